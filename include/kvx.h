@@ -1,0 +1,326 @@
+/*
+ * kvx.h -- C ABI of the MI355X-native paged KV-cache path.
+ *
+ * A drop-in for RichEngine's KV data plane: page storage in extents, page
+ * tables of extent-address|index entries, quantize-on-append, paged
+ * gather-dequant attention (decode / speculative verify / chunked prefill) with
+ * split partials and a fixed-order merge, tree-path compaction and whole-page
+ * copy, plus the page pool that owns page references.  The page format is the
+ * reference's, byte for byte.  Every entry point cites the reference interface
+ * it replaces (paths relative to the reference checkout).
+ *
+ * Conventions
+ *  - Plain pointers and sizes only.  `stream` is a hipStream_t passed as void*
+ *    (NULL = the default stream).  Work is enqueued on it and not waited for.
+ *  - Device pointers are caller-owned HBM; the library owns extents only and
+ *    allocates nothing on the launch path.
+ *  - Status codes replace the reference's exceptions; nothing is enqueued when
+ *    a call fails.  kvx_last_error() gives the message of the calling thread's
+ *    last failure.
+ *  - Lanes whose parameters fail the kernel contract write nothing (as the
+ *    reference kernels do); host-side validation reports them first.
+ *  - One caller thread per storage/pool (as the reference's engine thread).
+ */
+#ifndef KVX_H
+#define KVX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status: the reference's exception classes as values ---- */
+#define KVX_OK 0
+#define KVX_EINVAL (-1)  /* std::invalid_argument: bad geometry / parameters  */
+#define KVX_ESTATE (-2)  /* std::logic_error: lifecycle misuse                */
+#define KVX_ENOMEM (-3)  /* allocation refused (metal::AllocationResult)      */
+#define KVX_ERANGE (-4)  /* std::out_of_range: page / extent id past the pool */
+#define KVX_EDEVICE (-5) /* a HIP call failed                                 */
+const char *kvx_last_error(void);
+
+/* ---- formats and limits ---- */
+/* runtime/ops/PagedKv.hpp:16 (kv::Format), same values */
+#define KVX_FMT_INT8 1u
+#define KVX_FMT_BF16 2u
+#define KVX_FMT_INT4 3u
+#define KVX_FMT_FP8E4M3 4u
+/* runtime/metal/abi/KvExtent.h:27-30 */
+#define KVX_KEYS 0u
+#define KVX_KEY_SCALES 1u
+#define KVX_VALUES 2u
+#define KVX_VALUE_SCALES 3u
+/* runtime/metal/abi/ExecutionGeometry.h:7-39, abi/KvExtent.h:19 */
+#define KVX_PAGE_TOKENS 32u
+#define KVX_PAGE_INDEX_BITS 14u
+#define KVX_PAGE_INDEX_MASK ((1u << KVX_PAGE_INDEX_BITS) - 1u)
+#define KVX_VERIFY_ROWS 8u
+#define KVX_TREE_NODES 16u
+#define KVX_MAX_CONTEXT_TOKENS 262144u
+#define KVX_MAX_PHYSICAL_TOKENS (KVX_MAX_CONTEXT_TOKENS + KVX_TREE_NODES - 1u)
+#define KVX_PREFILL_TOKEN_BUDGET 2048u
+#define KVX_PREFILL_TILE_ROWS 8u
+#define KVX_PREFILL_MAX_SPLITS 32u
+#define KVX_VERIFY_MAX_SPLITS 128u
+#define KVX_VERIFY_CHUNK_STRIDE 32u
+/* The reference batches at most 4 lanes (abi/ExecutionGeometry.h:22); this
+   library takes any lane count and launches in groups of KVX_LANES_PER_LAUNCH. */
+#define KVX_LANES_PER_LAUNCH 32u
+
+/* runtime/ops/PagedKv.hpp:125-136 (kv::Layout) */
+typedef struct kvx_layout {
+  uint32_t layers;
+  uint32_t kv_heads;
+  uint32_t head_dim;
+  uint32_t format;
+  float score_scale; /* 0 selects 1/sqrt(head_dim) */
+} kvx_layout;
+
+/* runtime/metal/abi/KvExtent.h:93-96 (RichKvLayer) */
+typedef struct kvx_kv_layer {
+  uint32_t extent_pages;
+  uint32_t offset;
+} kvx_kv_layer;
+
+/* runtime/metal/abi/PagedAttention.h:39-45 (RichChunkedPrefillParams, 24 B) */
+typedef struct kvx_chunk_params {
+  uint32_t committed_tokens;
+  uint32_t chunk_tokens;
+  uint32_t chunk_stride;
+  uint32_t page_table_entries;
+  kvx_kv_layer kv; /* filled by the library from `layer` */
+} kvx_chunk_params;
+
+/* runtime/metal/abi/PagedAttention.h:52-61 (RichPrefillAttentionParams, 32 B) */
+typedef struct kvx_prefill_params {
+  uint32_t committed_tokens;
+  uint32_t rows;
+  uint32_t chunk_stride;
+  uint32_t page_table_entries;
+  kvx_kv_layer kv;
+  uint32_t split_count;
+  float score_scale;
+} kvx_prefill_params;
+
+/* runtime/metal/abi/PagedAttention.h:72-84 (RichVerifyAttentionParams, 36 B) */
+typedef struct kvx_verify_params {
+  uint32_t committed_tokens;
+  uint32_t page_table_entries;
+  kvx_kv_layer kv;
+  uint32_t split_count;
+  uint32_t slot_splits;
+  uint32_t active_rows;
+  uint32_t row_capacity;
+  float score_scale;
+} kvx_verify_params;
+
+/* runtime/ops/PagedKv.hpp:48-51 (kv::PageCopy) */
+typedef struct kvx_page_copy {
+  uint32_t from;
+  uint32_t to;
+} kvx_page_copy;
+
+/* ---- layout geometry: kv::Layout members, runtime/ops/PagedKv.hpp:137-230 ---- */
+int kvx_layout_valid(const kvx_layout *layout);
+uint64_t kvx_layout_data_bytes_per_layer_page(const kvx_layout *layout);
+uint64_t kvx_layout_scale_bytes_per_layer_page(const kvx_layout *layout);
+uint64_t kvx_layout_bytes_per_layer_page(const kvx_layout *layout);
+uint64_t kvx_layout_bytes_per_model_page(const kvx_layout *layout);
+uint32_t kvx_layout_extent_alignment_pages(const kvx_layout *layout);
+uint32_t kvx_layout_minimum_extent_pages(const kvx_layout *layout);
+uint32_t kvx_layout_maximum_extent_pages(const kvx_layout *layout);
+uint32_t kvx_layout_extent_pages_for(const kvx_layout *layout, uint64_t pages);
+/* The largest extent the page entry and the 32-bit layer offset allow: whole
+   alignment units, at most 16383 pages, below 4 GiB.  MI355X pools want few,
+   large extents (fewer allocations, better TLB reach); the reference's 128 MiB
+   target (extent_pages_for) stays available for parity. */
+uint32_t kvx_layout_largest_extent_pages(const kvx_layout *layout);
+/* runtime/metal/abi/KvExtent.h:76-89 (richengine_kv_offset) */
+uint64_t kvx_kv_offset(uint32_t extent_pages, uint32_t data_bytes, uint32_t scale_bytes,
+                       uint32_t layer, uint32_t tensor, uint32_t index);
+
+/* ---- planning: runtime/ops/PagedAttention.hpp:54-95, PagedAttention.cpp:23-32,200-297 ---- */
+/* kv::verifyAttentionSplits: clamp(ceil(pages/16), 32, 128) */
+uint32_t kvx_verify_splits(uint32_t committed_tokens, uint32_t rows);
+/* prefillSplits: clamp(32 / tiles, 1, 32) with tiles = ceil(rows / 8) */
+uint32_t kvx_prefill_splits(uint32_t rows);
+/* The batched-decode rule of this library: one split per
+   KVX_DECODE_PAGES_PER_SPLIT visible pages, at least 1, at most 128.  Decode at
+   batch 32 has enough (lane, head) parallelism that the reference's 32-split
+   floor would only add partial traffic. */
+#define KVX_DECODE_PAGES_PER_SPLIT 16u
+uint32_t kvx_decode_splits(uint32_t committed_tokens, uint32_t rows);
+/* kv::chunkedPrefillValidationError: 0 ok, 1 chunk_tokens_out_of_range,
+   2 context_out_of_range, 3 chunk_stride_invalid, 4 page_table_too_short */
+int kvx_chunk_validation(const kvx_chunk_params *params);
+/* ops::PagedAttention::prefillPlan(...).workspace / prefillWorkspace / verifyWorkspace.
+   Bytes of partials and statistics; a workspace buffer holds partials first,
+   then statistics at the next 256-byte boundary. */
+int kvx_prefill_workspace(uint32_t rows, uint32_t query_heads, const kvx_layout *layout,
+                          uint64_t *partials_bytes, uint64_t *statistics_bytes);
+int kvx_prefill_workspace_bound(uint32_t maximum_rows, uint32_t query_heads,
+                                const kvx_layout *layout, uint64_t *partials_bytes,
+                                uint64_t *statistics_bytes);
+int kvx_verify_workspace(uint32_t lanes, uint32_t row_capacity, uint32_t query_heads,
+                         const kvx_layout *layout, uint64_t *partials_bytes,
+                         uint64_t *statistics_bytes);
+/* Total bytes of one workspace buffer for an attend call over these lanes
+   (sum over lanes of slot_splits * kv_heads * row_capacity * group fused rows). */
+uint64_t kvx_attend_workspace_bytes(const kvx_verify_params *lanes, uint32_t n_lanes,
+                                    uint32_t query_heads, const kvx_layout *layout);
+
+/* ---- page storage: kv::PageStorage / kv::ExtentStorage,
+        runtime/ops/PageStorage.hpp:27-102, runtime/ops/PagedKv.hpp:56-76 ---- */
+typedef struct kvx_storage kvx_storage;
+/* PageStorage::PageStorage (PageStorage.mm:12-46).  aligned != 0 enforces whole
+   alignment units per extent as production does; 0 takes any extent size the
+   page index allows (dev/tuning/HostKvExtents.hpp:158-169, test pools). */
+int kvx_storage_create(const kvx_layout *layout, uint32_t page_count, uint32_t extent_pages,
+                       int aligned, kvx_storage **out);
+void kvx_storage_destroy(kvx_storage *storage);
+uint32_t kvx_storage_page_count(const kvx_storage *storage);
+uint32_t kvx_storage_extent_pages(const kvx_storage *storage);
+uint64_t kvx_storage_bytes_per_page(const kvx_storage *storage);
+uint64_t kvx_storage_extent_bytes(const kvx_storage *storage);
+uint64_t kvx_storage_allocated_bytes(const kvx_storage *storage);
+int kvx_storage_is_allocated(const kvx_storage *storage, uint32_t page);
+/* ExtentStorage::allocateExtent / releaseExtent (PageStorage.mm:64-93).
+   KVX_ENOMEM when hipMalloc refuses; KVX_ESTATE for an (un)allocated extent.
+   A new extent is zero-filled.  Release synchronises the device first. */
+int kvx_storage_allocate_extent(kvx_storage *storage, uint32_t extent);
+int kvx_storage_release_extent(kvx_storage *storage, uint32_t extent);
+/* A budget in bytes past which allocate_extent answers KVX_ENOMEM (the
+   reference's admission callback, runtime/metal/MetalBackend.hpp:18-45); 0 = none. */
+void kvx_storage_set_budget(kvx_storage *storage, uint64_t bytes);
+/* PageStorage::layers()[layer] */
+int kvx_storage_layer(const kvx_storage *storage, uint32_t layer, kvx_kv_layer *out);
+/* PageStorage::writeEntries (PageStorage.mm:127-141): entries [first, n) of the
+   pages' table.  The first form fills a host array; the second copies them to
+   a device table on `stream` (entries before `first` are left as they are). */
+int kvx_storage_entries(const kvx_storage *storage, const uint32_t *pages, uint32_t n,
+                        uint32_t first, uint64_t *table_host);
+int kvx_storage_write_entries(const kvx_storage *storage, const uint32_t *pages, uint32_t n,
+                              uint32_t first, uint64_t *table_device, uint64_t table_capacity,
+                              void *stream);
+/* PageStorage::spans (PageStorage.mm:143-167) for memory the host cannot map:
+   the page's bytes, layer by layer as keys, key scales, values, value scales
+   (bytes_per_page long), copied to / from host memory.  Synchronous. */
+int kvx_storage_page_read(const kvx_storage *storage, uint32_t page, void *host_bytes);
+int kvx_storage_page_write(kvx_storage *storage, uint32_t page, const void *host_bytes);
+/* Raw extent bytes, for tests that compare whole extents.  Synchronous. */
+int kvx_storage_extent_read(const kvx_storage *storage, uint32_t extent, uint64_t offset,
+                            uint64_t bytes, void *host_bytes);
+int kvx_storage_extent_write(kvx_storage *storage, uint32_t extent, uint64_t offset,
+                             uint64_t bytes, const void *host_bytes);
+
+/* ExtentStorage::copyPages (PageStorage.mm:95-114): every tensor of every layer
+   of each page, on `stream`.  All-or-nothing validation first: KVX_ESTATE and no
+   copy when any page sits in an unallocated extent, KVX_ERANGE past the pool,
+   KVX_EINVAL when a destination is also a source of the batch (the reference
+   copies in order on the host; the device copies all pages at once). */
+int kv_page_copy(kvx_storage *storage, const kvx_page_copy *copies, uint32_t n, void *stream);
+
+/* ---- page pool: engine::KvPool, runtime/engine/cache/KvPool.hpp:75-115 ---- */
+typedef struct kvx_pool kvx_pool;
+typedef struct kvx_pool_snapshot { /* KvPool.hpp:12-35 (KvPoolSnapshot) */
+  uint32_t pages_allocated, pages_free, pages_active, pages_prefix;
+  uint64_t allocated_bytes, reclaimable_bytes;
+  uint64_t extent_allocations, extent_releases;
+  double extent_allocate_max_ms, extent_release_max_ms;
+  uint64_t extent_compactions, pages_moved;
+} kvx_pool_snapshot;
+/* KvPool::KvPool (KvPool.cpp:14-33): allocates the runway. */
+int kvx_pool_create(kvx_storage *storage, uint32_t runway_pages, kvx_pool **out);
+void kvx_pool_destroy(kvx_pool *pool);
+/* KvPool::acquirePages (KvPool.cpp:35-72): `count` pages with one active
+   reference each, or KVX_ENOMEM with no page held (extents allocated on the
+   way stay, reclaimable). */
+int kvx_pool_acquire(kvx_pool *pool, uint32_t count, uint32_t *pages);
+int kvx_pool_retain(kvx_pool *pool, uint32_t page, int prefix_owner);  /* KvPool.cpp:74-91 */
+int kvx_pool_release(kvx_pool *pool, uint32_t page, int prefix_owner); /* KvPool.cpp:93-105 */
+int kvx_pool_page_active(const kvx_pool *pool, uint32_t page);
+uint32_t kvx_pool_free_pages(const kvx_pool *pool);
+/* KvPool::reclaimEmptyExtents (KvPool.cpp:125-141): bytes released via *released. */
+int kvx_pool_reclaim_empty(kvx_pool *pool, int keep_runway, uint32_t limit, uint64_t *released);
+/* KvPool::compactExtent (KvPool.cpp:165-230): empties the sparsest extent into
+   the fullest others through kv_page_copy on `stream`.  *moved_pages = 0 when
+   nothing moved; otherwise *first_page and destinations[extent_pages] say where
+   each page of the emptied extent went (KvPageMoves, KvPool.hpp:39-52). */
+int kvx_pool_compact_extent(kvx_pool *pool, const uint32_t *fixed, uint32_t n_fixed,
+                            uint32_t *first_page, uint32_t *destinations,
+                            uint32_t *moved_pages, void *stream);
+int kvx_pool_snapshot_get(const kvx_pool *pool, kvx_pool_snapshot *out);
+
+/* ---- the hot path ---- */
+
+/* Quantize-on-append + scatter through page tables.
+   Replaces ops::PagedAttention::addPrefillStore (runtime/ops/PagedAttention.cpp:424-440;
+   kernels prefill/paged_attention_store.metal:7-148) when verify_max_rows == 0,
+   and the store dispatch of ops::PagedAttention::addVerify
+   (PagedAttention.cpp:467-500; decode/paged_attention_store.metal:3-186) otherwise.
+   chunk_keys is bf16 [lane][kv head][chunk_stride][D], chunk_values bf16
+   [lane][kv head][D][chunk_stride]; lanes lie lane_stride elements apart.
+   page_tables[lane] is the device address of that lane's entries.
+   verify_max_rows > 0 applies the verify contract: chunk_stride == 32 and
+   chunk_tokens <= verify_max_rows (15 in the reference; up to 16 here).
+   Host validation follows kv::chunkedPrefillValidationError; the kernel keeps the
+   contract check of common/paged_store_row.h:14-29. */
+int kv_append(const kvx_storage *storage, uint32_t layer, const void *chunk_keys,
+              const void *chunk_values, const uint64_t *const *page_tables,
+              const kvx_chunk_params *lanes, uint32_t n_lanes, uint64_t lane_stride,
+              uint32_t verify_max_rows, void *stream);
+
+/* Paged attention of `active_rows` query rows per lane over committed history
+   plus those rows (chain: causal; tree: row_masks).  Replaces the split and
+   reduce dispatches of ops::PagedAttention::addVerify (PagedAttention.cpp:506-544;
+   kernels decode/paged_attention.metal:23-464, common/paged_attention_tile.h).
+   queries / output: bf16 [lane][kv head][row_stride][group][D]
+   (dev/tuning/AttentionFixture.hpp:167-173; row_stride = 32 in the reference).
+   row_masks: NULL, or u32 [lane][row_capacity] ancestor bitmasks
+   (shared/embedding.metal:248-281).  Each lane's split_count partitions its
+   pages as ceil(pages / split_count) per split; slot_splits is ignored (slots
+   are packed per lane).  Output rows >= active_rows up to row_capacity are
+   written as zeros.  workspace: device memory of at least
+   kvx_attend_workspace_bytes(). */
+int kv_attend_verify(const kvx_storage *storage, uint32_t layer, uint32_t query_heads,
+                     const void *queries, void *output, const uint64_t *const *page_tables,
+                     const kvx_verify_params *lanes, uint32_t n_lanes,
+                     const uint32_t *row_masks, uint32_t row_stride, void *workspace,
+                     uint64_t workspace_bytes, void *stream);
+
+/* One-row decode attention per lane: kv_attend_verify with active_rows =
+   row_capacity = 1 on the bandwidth-tuned kernels (the reference reaches decode
+   through its prefill entries with rows = 1, prefill/paged_attention.metal:7-67,
+   pinned by dev/tests/engine/paged_attention_plan_test.mm:1019). */
+int kv_attend_decode(const kvx_storage *storage, uint32_t layer, uint32_t query_heads,
+                     const void *queries, void *output, const uint64_t *const *page_tables,
+                     const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                     void *workspace, uint64_t workspace_bytes, void *stream);
+
+/* Chunked prefill attention of one sequence: rows in tiles of 8, each tile
+   causal over committed + its rows.  Replaces ops::PagedAttention::addPrefill
+   (PagedAttention.cpp:442-465; kernels prefill/paged_attention.metal:7-206).
+   queries / output: bf16 [kv head][chunk_stride][group][D].  workspace: at
+   least kvx_prefill_workspace() partials + statistics. */
+int kv_attend_prefill(const kvx_storage *storage, uint32_t layer, uint32_t query_heads,
+                      const void *queries, void *output, const uint64_t *page_table,
+                      const kvx_prefill_params *params, void *workspace,
+                      uint64_t workspace_bytes, void *stream);
+
+/* Tree-path compaction after acceptance: for i < retained_count[lane], the
+   row at committed + retained_path[lane * path_stride + i] moves to
+   committed + i.  Replaces ops::PagedAttention::addVerifyTreeCompact
+   (PagedAttention.cpp:546-573; kernel decode/paged_attention_store.metal:198-309).
+   retained_path / retained_count are device arrays (the acceptance kernel
+   writes them, decode/sampling.metal:1927-1989); path_stride is 8 in the
+   reference.  layer = UINT32_MAX compacts every layer. */
+int kv_compact_path(const kvx_storage *storage, uint32_t layer,
+                    const uint64_t *const *page_tables, const kvx_chunk_params *lanes,
+                    uint32_t n_lanes, const uint32_t *retained_path,
+                    const uint32_t *retained_count, uint32_t path_stride, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KVX_H */

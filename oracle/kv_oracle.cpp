@@ -199,8 +199,10 @@ void store_row(uint32_t format, uint32_t kv_heads, uint32_t head_dim,
     const int limit = format == KO_INT4 ? 7 : 127;
     int code = 0;
     if (maximum != 0.0f) {
-      const float scaled = v * qmax / maximum;
-      code = std::clamp(int(std::nearbyint(scaled)), -limit, limit);
+      // Clamped as a float first: a product that overflowed to infinity must
+      // saturate like the GPU's float-to-int conversion, not wrap.
+      const float rounded = std::nearbyint(v * qmax / maximum);
+      code = rounded != rounded ? 0 : int(std::min(std::max(rounded, float(-limit)), float(limit)));
     }
     if (format == KO_INT8) {
       reinterpret_cast<int8_t *>(

@@ -1,0 +1,38 @@
+"""Builds libkvx.so (HIP kernels + C ABI) for gfx950, in-tree."""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libkvx.so")
+SOURCES = ["kvx_host.cpp", "kvx_pool.cpp", "kvx_pool_abi.cpp", "kvx_kernels.hip",
+           "kvx_decode_int4.hip"]
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
+         # packed fp32 instructions stay off for every kernel of this library
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-I", os.path.join(ROOT, "include"), "-I", CSRC]
+
+
+def build(verbose=True):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    objects = []
+    os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    for src in SOURCES:
+        obj = os.path.join(HERE, "build", src + ".o")
+        cmd = [hipcc, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + FLAGS
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
+        objects.append(obj)
+    cmd = [hipcc, "-shared", "-o", LIB] + objects + ["--offload-arch=gfx950"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()
+    print(LIB)

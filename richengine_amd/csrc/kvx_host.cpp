@@ -1,0 +1,400 @@
+// Host side of libkvx: layout geometry, planning rules, extent storage and the
+// page pool.  No kernels here; device memory is reached through the HIP runtime.
+#include "kvx_internal.h"
+
+#include <algorithm>
+#include <chrono>
+#include <cstring>
+#include <limits>
+#include <numeric>
+
+namespace kvx {
+
+static thread_local std::string g_last_error;
+
+int fail(int code, const std::string &message) {
+  g_last_error = message;
+  return code;
+}
+int hip_fail(hipError_t error, const char *what) {
+  g_last_error = std::string(what) + ": " + hipGetErrorString(error);
+  (void)hipGetLastError();
+  return KVX_EDEVICE;
+}
+
+uint64_t Storage::extent_bytes() const { return uint64_t(extent_pages) * bytes_per_page(); }
+uint64_t Storage::bytes_per_page() const {
+  return uint64_t(layout.layers) * 2 * (uint64_t(data_bytes) + scale_bytes);
+}
+uint32_t Storage::allocated_extents() const {
+  uint32_t n = 0;
+  for (void *e : extents) n += e != nullptr;
+  return n;
+}
+
+namespace {
+
+constexpr uint64_t kRegionAlignment = 64 * 1024;            // PagedKv.hpp:89
+constexpr uint64_t kExtentTargetBytes = 128ull << 20;       // PagedKv.hpp:94
+
+uint64_t gcd(uint64_t a, uint64_t b) { return b ? gcd(b, a % b) : a; }
+uint64_t lcm(uint64_t a, uint64_t b) { return a && b ? a / gcd(a, b) * b : 0; }
+uint64_t aligned_region_pages(uint64_t bytes) {
+  return bytes ? kRegionAlignment / gcd(kRegionAlignment, bytes) : 0;
+}
+bool valid_format(uint32_t f) { return f >= KVX_FMT_INT8 && f <= KVX_FMT_FP8E4M3; }
+
+}  // namespace
+}  // namespace kvx
+
+using namespace kvx;
+
+// The page's spans in the reference's order: layer by layer, keys, key scales,
+// values, value scales.
+template <class F>
+static int for_each_span(const kvx_storage *s, uint32_t page, F &&f) {
+  if (page >= s->page_count) return fail(KVX_ERANGE, "invalid KV page id");
+  auto *extent = static_cast<uint8_t *>(s->extents[page / s->extent_pages]);
+  if (!extent)
+    return fail(KVX_ESTATE,
+                "KV page " + std::to_string(page) + " is in an extent that is not allocated");
+  const uint32_t index = page % s->extent_pages;
+  for (uint32_t layer = 0; layer < s->layout.layers; ++layer)
+    for (uint32_t tensor = KVX_KEYS; tensor <= KVX_VALUE_SCALES; ++tensor) {
+      const uint32_t bytes = (tensor & 1) ? s->scale_bytes : s->data_bytes;
+      if (!bytes) continue;
+      if (int rc = f(extent + kvx_kv_offset(s->extent_pages, s->data_bytes, s->scale_bytes, layer,
+                                            tensor, index),
+                     bytes))
+        return rc;
+    }
+  return KVX_OK;
+}
+extern "C" {
+
+const char *kvx_last_error(void) { return g_last_error.c_str(); }
+
+// ---------------------------------------------------------------- layout ---
+int kvx_layout_valid(const kvx_layout *l) {
+  return l && l->layers && l->kv_heads && l->head_dim && valid_format(l->format);
+}
+uint64_t kvx_layout_data_bytes_per_layer_page(const kvx_layout *l) {
+  return data_bytes_of(l->format, l->kv_heads, l->head_dim);
+}
+uint64_t kvx_layout_scale_bytes_per_layer_page(const kvx_layout *l) {
+  return scale_bytes_of(l->format, l->kv_heads);
+}
+uint64_t kvx_layout_bytes_per_layer_page(const kvx_layout *l) {
+  return 2 * (kvx_layout_data_bytes_per_layer_page(l) + kvx_layout_scale_bytes_per_layer_page(l));
+}
+uint64_t kvx_layout_bytes_per_model_page(const kvx_layout *l) {
+  return uint64_t(l->layers) * kvx_layout_bytes_per_layer_page(l);
+}
+uint32_t kvx_layout_extent_alignment_pages(const kvx_layout *l) {
+  const uint64_t data = aligned_region_pages(kvx_layout_data_bytes_per_layer_page(l));
+  if (l->format == KVX_FMT_BF16) return uint32_t(data);
+  return uint32_t(lcm(data, aligned_region_pages(kvx_layout_scale_bytes_per_layer_page(l))));
+}
+uint32_t kvx_layout_minimum_extent_pages(const kvx_layout *l) {
+  const uint64_t align = kvx_layout_extent_alignment_pages(l);
+  const uint64_t unit = align * kvx_layout_bytes_per_model_page(l);
+  if (!unit) return 0;
+  const uint64_t units = std::max<uint64_t>(1, (kExtentTargetBytes / 2 + unit - 1) / unit);
+  return uint32_t(units * align);
+}
+uint32_t kvx_layout_maximum_extent_pages(const kvx_layout *l) {
+  const uint64_t align = kvx_layout_extent_alignment_pages(l);
+  const uint64_t unit = align * kvx_layout_bytes_per_model_page(l);
+  if (!unit) return 0;
+  const uint64_t units = kExtentTargetBytes * 3 / 2 / unit;
+  return std::max(uint32_t(units * align), kvx_layout_minimum_extent_pages(l));
+}
+uint32_t kvx_layout_extent_pages_for(const kvx_layout *l, uint64_t pages) {
+  const uint32_t step = kvx_layout_extent_alignment_pages(l);
+  const uint64_t smallest = kvx_layout_minimum_extent_pages(l);
+  if (!smallest || pages < smallest) return 0;
+  const uint64_t largest = std::min<uint64_t>(kvx_layout_maximum_extent_pages(l), pages);
+  const uint64_t page_bytes = kvx_layout_bytes_per_model_page(l);
+  uint64_t best = 0, best_left = 0, best_distance = 0;
+  for (uint64_t candidate = smallest; candidate <= largest; candidate += step) {
+    const uint64_t bytes = candidate * page_bytes;
+    const uint64_t distance =
+        bytes > kExtentTargetBytes ? bytes - kExtentTargetBytes : kExtentTargetBytes - bytes;
+    const uint64_t left = pages % candidate;
+    if (!best || left < best_left || (left == best_left && distance < best_distance)) {
+      best = candidate;
+      best_left = left;
+      best_distance = distance;
+    }
+  }
+  return uint32_t(best);
+}
+uint32_t kvx_layout_largest_extent_pages(const kvx_layout *l) {
+  const uint64_t align = kvx_layout_extent_alignment_pages(l);
+  const uint64_t page_bytes = kvx_layout_bytes_per_model_page(l);
+  if (!align || !page_bytes) return 0;
+  uint64_t pages = std::min<uint64_t>(KVX_PAGE_INDEX_MASK,
+                                      std::numeric_limits<uint32_t>::max() / page_bytes);
+  pages = pages / align * align;
+  return uint32_t(pages);
+}
+uint64_t kvx_kv_offset(uint32_t extent_pages, uint32_t db, uint32_t sb, uint32_t layer,
+                       uint32_t tensor, uint32_t index) {
+  const RegionOffsets r = region_offsets(extent_pages, db, sb);
+  const uint64_t region = uint64_t(layer) * extent_pages * 2 * (uint64_t(db) + sb);
+  const uint64_t start[4] = {0, r.key_scales, r.values, r.value_scales};
+  return region + start[tensor & 3] + uint64_t(index) * ((tensor & 1) ? sb : db);
+}
+
+// -------------------------------------------------------------- planning ---
+static uint32_t pages_of(uint64_t tokens) {
+  return uint32_t((tokens + KVX_PAGE_TOKENS - 1) / KVX_PAGE_TOKENS);
+}
+uint32_t kvx_verify_splits(uint32_t committed, uint32_t rows) {
+  const uint32_t scaled = (pages_of(uint64_t(committed) + rows) + 15) / 16;
+  return std::min(std::max(32u, scaled), KVX_VERIFY_MAX_SPLITS);
+}
+uint32_t kvx_prefill_splits(uint32_t rows) {
+  const uint32_t tiles = (rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+  if (!tiles) return KVX_PREFILL_MAX_SPLITS;
+  return std::min(std::max(KVX_PREFILL_MAX_SPLITS / tiles, 1u), KVX_PREFILL_MAX_SPLITS);
+}
+uint32_t kvx_decode_splits(uint32_t committed, uint32_t rows) {
+  const uint32_t pages = pages_of(uint64_t(committed) + rows);
+  const uint32_t wanted = (pages + KVX_DECODE_PAGES_PER_SPLIT - 1) / KVX_DECODE_PAGES_PER_SPLIT;
+  return std::min(std::max(1u, wanted), KVX_VERIFY_MAX_SPLITS);
+}
+int kvx_chunk_validation(const kvx_chunk_params *p) {
+  if (!p->chunk_tokens || p->chunk_tokens > KVX_PREFILL_TOKEN_BUDGET) return 1;
+  if (uint64_t(p->committed_tokens) + p->chunk_tokens > KVX_MAX_PHYSICAL_TOKENS) return 2;
+  if (p->chunk_stride < p->chunk_tokens || p->chunk_stride > KVX_PREFILL_TOKEN_BUDGET ||
+      p->chunk_stride % KVX_PAGE_TOKENS)
+    return 3;
+  if (p->page_table_entries < pages_of(uint64_t(p->committed_tokens) + p->chunk_tokens)) return 4;
+  return 0;
+}
+static int geometry_ok(uint32_t query_heads, const kvx_layout *l) {
+  if (!kvx_layout_valid(l) || !query_heads || query_heads % l->kv_heads)
+    return fail(KVX_EINVAL, "query heads are not a multiple of the layout's KV heads");
+  return KVX_OK;
+}
+static void workspace_rows(uint64_t rows, uint32_t head_dim, uint64_t *pb, uint64_t *sb) {
+  if (pb) *pb = rows * head_dim * sizeof(float);
+  if (sb) *sb = rows * 2 * sizeof(float);
+}
+int kvx_prefill_workspace(uint32_t rows, uint32_t query_heads, const kvx_layout *l, uint64_t *pb,
+                          uint64_t *sb) {
+  if (int rc = geometry_ok(query_heads, l)) return rc;
+  if (!rows || rows > KVX_PREFILL_TOKEN_BUDGET)
+    return fail(KVX_EINVAL, "invalid paged prefill attention geometry");
+  const uint64_t tiles = (rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+  workspace_rows(tiles * kvx_prefill_splits(rows) * KVX_PREFILL_TILE_ROWS * query_heads,
+                 l->head_dim, pb, sb);
+  return KVX_OK;
+}
+int kvx_prefill_workspace_bound(uint32_t maximum_rows, uint32_t query_heads, const kvx_layout *l,
+                                uint64_t *pb, uint64_t *sb) {
+  if (int rc = geometry_ok(query_heads, l)) return rc;
+  if (!maximum_rows || maximum_rows > KVX_PREFILL_TOKEN_BUDGET)
+    return fail(KVX_EINVAL, "invalid attention workspace rows");
+  uint64_t slots = 0;
+  for (uint32_t rows = 1; rows <= maximum_rows; rows += KVX_PREFILL_TILE_ROWS) {
+    const uint64_t tiles = (rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+    slots = std::max(slots, tiles * kvx_prefill_splits(rows));
+  }
+  workspace_rows(slots * KVX_PREFILL_TILE_ROWS * query_heads, l->head_dim, pb, sb);
+  return KVX_OK;
+}
+int kvx_verify_workspace(uint32_t lanes, uint32_t row_capacity, uint32_t query_heads,
+                         const kvx_layout *l, uint64_t *pb, uint64_t *sb) {
+  if (int rc = geometry_ok(query_heads, l)) return rc;
+  if (!lanes || !row_capacity) return fail(KVX_EINVAL, "invalid attention workspace batch width");
+  workspace_rows(uint64_t(lanes) * row_capacity * KVX_VERIFY_MAX_SPLITS * query_heads, l->head_dim,
+                 pb, sb);
+  return KVX_OK;
+}
+uint64_t kvx_attend_workspace_bytes(const kvx_verify_params *lanes, uint32_t n, uint32_t query_heads,
+                                    const kvx_layout *l) {
+  uint64_t rows = 0;
+  for (uint32_t i = 0; i < n; ++i)
+    rows += uint64_t(lanes[i].split_count) * lanes[i].row_capacity * query_heads;
+  const uint64_t partials = (rows * l->head_dim * sizeof(float) + 255) / 256 * 256;
+  return partials + rows * 2 * sizeof(float);
+}
+
+// --------------------------------------------------------------- storage ---
+int kvx_storage_create(const kvx_layout *layout, uint32_t page_count, uint32_t extent_pages,
+                       int aligned, kvx_storage **out) {
+  if (!out) return fail(KVX_EINVAL, "null output");
+  *out = nullptr;
+  if (!kvx_layout_valid(layout)) return fail(KVX_EINVAL, "KV page storage layout is invalid");
+  if (layout->head_dim != 64 && layout->head_dim != 128 && layout->head_dim != 256)
+    return fail(KVX_EINVAL, "head dimension must be 64, 128 or 256");
+  const uint64_t extent_bytes = uint64_t(extent_pages) * kvx_layout_bytes_per_model_page(layout);
+  if (!extent_pages || (aligned && extent_pages % kvx_layout_extent_alignment_pages(layout)) ||
+      extent_pages > KVX_PAGE_INDEX_MASK ||
+      extent_bytes > std::numeric_limits<uint32_t>::max())
+    return fail(KVX_EINVAL, "KV extent geometry is invalid");
+  if (!page_count || page_count % extent_pages)
+    return fail(KVX_EINVAL, "KV page pool is not a whole number of extents");
+  auto *s = new kvx_storage;
+  s->layout = *layout;
+  s->page_count = page_count;
+  s->extent_pages = extent_pages;
+  s->data_bytes = uint32_t(kvx_layout_data_bytes_per_layer_page(layout));
+  s->scale_bytes = uint32_t(kvx_layout_scale_bytes_per_layer_page(layout));
+  s->extents.assign(page_count / extent_pages, nullptr);
+  s->allocations.assign(page_count / extent_pages, nullptr);
+  if (hipGetDevice(&s->device) != hipSuccess) {
+    delete s;
+    return fail(KVX_EDEVICE, "no HIP device: the paged KV path needs a GPU");
+  }
+  *out = s;
+  return KVX_OK;
+}
+void kvx_storage_destroy(kvx_storage *s) {
+  if (!s) return;
+  (void)hipDeviceSynchronize();
+  for (void *raw : s->allocations)
+    if (raw) (void)hipFree(raw);
+  delete s;
+}
+uint32_t kvx_storage_page_count(const kvx_storage *s) { return s->page_count; }
+uint32_t kvx_storage_extent_pages(const kvx_storage *s) { return s->extent_pages; }
+uint64_t kvx_storage_bytes_per_page(const kvx_storage *s) { return s->bytes_per_page(); }
+uint64_t kvx_storage_extent_bytes(const kvx_storage *s) { return s->extent_bytes(); }
+uint64_t kvx_storage_allocated_bytes(const kvx_storage *s) {
+  return uint64_t(s->allocated_extents()) * s->extent_bytes();
+}
+int kvx_storage_is_allocated(const kvx_storage *s, uint32_t page) {
+  return page < s->page_count && s->extents[page / s->extent_pages] != nullptr;
+}
+void kvx_storage_set_budget(kvx_storage *s, uint64_t bytes) { s->budget_bytes = bytes; }
+
+int kvx_storage_allocate_extent(kvx_storage *s, uint32_t extent) {
+  if (extent >= s->extents.size()) return fail(KVX_ERANGE, "KV extent is past the pool");
+  if (s->extents[extent])
+    return fail(KVX_ESTATE, "KV extent " + std::to_string(extent) + " is already allocated");
+  const uint64_t bytes = s->extent_bytes();
+  if (s->budget_bytes && kvx_storage_allocated_bytes(s) + bytes > s->budget_bytes)
+    return fail(KVX_ENOMEM, "KV extent refused by the storage budget");
+  // Page entries keep the page index in the low 14 bits of the extent address.
+  // Large allocations come back aligned far beyond that; a small test extent
+  // may not, and is then allocated again with room to align inside it.
+  constexpr uint64_t kAlign = uint64_t(KVX_PAGE_INDEX_MASK) + 1;
+  void *raw = nullptr;
+  if (hipMalloc(&raw, bytes) != hipSuccess || !raw) {
+    (void)hipGetLastError();
+    return fail(KVX_ENOMEM, "hipMalloc refused a KV extent of " + std::to_string(bytes) + " bytes");
+  }
+  if (reinterpret_cast<uint64_t>(raw) & KVX_PAGE_INDEX_MASK) {
+    (void)hipFree(raw);
+    raw = nullptr;
+    if (hipMalloc(&raw, bytes + kAlign) != hipSuccess || !raw) {
+      (void)hipGetLastError();
+      return fail(KVX_ENOMEM, "hipMalloc refused a KV extent of " + std::to_string(bytes) + " bytes");
+    }
+  }
+  void *p = reinterpret_cast<void *>((reinterpret_cast<uint64_t>(raw) + kAlign - 1) & ~(kAlign - 1));
+  if (hipMemset(p, 0, bytes) != hipSuccess) {
+    (void)hipFree(raw);
+    return hip_fail(hipGetLastError(), "hipMemset(extent)");
+  }
+  s->extents[extent] = p;
+  s->allocations[extent] = raw;
+  return KVX_OK;
+}
+int kvx_storage_release_extent(kvx_storage *s, uint32_t extent) {
+  if (extent >= s->extents.size()) return fail(KVX_ERANGE, "KV extent is past the pool");
+  if (!s->extents[extent])
+    return fail(KVX_ESTATE, "KV extent " + std::to_string(extent) + " is not allocated");
+  // Kernels reach extents through page tables without retaining them: wait for
+  // everything in flight before the memory goes away.
+  KVX_HIP(hipDeviceSynchronize());
+  KVX_HIP(hipFree(s->allocations[extent]));
+  s->extents[extent] = nullptr;
+  s->allocations[extent] = nullptr;
+  return KVX_OK;
+}
+int kvx_storage_layer(const kvx_storage *s, uint32_t layer, kvx_kv_layer *out) {
+  if (layer >= s->layout.layers) return fail(KVX_ERANGE, "KV layer is outside the layout");
+  out->extent_pages = s->extent_pages;
+  out->offset = uint32_t(kvx_kv_offset(s->extent_pages, s->data_bytes, s->scale_bytes, layer,
+                                       KVX_KEYS, 0));
+  return KVX_OK;
+}
+int kvx_storage_entries(const kvx_storage *s, const uint32_t *pages, uint32_t n, uint32_t first,
+                        uint64_t *table) {
+  if (first > n)
+    return fail(KVX_EINVAL, "KV page table entries start past the end of its pages");
+  for (uint32_t i = first; i < n; ++i) {
+    if (pages[i] >= s->page_count) return fail(KVX_ERANGE, "invalid KV page id");
+    const uint32_t extent = pages[i] / s->extent_pages;
+    if (!s->extents[extent])
+      return fail(KVX_ESTATE, "KV page " + std::to_string(pages[i]) +
+                                  " is in an extent that is not allocated");
+  }
+  for (uint32_t i = first; i < n; ++i) {
+    const uint32_t extent = pages[i] / s->extent_pages;
+    table[i] = reinterpret_cast<uint64_t>(s->extents[extent]) | (pages[i] - extent * s->extent_pages);
+  }
+  return KVX_OK;
+}
+int kvx_storage_write_entries(const kvx_storage *s, const uint32_t *pages, uint32_t n,
+                              uint32_t first, uint64_t *table_device, uint64_t capacity,
+                              void *stream) {
+  if (!table_device || capacity < n)
+    return fail(KVX_ESTATE, "KV page table is missing or too small for its entries");
+  std::vector<uint64_t> host(n);
+  if (int rc = kvx_storage_entries(s, pages, n, first, host.data())) return rc;
+  if (first == n) return KVX_OK;
+  // The staging vector dies with this call, so the copy completes here.
+  KVX_HIP(hipMemcpyAsync(table_device + first, host.data() + first, (n - first) * sizeof(uint64_t),
+                         hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+  KVX_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return KVX_OK;
+}
+
+int kvx_storage_page_read(const kvx_storage *s, uint32_t page, void *host) {
+  auto *out = static_cast<uint8_t *>(host);
+  KVX_HIP(hipDeviceSynchronize());
+  return for_each_span(s, page, [&](uint8_t *device, uint32_t bytes) -> int {
+    KVX_HIP(hipMemcpy(out, device, bytes, hipMemcpyDeviceToHost));
+    out += bytes;
+    return KVX_OK;
+  });
+}
+int kvx_storage_page_write(kvx_storage *s, uint32_t page, const void *host) {
+  auto *in = static_cast<const uint8_t *>(host);
+  KVX_HIP(hipDeviceSynchronize());
+  return for_each_span(s, page, [&](uint8_t *device, uint32_t bytes) -> int {
+    KVX_HIP(hipMemcpy(device, in, bytes, hipMemcpyHostToDevice));
+    in += bytes;
+    return KVX_OK;
+  });
+}
+static int extent_range(const kvx_storage *s, uint32_t extent, uint64_t offset, uint64_t bytes) {
+  if (extent >= s->extents.size()) return fail(KVX_ERANGE, "KV extent is past the pool");
+  if (!s->extents[extent]) return fail(KVX_ESTATE, "KV extent is not allocated");
+  if (offset > s->extent_bytes() || bytes > s->extent_bytes() - offset)
+    return fail(KVX_ERANGE, "range is outside the extent");
+  return KVX_OK;
+}
+int kvx_storage_extent_read(const kvx_storage *s, uint32_t extent, uint64_t offset, uint64_t bytes,
+                            void *host) {
+  if (int rc = extent_range(s, extent, offset, bytes)) return rc;
+  KVX_HIP(hipDeviceSynchronize());
+  KVX_HIP(hipMemcpy(host, static_cast<uint8_t *>(s->extents[extent]) + offset, bytes,
+                    hipMemcpyDeviceToHost));
+  return KVX_OK;
+}
+int kvx_storage_extent_write(kvx_storage *s, uint32_t extent, uint64_t offset, uint64_t bytes,
+                             const void *host) {
+  if (int rc = extent_range(s, extent, offset, bytes)) return rc;
+  KVX_HIP(hipDeviceSynchronize());
+  KVX_HIP(hipMemcpy(static_cast<uint8_t *>(s->extents[extent]) + offset, host, bytes,
+                    hipMemcpyHostToDevice));
+  return KVX_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,94 @@
+// Internal definitions shared by the host side and the kernels of libkvx.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "kvx.h"
+
+namespace kvx {
+
+// ---- errors -----------------------------------------------------------------
+int fail(int code, const std::string &message);
+int hip_fail(hipError_t error, const char *what);
+#define KVX_HIP(call)                                     \
+  do {                                                    \
+    hipError_t kvx_e_ = (call);                           \
+    if (kvx_e_ != hipSuccess) return ::kvx::hip_fail(kvx_e_, #call); \
+  } while (0)
+
+// ---- geometry (host and device) --------------------------------------------
+__host__ __device__ inline bool quantized(uint32_t format) { return format != KVX_FMT_BF16; }
+
+__host__ __device__ inline uint32_t data_bytes_of(uint32_t format, uint32_t kv_heads,
+                                                  uint32_t head_dim) {
+  const uint32_t elements = KVX_PAGE_TOKENS * kv_heads * head_dim;
+  return format == KVX_FMT_BF16 ? elements * 2 : format == KVX_FMT_INT4 ? elements / 2 : elements;
+}
+__host__ __device__ inline uint32_t scale_bytes_of(uint32_t format, uint32_t kv_heads) {
+  return quantized(format) ? KVX_PAGE_TOKENS * kv_heads * 4 : 0;
+}
+
+// Where the four tensors of a layer start inside the layer's region of an
+// extent, in bytes: keys | key scales | values | value scales, each holding
+// every page of the extent (reference: abi/KvExtent.h:76-89).
+struct RegionOffsets {
+  uint64_t key_scales;
+  uint64_t values;
+  uint64_t value_scales;
+};
+__host__ __device__ inline RegionOffsets region_offsets(uint32_t extent_pages, uint32_t db,
+                                                        uint32_t sb) {
+  RegionOffsets r;
+  r.key_scales = uint64_t(extent_pages) * db;
+  r.values = uint64_t(extent_pages) * (uint64_t(db) + sb);
+  r.value_scales = uint64_t(extent_pages) * (2ull * db + sb);
+  return r;
+}
+
+// One KV head's slab of each tensor of a page in one layer.
+struct Slab {
+  uint8_t *keys;
+  uint8_t *values;
+  float *key_scales;
+  float *value_scales;
+};
+__device__ inline Slab slab_of(uint32_t format, uint32_t kv_heads, uint32_t head_dim,
+                               kvx_kv_layer kv, uint32_t head, uint64_t entry) {
+  const uint32_t index = uint32_t(entry) & KVX_PAGE_INDEX_MASK;
+  uint8_t *region = reinterpret_cast<uint8_t *>(entry - index) + kv.offset;
+  const uint32_t db = data_bytes_of(format, kv_heads, head_dim);
+  const uint32_t sb = scale_bytes_of(format, kv_heads);
+  const RegionOffsets r = region_offsets(kv.extent_pages, db, sb);
+  const uint32_t head_bytes = db / kv_heads;
+  Slab s;
+  s.keys = region + uint64_t(index) * db + head * head_bytes;
+  s.values = region + r.values + uint64_t(index) * db + head * head_bytes;
+  const uint64_t scale_index = (uint64_t(index) * kv_heads + head) * KVX_PAGE_TOKENS;
+  s.key_scales = reinterpret_cast<float *>(region + r.key_scales) + scale_index;
+  s.value_scales = reinterpret_cast<float *>(region + r.value_scales) + scale_index;
+  return s;
+}
+
+// ---- storage ----------------------------------------------------------------
+struct Storage {
+  kvx_layout layout;
+  uint32_t page_count = 0;
+  uint32_t extent_pages = 0;
+  uint32_t data_bytes = 0;
+  uint32_t scale_bytes = 0;
+  uint64_t budget_bytes = 0;
+  int device = 0;
+  std::vector<void *> extents;      // 16 KiB-aligned base; nullptr while not allocated
+  std::vector<void *> allocations;  // what hipMalloc returned for each extent
+  uint64_t extent_bytes() const;
+  uint64_t bytes_per_page() const;
+  uint32_t allocated_extents() const;
+};
+
+}  // namespace kvx
+
+struct kvx_storage : kvx::Storage {};

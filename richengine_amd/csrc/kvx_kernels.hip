@@ -1,0 +1,868 @@
+// Kernels of the paged-KV path that are bandwidth-trivial or format-generic:
+// quantize-on-append, the format-generic attention tile with its fixed-order
+// merge, tree-path compaction and whole-page copy, with their launchers.
+// The arithmetic of every kernel here keeps the operation order of the
+// reference kernels it replaces (cited per kernel), with products and sums
+// left unfused so the fp32 results do not depend on contraction.
+#include <algorithm>
+#include <vector>
+
+#include "kvx_device.h"
+
+namespace kvx {
+
+constexpr uint32_t kPage = KVX_PAGE_TOKENS;
+constexpr uint32_t kLanes = KVX_LANES_PER_LAUNCH;
+
+// ============================================================== append ====
+struct AppendLane {
+  const uint64_t *table;
+  uint32_t committed, tokens, stride, entries;
+  uint32_t group_base;  // first workgroup of this lane
+  uint32_t pad;
+};
+struct AppendArgs {
+  AppendLane lane[kLanes];
+  uint32_t n_lanes;
+  uint32_t kv_heads, head_dim;
+  uint32_t verify_max_rows;
+  kvx_kv_layer kv;
+  uint64_t lane_stride;
+};
+
+// The kernel-side contract of a store lane (reference:
+// common/paged_store_row.h:14-29; verify adds rows <= bound and stride == 32,
+// decode/paged_attention_store.metal:22-27).  A lane that fails writes nothing.
+__device__ inline bool append_contract(const AppendLane &l, const AppendArgs &a) {
+  const uint64_t required = (uint64_t(l.committed) + l.tokens + kPage - 1) / kPage;
+  bool ok = l.committed <= KVX_MAX_PHYSICAL_TOKENS && l.tokens > 0 &&
+            l.tokens <= KVX_PREFILL_TOKEN_BUDGET &&
+            uint64_t(l.committed) + l.tokens <= KVX_MAX_PHYSICAL_TOKENS &&
+            l.stride >= l.tokens && l.stride <= KVX_PREFILL_TOKEN_BUDGET &&
+            l.stride % kPage == 0 && l.entries >= required && a.kv.extent_pages > 0;
+  if (a.verify_max_rows)
+    ok = ok && l.tokens <= a.verify_max_rows && l.stride == KVX_VERIFY_CHUNK_STRIDE;
+  return ok;
+}
+
+// One workgroup stores one row (one tensor, one head, one token) of one lane:
+// head_dim threads, one per dimension (reference:
+// common/paged_store_row.h:47-147, paged_store_row_fp8.h:28-78).
+template <uint32_t FMT>
+__global__ __launch_bounds__(256) void append_kernel(const uint16_t *__restrict__ chunk_keys,
+                                                     const uint16_t *__restrict__ chunk_values,
+                                                     AppendArgs a) {
+  __shared__ float wave_max[4];
+  const uint32_t group = blockIdx.x;
+  uint32_t li = 0;
+  for (uint32_t i = 1; i < a.n_lanes; ++i)
+    if (group >= a.lane[i].group_base) li = i;
+  const AppendLane &l = a.lane[li];
+  if (!append_contract(l, a)) return;
+  const uint32_t D = a.head_dim, H = a.kv_heads;
+  const uint32_t local = group - l.group_base;
+  const uint32_t rows = l.tokens * H;
+  if (local >= 2 * rows) return;
+  const bool value_tensor = local >= rows;
+  const uint32_t row = value_tensor ? local - rows : local;
+  const uint32_t token = row % l.tokens, head = row / l.tokens;
+  const uint32_t d = threadIdx.x;
+  const uint32_t logical = l.committed + token;
+  const Slab s = slab_of(FMT, H, D, a.kv, head, l.table[logical / kPage]);
+  const uint32_t slot = logical % kPage;
+  const uint16_t source =
+      value_tensor ? chunk_values[li * a.lane_stride + (uint64_t(head) * D + d) * l.stride + token]
+                   : chunk_keys[li * a.lane_stride + (uint64_t(head) * l.stride + token) * D + d];
+  uint8_t *data = value_tensor ? s.values : s.keys;
+  // Element index inside the head's slab: keys token-major, values
+  // dimension-major (packed int4: both token-major).
+  const uint32_t element = (value_tensor && FMT != KVX_FMT_INT4) ? d * kPage + slot : slot * D + d;
+
+  if constexpr (FMT == KVX_FMT_BF16) {
+    reinterpret_cast<uint16_t *>(data)[element] = source;
+    return;
+  } else {
+    const float v = bf16_to_f32(source);
+    float m = fabsf(v);
+    for (int offset = 32; offset; offset >>= 1) m = fmaxf(m, __shfl_xor(m, offset));
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    float maximum = wave_max[0];
+    for (uint32_t w = 1; w < (D + 63) / 64; ++w) maximum = fmaxf(maximum, wave_max[w]);
+    constexpr float qmax = FMT == KVX_FMT_INT4 ? 7.0f : FMT == KVX_FMT_INT8 ? 127.0f : 448.0f;
+    const float scale = maximum == 0.0f ? 0.0f : __fdiv_rn(maximum, qmax);
+    if (d == 0) (value_tensor ? s.value_scales : s.key_scales)[slot] = scale;
+    const float scaled = maximum == 0.0f ? 0.0f : __fdiv_rn(__fmul_rn(v, qmax), maximum);
+    if constexpr (FMT == KVX_FMT_FP8E4M3) {
+      data[element] = maximum == 0.0f ? uint8_t(0) : uint8_t(f32_to_e4m3(scaled));
+    } else {
+      constexpr int limit = FMT == KVX_FMT_INT4 ? 7 : 127;
+      int code = int(rintf(scaled));
+      code = code < -limit ? -limit : code > limit ? limit : code;
+      if (maximum == 0.0f) code = 0;
+      if constexpr (FMT == KVX_FMT_INT8) {
+        reinterpret_cast<int8_t *>(data)[element] = int8_t(code);
+      } else {
+        // Even dimension in the low nibble; the even thread writes the byte.
+        const uint32_t nibble = uint32_t(code) & 0xfu;
+        const uint32_t partner = __shfl_xor(nibble, 1);
+        if ((d & 1) == 0) data[element >> 1] = uint8_t(nibble | (partner << 4));
+      }
+    }
+  }
+}
+
+// ===================================================== generic attention ====
+// One tile = row_capacity query rows x `group` query heads of one KV head
+// (M fused rows) over the pages of one split.
+struct AttendLane {
+  const uint64_t *table;
+  uint32_t committed, entries, split_count, active_rows;
+  uint64_t row_base;   // first fused row of this lane's slots in the workspace
+  uint64_t q_offset;   // element offset of the lane's queries / output
+  uint32_t mask_offset;
+  float score_scale;
+};
+struct AttendArgs {
+  AttendLane lane[kLanes];
+  uint32_t n_lanes;
+  uint32_t kv_heads, group, head_dim;
+  uint32_t row_capacity;
+  uint32_t row_stride;  // rows between KV heads in queries / output
+  kvx_kv_layer kv;
+};
+struct PrefillArgs {
+  const uint64_t *table;
+  uint32_t committed, rows, stride, entries, splits;
+  uint32_t kv_heads, group, head_dim;
+  float score_scale;
+  kvx_kv_layer kv;
+};
+
+__device__ inline bool attend_contract(const AttendLane &l, const AttendArgs &a) {
+  return l.active_rows > 0 && l.active_rows <= a.row_capacity &&
+         l.entries >= (uint64_t(l.committed) + l.active_rows + kPage - 1) / kPage &&
+         a.kv.extent_pages > 0 &&
+         uint64_t(l.committed) + l.active_rows <= uint64_t(KVX_MAX_PHYSICAL_TOKENS) &&
+         l.split_count > 0 && l.split_count <= KVX_VERIFY_MAX_SPLITS;
+}
+__device__ inline bool prefill_contract(const PrefillArgs &p) {
+  return p.rows > 0 && p.rows <= KVX_PREFILL_TOKEN_BUDGET && p.stride >= p.rows &&
+         p.stride <= KVX_PREFILL_TOKEN_BUDGET && p.stride % kPage == 0 &&
+         p.entries >= (uint64_t(p.committed) + p.rows + kPage - 1) / kPage &&
+         p.kv.extent_pages > 0 && p.splits > 0 && p.splits <= KVX_PREFILL_MAX_SPLITS &&
+         uint64_t(p.committed) + p.rows <= uint64_t(KVX_MAX_PHYSICAL_TOKENS);
+}
+
+constexpr uint32_t kTileThreads = 256;
+constexpr uint32_t kMaxD = 256;
+constexpr uint32_t kKeyPitch = kMaxD + 2;  // bf16 elements; odd word pitch avoids bank conflicts
+
+// The page loop of one tile over one split (reference:
+// common/paged_attention_tile.h:85-349; fp8: paged_attention_fp8_tile.h:34-265).
+// MAXM bounds the fused rows a thread accumulates in registers.
+// K and V codes are staged in LDS as bf16, which holds every int4 / int8 /
+// e4m3 / bf16 code exactly.
+template <uint32_t FMT, uint32_t MAXM>
+__device__ void attention_tile(const uint16_t *__restrict__ tile_queries,
+                               const uint64_t *__restrict__ table, kvx_kv_layer kv,
+                               uint32_t H, uint32_t G, uint32_t D, uint32_t row_capacity,
+                               uint32_t head, uint32_t committed, uint32_t active_rows,
+                               uint32_t splits, uint32_t split, float *__restrict__ partials,
+                               float *__restrict__ statistics, uint64_t slot_row,
+                               const uint32_t *__restrict__ row_masks, float score_scale_in) {
+  __shared__ uint16_t k_lds[kPage * kKeyPitch];
+  __shared__ uint16_t v_lds[kPage * kMaxD];
+  __shared__ float w_lds[MAXM * (kPage + 1)];
+  __shared__ float rescale_lds[MAXM];
+  __shared__ uint32_t admit_lds[MAXM];
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t M = row_capacity * G;
+  const uint32_t visible = committed + active_rows;
+  const uint32_t pages = (visible + kPage - 1) / kPage;
+  const uint32_t per = (pages + splits - 1) / splits;
+  const uint32_t begin = split * per;
+  if (begin >= pages) return;
+  const uint32_t end = min(pages, begin + per);
+  constexpr bool kFp8 = FMT == KVX_FMT_FP8E4M3;
+  constexpr bool kQuant = FMT != KVX_FMT_BF16;
+  const float score_scale = default_score_scale(D, score_scale_in);
+
+  float acc[MAXM];
+#pragma unroll
+  for (uint32_t r = 0; r < MAXM; ++r) acc[r] = 0.0f;
+  // Thread r (< M) owns the running statistics of fused row r.
+  float row_max = -INFINITY, row_sum = 0.0f;
+  const uint32_t my_query_row = tid / G;
+  const bool owns_row = tid < M && my_query_row < active_rows;
+  uint32_t my_limit = 0, my_mask = 0;
+  if (owns_row) {
+    const uint32_t causal_end = committed + min(my_query_row, active_rows - 1) + 1;
+    my_limit = min(visible, causal_end);
+    my_mask = row_masks ? row_masks[my_query_row] : 0u;
+  }
+
+  for (uint32_t page = begin; page < end; ++page) {
+    const Slab s = slab_of(FMT, H, D, kv, head, table[page]);
+    const uint32_t token_start = page * kPage;
+    __syncthreads();  // the previous page's PV is done with the staging
+    for (uint32_t e = tid; e < kPage * D; e += kTileThreads) {
+      const uint32_t j = e / D, d = e % D;
+      k_lds[j * kKeyPitch + d] = f32_to_bf16(load_key_code<FMT>(s.keys, D, j, d));
+      v_lds[j * kMaxD + d] = f32_to_bf16(load_value_code<FMT>(s.values, D, j, d));
+    }
+    if (tid < M) {
+      uint32_t admit = 0;
+      if (owns_row) {
+        for (uint32_t j = 0; j < kPage; ++j) {
+          const uint32_t t = token_start + j;
+          const bool in = !row_masks ? t < my_limit
+                                     : (t < committed) ||
+                                           (t < visible && ((my_mask >> (t - committed)) & 1u));
+          admit |= uint32_t(in) << j;
+        }
+      }
+      admit_lds[tid] = admit;
+    }
+    __syncthreads();
+
+    // Scores: thread (token j, row group) walks the fused rows r = rg, rg+8, ...
+    {
+      const uint32_t j = tid & 31, rg = tid >> 5;
+      const float key_scale = kQuant ? s.key_scales[j] : 1.0f;
+      for (uint32_t r = rg; r < M; r += 8) {
+        float score = -INFINITY;
+        if ((admit_lds[r] >> j) & 1u) {
+          const uint16_t *q = tile_queries + uint64_t(r) * D;
+          float dot = 0.0f;
+          for (uint32_t d = 0; d < D; ++d) {
+            float qv = bf16_to_f32(q[d]);
+            if constexpr (kFp8) qv = round_f16(qv);  // the fp8 tile stages queries as fp16
+            dot = __fadd_rn(dot, __fmul_rn(qv, bf16_to_f32(k_lds[j * kKeyPitch + d])));
+          }
+          if constexpr (kQuant) dot = __fmul_rn(dot, key_scale);
+          score = __fmul_rn(dot, score_scale);
+        }
+        w_lds[r * (kPage + 1) + j] = score;
+      }
+    }
+    __syncthreads();
+
+    // Online softmax of one page, one thread per fused row, in the reference's
+    // order: four groups of eight tokens summed, then paired.
+    if (tid < M) {
+      float rescale = 1.0f;
+      if (owns_row) {
+        const uint32_t admit = admit_lds[tid];
+        float *w = w_lds + tid * (kPage + 1);
+        float local_max = -INFINITY;
+        for (uint32_t j = 0; j < kPage; ++j) local_max = fmaxf(local_max, w[j]);
+        const float next_max = fmaxf(row_max, local_max);
+        float lane_sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (uint32_t j = 0; j < kPage; ++j) {
+          const bool in = (admit >> j) & 1u;
+          const float p = in ? expf(__fsub_rn(w[j], next_max)) : 0.0f;
+          lane_sum[j >> 3] = __fadd_rn(lane_sum[j >> 3], p);
+          float weight = 0.0f;
+          if (in && w[j] > -INFINITY)
+            weight = kQuant ? __fmul_rn(p, s.value_scales[j]) : p;
+          w[j] = kFp8 ? round_f16(weight) : round_bf16(weight);
+        }
+        const float local_sum =
+            __fadd_rn(__fadd_rn(lane_sum[0], lane_sum[1]), __fadd_rn(lane_sum[2], lane_sum[3]));
+        rescale = (next_max == -INFINITY || next_max == row_max)
+                      ? 1.0f
+                      : expf(__fsub_rn(row_max, next_max));
+        row_sum = __fadd_rn(__fmul_rn(row_sum, rescale), local_sum);
+        row_max = next_max;
+      }
+      rescale_lds[tid] = rescale;
+    }
+    __syncthreads();
+
+    // PV: thread d accumulates dimension d of every fused row.
+    if (tid < D) {
+#pragma unroll
+      for (uint32_t r = 0; r < MAXM; ++r) {
+        if (r < M) {
+          const uint32_t admit = admit_lds[r];
+          if (r / G < active_rows) {
+            float sum = 0.0f;
+            for (uint32_t j = 0; j < kPage; ++j)
+              if ((admit >> j) & 1u)
+                sum = __fadd_rn(sum, __fmul_rn(w_lds[r * (kPage + 1) + j],
+                                               bf16_to_f32(v_lds[j * kMaxD + tid])));
+            const float scale = rescale_lds[r];
+            acc[r] = __fadd_rn(scale != 1.0f ? __fmul_rn(acc[r], scale) : acc[r], sum);
+          }
+        }
+      }
+    }
+  }
+
+  if (tid < D) {
+#pragma unroll
+    for (uint32_t r = 0; r < MAXM; ++r)
+      if (r < M && r / G < active_rows) partials[(slot_row + r) * D + tid] = acc[r];
+  }
+  if (owns_row) {
+    statistics[(slot_row + tid) * 2] = row_max;
+    statistics[(slot_row + tid) * 2 + 1] = row_sum;
+  }
+}
+
+template <uint32_t FMT, uint32_t MAXM>
+__global__ __launch_bounds__(kTileThreads) void attend_split_kernel(
+    const uint16_t *__restrict__ queries, float *__restrict__ partials,
+    float *__restrict__ statistics, const uint32_t *__restrict__ row_masks, AttendArgs a) {
+  const uint32_t split = blockIdx.x, head = blockIdx.y, li = blockIdx.z;
+  const AttendLane &l = a.lane[li];
+  if (!attend_contract(l, a) || split >= l.split_count) return;
+  const uint32_t M = a.row_capacity * a.group;
+  const uint16_t *tile_q =
+      queries + l.q_offset + uint64_t(head) * a.row_stride * a.group * a.head_dim;
+  const uint64_t slot_row = l.row_base + (uint64_t(head) * l.split_count + split) * M;
+  attention_tile<FMT, MAXM>(tile_q, l.table, a.kv, a.kv_heads, a.group, a.head_dim,
+                            a.row_capacity, head, l.committed, l.active_rows, l.split_count,
+                            split, partials, statistics, slot_row,
+                            row_masks ? row_masks + l.mask_offset : nullptr, l.score_scale);
+}
+
+// Prefill: KV heads, query tiles of eight rows, history splits (reference:
+// prefill/paged_attention.metal:7-67); slots are [tile][head][split].
+template <uint32_t FMT, uint32_t MAXM>
+__global__ __launch_bounds__(kTileThreads) void prefill_split_kernel(
+    const uint16_t *__restrict__ queries, float *__restrict__ partials,
+    float *__restrict__ statistics, PrefillArgs p) {
+  const uint32_t split = blockIdx.x, head = blockIdx.y, tile = blockIdx.z;
+  const uint32_t tile_start = tile * KVX_PREFILL_TILE_ROWS;
+  if (!prefill_contract(p) || tile_start >= p.rows) return;
+  const uint32_t active = min(KVX_PREFILL_TILE_ROWS, p.rows - tile_start);
+  const uint32_t M = KVX_PREFILL_TILE_ROWS * p.group;
+  const uint64_t tile_offset = (uint64_t(head) * p.stride + tile_start) * p.group * p.head_dim;
+  const uint64_t slot_row = ((uint64_t(tile) * p.kv_heads + head) * p.splits + split) * M;
+  attention_tile<FMT, MAXM>(queries + tile_offset, p.table, p.kv, p.kv_heads, p.group, p.head_dim,
+                            KVX_PREFILL_TILE_ROWS, head, p.committed + tile_start, active, p.splits,
+                            split, partials, statistics, slot_row, nullptr, p.score_scale);
+}
+
+// Fixed-order merge of one fused row's splits (reference:
+// common/paged_attention_tile.h:362-417).  head_dim threads, one per dimension.
+__device__ void reduce_row(const float *__restrict__ partials, const float *__restrict__ statistics,
+                           uint16_t *__restrict__ out_row, uint32_t G, uint32_t D, uint32_t M,
+                           uint32_t committed, uint32_t active_rows, uint32_t splits,
+                           uint64_t head_row, uint32_t fused_row) {
+  const uint32_t d = threadIdx.x;
+  if (fused_row / G >= active_rows) {
+    out_row[d] = 0;
+    return;
+  }
+  const uint32_t pages = (committed + active_rows + kPage - 1) / kPage;
+  const uint32_t per = (pages + splits - 1) / splits;
+  const uint32_t written = (pages + per - 1) / per;
+  float maximum = -INFINITY;
+  for (uint32_t s = 0; s < written; ++s)
+    maximum = fmaxf(maximum, statistics[(head_row + uint64_t(s) * M + fused_row) * 2]);
+  float numerator = 0.0f, denominator = 0.0f;
+  for (uint32_t s = 0; s < written; ++s) {  // split order is part of the contract
+    const uint64_t row = head_row + uint64_t(s) * M + fused_row;
+    const float weight = expf(__fsub_rn(statistics[row * 2], maximum));
+    numerator = __fadd_rn(numerator, __fmul_rn(weight, partials[row * D + d]));
+    denominator = __fadd_rn(denominator, __fmul_rn(weight, statistics[row * 2 + 1]));
+  }
+  out_row[d] = f32_to_bf16(denominator > 0.0f ? __fdiv_rn(numerator, denominator) : 0.0f);
+}
+
+__global__ __launch_bounds__(256) void attend_reduce_kernel(const float *__restrict__ partials,
+                                                            const float *__restrict__ statistics,
+                                                            uint16_t *__restrict__ output,
+                                                            AttendArgs a) {
+  const uint32_t fused_row = blockIdx.x, head = blockIdx.y, li = blockIdx.z;
+  const AttendLane &l = a.lane[li];
+  if (!attend_contract(l, a)) return;
+  const uint32_t M = a.row_capacity * a.group, D = a.head_dim;
+  uint16_t *out = output + l.q_offset + uint64_t(head) * a.row_stride * a.group * D +
+                  uint64_t(fused_row) * D;
+  reduce_row(partials, statistics, out, a.group, D, M, l.committed, l.active_rows, l.split_count,
+             l.row_base + uint64_t(head) * l.split_count * M, fused_row);
+}
+
+__global__ __launch_bounds__(256) void prefill_reduce_kernel(const float *__restrict__ partials,
+                                                             const float *__restrict__ statistics,
+                                                             uint16_t *__restrict__ output,
+                                                             PrefillArgs p) {
+  const uint32_t fused_row = blockIdx.x, head = blockIdx.y, tile = blockIdx.z;
+  const uint32_t tile_start = tile * KVX_PREFILL_TILE_ROWS;
+  if (!prefill_contract(p) || tile_start >= p.rows) return;
+  const uint32_t active = min(KVX_PREFILL_TILE_ROWS, p.rows - tile_start);
+  const uint32_t M = KVX_PREFILL_TILE_ROWS * p.group, D = p.head_dim;
+  const uint64_t tile_offset = (uint64_t(head) * p.stride + tile_start) * p.group * D;
+  reduce_row(partials, statistics, output + tile_offset + uint64_t(fused_row) * D, p.group, D, M,
+             p.committed + tile_start, active, p.splits,
+             (uint64_t(tile) * p.kv_heads + head) * p.splits * M, fused_row);
+}
+
+// =========================================================== compaction ====
+struct CompactLane {
+  const uint64_t *table;
+  uint32_t committed, tokens, entries, pad;
+};
+struct CompactArgs {
+  CompactLane lane[kLanes];
+  uint32_t n_lanes, kv_heads, head_dim, format;
+  uint32_t first_layer, path_stride;
+  uint32_t extent_pages, data_bytes, scale_bytes;
+};
+
+// Forward-order copy of the retained path's rows to their path slots, one
+// workgroup per (head, lane, layer) (reference:
+// decode/paged_attention_store.metal:198-278).  All loads of a row complete
+// before its stores.  A lane whose path is not a strictly increasing list of
+// stored rows, or whose slots fall outside its table, moves nothing.
+__global__ __launch_bounds__(256) void compact_kernel(const uint32_t *__restrict__ retained_path,
+                                                      const uint32_t *__restrict__ retained_count,
+                                                      uint32_t lane_first, CompactArgs a) {
+  const uint32_t head = blockIdx.x, li = blockIdx.y, layer = a.first_layer + blockIdx.z;
+  const CompactLane &l = a.lane[li];
+  const uint32_t lane = lane_first + li;
+  const uint32_t count = retained_count[lane];
+  const uint32_t *path = retained_path + uint64_t(lane) * a.path_stride;
+  if (count == 0 || count > a.path_stride || count > l.tokens) return;
+  if (l.entries < (uint64_t(l.committed) + l.tokens + kPage - 1) / kPage) return;
+  for (uint32_t i = 0; i < count; ++i)
+    if (path[i] >= l.tokens || path[i] < i || (i && path[i] <= path[i - 1])) return;
+  const uint32_t D = a.head_dim, H = a.kv_heads, F = a.format;
+  kvx_kv_layer kv;
+  kv.extent_pages = a.extent_pages;
+  kv.offset = uint32_t(uint64_t(layer) * a.extent_pages * 2 * (uint64_t(a.data_bytes) + a.scale_bytes));
+  const uint32_t d = threadIdx.x;
+  const uint32_t element_bytes = F == KVX_FMT_BF16 ? 2 : 1;
+  const uint32_t row_units = F == KVX_FMT_INT4 ? D / 2 : D;  // elements (bytes for int4) per row
+  for (uint32_t i = 0; i < count; ++i) {
+    const uint32_t src_row = path[i];
+    if (src_row == i) continue;
+    const uint32_t src_token = l.committed + src_row, dst_token = l.committed + i;
+    const Slab src = slab_of(F, H, D, kv, head, l.table[src_token / kPage]);
+    const Slab dst = slab_of(F, H, D, kv, head, l.table[dst_token / kPage]);
+    const uint32_t so = src_token % kPage, dof = dst_token % kPage;
+    uint16_t key = 0, value = 0;
+    float key_scale = 0.0f, value_scale = 0.0f;
+    const bool active = d < row_units;
+    if (active) {
+      const uint32_t ks = so * row_units + d;
+      const uint32_t vs = F == KVX_FMT_INT4 ? ks : d * kPage + so;
+      if (element_bytes == 2) {
+        key = reinterpret_cast<const uint16_t *>(src.keys)[ks];
+        value = reinterpret_cast<const uint16_t *>(src.values)[vs];
+      } else {
+        key = src.keys[ks];
+        value = src.values[vs];
+      }
+    }
+    if (d == 0 && F != KVX_FMT_BF16) {
+      key_scale = src.key_scales[so];
+      value_scale = src.value_scales[so];
+    }
+    __syncthreads();
+    if (active) {
+      const uint32_t kd = dof * row_units + d;
+      const uint32_t vd = F == KVX_FMT_INT4 ? kd : d * kPage + dof;
+      if (element_bytes == 2) {
+        reinterpret_cast<uint16_t *>(dst.keys)[kd] = key;
+        reinterpret_cast<uint16_t *>(dst.values)[vd] = value;
+      } else {
+        dst.keys[kd] = uint8_t(key);
+        dst.values[vd] = uint8_t(value);
+      }
+    }
+    if (d == 0 && F != KVX_FMT_BF16) {
+      dst.key_scales[dof] = key_scale;
+      dst.value_scales[dof] = value_scale;
+    }
+    __threadfence_block();
+    __syncthreads();
+  }
+}
+
+// ============================================================ page copy ====
+constexpr uint32_t kCopiesPerLaunch = 128;
+constexpr uint32_t kCopyChunk = 16384;
+struct CopyArgs {
+  uint64_t from[kCopiesPerLaunch];
+  uint64_t to[kCopiesPerLaunch];
+  uint32_t extent_pages, data_bytes, scale_bytes, layers;
+};
+
+// Every tensor of every layer of each page, 16 bytes per thread per step
+// (reference: runtime/ops/PageStorage.mm:95-167 copies the same spans on the
+// host).  blockIdx = (chunk of the span, layer * 4 + tensor, copy).
+__global__ __launch_bounds__(256) void page_copy_kernel(CopyArgs a) {
+  const uint32_t tensor = blockIdx.y & 3, layer = blockIdx.y >> 2;
+  const uint32_t bytes = (tensor & 1) ? a.scale_bytes : a.data_bytes;
+  const uint32_t begin = blockIdx.x * kCopyChunk;
+  if (begin >= bytes) return;
+  const uint32_t end = min(bytes, begin + kCopyChunk);
+  const uint64_t from = a.from[blockIdx.z], to = a.to[blockIdx.z];
+  const uint32_t fi = uint32_t(from) & KVX_PAGE_INDEX_MASK, ti = uint32_t(to) & KVX_PAGE_INDEX_MASK;
+  const RegionOffsets r = region_offsets(a.extent_pages, a.data_bytes, a.scale_bytes);
+  const uint64_t region = uint64_t(layer) * a.extent_pages * 2 * (uint64_t(a.data_bytes) + a.scale_bytes);
+  const uint64_t start = tensor == 0 ? 0 : tensor == 1 ? r.key_scales : tensor == 2 ? r.values : r.value_scales;
+  const uint8_t *src = reinterpret_cast<const uint8_t *>(from - fi) + region + start + uint64_t(fi) * bytes;
+  uint8_t *dst = reinterpret_cast<uint8_t *>(to - ti) + region + start + uint64_t(ti) * bytes;
+  for (uint32_t o = begin + threadIdx.x * 16; o < end; o += 256 * 16)
+    *reinterpret_cast<uint4 *>(dst + o) = *reinterpret_cast<const uint4 *>(src + o);
+}
+
+// ============================================================= launchers ====
+namespace {
+
+template <class F>
+int dispatch_format(uint32_t format, F &&f) {
+  switch (format) {
+  case KVX_FMT_INT8: return f(std::integral_constant<uint32_t, KVX_FMT_INT8>{});
+  case KVX_FMT_BF16: return f(std::integral_constant<uint32_t, KVX_FMT_BF16>{});
+  case KVX_FMT_INT4: return f(std::integral_constant<uint32_t, KVX_FMT_INT4>{});
+  case KVX_FMT_FP8E4M3: return f(std::integral_constant<uint32_t, KVX_FMT_FP8E4M3>{});
+  }
+  return fail(KVX_EINVAL, "invalid KV format");
+}
+
+template <class F>
+int dispatch_rows(uint32_t M, F &&f) {
+  if (M <= 8) return f(std::integral_constant<uint32_t, 8>{});
+  if (M <= 48) return f(std::integral_constant<uint32_t, 48>{});
+  if (M <= 64) return f(std::integral_constant<uint32_t, 64>{});
+  if (M <= 96) return f(std::integral_constant<uint32_t, 96>{});
+  if (M <= 128) return f(std::integral_constant<uint32_t, 128>{});
+  return fail(KVX_EINVAL, "tile holds more than 128 fused rows");
+}
+
+int check_launch(const char *what) {
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? KVX_OK : hip_fail(e, what);
+}
+
+}  // namespace
+}  // namespace kvx
+
+using namespace kvx;
+
+// Implemented by the int4 decode kernels; declines (returns 1) shapes it does
+// not cover so the generic tile takes them.
+int kvx_decode_int4_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t query_heads,
+                           const void *queries, void *output, const uint64_t *const *page_tables,
+                           const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                           void *workspace, uint64_t workspace_bytes, hipStream_t stream);
+
+extern "C" {
+
+int kv_append(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
+              const void *chunk_values, const uint64_t *const *page_tables,
+              const kvx_chunk_params *lanes, uint32_t n_lanes, uint64_t lane_stride,
+              uint32_t verify_max_rows, void *stream) {
+  if (!s || !chunk_keys || !chunk_values || !page_tables || !lanes || !n_lanes)
+    return fail(KVX_EINVAL, "kv_append: null argument or no lanes");
+  kvx_kv_layer kv;
+  if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
+  if (verify_max_rows > KVX_TREE_NODES)
+    return fail(KVX_EINVAL, "verify stores hold at most 16 rows per lane");
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    static const char *const names[] = {"", "chunk_tokens_out_of_range", "context_out_of_range",
+                                        "chunk_stride_invalid", "page_table_too_short"};
+    if (const int e = kvx_chunk_validation(&lanes[i])) return fail(KVX_EINVAL, names[e]);
+    if (verify_max_rows && (lanes[i].chunk_tokens > verify_max_rows ||
+                            lanes[i].chunk_stride != KVX_VERIFY_CHUNK_STRIDE))
+      return fail(KVX_EINVAL, "verify store rows or stride are out of range");
+    if (!page_tables[i]) return fail(KVX_EINVAL, "kv_append: null page table");
+  }
+  const uint32_t H = s->layout.kv_heads, D = s->layout.head_dim;
+  for (uint32_t first = 0; first < n_lanes; first += kLanes) {
+    AppendArgs a{};
+    a.n_lanes = std::min(kLanes, n_lanes - first);
+    a.kv_heads = H;
+    a.head_dim = D;
+    a.verify_max_rows = verify_max_rows;
+    a.kv = kv;
+    a.lane_stride = lane_stride;
+    uint32_t groups = 0;
+    for (uint32_t i = 0; i < a.n_lanes; ++i) {
+      const kvx_chunk_params &p = lanes[first + i];
+      a.lane[i] = {page_tables[first + i], p.committed_tokens, p.chunk_tokens, p.chunk_stride,
+                   p.page_table_entries, groups, 0};
+      groups += 2 * p.chunk_tokens * H;
+    }
+    const auto *keys = static_cast<const uint16_t *>(chunk_keys) + uint64_t(first) * lane_stride;
+    const auto *values = static_cast<const uint16_t *>(chunk_values) + uint64_t(first) * lane_stride;
+    const int rc = dispatch_format(s->layout.format, [&](auto fmt) {
+      hipLaunchKernelGGL((append_kernel<decltype(fmt)::value>), dim3(groups), dim3(D), 0,
+                         static_cast<hipStream_t>(stream), keys, values, a);
+      return check_launch("append_kernel");
+    });
+    if (rc) return rc;
+  }
+  return KVX_OK;
+}
+
+static int validate_attend(const kvx_storage *s, uint32_t query_heads,
+                           const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                           const uint64_t *const *page_tables, uint64_t workspace_bytes) {
+  const kvx_layout &l = s->layout;
+  if (!query_heads || query_heads % l.kv_heads)
+    return fail(KVX_EINVAL, "query heads are not a multiple of the KV heads");
+  const uint32_t capacity = lanes[0].row_capacity;
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    const kvx_verify_params &p = lanes[i];
+    if (p.row_capacity != capacity || !capacity || capacity > row_stride)
+      return fail(KVX_EINVAL, "verify lanes must share one row capacity within the row stride");
+    if (!p.active_rows || p.active_rows > capacity)
+      return fail(KVX_EINVAL, "verify active rows are out of range");
+    if (uint64_t(p.committed_tokens) + p.active_rows > KVX_MAX_PHYSICAL_TOKENS)
+      return fail(KVX_EINVAL, "verify attention history exceeds physical context");
+    if (p.page_table_entries < (uint64_t(p.committed_tokens) + p.active_rows + 31) / 32)
+      return fail(KVX_EINVAL, "page_table_too_short");
+    if (!p.split_count || p.split_count > KVX_VERIFY_MAX_SPLITS)
+      return fail(KVX_EINVAL, "verify split count is out of range");
+    if (!page_tables[i]) return fail(KVX_EINVAL, "null page table");
+  }
+  if (capacity * (query_heads / l.kv_heads) > 128)
+    return fail(KVX_EINVAL, "tile holds more than 128 fused rows");
+  if (workspace_bytes < kvx_attend_workspace_bytes(lanes, n_lanes, query_heads, &l))
+    return fail(KVX_EINVAL, "verify attention scratch is smaller than its bound");
+  return KVX_OK;
+}
+
+static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_heads,
+                          const void *queries, void *output, const uint64_t *const *page_tables,
+                          const kvx_verify_params *lanes, uint32_t n_lanes,
+                          const uint32_t *row_masks, uint32_t row_stride, void *workspace,
+                          hipStream_t stream) {
+  const kvx_layout &l = s->layout;
+  const uint32_t H = l.kv_heads, G = query_heads / H, D = l.head_dim;
+  const uint32_t capacity = lanes[0].row_capacity, M = capacity * G;
+  uint64_t total_rows = 0;
+  for (uint32_t i = 0; i < n_lanes; ++i) total_rows += uint64_t(lanes[i].split_count) * H * M;
+  float *partials = static_cast<float *>(workspace);
+  float *statistics = reinterpret_cast<float *>(
+      static_cast<uint8_t *>(workspace) + (total_rows * D * sizeof(float) + 255) / 256 * 256);
+  uint64_t row_base = 0;
+  for (uint32_t first = 0; first < n_lanes; first += kLanes) {
+    AttendArgs a{};
+    a.n_lanes = std::min(kLanes, n_lanes - first);
+    a.kv_heads = H;
+    a.group = G;
+    a.head_dim = D;
+    a.row_capacity = capacity;
+    a.row_stride = row_stride;
+    a.kv = kv;
+    uint32_t max_splits = 0;
+    for (uint32_t i = 0; i < a.n_lanes; ++i) {
+      const kvx_verify_params &p = lanes[first + i];
+      AttendLane &al = a.lane[i];
+      al.table = page_tables[first + i];
+      al.committed = p.committed_tokens;
+      al.entries = p.page_table_entries;
+      al.split_count = p.split_count;
+      al.active_rows = p.active_rows;
+      al.row_base = row_base;
+      al.q_offset = uint64_t(first + i) * H * row_stride * G * D;
+      al.mask_offset = (first + i) * capacity;
+      al.score_scale = p.score_scale != 0.0f ? p.score_scale : l.score_scale;
+      row_base += uint64_t(p.split_count) * H * M;
+      max_splits = std::max(max_splits, p.split_count);
+    }
+    int rc = dispatch_format(l.format, [&](auto fmt) {
+      return dispatch_rows(M, [&](auto maxm) {
+        hipLaunchKernelGGL((attend_split_kernel<decltype(fmt)::value, decltype(maxm)::value>),
+                           dim3(max_splits, H, a.n_lanes), dim3(kTileThreads), 0, stream,
+                           static_cast<const uint16_t *>(queries), partials, statistics, row_masks,
+                           a);
+        return check_launch("attend_split_kernel");
+      });
+    });
+    if (rc) return rc;
+    hipLaunchKernelGGL(attend_reduce_kernel, dim3(M, H, a.n_lanes), dim3(D), 0, stream, partials,
+                       statistics, static_cast<uint16_t *>(output), a);
+    if ((rc = check_launch("attend_reduce_kernel"))) return rc;
+  }
+  return KVX_OK;
+}
+
+int kv_attend_verify(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
+                     const void *queries, void *output, const uint64_t *const *page_tables,
+                     const kvx_verify_params *lanes, uint32_t n_lanes, const uint32_t *row_masks,
+                     uint32_t row_stride, void *workspace, uint64_t workspace_bytes, void *stream) {
+  if (!s || !queries || !output || !page_tables || !lanes || !n_lanes || !workspace)
+    return fail(KVX_EINVAL, "kv_attend_verify: null argument or no lanes");
+  if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
+  kvx_kv_layer kv;
+  if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
+  if (row_masks && s->layout.format == KVX_FMT_FP8E4M3)
+    return fail(KVX_EINVAL, "tree verify has no fp8 kernels");
+  if (int rc = validate_attend(s, query_heads, lanes, n_lanes, row_stride, page_tables,
+                               workspace_bytes))
+    return rc;
+  return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks,
+                        row_stride, workspace, static_cast<hipStream_t>(stream));
+}
+
+int kv_attend_decode(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
+                     const void *queries, void *output, const uint64_t *const *page_tables,
+                     const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                     void *workspace, uint64_t workspace_bytes, void *stream) {
+  if (!s || !queries || !output || !page_tables || !lanes || !n_lanes || !workspace)
+    return fail(KVX_EINVAL, "kv_attend_decode: null argument or no lanes");
+  if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
+  kvx_kv_layer kv;
+  if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
+  for (uint32_t i = 0; i < n_lanes; ++i)
+    if (lanes[i].active_rows != 1 || lanes[i].row_capacity != 1)
+      return fail(KVX_EINVAL, "decode attends exactly one row per lane");
+  if (int rc = validate_attend(s, query_heads, lanes, n_lanes, row_stride, page_tables,
+                               workspace_bytes))
+    return rc;
+  const int fast = kvx_decode_int4_launch(s, kv, query_heads, queries, output, page_tables, lanes,
+                                          n_lanes, row_stride, workspace, workspace_bytes,
+                                          static_cast<hipStream_t>(stream));
+  if (fast <= 0) return fast;
+  return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, nullptr,
+                        row_stride, workspace, static_cast<hipStream_t>(stream));
+}
+
+int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
+                      const void *queries, void *output, const uint64_t *page_table,
+                      const kvx_prefill_params *params, void *workspace, uint64_t workspace_bytes,
+                      void *stream) {
+  if (!s || !queries || !output || !page_table || !params || !workspace)
+    return fail(KVX_EINVAL, "kv_attend_prefill: null argument");
+  if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
+  const kvx_layout &l = s->layout;
+  kvx_kv_layer kv;
+  if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
+  if (!query_heads || query_heads % l.kv_heads)
+    return fail(KVX_EINVAL, "query heads are not a multiple of the KV heads");
+  const kvx_chunk_params chunk{params->committed_tokens, params->rows, params->chunk_stride,
+                               params->page_table_entries, {}};
+  static const char *const names[] = {"", "chunk_tokens_out_of_range", "context_out_of_range",
+                                      "chunk_stride_invalid", "page_table_too_short"};
+  if (const int e = kvx_chunk_validation(&chunk)) return fail(KVX_EINVAL, names[e]);
+  if (!params->split_count || params->split_count > KVX_PREFILL_MAX_SPLITS)
+    return fail(KVX_EINVAL, "prefill split count is out of range");
+  const uint32_t H = l.kv_heads, G = query_heads / H, D = l.head_dim;
+  const uint32_t tiles = (params->rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+  const uint32_t M = KVX_PREFILL_TILE_ROWS * G;
+  if (M > 128) return fail(KVX_EINVAL, "tile holds more than 128 fused rows");
+  const uint64_t rows = uint64_t(tiles) * H * params->split_count * M;
+  const uint64_t partial_bytes = rows * D * sizeof(float);
+  if (workspace_bytes < partial_bytes + rows * 2 * sizeof(float))
+    return fail(KVX_EINVAL, "prefill attention scratch is smaller than its bound");
+  float *partials = static_cast<float *>(workspace);
+  float *statistics = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + partial_bytes);
+  PrefillArgs p{page_table, params->committed_tokens, params->rows, params->chunk_stride,
+                params->page_table_entries, params->split_count, H, G, D,
+                params->score_scale != 0.0f ? params->score_scale : l.score_scale, kv};
+  auto st = static_cast<hipStream_t>(stream);
+  int rc = dispatch_format(l.format, [&](auto fmt) {
+    return dispatch_rows(M, [&](auto maxm) {
+      hipLaunchKernelGGL((prefill_split_kernel<decltype(fmt)::value, decltype(maxm)::value>),
+                         dim3(params->split_count, H, tiles), dim3(kTileThreads), 0, st,
+                         static_cast<const uint16_t *>(queries), partials, statistics, p);
+      return check_launch("prefill_split_kernel");
+    });
+  });
+  if (rc) return rc;
+  hipLaunchKernelGGL(prefill_reduce_kernel, dim3(M, H, tiles), dim3(D), 0, st, partials, statistics,
+                     static_cast<uint16_t *>(output), p);
+  return check_launch("prefill_reduce_kernel");
+}
+
+int kv_compact_path(const kvx_storage *s, uint32_t layer, const uint64_t *const *page_tables,
+                    const kvx_chunk_params *lanes, uint32_t n_lanes,
+                    const uint32_t *retained_path, const uint32_t *retained_count,
+                    uint32_t path_stride, void *stream) {
+  if (!s || !page_tables || !lanes || !n_lanes || !retained_path || !retained_count)
+    return fail(KVX_EINVAL, "kv_compact_path: null argument or no lanes");
+  const kvx_layout &l = s->layout;
+  if (layer != UINT32_MAX && layer >= l.layers)
+    return fail(KVX_ERANGE, "KV layer is outside the layout");
+  if (!path_stride || path_stride > KVX_TREE_NODES)
+    return fail(KVX_EINVAL, "retained path stride is out of range");
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    static const char *const names[] = {"", "chunk_tokens_out_of_range", "context_out_of_range",
+                                        "chunk_stride_invalid", "page_table_too_short"};
+    if (const int e = kvx_chunk_validation(&lanes[i])) return fail(KVX_EINVAL, names[e]);
+    if (lanes[i].chunk_tokens > KVX_TREE_NODES)
+      return fail(KVX_EINVAL, "a tree lane holds at most 16 rows");
+    if (!page_tables[i]) return fail(KVX_EINVAL, "null page table");
+  }
+  for (uint32_t first = 0; first < n_lanes; first += kLanes) {
+    CompactArgs a{};
+    a.n_lanes = std::min(kLanes, n_lanes - first);
+    a.kv_heads = l.kv_heads;
+    a.head_dim = l.head_dim;
+    a.format = l.format;
+    a.first_layer = layer == UINT32_MAX ? 0 : layer;
+    a.path_stride = path_stride;
+    a.extent_pages = s->extent_pages;
+    a.data_bytes = s->data_bytes;
+    a.scale_bytes = s->scale_bytes;
+    for (uint32_t i = 0; i < a.n_lanes; ++i) {
+      const kvx_chunk_params &p = lanes[first + i];
+      a.lane[i] = {page_tables[first + i], p.committed_tokens, p.chunk_tokens,
+                   p.page_table_entries, 0};
+    }
+    const uint32_t layers = layer == UINT32_MAX ? l.layers : 1;
+    hipLaunchKernelGGL(compact_kernel, dim3(l.kv_heads, a.n_lanes, layers), dim3(l.head_dim), 0,
+                       static_cast<hipStream_t>(stream), retained_path, retained_count, first, a);
+    if (int rc = check_launch("compact_kernel")) return rc;
+  }
+  return KVX_OK;
+}
+
+int kv_page_copy(kvx_storage *s, const kvx_page_copy *copies, uint32_t n, void *stream) {
+  if (!s || (n && !copies)) return fail(KVX_EINVAL, "kv_page_copy: null argument");
+  // All-or-nothing: validate every page before any copy is enqueued.
+  for (uint32_t i = 0; i < n; ++i) {
+    if (copies[i].from >= s->page_count || copies[i].to >= s->page_count)
+      return fail(KVX_ERANGE, "invalid KV page id");
+    if (!s->extents[copies[i].from / s->extent_pages] || !s->extents[copies[i].to / s->extent_pages])
+      return fail(KVX_ESTATE, "cannot copy a KV page of an extent that is not allocated");
+  }
+  {
+    std::vector<uint32_t> sources(n);
+    for (uint32_t i = 0; i < n; ++i) sources[i] = copies[i].from;
+    std::sort(sources.begin(), sources.end());
+    std::vector<uint32_t> targets(n);
+    for (uint32_t i = 0; i < n; ++i) targets[i] = copies[i].to;
+    std::sort(targets.begin(), targets.end());
+    for (uint32_t i = 0; i < n; ++i) {
+      if (std::binary_search(sources.begin(), sources.end(), copies[i].to))
+        return fail(KVX_EINVAL, "a page copy destination is also a source of the batch");
+      if (i && targets[i] == targets[i - 1])
+        return fail(KVX_EINVAL, "two page copies share a destination");
+    }
+  }
+  const uint32_t span = std::max(s->data_bytes, s->scale_bytes);
+  const uint32_t chunks = (span + kCopyChunk - 1) / kCopyChunk;
+  for (uint32_t first = 0; first < n; first += kCopiesPerLaunch) {
+    CopyArgs a{};
+    const uint32_t count = std::min(kCopiesPerLaunch, n - first);
+    a.extent_pages = s->extent_pages;
+    a.data_bytes = s->data_bytes;
+    a.scale_bytes = s->scale_bytes;
+    a.layers = s->layout.layers;
+    for (uint32_t i = 0; i < count; ++i) {
+      const kvx_page_copy &c = copies[first + i];
+      a.from[i] = reinterpret_cast<uint64_t>(s->extents[c.from / s->extent_pages]) |
+                  (c.from % s->extent_pages);
+      a.to[i] = reinterpret_cast<uint64_t>(s->extents[c.to / s->extent_pages]) |
+                (c.to % s->extent_pages);
+    }
+    hipLaunchKernelGGL(page_copy_kernel, dim3(chunks, s->layout.layers * 4, count), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), a);
+    if (int rc = check_launch("page_copy_kernel")) return rc;
+  }
+  return KVX_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,377 @@
+"""ctypes binding of include/kvx.h.
+
+There is no CPU fallback: every hot-path call goes to the HIP library, and
+loading fails loudly when ``libkvx.so`` is missing.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libkvx.so")
+
+INT8, BF16, INT4, FP8 = 1, 2, 3, 4
+KEYS, KEY_SCALES, VALUES, VALUE_SCALES = 0, 1, 2, 3
+OK, EINVAL, ESTATE, ENOMEM, ERANGE, EDEVICE = 0, -1, -2, -3, -4, -5
+PAGE = 32
+ALL_LAYERS = 0xFFFFFFFF
+BYTES_PER_TOKEN_LAYER = {INT4: 1056, INT8: 2080, FP8: 2080, BF16: 4096}
+
+SYMBOLS = [
+    "kvx_last_error", "kvx_layout_valid", "kvx_layout_data_bytes_per_layer_page",
+    "kvx_layout_scale_bytes_per_layer_page", "kvx_layout_bytes_per_layer_page",
+    "kvx_layout_bytes_per_model_page", "kvx_layout_extent_alignment_pages",
+    "kvx_layout_minimum_extent_pages", "kvx_layout_maximum_extent_pages",
+    "kvx_layout_extent_pages_for", "kvx_layout_largest_extent_pages", "kvx_kv_offset",
+    "kvx_verify_splits", "kvx_prefill_splits", "kvx_decode_splits", "kvx_chunk_validation",
+    "kvx_prefill_workspace", "kvx_prefill_workspace_bound", "kvx_verify_workspace",
+    "kvx_attend_workspace_bytes", "kvx_storage_create", "kvx_storage_destroy",
+    "kvx_storage_page_count", "kvx_storage_extent_pages", "kvx_storage_bytes_per_page",
+    "kvx_storage_extent_bytes", "kvx_storage_allocated_bytes", "kvx_storage_is_allocated",
+    "kvx_storage_allocate_extent", "kvx_storage_release_extent", "kvx_storage_set_budget",
+    "kvx_storage_layer", "kvx_storage_entries", "kvx_storage_write_entries",
+    "kvx_storage_page_read", "kvx_storage_page_write", "kvx_storage_extent_read",
+    "kvx_storage_extent_write", "kv_page_copy", "kvx_pool_create", "kvx_pool_destroy",
+    "kvx_pool_acquire", "kvx_pool_retain", "kvx_pool_release", "kvx_pool_page_active",
+    "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
+    "kvx_pool_snapshot_get", "kv_append", "kv_attend_verify", "kv_attend_decode",
+    "kv_attend_prefill", "kv_compact_path",
+]
+
+
+class Layout(C.Structure):
+    _fields_ = [("layers", C.c_uint32), ("kv_heads", C.c_uint32), ("head_dim", C.c_uint32),
+                ("format", C.c_uint32), ("score_scale", C.c_float)]
+
+
+class KvLayer(C.Structure):
+    _fields_ = [("extent_pages", C.c_uint32), ("offset", C.c_uint32)]
+
+
+class ChunkParams(C.Structure):
+    _fields_ = [("committed_tokens", C.c_uint32), ("chunk_tokens", C.c_uint32),
+                ("chunk_stride", C.c_uint32), ("page_table_entries", C.c_uint32),
+                ("kv", KvLayer)]
+
+
+class PrefillParams(C.Structure):
+    _fields_ = [("committed_tokens", C.c_uint32), ("rows", C.c_uint32),
+                ("chunk_stride", C.c_uint32), ("page_table_entries", C.c_uint32),
+                ("kv", KvLayer), ("split_count", C.c_uint32), ("score_scale", C.c_float)]
+
+
+class VerifyParams(C.Structure):
+    _fields_ = [("committed_tokens", C.c_uint32), ("page_table_entries", C.c_uint32),
+                ("kv", KvLayer), ("split_count", C.c_uint32), ("slot_splits", C.c_uint32),
+                ("active_rows", C.c_uint32), ("row_capacity", C.c_uint32),
+                ("score_scale", C.c_float)]
+
+
+class PageCopy(C.Structure):
+    _fields_ = [("from_", C.c_uint32), ("to", C.c_uint32)]
+
+
+class PoolSnapshot(C.Structure):
+    _fields_ = [("pages_allocated", C.c_uint32), ("pages_free", C.c_uint32),
+                ("pages_active", C.c_uint32), ("pages_prefix", C.c_uint32),
+                ("allocated_bytes", C.c_uint64), ("reclaimable_bytes", C.c_uint64),
+                ("extent_allocations", C.c_uint64), ("extent_releases", C.c_uint64),
+                ("extent_allocate_max_ms", C.c_double), ("extent_release_max_ms", C.c_double),
+                ("extent_compactions", C.c_uint64), ("pages_moved", C.c_uint64)]
+
+
+class KvxError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"kvx error {code}: {message}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """Loads libkvx.so; raises when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -m richengine_amd.build` "
+                "(there is no CPU fallback for the KV path)")
+        L = C.CDLL(LIB_PATH)
+        _declare(L)
+        _lib = L
+    return _lib
+
+
+def _declare(L):
+    u32, u64, vp, i = C.c_uint32, C.c_uint64, C.c_void_p, C.c_int
+    LP = C.POINTER(Layout)
+    L.kvx_last_error.restype = C.c_char_p
+    for n in ("kvx_layout_data_bytes_per_layer_page", "kvx_layout_scale_bytes_per_layer_page",
+              "kvx_layout_bytes_per_layer_page", "kvx_layout_bytes_per_model_page"):
+        getattr(L, n).argtypes, getattr(L, n).restype = [LP], u64
+    for n in ("kvx_layout_extent_alignment_pages", "kvx_layout_minimum_extent_pages",
+              "kvx_layout_maximum_extent_pages", "kvx_layout_largest_extent_pages"):
+        getattr(L, n).argtypes, getattr(L, n).restype = [LP], u32
+    L.kvx_layout_valid.argtypes = [LP]
+    L.kvx_layout_extent_pages_for.argtypes, L.kvx_layout_extent_pages_for.restype = [LP, u64], u32
+    L.kvx_kv_offset.argtypes, L.kvx_kv_offset.restype = [u32] * 6, u64
+    for n in ("kvx_verify_splits", "kvx_decode_splits"):
+        getattr(L, n).argtypes, getattr(L, n).restype = [u32, u32], u32
+    L.kvx_prefill_splits.argtypes, L.kvx_prefill_splits.restype = [u32], u32
+    L.kvx_chunk_validation.argtypes = [C.POINTER(ChunkParams)]
+    P64 = C.POINTER(u64)
+    L.kvx_prefill_workspace.argtypes = [u32, u32, LP, P64, P64]
+    L.kvx_prefill_workspace_bound.argtypes = [u32, u32, LP, P64, P64]
+    L.kvx_verify_workspace.argtypes = [u32, u32, u32, LP, P64, P64]
+    L.kvx_attend_workspace_bytes.argtypes = [vp, u32, u32, LP]
+    L.kvx_attend_workspace_bytes.restype = u64
+    L.kvx_storage_create.argtypes = [LP, u32, u32, i, C.POINTER(vp)]
+    L.kvx_storage_destroy.argtypes = [vp]
+    L.kvx_storage_destroy.restype = None
+    for n in ("kvx_storage_page_count", "kvx_storage_extent_pages"):
+        getattr(L, n).argtypes, getattr(L, n).restype = [vp], u32
+    for n in ("kvx_storage_bytes_per_page", "kvx_storage_extent_bytes",
+              "kvx_storage_allocated_bytes"):
+        getattr(L, n).argtypes, getattr(L, n).restype = [vp], u64
+    L.kvx_storage_is_allocated.argtypes = [vp, u32]
+    L.kvx_storage_allocate_extent.argtypes = [vp, u32]
+    L.kvx_storage_release_extent.argtypes = [vp, u32]
+    L.kvx_storage_set_budget.argtypes, L.kvx_storage_set_budget.restype = [vp, u64], None
+    L.kvx_storage_layer.argtypes = [vp, u32, C.POINTER(KvLayer)]
+    L.kvx_storage_entries.argtypes = [vp, vp, u32, u32, vp]
+    L.kvx_storage_write_entries.argtypes = [vp, vp, u32, u32, vp, u64, vp]
+    L.kvx_storage_page_read.argtypes = [vp, u32, vp]
+    L.kvx_storage_page_write.argtypes = [vp, u32, vp]
+    L.kvx_storage_extent_read.argtypes = [vp, u32, u64, u64, vp]
+    L.kvx_storage_extent_write.argtypes = [vp, u32, u64, u64, vp]
+    L.kv_page_copy.argtypes = [vp, vp, u32, vp]
+    L.kvx_pool_create.argtypes = [vp, u32, C.POINTER(vp)]
+    L.kvx_pool_destroy.argtypes, L.kvx_pool_destroy.restype = [vp], None
+    L.kvx_pool_acquire.argtypes = [vp, u32, vp]
+    L.kvx_pool_retain.argtypes = [vp, u32, i]
+    L.kvx_pool_release.argtypes = [vp, u32, i]
+    L.kvx_pool_page_active.argtypes = [vp, u32]
+    L.kvx_pool_free_pages.argtypes, L.kvx_pool_free_pages.restype = [vp], u32
+    L.kvx_pool_reclaim_empty.argtypes = [vp, i, u32, P64]
+    L.kvx_pool_compact_extent.argtypes = [vp, vp, u32, C.POINTER(u32), vp, C.POINTER(u32), vp]
+    L.kvx_pool_snapshot_get.argtypes = [vp, C.POINTER(PoolSnapshot)]
+    L.kv_append.argtypes = [vp, u32, vp, vp, vp, vp, u32, u64, u32, vp]
+    L.kv_attend_verify.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, vp, u32, vp, u64, vp]
+    L.kv_attend_decode.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, u32, vp, u64, vp]
+    L.kv_attend_prefill.argtypes = [vp, u32, u32, vp, vp, vp, C.POINTER(PrefillParams), vp, u64, vp]
+    L.kv_compact_path.argtypes = [vp, u32, vp, vp, u32, vp, vp, u32, vp]
+
+
+def check(rc):
+    if rc != OK:
+        raise KvxError(rc, lib().kvx_last_error().decode())
+    return rc
+
+
+def _stream(stream):
+    if stream is not None:
+        return C.c_void_p(stream)
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    """Device address of a torch tensor (or an int / None)."""
+    if t is None:
+        return None
+    return t if isinstance(t, int) else t.data_ptr()
+
+
+def _table_array(tables):
+    return (C.c_void_p * len(tables))(*[_ptr(t) for t in tables])
+
+
+class Storage:
+    """Page storage in device extents (the reference's kv::PageStorage)."""
+
+    def __init__(self, layers, kv_heads, head_dim, fmt, page_count, extent_pages, aligned=False,
+                 score_scale=0.0):
+        self.layout = Layout(layers, kv_heads, head_dim, fmt, score_scale)
+        h = C.c_void_p()
+        check(lib().kvx_storage_create(C.byref(self.layout), page_count, extent_pages,
+                                       int(aligned), C.byref(h)))
+        self.h = h
+        self.page_count, self.extent_pages = page_count, extent_pages
+        self.extents = page_count // extent_pages
+        self.extent_bytes = lib().kvx_storage_extent_bytes(h)
+        self.bytes_per_page = lib().kvx_storage_bytes_per_page(h)
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().kvx_storage_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        self.close()
+
+    def allocate(self, extent):
+        return check(lib().kvx_storage_allocate_extent(self.h, extent))
+
+    def allocate_all(self):
+        for e in range(self.extents):
+            self.allocate(e)
+        return self
+
+    def release(self, extent):
+        return check(lib().kvx_storage_release_extent(self.h, extent))
+
+    def layer(self, layer):
+        out = KvLayer()
+        check(lib().kvx_storage_layer(self.h, layer, C.byref(out)))
+        return out
+
+    def entries_host(self, pages, first=0):
+        import numpy as np
+        pages = np.ascontiguousarray(pages, dtype=np.uint32)
+        table = np.zeros(len(pages), dtype=np.uint64)
+        check(lib().kvx_storage_entries(self.h, pages.ctypes.data, len(pages), first,
+                                        table.ctypes.data))
+        return table
+
+    def table(self, pages):
+        """A device page table (torch int64 tensor holding the u64 entries)."""
+        import torch
+        host = self.entries_host(pages)
+        return torch.from_numpy(host.view("int64")).cuda()
+
+    def page_read(self, page):
+        import numpy as np
+        out = np.empty(self.bytes_per_page, dtype=np.uint8)
+        check(lib().kvx_storage_page_read(self.h, page, out.ctypes.data))
+        return out
+
+    def page_write(self, page, data):
+        import numpy as np
+        data = np.ascontiguousarray(data, dtype=np.uint8)
+        assert data.size == self.bytes_per_page
+        return check(lib().kvx_storage_page_write(self.h, page, data.ctypes.data))
+
+    def extent_read(self, extent, offset=0, nbytes=None):
+        import numpy as np
+        nbytes = self.extent_bytes - offset if nbytes is None else nbytes
+        out = np.empty(nbytes, dtype=np.uint8)
+        check(lib().kvx_storage_extent_read(self.h, extent, offset, nbytes, out.ctypes.data))
+        return out
+
+    def extent_write(self, extent, data, offset=0):
+        import numpy as np
+        data = np.ascontiguousarray(data, dtype=np.uint8)
+        return check(lib().kvx_storage_extent_write(self.h, extent, offset, data.size,
+                                                    data.ctypes.data))
+
+    def copy_pages(self, copies, stream=None):
+        arr = (PageCopy * len(copies))(*[PageCopy(a, b) for a, b in copies])
+        return check(lib().kv_page_copy(self.h, arr, len(copies), _stream(stream)))
+
+
+def append(storage, layer, chunk_keys, chunk_values, tables, lanes, lane_stride,
+           verify_max_rows=0, stream=None):
+    arr = (ChunkParams * len(lanes))(*lanes)
+    return check(lib().kv_append(storage.h, layer, _ptr(chunk_keys), _ptr(chunk_values),
+                                 _table_array(tables), arr, len(lanes), lane_stride,
+                                 verify_max_rows, _stream(stream)))
+
+
+def attend_workspace_bytes(storage, lanes, query_heads):
+    arr = (VerifyParams * len(lanes))(*lanes)
+    return lib().kvx_attend_workspace_bytes(arr, len(lanes), query_heads, C.byref(storage.layout))
+
+
+def attend_verify(storage, layer, query_heads, queries, output, tables, lanes, row_masks,
+                  row_stride, workspace, stream=None):
+    arr = (VerifyParams * len(lanes))(*lanes)
+    return check(lib().kv_attend_verify(storage.h, layer, query_heads, _ptr(queries), _ptr(output),
+                                        _table_array(tables), arr, len(lanes), _ptr(row_masks),
+                                        row_stride, _ptr(workspace),
+                                        workspace.numel() * workspace.element_size(),
+                                        _stream(stream)))
+
+
+def attend_decode(storage, layer, query_heads, queries, output, tables, lanes, row_stride,
+                  workspace, stream=None):
+    arr = (VerifyParams * len(lanes))(*lanes)
+    return check(lib().kv_attend_decode(storage.h, layer, query_heads, _ptr(queries), _ptr(output),
+                                        _table_array(tables), arr, len(lanes), row_stride,
+                                        _ptr(workspace),
+                                        workspace.numel() * workspace.element_size(),
+                                        _stream(stream)))
+
+
+def prefill_workspace_bytes(storage, rows, query_heads):
+    pb, sb = C.c_uint64(), C.c_uint64()
+    check(lib().kvx_prefill_workspace(rows, query_heads, C.byref(storage.layout), C.byref(pb),
+                                      C.byref(sb)))
+    return pb.value + sb.value
+
+
+def attend_prefill(storage, layer, query_heads, queries, output, table, params, workspace,
+                   stream=None):
+    return check(lib().kv_attend_prefill(storage.h, layer, query_heads, _ptr(queries),
+                                         _ptr(output), _ptr(table), C.byref(params),
+                                         _ptr(workspace),
+                                         workspace.numel() * workspace.element_size(),
+                                         _stream(stream)))
+
+
+def compact_path(storage, layer, tables, lanes, retained_path, retained_count, path_stride,
+                 stream=None):
+    arr = (ChunkParams * len(lanes))(*lanes)
+    return check(lib().kv_compact_path(storage.h, layer, _table_array(tables), arr, len(lanes),
+                                       _ptr(retained_path), _ptr(retained_count), path_stride,
+                                       _stream(stream)))
+
+
+class Pool:
+    """Page references and extent lifetime (the reference's engine::KvPool)."""
+
+    def __init__(self, storage, runway_pages):
+        h = C.c_void_p()
+        check(lib().kvx_pool_create(storage.h, runway_pages, C.byref(h)))
+        self.h, self.storage = h, storage
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().kvx_pool_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        self.close()
+
+    def acquire(self, count):
+        out = (C.c_uint32 * max(count, 1))()
+        check(lib().kvx_pool_acquire(self.h, count, out))
+        return list(out[:count])
+
+    def retain(self, page, prefix_owner=False):
+        return check(lib().kvx_pool_retain(self.h, page, int(prefix_owner)))
+
+    def release(self, page, prefix_owner=False):
+        return check(lib().kvx_pool_release(self.h, page, int(prefix_owner)))
+
+    def page_active(self, page):
+        return bool(lib().kvx_pool_page_active(self.h, page))
+
+    def reclaim_empty(self, keep_runway, limit=0xFFFFFFFF):
+        out = C.c_uint64()
+        check(lib().kvx_pool_reclaim_empty(self.h, int(keep_runway), limit, C.byref(out)))
+        return out.value
+
+    def compact_extent(self, fixed=(), stream=None):
+        fixed_arr = (C.c_uint32 * max(len(fixed), 1))(*fixed)
+        first, moved = C.c_uint32(), C.c_uint32()
+        dest = (C.c_uint32 * self.storage.extent_pages)()
+        check(lib().kvx_pool_compact_extent(self.h, fixed_arr, len(fixed), C.byref(first), dest,
+                                            C.byref(moved), _stream(stream)))
+        if not moved.value:
+            return None
+        return {"first": first.value, "dest": list(dest), "moved": moved.value}
+
+    def snapshot(self):
+        s = PoolSnapshot()
+        check(lib().kvx_pool_snapshot_get(self.h, C.byref(s)))
+        return s

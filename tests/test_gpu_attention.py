@@ -1,0 +1,313 @@
+"""GPU parity of paged attention (decode, chain / tree verify, chunked prefill)
+against the oracle on the same seeded inputs, through the C ABI.
+
+Bar: per output row, ||gpu - oracle||2 / ||oracle||2 <= 2e-3 for int4 / int8 /
+bf16 pages and <= 1e-2 for fp8 pages, on the bf16 outputs (gpulib.check_attention
+says why the oracle's fp32 value gets 2e-3 more).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import kvoracle as ko
+from richengine_amd import kvx
+import kvtestlib as T
+import gpulib as Gp
+
+pytestmark = pytest.mark.gpu
+H, G, D = 4, 6, 256
+QH = H * G
+FORMATS = [ko.INT4, ko.INT8, ko.BF16, ko.FP8]
+
+
+def tol(fmt):
+    return 1e-2 if fmt == ko.FP8 else 2e-3
+
+
+def fill(tw, total, seed, layer=1, scale=1.0):
+    """Appends `total` tokens on the device (the path under test) and mirrors
+    them into the oracle store by copying the device bytes back."""
+    n_pages = (total + 31) // 32
+    pages = tw.pages(n_pages, seed)
+    th, td = tw.tables(pages)
+    rng = np.random.default_rng(seed)
+    done = 0
+    while done < total:
+        n = min(2048, total - done)
+        k = (rng.standard_normal((H, n, D)) * scale).astype(np.float32)
+        v = (rng.standard_normal((H, n, D)) * scale).astype(np.float32)
+        k[:, :, [3, 77, 130, 255]] *= 20
+        stride = (n + 31) // 32 * 32
+        ck, cv = T.chunk_buffers(k, v, stride)
+        kvx.append(tw.dev, layer, Gp.dev(ck), Gp.dev(cv), [td],
+                   [kvx.ChunkParams(done, n, stride, n_pages)], H * stride * D)
+        p = ko.ChunkParams(done, n, stride, n_pages, tw.host.layer(layer))
+        assert ko.store_chunk(tw.fmt, H, D, ck, cv, th, p) == 1
+        done += n
+    torch.cuda.synchronize()
+    return pages, th, td
+
+
+def queries(shape_rows, seed):
+    """bf16 queries for [..., rows, G, D]-shaped tiles."""
+    rng = np.random.default_rng(seed + 999)
+    return ko.f32_to_bf16(rng.standard_normal(shape_rows).astype(np.float32)).reshape(shape_rows)
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("committed,rows", [(0, 1), (33, 7), (255, 17), (1023, 8), (100, 77),
+                                            (2000, 130)])
+def test_prefill_matches_oracle(fmt, committed, rows):
+    tw = Gp.Twin(fmt, H, D, 2, (committed + rows + 31) // 32)
+    pages, th, td = fill(tw, committed + rows, seed=committed + rows)
+    tw.assert_same_bytes()
+    stride = (rows + 31) // 32 * 32
+    q = np.zeros((H, stride, G, D), dtype=np.uint16)
+    q[:, :rows] = queries((H, rows, G, D), committed)
+    splits = kvx.lib().kvx_prefill_splits(rows)
+    hp = ko.PrefillParams(committed, rows, stride, len(pages), tw.host.layer(1), splits, 0.0)
+    ok, want, want32 = ko.attend_prefill(fmt, H, G, D, q, th, hp)
+    assert ok == 1
+    out = torch.full((H, stride, G, D), 0x5A5A, dtype=torch.int16, device="cuda")
+    ws = torch.empty(kvx.prefill_workspace_bytes(tw.dev, rows, QH), dtype=torch.uint8, device="cuda")
+    kvx.attend_prefill(tw.dev, 1, QH, Gp.dev(q), out, td,
+                       kvx.PrefillParams(committed, rows, stride, len(pages), kvx.KvLayer(), splits, 0.0), ws)
+    torch.cuda.synchronize()
+    got = Gp.host_u16(out)
+    live = np.zeros((H, stride), dtype=bool)
+    live[:, :rows] = True
+    stats = Gp.check_attention(got, want, want32, live, tol(fmt), f"prefill fmt={fmt}")
+    # the format-generic tile keeps the oracle's operation order: nearly every
+    # output has the oracle's bits (expf differs in the last place)
+    assert stats["exact"] > 0.98
+    # rows of the last tile past the chunk are zeros; rows past the tiles are untouched
+    tile_end = (rows + 7) // 8 * 8
+    assert not got[:, rows:tile_end].any()
+    assert (got[:, tile_end:] == 0x5A5A).all()
+    tw.close()
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+def test_verify_chain_matches_oracle(fmt):
+    committed = [0, 1023, 1023 + 649, 40]
+    lanes = len(committed)
+    counts = [(c + 8 + 31) // 32 for c in committed]
+    tws, hts, dts = [], [], []
+    for lane, c in enumerate(committed):
+        tw = Gp.Twin(fmt, H, D, 2, counts[lane])
+        pages, th, td = fill(tw, c + 8, seed=300 + lane)
+        tws.append(tw)
+        hts.append(th)
+        dts.append(td)
+    # every lane has its own storage here only on the oracle side; the device
+    # call needs one storage, so lanes are checked one per call and then batched
+    for lane in range(lanes):
+        tw = tws[lane]
+        q = np.zeros((1, H, 32, G, D), dtype=np.uint16)
+        q[:, :, :8] = queries((1, H, 8, G, D), lane)
+        splits = kvx.lib().kvx_verify_splits(committed[lane], 8)
+        hp = ko.VerifyParams(committed[lane], counts[lane], tw.host.layer(1), splits, 128, 8, 8, 0.0)
+        n, want, want32 = ko.attend_verify(fmt, H, G, D, q, [hts[lane]], [hp])
+        assert n == 1
+        dp = [kvx.VerifyParams(committed[lane], counts[lane], kvx.KvLayer(), splits, splits, 8, 8, 0.0)]
+        out = torch.full((1, H, 32, G, D), 0x5A5A, dtype=torch.int16, device="cuda")
+        ws = torch.empty(kvx.attend_workspace_bytes(tw.dev, dp, QH), dtype=torch.uint8, device="cuda")
+        kvx.attend_verify(tw.dev, 1, QH, Gp.dev(q), out, [dts[lane]], dp, None, 32, ws)
+        torch.cuda.synchronize()
+        got = Gp.host_u16(out)
+        live = np.zeros((1, H, 32), dtype=bool)
+        live[:, :, :8] = True
+        Gp.check_attention(got, want, want32, live, tol(fmt), f"verify lane {lane}")
+        assert (got[:, :, 8:] == 0x5A5A).all()
+    for tw in tws:
+        tw.close()
+
+
+def shared_pool_lanes(fmt, committed, rows, seed, layers=2, layer=1):
+    """Lanes with their own page tables inside one pool (the batched case)."""
+    counts = [(c + rows + 31) // 32 for c in committed]
+    tw = Gp.Twin(fmt, H, D, layers, sum(counts))
+    ids = tw.pages(sum(counts), seed)
+    hts, dts, first = [], [], 0
+    rng = np.random.default_rng(seed)
+    for lane, n in enumerate(counts):
+        th, td = tw.tables(ids[first:first + n])
+        first += n
+        hts.append(th)
+        dts.append(td)
+        total = committed[lane] + rows
+        done = 0
+        while done < total:
+            m = min(2048, total - done)
+            k = rng.standard_normal((H, m, D)).astype(np.float32)
+            v = rng.standard_normal((H, m, D)).astype(np.float32)
+            stride = (m + 31) // 32 * 32
+            ck, cv = T.chunk_buffers(k, v, stride)
+            kvx.append(tw.dev, layer, Gp.dev(ck), Gp.dev(cv), [td],
+                       [kvx.ChunkParams(done, m, stride, n)], H * stride * D)
+            p = ko.ChunkParams(done, m, stride, n, tw.host.layer(layer))
+            assert ko.store_chunk(fmt, H, D, ck, cv, th, p) == 1
+            done += m
+    torch.cuda.synchronize()
+    return tw, counts, hts, dts
+
+
+@pytest.mark.parametrize("fmt", [ko.INT4, ko.INT8, ko.BF16])
+def test_batched_verify_chain_matches_oracle(fmt):
+    committed = [0, 1023, 1672, 31]
+    tw, counts, hts, dts = shared_pool_lanes(fmt, committed, 8, seed=41)
+    lanes = len(committed)
+    q = np.zeros((lanes, H, 32, G, D), dtype=np.uint16)
+    q[:, :, :8] = queries((lanes, H, 8, G, D), 5)
+    splits = [kvx.lib().kvx_verify_splits(c, 8) for c in committed]
+    hp = [ko.VerifyParams(committed[i], counts[i], tw.host.layer(1), splits[i], 128, 8, 8, 0.0)
+          for i in range(lanes)]
+    n, want, want32 = ko.attend_verify(fmt, H, G, D, q, hts, hp)
+    assert n == lanes
+    dp = [kvx.VerifyParams(committed[i], counts[i], kvx.KvLayer(), splits[i], 128, 8, 8, 0.0)
+          for i in range(lanes)]
+    out = torch.zeros((lanes, H, 32, G, D), dtype=torch.int16, device="cuda")
+    ws = torch.empty(kvx.attend_workspace_bytes(tw.dev, dp, QH), dtype=torch.uint8, device="cuda")
+    kvx.attend_verify(tw.dev, 1, QH, Gp.dev(q), out, dts, dp, None, 32, ws)
+    torch.cuda.synchronize()
+    live = np.zeros((lanes, H, 32), dtype=bool)
+    live[:, :, :8] = True
+    Gp.check_attention(Gp.host_u16(out), want, want32, live, tol(fmt), "batched verify")
+    # a repeat submission gives the same bits
+    out2 = torch.zeros_like(out)
+    kvx.attend_verify(tw.dev, 1, QH, Gp.dev(q), out2, dts, dp, None, 32, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+    tw.close()
+
+
+def tree_masks(parents):
+    masks = []
+    for row, parent in enumerate(parents):
+        masks.append((1 << row) | (masks[parent] if parent >= 0 else 0))
+    return masks
+
+
+@pytest.mark.parametrize("fmt", [ko.INT4, ko.INT8, ko.BF16])
+@pytest.mark.parametrize("nodes", [15, 16])
+def test_tree_verify_matches_oracle(fmt, nodes):
+    committed = [260, 31, 4000]
+    lanes = len(committed)
+    tw, counts, hts, dts = shared_pool_lanes(fmt, committed, nodes, seed=61 + nodes)
+    rng = np.random.default_rng(nodes)
+    masks = np.zeros((lanes, 16), dtype=np.uint32)
+    for lane in range(lanes):
+        parents = [-1] + [int(rng.integers(max(0, i - 3), i)) for i in range(1, nodes)]
+        masks[lane, :nodes] = tree_masks(parents)
+    q = np.zeros((lanes, H, 32, G, D), dtype=np.uint16)
+    q[:, :, :16] = queries((lanes, H, 16, G, D), 7)
+    splits = [kvx.lib().kvx_verify_splits(c, nodes) for c in committed]
+    hp = [ko.VerifyParams(committed[i], counts[i], tw.host.layer(1), splits[i], 128, nodes, 16, 0.0)
+          for i in range(lanes)]
+    n, want, want32 = ko.attend_verify(fmt, H, G, D, q, hts, hp, masks)
+    assert n == lanes
+    dp = [kvx.VerifyParams(committed[i], counts[i], kvx.KvLayer(), splits[i], 128, nodes, 16, 0.0)
+          for i in range(lanes)]
+    out = torch.full((lanes, H, 32, G, D), 0x5A5A, dtype=torch.int16, device="cuda")
+    ws = torch.empty(kvx.attend_workspace_bytes(tw.dev, dp, QH), dtype=torch.uint8, device="cuda")
+    kvx.attend_verify(tw.dev, 1, QH, Gp.dev(q), out, dts, dp, Gp.dev(masks), 32, ws)
+    torch.cuda.synchronize()
+    got = Gp.host_u16(out)
+    live = np.zeros((lanes, H, 32), dtype=bool)
+    live[:, :, :nodes] = True
+    Gp.check_attention(got, want, want32, live, tol(fmt), "tree verify")
+    assert not got[:, :, nodes:16].any() and (got[:, :, 16:] == 0x5A5A).all()
+    tw.close()
+
+
+def decode_case(fmt, committed, seed, row_stride=1, layers=2, layer=1):
+    lanes = len(committed)
+    tw, counts, hts, dts = shared_pool_lanes(fmt, committed, 1, seed=seed, layers=layers, layer=layer)
+    q = np.zeros((lanes, H, row_stride, G, D), dtype=np.uint16)
+    q[:, :, 0] = queries((lanes, H, G, D), seed)
+    splits = [kvx.lib().kvx_decode_splits(c, 1) for c in committed]
+    want = np.zeros((lanes, H, G, D), dtype=np.uint16)
+    want32 = np.zeros((lanes, H, G, D), dtype=np.float32)
+    for i in range(lanes):
+        # the oracle's decode is its prefill entry with one row; its contract
+        # bounds the split count at 32, the verify entry at 128
+        q1 = np.zeros((1, H, 32, G, D), dtype=np.uint16)
+        q1[0, :, 0] = q[i, :, 0]
+        hp = ko.VerifyParams(committed[i], counts[i], tw.host.layer(layer), splits[i], 128, 1, 1, 0.0)
+        n, o, o32 = ko.attend_verify(fmt, H, G, D, q1, [hts[i]], [hp])
+        assert n == 1
+        want[i], want32[i] = o[0, :, 0], o32[0, :, 0]
+    dp = [kvx.VerifyParams(committed[i], counts[i], kvx.KvLayer(), splits[i], splits[i], 1, 1, 0.0)
+          for i in range(lanes)]
+    out = torch.full((lanes, H, row_stride, G, D), 0x5A5A, dtype=torch.int16, device="cuda")
+    ws = torch.empty(kvx.attend_workspace_bytes(tw.dev, dp, QH), dtype=torch.uint8, device="cuda")
+    kvx.attend_decode(tw.dev, layer, QH, Gp.dev(q), out, dts, dp, row_stride, ws)
+    torch.cuda.synchronize()
+    got = Gp.host_u16(out)
+    stats = Gp.check_attention(got[:, :, 0], want, want32, np.ones((lanes, H), dtype=bool), tol(fmt),
+                               f"decode fmt={fmt}")
+    if row_stride > 1:
+        assert (got[:, :, 1:] == 0x5A5A).all()
+    tw.close()
+    return stats
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+def test_decode_matches_oracle(fmt):
+    decode_case(fmt, [0, 1, 31, 32, 511, 512, 1000, 2047, 4095, 600, 33, 5000], seed=80 + fmt)
+
+
+@pytest.mark.parametrize("row_stride", [1, 32])
+def test_int4_decode_many_lanes_and_strides(row_stride):
+    rng = np.random.default_rng(row_stride)
+    committed = [int(x) for x in rng.integers(0, 3000, 40)]
+    decode_case(ko.INT4, committed, seed=5 + row_stride, row_stride=row_stride)
+
+
+def test_int4_decode_single_token_is_the_value_row():
+    tw, counts, hts, dts = shared_pool_lanes(ko.INT4, [0], 1, seed=3)
+    q = queries((1, H, 1, G, D), 1)
+    dp = [kvx.VerifyParams(0, 1, kvx.KvLayer(), 1, 1, 1, 1, 0.0)]
+    out = torch.zeros((1, H, 1, G, D), dtype=torch.int16, device="cuda")
+    ws = torch.empty(kvx.attend_workspace_bytes(tw.dev, dp, QH), dtype=torch.uint8, device="cuda")
+    kvx.attend_decode(tw.dev, 1, QH, Gp.dev(q), out, dts, dp, 1, ws)
+    torch.cuda.synchronize()
+    got = ko.bf16_to_f32(Gp.host_u16(out)).reshape(H, G, D)
+    page = int((hts[0][0] & 0x3FFF)) + 0  # index inside its extent
+    kc, ks, vc, vs = T.page_codes(tw.host, 1, int(tw.pages(1, 3)[0]))
+    for h in range(H):
+        w = ko.bf16_to_f32(ko.f32_to_bf16(vs[h, :1]))[0]
+        want = ko.bf16_to_f32(ko.f32_to_bf16((w * vc[h, 0]).astype(np.float32)))
+        for g in range(G):
+            assert np.array_equal(got[h, g], want)
+    tw.close()
+
+
+def test_invalid_attention_parameters_enqueue_nothing():
+    tw, counts, hts, dts = shared_pool_lanes(ko.INT8, [40], 8, seed=9)
+    q = Gp.dev(queries((1, H, 32, G, D), 2))
+    out = torch.full((1, H, 32, G, D), 0x5A5A, dtype=torch.int16, device="cuda")
+    good = kvx.VerifyParams(40, counts[0], kvx.KvLayer(), 32, 32, 8, 8, 0.0)
+    ws = torch.full((kvx.attend_workspace_bytes(tw.dev, [good], QH),), 0xA5, dtype=torch.uint8, device="cuda")
+    cases = []
+    for field, value in (("page_table_entries", 1), ("split_count", 0), ("split_count", 129),
+                         ("active_rows", 0), ("active_rows", 9), ("committed_tokens", 262159)):
+        p = kvx.VerifyParams(40, counts[0], kvx.KvLayer(), 32, 32, 8, 8, 0.0)
+        setattr(p, field, value)
+        cases.append(p)
+    for p in cases:
+        with pytest.raises(kvx.KvxError) as err:
+            kvx.attend_verify(tw.dev, 1, QH, q, out, dts, [p], None, 32, ws)
+        assert err.value.code == kvx.EINVAL
+    with pytest.raises(kvx.KvxError):  # undersized scratch
+        kvx.attend_verify(tw.dev, 1, QH, q, out, dts, [good], None, 32, ws[:-4])
+    with pytest.raises(kvx.KvxError):  # query heads not a multiple of the KV heads
+        kvx.attend_verify(tw.dev, 1, QH + 1, q, out, dts, [good], None, 32, ws)
+    with pytest.raises(kvx.KvxError):  # aliasing
+        kvx.attend_verify(tw.dev, 1, QH, q, q, dts, [good], None, 32, ws)
+    bad_prefill = kvx.PrefillParams(40, 8, 32, 1, kvx.KvLayer(), 4, 0.0)
+    with pytest.raises(kvx.KvxError):
+        kvx.attend_prefill(tw.dev, 1, QH, q, out, dts[0], bad_prefill, ws)
+    torch.cuda.synchronize()
+    assert (out == 0x5A5A).all() and (ws == 0xA5).all()
+    tw.close()
