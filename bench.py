@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged-KV decode path on one MI355X.
+
+Workload (BASELINE.json configs[2], the one the metric is quoted on): int4 KV,
+16 layers, 4 KV heads x 256, 24 query heads, batch 32 with contexts drawn
+uniformly from [512, 32768]; pages come from a device-sized pool in a
+seed-shuffled order, reached through per-sequence page tables.  One step is one
+decode step of the whole batch: per layer, append one token per sequence
+(quantize + scatter) and run paged decode attention (split partials + merge).
+
+Prints ONE JSON line: whole-step KV GB/s (algorithmic KV bytes read by attention
+/ step time), decode tokens/s, the roofline of the dominant kernel measured
+with events on the launch stream, and the CPU oracle timed on a bounded sample.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+H, G, D, LAYERS = 4, 6, 256, 16
+QH = H * G
+BATCH = 32
+BYTES_PER_TOKEN_LAYER = 1056  # int4: 2 * (4 heads * 128 B + 4 * 4 B scales)
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--seed", type=int, default=20261125)
+    ap.add_argument("--pool-gb", type=float, default=0.0,
+                    help="KV pool size; 0 = 80%% of free HBM, at most 256 GB")
+    ap.add_argument("--contiguous", action="store_true",
+                    help="hand out pages in order instead of shuffled (TLB comparison)")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0,
+                    help="CPU oracle budget; 0 skips the CPU baseline")
+    ap.add_argument("--kernel-iters", type=int, default=20)
+    ap.add_argument("--pages-per-split", type=int, default=0,
+                    help="override the library's decode split rule (experiments)")
+    return ap.parse_args()
+
+
+def cpu_baseline(contexts, seed, budget_s):
+    """The oracle (scalar port, one thread) on a bounded sample of the same
+    workload: the first sequences of the batch, one layer, one token appended
+    then one decode attention each."""
+    import numpy as np
+    from oracle import kvoracle as ko
+
+    rng = np.random.default_rng(seed)
+    bytes_done, tokens_done, spent, lanes_done = 0, 0, 0.0, 0
+    order = np.argsort(contexts)  # shortest first so the sample stays bounded
+    for lane in order:
+        ctx = int(contexts[lane])
+        if spent > 0 and spent + spent / max(tokens_done, 1) * ctx > budget_s:
+            break
+        n_pages = (ctx + 1 + 31) // 32
+        store = ko.Store(1, H, D, ko.INT4, n_pages, n_pages)
+        store.allocate(0)
+        table = store.entries(np.arange(n_pages, dtype=np.uint32))
+        # history is filled outside the timed region
+        done = 0
+        while done < ctx:
+            n = min(2048, ctx - done)
+            stride = (n + 31) // 32 * 32
+            k = ko.f32_to_bf16(rng.standard_normal((H, stride, D)).astype(np.float32)).reshape(H, stride, D)
+            v = ko.f32_to_bf16(rng.standard_normal((H, D, stride)).astype(np.float32)).reshape(H, D, stride)
+            ko.store_chunk(ko.INT4, H, D, k, v, table, ko.ChunkParams(done, n, stride, n_pages, store.layer(0)))
+            done += n
+        k = ko.f32_to_bf16(rng.standard_normal((H, 32, D)).astype(np.float32)).reshape(H, 32, D)
+        v = ko.f32_to_bf16(rng.standard_normal((H, D, 32)).astype(np.float32)).reshape(H, D, 32)
+        q = np.zeros((1, H, 32, G, D), dtype=np.uint16)
+        q[0, :, 0] = ko.f32_to_bf16(rng.standard_normal((H, G, D)).astype(np.float32)).reshape(H, G, D)
+        splits = min(max(1, ((ctx + 1 + 31) // 32 + 31) // 32), 128)
+        t0 = time.perf_counter()
+        ko.store_chunk(ko.INT4, H, D, k, v, table, ko.ChunkParams(ctx, 1, 32, n_pages, store.layer(0)))
+        ko.attend_verify(ko.INT4, H, G, D, q, [table],
+                         [ko.VerifyParams(ctx, n_pages, store.layer(0), splits, 128, 1, 1, 0.0)],
+                         want_f32=False)
+        spent += time.perf_counter() - t0
+        bytes_done += (ctx + 1) * BYTES_PER_TOKEN_LAYER
+        tokens_done += ctx + 1
+        lanes_done += 1
+        store.close()
+    return {
+        "value": bytes_done / spent / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": f"{lanes_done} shortest sequences of the batch ({tokens_done} tokens), one layer: "
+                  f"append 1 token + decode attention each, {spent:.1f} s of scalar C++ oracle",
+        "decode_tokens_per_s_one_layer": lanes_done / spent,
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: the KV path of this build has no multi-GPU leg "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+    from richengine_amd import kvx
+
+    if not os.path.exists(kvx.LIB_PATH):
+        from richengine_amd import build as kvx_build
+        kvx_build.build(verbose=False)
+    L = kvx.lib()
+    torch.cuda.set_device(0)
+    rng = np.random.default_rng(args.seed)
+
+    # ---- pool -----------------------------------------------------------------
+    layout = kvx.Layout(LAYERS, H, D, kvx.INT4, 0.0)
+    extent_pages = L.kvx_layout_largest_extent_pages(C.byref(layout))
+    page_bytes = L.kvx_layout_bytes_per_model_page(C.byref(layout))
+    extent_bytes = extent_pages * page_bytes
+    free, _total = torch.cuda.mem_get_info()
+    pool_bytes = args.pool_gb * 1e9 if args.pool_gb > 0 else min(0.8 * free, 256e9)
+    extents = max(1, int(pool_bytes // extent_bytes))
+    contexts = rng.integers(512, 32769, BATCH)
+    total_steps = args.warmup + args.steps + args.kernel_iters + 8
+    lane_pages = [(int(c) + total_steps + 31) // 32 for c in contexts]
+    while extents * extent_pages < sum(lane_pages):
+        extents += 1
+    storage = kvx.Storage(LAYERS, H, D, kvx.INT4, extents * extent_pages, extent_pages, aligned=True)
+    storage.allocate_all()
+    pool_pages = extents * extent_pages
+    ids = (np.arange(pool_pages) if args.contiguous else rng.permutation(pool_pages))
+    ids = ids[:sum(lane_pages)].astype(np.uint32)
+    tables, first = [], 0
+    for n in lane_pages:
+        tables.append(storage.table(ids[first:first + n]))
+        first += n
+
+    # ---- history: quantize-on-append through the library ----------------------
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(args.seed)
+    for lane, ctx in enumerate(contexts):
+        ctx, done = int(ctx), 0
+        while done < ctx:
+            n = min(2048, ctx - done)
+            stride = (n + 31) // 32 * 32
+            k = torch.randn((H, stride, D), generator=gen, device="cuda", dtype=torch.float32).bfloat16()
+            v = torch.randn((H, D, stride), generator=gen, device="cuda", dtype=torch.float32).bfloat16()
+            for layer in range(LAYERS):
+                kvx.append(storage, layer, k, v, [tables[lane]],
+                           [kvx.ChunkParams(done, n, stride, lane_pages[lane])], H * stride * D)
+            done += n
+    torch.cuda.synchronize()
+
+    # ---- step buffers -----------------------------------------------------------
+    chunk_k = torch.randn((BATCH, H, 32, D), generator=gen, device="cuda").bfloat16()
+    chunk_v = torch.randn((BATCH, H, D, 32), generator=gen, device="cuda").bfloat16()
+    queries = torch.randn((BATCH, H, 1, G, D), generator=gen, device="cuda").bfloat16()
+    output = torch.zeros_like(queries)
+    committed = [int(c) for c in contexts]
+
+    def lane_params():
+        ap = [kvx.ChunkParams(committed[i], 1, 32, lane_pages[i]) for i in range(BATCH)]
+        vp = []
+        for i in range(BATCH):
+            s = L.kvx_decode_splits(committed[i], 1)
+            if args.pages_per_split:
+                pages = (committed[i] + 1 + 31) // 32
+                s = min(max(1, -(-pages // args.pages_per_split)), 128)
+            vp.append(kvx.VerifyParams(committed[i], lane_pages[i], kvx.KvLayer(), s, s, 1, 1, 0.0))
+        return ap, vp
+
+    _, vp_max = lane_params()
+    ws_bytes = 2 * kvx.attend_workspace_bytes(storage, vp_max, QH) + (1 << 20)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    table_arr = (C.c_void_p * BATCH)(*[t.data_ptr() for t in tables])
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    lane_stride = H * 32 * D
+
+    def step():
+        ap, vp = lane_params()
+        ap_arr = (kvx.ChunkParams * BATCH)(*ap)
+        vp_arr = (kvx.VerifyParams * BATCH)(*vp)
+        for layer in range(LAYERS):
+            rc = L.kv_append(storage.h, layer, chunk_k.data_ptr(), chunk_v.data_ptr(), table_arr,
+                             ap_arr, BATCH, lane_stride, 15, stream)
+            if rc:
+                kvx.check(rc)
+            rc = L.kv_attend_decode(storage.h, layer, QH, queries.data_ptr(), output.data_ptr(),
+                                    table_arr, vp_arr, BATCH, 1, workspace.data_ptr(), ws_bytes, stream)
+            if rc:
+                kvx.check(rc)
+        for i in range(BATCH):
+            committed[i] += 1
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    kv_bytes = 0
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        kv_bytes += sum(c + 1 for c in committed) * BYTES_PER_TOKEN_LAYER * LAYERS
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    gpu_ms = start.elapsed_time(stop)
+    ms_per_step = wall * 1e3 / args.steps
+    value = kv_bytes / wall / 1e9
+
+    # ---- dominant kernel: decode attention (split + merge), one layer per launch
+    # Same inputs as a step's attention; events sit on the launch stream.
+    _, vp = lane_params()
+    vp_arr = (kvx.VerifyParams * BATCH)(*vp)
+    launch_bytes = sum(c + 1 for c in committed) * BYTES_PER_TOKEN_LAYER
+    for layer in range(2):
+        L.kv_attend_decode(storage.h, layer, QH, queries.data_ptr(), output.data_ptr(), table_arr,
+                           vp_arr, BATCH, 1, workspace.data_ptr(), ws_bytes, stream)
+    torch.cuda.synchronize()
+    k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    k0.record()
+    for it in range(args.kernel_iters):
+        L.kv_attend_decode(storage.h, it % LAYERS, QH, queries.data_ptr(), output.data_ptr(),
+                           table_arr, vp_arr, BATCH, 1, workspace.data_ptr(), ws_bytes, stream)
+    k1.record()
+    torch.cuda.synchronize()
+    kernel_ms = k0.elapsed_time(k1) / args.kernel_iters
+    achieved = launch_bytes / (kernel_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "int4 paged decode attn: KV GB/s (% HBM peak) + decode tokens/s, bs=32",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int4 pages, bf16 MFMA, fp32 accumulate",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE configs[2]: batched mixed-length int4 decode, batch 32, contexts "
+                        "U[512,32768], 16 layers, 4 KV heads x 256, 24 query heads, 1-token append "
+                        "+ split-K paged attention per layer",
+            "batch": BATCH, "layers": LAYERS, "context_tokens_total": int(sum(committed)),
+            "pool_gb": round(extents * extent_bytes / 1e9, 1), "extents": extents,
+            "page_order": "contiguous" if args.contiguous else "seed-shuffled",
+            "seed": args.seed,
+        },
+        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "decode_tokens_per_s": round(BATCH * args.steps / wall, 1),
+        "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
+        "roofline": {
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel": "decode_int4_kernel (paged decode attention split kernel; merge kernel timed with it), one layer of the batch per launch",
+            "bytes_per_launch": launch_bytes, "ms_per_launch": round(kernel_ms, 4),
+        },
+    }
+    storage.close()
+    if args.cpu_seconds > 0:
+        result["cpu_baseline"] = cpu_baseline(contexts, args.seed, args.cpu_seconds)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -149,7 +149,7 @@ uint32_t kvx_prefill_splits(uint32_t rows);
    KVX_DECODE_PAGES_PER_SPLIT visible pages, at least 1, at most 128.  Decode at
    batch 32 has enough (lane, head) parallelism that the reference's 32-split
    floor would only add partial traffic. */
-#define KVX_DECODE_PAGES_PER_SPLIT 16u
+#define KVX_DECODE_PAGES_PER_SPLIT 32u
 uint32_t kvx_decode_splits(uint32_t committed_tokens, uint32_t rows);
 /* kv::chunkedPrefillValidationError: 0 ok, 1 chunk_tokens_out_of_range,
    2 context_out_of_range, 3 chunk_stride_invalid, 4 page_table_too_short */
@@ -319,6 +319,12 @@ int kv_compact_path(const kvx_storage *storage, uint32_t layer,
                     const uint64_t *const *page_tables, const kvx_chunk_params *lanes,
                     uint32_t n_lanes, const uint32_t *retained_path,
                     const uint32_t *retained_count, uint32_t path_stride, void *stream);
+
+/* Profiling aid with no counterpart in the reference: selects which phases the
+   attend entries launch (bit 0 = split kernel, bit 1 = merge kernel; default 3)
+   so a harness can time one kernel alone with events on its stream.  Outputs
+   are only meaningful with both bits set. */
+void kvx_debug_set_attend_phases(uint32_t phases);
 
 #ifdef __cplusplus
 }

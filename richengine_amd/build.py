@@ -15,22 +15,22 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
          "-I", os.path.join(ROOT, "include"), "-I", CSRC]
 
 
-def build(verbose=True):
+def build(verbose=True, lib=LIB, extra_flags=(), tag=""):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objects = []
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
     for src in SOURCES:
-        obj = os.path.join(HERE, "build", src + ".o")
-        cmd = [hipcc, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + FLAGS
+        obj = os.path.join(HERE, "build", src + tag + ".o")
+        cmd = [hipcc, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + FLAGS + list(extra_flags)
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)
         objects.append(obj)
-    cmd = [hipcc, "-shared", "-o", LIB] + objects + ["--offload-arch=gfx950"]
+    cmd = [hipcc, "-shared", "-o", lib] + objects + ["--offload-arch=gfx950"]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
-    return LIB
+    return lib
 
 
 if __name__ == "__main__":

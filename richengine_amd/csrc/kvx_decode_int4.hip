@@ -1,8 +1,490 @@
-// int4 decode attention kernels (placeholder launcher until the kernel lands).
+// int4 paged decode attention for gfx950: the split kernel of kv_attend_decode
+// for packed-nibble pages with head dimension 256.
+//
+// One wave per (sequence, split, KV head) streams the split's pages once:
+// coalesced 128-bit key loads and 64-bit value loads, the page's fp32 scales,
+// bf16 MFMA (16x16x32) for q.k and p.v with the GQA group as the 16-wide N
+// side, page-granular online softmax in registers.  The arithmetic follows the
+// reference tile (common/paged_attention_tile.h:85-349): scores are the raw
+// code dot product times the key scale times the score scale, the running
+// maximum moves once per 32-token page, and probability x value scale is
+// rounded to bf16 before it meets the value codes.
+//
+// Nibble -> bf16 without a table: OR-ing a 4-bit field into the mantissa of
+// 0x4300 gives 128 + field exactly.  With the stored two's-complement code c,
+// field = (c & 15) ^ 8 = c + 8 gives 136 + c and field = (c & 15) ^ 7 = 7 - c
+// gives 135 - c.  Even positions use the first form, odd positions the second
+// with the other operand negated, so the products are q.c + 136 q and
+// q.c - 135 q: the constant parts largely cancel pairwise and what is left is
+// tracked in fp32 and subtracted (keys: once per q row; values: per page,
+// rescaled with the accumulator).  Positions are dimensions for q.k and tokens
+// for p.v.
+#include <algorithm>
+
 #include "kvx_device.h"
 
-int kvx_decode_int4_launch(const kvx_storage *, kvx_kv_layer, uint32_t, const void *, void *,
-                           const uint64_t *const *, const kvx_verify_params *, uint32_t, uint32_t,
-                           void *, uint64_t, hipStream_t) {
-  return 1;  // declined: the caller runs the generic tile
+namespace kvx {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+#define KVX_GLOBAL __attribute__((address_space(1)))
+
+// Loads through pointers rebuilt from page entries: say they are global memory
+// so the compiler emits global_load rather than flat_load.
+template <class T>
+__device__ __forceinline__ T load_streaming(const uint8_t *p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const KVX_GLOBAL T *>(
+      reinterpret_cast<uintptr_t>(p)));
+}
+template <class T>
+__device__ __forceinline__ T load_global(const void *p) {
+  return *reinterpret_cast<const KVX_GLOBAL T *>(reinterpret_cast<uintptr_t>(p));
+}
+
+constexpr uint32_t kPage = KVX_PAGE_TOKENS;
+constexpr uint32_t kLanes = KVX_LANES_PER_LAUNCH;
+constexpr uint32_t kD = 256;
+constexpr uint32_t kRowBytes = kD / 2;                // one token's packed row
+constexpr uint32_t kHeadSlabBytes = kPage * kRowBytes;  // 4 KiB per (head, page, tensor)
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct DecodeLane {
+  const uint64_t *table;
+  uint32_t committed;
+  uint32_t split_count;
+  uint32_t first_item;  // first (lane, split) work item of this lane
+  float score_scale;
+  uint64_t row_base;    // first fused row of the lane's slots in the workspace
+  uint64_t q_offset;    // element offset of the lane's queries
+};
+struct DecodeArgs {
+  DecodeLane lane[kLanes];
+  uint32_t n_lanes;
+  uint32_t kv_heads;
+  uint32_t group;
+  uint32_t row_stride;
+  kvx_kv_layer kv;
+};
+
+// What one lane holds of one page.
+struct PageRegs {
+  u32x4 k[4];   // [token block * 2 + half row]: 16 bytes of the lane's key token
+  u32x2 v[8];   // [token slot]: 8 bytes (16 dims) of each of the lane's 8 tokens
+  f32x4 ks[2];  // key scales of the lane's score tokens, per token block
+  f32x4 vs[2];  // value scales, same tokens
+};
+
+__device__ __forceinline__ f32x4 mfma_bf16(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// Lane geometry: t = lane & 15, g = lane >> 4.
+//  q.k : A = keys, row t = token 16*tb + t of the page; k-slots = the 8 nibbles
+//        of one dword of that token's row.  B = queries, column t = q head.
+//        Output column t = q head, rows 4g..4g+3 = tokens 16*tb + 4g + r.
+//  p.v : A = values, row t = dims 16t..16t+15 (one MFMA per nibble position),
+//        k-slots = the lane group's 8 tokens 4g..4g+3, 16+4g..16+4g+3.
+//        B = probabilities, column t = q head: exactly the q.k output registers.
+__device__ __forceinline__ void load_page(PageRegs &r, uint64_t entry, uint32_t head,
+                                          uint32_t kv_heads, uint32_t layer_offset,
+                                          uint64_t key_scales_off, uint64_t values_off,
+                                          uint64_t value_scales_off, uint32_t t, uint32_t g) {
+  const uint32_t index = uint32_t(entry) & KVX_PAGE_INDEX_MASK;
+  const uint8_t *region = reinterpret_cast<const uint8_t *>(entry - index) + layer_offset;
+  const uint64_t slab = (uint64_t(index) * kv_heads + head) * kHeadSlabBytes;
+  const uint8_t *keys = region + slab;
+  const uint8_t *values = region + values_off + slab;
+  const uint64_t scale_index = (uint64_t(index) * kv_heads + head) * kPage;
+  const float *key_scales = reinterpret_cast<const float *>(region + key_scales_off) + scale_index;
+  const float *value_scales =
+      reinterpret_cast<const float *>(region + value_scales_off) + scale_index;
+#pragma unroll
+  for (uint32_t tb = 0; tb < 2; ++tb)
+#pragma unroll
+    for (uint32_t half = 0; half < 2; ++half)
+      r.k[tb * 2 + half] =
+          load_streaming<u32x4>(keys + (16 * tb + t) * kRowBytes + 64 * half + 16 * g);
+#pragma unroll
+  for (uint32_t s = 0; s < 8; ++s) {
+    const uint32_t token = (s < 4 ? 0 : 16) + 4 * g + (s & 3);
+    r.v[s] = load_streaming<u32x2>(values + token * kRowBytes + 8 * t);
+  }
+#pragma unroll
+  for (uint32_t tb = 0; tb < 2; ++tb) {
+    r.ks[tb] = load_global<f32x4>(key_scales + 16 * tb + 4 * g);
+    r.vs[tb] = load_global<f32x4>(value_scales + 16 * tb + 4 * g);
+  }
+}
+
+// Four bf16 pairs from one dword of eight nibbles: register p holds nibble p
+// (low half) and nibble p + 4 (high half).  Even nibbles become 136 + c, odd
+// ones 135 - c.
+__device__ __forceinline__ u32x4 expand_key_dword(uint32_t x) {
+  u32x4 out;
+  out[0] = (x & 0x000F000Fu) ^ 0x43084308u;
+  out[1] = ((x >> 4) & 0x000F000Fu) ^ 0x43074307u;
+  out[2] = ((x >> 8) & 0x000F000Fu) ^ 0x43084308u;
+  out[3] = ((x >> 12) & 0x000F000Fu) ^ 0x43074307u;
+  return out;
+}
+
+struct State {
+  f32x4 acc[16];  // [nibble position m]: dims 16*(4g + r) + m of q head t
+  float row_max;
+  float row_sum;   // this lane's tokens only; lanes of a q head are summed at the end
+  float bias;      // constant part carried by acc, this lane's tokens only
+};
+
+__device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 *q_lds, float q_bias,
+                                            float score_scale, uint32_t first_token,
+                                            uint32_t visible, uint32_t lane, uint32_t g,
+                                            State &st) {
+#ifdef KVX_PROBE_STREAM_ONLY
+  // Measurement build: consume every loaded register with almost no arithmetic,
+  // to see what the memory system delivers for this access pattern.
+  uint32_t x = 0;
+  for (uint32_t i = 0; i < 4; ++i) x ^= r.k[i][0] ^ r.k[i][1] ^ r.k[i][2] ^ r.k[i][3];
+  for (uint32_t i = 0; i < 8; ++i) x ^= r.v[i][0] ^ r.v[i][1];
+  st.row_sum += r.ks[0][0] + r.ks[1][3] + r.vs[0][1] + r.vs[1][2] + __uint_as_float(x & 0xffu);
+  return;
+#endif
+  // ---- q.k ----
+  f32x4 s[2];
+  s[0] = s[1] = f32x4{-q_bias, -q_bias, -q_bias, -q_bias};
+#pragma unroll
+  for (uint32_t kb = 0; kb < 8; ++kb) {
+    const u32x4 q = q_lds[kb * 64 + lane];
+#pragma unroll
+    for (uint32_t tb = 0; tb < 2; ++tb)
+      s[tb] = mfma_bf16(expand_key_dword(r.k[tb * 2 + (kb >> 2)][kb & 3]), q, s[tb]);
+  }
+  // ---- page softmax ----
+  float score[8], local_max = -INFINITY;
+  bool live[8];
+#pragma unroll
+  for (uint32_t i = 0; i < 8; ++i) {
+    const uint32_t tb = i >> 2, rr = i & 3;
+    float v = s[tb][rr] * r.ks[tb][rr];
+    v *= score_scale;
+    live[i] = first_token + 16 * tb + 4 * g + rr < visible;
+    score[i] = live[i] ? v : -INFINITY;
+    local_max = fmaxf(local_max, score[i]);
+  }
+  local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
+  local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
+  const float next_max = fmaxf(st.row_max, local_max);
+  const float rescale = __builtin_amdgcn_exp2f((st.row_max - next_max) * kLog2e);
+  float weight[8], page_sum = 0.0f;
+#pragma unroll
+  for (uint32_t i = 0; i < 8; ++i) {
+    // The difference first, so the page's maximum gets exactly 1.
+    const float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
+    page_sum += p;
+    const float w = p * r.vs[i >> 2][i & 3];
+    weight[i] = live[i] ? w : 0.0f;
+  }
+  st.row_sum = fmaf(st.row_sum, rescale, page_sum);
+  st.row_max = next_max;
+  // bf16 probabilities (round to nearest even): even tokens as they are, odd
+  // tokens negated (their value codes are expanded as 135 - c).
+  u32x4 pb;
+  float page_bias = 0.0f;
+#pragma unroll
+  for (uint32_t p = 0; p < 4; ++p) {
+    const f32x2 pair = {weight[2 * p], weight[2 * p + 1]};
+    const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+    page_bias = fmaf(136.0f, __uint_as_float(bits << 16), page_bias);
+    page_bias = fmaf(-135.0f, __uint_as_float(bits & 0xffff0000u), page_bias);
+    pb[p] = bits ^ 0x80000000u;
+  }
+  st.bias = fmaf(st.bias, rescale, page_bias);
+  if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
+#pragma unroll
+    for (uint32_t m = 0; m < 16; ++m) st.acc[m] *= rescale;
+  }
+  // ---- p.v ----
+#pragma unroll
+  for (uint32_t half = 0; half < 2; ++half) {
+#pragma unroll
+    for (uint32_t part = 0; part < 2; ++part) {  // nibbles 0..3, then 4..7 of the dword
+      u32x4 vop[4];
+#pragma unroll
+      for (uint32_t p = 0; p < 4; ++p) {
+        const uint32_t even = r.v[2 * p][half], odd = r.v[2 * p + 1][half];
+        const uint32_t both =
+            __builtin_amdgcn_perm(odd, even, part ? 0x07060302u : 0x05040100u);
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i)
+          vop[i][p] = ((both >> (4 * i)) & 0x000F000Fu) ^ 0x43074308u;
+      }
+#pragma unroll
+      for (uint32_t i = 0; i < 4; ++i) {
+        const uint32_t m = 8 * half + 4 * part + i;
+        st.acc[m] = mfma_bf16(vop[i], pb, st.acc[m]);
+      }
+    }
+  }
+}
+
+#ifndef KVX_DECODE_DEPTH
+#define KVX_DECODE_DEPTH 2
+#endif
+#ifndef KVX_DECODE_WAVES
+#define KVX_DECODE_WAVES 2
+#endif
+constexpr uint32_t kDepth = KVX_DECODE_DEPTH;
+
+// Fixed-order merge of one q head's row over the splits of its (sequence, KV
+// head) (reference: common/paged_attention_tile.h:362-417).  One wave per row;
+// each lane owns four consecutive dimensions.
+__device__ __forceinline__ void merge_row(const float *__restrict__ partials,
+                                          const float *__restrict__ statistics,
+                                          uint16_t *__restrict__ out_row, uint64_t first_row,
+                                          uint32_t written, uint32_t G, uint32_t lane) {
+  float maximum = -INFINITY;
+  for (uint32_t s = 0; s < written; ++s)
+    maximum = fmaxf(maximum, load_global<float>(statistics + (first_row + uint64_t(s) * G) * 2));
+  f32x4 numerator = {0.0f, 0.0f, 0.0f, 0.0f};
+  float denominator = 0.0f;
+#pragma unroll 8
+  for (uint32_t s = 0; s < written; ++s) {  // split order is part of the contract
+    const uint64_t row = first_row + uint64_t(s) * G;
+    const f32x2 stat = load_global<f32x2>(statistics + row * 2);
+    const float weight = expf(__fsub_rn(stat[0], maximum));
+    const f32x4 part = load_global<f32x4>(partials + row * kD + 4 * lane);
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i)
+      numerator[i] = __fadd_rn(numerator[i], __fmul_rn(weight, part[i]));
+    denominator = __fadd_rn(denominator, __fmul_rn(weight, stat[1]));
+  }
+  u32x2 packed;
+#pragma unroll
+  for (uint32_t i = 0; i < 2; ++i) {
+    const float lo = denominator > 0.0f ? __fdiv_rn(numerator[2 * i], denominator) : 0.0f;
+    const float hi = denominator > 0.0f ? __fdiv_rn(numerator[2 * i + 1], denominator) : 0.0f;
+    packed[i] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
+  }
+  *reinterpret_cast<u32x2 *>(out_row + 4 * lane) = packed;
+}
+
+// grid (q head in group, KV head, lane).  Lanes whose pages fit one split were
+// written by the split kernel itself.
+__global__ __launch_bounds__(64) void decode_int4_merge_kernel(
+    uint16_t *__restrict__ output, const float *__restrict__ partials,
+    const float *__restrict__ statistics, DecodeArgs a) {
+  const uint32_t j = blockIdx.x, head = blockIdx.y;
+  const DecodeLane &l = a.lane[blockIdx.z];
+  const uint32_t pages = (l.committed + 1 + kPage - 1) / kPage;
+  const uint32_t per = (pages + l.split_count - 1) / l.split_count;
+  const uint32_t written = (pages + per - 1) / per;
+  if (written <= 1) return;
+  const uint32_t G = a.group;
+  uint16_t *out_row =
+      output + l.q_offset + uint64_t(head) * a.row_stride * G * kD + uint64_t(j) * kD;
+  merge_row(partials, statistics, out_row, l.row_base + uint64_t(head) * l.split_count * G + j,
+            written, G, threadIdx.x);
+}
+
+__global__ __launch_bounds__(64)
+__attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void decode_int4_kernel(
+    const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
+    float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
+  const uint32_t item = blockIdx.x, head = blockIdx.y;
+  uint32_t li = 0;
+  for (uint32_t i = 1; i < a.n_lanes; ++i)
+    if (item >= a.lane[i].first_item) li = i;
+  const DecodeLane &l = a.lane[li];
+  const uint32_t split = item - l.first_item;
+  if (split >= l.split_count) return;
+  const uint32_t visible = l.committed + 1;
+  const uint32_t pages = (visible + kPage - 1) / kPage;
+  const uint32_t per = (pages + l.split_count - 1) / l.split_count;
+  const uint32_t written = (pages + per - 1) / per;  // splits that own a page
+  const uint32_t begin = split * per;
+  if (begin >= pages) return;
+  const uint32_t end = min(pages, begin + per);
+
+  const uint32_t lane = threadIdx.x, t = lane & 15, g = lane >> 4;
+  const uint32_t H = a.kv_heads, G = a.group;
+  const uint32_t db = kPage * H * kRowBytes, sb = kPage * H * 4;
+  const RegionOffsets ro = region_offsets(a.kv.extent_pages, db, sb);
+  const float score_scale = default_score_scale(kD, l.score_scale);
+
+  // kDepth register sets rotate: a set is refilled with the page kDepth ahead as
+  // soon as its page has been consumed, so up to kDepth pages are in flight.
+  // The first pages are requested before anything else so their latency
+  // overlaps the query set-up.
+  PageRegs r[kDepth];
+#pragma unroll
+  for (uint32_t d = 0; d < kDepth; ++d)
+    if (begin + d < end)
+      load_page(r[d], l.table[begin + d], head, H, a.kv.offset, ro.key_scales, ro.values,
+                ro.value_scales, t, g);
+
+  // Queries of this KV head: [g][D] bf16, q head t < G.  Register kb holds the
+  // 8 dims of dword w = 16*(kb>>2) + 4g + (kb&3) of a key row in expansion
+  // order; odd dims are negated.  q_bias is the constant part of every score.
+  const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
+  __shared__ u32x4 q_lds[8 * 64];
+  float q_bias = 0.0f;
+  const uint16_t *q_row = q_head + uint64_t(t < G ? t : 0) * kD;
+#pragma unroll
+  for (uint32_t kb = 0; kb < 8; ++kb) {
+    const uint32_t w = 16 * (kb >> 2) + 4 * g + (kb & 3);
+    // dims 8w .. 8w+7 as four bf16 pairs, regrouped to (p, p+4) pairs
+    const u32x4 raw = load_global<u32x4>(q_row + 8 * w);
+    u32x4 q_reg;
+    q_reg[0] = __builtin_amdgcn_perm(raw[2], raw[0], 0x05040100u);
+    q_reg[1] = __builtin_amdgcn_perm(raw[2], raw[0], 0x07060302u) ^ 0x80008000u;
+    q_reg[2] = __builtin_amdgcn_perm(raw[3], raw[1], 0x05040100u);
+    q_reg[3] = __builtin_amdgcn_perm(raw[3], raw[1], 0x07060302u) ^ 0x80008000u;
+    if (t >= G) q_reg = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (uint32_t p = 0; p < 4; ++p) {
+      // even dims carry +136 q, odd dims (stored negated) -135 q = +135 stored
+      const float pair_sum =
+          __uint_as_float(q_reg[p] << 16) + __uint_as_float(q_reg[p] & 0xffff0000u);
+      q_bias = fmaf((p & 1) ? 135.0f : 136.0f, pair_sum, q_bias);
+    }
+    q_lds[kb * 64 + lane] = q_reg;
+  }
+  q_bias += __shfl_xor(q_bias, 16);
+  q_bias += __shfl_xor(q_bias, 32);
+
+  State st;
+#pragma unroll
+  for (uint32_t m = 0; m < 16; ++m) st.acc[m] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  st.row_max = -INFINITY;
+  st.row_sum = 0.0f;
+  st.bias = 0.0f;
+
+  for (uint32_t page = begin; page < end; page += kDepth) {
+#pragma unroll
+    for (uint32_t d = 0; d < kDepth; ++d) {
+      if (page + d < end) {
+        attend_page(r[d], q_lds, q_bias, score_scale, (page + d) * kPage, visible, lane, g, st);
+        if (page + d + kDepth < end)
+          load_page(r[d], l.table[page + d + kDepth], head, H, a.kv.offset, ro.key_scales,
+                    ro.values, ro.value_scales, t, g);
+      }
+    }
+  }
+
+  // Lanes of one q head hold disjoint tokens: combine their sums and the
+  // constant part, then take the constant part out of the accumulators.
+  float row_sum = st.row_sum, bias = st.bias;
+  row_sum += __shfl_xor(row_sum, 16);
+  row_sum += __shfl_xor(row_sum, 32);
+  bias += __shfl_xor(bias, 16);
+  bias += __shfl_xor(bias, 32);
+  uint16_t *out_head = output + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
+
+  if (written == 1) {
+    // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
+    if (t < G) {
+      const float denominator = row_sum;
+#pragma unroll
+      for (uint32_t rr = 0; rr < 4; ++rr)
+#pragma unroll
+        for (uint32_t m4 = 0; m4 < 4; ++m4) {
+          u32x2 packed;
+#pragma unroll
+          for (uint32_t i = 0; i < 2; ++i) {
+            const float lo = st.acc[4 * m4 + 2 * i][rr] - bias;
+            const float hi = st.acc[4 * m4 + 2 * i + 1][rr] - bias;
+            const float qlo = denominator > 0.0f ? __fdiv_rn(lo, denominator) : 0.0f;
+            const float qhi = denominator > 0.0f ? __fdiv_rn(hi, denominator) : 0.0f;
+            packed[i] = uint32_t(f32_to_bf16(qlo)) | (uint32_t(f32_to_bf16(qhi)) << 16);
+          }
+          *reinterpret_cast<u32x2 *>(out_head + uint64_t(t) * kD + 16 * (4 * g + rr) + 4 * m4) =
+              packed;
+        }
+    }
+    return;
+  }
+
+  const uint64_t head_row = l.row_base + uint64_t(head) * l.split_count * G;
+  if (t < G) {
+    const uint64_t row = head_row + uint64_t(split) * G + t;
+    float *out = partials + row * kD;
+#pragma unroll
+    for (uint32_t rr = 0; rr < 4; ++rr)
+#pragma unroll
+      for (uint32_t m4 = 0; m4 < 4; ++m4) {
+        f32x4 v;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) v[i] = st.acc[4 * m4 + i][rr] - bias;
+        *reinterpret_cast<f32x4 *>(out + 16 * (4 * g + rr) + 4 * m4) = v;
+      }
+    if (g == 0) {
+      statistics[row * 2] = st.row_max;
+      statistics[row * 2 + 1] = row_sum;
+    }
+  }
+}
+
+}  // namespace
+}  // namespace kvx
+
+using namespace kvx;
+
+// Runs decode attention (split kernel, then the merge of multi-split lanes) for int4 pages of head
+// dimension 256; returns 1 (declined) for shapes it does not cover so the
+// caller runs the format-generic kernels, 0 when enqueued, or a negative status.
+int kvx_decode_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_heads,
+                           const void *queries, void *output, const uint64_t *const *page_tables,
+                           const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                           void *workspace, hipStream_t stream) {
+  const kvx_layout &l = s->layout;
+  if (l.format != KVX_FMT_INT4 || l.head_dim != kD) return 1;
+  const uint32_t H = l.kv_heads, G = query_heads / H;
+  if (G > 16) return 1;
+  uint64_t total_rows = 0;
+  for (uint32_t i = 0; i < n_lanes; ++i) total_rows += uint64_t(lanes[i].split_count) * H * G;
+  float *partials = static_cast<float *>(workspace);
+  float *statistics = reinterpret_cast<float *>(
+      static_cast<uint8_t *>(workspace) + (total_rows * kD * sizeof(float) + 255) / 256 * 256);
+  uint64_t row_base = 0;
+  for (uint32_t first = 0; first < n_lanes; first += kLanes) {
+    DecodeArgs a{};
+    a.n_lanes = std::min(kLanes, n_lanes - first);
+    a.kv_heads = H;
+    a.group = G;
+    a.row_stride = row_stride;
+    a.kv = kv;
+    uint32_t items = 0;
+    for (uint32_t i = 0; i < a.n_lanes; ++i) {
+      const kvx_verify_params &p = lanes[first + i];
+      DecodeLane &dl = a.lane[i];
+      dl.table = page_tables[first + i];
+      dl.committed = p.committed_tokens;
+      dl.split_count = p.split_count;
+      dl.first_item = items;
+      dl.score_scale = p.score_scale != 0.0f ? p.score_scale : l.score_scale;
+      dl.row_base = row_base;
+      dl.q_offset = uint64_t(first + i) * H * row_stride * G * kD;
+      items += p.split_count;
+      row_base += uint64_t(p.split_count) * H * G;
+    }
+    uint32_t max_splits = 0;
+    for (uint32_t i = 0; i < a.n_lanes; ++i) max_splits = std::max(max_splits, a.lane[i].split_count);
+    hipLaunchKernelGGL(decode_int4_kernel, dim3(items, H), dim3(64), 0, stream,
+                       static_cast<const uint16_t *>(queries), static_cast<uint16_t *>(output),
+                       partials, statistics, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, "decode_int4_kernel");
+    if (max_splits > 1) {
+      hipLaunchKernelGGL(decode_int4_merge_kernel, dim3(G, H, a.n_lanes), dim3(64), 0, stream,
+                         static_cast<uint16_t *>(output), partials, statistics, a);
+      e = hipGetLastError();
+      if (e != hipSuccess) return hip_fail(e, "decode_int4_merge_kernel");
+    }
+  }
+  return 0;
 }

@@ -538,6 +538,10 @@ int dispatch_rows(uint32_t M, F &&f) {
   return fail(KVX_EINVAL, "tile holds more than 128 fused rows");
 }
 
+// Which attention phases the attend entries launch: bit 0 the split kernel,
+// bit 1 the merge.  Profiling harnesses clear a bit to time one kernel alone.
+uint32_t g_attend_phases = 3;
+
 int check_launch(const char *what) {
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? KVX_OK : hip_fail(e, what);
@@ -548,14 +552,18 @@ int check_launch(const char *what) {
 
 using namespace kvx;
 
-// Implemented by the int4 decode kernels; declines (returns 1) shapes it does
-// not cover so the generic tile takes them.
+// Implemented by the int4 decode kernels: enqueues the whole attention and
+// returns 0, or declines (returns 1) shapes it does not cover.
 int kvx_decode_int4_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t query_heads,
                            const void *queries, void *output, const uint64_t *const *page_tables,
                            const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
-                           void *workspace, uint64_t workspace_bytes, hipStream_t stream);
+                           void *workspace, hipStream_t stream);
+
+uint32_t kvx_attend_phases() { return kvx::g_attend_phases; }
 
 extern "C" {
+
+void kvx_debug_set_attend_phases(uint32_t phases) { kvx::g_attend_phases = phases & 3u; }
 
 int kv_append(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
               const void *chunk_values, const uint64_t *const *page_tables,
@@ -636,10 +644,11 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
                           const void *queries, void *output, const uint64_t *const *page_tables,
                           const kvx_verify_params *lanes, uint32_t n_lanes,
                           const uint32_t *row_masks, uint32_t row_stride, void *workspace,
-                          hipStream_t stream) {
+                          hipStream_t stream, uint32_t phases) {
   const kvx_layout &l = s->layout;
   const uint32_t H = l.kv_heads, G = query_heads / H, D = l.head_dim;
   const uint32_t capacity = lanes[0].row_capacity, M = capacity * G;
+  phases &= g_attend_phases;
   uint64_t total_rows = 0;
   for (uint32_t i = 0; i < n_lanes; ++i) total_rows += uint64_t(lanes[i].split_count) * H * M;
   float *partials = static_cast<float *>(workspace);
@@ -671,19 +680,23 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
       row_base += uint64_t(p.split_count) * H * M;
       max_splits = std::max(max_splits, p.split_count);
     }
-    int rc = dispatch_format(l.format, [&](auto fmt) {
-      return dispatch_rows(M, [&](auto maxm) {
-        hipLaunchKernelGGL((attend_split_kernel<decltype(fmt)::value, decltype(maxm)::value>),
-                           dim3(max_splits, H, a.n_lanes), dim3(kTileThreads), 0, stream,
-                           static_cast<const uint16_t *>(queries), partials, statistics, row_masks,
-                           a);
-        return check_launch("attend_split_kernel");
+    int rc = KVX_OK;
+    if (phases & 1u)
+      rc = dispatch_format(l.format, [&](auto fmt) {
+        return dispatch_rows(M, [&](auto maxm) {
+          hipLaunchKernelGGL((attend_split_kernel<decltype(fmt)::value, decltype(maxm)::value>),
+                             dim3(max_splits, H, a.n_lanes), dim3(kTileThreads), 0, stream,
+                             static_cast<const uint16_t *>(queries), partials, statistics,
+                             row_masks, a);
+          return check_launch("attend_split_kernel");
+        });
       });
-    });
     if (rc) return rc;
-    hipLaunchKernelGGL(attend_reduce_kernel, dim3(M, H, a.n_lanes), dim3(D), 0, stream, partials,
-                       statistics, static_cast<uint16_t *>(output), a);
-    if ((rc = check_launch("attend_reduce_kernel"))) return rc;
+    if (phases & 2u) {
+      hipLaunchKernelGGL(attend_reduce_kernel, dim3(M, H, a.n_lanes), dim3(D), 0, stream, partials,
+                         statistics, static_cast<uint16_t *>(output), a);
+      if ((rc = check_launch("attend_reduce_kernel"))) return rc;
+    }
   }
   return KVX_OK;
 }
@@ -703,7 +716,7 @@ int kv_attend_verify(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
                                workspace_bytes))
     return rc;
   return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks,
-                        row_stride, workspace, static_cast<hipStream_t>(stream));
+                        row_stride, workspace, static_cast<hipStream_t>(stream), 3);
 }
 
 int kv_attend_decode(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
@@ -722,11 +735,11 @@ int kv_attend_decode(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
                                workspace_bytes))
     return rc;
   const int fast = kvx_decode_int4_launch(s, kv, query_heads, queries, output, page_tables, lanes,
-                                          n_lanes, row_stride, workspace, workspace_bytes,
+                                          n_lanes, row_stride, workspace,
                                           static_cast<hipStream_t>(stream));
   if (fast <= 0) return fast;
   return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, nullptr,
-                        row_stride, workspace, static_cast<hipStream_t>(stream));
+                        row_stride, workspace, static_cast<hipStream_t>(stream), 3);
 }
 
 int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads,

@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libkvx.so")
+# KVX_LIB_PATH selects another build of the same library (profiling variants).
+LIB_PATH = os.environ.get("KVX_LIB_PATH") or os.path.join(HERE, "libkvx.so")
 
 INT8, BF16, INT4, FP8 = 1, 2, 3, 4
 KEYS, KEY_SCALES, VALUES, VALUE_SCALES = 0, 1, 2, 3
@@ -34,7 +35,7 @@ SYMBOLS = [
     "kvx_pool_acquire", "kvx_pool_retain", "kvx_pool_release", "kvx_pool_page_active",
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
     "kvx_pool_snapshot_get", "kv_append", "kv_attend_verify", "kv_attend_decode",
-    "kv_attend_prefill", "kv_compact_path",
+    "kv_attend_prefill", "kv_compact_path", "kvx_debug_set_attend_phases",
 ]
 
 
@@ -160,6 +161,7 @@ def _declare(L):
     L.kv_attend_decode.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, u32, vp, u64, vp]
     L.kv_attend_prefill.argtypes = [vp, u32, u32, vp, vp, vp, C.POINTER(PrefillParams), vp, u64, vp]
     L.kv_compact_path.argtypes = [vp, u32, vp, vp, u32, vp, vp, u32, vp]
+    L.kvx_debug_set_attend_phases.argtypes, L.kvx_debug_set_attend_phases.restype = [u32], None
 
 
 def check(rc):

@@ -79,7 +79,7 @@ def bf16_ulp_diff(a_bits, b_bits):
     return np.abs(key(a_bits) - key(b_bits))
 
 
-def check_attention(out_bits, want_bits, want_f32, rows_mask, tol, label=""):
+def check_attention(out_bits, want_bits, want_f32, rows_mask, tol, label="", matrix_core=False):
     """out_bits / want_bits: bf16 outputs (GPU, oracle); want_f32: the oracle's
     value before its final rounding.  rows_mask selects live rows (last axis D).
 
@@ -87,15 +87,29 @@ def check_attention(out_bits, want_bits, want_f32, rows_mask, tol, label=""):
     outputs both sides produce.  Against the oracle's fp32 value the bound is
     tol + 2e-3, because rounding a row to bf16 alone moves it by 1.6e-3 to
     2.0e-3 in this norm (the oracle's own bf16 output is that far from its
-    fp32 value), which would leave no room for anything else."""
+    fp32 value), which would leave no room for anything else.
+
+    matrix_core: kernels that sum q.k on the matrix cores cannot keep the
+    oracle's summation order, so a score can differ in its last bits and the
+    bf16 rounding of one probability can fall the other way.  When that
+    probability dominates its row, the row moves by up to half a bf16 step
+    (2e-3) on top of everything else.  For those kernels at least 99% of the
+    rows must meet tol and every row tol + 2e-3."""
     got = ko.bf16_to_f32(out_bits).reshape(out_bits.shape)
     want = ko.bf16_to_f32(want_bits).reshape(want_bits.shape)
     assert np.isfinite(got).all(), f"{label}: non-finite attention output"
     rel = T.rel_l2(got[rows_mask], want[rows_mask])
-    assert rel.max() <= tol, f"{label}: relative L2 vs oracle bf16 {rel.max():.3e} > {tol}"
+    flat = np.unravel_index(int(np.argmax(rel)), rel.shape)
+    worst = tuple(int(x) for x in np.argwhere(rows_mask)[flat[0]]) + tuple(int(x) for x in flat[1:])
+    hard = tol + 2e-3 if matrix_core else tol
+    assert rel.max() <= hard, (f"{label}: relative L2 vs oracle bf16 {rel.max():.3e} > {hard} "
+                               f"at row {worst}")
+    within = float((rel <= tol).mean())
+    assert within >= 0.99, f"{label}: only {within:.4f} of the rows are within {tol}"
     rel32 = T.rel_l2(got[rows_mask], want_f32[rows_mask])
     assert rel32.max() <= tol + 2e-3, f"{label}: relative L2 vs oracle fp32 {rel32.max():.3e}"
     ulps = bf16_ulp_diff(out_bits[rows_mask], want_bits[rows_mask])
-    return dict(rel_l2=float(rel.max()), rel_l2_fp32=float(rel32.max()),
+    return dict(rel_l2=float(rel.max()), rel_l2_mean=float(rel.mean()), rows_within_tol=within,
+                rel_l2_fp32=float(rel32.max()),
                 max_abs=float(np.abs(got[rows_mask] - want_f32[rows_mask]).max()),
                 exact=float((ulps == 0).mean()), max_ulp=int(ulps.max()))

@@ -73,7 +73,7 @@ def test_planning_rules_agree_with_the_oracle():
         committed, rows = rng.randrange(0, 262159), rng.choice([1, 8, 15, 16])
         assert L.kvx_verify_splits(committed, rows) == O.ko_verify_splits(committed, rows)
         pages = (committed + rows + 31) // 32
-        assert L.kvx_decode_splits(committed, rows) == min(max(1, (pages + 15) // 16), 128)
+        assert L.kvx_decode_splits(committed, rows) == min(max(1, (pages + 31) // 32), 128)
         tokens = rng.choice([0, 1, 8, 2048, 2049, rng.randrange(0, 2100)])
         stride = rng.choice([0, 31, 32, 2048, 2080, (tokens + 31) // 32 * 32])
         entries = rng.choice([0, (committed + tokens + 31) // 32, max((committed + tokens + 31) // 32 - 1, 0), 9000])
