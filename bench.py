@@ -43,6 +43,8 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=15.0,
                     help="CPU oracle budget; 0 skips the CPU baseline")
     ap.add_argument("--kernel-iters", type=int, default=20)
+    ap.add_argument("--uniform-context", type=int, default=0,
+                    help="give every sequence this context instead of U[512,32768] (experiments)")
     ap.add_argument("--pages-per-split", type=int, default=0,
                     help="override the library's decode split rule (experiments)")
     return ap.parse_args()
@@ -124,6 +126,8 @@ def main():
     pool_bytes = args.pool_gb * 1e9 if args.pool_gb > 0 else min(0.8 * free, 256e9)
     extents = max(1, int(pool_bytes // extent_bytes))
     contexts = rng.integers(512, 32769, BATCH)
+    if args.uniform_context:
+        contexts[:] = args.uniform_context
     total_steps = args.warmup + args.steps + args.kernel_iters + 8
     lane_pages = [(int(c) + total_steps + 31) // 32 for c in contexts]
     while extents * extent_pages < sum(lane_pages):

@@ -370,8 +370,15 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
       if (page + d < end) {
         attend_page(r[d], q_lds, q_bias, score_scale, (page + d) * kPage, visible, lane, g, st);
         if (page + d + kDepth < end)
+#ifdef KVX_PROBE_SAME_PAGE
+          // Measurement build: every page is the split's first one, so loads hit
+          // the caches and the time left is the kernel's own arithmetic.
+          load_page(r[d], l.table[begin], head, H, a.kv.offset, ro.key_scales, ro.values,
+                    ro.value_scales, t, g);
+#else
           load_page(r[d], l.table[page + d + kDepth], head, H, a.kv.offset, ro.key_scales,
                     ro.values, ro.value_scales, t, g);
+#endif
       }
     }
   }
