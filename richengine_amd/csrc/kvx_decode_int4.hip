@@ -52,6 +52,7 @@ constexpr uint32_t kD = 256;
 constexpr uint32_t kRowBytes = kD / 2;                // one token's packed row
 constexpr uint32_t kHeadSlabBytes = kPage * kRowBytes;  // 4 KiB per (head, page, tensor)
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr uint32_t kTableSlots = 1024;  // page entries of one split staged in LDS
 
 struct DecodeLane {
   const uint64_t *table;
@@ -141,6 +142,9 @@ struct State {
   float bias;      // constant part carried by acc, this lane's tokens only
 };
 
+// MASKED: the page may hold tokens at or past `visible` (only the last page of
+// a sequence can); other pages skip the per-token test.
+template <bool MASKED>
 __device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 *q_lds, float q_bias,
                                             float score_scale, uint32_t first_token,
                                             uint32_t visible, uint32_t lane, uint32_t g,
@@ -172,7 +176,7 @@ __device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 *q_ld
     const uint32_t tb = i >> 2, rr = i & 3;
     float v = s[tb][rr] * r.ks[tb][rr];
     v *= score_scale;
-    live[i] = first_token + 16 * tb + 4 * g + rr < visible;
+    live[i] = !MASKED || first_token + 16 * tb + 4 * g + rr < visible;
     score[i] = live[i] ? v : -INFINITY;
     local_max = fmaxf(local_max, score[i]);
   }
@@ -242,26 +246,50 @@ constexpr uint32_t kDepth = KVX_DECODE_DEPTH;
 
 // Fixed-order merge of one q head's row over the splits of its (sequence, KV
 // head) (reference: common/paged_attention_tile.h:362-417).  One wave per row;
-// each lane owns four consecutive dimensions.
+// each lane owns four consecutive dimensions.  The statistics of up to 64
+// splits are fetched at once, one split per lane, so the maximum and the
+// weights cost one load latency; the partial rows then stream with several
+// loads in flight.  Sums run in split order, which is part of the contract.
 __device__ __forceinline__ void merge_row(const float *__restrict__ partials,
                                           const float *__restrict__ statistics,
                                           uint16_t *__restrict__ out_row, uint64_t first_row,
                                           uint32_t written, uint32_t G, uint32_t lane) {
   float maximum = -INFINITY;
-  for (uint32_t s = 0; s < written; ++s)
-    maximum = fmaxf(maximum, load_global<float>(statistics + (first_row + uint64_t(s) * G) * 2));
+  for (uint32_t base = 0; base < written; base += 64) {
+    const uint32_t s = base + lane;
+    float m = s < written ? load_global<float>(statistics + (first_row + uint64_t(s) * G) * 2)
+                          : -INFINITY;
+#pragma unroll
+    for (uint32_t step = 32; step > 0; step >>= 1) m = fmaxf(m, __shfl_xor(m, step));
+    maximum = fmaxf(maximum, m);
+  }
   f32x4 numerator = {0.0f, 0.0f, 0.0f, 0.0f};
   float denominator = 0.0f;
-#pragma unroll 8
-  for (uint32_t s = 0; s < written; ++s) {  // split order is part of the contract
-    const uint64_t row = first_row + uint64_t(s) * G;
-    const f32x2 stat = load_global<f32x2>(statistics + row * 2);
-    const float weight = expf(__fsub_rn(stat[0], maximum));
-    const f32x4 part = load_global<f32x4>(partials + row * kD + 4 * lane);
+  for (uint32_t base = 0; base < written; base += 64) {
+    const uint32_t mine = base + lane;
+    f32x2 stat = {-INFINITY, 0.0f};
+    if (mine < written) stat = load_global<f32x2>(statistics + (first_row + uint64_t(mine) * G) * 2);
+    const float my_weight = expf(__fsub_rn(stat[0], maximum));
+    const float my_term = __fmul_rn(my_weight, stat[1]);
+    const uint32_t count = min(64u, written - base);
+    for (uint32_t i = 0; i < count; i += 8) {
+      f32x4 part[8];
 #pragma unroll
-    for (uint32_t i = 0; i < 4; ++i)
-      numerator[i] = __fadd_rn(numerator[i], __fmul_rn(weight, part[i]));
-    denominator = __fadd_rn(denominator, __fmul_rn(weight, stat[1]));
+      for (uint32_t u = 0; u < 8; ++u) {
+        const uint64_t row = first_row + uint64_t(base + min(i + u, count - 1)) * G;
+        part[u] = load_global<f32x4>(partials + row * kD + 4 * lane);
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < 8; ++u) {
+        if (i + u < count) {
+          const float weight = __shfl(my_weight, i + u);
+#pragma unroll
+          for (uint32_t c = 0; c < 4; ++c)
+            numerator[c] = __fadd_rn(numerator[c], __fmul_rn(weight, part[u][c]));
+          denominator = __fadd_rn(denominator, __shfl(my_term, i + u));
+        }
+      }
+    }
   }
   u32x2 packed;
 #pragma unroll
@@ -316,29 +344,57 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
   const RegionOffsets ro = region_offsets(a.kv.extent_pages, db, sb);
   const float score_scale = default_score_scale(kD, l.score_scale);
 
+  // Queries of this KV head: [g][D] bf16, q head t < G.  Their loads go out
+  // first; everything behind them returns later, so the wait for the queries
+  // leaves the page loads in flight.
+  const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
+  const uint16_t *q_row = q_head + uint64_t(t < G ? t : 0) * kD;
+  u32x4 q_raw[8];
+#pragma unroll
+  for (uint32_t kb = 0; kb < 8; ++kb)
+    q_raw[kb] = load_global<u32x4>(q_row + 8 * (16 * (kb >> 2) + 4 * g + (kb & 3)));
+
+  // The split's page entries (at most kTableSlots; the launcher declines longer
+  // splits) go through LDS and are read back with uniform LDS loads.  (Fetched from memory one by one they would be
+  // vector loads in the steady loop, and since loads return in order the wait for
+  // an entry would drain every page load in flight.)
+  __shared__ uint64_t table_lds[kTableSlots];
+  for (uint32_t i = lane; i < end - begin; i += 64)
+    table_lds[i] = load_global<uint64_t>(l.table + begin + i);
+  __syncthreads();
   // kDepth register sets rotate: a set is refilled with the page kDepth ahead as
   // soon as its page has been consumed, so up to kDepth pages are in flight.
-  // The first pages are requested before anything else so their latency
-  // overlaps the query set-up.
   PageRegs r[kDepth];
+  auto fill = [&](PageRegs &set, uint32_t slot) {
+#ifdef KVX_PROBE_SAME_PAGE
+    // Measurement build: every refill is the split's first page, so loads hit the
+    // caches and the time left is the kernel's own arithmetic.
+    slot = 0;
+#endif
+    // The empty asm statements pin the loads of one fill together and in place:
+    // moved up into the arithmetic that still reads the set they would need a
+    // second copy of its registers, and interleaved with another fill's loads
+    // they would make every wait cover both.
+    asm volatile("");
+    load_page(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values,
+              ro.value_scales, t, g);
+    asm volatile("");
+  };
+  // The first fills are unconditional too (a split shorter than kDepth pages
+  // loads its last page again): the steady loop must be entered with the same
+  // loads in flight, in the same order, as its own iterations leave behind.
 #pragma unroll
-  for (uint32_t d = 0; d < kDepth; ++d)
-    if (begin + d < end)
-      load_page(r[d], l.table[begin + d], head, H, a.kv.offset, ro.key_scales, ro.values,
-                ro.value_scales, t, g);
+  for (uint32_t d = 0; d < kDepth; ++d) fill(r[d], min(d, end - begin - 1));
 
-  // Queries of this KV head: [g][D] bf16, q head t < G.  Register kb holds the
-  // 8 dims of dword w = 16*(kb>>2) + 4g + (kb&3) of a key row in expansion
-  // order; odd dims are negated.  q_bias is the constant part of every score.
-  const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
+  // Register kb of the staged queries holds the 8 dims of dword
+  // w = 16*(kb>>2) + 4g + (kb&3) of a key row in expansion order; odd dims are
+  // negated.  q_bias is the constant part of every score.
   __shared__ u32x4 q_lds[8 * 64];
   float q_bias = 0.0f;
-  const uint16_t *q_row = q_head + uint64_t(t < G ? t : 0) * kD;
 #pragma unroll
   for (uint32_t kb = 0; kb < 8; ++kb) {
-    const uint32_t w = 16 * (kb >> 2) + 4 * g + (kb & 3);
     // dims 8w .. 8w+7 as four bf16 pairs, regrouped to (p, p+4) pairs
-    const u32x4 raw = load_global<u32x4>(q_row + 8 * w);
+    const u32x4 raw = q_raw[kb];
     u32x4 q_reg;
     q_reg[0] = __builtin_amdgcn_perm(raw[2], raw[0], 0x05040100u);
     q_reg[1] = __builtin_amdgcn_perm(raw[2], raw[0], 0x07060302u) ^ 0x80008000u;
@@ -364,22 +420,28 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
   st.row_sum = 0.0f;
   st.bias = 0.0f;
 
-  for (uint32_t page = begin; page < end; page += kDepth) {
+  // Steady state: every refill is unconditional, so the loop body is straight
+  // line code and the wait for a set counts exactly the loads issued after it;
+  // a refill under a branch would make each wait cover the newest loads too.
+  // The last page of the split is never consumed here, so no token test.
+  uint32_t page = begin;
+  for (; page + 2 * kDepth <= end; page += kDepth) {
 #pragma unroll
     for (uint32_t d = 0; d < kDepth; ++d) {
-      if (page + d < end) {
-        attend_page(r[d], q_lds, q_bias, score_scale, (page + d) * kPage, visible, lane, g, st);
-        if (page + d + kDepth < end)
-#ifdef KVX_PROBE_SAME_PAGE
-          // Measurement build: every page is the split's first one, so loads hit
-          // the caches and the time left is the kernel's own arithmetic.
-          load_page(r[d], l.table[begin], head, H, a.kv.offset, ro.key_scales, ro.values,
-                    ro.value_scales, t, g);
-#else
-          load_page(r[d], l.table[page + d + kDepth], head, H, a.kv.offset, ro.key_scales,
-                    ro.values, ro.value_scales, t, g);
-#endif
-      }
+      attend_page<false>(r[d], q_lds, q_bias, score_scale, (page + d) * kPage, visible, lane, g,
+                         st);
+      fill(r[d], page + d + kDepth - begin);
+    }
+  }
+  // Tail: at most 2 * kDepth - 1 pages are left, the first kDepth of them loaded.
+#pragma unroll
+  for (uint32_t k = 0; k < 2 * kDepth - 1; ++k) {
+    const uint32_t d = k % kDepth;
+    if (page + k < end) {
+      attend_page<true>(r[d], q_lds, q_bias, score_scale, (page + k) * kPage, visible, lane, g,
+                        st);
+      if (k + kDepth < 2 * kDepth - 1 && page + k + kDepth < end)
+        fill(r[d], page + k + kDepth - begin);
     }
   }
 
@@ -452,6 +514,11 @@ int kvx_decode_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   if (l.format != KVX_FMT_INT4 || l.head_dim != kD) return 1;
   const uint32_t H = l.kv_heads, G = query_heads / H;
   if (G > 16) return 1;
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    const uint32_t pages = lanes[i].committed_tokens / kPage + 1;
+    const uint32_t splits = std::max(1u, lanes[i].split_count);
+    if ((pages + splits - 1) / splits > kTableSlots) return 1;
+  }
   uint64_t total_rows = 0;
   for (uint32_t i = 0; i < n_lanes; ++i) total_rows += uint64_t(lanes[i].split_count) * H * G;
   float *partials = static_cast<float *>(workspace);
