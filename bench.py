@@ -45,6 +45,9 @@ def parse():
     ap.add_argument("--kernel-iters", type=int, default=20)
     ap.add_argument("--uniform-context", type=int, default=0,
                     help="give every sequence this context instead of U[512,32768] (experiments)")
+    ap.add_argument("--copy-calibration-pages", type=int, default=0,
+                    help="before the timed region copy this many pool pages once with "
+                         "kv_page_copy: a plain copy of known size to scale HBM counters by")
     ap.add_argument("--pages-per-split", type=int, default=0,
                     help="override the library's decode split rule (experiments)")
     return ap.parse_args()
@@ -100,6 +103,21 @@ def cpu_baseline(contexts, seed, budget_s):
     }
 
 
+def profiled_traffic():
+    """HBM bytes per launch of the split kernel on this workload, from the
+    committed counter summary (two rocprofv3 --pmc runs of this script, scaled by
+    what the same counters read for the library's page-copy kernel); None when
+    the summary is absent."""
+    path = os.path.join(ROOT, "profiles", "decode_int4_batch32_hbm_traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(float(line.split(":", 1)[1]))
+    except OSError:
+        pass
+    return None
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -135,8 +153,8 @@ def main():
     storage = kvx.Storage(LAYERS, H, D, kvx.INT4, extents * extent_pages, extent_pages, aligned=True)
     storage.allocate_all()
     pool_pages = extents * extent_pages
-    ids = (np.arange(pool_pages) if args.contiguous else rng.permutation(pool_pages))
-    ids = ids[:sum(lane_pages)].astype(np.uint32)
+    ids_all = (np.arange(pool_pages) if args.contiguous else rng.permutation(pool_pages))
+    ids = ids_all[:sum(lane_pages)].astype(np.uint32)
     tables, first = [], 0
     for n in lane_pages:
         tables.append(storage.table(ids[first:first + n]))
@@ -199,6 +217,15 @@ def main():
         for i in range(BATCH):
             committed[i] += 1
 
+    if args.copy_calibration_pages:
+        # Spare pages at the end of the shuffled order: read N pages, write N pages.
+        n = min(args.copy_calibration_pages, (pool_pages - sum(lane_pages)) // 2)
+        order = ids_all[sum(lane_pages):sum(lane_pages) + 2 * n]
+        storage.copy_pages([(int(order[i]), int(order[n + i])) for i in range(n)])
+        torch.cuda.synchronize()
+        print(f"copy calibration: {n} pages, {n * page_bytes} bytes read and as many written",
+              file=sys.stderr)
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -216,24 +243,34 @@ def main():
     ms_per_step = wall * 1e3 / args.steps
     value = kv_bytes / wall / 1e9
 
-    # ---- dominant kernel: decode attention (split + merge), one layer per launch
-    # Same inputs as a step's attention; events sit on the launch stream.
+    # ---- dominant kernel: the split kernel of decode attention, one layer of the
+    # batch per launch.  Same inputs as a step's attention; events sit on the
+    # launch stream.  The merge kernel and both together are timed the same way.
     _, vp = lane_params()
     vp_arr = (kvx.VerifyParams * BATCH)(*vp)
     launch_bytes = sum(c + 1 for c in committed) * BYTES_PER_TOKEN_LAYER
-    for layer in range(2):
-        L.kv_attend_decode(storage.h, layer, QH, queries.data_ptr(), output.data_ptr(), table_arr,
-                           vp_arr, BATCH, 1, workspace.data_ptr(), ws_bytes, stream)
-    torch.cuda.synchronize()
-    k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    k0.record()
-    for it in range(args.kernel_iters):
-        L.kv_attend_decode(storage.h, it % LAYERS, QH, queries.data_ptr(), output.data_ptr(),
-                           table_arr, vp_arr, BATCH, 1, workspace.data_ptr(), ws_bytes, stream)
-    k1.record()
-    torch.cuda.synchronize()
-    kernel_ms = k0.elapsed_time(k1) / args.kernel_iters
+
+    def time_attend(phases):
+        L.kvx_debug_set_attend_phases(phases)
+        for layer in range(2):
+            L.kv_attend_decode(storage.h, layer, QH, queries.data_ptr(), output.data_ptr(), table_arr,
+                               vp_arr, BATCH, 1, workspace.data_ptr(), ws_bytes, stream)
+        torch.cuda.synchronize()
+        k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        k0.record()
+        for it in range(args.kernel_iters):
+            L.kv_attend_decode(storage.h, it % LAYERS, QH, queries.data_ptr(), output.data_ptr(),
+                               table_arr, vp_arr, BATCH, 1, workspace.data_ptr(), ws_bytes, stream)
+        k1.record()
+        torch.cuda.synchronize()
+        L.kvx_debug_set_attend_phases(3)
+        return k0.elapsed_time(k1) / args.kernel_iters
+
+    both_ms = time_attend(3)
+    merge_ms = time_attend(2)
+    kernel_ms = time_attend(1)
     achieved = launch_bytes / (kernel_ms * 1e-3) / 1e9
+    traffic = profiled_traffic()
 
     result = {
         "metric": "int4 paged decode attn: KV GB/s (% HBM peak) + decode tokens/s, bs=32",
@@ -255,9 +292,11 @@ def main():
         "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-            "kernel": "decode_int4_kernel (paged decode attention split kernel; merge kernel timed with it), one layer of the batch per launch",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+            "kernel": "decode_int4_kernel (split kernel of paged decode attention), one layer of the batch per launch",
             "bytes_per_launch": launch_bytes, "ms_per_launch": round(kernel_ms, 4),
+            "merge_ms_per_launch": round(merge_ms, 4), "split_plus_merge_ms": round(both_ms, 4),
+            "split_plus_merge_gbs": round(launch_bytes / (both_ms * 1e-3) / 1e9, 1),
         },
     }
     storage.close()

@@ -503,6 +503,8 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
 
 using namespace kvx;
 
+uint32_t kvx_attend_phases();  // bit 0 = split kernel, bit 1 = merge kernel
+
 // Runs decode attention (split kernel, then the merge of multi-split lanes) for int4 pages of head
 // dimension 256; returns 1 (declined) for shapes it does not cover so the
 // caller runs the format-generic kernels, 0 when enqueued, or a negative status.
@@ -548,12 +550,16 @@ int kvx_decode_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
     }
     uint32_t max_splits = 0;
     for (uint32_t i = 0; i < a.n_lanes; ++i) max_splits = std::max(max_splits, a.lane[i].split_count);
-    hipLaunchKernelGGL(decode_int4_kernel, dim3(items, H), dim3(64), 0, stream,
-                       static_cast<const uint16_t *>(queries), static_cast<uint16_t *>(output),
-                       partials, statistics, a);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return hip_fail(e, "decode_int4_kernel");
-    if (max_splits > 1) {
+    const uint32_t phases = kvx_attend_phases();
+    hipError_t e = hipSuccess;
+    if (phases & 1u) {
+      hipLaunchKernelGGL(decode_int4_kernel, dim3(items, H), dim3(64), 0, stream,
+                         static_cast<const uint16_t *>(queries), static_cast<uint16_t *>(output),
+                         partials, statistics, a);
+      e = hipGetLastError();
+      if (e != hipSuccess) return hip_fail(e, "decode_int4_kernel");
+    }
+    if (max_splits > 1 && (phases & 2u)) {
       hipLaunchKernelGGL(decode_int4_merge_kernel, dim3(G, H, a.n_lanes), dim3(64), 0, stream,
                          static_cast<uint16_t *>(output), partials, statistics, a);
       e = hipGetLastError();
