@@ -33,6 +33,25 @@ def build(verbose=True, lib=LIB, extra_flags=(), tag=""):
     return lib
 
 
+HOST_TEST_SRC = os.path.join(ROOT, "tests", "cpp", "kvx_host_test.cpp")
+HOST_TEST_BIN = os.path.join(ROOT, "tests", "cpp", "kvx_host_test")
+
+
+def build_host_test(verbose=True):
+    """The C++ test of the host mirror (include/kvx.hpp): host code only, linked
+    against libkvx.so and the HIP runtime."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, "-x", "c++", "-std=c++17", "-O1", "-Wall", "-D__HIP_PLATFORM_AMD__",
+           "-I", os.path.join(ROOT, "include"), "-I", "/opt/rocm/include", HOST_TEST_SRC,
+           "-o", HOST_TEST_BIN, "-L", HERE, "-lkvx", "-L", "/opt/rocm/lib", "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN/../../richengine_amd"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return HOST_TEST_BIN
+
+
 if __name__ == "__main__":
     build()
+    build_host_test()
     print(LIB)

@@ -1,0 +1,328 @@
+// Tests of the C++ host mirror (include/kvx.hpp) written the way the
+// reference's own host tests are: known answers first, then behaviour.
+//   kvx_host_test host    -- no GPU needed (layout, planning, validation)
+//   kvx_host_test device  -- storage, pool, append, decode on the GPU
+// Known answers come from the reference's tests:
+//   dev/tests/engine/q8_paged_kv_test.cc:17-61 (byte accounting),
+//   dev/tests/engine/q8_flash_attention_metal_test.mm:53-56 (verify splits),
+//   dev/tests/engine/paged_attention_plan_test.mm:104-176 (plans, validation).
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <numeric>
+#include <vector>
+
+#include "kvx.hpp"
+
+using namespace kvx;
+using kv::Format;
+using kv::Layout;
+
+namespace {
+
+int failures = 0;
+#define EXPECT(condition)                                                          \
+  do {                                                                             \
+    if (!(condition)) {                                                            \
+      std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #condition);           \
+      ++failures;                                                                  \
+    }                                                                              \
+  } while (0)
+
+template <class Exception> bool throws(const std::function<void()> &f) {
+  try {
+    f();
+  } catch (const Exception &) {
+    return true;
+  } catch (...) {
+    return false;
+  }
+  return false;
+}
+
+void hip(hipError_t e) {
+  if (e != hipSuccess) {
+    std::printf("HIP error: %s\n", hipGetErrorString(e));
+    std::exit(2);
+  }
+}
+
+uint16_t bf16(float f) {
+  uint32_t bits;
+  std::memcpy(&bits, &f, 4);
+  return static_cast<uint16_t>((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+}
+float f32(uint16_t h) {
+  const uint32_t bits = uint32_t{h} << 16;
+  float f;
+  std::memcpy(&f, &bits, 4);
+  return f;
+}
+
+constexpr Layout kOracleLayout{16, 4, 256, Format::Int8};
+
+void testByteAccounting() {
+  const Layout bf16Layout{16, 4, 256, Format::BFloat16};
+  EXPECT(bf16Layout.valid());
+  EXPECT(bf16Layout.bytesPerModelPage() == 2'097'152);
+  EXPECT(bf16Layout.extentAlignmentPages() == 1);
+  EXPECT(bf16Layout.minimumExtentPages() == 32 && bf16Layout.maximumExtentPages() == 96);
+  EXPECT(bf16Layout.scaleBytesPerLayerPage() == 0);
+  const Layout compact{10, 2, 256, Format::BFloat16};
+  EXPECT(compact.bytesPerModelPage() == 655'360);
+  EXPECT(compact.extentAlignmentPages() == 2);
+  EXPECT(compact.minimumExtentPages() == 104 && compact.maximumExtentPages() == 306);
+  EXPECT(kOracleLayout.extentAlignmentPages() == 128);
+  EXPECT(kOracleLayout.minimumExtentPages() == 128 && kOracleLayout.maximumExtentPages() == 128);
+  EXPECT(kOracleLayout.extentPagesFor(127) == 0 && kOracleLayout.extentPagesFor(128) == 128 &&
+         kOracleLayout.extentPagesFor(1000) == 128);
+  const Layout compactInt8{10, 2, 256, Format::Int8};
+  EXPECT(compactInt8.bytesPerModelPage() == 332'800);
+  EXPECT(compactInt8.extentAlignmentPages() == 256);
+  EXPECT(compactInt8.minimumExtentPages() == 256 && compactInt8.maximumExtentPages() == 512);
+  EXPECT(compactInt8.extentPagesFor(255) == 0 && compactInt8.extentPagesFor(511) == 256);
+  EXPECT(compactInt8.extentPagesFor(10'240) == 512);
+  EXPECT(compactInt8.extentPagesFor(10'496) == 256);
+  EXPECT(bf16Layout.extentPagesFor(31) == 0 && bf16Layout.extentPagesFor(448) == 64 &&
+         bf16Layout.extentPagesFor(97) == 48);
+  EXPECT(!(Layout{16, 4, 256, static_cast<Format>(0)}.valid()));
+  EXPECT(kOracleLayout.bytesPerModelPage() == 1'064'960);
+  EXPECT(4608 * kOracleLayout.bytesPerModelPage() == 4'907'335'680ULL);
+  const Layout int4{16, 4, 256, Format::Int4};
+  EXPECT(int4.dataBytesPerLayerPage() == 16'384 && int4.scaleBytesPerLayerPage() == 512);
+  EXPECT(int4.bytesPerModelPage() == 540'672);
+  // The largest extent stays a whole number of alignment units, indexable in
+  // 14 bits and below 4 GiB.
+  EXPECT(int4.largestExtentPages() % int4.extentAlignmentPages() == 0);
+  EXPECT(int4.largestExtentPages() <= 16383);
+  EXPECT(uint64_t{int4.largestExtentPages()} * int4.bytesPerModelPage() < (1ULL << 32));
+}
+
+void testPlans() {
+  EXPECT(kv::verifyAttentionSplits(0) == 32);
+  EXPECT(kv::verifyAttentionSplits(16384) == 33);
+  EXPECT(kv::verifyAttentionSplits(131072) == 128);
+  const Layout layout{16, 4, 256, Format::Int8};
+  const auto one = ops::PagedAttention::prefillPlan(1, 24, layout);
+  EXPECT(one.splits == 32);
+  const auto full = ops::PagedAttention::prefillPlan(2048, 24, layout);
+  EXPECT(full.splits == 1);
+  // rows * D * 4 partial bytes and rows * 2 * 4 statistic bytes per slot
+  // (runtime/ops/PagedAttention.cpp:29-32); slots = tiles * kv heads * splits,
+  // rows per slot = 8 * group.
+  EXPECT(full.workspace.partialsBytes == uint64_t{256} * 4 * 1 * 48 * 256 * 4);
+  EXPECT(full.workspace.statisticsBytes == uint64_t{256} * 4 * 1 * 48 * 2 * 4);
+  const auto bound = ops::PagedAttention::prefillWorkspace(2048, 24, layout);
+  EXPECT(bound.partialsBytes >= full.workspace.partialsBytes);
+  const auto verify = ops::PagedAttention::verifyPlan(2, 24, layout, {0, 131072});
+  EXPECT(verify.laneSplits[0] == 32 && verify.laneSplits[1] == 128 && verify.splits == 128);
+  EXPECT(verify.rowCapacity == kv::kVerifyRows);
+  const auto decode = ops::PagedAttention::verifyPlan(2, 24, layout, {31, 32 * 64}, false, true);
+  EXPECT(decode.laneSplits[0] == 1 && decode.laneSplits[1] == 3 && decode.rowCapacity == 1);
+  EXPECT(throws<std::invalid_argument>([&] { (void)ops::PagedAttention::prefillPlan(0, 24, layout); }));
+  EXPECT(throws<std::invalid_argument>([&] { (void)ops::PagedAttention::prefillPlan(2049, 24, layout); }));
+  EXPECT(throws<std::invalid_argument>([&] { (void)ops::PagedAttention::prefillPlan(8, 25, layout); }));
+  EXPECT(throws<std::invalid_argument>(
+      [&] { (void)ops::PagedAttention::verifyPlan(1, 24, {16, 4, 256, Format::Float8E4M3}, {0}, true); }));
+}
+
+void testParams() {
+  const auto p = ops::PagedAttention::prefillParams(4093, 77, 96, 131);
+  EXPECT(p.committed_tokens == 4093 && p.chunk_tokens == 77 && p.chunk_stride == 96);
+  EXPECT(sizeof(kv::ChunkedPrefillParams) == 24 && sizeof(kv::PrefillAttentionParams) == 32 &&
+         sizeof(kv::VerifyAttentionParams) == 36);
+  // chunk_tokens 0 or past the stride, stride not a page multiple, table too
+  // short, context past the limit: each is refused before anything runs.
+  EXPECT(throws<std::invalid_argument>([] { (void)ops::PagedAttention::prefillParams(0, 0, 32, 1); }));
+  EXPECT(throws<std::invalid_argument>([] { (void)ops::PagedAttention::prefillParams(0, 33, 32, 2); }));
+  EXPECT(throws<std::invalid_argument>([] { (void)ops::PagedAttention::prefillParams(0, 8, 24, 1); }));
+  EXPECT(throws<std::invalid_argument>([] { (void)ops::PagedAttention::prefillParams(32, 1, 32, 1); }));
+  EXPECT(throws<std::invalid_argument>(
+      [] { (void)ops::PagedAttention::prefillParams(KVX_MAX_PHYSICAL_TOKENS, 1, 32, 1 << 14); }));
+  const auto v = ops::PagedAttention::verifyParams(100, 4);
+  EXPECT(v.chunk_tokens == kv::kVerifyRows && v.chunk_stride == kv::kVerifyChunkStride);
+  const auto t = ops::PagedAttention::verifyTreeParams(100, 4);
+  EXPECT(t.chunk_tokens == 15);
+}
+
+// ---- device ------------------------------------------------------------------
+
+void testStorageLifecycle() {
+  const Layout layout{2, 2, 64, Format::Int8};
+  kv::PageStorage storage(layout, 12, 4, /*aligned=*/false);
+  EXPECT(storage.pageCount() == 12 && storage.extentPages() == 4);
+  EXPECT(storage.bytesPerPage() == layout.bytesPerModelPage());
+  EXPECT(!storage.allocated(0));
+  EXPECT(storage.allocateExtent(0) == kv::AllocationFailure::None);
+  EXPECT(storage.allocated(3) && !storage.allocated(4));
+  EXPECT(throws<std::logic_error>([&] { (void)storage.allocateExtent(0); }));
+  EXPECT(throws<std::logic_error>([&] { storage.releaseExtent(1); }));
+  EXPECT(throws<std::out_of_range>([&] { (void)storage.allocateExtent(3); }));
+  // copying a page of an unallocated extent copies nothing
+  EXPECT(throws<std::logic_error>([&] { storage.copyPages({{0, 4}}); }));
+  // a refused allocation is a value and leaves nothing allocated
+  storage.setBudget(storage.extentBytes());
+  EXPECT(storage.allocateExtent(1) == kv::AllocationFailure::EngineBudget);
+  EXPECT(!storage.allocated(4) && storage.allocatedBytes() == storage.extentBytes());
+  storage.setBudget(0);
+  EXPECT(storage.allocateExtent(1) == kv::AllocationFailure::None);
+  // a new extent reads as zeros; page bytes round-trip; copies are byte-identical
+  std::vector<uint8_t> zero = storage.readPage(5);
+  EXPECT(std::all_of(zero.begin(), zero.end(), [](uint8_t b) { return b == 0; }));
+  std::vector<uint8_t> bytes(storage.bytesPerPage());
+  for (size_t i = 0; i < bytes.size(); ++i) bytes[i] = static_cast<uint8_t>(i * 131 + 7);
+  storage.writePage(1, bytes);
+  storage.copyPages({{1, 6}});
+  hip(hipDeviceSynchronize());
+  EXPECT(storage.readPage(6) == bytes && storage.readPage(1) == bytes);
+  // a destination that is also a source of the batch is refused
+  EXPECT(throws<std::invalid_argument>([&] { storage.copyPages({{1, 2}, {2, 3}}); }));
+  // entries decode to (extent base, index)
+  std::vector<uint64_t> table(3);
+  storage.entries({0, 3, 5}, 0, table.data());
+  EXPECT((table[0] & KVX_PAGE_INDEX_MASK) == 0 && (table[1] & KVX_PAGE_INDEX_MASK) == 3 &&
+         (table[2] & KVX_PAGE_INDEX_MASK) == 1);
+  EXPECT((table[0] & ~uint64_t{KVX_PAGE_INDEX_MASK}) == (table[1] & ~uint64_t{KVX_PAGE_INDEX_MASK}));
+  EXPECT((table[0] & ~uint64_t{KVX_PAGE_INDEX_MASK}) != (table[2] & ~uint64_t{KVX_PAGE_INDEX_MASK}));
+  storage.releaseExtent(1);
+  EXPECT(!storage.allocated(4));
+}
+
+void testPoolCompaction() {
+  const Layout layout{2, 2, 64, Format::Int4};
+  kv::PageStorage storage(layout, 12, 4, /*aligned=*/false);
+  engine::KvPool pool(storage, 4);
+  EXPECT(pool.freePageCount() == 4);
+  auto got = pool.acquirePages(10);
+  EXPECT(got.granted() && got.pages.size() == 10);
+  // every page gets its own content
+  std::vector<std::vector<uint8_t>> content(12);
+  for (uint32_t page : got.pages) {
+    content[page].resize(storage.bytesPerPage());
+    for (size_t i = 0; i < content[page].size(); ++i)
+      content[page][i] = static_cast<uint8_t>(page * 37 + i * 11);
+    storage.writePage(page, content[page]);
+  }
+  // leave one extent with a single held page and the others with room for it
+  std::vector<uint32_t> byExtent[3];
+  for (uint32_t page : got.pages) byExtent[page / 4].push_back(page);
+  uint32_t sparse = 0;
+  for (uint32_t e = 1; e < 3; ++e)
+    if (byExtent[e].size() < byExtent[sparse].size()) sparse = e;
+  std::vector<uint32_t> held;
+  for (uint32_t e = 0; e < 3; ++e)
+    for (size_t i = 0; i < byExtent[e].size(); ++i) {
+      const bool keep = e == sparse ? i == 0 : i + 1 < byExtent[e].size();
+      if (keep) held.push_back(byExtent[e][i]);
+      else pool.releasePage(byExtent[e][i], false);
+    }
+  const auto moves = pool.compactExtent();
+  hip(hipDeviceSynchronize());
+  EXPECT(!moves.empty() && moves.firstPage == sparse * 4);
+  for (uint32_t page : held) {
+    const uint32_t now = moves.follow(page);
+    EXPECT(pool.pageActive(now));
+    EXPECT(storage.readPage(now) == content[page]);
+    if (page / 4 == sparse) EXPECT(now / 4 != sparse);
+    else EXPECT(now == page);
+  }
+  EXPECT(pool.snapshot().extent_compactions == 1 && pool.snapshot().pages_moved == 1);
+  EXPECT(pool.reclaimEmptyExtents(false, 8) == storage.extentBytes());
+  EXPECT(throws<std::out_of_range>([&] { pool.retainPage(12, false); }));
+  EXPECT(throws<std::logic_error>([&] { pool.releasePage(moves.firstPage, false); }));
+}
+
+template <class T> T *toDevice(const std::vector<T> &host) {
+  T *device = nullptr;
+  hip(hipMalloc(&device, host.size() * sizeof(T)));
+  hip(hipMemcpy(device, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice));
+  return device;
+}
+
+// One appended token attended by one decode row: the probability is exactly 1,
+// so every query head's output is the dequantised value row, bf16(scale * code).
+void testAppendDecodeSingleToken() {
+  const Layout layout{2, 4, 256, Format::Int4};
+  const uint32_t H = 4, G = 6, D = 256, QH = H * G;
+  kv::PageStorage storage(layout, 8, 4, /*aligned=*/false);
+  engine::KvPool pool(storage, 8);
+  const auto got = pool.acquirePages(2);
+  std::vector<uint64_t> table(2);
+  storage.entries(got.pages, 0, table.data());
+  uint64_t *tableDevice = toDevice(table);
+  const uint64_t *tables[1] = {tableDevice};
+
+  std::vector<uint16_t> keys(H * 32 * D, 0), values(H * D * 32, 0), queries(H * G * D);
+  for (uint32_t h = 0; h < H; ++h)
+    for (uint32_t d = 0; d < D; ++d) {
+      keys[(h * 32 + 0) * D + d] = bf16(std::sin(0.37f * d + h));
+      // codes d % 15 - 7 with scale 0.5 * (h + 1): exactly representable
+      values[(h * D + d) * 32 + 0] = bf16(0.5f * (h + 1) * (float(d % 15) - 7.0f));
+    }
+  for (size_t i = 0; i < queries.size(); ++i) queries[i] = bf16(std::cos(0.11f * i));
+  uint16_t *keysDevice = toDevice(keys), *valuesDevice = toDevice(values), *queriesDevice = toDevice(queries);
+  uint16_t *outputDevice = nullptr;
+  hip(hipMalloc(&outputDevice, queries.size() * 2));
+
+  for (uint32_t layer = 0; layer < 2; ++layer) {
+    const auto chunk = ops::PagedAttention::prefillParams(0, 1, 32, 2);
+    ops::PagedAttention::addPrefillStore(nullptr, storage, layer, keysDevice, valuesDevice, tableDevice, chunk);
+    const auto plan = ops::PagedAttention::verifyPlan(1, QH, layout, {0}, false, true);
+    void *workspace = nullptr;
+    hip(hipMalloc(&workspace, plan.workspace.bytes() + 256));
+    ops::PagedVerifyBuffers buffers;
+    buffers.queries = queriesDevice;
+    buffers.output = outputDevice;
+    buffers.workspace = workspace;
+    buffers.workspaceBytes = plan.workspace.bytes() + 256;
+    buffers.pageTables = tables;
+    hip(hipMemset(outputDevice, 0xff, queries.size() * 2));
+    ops::PagedAttention::attend(nullptr, storage, layer, buffers, {chunk}, plan);
+    hip(hipDeviceSynchronize());
+    std::vector<uint16_t> output(queries.size());
+    hip(hipMemcpy(output.data(), outputDevice, output.size() * 2, hipMemcpyDeviceToHost));
+    uint32_t wrong = 0;
+    for (uint32_t h = 0; h < H; ++h)
+      for (uint32_t g = 0; g < G; ++g)
+        for (uint32_t d = 0; d < D; ++d)
+          wrong += f32(output[(h * G + g) * D + d]) != 0.5f * (h + 1) * (float(d % 15) - 7.0f);
+    EXPECT(wrong == 0);
+    hip(hipFree(workspace));
+  }
+  // an invalid chunk is refused before anything is enqueued
+  kv::ChunkedPrefillParams bad{0, 1, 32, 0, {}};
+  EXPECT(throws<std::invalid_argument>(
+      [&] { ops::PagedAttention::addPrefillStore(nullptr, storage, 0, keysDevice, valuesDevice, tableDevice, bad); }));
+  EXPECT(throws<std::out_of_range>([&] {  // a layer past the layout
+    ops::PagedAttention::addPrefillStore(nullptr, storage, 2, keysDevice, valuesDevice, tableDevice,
+                                         ops::PagedAttention::prefillParams(0, 1, 32, 2));
+  }));
+  hip(hipFree(tableDevice));
+  hip(hipFree(keysDevice));
+  hip(hipFree(valuesDevice));
+  hip(hipFree(queriesDevice));
+  hip(hipFree(outputDevice));
+}
+
+}  // namespace
+
+int main(int argc, char **argv) {
+  const std::string mode = argc > 1 ? argv[1] : "host";
+  testByteAccounting();
+  testPlans();
+  testParams();
+  if (mode == "device") {
+    testStorageLifecycle();
+    testPoolCompaction();
+    testAppendDecodeSingleToken();
+  }
+  if (failures) {
+    std::printf("kvx_host_test (%s): %d failure(s)\n", mode.c_str(), failures);
+    return 1;
+  }
+  std::printf("kvx_host_test (%s): ok\n", mode.c_str());
+  return 0;
+}
