@@ -178,6 +178,13 @@ typedef struct kvx_storage kvx_storage;
    page index allows (dev/tuning/HostKvExtents.hpp:158-169, test pools). */
 int kvx_storage_create(const kvx_layout *layout, uint32_t page_count, uint32_t extent_pages,
                        int aligned, kvx_storage **out);
+/* Storage with no memory behind its extents, for the page bookkeeping alone (pool,
+   prefix cache, sequences): the counterpart of the reference's deterministic test
+   storage (test::TestKvStorage, dev/tests/engine/TestKvPool.hpp).  Needs no GPU.  Allocation, release,
+   budget and kv_page_copy validation behave as usual; page and extent reads/writes, table
+   uploads and every hot-path entry answer KVX_ESTATE. */
+int kvx_storage_create_accounting(const kvx_layout *layout, uint32_t page_count,
+                                  uint32_t extent_pages, int aligned, kvx_storage **out);
 void kvx_storage_destroy(kvx_storage *storage);
 uint32_t kvx_storage_page_count(const kvx_storage *storage);
 uint32_t kvx_storage_extent_pages(const kvx_storage *storage);
@@ -251,6 +258,92 @@ int kvx_pool_compact_extent(kvx_pool *pool, const uint32_t *fixed, uint32_t n_fi
                             uint32_t *first_page, uint32_t *destinations,
                             uint32_t *moved_pages, void *stream);
 int kvx_pool_snapshot_get(const kvx_pool *pool, kvx_pool_snapshot *out);
+
+/* ---- prefix page cache: engine::KvCache, resident tier
+        (runtime/engine/cache/KvCache.hpp:40-241, KvCache.cpp:66-158, 227-283, 393-409, 480-484,
+        515-559).  Blocks are keyed by (parent block, the page's 32 tokens, image identity) and own
+        one prefix reference of their page in the pool.  The disk tier, recurrent states and
+        poisoning are outside the KV data path and have no counterpart. ---- */
+typedef struct kvx_prefix kvx_prefix;
+#define KVX_NO_PAGE 0xffffffffu
+int kvx_prefix_create(kvx_pool *pool, kvx_prefix **out);
+void kvx_prefix_destroy(kvx_prefix *prefix); /* gives every block's page back (KvCache::~KvCache) */
+/* KvCache::find: 1 with *block / *page when the exact key exists, else 0.  parent 0 = root. */
+int kvx_prefix_find(const kvx_prefix *prefix, uint64_t parent, const uint32_t *tokens,
+                    uint32_t n_tokens, uint64_t image_lo, uint64_t image_hi, uint64_t *block,
+                    uint32_t *page);
+/* KvCache::insert: existing content is returned as it is (*canonical_page may differ from
+   `page`).  KVX_EINVAL for a partial page or an unknown parent, KVX_ERANGE for a page past the
+   pool, KVX_ESTATE when the page already holds a block. */
+int kvx_prefix_insert(kvx_prefix *prefix, uint64_t parent, const uint32_t *tokens,
+                      uint32_t n_tokens, uint32_t page, uint64_t image_lo, uint64_t image_hi,
+                      uint64_t *block, uint32_t *canonical_page);
+int kvx_prefix_contains(const kvx_prefix *prefix, uint64_t block);
+uint64_t kvx_prefix_generation(const kvx_prefix *prefix);
+uint64_t kvx_prefix_block_count(const kvx_prefix *prefix);
+/* KvCache::chain, root first; *length = KvCache::chainLength. */
+int kvx_prefix_chain(const kvx_prefix *prefix, uint64_t block, uint64_t *blocks, uint32_t *pages,
+                     uint32_t capacity, uint32_t *length);
+int kvx_prefix_retain_active(kvx_prefix *prefix, uint64_t block);
+int kvx_prefix_release_active(kvx_prefix *prefix, uint64_t block);
+int kvx_prefix_touch(kvx_prefix *prefix, uint64_t block);
+/* KvCache::evictionCandidate: idle leaves, least recently used first; after = 0 starts the scan.
+   1 with *block, or 0 when there is no further candidate. */
+int kvx_prefix_eviction_candidate(const kvx_prefix *prefix, uint64_t after, uint64_t *block);
+/* KvCache::erase: KVX_ESTATE for a block with children or users. */
+int kvx_prefix_erase(kvx_prefix *prefix, uint64_t block);
+/* KvCache::followPages: after kvx_pool_compact_extent moved pages. */
+void kvx_prefix_follow_pages(kvx_prefix *prefix, uint32_t first_page, const uint32_t *destinations,
+                             uint32_t n);
+/* Cache::extendMatch (runtime/engine/cache/Cache.cpp:179-199), text-only prompts: the chain of
+   cached blocks that covers the prompt's leading whole pages, leaving at least one prompt token
+   unmatched.  Returns the number of pages looked up. */
+uint64_t kvx_prefix_match(const kvx_prefix *prefix, const uint32_t *prompt, uint64_t n_tokens,
+                          uint64_t *blocks, uint32_t capacity, uint32_t *matched);
+
+/* ---- per-sequence page lists: the Request records of engine::Cache
+        (runtime/engine/cache/Cache.cpp:143-166, 284-333, 381-413, 700-731, 748-785) ---- */
+typedef struct kvx_sequences kvx_sequences;
+typedef struct kvx_sequence_pages { /* Cache::pageTable -> PageTableView, plus the cached blocks */
+  const uint32_t *pages;
+  uint32_t page_count;
+  uint64_t revision;      /* bumped whenever a page id changed */
+  uint32_t first_changed; /* first logical page of the latest change */
+  const uint64_t *blocks;
+  uint32_t block_count;
+} kvx_sequence_pages;
+int kvx_sequences_create(kvx_pool *pool, kvx_prefix *prefix, kvx_sequences **out);
+void kvx_sequences_destroy(kvx_sequences *sequences);
+int kvx_sequence_begin(kvx_sequences *sequences, uint64_t id); /* Cache::beginRequest */
+int kvx_sequence_end(kvx_sequences *sequences, uint64_t id);   /* Cache::endRequest */
+/* Cache::restoreRequest for a resident chain: the sequence takes the chain of `last_block` as its
+   first pages (one active reference each) and becomes the block's user. */
+int kvx_sequence_restore(kvx_sequences *sequences, uint64_t id, uint64_t last_block);
+/* Cache::ensureTokens: pages for `tokens` tokens, or KVX_ENOMEM with nothing taken. */
+int kvx_sequence_ensure_tokens(kvx_sequences *sequences, uint64_t id, uint64_t tokens);
+/* Cache::publishCommittedBlocks: every newly full page becomes a block; where the content is
+   cached already the sequence moves to the canonical page (copy-free dedup) and the view's
+   revision / first_changed say so. */
+int kvx_sequence_publish(kvx_sequences *sequences, uint64_t id, const uint32_t *tokens,
+                         uint64_t n_tokens, uint32_t committed_tokens);
+int kvx_sequence_view(const kvx_sequences *sequences, uint64_t id, kvx_sequence_pages *out);
+/* Cache::compactExtent: kvx_pool_compact_extent, then blocks and sequences follow their pages. */
+int kvx_sequences_compact_extent(kvx_sequences *sequences, uint32_t *first_page,
+                                 uint32_t *destinations, uint32_t *moved_pages, void *stream);
+
+/* ---- producers of the verify inputs, host versions ---- */
+/* Ancestor bitmasks of a verify tree (kernel verify_input_tree_tokens,
+   runtime/metal/kernels/shared/embedding.metal:248-281): masks[row] = 1 << row | bits of its
+   ancestors.  parents[row] < row; KVX_TREE_NO_PARENT marks the root (row 0) and, on any later
+   row, a dead row, whose mask is 0.  KVX_EINVAL for rows > 32 or a parent that is not an
+   earlier row. */
+#define KVX_TREE_NO_PARENT 0xffffffffu
+int kvx_tree_masks(const uint32_t *parents, uint32_t rows, uint32_t *masks);
+/* The contract of a retained path (kernel decode_accept_tree,
+   runtime/metal/kernels/decode/sampling.metal:1927-1989): starts at row 0, rows strictly
+   increase, each row is a child of the one before.  1 valid, 0 not. */
+int kvx_tree_path_valid(const uint32_t *parents, uint32_t rows, const uint32_t *path,
+                        uint32_t retained);
 
 /* ---- the hot path ---- */
 

@@ -7,7 +7,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libkvx.so")
-SOURCES = ["kvx_host.cpp", "kvx_pool.cpp", "kvx_pool_abi.cpp", "kvx_kernels.hip",
+SOURCES = ["kvx_host.cpp", "kvx_pool.cpp", "kvx_pool_abi.cpp", "kvx_prefix.cpp",
+           "kvx_prefix_abi.cpp", "kvx_kernels.hip",
            "kvx_decode_int4.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
          # packed fp32 instructions stay off for every kernel of this library

@@ -223,8 +223,8 @@ uint64_t kvx_attend_workspace_bytes(const kvx_verify_params *lanes, uint32_t n, 
 }
 
 // --------------------------------------------------------------- storage ---
-int kvx_storage_create(const kvx_layout *layout, uint32_t page_count, uint32_t extent_pages,
-                       int aligned, kvx_storage **out) {
+static int storage_create(const kvx_layout *layout, uint32_t page_count, uint32_t extent_pages,
+                          int aligned, bool accounting, kvx_storage **out) {
   if (!out) return fail(KVX_EINVAL, "null output");
   *out = nullptr;
   if (!kvx_layout_valid(layout)) return fail(KVX_EINVAL, "KV page storage layout is invalid");
@@ -245,16 +245,25 @@ int kvx_storage_create(const kvx_layout *layout, uint32_t page_count, uint32_t e
   s->scale_bytes = uint32_t(kvx_layout_scale_bytes_per_layer_page(layout));
   s->extents.assign(page_count / extent_pages, nullptr);
   s->allocations.assign(page_count / extent_pages, nullptr);
-  if (hipGetDevice(&s->device) != hipSuccess) {
+  s->accounting = accounting;
+  if (!accounting && hipGetDevice(&s->device) != hipSuccess) {
     delete s;
     return fail(KVX_EDEVICE, "no HIP device: the paged KV path needs a GPU");
   }
   *out = s;
   return KVX_OK;
 }
+int kvx_storage_create(const kvx_layout *layout, uint32_t page_count, uint32_t extent_pages,
+                       int aligned, kvx_storage **out) {
+  return storage_create(layout, page_count, extent_pages, aligned, false, out);
+}
+int kvx_storage_create_accounting(const kvx_layout *layout, uint32_t page_count,
+                                  uint32_t extent_pages, int aligned, kvx_storage **out) {
+  return storage_create(layout, page_count, extent_pages, aligned, true, out);
+}
 void kvx_storage_destroy(kvx_storage *s) {
   if (!s) return;
-  (void)hipDeviceSynchronize();
+  if (!s->accounting) (void)hipDeviceSynchronize();
   for (void *raw : s->allocations)
     if (raw) (void)hipFree(raw);
   delete s;
@@ -282,6 +291,10 @@ int kvx_storage_allocate_extent(kvx_storage *s, uint32_t extent) {
   // Large allocations come back aligned far beyond that; a small test extent
   // may not, and is then allocated again with room to align inside it.
   constexpr uint64_t kAlign = uint64_t(KVX_PAGE_INDEX_MASK) + 1;
+  if (s->accounting) {  // a distinct, aligned, never dereferenced address per extent
+    s->extents[extent] = reinterpret_cast<void *>(uint64_t(extent + 1) << 32);
+    return KVX_OK;
+  }
   void *raw = nullptr;
   if (hipMalloc(&raw, bytes) != hipSuccess || !raw) {
     (void)hipGetLastError();
@@ -308,6 +321,10 @@ int kvx_storage_release_extent(kvx_storage *s, uint32_t extent) {
   if (extent >= s->extents.size()) return fail(KVX_ERANGE, "KV extent is past the pool");
   if (!s->extents[extent])
     return fail(KVX_ESTATE, "KV extent " + std::to_string(extent) + " is not allocated");
+  if (s->accounting) {
+    s->extents[extent] = nullptr;
+    return KVX_OK;
+  }
   // Kernels reach extents through page tables without retaining them: wait for
   // everything in flight before the memory goes away.
   KVX_HIP(hipDeviceSynchronize());
@@ -343,6 +360,7 @@ int kvx_storage_entries(const kvx_storage *s, const uint32_t *pages, uint32_t n,
 int kvx_storage_write_entries(const kvx_storage *s, const uint32_t *pages, uint32_t n,
                               uint32_t first, uint64_t *table_device, uint64_t capacity,
                               void *stream) {
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory");
   if (!table_device || capacity < n)
     return fail(KVX_ESTATE, "KV page table is missing or too small for its entries");
   std::vector<uint64_t> host(n);
@@ -356,6 +374,7 @@ int kvx_storage_write_entries(const kvx_storage *s, const uint32_t *pages, uint3
 }
 
 int kvx_storage_page_read(const kvx_storage *s, uint32_t page, void *host) {
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory");
   auto *out = static_cast<uint8_t *>(host);
   KVX_HIP(hipDeviceSynchronize());
   return for_each_span(s, page, [&](uint8_t *device, uint32_t bytes) -> int {
@@ -365,6 +384,7 @@ int kvx_storage_page_read(const kvx_storage *s, uint32_t page, void *host) {
   });
 }
 int kvx_storage_page_write(kvx_storage *s, uint32_t page, const void *host) {
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory");
   auto *in = static_cast<const uint8_t *>(host);
   KVX_HIP(hipDeviceSynchronize());
   return for_each_span(s, page, [&](uint8_t *device, uint32_t bytes) -> int {
@@ -374,6 +394,7 @@ int kvx_storage_page_write(kvx_storage *s, uint32_t page, const void *host) {
   });
 }
 static int extent_range(const kvx_storage *s, uint32_t extent, uint64_t offset, uint64_t bytes) {
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory");
   if (extent >= s->extents.size()) return fail(KVX_ERANGE, "KV extent is past the pool");
   if (!s->extents[extent]) return fail(KVX_ESTATE, "KV extent is not allocated");
   if (offset > s->extent_bytes() || bytes > s->extent_bytes() - offset)
@@ -395,6 +416,33 @@ int kvx_storage_extent_write(kvx_storage *s, uint32_t extent, uint64_t offset, u
   KVX_HIP(hipMemcpy(static_cast<uint8_t *>(s->extents[extent]) + offset, host, bytes,
                     hipMemcpyHostToDevice));
   return KVX_OK;
+}
+
+int kvx_tree_masks(const uint32_t *parents, uint32_t rows, uint32_t *masks) {
+  if (!parents || !masks || rows > 32) return kvx::fail(KVX_EINVAL, "verify tree has at most 32 rows");
+  for (uint32_t row = 0; row < rows; ++row) {
+    const uint32_t parent = parents[row];
+    if (parent != KVX_TREE_NO_PARENT && parent >= row)
+      return kvx::fail(KVX_EINVAL, "a tree row's parent must be an earlier row");
+    // Row 0 is the anchor; a later row without a parent is dead.
+    if (row && parent == KVX_TREE_NO_PARENT) {
+      masks[row] = 0;
+      continue;
+    }
+    uint32_t mask = 1u << row;
+    for (uint32_t above = parent; above != KVX_TREE_NO_PARENT; above = parents[above])
+      mask |= 1u << above;
+    masks[row] = mask;
+  }
+  return KVX_OK;
+}
+
+int kvx_tree_path_valid(const uint32_t *parents, uint32_t rows, const uint32_t *path,
+                        uint32_t retained) {
+  if (!parents || !path || !retained || path[0] != 0) return 0;
+  for (uint32_t i = 1; i < retained; ++i)
+    if (path[i] >= rows || path[i] <= path[i - 1] || parents[path[i]] != path[i - 1]) return 0;
+  return 1;
 }
 
 }  // extern "C"

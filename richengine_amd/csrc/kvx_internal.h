@@ -82,6 +82,7 @@ struct Storage {
   uint32_t scale_bytes = 0;
   uint64_t budget_bytes = 0;
   int device = 0;
+  bool accounting = false;  // no memory behind the extents: page bookkeeping only
   std::vector<void *> extents;      // 16 KiB-aligned base; nullptr while not allocated
   std::vector<void *> allocations;  // what hipMalloc returned for each extent
   uint64_t extent_bytes() const;

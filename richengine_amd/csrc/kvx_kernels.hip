@@ -571,6 +571,7 @@ int kv_append(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
               uint32_t verify_max_rows, void *stream) {
   if (!s || !chunk_keys || !chunk_values || !page_tables || !lanes || !n_lanes)
     return fail(KVX_EINVAL, "kv_append: null argument or no lanes");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
   kvx_kv_layer kv;
   if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
   if (verify_max_rows > KVX_TREE_NODES)
@@ -707,6 +708,7 @@ int kv_attend_verify(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
                      uint32_t row_stride, void *workspace, uint64_t workspace_bytes, void *stream) {
   if (!s || !queries || !output || !page_tables || !lanes || !n_lanes || !workspace)
     return fail(KVX_EINVAL, "kv_attend_verify: null argument or no lanes");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
   if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
   kvx_kv_layer kv;
   if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
@@ -725,6 +727,7 @@ int kv_attend_decode(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
                      void *workspace, uint64_t workspace_bytes, void *stream) {
   if (!s || !queries || !output || !page_tables || !lanes || !n_lanes || !workspace)
     return fail(KVX_EINVAL, "kv_attend_decode: null argument or no lanes");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
   if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
   kvx_kv_layer kv;
   if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
@@ -748,6 +751,7 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
                       void *stream) {
   if (!s || !queries || !output || !page_table || !params || !workspace)
     return fail(KVX_EINVAL, "kv_attend_prefill: null argument");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
   if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
   const kvx_layout &l = s->layout;
   kvx_kv_layer kv;
@@ -795,6 +799,7 @@ int kv_compact_path(const kvx_storage *s, uint32_t layer, const uint64_t *const 
                     uint32_t path_stride, void *stream) {
   if (!s || !page_tables || !lanes || !n_lanes || !retained_path || !retained_count)
     return fail(KVX_EINVAL, "kv_compact_path: null argument or no lanes");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
   const kvx_layout &l = s->layout;
   if (layer != UINT32_MAX && layer >= l.layers)
     return fail(KVX_ERANGE, "KV layer is outside the layout");
@@ -855,6 +860,7 @@ int kv_page_copy(kvx_storage *s, const kvx_page_copy *copies, uint32_t n, void *
         return fail(KVX_EINVAL, "two page copies share a destination");
     }
   }
+  if (s->accounting) return KVX_OK;  // nothing behind the pages: the bookkeeping is the copy
   const uint32_t span = std::max(s->data_bytes, s->scale_bytes);
   const uint32_t chunks = (span + kCopyChunk - 1) / kCopyChunk;
   for (uint32_t first = 0; first < n; first += kCopiesPerLaunch) {

@@ -35,6 +35,9 @@ struct kvx_pool {
   kvx_pool(kvx_storage *storage, uint32_t runway) : extents(storage), pool(extents, runway) {}
 };
 
+kvx::KvPool &kvx_pool_object(kvx_pool *pool) { return pool->pool; }
+void kvx_pool_set_stream(kvx_pool *pool, void *stream) { pool->extents.stream = stream; }
+
 extern "C" {
 
 int kvx_pool_create(kvx_storage *storage, uint32_t runway_pages, kvx_pool **out) {

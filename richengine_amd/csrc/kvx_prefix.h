@@ -1,0 +1,114 @@
+// Prefix reuse at whole-page granularity: the RAM tier of the reference's
+// engine::KvCache (runtime/engine/cache/KvCache.hpp:40-241, KvCache.cpp) and
+// the part of engine::Cache that keeps each sequence's page list
+// (runtime/engine/cache/Cache.cpp:143-166, 179-199, 284-333, 381-413, 700-731,
+// 748-785).  Blocks are keyed by (parent block, the page's 32 tokens, image
+// identity); a block owns one prefix reference of its page in the pool.  The
+// disk tier, recurrent states and poisoning of the reference are not part of
+// the KV data path and have no counterpart here.
+#pragma once
+
+#include <array>
+#include <cstdint>
+#include <map>
+#include <unordered_map>
+#include <utility>
+#include <vector>
+
+#include "kvx_pool.h"
+
+namespace kvx {
+
+class PrefixCache {
+public:
+  static constexpr uint32_t kNoPage = 0xffffffffu;
+  explicit PrefixCache(KvPool &pool) : pool_(pool), block_on_page_(pool.page_count(), 0) {}
+  ~PrefixCache();
+  PrefixCache(const PrefixCache &) = delete;
+  PrefixCache &operator=(const PrefixCache &) = delete;
+
+  // KvCache::find: true with the block and its page when the exact key exists.
+  bool find(uint64_t parent, const uint32_t *tokens, uint32_t n_tokens, uint64_t image_lo,
+            uint64_t image_hi, uint64_t *block, uint32_t *page) const;
+  // KvCache::insert: existing content is returned as it is.
+  int insert(uint64_t parent, const uint32_t *tokens, uint32_t n_tokens, uint32_t page,
+             uint64_t image_lo, uint64_t image_hi, uint64_t *block, uint32_t *canonical_page);
+  bool contains(uint64_t block) const { return blocks_.count(block) != 0; }
+  int chain_length(uint64_t block, uint32_t *length) const;
+  int chain(uint64_t block, std::vector<uint64_t> *blocks, std::vector<uint32_t> *pages) const;
+  int page_of(uint64_t block, uint32_t *page) const;
+  int retain_active(uint64_t block);
+  int release_active(uint64_t block);
+  int touch(uint64_t block);
+  // KvCache::evictionCandidate: idle resident leaves, oldest first; `after` = 0
+  // starts the scan.  False when there is none.
+  int eviction_candidate(uint64_t after, uint64_t *block, bool *found) const;
+  int erase(uint64_t block);
+  // KvCache::followPages after an extent compaction.
+  void follow_pages(const PageMoves &moves);
+  // Cache::extendMatch for text-only prompts: appends matched blocks, leaving at
+  // least one prompt token unmatched; returns how many pages were looked up.
+  uint64_t extend_match(std::vector<uint64_t> *blocks, const uint32_t *prompt, uint64_t n) const;
+  uint64_t generation() const { return generation_; }
+  uint64_t block_count() const { return blocks_.size(); }
+
+private:
+  struct Block {
+    uint64_t id = 0, parent = 0, index_hash = 0;
+    std::array<uint32_t, KVX_PAGE_TOKENS> tokens{};
+    uint64_t image_lo = 0, image_hi = 0;
+    uint32_t page = kNoPage, depth = 0, children = 0, active_users = 0;
+    uint64_t last_used = 0, listed_at = 0;
+    bool listed = false;
+  };
+  const Block *get(uint64_t id) const;
+  Block *get(uint64_t id);
+  void reindex(Block &b);
+
+  KvPool &pool_;
+  std::unordered_map<uint64_t, Block> blocks_;
+  std::unordered_multimap<uint64_t, uint64_t> index_;
+  std::map<std::pair<uint64_t, uint64_t>, uint64_t> leaves_;  // (last used, id) -> id
+  std::vector<uint64_t> block_on_page_;
+  uint64_t next_id_ = 1, clock_ = 0, generation_ = 0;
+};
+
+// One sequence's pages: engine::Cache's Request record.
+class SequenceCache {
+public:
+  SequenceCache(KvPool &pool, PrefixCache &prefix) : pool_(pool), prefix_(prefix) {}
+  ~SequenceCache();
+  int begin(uint64_t id);                                   // Cache::beginRequest
+  int end(uint64_t id);                                     // Cache::endRequest
+  int restore(uint64_t id, uint64_t last_block);            // Cache::restoreRequest, resident chain
+  int ensure_tokens(uint64_t id, uint64_t tokens);          // Cache::ensureTokens
+  int publish(uint64_t id, const uint32_t *tokens, uint64_t n_tokens, uint32_t committed);
+  struct View {                                             // Cache::pageTable
+    const uint32_t *pages;
+    uint32_t count;
+    uint64_t revision;
+    uint32_t first_changed;
+    const uint64_t *blocks;
+    uint32_t block_count;
+  };
+  int view(uint64_t id, View *out) const;
+  // Cache::compactExtent: empties one extent, re-points blocks and sequences.
+  int compact_extent(PageMoves *moves);
+
+private:
+  struct Sequence {
+    std::vector<uint32_t> pages;
+    std::vector<uint64_t> blocks;
+    uint64_t revision = 0;
+    uint32_t first_changed = 0;
+  };
+  static void changed(Sequence &s, uint32_t first) {
+    ++s.revision;
+    s.first_changed = first;
+  }
+  KvPool &pool_;
+  PrefixCache &prefix_;
+  std::unordered_map<uint64_t, Sequence> sequences_;
+};
+
+}  // namespace kvx

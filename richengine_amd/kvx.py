@@ -36,6 +36,14 @@ SYMBOLS = [
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
     "kvx_pool_snapshot_get", "kv_append", "kv_attend_verify", "kv_attend_decode",
     "kv_attend_prefill", "kv_compact_path", "kvx_debug_set_attend_phases",
+    "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
+    "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
+    "kvx_prefix_chain", "kvx_prefix_retain_active", "kvx_prefix_release_active",
+    "kvx_prefix_touch", "kvx_prefix_eviction_candidate", "kvx_prefix_erase",
+    "kvx_prefix_follow_pages", "kvx_prefix_match", "kvx_sequences_create",
+    "kvx_sequences_destroy", "kvx_sequence_begin", "kvx_sequence_end", "kvx_sequence_restore",
+    "kvx_sequence_ensure_tokens", "kvx_sequence_publish", "kvx_sequence_view",
+    "kvx_sequences_compact_extent", "kvx_tree_masks", "kvx_tree_path_valid",
 ]
 
 
@@ -69,6 +77,12 @@ class VerifyParams(C.Structure):
 
 class PageCopy(C.Structure):
     _fields_ = [("from_", C.c_uint32), ("to", C.c_uint32)]
+
+
+class SequencePages(C.Structure):
+    _fields_ = [("pages", C.POINTER(C.c_uint32)), ("page_count", C.c_uint32),
+                ("revision", C.c_uint64), ("first_changed", C.c_uint32),
+                ("blocks", C.POINTER(C.c_uint64)), ("block_count", C.c_uint32)]
 
 
 class PoolSnapshot(C.Structure):
@@ -127,6 +141,33 @@ def _declare(L):
     L.kvx_attend_workspace_bytes.argtypes = [vp, u32, u32, LP]
     L.kvx_attend_workspace_bytes.restype = u64
     L.kvx_storage_create.argtypes = [LP, u32, u32, i, C.POINTER(vp)]
+    L.kvx_storage_create_accounting.argtypes = [LP, u32, u32, i, C.POINTER(vp)]
+    PU32, PU64 = C.POINTER(u32), C.POINTER(u64)
+    L.kvx_prefix_create.argtypes = [vp, C.POINTER(vp)]
+    L.kvx_prefix_destroy.argtypes, L.kvx_prefix_destroy.restype = [vp], None
+    L.kvx_prefix_find.argtypes = [vp, u64, vp, u32, u64, u64, PU64, PU32]
+    L.kvx_prefix_insert.argtypes = [vp, u64, vp, u32, u32, u64, u64, PU64, PU32]
+    L.kvx_prefix_contains.argtypes = [vp, u64]
+    L.kvx_prefix_generation.argtypes, L.kvx_prefix_generation.restype = [vp], u64
+    L.kvx_prefix_block_count.argtypes, L.kvx_prefix_block_count.restype = [vp], u64
+    L.kvx_prefix_chain.argtypes = [vp, u64, vp, vp, u32, PU32]
+    for n in ("kvx_prefix_retain_active", "kvx_prefix_release_active", "kvx_prefix_touch",
+              "kvx_prefix_erase"):
+        getattr(L, n).argtypes = [vp, u64]
+    L.kvx_prefix_eviction_candidate.argtypes = [vp, u64, PU64]
+    L.kvx_prefix_follow_pages.argtypes, L.kvx_prefix_follow_pages.restype = [vp, u32, vp, u32], None
+    L.kvx_prefix_match.argtypes, L.kvx_prefix_match.restype = [vp, vp, u64, vp, u32, PU32], u64
+    L.kvx_sequences_create.argtypes = [vp, vp, C.POINTER(vp)]
+    L.kvx_sequences_destroy.argtypes, L.kvx_sequences_destroy.restype = [vp], None
+    L.kvx_sequence_begin.argtypes = [vp, u64]
+    L.kvx_sequence_end.argtypes = [vp, u64]
+    L.kvx_sequence_restore.argtypes = [vp, u64, u64]
+    L.kvx_sequence_ensure_tokens.argtypes = [vp, u64, u64]
+    L.kvx_sequence_publish.argtypes = [vp, u64, vp, u64, u32]
+    L.kvx_sequence_view.argtypes = [vp, u64, C.POINTER(SequencePages)]
+    L.kvx_sequences_compact_extent.argtypes = [vp, PU32, vp, PU32, vp]
+    L.kvx_tree_masks.argtypes = [vp, u32, vp]
+    L.kvx_tree_path_valid.argtypes = [vp, u32, vp, u32]
     L.kvx_storage_destroy.argtypes = [vp]
     L.kvx_storage_destroy.restype = None
     for n in ("kvx_storage_page_count", "kvx_storage_extent_pages"):
@@ -172,7 +213,7 @@ def check(rc):
 
 def _stream(stream):
     if stream is not None:
-        return C.c_void_p(stream)
+        return C.c_void_p(stream or None)  # 0 = the default stream
     import torch
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -192,11 +233,12 @@ class Storage:
     """Page storage in device extents (the reference's kv::PageStorage)."""
 
     def __init__(self, layers, kv_heads, head_dim, fmt, page_count, extent_pages, aligned=False,
-                 score_scale=0.0):
+                 score_scale=0.0, accounting=False):
         self.layout = Layout(layers, kv_heads, head_dim, fmt, score_scale)
+        self.accounting = accounting
         h = C.c_void_p()
-        check(lib().kvx_storage_create(C.byref(self.layout), page_count, extent_pages,
-                                       int(aligned), C.byref(h)))
+        create = lib().kvx_storage_create_accounting if accounting else lib().kvx_storage_create
+        check(create(C.byref(self.layout), page_count, extent_pages, int(aligned), C.byref(h)))
         self.h = h
         self.page_count, self.extent_pages = page_count, extent_pages
         self.extents = page_count // extent_pages
@@ -367,6 +409,8 @@ class Pool:
         fixed_arr = (C.c_uint32 * max(len(fixed), 1))(*fixed)
         first, moved = C.c_uint32(), C.c_uint32()
         dest = (C.c_uint32 * self.storage.extent_pages)()
+        if stream is None and self.storage.accounting:
+            stream = 0
         check(lib().kvx_pool_compact_extent(self.h, fixed_arr, len(fixed), C.byref(first), dest,
                                             C.byref(moved), _stream(stream)))
         if not moved.value:
@@ -377,3 +421,144 @@ class Pool:
         s = PoolSnapshot()
         check(lib().kvx_pool_snapshot_get(self.h, C.byref(s)))
         return s
+
+
+def _u32(values):
+    return (C.c_uint32 * max(len(values), 1))(*[int(v) for v in values])
+
+
+class Prefix:
+    """Prefix page cache, resident tier (the reference's engine::KvCache)."""
+
+    def __init__(self, pool):
+        h = C.c_void_p()
+        check(lib().kvx_prefix_create(pool.h, C.byref(h)))
+        self.h, self.pool = h, pool
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().kvx_prefix_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        self.close()
+
+    def find(self, parent, tokens, images=(0, 0)):
+        block, page = C.c_uint64(), C.c_uint32()
+        found = lib().kvx_prefix_find(self.h, parent, _u32(tokens), len(tokens), images[0],
+                                      images[1], C.byref(block), C.byref(page))
+        return (block.value, page.value) if found else None
+
+    def insert(self, parent, tokens, page, images=(0, 0)):
+        block, canonical = C.c_uint64(), C.c_uint32()
+        check(lib().kvx_prefix_insert(self.h, parent, _u32(tokens), len(tokens), page, images[0],
+                                      images[1], C.byref(block), C.byref(canonical)))
+        return block.value, canonical.value
+
+    def contains(self, block):
+        return bool(lib().kvx_prefix_contains(self.h, block))
+
+    def generation(self):
+        return lib().kvx_prefix_generation(self.h)
+
+    def block_count(self):
+        return lib().kvx_prefix_block_count(self.h)
+
+    def chain(self, block):
+        length = C.c_uint32()
+        check(lib().kvx_prefix_chain(self.h, block, None, None, 0, C.byref(length)))
+        blocks, pages = (C.c_uint64 * max(length.value, 1))(), (C.c_uint32 * max(length.value, 1))()
+        check(lib().kvx_prefix_chain(self.h, block, blocks, pages, length.value, C.byref(length)))
+        return list(blocks[:length.value]), list(pages[:length.value])
+
+    def retain_active(self, block):
+        return check(lib().kvx_prefix_retain_active(self.h, block))
+
+    def release_active(self, block):
+        return check(lib().kvx_prefix_release_active(self.h, block))
+
+    def touch(self, block):
+        return check(lib().kvx_prefix_touch(self.h, block))
+
+    def eviction_candidate(self, after=0):
+        block = C.c_uint64()
+        rc = lib().kvx_prefix_eviction_candidate(self.h, after, C.byref(block))
+        if rc < 0:
+            check(rc)
+        return block.value if rc else None
+
+    def erase(self, block):
+        return check(lib().kvx_prefix_erase(self.h, block))
+
+    def follow_pages(self, moves):
+        if moves:
+            dest = _u32(moves["dest"])
+            lib().kvx_prefix_follow_pages(self.h, moves["first"], dest, len(moves["dest"]))
+
+    def match(self, prompt):
+        capacity = max(len(prompt) // 32, 1)
+        blocks, matched = (C.c_uint64 * capacity)(), C.c_uint32()
+        hashed = lib().kvx_prefix_match(self.h, _u32(prompt), len(prompt), blocks, capacity,
+                                        C.byref(matched))
+        return list(blocks[:matched.value]), hashed
+
+
+class Sequences:
+    """Per-sequence page lists (the Request records of the reference's engine::Cache)."""
+
+    def __init__(self, pool, prefix):
+        h = C.c_void_p()
+        check(lib().kvx_sequences_create(pool.h, prefix.h, C.byref(h)))
+        self.h, self.pool, self.prefix = h, pool, prefix
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().kvx_sequences_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        self.close()
+
+    def begin(self, sequence):
+        return check(lib().kvx_sequence_begin(self.h, sequence))
+
+    def end(self, sequence):
+        return check(lib().kvx_sequence_end(self.h, sequence))
+
+    def restore(self, sequence, last_block):
+        return check(lib().kvx_sequence_restore(self.h, sequence, last_block))
+
+    def ensure_tokens(self, sequence, tokens):
+        return check(lib().kvx_sequence_ensure_tokens(self.h, sequence, tokens))
+
+    def publish(self, sequence, tokens, committed):
+        return check(lib().kvx_sequence_publish(self.h, sequence, _u32(tokens), len(tokens),
+                                                committed))
+
+    def view(self, sequence):
+        out = SequencePages()
+        check(lib().kvx_sequence_view(self.h, sequence, C.byref(out)))
+        return {"pages": [out.pages[i] for i in range(out.page_count)],
+                "revision": out.revision, "first_changed": out.first_changed,
+                "blocks": [out.blocks[i] for i in range(out.block_count)]}
+
+    def compact_extent(self, stream=None):
+        if stream is None and self.pool.storage.accounting:
+            stream = 0
+        first, moved = C.c_uint32(), C.c_uint32()
+        dest = (C.c_uint32 * self.pool.storage.extent_pages)()
+        check(lib().kvx_sequences_compact_extent(self.h, C.byref(first), dest, C.byref(moved),
+                                                 _stream(stream)))
+        if not moved.value:
+            return None
+        return {"first": first.value, "dest": list(dest), "moved": moved.value}
+
+
+def tree_masks(parents):
+    masks = (C.c_uint32 * max(len(parents), 1))()
+    check(lib().kvx_tree_masks(_u32(parents), len(parents), masks))
+    return list(masks[:len(parents)])
+
+
+def tree_path_valid(parents, path):
+    return bool(lib().kvx_tree_path_valid(_u32(parents), len(parents), _u32(path), len(path)))
