@@ -418,6 +418,10 @@ int kv_compact_path(const kvx_storage *storage, uint32_t layer,
    so a harness can time one kernel alone with events on its stream.  Outputs
    are only meaningful with both bits set. */
 void kvx_debug_set_attend_phases(uint32_t phases);
+/* Also no counterpart in the reference: how many attend calls of this process went to the
+   format-generic kernels and how many to the matrix-core (MFMA) kernels, so tests can tell
+   which path they measured. */
+void kvx_debug_attend_paths(uint64_t *generic_calls, uint64_t *matrix_core_calls);
 
 #ifdef __cplusplus
 }

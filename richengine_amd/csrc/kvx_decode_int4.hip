@@ -1,7 +1,9 @@
-// int4 paged decode attention for gfx950: the split kernel of kv_attend_decode
-// for packed-nibble pages with head dimension 256.
+// int4 paged attention for gfx950: the split and merge kernels of
+// kv_attend_decode, kv_attend_verify (chain and tree) and kv_attend_prefill for
+// packed-nibble pages with head dimension 256.
 //
-// One wave per (sequence, split, KV head) streams the split's pages once:
+// One wave per (sequence or prefill tile, split, KV head, block of 16 fused
+// query rows) streams the split's pages once:
 // coalesced 128-bit key loads and 64-bit value loads, the page's fp32 scales,
 // bf16 MFMA (16x16x32) for q.k and p.v with the GQA group as the 16-wide N
 // side, page-granular online softmax in registers.  The arithmetic follows the
@@ -56,7 +58,9 @@ constexpr uint32_t kTableSlots = 1024;  // page entries of one split staged in L
 
 struct DecodeLane {
   const uint64_t *table;
+  const uint32_t *masks;  // tree verify: ancestor bitmask per row; null = causal chain
   uint32_t committed;
+  uint32_t active_rows;   // query rows attended (1 for decode)
   uint32_t split_count;
   uint32_t first_item;  // first (lane, split) work item of this lane
   float score_scale;
@@ -69,7 +73,23 @@ struct DecodeArgs {
   uint32_t kv_heads;
   uint32_t group;
   uint32_t row_stride;
+  uint32_t fused_rows;  // row capacity x group: fused query rows per (lane, KV head)
   kvx_kv_layer kv;
+};
+
+// Which tokens one fused query row (an MFMA column) may see
+// (reference: common/paged_attention_tile.h:141-143).
+struct Sight {
+  uint32_t committed;
+  uint32_t visible;  // committed + active rows
+  uint32_t limit;    // chain: first token the row may not see
+  uint32_t mask;     // tree: the row's ancestor bits over tokens committed + i
+  bool tree;
+  __device__ __forceinline__ bool sees(uint32_t token) const {
+    if (tree)
+      return token < committed || (token < visible && ((mask >> ((token - committed) & 31u)) & 1u));
+    return token < limit;
+  }
 };
 
 // What one lane holds of one page.
@@ -142,12 +162,12 @@ struct State {
   float bias;      // constant part carried by acc, this lane's tokens only
 };
 
-// MASKED: the page may hold tokens at or past `visible` (only the last page of
-// a sequence can); other pages skip the per-token test.
+// MASKED: the page may hold tokens some row does not see (only the last two
+// pages of a sequence can); other pages skip the per-token test.
 template <bool MASKED>
 __device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 *q_lds, float q_bias,
                                             float score_scale, uint32_t first_token,
-                                            uint32_t visible, uint32_t lane, uint32_t g,
+                                            const Sight &sight, uint32_t lane, uint32_t g,
                                             State &st) {
 #ifdef KVX_PROBE_STREAM_ONLY
   // Measurement build: consume every loaded register with almost no arithmetic,
@@ -176,19 +196,23 @@ __device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 *q_ld
     const uint32_t tb = i >> 2, rr = i & 3;
     float v = s[tb][rr] * r.ks[tb][rr];
     v *= score_scale;
-    live[i] = !MASKED || first_token + 16 * tb + 4 * g + rr < visible;
+    live[i] = !MASKED || sight.sees(first_token + 16 * tb + 4 * g + rr);
     score[i] = live[i] ? v : -INFINITY;
     local_max = fmaxf(local_max, score[i]);
   }
   local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
   local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
   const float next_max = fmaxf(st.row_max, local_max);
-  const float rescale = __builtin_amdgcn_exp2f((st.row_max - next_max) * kLog2e);
+  // A row that has seen nothing yet keeps -inf; its rescale is 1, not exp(nan).
+  const float rescale = next_max == st.row_max
+                            ? 1.0f
+                            : __builtin_amdgcn_exp2f((st.row_max - next_max) * kLog2e);
   float weight[8], page_sum = 0.0f;
 #pragma unroll
   for (uint32_t i = 0; i < 8; ++i) {
     // The difference first, so the page's maximum gets exactly 1.
-    const float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
+    float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
+    if (MASKED) p = live[i] ? p : 0.0f;
     page_sum += p;
     const float w = p * r.vs[i >> 2][i & 3];
     weight[i] = live[i] ? w : 0.0f;
@@ -301,22 +325,26 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ partials,
   *reinterpret_cast<u32x2 *>(out_row + 4 * lane) = packed;
 }
 
-// grid (q head in group, KV head, lane).  Lanes whose pages fit one split were
+// grid (fused query row, KV head, lane).  Lanes whose pages fit one split were
 // written by the split kernel itself.
 __global__ __launch_bounds__(64) void decode_int4_merge_kernel(
     uint16_t *__restrict__ output, const float *__restrict__ partials,
     const float *__restrict__ statistics, DecodeArgs a) {
   const uint32_t j = blockIdx.x, head = blockIdx.y;
   const DecodeLane &l = a.lane[blockIdx.z];
-  const uint32_t pages = (l.committed + 1 + kPage - 1) / kPage;
+  const uint32_t pages = (l.committed + l.active_rows + kPage - 1) / kPage;
   const uint32_t per = (pages + l.split_count - 1) / l.split_count;
   const uint32_t written = (pages + per - 1) / per;
   if (written <= 1) return;
-  const uint32_t G = a.group;
+  const uint32_t G = a.group, M = a.fused_rows;
   uint16_t *out_row =
       output + l.q_offset + uint64_t(head) * a.row_stride * G * kD + uint64_t(j) * kD;
-  merge_row(partials, statistics, out_row, l.row_base + uint64_t(head) * l.split_count * G + j,
-            written, G, threadIdx.x);
+  if (j / G >= l.active_rows) {  // rows past the live ones read as zeros
+    *reinterpret_cast<u32x2 *>(out_row + 4 * threadIdx.x) = u32x2{0u, 0u};
+    return;
+  }
+  merge_row(partials, statistics, out_row, l.row_base + uint64_t(head) * l.split_count * M + j,
+            written, M, threadIdx.x);
 }
 
 __global__ __launch_bounds__(64)
@@ -330,7 +358,7 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
   const DecodeLane &l = a.lane[li];
   const uint32_t split = item - l.first_item;
   if (split >= l.split_count) return;
-  const uint32_t visible = l.committed + 1;
+  const uint32_t visible = l.committed + l.active_rows;
   const uint32_t pages = (visible + kPage - 1) / kPage;
   const uint32_t per = (pages + l.split_count - 1) / l.split_count;
   const uint32_t written = (pages + per - 1) / per;  // splits that own a page
@@ -339,16 +367,26 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
   const uint32_t end = min(pages, begin + per);
 
   const uint32_t lane = threadIdx.x, t = lane & 15, g = lane >> 4;
-  const uint32_t H = a.kv_heads, G = a.group;
+  const uint32_t H = a.kv_heads, G = a.group, M = a.fused_rows;
+  // This wave's MFMA columns are fused rows 16 z .. 16 z + 15 of the tile; a fused
+  // row is (query row, head in group) = (m / G, m % G).
+  const uint32_t m = 16 * blockIdx.z + t, query_row = m / G;
+  const bool in_tile = m < M, live_row = in_tile && query_row < l.active_rows;
+  Sight sight;
+  sight.committed = l.committed;
+  sight.visible = visible;
+  sight.limit = live_row ? min(visible, l.committed + min(query_row, l.active_rows - 1) + 1) : visible;
+  sight.tree = live_row && l.masks != nullptr;
+  sight.mask = sight.tree ? l.masks[query_row] : 0u;
   const uint32_t db = kPage * H * kRowBytes, sb = kPage * H * 4;
   const RegionOffsets ro = region_offsets(a.kv.extent_pages, db, sb);
   const float score_scale = default_score_scale(kD, l.score_scale);
 
-  // Queries of this KV head: [g][D] bf16, q head t < G.  Their loads go out
+  // Queries of this KV head: [row][g][D] bf16, fused row m.  Their loads go out
   // first; everything behind them returns later, so the wait for the queries
-  // leaves the page loads in flight.
+  // leaves the page loads in flight.  Columns without a live row carry zeros.
   const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
-  const uint16_t *q_row = q_head + uint64_t(t < G ? t : 0) * kD;
+  const uint16_t *q_row = q_head + uint64_t(live_row ? m : 0) * kD;
   u32x4 q_raw[8];
 #pragma unroll
   for (uint32_t kb = 0; kb < 8; ++kb)
@@ -400,7 +438,7 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
     q_reg[1] = __builtin_amdgcn_perm(raw[2], raw[0], 0x07060302u) ^ 0x80008000u;
     q_reg[2] = __builtin_amdgcn_perm(raw[3], raw[1], 0x05040100u);
     q_reg[3] = __builtin_amdgcn_perm(raw[3], raw[1], 0x07060302u) ^ 0x80008000u;
-    if (t >= G) q_reg = u32x4{0u, 0u, 0u, 0u};
+    if (!live_row) q_reg = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
     for (uint32_t p = 0; p < 4; ++p) {
       // even dims carry +136 q, odd dims (stored negated) -135 q = +135 stored
@@ -428,7 +466,7 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
   for (; page + 2 * kDepth <= end; page += kDepth) {
 #pragma unroll
     for (uint32_t d = 0; d < kDepth; ++d) {
-      attend_page<false>(r[d], q_lds, q_bias, score_scale, (page + d) * kPage, visible, lane, g,
+      attend_page<false>(r[d], q_lds, q_bias, score_scale, (page + d) * kPage, sight, lane, g,
                          st);
       fill(r[d], page + d + kDepth - begin);
     }
@@ -438,7 +476,7 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
   for (uint32_t k = 0; k < 2 * kDepth - 1; ++k) {
     const uint32_t d = k % kDepth;
     if (page + k < end) {
-      attend_page<true>(r[d], q_lds, q_bias, score_scale, (page + k) * kPage, visible, lane, g,
+      attend_page<true>(r[d], q_lds, q_bias, score_scale, (page + k) * kPage, sight, lane, g,
                         st);
       if (k + kDepth < 2 * kDepth - 1 && page + k + kDepth < end)
         fill(r[d], page + k + kDepth - begin);
@@ -456,8 +494,9 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
 
   if (written == 1) {
     // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
-    if (t < G) {
-      const float denominator = row_sum;
+    // Rows of the tile past the live ones read as zeros (row_sum is 0 there).
+    if (in_tile) {
+      const float denominator = live_row ? row_sum : 0.0f;
 #pragma unroll
       for (uint32_t rr = 0; rr < 4; ++rr)
 #pragma unroll
@@ -471,16 +510,16 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
             const float qhi = denominator > 0.0f ? __fdiv_rn(hi, denominator) : 0.0f;
             packed[i] = uint32_t(f32_to_bf16(qlo)) | (uint32_t(f32_to_bf16(qhi)) << 16);
           }
-          *reinterpret_cast<u32x2 *>(out_head + uint64_t(t) * kD + 16 * (4 * g + rr) + 4 * m4) =
+          *reinterpret_cast<u32x2 *>(out_head + uint64_t(m) * kD + 16 * (4 * g + rr) + 4 * m4) =
               packed;
         }
     }
     return;
   }
 
-  const uint64_t head_row = l.row_base + uint64_t(head) * l.split_count * G;
-  if (t < G) {
-    const uint64_t row = head_row + uint64_t(split) * G + t;
+  const uint64_t head_row = l.row_base + uint64_t(head) * l.split_count * M;
+  if (live_row) {
+    const uint64_t row = head_row + uint64_t(split) * M + m;
     float *out = partials + row * kD;
 #pragma unroll
     for (uint32_t rr = 0; rr < 4; ++rr)
@@ -505,27 +544,36 @@ using namespace kvx;
 
 uint32_t kvx_attend_phases();  // bit 0 = split kernel, bit 1 = merge kernel
 
-// Runs decode attention (split kernel, then the merge of multi-split lanes) for int4 pages of head
-// dimension 256; returns 1 (declined) for shapes it does not cover so the
-// caller runs the format-generic kernels, 0 when enqueued, or a negative status.
-int kvx_decode_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_heads,
+// Runs paged attention (split kernel, then the merge of multi-split lanes) for
+// int4 pages of head dimension 256; returns 1 (declined) for shapes it does not
+// cover so the caller runs the format-generic kernels, 0 when enqueued, or a
+// negative status.  Lane i reads its queries and writes its rows at element
+// offset i * lane_stride; the rows of one KV head lie row_stride * group * 256
+// elements apart.  row_masks: null, or one ancestor bitmask per (lane, row of
+// capacity).  Every lane has the row capacity of the first.
+int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_heads,
                            const void *queries, void *output, const uint64_t *const *page_tables,
-                           const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
-                           void *workspace, hipStream_t stream) {
+                           const kvx_verify_params *lanes, uint32_t n_lanes,
+                           const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
+                           void *workspace, uint64_t workspace_bytes, hipStream_t stream) {
   const kvx_layout &l = s->layout;
   if (l.format != KVX_FMT_INT4 || l.head_dim != kD) return 1;
   const uint32_t H = l.kv_heads, G = query_heads / H;
-  if (G > 16) return 1;
-  for (uint32_t i = 0; i < n_lanes; ++i) {
-    const uint32_t pages = lanes[i].committed_tokens / kPage + 1;
-    const uint32_t splits = std::max(1u, lanes[i].split_count);
-    if ((pages + splits - 1) / splits > kTableSlots) return 1;
-  }
+  const uint32_t capacity = lanes[0].row_capacity, M = capacity * G;
+  if (G > 16 || !capacity || capacity > KVX_TREE_NODES) return 1;
   uint64_t total_rows = 0;
-  for (uint32_t i = 0; i < n_lanes; ++i) total_rows += uint64_t(lanes[i].split_count) * H * G;
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    const kvx_verify_params &p = lanes[i];
+    if (p.row_capacity != capacity || !p.active_rows || p.active_rows > capacity) return 1;
+    const uint32_t pages = (p.committed_tokens + p.active_rows + kPage - 1) / kPage;
+    const uint32_t splits = std::max(1u, p.split_count);
+    if ((pages + splits - 1) / splits > kTableSlots) return 1;
+    total_rows += uint64_t(p.split_count) * H * M;
+  }
+  const uint64_t statistics_offset = (total_rows * kD * sizeof(float) + 255) / 256 * 256;
+  if (workspace_bytes < statistics_offset + total_rows * 2 * sizeof(float)) return 1;
   float *partials = static_cast<float *>(workspace);
-  float *statistics = reinterpret_cast<float *>(
-      static_cast<uint8_t *>(workspace) + (total_rows * kD * sizeof(float) + 255) / 256 * 256);
+  float *statistics = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + statistics_offset);
   uint64_t row_base = 0;
   for (uint32_t first = 0; first < n_lanes; first += kLanes) {
     DecodeArgs a{};
@@ -533,34 +581,37 @@ int kvx_decode_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
     a.kv_heads = H;
     a.group = G;
     a.row_stride = row_stride;
+    a.fused_rows = M;
     a.kv = kv;
     uint32_t items = 0;
     for (uint32_t i = 0; i < a.n_lanes; ++i) {
       const kvx_verify_params &p = lanes[first + i];
       DecodeLane &dl = a.lane[i];
       dl.table = page_tables[first + i];
+      dl.masks = row_masks ? row_masks + uint64_t(first + i) * capacity : nullptr;
       dl.committed = p.committed_tokens;
+      dl.active_rows = p.active_rows;
       dl.split_count = p.split_count;
       dl.first_item = items;
       dl.score_scale = p.score_scale != 0.0f ? p.score_scale : l.score_scale;
       dl.row_base = row_base;
-      dl.q_offset = uint64_t(first + i) * H * row_stride * G * kD;
+      dl.q_offset = uint64_t(first + i) * lane_stride;
       items += p.split_count;
-      row_base += uint64_t(p.split_count) * H * G;
+      row_base += uint64_t(p.split_count) * H * M;
     }
     uint32_t max_splits = 0;
     for (uint32_t i = 0; i < a.n_lanes; ++i) max_splits = std::max(max_splits, a.lane[i].split_count);
     const uint32_t phases = kvx_attend_phases();
     hipError_t e = hipSuccess;
     if (phases & 1u) {
-      hipLaunchKernelGGL(decode_int4_kernel, dim3(items, H), dim3(64), 0, stream,
+      hipLaunchKernelGGL(decode_int4_kernel, dim3(items, H, (M + 15) / 16), dim3(64), 0, stream,
                          static_cast<const uint16_t *>(queries), static_cast<uint16_t *>(output),
                          partials, statistics, a);
       e = hipGetLastError();
       if (e != hipSuccess) return hip_fail(e, "decode_int4_kernel");
     }
     if (max_splits > 1 && (phases & 2u)) {
-      hipLaunchKernelGGL(decode_int4_merge_kernel, dim3(G, H, a.n_lanes), dim3(64), 0, stream,
+      hipLaunchKernelGGL(decode_int4_merge_kernel, dim3(M, H, a.n_lanes), dim3(64), 0, stream,
                          static_cast<uint16_t *>(output), partials, statistics, a);
       e = hipGetLastError();
       if (e != hipSuccess) return hip_fail(e, "decode_int4_merge_kernel");

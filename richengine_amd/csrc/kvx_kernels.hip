@@ -552,18 +552,32 @@ int check_launch(const char *what) {
 
 using namespace kvx;
 
-// Implemented by the int4 decode kernels: enqueues the whole attention and
+// Implemented by the int4 MFMA kernels: enqueues the whole attention and
 // returns 0, or declines (returns 1) shapes it does not cover.
-int kvx_decode_int4_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t query_heads,
+int kvx_attend_int4_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t query_heads,
                            const void *queries, void *output, const uint64_t *const *page_tables,
-                           const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
-                           void *workspace, hipStream_t stream);
+                           const kvx_verify_params *lanes, uint32_t n_lanes,
+                           const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
+                           void *workspace, uint64_t workspace_bytes, hipStream_t stream);
 
 uint32_t kvx_attend_phases() { return kvx::g_attend_phases; }
+
+namespace {
+uint64_t g_generic_attends = 0, g_matrix_attends = 0;
+int took(int fast) {  // counts which kernels an attend call went to
+  if (fast == 0) ++g_matrix_attends;
+  if (fast > 0) ++g_generic_attends;
+  return fast;
+}
+}  // namespace
 
 extern "C" {
 
 void kvx_debug_set_attend_phases(uint32_t phases) { kvx::g_attend_phases = phases & 3u; }
+void kvx_debug_attend_paths(uint64_t *generic_calls, uint64_t *matrix_core_calls) {
+  if (generic_calls) *generic_calls = g_generic_attends;
+  if (matrix_core_calls) *matrix_core_calls = g_matrix_attends;
+}
 
 int kv_append(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
               const void *chunk_values, const uint64_t *const *page_tables,
@@ -717,6 +731,12 @@ int kv_attend_verify(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
   if (int rc = validate_attend(s, query_heads, lanes, n_lanes, row_stride, page_tables,
                                workspace_bytes))
     return rc;
+  const uint32_t group = query_heads / s->layout.kv_heads;
+  const int fast = took(kvx_attend_int4_launch(
+      s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks, row_stride,
+      uint64_t(s->layout.kv_heads) * row_stride * group * s->layout.head_dim, workspace,
+      workspace_bytes, static_cast<hipStream_t>(stream)));
+  if (fast <= 0) return fast;
   return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks,
                         row_stride, workspace, static_cast<hipStream_t>(stream), 3);
 }
@@ -737,9 +757,11 @@ int kv_attend_decode(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
   if (int rc = validate_attend(s, query_heads, lanes, n_lanes, row_stride, page_tables,
                                workspace_bytes))
     return rc;
-  const int fast = kvx_decode_int4_launch(s, kv, query_heads, queries, output, page_tables, lanes,
-                                          n_lanes, row_stride, workspace,
-                                          static_cast<hipStream_t>(stream));
+  const uint32_t group = query_heads / s->layout.kv_heads;
+  const int fast = took(kvx_attend_int4_launch(
+      s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, nullptr, row_stride,
+      uint64_t(s->layout.kv_heads) * row_stride * group * s->layout.head_dim, workspace,
+      workspace_bytes, static_cast<hipStream_t>(stream)));
   if (fast <= 0) return fast;
   return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, nullptr,
                         row_stride, workspace, static_cast<hipStream_t>(stream), 3);
@@ -773,12 +795,31 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
   const uint64_t partial_bytes = rows * D * sizeof(float);
   if (workspace_bytes < partial_bytes + rows * 2 * sizeof(float))
     return fail(KVX_EINVAL, "prefill attention scratch is smaller than its bound");
+  auto st = static_cast<hipStream_t>(stream);
+  {
+    // The int4 MFMA kernels take the tiles as lanes: tile t attends rows 8t..8t+7
+    // over committed + 8t tokens, its queries 8 rows further on in the chunk.
+    std::vector<kvx_verify_params> tile_lanes(tiles);
+    std::vector<const uint64_t *> tile_tables(tiles, page_table);
+    for (uint32_t t = 0; t < tiles; ++t)
+      tile_lanes[t] = {params->committed_tokens + KVX_PREFILL_TILE_ROWS * t,
+                       params->page_table_entries,
+                       {},
+                       params->split_count,
+                       params->split_count,
+                       std::min(KVX_PREFILL_TILE_ROWS, params->rows - KVX_PREFILL_TILE_ROWS * t),
+                       KVX_PREFILL_TILE_ROWS,
+                       params->score_scale};
+    const int fast = took(kvx_attend_int4_launch(
+        s, kv, query_heads, queries, output, tile_tables.data(), tile_lanes.data(), tiles, nullptr,
+        params->chunk_stride, uint64_t(KVX_PREFILL_TILE_ROWS) * G * D, workspace, workspace_bytes, st));
+    if (fast <= 0) return fast;
+  }
   float *partials = static_cast<float *>(workspace);
   float *statistics = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + partial_bytes);
   PrefillArgs p{page_table, params->committed_tokens, params->rows, params->chunk_stride,
                 params->page_table_entries, params->split_count, H, G, D,
                 params->score_scale != 0.0f ? params->score_scale : l.score_scale, kv};
-  auto st = static_cast<hipStream_t>(stream);
   int rc = dispatch_format(l.format, [&](auto fmt) {
     return dispatch_rows(M, [&](auto maxm) {
       hipLaunchKernelGGL((prefill_split_kernel<decltype(fmt)::value, decltype(maxm)::value>),
