@@ -186,8 +186,9 @@ def main():
     def lane_params():
         ap = [kvx.ChunkParams(committed[i], 1, 32, lane_pages[i]) for i in range(BATCH)]
         vp = []
+        plan = kvx.decode_plan(committed, H)
         for i in range(BATCH):
-            s = L.kvx_decode_splits(committed[i], 1)
+            s = plan[i]
             if args.pages_per_split:
                 pages = (committed[i] + 1 + 31) // 32
                 s = min(max(1, -(-pages // args.pages_per_split)), 128)

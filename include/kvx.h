@@ -151,6 +151,14 @@ uint32_t kvx_prefill_splits(uint32_t rows);
    floor would only add partial traffic. */
 #define KVX_DECODE_PAGES_PER_SPLIT 32u
 uint32_t kvx_decode_splits(uint32_t committed_tokens, uint32_t rows);
+/* The same rule for a whole decode batch, which also fills the GPU when the batch is small:
+   pages per split = clamp(ceil(total page-heads / 1024 waves), 8, 32), and each lane gets
+   clamp(ceil(its pages / that), 1, KVX_DECODE_MAX_SPLITS) splits.  One-row decode lanes may
+   use up to KVX_DECODE_MAX_SPLITS splits; every other attend entry keeps the reference's
+   KVX_VERIFY_MAX_SPLITS. */
+#define KVX_DECODE_MAX_SPLITS 512u
+int kvx_decode_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t kv_heads,
+                    uint32_t *split_counts);
 /* kv::chunkedPrefillValidationError: 0 ok, 1 chunk_tokens_out_of_range,
    2 context_out_of_range, 3 chunk_stride_invalid, 4 page_table_too_short */
 int kvx_chunk_validation(const kvx_chunk_params *params);

@@ -149,15 +149,18 @@ bool prefill_contract_valid(const ko_prefill_params &p) {
          uint64_t{p.committed_tokens} + p.rows <= uint64_t{KO_MAX_PHYSICAL};
 }
 
-// common/paged_attention_tile.h:44-59
+// common/paged_attention_tile.h:44-59.  One-row decode lanes may use up to
+// KO_DECODE_MAX_SPLITS splits (a rule of the MI355X build for small batches, not
+// of the reference, whose bound is KO_VERIFY_MAX_SPLITS).
 bool verify_contract_valid(const ko_verify_params &p) {
+  const uint32_t max_splits = p.row_capacity == 1 ? KO_DECODE_MAX_SPLITS : KO_VERIFY_MAX_SPLITS;
   return p.active_rows > 0 && p.active_rows <= p.row_capacity &&
          p.page_table_entries >=
              (uint64_t{p.committed_tokens} + p.active_rows + kPage - 1) / kPage &&
          p.kv.extent_pages > 0 &&
          uint64_t{p.committed_tokens} + p.active_rows <= uint64_t{KO_MAX_PHYSICAL} &&
-         p.split_count > 0 && p.split_count <= KO_VERIFY_MAX_SPLITS &&
-         p.slot_splits >= p.split_count && p.slot_splits <= KO_VERIFY_MAX_SPLITS;
+         p.split_count > 0 && p.split_count <= max_splits &&
+         p.slot_splits >= p.split_count && p.slot_splits <= max_splits;
 }
 
 // common/paged_store_row.h:47-147 and paged_store_row_fp8.h:28-78: one row of

@@ -47,6 +47,7 @@ enum { KO_KEYS = 0, KO_KEY_SCALES = 1, KO_VALUES = 2, KO_VALUE_SCALES = 3 };
 #define KO_PREFILL_TILE_ROWS 8u      /* abi/ExecutionGeometry.h:32 */
 #define KO_PREFILL_MAX_SPLITS 32u    /* abi/ExecutionGeometry.h:33 */
 #define KO_VERIFY_MAX_SPLITS 128u    /* abi/ExecutionGeometry.h:39 */
+#define KO_DECODE_MAX_SPLITS 512u    /* one-row decode lanes of the MI355X build; no reference counterpart */
 #define KO_VERIFY_STRIDE 32u         /* abi/ExecutionGeometry.h:31 */
 
 /* runtime/ops/PagedKv.hpp:125-136 */

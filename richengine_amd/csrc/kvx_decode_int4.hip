@@ -268,39 +268,45 @@ __device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 *q_ld
 #endif
 constexpr uint32_t kDepth = KVX_DECODE_DEPTH;
 
-// Fixed-order merge of one q head's row over the splits of its (sequence, KV
-// head) (reference: common/paged_attention_tile.h:362-417).  One wave per row;
-// each lane owns four consecutive dimensions.  The statistics of up to 64
-// splits are fetched at once, one split per lane, so the maximum and the
-// weights cost one load latency; the partial rows then stream with several
-// loads in flight.  Sums run in split order, which is part of the contract.
-__device__ __forceinline__ void merge_row(const float *__restrict__ partials,
-                                          const float *__restrict__ statistics,
-                                          uint16_t *__restrict__ out_row, uint64_t first_row,
-                                          uint32_t written, uint32_t G, uint32_t lane) {
-  float maximum = -INFINITY;
-  for (uint32_t base = 0; base < written; base += 64) {
-    const uint32_t s = base + lane;
-    float m = s < written ? load_global<float>(statistics + (first_row + uint64_t(s) * G) * 2)
-                          : -INFINITY;
-#pragma unroll
-    for (uint32_t step = 32; step > 0; step >>= 1) m = fmaxf(m, __shfl_xor(m, step));
-    maximum = fmaxf(maximum, m);
-  }
-  f32x4 numerator = {0.0f, 0.0f, 0.0f, 0.0f};
-  float denominator = 0.0f;
-  for (uint32_t base = 0; base < written; base += 64) {
+// Merge of one fused query row over the splits of its (sequence, KV head)
+// (reference: common/paged_attention_tile.h:362-417).  Each lane owns four
+// consecutive dimensions.  The statistics of up to 64 splits are fetched at
+// once, one split per lane, so the maximum and the weights cost one load
+// latency; the partial rows then stream with several loads in flight.
+//
+// The order of the sums is fixed, which keeps the result a function of the
+// inputs and the split count alone: up to kMergeSequential splits are summed
+// in split order by one wave, as the reference does; longer lists (small
+// batches over long contexts) are cut into kMergeWaves consecutive ranges, one
+// per wave, each summed in split order, and the ranges are then added in range
+// order.
+constexpr uint32_t kMergeSequential = 32;
+constexpr uint32_t kMergeWaves = 4;
+
+struct MergeSums {
+  f32x4 numerator;
+  float denominator;
+};
+
+// Sums splits [first, last) of the row in split order; `maximum` is the row's
+// maximum over all splits.
+__device__ __forceinline__ MergeSums merge_range(const float *__restrict__ partials,
+                                                 const float *__restrict__ statistics,
+                                                 uint64_t first_row, uint32_t first, uint32_t last,
+                                                 uint32_t M, float maximum, uint32_t lane) {
+  MergeSums sums{{0.0f, 0.0f, 0.0f, 0.0f}, 0.0f};
+  for (uint32_t base = first; base < last; base += 64) {
     const uint32_t mine = base + lane;
     f32x2 stat = {-INFINITY, 0.0f};
-    if (mine < written) stat = load_global<f32x2>(statistics + (first_row + uint64_t(mine) * G) * 2);
+    if (mine < last) stat = load_global<f32x2>(statistics + (first_row + uint64_t(mine) * M) * 2);
     const float my_weight = expf(__fsub_rn(stat[0], maximum));
     const float my_term = __fmul_rn(my_weight, stat[1]);
-    const uint32_t count = min(64u, written - base);
+    const uint32_t count = min(64u, last - base);
     for (uint32_t i = 0; i < count; i += 8) {
       f32x4 part[8];
 #pragma unroll
       for (uint32_t u = 0; u < 8; ++u) {
-        const uint64_t row = first_row + uint64_t(base + min(i + u, count - 1)) * G;
+        const uint64_t row = first_row + uint64_t(base + min(i + u, count - 1)) * M;
         part[u] = load_global<f32x4>(partials + row * kD + 4 * lane);
       }
 #pragma unroll
@@ -309,28 +315,22 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ partials,
           const float weight = __shfl(my_weight, i + u);
 #pragma unroll
           for (uint32_t c = 0; c < 4; ++c)
-            numerator[c] = __fadd_rn(numerator[c], __fmul_rn(weight, part[u][c]));
-          denominator = __fadd_rn(denominator, __shfl(my_term, i + u));
+            sums.numerator[c] = __fadd_rn(sums.numerator[c], __fmul_rn(weight, part[u][c]));
+          sums.denominator = __fadd_rn(sums.denominator, __shfl(my_term, i + u));
         }
       }
     }
   }
-  u32x2 packed;
-#pragma unroll
-  for (uint32_t i = 0; i < 2; ++i) {
-    const float lo = denominator > 0.0f ? __fdiv_rn(numerator[2 * i], denominator) : 0.0f;
-    const float hi = denominator > 0.0f ? __fdiv_rn(numerator[2 * i + 1], denominator) : 0.0f;
-    packed[i] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
-  }
-  *reinterpret_cast<u32x2 *>(out_row + 4 * lane) = packed;
+  return sums;
 }
 
-// grid (fused query row, KV head, lane).  Lanes whose pages fit one split were
-// written by the split kernel itself.
-__global__ __launch_bounds__(64) void decode_int4_merge_kernel(
+// grid (fused query row, KV head, lane), kMergeWaves waves per row.  Lanes whose
+// pages fit one split were written by the split kernel itself.
+__global__ __launch_bounds__(64 * kMergeWaves) void decode_int4_merge_kernel(
     uint16_t *__restrict__ output, const float *__restrict__ partials,
     const float *__restrict__ statistics, DecodeArgs a) {
   const uint32_t j = blockIdx.x, head = blockIdx.y;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const DecodeLane &l = a.lane[blockIdx.z];
   const uint32_t pages = (l.committed + l.active_rows + kPage - 1) / kPage;
   const uint32_t per = (pages + l.split_count - 1) / l.split_count;
@@ -340,11 +340,52 @@ __global__ __launch_bounds__(64) void decode_int4_merge_kernel(
   uint16_t *out_row =
       output + l.q_offset + uint64_t(head) * a.row_stride * G * kD + uint64_t(j) * kD;
   if (j / G >= l.active_rows) {  // rows past the live ones read as zeros
-    *reinterpret_cast<u32x2 *>(out_row + 4 * threadIdx.x) = u32x2{0u, 0u};
+    if (wave == 0) *reinterpret_cast<u32x2 *>(out_row + 4 * lane) = u32x2{0u, 0u};
     return;
   }
-  merge_row(partials, statistics, out_row, l.row_base + uint64_t(head) * l.split_count * M + j,
-            written, M, threadIdx.x);
+  const uint64_t first_row = l.row_base + uint64_t(head) * l.split_count * M + j;
+  const bool sequential = written <= kMergeSequential;
+  if (sequential && wave) return;
+  float maximum = -INFINITY;
+  for (uint32_t base = 0; base < written; base += 64) {
+    const uint32_t s = base + lane;
+    float m = s < written ? load_global<float>(statistics + (first_row + uint64_t(s) * M) * 2)
+                          : -INFINITY;
+#pragma unroll
+    for (uint32_t step = 32; step > 0; step >>= 1) m = fmaxf(m, __shfl_xor(m, step));
+    maximum = fmaxf(maximum, m);
+  }
+  MergeSums sums;
+  if (sequential) {
+    sums = merge_range(partials, statistics, first_row, 0, written, M, maximum, lane);
+  } else {
+    const uint32_t share = (written + kMergeWaves - 1) / kMergeWaves;
+    const uint32_t first = min(written, wave * share), last = min(written, first + share);
+    const MergeSums mine = merge_range(partials, statistics, first_row, first, last, M, maximum, lane);
+    __shared__ f32x4 numerators[kMergeWaves][64];
+    __shared__ float denominators[kMergeWaves][64];
+    numerators[wave][lane] = mine.numerator;
+    denominators[wave][lane] = mine.denominator;
+    __syncthreads();
+    if (wave) return;
+    sums = mine;
+#pragma unroll
+    for (uint32_t w = 1; w < kMergeWaves; ++w) {
+      const f32x4 other = numerators[w][lane];
+#pragma unroll
+      for (uint32_t c = 0; c < 4; ++c) sums.numerator[c] = __fadd_rn(sums.numerator[c], other[c]);
+      sums.denominator = __fadd_rn(sums.denominator, denominators[w][lane]);
+    }
+  }
+  u32x2 packed;
+#pragma unroll
+  for (uint32_t i = 0; i < 2; ++i) {
+    const float lo = sums.denominator > 0.0f ? __fdiv_rn(sums.numerator[2 * i], sums.denominator) : 0.0f;
+    const float hi =
+        sums.denominator > 0.0f ? __fdiv_rn(sums.numerator[2 * i + 1], sums.denominator) : 0.0f;
+    packed[i] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
+  }
+  *reinterpret_cast<u32x2 *>(out_row + 4 * lane) = packed;
 }
 
 __global__ __launch_bounds__(64)
@@ -611,7 +652,8 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
       if (e != hipSuccess) return hip_fail(e, "decode_int4_kernel");
     }
     if (max_splits > 1 && (phases & 2u)) {
-      hipLaunchKernelGGL(decode_int4_merge_kernel, dim3(M, H, a.n_lanes), dim3(64), 0, stream,
+      hipLaunchKernelGGL(decode_int4_merge_kernel, dim3(M, H, a.n_lanes), dim3(64 * kMergeWaves), 0,
+                         stream,
                          static_cast<uint16_t *>(output), partials, statistics, a);
       e = hipGetLastError();
       if (e != hipSuccess) return hip_fail(e, "decode_int4_merge_kernel");

@@ -164,6 +164,24 @@ uint32_t kvx_decode_splits(uint32_t committed, uint32_t rows) {
   const uint32_t wanted = (pages + KVX_DECODE_PAGES_PER_SPLIT - 1) / KVX_DECODE_PAGES_PER_SPLIT;
   return std::min(std::max(1u, wanted), KVX_VERIFY_MAX_SPLITS);
 }
+int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_heads,
+                    uint32_t *split_counts) {
+  if (!committed || !split_counts || !n_lanes || !kv_heads)
+    return fail(KVX_EINVAL, "kvx_decode_plan: null argument or empty batch");
+  // One wave per SIMD of 256 CUs x 4 SIMDs is the least that fills the GPU;
+  // shorter splits than 8 pages cost more in set-up and partial rows than they
+  // win, and once the batch is large 32 pages per split measure best.
+  constexpr uint64_t kWaves = 1024;
+  uint64_t page_heads = 0;
+  for (uint32_t i = 0; i < n_lanes; ++i) page_heads += uint64_t(pages_of(uint64_t(committed[i]) + 1)) * kv_heads;
+  const uint32_t per = uint32_t(std::min<uint64_t>(
+      std::max<uint64_t>((page_heads + kWaves - 1) / kWaves, 8), KVX_DECODE_PAGES_PER_SPLIT));
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    const uint32_t pages = pages_of(uint64_t(committed[i]) + 1);
+    split_counts[i] = std::min(std::max(1u, (pages + per - 1) / per), KVX_DECODE_MAX_SPLITS);
+  }
+  return KVX_OK;
+}
 int kvx_chunk_validation(const kvx_chunk_params *p) {
   if (!p->chunk_tokens || p->chunk_tokens > KVX_PREFILL_TOKEN_BUDGET) return 1;
   if (uint64_t(p->committed_tokens) + p->chunk_tokens > KVX_MAX_PHYSICAL_TOKENS) return 2;

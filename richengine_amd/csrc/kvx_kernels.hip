@@ -144,7 +144,8 @@ __device__ inline bool attend_contract(const AttendLane &l, const AttendArgs &a)
          l.entries >= (uint64_t(l.committed) + l.active_rows + kPage - 1) / kPage &&
          a.kv.extent_pages > 0 &&
          uint64_t(l.committed) + l.active_rows <= uint64_t(KVX_MAX_PHYSICAL_TOKENS) &&
-         l.split_count > 0 && l.split_count <= KVX_VERIFY_MAX_SPLITS;
+         l.split_count > 0 &&
+         l.split_count <= (a.row_capacity == 1 ? KVX_DECODE_MAX_SPLITS : KVX_VERIFY_MAX_SPLITS);
 }
 __device__ inline bool prefill_contract(const PrefillArgs &p) {
   return p.rows > 0 && p.rows <= KVX_PREFILL_TOKEN_BUDGET && p.stride >= p.rows &&
@@ -634,6 +635,7 @@ static int validate_attend(const kvx_storage *s, uint32_t query_heads,
   if (!query_heads || query_heads % l.kv_heads)
     return fail(KVX_EINVAL, "query heads are not a multiple of the KV heads");
   const uint32_t capacity = lanes[0].row_capacity;
+  const uint32_t max_splits = capacity == 1 ? KVX_DECODE_MAX_SPLITS : KVX_VERIFY_MAX_SPLITS;
   for (uint32_t i = 0; i < n_lanes; ++i) {
     const kvx_verify_params &p = lanes[i];
     if (p.row_capacity != capacity || !capacity || capacity > row_stride)
@@ -644,7 +646,7 @@ static int validate_attend(const kvx_storage *s, uint32_t query_heads,
       return fail(KVX_EINVAL, "verify attention history exceeds physical context");
     if (p.page_table_entries < (uint64_t(p.committed_tokens) + p.active_rows + 31) / 32)
       return fail(KVX_EINVAL, "page_table_too_short");
-    if (!p.split_count || p.split_count > KVX_VERIFY_MAX_SPLITS)
+    if (!p.split_count || p.split_count > max_splits)
       return fail(KVX_EINVAL, "verify split count is out of range");
     if (!page_tables[i]) return fail(KVX_EINVAL, "null page table");
   }
