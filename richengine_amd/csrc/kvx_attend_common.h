@@ -1,0 +1,280 @@
+// Shared by the matrix-core (MFMA) attention kernels: lane arguments, the
+// per-row visibility rule, the merge kernel and the launch sequence.
+#pragma once
+
+#include <algorithm>
+
+#include "kvx_device.h"
+
+namespace kvx {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+#define KVX_GLOBAL __attribute__((address_space(1)))
+
+// Loads through pointers rebuilt from page entries: say they are global memory
+// so the compiler emits global_load rather than flat_load.
+template <class T>
+__device__ __forceinline__ T load_streaming(const uint8_t *p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const KVX_GLOBAL T *>(
+      reinterpret_cast<uintptr_t>(p)));
+}
+template <class T>
+__device__ __forceinline__ T load_global(const void *p) {
+  return *reinterpret_cast<const KVX_GLOBAL T *>(reinterpret_cast<uintptr_t>(p));
+}
+
+constexpr uint32_t kPage = KVX_PAGE_TOKENS;
+constexpr uint32_t kLanes = KVX_LANES_PER_LAUNCH;
+constexpr uint32_t kD = 256;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr uint32_t kTableSlots = 1024;  // page entries of one split staged in LDS
+
+struct DecodeLane {
+  const uint64_t *table;
+  const uint32_t *masks;  // tree verify: ancestor bitmask per row; null = causal chain
+  uint32_t committed;
+  uint32_t active_rows;   // query rows attended (1 for decode)
+  uint32_t split_count;
+  uint32_t first_item;  // first (lane, split) work item of this lane
+  float score_scale;
+  uint64_t row_base;    // first fused row of the lane's slots in the workspace
+  uint64_t q_offset;    // element offset of the lane's queries
+};
+struct DecodeArgs {
+  DecodeLane lane[kLanes];
+  uint32_t n_lanes;
+  uint32_t kv_heads;
+  uint32_t group;
+  uint32_t row_stride;
+  uint32_t fused_rows;  // row capacity x group: fused query rows per (lane, KV head)
+  kvx_kv_layer kv;
+};
+
+// Which tokens one fused query row (an MFMA column) may see
+// (reference: common/paged_attention_tile.h:141-143).
+struct Sight {
+  uint32_t committed;
+  uint32_t visible;  // committed + active rows
+  uint32_t limit;    // chain: first token the row may not see
+  uint32_t mask;     // tree: the row's ancestor bits over tokens committed + i
+  bool tree;
+  __device__ __forceinline__ bool sees(uint32_t token) const {
+    if (tree)
+      return token < committed || (token < visible && ((mask >> ((token - committed) & 31u)) & 1u));
+    return token < limit;
+  }
+};
+
+// Merge of one fused query row over the splits of its (sequence, KV head)
+// (reference: common/paged_attention_tile.h:362-417).  Each lane owns four
+// consecutive dimensions.  The statistics of up to 64 splits are fetched at
+// once, one split per lane, so the maximum and the weights cost one load
+// latency; the partial rows then stream with several loads in flight.
+//
+// The order of the sums is fixed, which keeps the result a function of the
+// inputs and the split count alone: up to kMergeSequential splits are summed
+// in split order by one wave, as the reference does; longer lists (small
+// batches over long contexts) are cut into kMergeWaves consecutive ranges, one
+// per wave, each summed in split order, and the ranges are then added in range
+// order.
+constexpr uint32_t kMergeSequential = 32;
+constexpr uint32_t kMergeWaves = 4;
+
+struct MergeSums {
+  f32x4 numerator;
+  float denominator;
+};
+
+// Sums splits [first, last) of the row in split order; `maximum` is the row's
+// maximum over all splits.
+__device__ __forceinline__ MergeSums merge_range(const float *__restrict__ partials,
+                                                 const float *__restrict__ statistics,
+                                                 uint64_t first_row, uint32_t first, uint32_t last,
+                                                 uint32_t M, float maximum, uint32_t lane) {
+  MergeSums sums{{0.0f, 0.0f, 0.0f, 0.0f}, 0.0f};
+  for (uint32_t base = first; base < last; base += 64) {
+    const uint32_t mine = base + lane;
+    f32x2 stat = {-INFINITY, 0.0f};
+    if (mine < last) stat = load_global<f32x2>(statistics + (first_row + uint64_t(mine) * M) * 2);
+    const float my_weight = expf(__fsub_rn(stat[0], maximum));
+    const float my_term = __fmul_rn(my_weight, stat[1]);
+    const uint32_t count = min(64u, last - base);
+    for (uint32_t i = 0; i < count; i += 8) {
+      f32x4 part[8];
+#pragma unroll
+      for (uint32_t u = 0; u < 8; ++u) {
+        const uint64_t row = first_row + uint64_t(base + min(i + u, count - 1)) * M;
+        part[u] = load_global<f32x4>(partials + row * kD + 4 * lane);
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < 8; ++u) {
+        if (i + u < count) {
+          const float weight = __shfl(my_weight, i + u);
+#pragma unroll
+          for (uint32_t c = 0; c < 4; ++c)
+            sums.numerator[c] = __fadd_rn(sums.numerator[c], __fmul_rn(weight, part[u][c]));
+          sums.denominator = __fadd_rn(sums.denominator, __shfl(my_term, i + u));
+        }
+      }
+    }
+  }
+  return sums;
+}
+
+// grid (fused query row, KV head, lane), kMergeWaves waves per row.  Lanes whose
+// pages fit one split were written by the split kernel itself.
+__global__ __launch_bounds__(64 * kMergeWaves) void matrix_merge_kernel(
+    uint16_t *__restrict__ output, const float *__restrict__ partials,
+    const float *__restrict__ statistics, DecodeArgs a) {
+  const uint32_t j = blockIdx.x, head = blockIdx.y;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const DecodeLane &l = a.lane[blockIdx.z];
+  const uint32_t pages = (l.committed + l.active_rows + kPage - 1) / kPage;
+  const uint32_t per = (pages + l.split_count - 1) / l.split_count;
+  const uint32_t written = (pages + per - 1) / per;
+  if (written <= 1) return;
+  const uint32_t G = a.group, M = a.fused_rows;
+  uint16_t *out_row =
+      output + l.q_offset + uint64_t(head) * a.row_stride * G * kD + uint64_t(j) * kD;
+  if (j / G >= l.active_rows) {  // rows past the live ones read as zeros
+    if (wave == 0) *reinterpret_cast<u32x2 *>(out_row + 4 * lane) = u32x2{0u, 0u};
+    return;
+  }
+  const uint64_t first_row = l.row_base + uint64_t(head) * l.split_count * M + j;
+  const bool sequential = written <= kMergeSequential;
+  if (sequential && wave) return;
+  float maximum = -INFINITY;
+  for (uint32_t base = 0; base < written; base += 64) {
+    const uint32_t s = base + lane;
+    float m = s < written ? load_global<float>(statistics + (first_row + uint64_t(s) * M) * 2)
+                          : -INFINITY;
+#pragma unroll
+    for (uint32_t step = 32; step > 0; step >>= 1) m = fmaxf(m, __shfl_xor(m, step));
+    maximum = fmaxf(maximum, m);
+  }
+  MergeSums sums;
+  if (sequential) {
+    sums = merge_range(partials, statistics, first_row, 0, written, M, maximum, lane);
+  } else {
+    const uint32_t share = (written + kMergeWaves - 1) / kMergeWaves;
+    const uint32_t first = min(written, wave * share), last = min(written, first + share);
+    const MergeSums mine = merge_range(partials, statistics, first_row, first, last, M, maximum, lane);
+    __shared__ f32x4 numerators[kMergeWaves][64];
+    __shared__ float denominators[kMergeWaves][64];
+    numerators[wave][lane] = mine.numerator;
+    denominators[wave][lane] = mine.denominator;
+    __syncthreads();
+    if (wave) return;
+    sums = mine;
+#pragma unroll
+    for (uint32_t w = 1; w < kMergeWaves; ++w) {
+      const f32x4 other = numerators[w][lane];
+#pragma unroll
+      for (uint32_t c = 0; c < 4; ++c) sums.numerator[c] = __fadd_rn(sums.numerator[c], other[c]);
+      sums.denominator = __fadd_rn(sums.denominator, denominators[w][lane]);
+    }
+  }
+  u32x2 packed;
+#pragma unroll
+  for (uint32_t i = 0; i < 2; ++i) {
+    const float lo = sums.denominator > 0.0f ? __fdiv_rn(sums.numerator[2 * i], sums.denominator) : 0.0f;
+    const float hi =
+        sums.denominator > 0.0f ? __fdiv_rn(sums.numerator[2 * i + 1], sums.denominator) : 0.0f;
+    packed[i] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
+  }
+  *reinterpret_cast<u32x2 *>(out_row + 4 * lane) = packed;
+}
+
+// Launches a split kernel over (work items, KV heads, column blocks) and then
+// the merge of the lanes that have more than one split.  `columns` is how many
+// fused query rows one workgroup of the split kernel covers.  Returns 1
+// (declined) when the workspace cannot hold the aligned layout, 0 when
+// enqueued, or a negative status.
+template <class SplitKernel>
+int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t columns,
+                            uint32_t threads, const kvx_storage *s, kvx_kv_layer kv,
+                            uint32_t query_heads, const void *queries, void *output,
+                            const uint64_t *const *page_tables, const kvx_verify_params *lanes,
+                            uint32_t n_lanes, const uint32_t *row_masks, uint32_t row_stride,
+                            uint64_t lane_stride, void *workspace, uint64_t workspace_bytes,
+                            uint32_t phases, hipStream_t stream) {
+  const kvx_layout &l = s->layout;
+  const uint32_t H = l.kv_heads, G = query_heads / H;
+  const uint32_t capacity = lanes[0].row_capacity, M = capacity * G;
+  uint64_t total_rows = 0;
+  for (uint32_t i = 0; i < n_lanes; ++i) total_rows += uint64_t(lanes[i].split_count) * H * M;
+  const uint64_t statistics_offset = (total_rows * kD * sizeof(float) + 255) / 256 * 256;
+  if (workspace_bytes < statistics_offset + total_rows * 2 * sizeof(float)) return 1;
+  float *partials = static_cast<float *>(workspace);
+  float *statistics = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + statistics_offset);
+  uint64_t row_base = 0;
+  for (uint32_t first = 0; first < n_lanes; first += kLanes) {
+    DecodeArgs a{};
+    a.n_lanes = std::min(kLanes, n_lanes - first);
+    a.kv_heads = H;
+    a.group = G;
+    a.row_stride = row_stride;
+    a.fused_rows = M;
+    a.kv = kv;
+    uint32_t items = 0, max_splits = 0;
+    for (uint32_t i = 0; i < a.n_lanes; ++i) {
+      const kvx_verify_params &p = lanes[first + i];
+      DecodeLane &dl = a.lane[i];
+      dl.table = page_tables[first + i];
+      dl.masks = row_masks ? row_masks + uint64_t(first + i) * capacity : nullptr;
+      dl.committed = p.committed_tokens;
+      dl.active_rows = p.active_rows;
+      dl.split_count = p.split_count;
+      dl.first_item = items;
+      dl.score_scale = p.score_scale != 0.0f ? p.score_scale : l.score_scale;
+      dl.row_base = row_base;
+      dl.q_offset = uint64_t(first + i) * lane_stride;
+      items += p.split_count;
+      max_splits = std::max(max_splits, p.split_count);
+      row_base += uint64_t(p.split_count) * H * M;
+    }
+    if (phases & 1u) {
+      hipLaunchKernelGGL(split_kernel, dim3(items, H, (M + columns - 1) / columns), dim3(threads), 0,
+                         stream, static_cast<const uint16_t *>(queries),
+                         static_cast<uint16_t *>(output), partials, statistics, a);
+      const hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return hip_fail(e, name);
+    }
+    if (max_splits > 1 && (phases & 2u)) {
+      hipLaunchKernelGGL(matrix_merge_kernel, dim3(M, H, a.n_lanes), dim3(64 * kMergeWaves), 0,
+                         stream, static_cast<uint16_t *>(output), partials, statistics, a);
+      const hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return hip_fail(e, "matrix_merge_kernel");
+    }
+  }
+  return 0;
+}
+
+// The shapes every matrix-core kernel of this library covers: head dimension
+// 256, a group of at most 16 query heads, at most KVX_TREE_NODES rows per lane,
+// every lane with the row capacity of the first, splits of at most kTableSlots
+// pages.
+inline bool matrix_attention_covers(const kvx_storage *s, uint32_t query_heads,
+                                    const kvx_verify_params *lanes, uint32_t n_lanes) {
+  const kvx_layout &l = s->layout;
+  if (l.head_dim != kD) return false;
+  const uint32_t G = query_heads / l.kv_heads, capacity = lanes[0].row_capacity;
+  if (G > 16 || !capacity || capacity > KVX_TREE_NODES) return false;
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    const kvx_verify_params &p = lanes[i];
+    if (p.row_capacity != capacity || !p.active_rows || p.active_rows > capacity) return false;
+    const uint32_t pages = (p.committed_tokens + p.active_rows + kPage - 1) / kPage;
+    const uint32_t splits = std::max(1u, p.split_count);
+    if ((pages + splits - 1) / splits > kTableSlots) return false;
+  }
+  return true;
+}
+
+}  // namespace
+}  // namespace kvx

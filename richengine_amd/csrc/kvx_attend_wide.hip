@@ -1,0 +1,417 @@
+// bf16 and fp8-e4m3 paged attention for gfx950: the split kernel of
+// kv_attend_decode, kv_attend_verify and kv_attend_prefill for pages whose
+// elements are two bytes (bf16) or one byte (fp8) wide, head dimension 256.
+//
+// One wave per (sequence or prefill tile, split, KV head, group of NB blocks of
+// 16 fused query rows).  The wave streams the split's pages once; keys and
+// values are the A operands of 16x16x32 MFMAs as they lie in the page (bf16) or
+// after an exact byte -> fp16 expansion (fp8), and all NB row blocks reuse
+// them.  The arithmetic follows the reference tiles
+// (common/paged_attention_tile.h:85-349 for bf16,
+// common/paged_attention_fp8_tile.h:34-265 for fp8): page-granular online
+// softmax, scores = raw dot x key scale x score scale, probabilities x value
+// scale rounded to bf16 (bf16 pages) or fp16 (fp8 pages, whose queries are
+// staged as fp16) before they meet the values.
+//
+// fp8 -> fp16 without a table: an e4m3 byte s.eeee.mmm placed at bits 14..7 of a
+// half (sign moved to bit 15) is the fp16 number 2^-8 times the e4m3 value,
+// subnormals included, because both formats then share mantissa alignment and
+// differ by the bias 15 - 7.  The factor 2^8 is applied in fp32, where it is
+// exact (to the scores with the key scale, to the accumulators at the end).
+#include "kvx_attend_common.h"
+
+namespace kvx {
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+template <uint32_t FMT>
+struct Wide {
+  static constexpr bool kFp8 = FMT == KVX_FMT_FP8E4M3;
+  static constexpr uint32_t kBytes = kFp8 ? 1 : 2;                   // per element
+  static constexpr uint32_t kSlab = kPage * kD * kBytes;             // per (head, page, tensor)
+  static constexpr uint32_t kDwords = kFp8 ? 2 : 4;                  // raw dwords per MFMA operand
+};
+
+template <uint32_t FMT>
+__device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+  if constexpr (Wide<FMT>::kFp8)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// Two e4m3 bytes (bytes `lo` and `hi` of x, selected by the perm pattern) to
+// two fp16 halves worth 2^-8 of their values.
+__device__ __forceinline__ uint32_t fp8_pair(uint32_t x, uint32_t select) {
+  const uint32_t y = __builtin_amdgcn_perm(0u, x, select);  // 0x00bb00aa
+  return ((y << 8) & 0x80008000u) | ((y << 7) & 0x3F803F80u);
+}
+// Eight consecutive bytes (two dwords) to eight fp16 in order.
+__device__ __forceinline__ u32x4 fp8_operand(uint32_t first, uint32_t second) {
+  return u32x4{fp8_pair(first, 0x0c010c00u), fp8_pair(first, 0x0c030c02u),
+               fp8_pair(second, 0x0c010c00u), fp8_pair(second, 0x0c030c02u)};
+}
+
+// What one lane holds of one page's keys / values.
+//  q.k : A = keys, row t = token 16*tb + t, k-slots = dims 32*kb + 8g .. + 7.
+//        B = queries, column t = fused query row, same dims.
+//        Output column t, rows 4g..4g+3 = tokens 16*tb + 4g + r.
+//  p.v : A = values (stored dimension-major), row t = dim 16*mb + t, k-slots =
+//        tokens 4g..4g+3 and 16+4g..16+4g+3: exactly the tokens whose scores the
+//        lane holds, so the probabilities are the B operand as they are.
+template <uint32_t FMT>
+struct KeyRegs {
+  uint32_t raw[2][8][Wide<FMT>::kDwords];  // [token block][dim block]
+};
+template <uint32_t FMT>
+struct ValueRegs {
+  uint32_t raw[16][Wide<FMT>::kDwords];  // [dim block]: tokens 4g.., then 16+4g..
+};
+
+struct PagePlace {
+  const uint8_t *keys, *values;
+  const float *key_scales, *value_scales;
+};
+template <uint32_t FMT>
+__device__ __forceinline__ PagePlace place_page(uint64_t entry, uint32_t head, uint32_t kv_heads,
+                                                uint32_t layer_offset, const RegionOffsets &ro) {
+  const uint32_t index = uint32_t(entry) & KVX_PAGE_INDEX_MASK;
+  const uint8_t *region = reinterpret_cast<const uint8_t *>(entry - index) + layer_offset;
+  const uint64_t slab = (uint64_t(index) * kv_heads + head) * Wide<FMT>::kSlab;
+  const uint64_t scale_index = (uint64_t(index) * kv_heads + head) * kPage;
+  PagePlace p;
+  p.keys = region + slab;
+  p.values = region + ro.values + slab;
+  p.key_scales = reinterpret_cast<const float *>(region + ro.key_scales) + scale_index;
+  p.value_scales = reinterpret_cast<const float *>(region + ro.value_scales) + scale_index;
+  return p;
+}
+
+template <uint32_t FMT>
+__device__ __forceinline__ void load_keys(KeyRegs<FMT> &k, const PagePlace &p, uint32_t t,
+                                          uint32_t g) {
+  constexpr uint32_t B = Wide<FMT>::kBytes;
+#pragma unroll
+  for (uint32_t tb = 0; tb < 2; ++tb)
+#pragma unroll
+    for (uint32_t kb = 0; kb < 8; ++kb) {
+      const uint8_t *at = p.keys + ((16 * tb + t) * kD + 32 * kb + 8 * g) * B;
+      if constexpr (Wide<FMT>::kFp8) {
+        const u32x2 v = load_streaming<u32x2>(at);
+        k.raw[tb][kb][0] = v[0];
+        k.raw[tb][kb][1] = v[1];
+      } else {
+        const u32x4 v = load_streaming<u32x4>(at);
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) k.raw[tb][kb][i] = v[i];
+      }
+    }
+}
+template <uint32_t FMT>
+__device__ __forceinline__ void load_values(ValueRegs<FMT> &v, const PagePlace &p, uint32_t t,
+                                            uint32_t g) {
+  constexpr uint32_t B = Wide<FMT>::kBytes;
+#pragma unroll
+  for (uint32_t mb = 0; mb < 16; ++mb)
+#pragma unroll
+    for (uint32_t half = 0; half < 2; ++half) {
+      const uint8_t *at = p.values + ((16 * mb + t) * kPage + 16 * half + 4 * g) * B;
+      if constexpr (Wide<FMT>::kFp8) {
+        v.raw[mb][half] = load_streaming<uint32_t>(at);
+      } else {
+        const u32x2 x = load_streaming<u32x2>(at);
+        v.raw[mb][2 * half] = x[0];
+        v.raw[mb][2 * half + 1] = x[1];
+      }
+    }
+}
+template <uint32_t FMT>
+__device__ __forceinline__ u32x4 key_operand(const KeyRegs<FMT> &k, uint32_t tb, uint32_t kb) {
+  if constexpr (Wide<FMT>::kFp8) return fp8_operand(k.raw[tb][kb][0], k.raw[tb][kb][1]);
+  else return u32x4{k.raw[tb][kb][0], k.raw[tb][kb][1], k.raw[tb][kb][2], k.raw[tb][kb][3]};
+}
+template <uint32_t FMT>
+__device__ __forceinline__ u32x4 value_operand(const ValueRegs<FMT> &v, uint32_t mb) {
+  if constexpr (Wide<FMT>::kFp8) return fp8_operand(v.raw[mb][0], v.raw[mb][1]);
+  else return u32x4{v.raw[mb][0], v.raw[mb][1], v.raw[mb][2], v.raw[mb][3]};
+}
+
+template <uint32_t FMT, uint32_t NB>
+__global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restrict__ queries,
+                                                         uint16_t *__restrict__ output,
+                                                         float *__restrict__ partials,
+                                                         float *__restrict__ statistics,
+                                                         DecodeArgs a) {
+  constexpr bool kFp8 = Wide<FMT>::kFp8;
+  const uint32_t item = blockIdx.x, head = blockIdx.y;
+  uint32_t li = 0;
+  for (uint32_t i = 1; i < a.n_lanes; ++i)
+    if (item >= a.lane[i].first_item) li = i;
+  const DecodeLane &l = a.lane[li];
+  const uint32_t split = item - l.first_item;
+  if (split >= l.split_count) return;
+  const uint32_t visible = l.committed + l.active_rows;
+  const uint32_t pages = (visible + kPage - 1) / kPage;
+  const uint32_t per = (pages + l.split_count - 1) / l.split_count;
+  const uint32_t written = (pages + per - 1) / per;  // splits that own a page
+  const uint32_t begin = split * per;
+  if (begin >= pages) return;
+  const uint32_t end = min(pages, begin + per);
+
+  const uint32_t lane = threadIdx.x, t = lane & 15, g = lane >> 4;
+  const uint32_t H = a.kv_heads, G = a.group, M = a.fused_rows;
+  const uint32_t db = Wide<FMT>::kSlab * H, sb = kFp8 ? kPage * H * 4 : 0;
+  const RegionOffsets ro = region_offsets(a.kv.extent_pages, db, sb);
+  const float score_scale = default_score_scale(kD, l.score_scale);
+
+  // Column t of block nb is fused row m = (query row, head in group).
+  uint32_t m[NB];
+  bool in_tile[NB], live_row[NB];
+  Sight sight[NB];
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    m[nb] = 16 * (NB * blockIdx.z + nb) + t;
+    const uint32_t query_row = m[nb] / G;
+    in_tile[nb] = m[nb] < M;
+    live_row[nb] = in_tile[nb] && query_row < l.active_rows;
+    sight[nb].committed = l.committed;
+    sight[nb].visible = visible;
+    sight[nb].limit =
+        live_row[nb] ? min(visible, l.committed + min(query_row, l.active_rows - 1) + 1) : visible;
+    sight[nb].tree = live_row[nb] && l.masks != nullptr;
+    sight[nb].mask = sight[nb].tree ? l.masks[query_row] : 0u;
+  }
+
+  // Queries: [row][g][D] bf16, fused row m; register kb of a column holds dims
+  // 32*kb + 8g .. + 7.  fp8 pages stage them as fp16.  Columns without a live row
+  // carry zeros.
+  const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
+  __shared__ u32x4 q_lds[NB][8][64];
+  __shared__ uint64_t table_lds[kTableSlots];
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    const uint16_t *q_row = q_head + uint64_t(live_row[nb] ? m[nb] : 0) * kD;
+#pragma unroll
+    for (uint32_t kb = 0; kb < 8; ++kb) {
+      u32x4 q = load_global<u32x4>(q_row + 32 * kb + 8 * g);
+      if constexpr (kFp8) {
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+          const f16x2 pair = {_Float16(__uint_as_float(q[i] << 16)),
+                              _Float16(__uint_as_float(q[i] & 0xffff0000u))};
+          q[i] = __builtin_bit_cast(uint32_t, pair);
+        }
+      }
+      if (!live_row[nb]) q = u32x4{0u, 0u, 0u, 0u};
+      q_lds[nb][kb][lane] = q;
+    }
+  }
+  // The split's page entries (at most kTableSlots; the launcher declines longer
+  // splits) go through LDS and are read back with uniform LDS loads.
+  for (uint32_t i = lane; i < end - begin; i += 64)
+    table_lds[i] = load_global<uint64_t>(l.table + begin + i);
+  __syncthreads();
+
+  KeyRegs<FMT> keys;
+  ValueRegs<FMT> values;
+  f32x4 ks[2], vs[2];  // fp8: scales of the lane's score tokens, per token block
+  auto fetch_keys = [&](uint32_t slot) {
+    const PagePlace p = place_page<FMT>(table_lds[slot], head, H, a.kv.offset, ro);
+    asm volatile("");  // the loads of one fetch stay together and in place
+    load_keys<FMT>(keys, p, t, g);
+    if constexpr (kFp8) {
+      ks[0] = load_global<f32x4>(p.key_scales + 4 * g);
+      ks[1] = load_global<f32x4>(p.key_scales + 16 + 4 * g);
+    }
+    asm volatile("");
+  };
+  auto fetch_values = [&](uint32_t slot) {
+    const PagePlace p = place_page<FMT>(table_lds[slot], head, H, a.kv.offset, ro);
+    asm volatile("");
+    load_values<FMT>(values, p, t, g);
+    if constexpr (kFp8) {
+      vs[0] = load_global<f32x4>(p.value_scales + 4 * g);
+      vs[1] = load_global<f32x4>(p.value_scales + 16 + 4 * g);
+    }
+    asm volatile("");
+  };
+  fetch_keys(0);
+  fetch_values(0);
+
+  f32x4 acc[NB][16];  // [block][dim block]: dims 16*mb + 4g + r of column t
+  float row_max[NB], row_sum[NB];
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+#pragma unroll
+    for (uint32_t mb = 0; mb < 16; ++mb) acc[nb][mb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    row_max[nb] = -INFINITY;
+    row_sum[nb] = 0.0f;
+  }
+  // fp8 operands are worth 2^-8 of their values; see the head of this file.
+  constexpr float kUnscale = kFp8 ? 256.0f : 1.0f;
+
+  for (uint32_t page = begin; page < end; ++page) {
+    // Refills are unconditional (the last page is fetched once more) so the loop
+    // body is straight-line code and each wait counts exactly the loads issued
+    // after the ones it needs.
+    const uint32_t next = min(page + 1, end - 1) - begin;
+    // ---- q.k ----
+    f32x4 s[NB][2];
+#pragma unroll
+    for (uint32_t nb = 0; nb < NB; ++nb) s[nb][0] = s[nb][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (uint32_t kb = 0; kb < 8; ++kb)
+#pragma unroll
+      for (uint32_t tb = 0; tb < 2; ++tb) {
+        const u32x4 k = key_operand<FMT>(keys, tb, kb);
+#pragma unroll
+        for (uint32_t nb = 0; nb < NB; ++nb) s[nb][tb] = mfma<FMT>(k, q_lds[nb][kb][lane], s[nb][tb]);
+      }
+    f32x4 page_ks[2];
+    if constexpr (kFp8) {
+      page_ks[0] = ks[0];
+      page_ks[1] = ks[1];
+    }
+    fetch_keys(next);
+    // ---- page softmax, per column block ----
+    const uint32_t first_token = page * kPage;
+    u32x4 pb[NB];
+    f32x4 page_vs[2];
+    if constexpr (kFp8) {
+      page_vs[0] = vs[0];
+      page_vs[1] = vs[1];
+    }
+#pragma unroll
+    for (uint32_t nb = 0; nb < NB; ++nb) {
+      float score[8], local_max = -INFINITY;
+      bool live[8];
+#pragma unroll
+      for (uint32_t i = 0; i < 8; ++i) {
+        const uint32_t tb = i >> 2, rr = i & 3;
+        float v = s[nb][tb][rr] * kUnscale;
+        if constexpr (kFp8) v *= page_ks[tb][rr];
+        v *= score_scale;
+        live[i] = sight[nb].sees(first_token + 16 * tb + 4 * g + rr);
+        score[i] = live[i] ? v : -INFINITY;
+        local_max = fmaxf(local_max, score[i]);
+      }
+      local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
+      local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
+      const float next_max = fmaxf(row_max[nb], local_max);
+      // A row that has seen nothing yet keeps -inf; its rescale is 1, not exp(nan).
+      const float rescale = next_max == row_max[nb]
+                                ? 1.0f
+                                : __builtin_amdgcn_exp2f((row_max[nb] - next_max) * kLog2e);
+      float weight[8], page_sum = 0.0f;
+#pragma unroll
+      for (uint32_t i = 0; i < 8; ++i) {
+        // The difference first, so the page's maximum gets exactly 1.
+        float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
+        p = live[i] ? p : 0.0f;
+        page_sum += p;
+        weight[i] = kFp8 ? p * page_vs[i >> 2][i & 3] : p;
+      }
+      row_sum[nb] = fmaf(row_sum[nb], rescale, page_sum);
+      row_max[nb] = next_max;
+#pragma unroll
+      for (uint32_t p = 0; p < 4; ++p) {
+        if constexpr (kFp8) {
+          const f16x2 pair = {_Float16(weight[2 * p]), _Float16(weight[2 * p + 1])};
+          pb[nb][p] = __builtin_bit_cast(uint32_t, pair);
+        } else {
+          const f32x2 pair = {weight[2 * p], weight[2 * p + 1]};
+          pb[nb][p] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+        }
+      }
+      if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
+#pragma unroll
+        for (uint32_t mb = 0; mb < 16; ++mb) acc[nb][mb] *= rescale;
+      }
+    }
+    // ---- p.v ----
+#pragma unroll
+    for (uint32_t mb = 0; mb < 16; ++mb) {
+      const u32x4 v = value_operand<FMT>(values, mb);
+#pragma unroll
+      for (uint32_t nb = 0; nb < NB; ++nb) acc[nb][mb] = mfma<FMT>(v, pb[nb], acc[nb][mb]);
+    }
+    fetch_values(next);
+  }
+
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    // Lanes of one column hold disjoint tokens: combine their sums.
+    float sum = row_sum[nb];
+    sum += __shfl_xor(sum, 16);
+    sum += __shfl_xor(sum, 32);
+    uint16_t *out_head = output + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
+    if (written == 1) {
+      // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
+      // Rows of the tile past the live ones read as zeros.
+      if (in_tile[nb]) {
+        const float denominator = live_row[nb] ? sum : 0.0f;
+#pragma unroll
+        for (uint32_t mb = 0; mb < 16; ++mb) {
+          u32x2 packed;
+#pragma unroll
+          for (uint32_t i = 0; i < 2; ++i) {
+            const float lo = acc[nb][mb][2 * i] * kUnscale, hi = acc[nb][mb][2 * i + 1] * kUnscale;
+            const float qlo = denominator > 0.0f ? __fdiv_rn(lo, denominator) : 0.0f;
+            const float qhi = denominator > 0.0f ? __fdiv_rn(hi, denominator) : 0.0f;
+            packed[i] = uint32_t(f32_to_bf16(qlo)) | (uint32_t(f32_to_bf16(qhi)) << 16);
+          }
+          *reinterpret_cast<u32x2 *>(out_head + uint64_t(m[nb]) * kD + 16 * mb + 4 * g) = packed;
+        }
+      }
+      continue;
+    }
+    if (live_row[nb]) {
+      const uint64_t row =
+          l.row_base + uint64_t(head) * l.split_count * M + uint64_t(split) * M + m[nb];
+      float *out = partials + row * kD;
+#pragma unroll
+      for (uint32_t mb = 0; mb < 16; ++mb)
+        *reinterpret_cast<f32x4 *>(out + 16 * mb + 4 * g) = acc[nb][mb] * kUnscale;
+      if (g == 0) {
+        statistics[row * 2] = row_max[nb];
+        statistics[row * 2 + 1] = sum;
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace kvx
+
+using namespace kvx;
+
+uint32_t kvx_attend_phases();  // bit 0 = split kernel, bit 1 = merge kernel
+
+// Runs paged attention for bf16 or fp8 pages of head dimension 256 on the
+// matrix cores; returns 1 (declined) for shapes it does not cover, 0 when
+// enqueued, or a negative status.  Arguments as kvx_attend_int4_launch.
+int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_heads,
+                           const void *queries, void *output, const uint64_t *const *page_tables,
+                           const kvx_verify_params *lanes, uint32_t n_lanes,
+                           const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
+                           void *workspace, uint64_t workspace_bytes, hipStream_t stream) {
+  const uint32_t format = s->layout.format;
+  if ((format != KVX_FMT_BF16 && format != KVX_FMT_FP8E4M3) ||
+      !matrix_attention_covers(s, query_heads, lanes, n_lanes))
+    return 1;
+  const uint32_t M = lanes[0].row_capacity * (query_heads / s->layout.kv_heads);
+  const uint32_t phases = kvx_attend_phases();
+#define KVX_WIDE(FMT, NB)                                                                        \
+  launch_matrix_attention(attend_wide_kernel<FMT, NB>, "attend_wide_kernel", 16 * NB, 64, s, kv, \
+                          query_heads, queries, output, page_tables, lanes, n_lanes, row_masks,  \
+                          row_stride, lane_stride, workspace, workspace_bytes, phases, stream)
+  // Two blocks of 16 fused rows per wave share every key and value operand; a
+  // third would not fit the register file next to a page of bf16 keys and values.
+  if (format == KVX_FMT_BF16) return M > 16 ? KVX_WIDE(KVX_FMT_BF16, 2) : KVX_WIDE(KVX_FMT_BF16, 1);
+  return M > 16 ? KVX_WIDE(KVX_FMT_FP8E4M3, 2) : KVX_WIDE(KVX_FMT_FP8E4M3, 1);
+#undef KVX_WIDE
+}

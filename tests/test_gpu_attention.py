@@ -18,13 +18,15 @@ pytestmark = pytest.mark.gpu
 H, G, D = 4, 6, 256
 QH = H * G
 FORMATS = [ko.INT4, ko.INT8, ko.BF16, ko.FP8]
+# formats whose pages of head dimension 256 run on the matrix-core kernels
+MATRIX = (ko.INT4, ko.BF16, ko.FP8)
 
 
 @pytest.fixture(autouse=True)
 def which_kernels_ran(request):
-    """int4 pages of head dimension 256 must run on the matrix-core kernels and
-    every other format on the format-generic ones: a test that passed through
-    the other path would not have tested what it names."""
+    """int4, bf16 and fp8 pages of head dimension 256 must run on the matrix-core
+    kernels and int8 pages on the format-generic ones: a test that passed
+    through the other path would not have tested what it names."""
     before = kvx.attend_paths()
     yield
     after = kvx.attend_paths()
@@ -32,7 +34,7 @@ def which_kernels_ran(request):
     if fmt is None:
         return
     generic, matrix = after[0] - before[0], after[1] - before[1]
-    if fmt == ko.INT4:
+    if fmt in MATRIX:
         assert matrix > 0 and generic == 0, (generic, matrix)
     else:
         assert generic > 0 and matrix == 0, (generic, matrix)
@@ -95,11 +97,11 @@ def test_prefill_matches_oracle(fmt, committed, rows):
     live = np.zeros((H, stride), dtype=bool)
     live[:, :rows] = True
     stats = Gp.check_attention(got, want, want32, live, tol(fmt), f"prefill fmt={fmt}",
-                               matrix_core=fmt == ko.INT4)
+                               matrix_core=fmt in MATRIX)
     # the format-generic tile keeps the oracle's operation order: nearly every
-    # output has the oracle's bits (expf differs in the last place); int4 runs
-    # on the matrix cores and sums in another order
-    if fmt != ko.INT4:
+    # output has the oracle's bits (expf differs in the last place); the other
+    # formats run on the matrix cores and sum in another order
+    if fmt not in MATRIX:
         assert stats["exact"] > 0.98
     else:
         assert stats["rel_l2_mean"] < 5e-4
@@ -141,7 +143,7 @@ def test_verify_chain_matches_oracle(fmt):
         live = np.zeros((1, H, 32), dtype=bool)
         live[:, :, :8] = True
         Gp.check_attention(got, want, want32, live, tol(fmt), f"verify lane {lane}",
-                           matrix_core=fmt == ko.INT4)
+                           matrix_core=fmt in MATRIX)
         assert (got[:, :, 8:] == 0x5A5A).all()
     for tw in tws:
         tw.close()
@@ -197,7 +199,7 @@ def test_batched_verify_chain_matches_oracle(fmt):
     live = np.zeros((lanes, H, 32), dtype=bool)
     live[:, :, :8] = True
     Gp.check_attention(Gp.host_u16(out), want, want32, live, tol(fmt), "batched verify",
-                       matrix_core=fmt == ko.INT4)
+                       matrix_core=fmt in MATRIX)
     # a repeat submission gives the same bits
     out2 = torch.zeros_like(out)
     kvx.attend_verify(tw.dev, 1, QH, Gp.dev(q), out2, dts, dp, None, 32, ws)
@@ -241,7 +243,7 @@ def test_tree_verify_matches_oracle(fmt, nodes):
     live = np.zeros((lanes, H, 32), dtype=bool)
     live[:, :, :nodes] = True
     Gp.check_attention(got, want, want32, live, tol(fmt), "tree verify",
-                       matrix_core=fmt == ko.INT4)
+                       matrix_core=fmt in MATRIX)
     assert not got[:, :, nodes:16].any() and (got[:, :, 16:] == 0x5A5A).all()
     tw.close()
 
@@ -271,7 +273,7 @@ def decode_case(fmt, committed, seed, row_stride=1, layers=2, layer=1):
     torch.cuda.synchronize()
     got = Gp.host_u16(out)
     stats = Gp.check_attention(got[:, :, 0], want, want32, np.ones((lanes, H), dtype=bool), tol(fmt),
-                               f"decode fmt={fmt} committed={committed}", matrix_core=fmt == ko.INT4)
+                               f"decode fmt={fmt} committed={committed}", matrix_core=fmt in MATRIX)
     assert stats["rel_l2_mean"] < 5e-4
     if row_stride > 1:
         assert (got[:, :, 1:] == 0x5A5A).all()
