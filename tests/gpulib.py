@@ -56,6 +56,12 @@ class Twin:
                 raise AssertionError(f"extent {e}: {bad.size} bytes differ, first at {bad[0]}: "
                                      f"got {got[bad[0]]:#x} want {want[bad[0]]:#x}")
 
+    def download(self):
+        """Copies the device extents' bytes into the oracle store (after device
+        appends whose bit-exactness other tests pin)."""
+        for e in range(self.extents):
+            self.host.extent(e)[:] = self.dev.extent_read(e)
+
     def upload(self):
         """Copies the oracle store's bytes into the device extents."""
         for e in range(self.extents):
@@ -105,7 +111,10 @@ def check_attention(out_bits, want_bits, want_f32, rows_mask, tol, label="", mat
     assert rel.max() <= hard, (f"{label}: relative L2 vs oracle bf16 {rel.max():.3e} > {hard} "
                                f"at row {worst}")
     within = float((rel <= tol).mean())
-    assert within >= 0.99, f"{label}: only {within:.4f} of the rows are within {tol}"
+    # 1% of the rows, and at least one where there are fewer than a hundred
+    allowed = max(1, int(0.01 * rel.size)) if matrix_core else 0
+    assert int((rel > tol).sum()) <= allowed, (
+        f"{label}: only {within:.4f} of the {rel.size} rows are within {tol}")
     rel32 = T.rel_l2(got[rows_mask], want_f32[rows_mask])
     assert rel32.max() <= tol + 2e-3, f"{label}: relative L2 vs oracle fp32 {rel32.max():.3e}"
     ulps = bf16_ulp_diff(out_bits[rows_mask], want_bits[rows_mask])
@@ -113,3 +122,27 @@ def check_attention(out_bits, want_bits, want_f32, rows_mask, tol, label="", mat
                 rel_l2_fp32=float(rel32.max()),
                 max_abs=float(np.abs(got[rows_mask] - want_f32[rows_mask]).max()),
                 exact=float((ulps == 0).mean()), max_ulp=int(ulps.max()))
+
+
+def oracle_tile(fmt, kv_heads, group, head_dim, tile_queries, table, kv, head, committed, active,
+                splits, capacity, masks=None, score_scale=0.0):
+    """The oracle's attention of one tile (capacity rows x group fused rows) of one
+    KV head: every split's partial tile, then the fixed-order merge of each live
+    fused row.  tile_queries: bf16 [capacity * group, D].  Returns (bf16, fp32)
+    outputs of that shape; rows past `active` are zeros."""
+    L = ko.lib()
+    M, D = capacity * group, head_dim
+    tile_queries = np.ascontiguousarray(tile_queries, dtype=np.uint16).reshape(M, D)
+    partials = np.zeros((splits, M, D), dtype=np.float32)
+    statistics = np.zeros((splits, M, 2), dtype=np.float32)
+    mask_ptr = ko.ptr(np.ascontiguousarray(masks, dtype=np.uint32)) if masks is not None else None
+    for split in range(splits):
+        L.ko_attention_tile(fmt, kv_heads, group, D, capacity, ko.ptr(tile_queries), ko.ptr(table), kv,
+                            head, committed, active, splits, split, ko.ptr(partials),
+                            ko.ptr(statistics), split, mask_ptr, score_scale)
+    out = np.zeros((M, D), dtype=np.uint16)
+    out32 = np.zeros((M, D), dtype=np.float32)
+    for row in range(M):
+        L.ko_attention_reduce_row(group, D, capacity, ko.ptr(partials), ko.ptr(statistics), committed,
+                                  active, splits, 0, row, ko.ptr(out[row]), ko.ptr(out32[row]))
+    return out, out32

@@ -1,0 +1,345 @@
+"""The five benchmark configurations at their full sizes, as parity tests.
+
+Where the scalar oracle finishes in seconds the device result is compared with
+it directly (configs 1-3, sampled tiles of 4 and 5); past that, size-independent
+properties carry the check: placement invariance (the same bytes behind any
+page ids give the same output bits), shared-prefix pages against private
+copies, append -> tree verify -> path compaction leaving exactly the oracle's
+page bytes.  Histories are written by the device append (pinned bit-exact in
+test_gpu_append.py) and copied into the oracle store.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import kvoracle as ko
+from richengine_amd import kvx
+import gpulib as Gp
+import kvtestlib as T
+
+pytestmark = pytest.mark.gpu
+
+H, G, D = 4, 6, 256
+QH = H * G
+
+
+def tol(fmt):
+    return 1e-2 if fmt == ko.FP8 else 2e-3
+
+
+def device_history(tw, layer, table_dev, entries, first, count, gen, outliers=False):
+    """Appends `count` random tokens at position `first` through kv_append."""
+    done = 0
+    while done < count:
+        n = min(2048, count - done)
+        stride = (n + 31) // 32 * 32
+        k = torch.randn((H, stride, D), generator=gen, device="cuda")
+        v = torch.randn((H, D, stride), generator=gen, device="cuda")
+        if outliers:  # a few channels 20x larger, as quantized KV caches see
+            k[:, :, [3, 77, 130, 255]] *= 20
+            v[:, [5, 64, 131, 250], :] *= 20
+        kvx.append(tw.dev, layer, k.bfloat16(), v.bfloat16(), [table_dev],
+                   [kvx.ChunkParams(first + done, n, stride, entries)], H * stride * D)
+        done += n
+
+
+def bf16_rows(shape, seed):
+    rng = np.random.default_rng(seed)
+    return ko.f32_to_bf16(rng.standard_normal(shape).astype(np.float32)).reshape(shape)
+
+
+def decode_on_device(tw, layer, q, tables, committed, counts, splits):
+    lanes = len(committed)
+    dp = [kvx.VerifyParams(committed[i], counts[i], kvx.KvLayer(), splits[i], splits[i], 1, 1, 0.0)
+          for i in range(lanes)]
+    out = torch.zeros((lanes, H, 1, G, D), dtype=torch.int16, device="cuda")
+    ws = torch.empty(kvx.attend_workspace_bytes(tw.dev, dp, QH) + 256, dtype=torch.uint8, device="cuda")
+    kvx.attend_decode(tw.dev, layer, QH, Gp.dev(q), out, tables, dp, 1, ws)
+    torch.cuda.synchronize()
+    return Gp.host_u16(out)[:, :, 0]
+
+
+def decode_on_oracle(tw, layer, q, tables, committed, counts, splits):
+    lanes = len(committed)
+    want = np.zeros((lanes, H, G, D), dtype=np.uint16)
+    want32 = np.zeros((lanes, H, G, D), dtype=np.float32)
+    for i in range(lanes):
+        q1 = np.zeros((1, H, 32, G, D), dtype=np.uint16)
+        q1[0, :, 0] = q[i, :, 0]
+        hp = ko.VerifyParams(committed[i], counts[i], tw.host.layer(layer), splits[i], splits[i], 1, 1, 0.0)
+        n, o, o32 = ko.attend_verify(tw.fmt, H, G, D, q1, [tables[i]], [hp])
+        assert n == 1
+        want[i], want32[i] = o[0, :, 0], o32[0, :, 0]
+    return want, want32
+
+
+def test_config1_int8_plumbing():
+    # int8, one layer, batch 1: 4096 tokens with outlier channels, one decode step
+    tw = Gp.Twin(ko.INT8, H, D, 1, 130)
+    pages = tw.pages(129, seed=1)
+    th, td = tw.tables(pages)
+    rng = np.random.default_rng(1)
+    done = 0
+    while done < 4097:   # both stores append the same chunks: bytes must agree
+        n = min(2048, 4097 - done)
+        k = rng.standard_normal((H, n, D)).astype(np.float32)
+        v = rng.standard_normal((H, n, D)).astype(np.float32)
+        k[:, :, [3, 77, 130, 255]] *= 20
+        stride = (n + 31) // 32 * 32
+        ck, cv = T.chunk_buffers(k, v, stride)
+        kvx.append(tw.dev, 0, Gp.dev(ck), Gp.dev(cv), [td], [kvx.ChunkParams(done, n, stride, 129)],
+                   H * stride * D)
+        assert ko.store_chunk(ko.INT8, H, D, ck, cv, th,
+                              ko.ChunkParams(done, n, stride, 129, tw.host.layer(0))) == 1
+        done += n
+    tw.assert_same_bytes()
+    q = bf16_rows((1, H, 1, G, D), 2)
+    splits = kvx.decode_plan([4096], H)
+    got = decode_on_device(tw, 0, q, [td], [4096], [129], splits)
+    want, want32 = decode_on_oracle(tw, 0, q, [th], [4096], [129], splits)
+    Gp.check_attention(got, want, want32, np.ones((1, H), dtype=bool), tol(ko.INT8), "config 1")
+    tw.close()
+
+
+def test_config2_int4_long_context_batch1():
+    # int4, batch 1, context 32768 behind a contiguous page table; one token is
+    # appended, then attended.  Then the same pages behind shuffled page ids.
+    committed, n_pages = 32768, 1025
+    tw = Gp.Twin(ko.INT4, H, D, 2, 2 * n_pages, one_extent=True)
+    pages = np.arange(n_pages, dtype=np.uint32)
+    th, td = tw.tables(pages)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(2)
+    device_history(tw, 1, td, n_pages, 0, committed, gen)
+    device_history(tw, 1, td, n_pages, committed, 1, gen)      # the decode step's append
+    tw.download()
+    q = bf16_rows((1, H, 1, G, D), 3)
+    splits = kvx.decode_plan([committed], H)
+    assert 32 < splits[0] <= 512                               # the small-batch rule is in force
+    got = decode_on_device(tw, 1, q, [td], [committed], [n_pages], splits)
+    want, want32 = decode_on_oracle(tw, 1, q, [th], [committed], [n_pages], splits)
+    stats = Gp.check_attention(got, want, want32, np.ones((1, H), dtype=bool), tol(ko.INT4),
+                               "config 2", matrix_core=True)
+    assert stats["rel_l2_mean"] < 1e-3
+    # placement invariance: move every page to a shuffled id, attend again
+    shuffled = (n_pages + np.random.default_rng(4).permutation(n_pages)).astype(np.uint32)
+    tw.dev.copy_pages([(int(a), int(b)) for a, b in zip(pages, shuffled)])
+    _, td2 = tw.tables(shuffled)
+    again = decode_on_device(tw, 1, q, [td2], [committed], [n_pages], splits)
+    assert np.array_equal(again, got)
+    tw.close()
+
+
+def test_config3_int4_mixed_batch32():
+    # int4, batch 32, contexts U[512, 32768], shuffled pages of one pool; one
+    # layer of the decode step against the oracle, every lane
+    rng = np.random.default_rng(20261125)
+    contexts = [int(c) for c in rng.integers(512, 32769, 32)]
+    counts = [(c + 1 + 31) // 32 for c in contexts]
+    tw = Gp.Twin(ko.INT4, H, D, 1, sum(counts), one_extent=True)
+    ids = np.random.default_rng(5).permutation(sum(counts)).astype(np.uint32)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    hts, dts, first = [], [], 0
+    for lane, n in enumerate(counts):
+        th, td = tw.tables(ids[first:first + n])
+        first += n
+        hts.append(th)
+        dts.append(td)
+        device_history(tw, 0, td, n, 0, contexts[lane] + 1, gen)
+    tw.download()
+    q = bf16_rows((32, H, 1, G, D), 6)
+    splits = kvx.decode_plan(contexts, H)
+    got = decode_on_device(tw, 0, q, dts, contexts, counts, splits)
+    want, want32 = decode_on_oracle(tw, 0, q, hts, contexts, counts, splits)
+    stats = Gp.check_attention(got, want, want32, np.ones((32, H), dtype=bool), tol(ko.INT4),
+                               "config 3", matrix_core=True)
+    assert stats["rel_l2_mean"] < 5e-4
+    tw.close()
+
+
+@pytest.mark.parametrize("fmt", [ko.BF16, ko.FP8])
+def test_config4_shared_prefix_chunked_prefill(fmt):
+    # batch 4: a 16384-token prefix computed once and shared through the prefix
+    # cache (512 whole pages), then a 2048-token chunk per sequence: quantize +
+    # scatter, causal attention of 2048 rows over 18432 tokens
+    prefix, chunk, sequences = 16384, 2048, 4
+    prefix_pages, chunk_pages = prefix // 32, chunk // 32
+    total_pages = prefix_pages + sequences * chunk_pages + prefix_pages   # + one private copy
+    tw = Gp.Twin(fmt, H, D, 1, total_pages, one_extent=True)
+    tw.dev.release(0)          # the pool allocates the device extent itself
+    pool = kvx.Pool(tw.dev, tw.dev.page_count)
+    cache = kvx.Prefix(pool)
+    seqs = kvx.Sequences(pool, cache)
+    tokens = [[(7 * i + 13 * s * (i >= prefix)) % 50021 for i in range(prefix + chunk)]
+              for s in range(sequences)]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7)
+    # sequence 1 computes the prefix and publishes it
+    seqs.begin(1)
+    seqs.ensure_tokens(1, prefix + chunk)
+    view = seqs.view(1)
+    table1 = tw.dev.table(np.array(view["pages"], dtype=np.uint32))
+    device_history(tw, 0, table1, len(view["pages"]), 0, prefix, gen)
+    seqs.publish(1, tokens[0], prefix)
+    # the others find it, adopt its pages and take pages of their own for the chunk
+    tables = {1: table1}
+    for s in range(2, sequences + 1):
+        seqs.begin(s)
+        blocks, hashed = cache.match(tokens[s - 1])
+        assert len(blocks) == prefix_pages and hashed == prefix_pages + 1
+        seqs.restore(s, blocks[-1])
+        seqs.ensure_tokens(s, prefix + chunk)
+        v = seqs.view(s)
+        assert v["pages"][:prefix_pages] == view["pages"][:prefix_pages]
+        assert not set(v["pages"][prefix_pages:]) & set(view["pages"])
+        tables[s] = tw.dev.table(np.array(v["pages"], dtype=np.uint32))
+    snap = pool.snapshot()
+    assert snap.pages_prefix == prefix_pages
+    assert snap.pages_active == prefix_pages + sequences * chunk_pages
+    # every sequence appends its chunk and attends it
+    n_entries = prefix_pages + chunk_pages
+    splits = kvx.lib().kvx_prefill_splits(chunk)
+    ws = torch.empty(kvx.prefill_workspace_bytes(tw.dev, chunk, QH) + 256, dtype=torch.uint8, device="cuda")
+    outs, chunks, qs = {}, {}, {}
+    for s in range(1, sequences + 1):
+        k = torch.randn((H, chunk, D), generator=gen, device="cuda").bfloat16()
+        v = torch.randn((H, D, chunk), generator=gen, device="cuda").bfloat16()
+        q = torch.randn((H, chunk, G, D), generator=gen, device="cuda").bfloat16()
+        chunks[s], qs[s] = (k, v), q
+        kvx.append(tw.dev, 0, k, v, [tables[s]], [kvx.ChunkParams(prefix, chunk, chunk, n_entries)],
+                   H * chunk * D)
+        out = torch.zeros((H, chunk, G, D), dtype=torch.int16, device="cuda")
+        kvx.attend_prefill(tw.dev, 0, QH, q, out, tables[s],
+                           kvx.PrefillParams(prefix, chunk, chunk, n_entries, kvx.KvLayer(), splits, 0.0), ws)
+        outs[s] = out
+    torch.cuda.synchronize()
+    # (a) shared pages against a private copy of the prefix: sequence 2 again,
+    # with its prefix pages copied to fresh pages -- the bits must not change
+    spare = pool.acquire(prefix_pages)
+    shared = seqs.view(2)["pages"]
+    tw.dev.copy_pages(list(zip(shared[:prefix_pages], spare)))
+    private = tw.dev.table(np.array(spare + shared[prefix_pages:], dtype=np.uint32))
+    out_private = torch.zeros((H, chunk, G, D), dtype=torch.int16, device="cuda")
+    kvx.attend_prefill(tw.dev, 0, QH, qs[2], out_private, private,
+                       kvx.PrefillParams(prefix, chunk, chunk, n_entries, kvx.KvLayer(), splits, 0.0), ws)
+    torch.cuda.synchronize()
+    assert torch.equal(out_private, outs[2])
+    # the copies are byte-identical and the sources untouched
+    for a, b in list(zip(shared[:prefix_pages], spare))[::97]:
+        assert np.array_equal(tw.dev.page_read(a), tw.dev.page_read(b))
+    # (b) the oracle on sampled tiles of sequence 2: first, middle, last
+    tw.download()
+    table_host = tw.host.entries(np.array(shared, dtype=np.uint32))
+    q_host = Gp.host_u16(qs[2].view(torch.int16))
+    got = Gp.host_u16(outs[2])
+    rels = []
+    for tile in (0, 127, 255):
+        for head in (0, 3):
+            tile_q = q_host[head, 8 * tile:8 * tile + 8].reshape(8 * G, D)
+            want, want32 = Gp.oracle_tile(fmt, H, G, D, tile_q, table_host, tw.host.layer(0), head,
+                                          prefix + 8 * tile, 8, splits, 8)
+            mine = got[head, 8 * tile:8 * tile + 8].reshape(8 * G, D)
+            stats = Gp.check_attention(mine, want, want32, np.ones(8 * G, dtype=bool), tol(fmt),
+                                       f"config 4 tile {tile} head {head}", matrix_core=True)
+            rels.append(stats["rel_l2_mean"])
+    assert np.mean(rels) < (4e-3 if fmt == ko.FP8 else 1e-3)
+    for s in range(1, sequences + 1):
+        seqs.end(s)
+    for p in spare:
+        pool.release(p)
+    assert pool.snapshot().pages_active == 0 and pool.snapshot().pages_prefix == prefix_pages
+    seqs.close()
+    cache.close()
+    pool.close()
+    tw.close()
+
+
+def test_config5_int4_tree_verify_and_rollback():
+    # int4, batch 4, context 65536, a 16-row tree per sequence: append the rows,
+    # masked verify, a root-to-leaf path per sequence, compaction; the page bytes
+    # after the rollback must be the oracle's, bit for bit
+    lanes, committed, nodes = 4, 65536, 16
+    n_pages = (committed + nodes + 31) // 32
+    tw = Gp.Twin(ko.INT4, H, D, 1, lanes * n_pages, one_extent=True)
+    ids = np.random.default_rng(8).permutation(lanes * n_pages).astype(np.uint32)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(8)
+    hts, dts = [], []
+    for lane in range(lanes):
+        th, td = tw.tables(ids[lane * n_pages:(lane + 1) * n_pages])
+        hts.append(th)
+        dts.append(td)
+        device_history(tw, 0, td, n_pages, 0, committed, gen)
+    tw.download()
+    rng = np.random.default_rng(9)
+    none = 0xFFFFFFFF
+    parents, masks = [], np.zeros((lanes, nodes), dtype=np.uint32)
+    for lane in range(lanes):
+        # topologically ordered, branching at most 3
+        p, children = [none], {0: 0}
+        for row in range(1, nodes):
+            choices = [c for c in range(row) if children.get(c, 0) < 3]
+            parent = int(rng.choice(choices[-4:]))
+            children[parent] = children.get(parent, 0) + 1
+            p.append(parent)
+        parents.append(p)
+        masks[lane] = kvx.tree_masks(p)
+    # the rows' K/V go through the verify store on both sides
+    k = rng.standard_normal((lanes, H, nodes, D)).astype(np.float32)
+    v = rng.standard_normal((lanes, H, nodes, D)).astype(np.float32)
+    ck = np.zeros((lanes, H, 32, D), dtype=np.uint16)
+    cv = np.zeros((lanes, H, D, 32), dtype=np.uint16)
+    for lane in range(lanes):
+        ck[lane], cv[lane] = T.chunk_buffers(k[lane], v[lane], 32)
+    dparams = [kvx.ChunkParams(committed, nodes, 32, n_pages) for _ in range(lanes)]
+    kvx.append(tw.dev, 0, Gp.dev(ck), Gp.dev(cv), dts, dparams, H * 32 * D, verify_max_rows=16)
+    hparams = [ko.ChunkParams(committed, nodes, 32, n_pages, tw.host.layer(0)) for _ in range(lanes)]
+    assert ko.store_verify(ko.INT4, H, D, ck, cv, hts, hparams, max_rows=16) == lanes
+    # masked verify on the device; the oracle on one lane, two heads
+    q = np.zeros((lanes, H, 32, G, D), dtype=np.uint16)
+    q[:, :, :nodes] = bf16_rows((lanes, H, nodes, G, D), 10)
+    splits = [kvx.lib().kvx_verify_splits(committed, nodes)] * lanes
+    dp = [kvx.VerifyParams(committed, n_pages, kvx.KvLayer(), splits[i], 128, nodes, 16, 0.0)
+          for i in range(lanes)]
+    out = torch.zeros((lanes, H, 32, G, D), dtype=torch.int16, device="cuda")
+    ws = torch.empty(kvx.attend_workspace_bytes(tw.dev, dp, QH) + 256, dtype=torch.uint8, device="cuda")
+    kvx.attend_verify(tw.dev, 0, QH, Gp.dev(q), out, dts, dp, Gp.dev(masks), 32, ws)
+    torch.cuda.synchronize()
+    got = Gp.host_u16(out)
+    lane = 2
+    for head in (0, 3):
+        tile_q = q[lane, head, :16].reshape(16 * G, D)
+        want, want32 = Gp.oracle_tile(ko.INT4, H, G, D, tile_q, hts[lane], tw.host.layer(0), head,
+                                      committed, nodes, splits[lane], 16, masks=masks[lane])
+        mine = got[lane, head, :16].reshape(16 * G, D)
+        Gp.check_attention(mine, want, want32, np.ones(16 * G, dtype=bool), tol(ko.INT4),
+                           f"config 5 lane {lane} head {head}", matrix_core=True)
+    # a tree that is a path must see exactly what the chain sees
+    chain_masks = np.zeros((lanes, nodes), dtype=np.uint32)
+    chain_masks[:] = kvx.tree_masks([none] + list(range(nodes - 1)))
+    out_path = torch.zeros_like(out)
+    kvx.attend_verify(tw.dev, 0, QH, Gp.dev(q), out_path, dts, dp, Gp.dev(chain_masks), 32, ws)
+    out_chain = torch.zeros_like(out)
+    kvx.attend_verify(tw.dev, 0, QH, Gp.dev(q), out_chain, dts, dp, None, 32, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(out_path, out_chain)
+    # acceptance: a seeded root-to-leaf walk per sequence; then compaction
+    paths = np.zeros((lanes, 16), dtype=np.uint32)
+    counts = np.zeros(lanes, dtype=np.uint32)
+    for i in range(lanes):
+        walk, row = [0], 0
+        while True:
+            kids = [c for c in range(nodes) if parents[i][c] == row]
+            if not kids:
+                break
+            row = int(rng.choice(kids))
+            walk.append(row)
+        assert kvx.tree_path_valid(parents[i], walk)
+        paths[i, :len(walk)] = walk
+        counts[i] = len(walk)
+    kvx.compact_path(tw.dev, 0, dts, dparams, Gp.dev(paths), Gp.dev(counts), 16)
+    torch.cuda.synchronize()
+    assert ko.compact_tree(ko.INT4, H, D, hts, hparams, paths, counts, 16) > 0   # rows moved
+    tw.assert_same_bytes()
+    tw.close()
