@@ -92,86 +92,99 @@ __device__ __forceinline__ u32x4 expand_key_dword(uint32_t x) {
   return out;
 }
 
+// Softmax state and accumulators of one block of 16 fused query rows.
 struct State {
-  f32x4 acc[16];  // [nibble position m]: dims 16*(4g + r) + m of q head t
+  f32x4 acc[16];  // [nibble position m]: dims 16*(4g + r) + m of column t
   float row_max;
-  float row_sum;   // this lane's tokens only; lanes of a q head are summed at the end
+  float row_sum;   // this lane's tokens only; lanes of a column are summed at the end
   float bias;      // constant part carried by acc, this lane's tokens only
 };
 
+// One page against NB blocks of 16 fused query rows; every key and value
+// operand is expanded once and used by all blocks.
 // MASKED: the page may hold tokens some row does not see (only the last two
 // pages of a sequence can); other pages skip the per-token test.
-template <bool MASKED>
-__device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 *q_lds, float q_bias,
-                                            float score_scale, uint32_t first_token,
-                                            const Sight &sight, uint32_t lane, uint32_t g,
-                                            State &st) {
+template <bool MASKED, uint32_t NB>
+__device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 (*q_lds)[8 * 64],
+                                            const float *q_bias, float score_scale,
+                                            uint32_t first_token, const Sight *sight,
+                                            uint32_t lane, uint32_t g, State *st) {
 #ifdef KVX_PROBE_STREAM_ONLY
   // Measurement build: consume every loaded register with almost no arithmetic,
   // to see what the memory system delivers for this access pattern.
   uint32_t x = 0;
   for (uint32_t i = 0; i < 4; ++i) x ^= r.k[i][0] ^ r.k[i][1] ^ r.k[i][2] ^ r.k[i][3];
   for (uint32_t i = 0; i < 8; ++i) x ^= r.v[i][0] ^ r.v[i][1];
-  st.row_sum += r.ks[0][0] + r.ks[1][3] + r.vs[0][1] + r.vs[1][2] + __uint_as_float(x & 0xffu);
+  st[0].row_sum += r.ks[0][0] + r.ks[1][3] + r.vs[0][1] + r.vs[1][2] + __uint_as_float(x & 0xffu);
   return;
 #endif
   // ---- q.k ----
-  f32x4 s[2];
-  s[0] = s[1] = f32x4{-q_bias, -q_bias, -q_bias, -q_bias};
+  f32x4 s[NB][2];
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb)
+    s[nb][0] = s[nb][1] = f32x4{-q_bias[nb], -q_bias[nb], -q_bias[nb], -q_bias[nb]};
 #pragma unroll
   for (uint32_t kb = 0; kb < 8; ++kb) {
-    const u32x4 q = q_lds[kb * 64 + lane];
+    u32x4 q[NB];
 #pragma unroll
-    for (uint32_t tb = 0; tb < 2; ++tb)
-      s[tb] = mfma_bf16(expand_key_dword(r.k[tb * 2 + (kb >> 2)][kb & 3]), q, s[tb]);
+    for (uint32_t nb = 0; nb < NB; ++nb) q[nb] = q_lds[nb][kb * 64 + lane];
+#pragma unroll
+    for (uint32_t tb = 0; tb < 2; ++tb) {
+      const u32x4 k = expand_key_dword(r.k[tb * 2 + (kb >> 2)][kb & 3]);
+#pragma unroll
+      for (uint32_t nb = 0; nb < NB; ++nb) s[nb][tb] = mfma_bf16(k, q[nb], s[nb][tb]);
+    }
   }
-  // ---- page softmax ----
-  float score[8], local_max = -INFINITY;
-  bool live[8];
+  // ---- page softmax, per block ----
+  u32x4 pb[NB];
 #pragma unroll
-  for (uint32_t i = 0; i < 8; ++i) {
-    const uint32_t tb = i >> 2, rr = i & 3;
-    float v = s[tb][rr] * r.ks[tb][rr];
-    v *= score_scale;
-    live[i] = !MASKED || sight.sees(first_token + 16 * tb + 4 * g + rr);
-    score[i] = live[i] ? v : -INFINITY;
-    local_max = fmaxf(local_max, score[i]);
-  }
-  local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
-  local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
-  const float next_max = fmaxf(st.row_max, local_max);
-  // A row that has seen nothing yet keeps -inf; its rescale is 1, not exp(nan).
-  const float rescale = next_max == st.row_max
-                            ? 1.0f
-                            : __builtin_amdgcn_exp2f((st.row_max - next_max) * kLog2e);
-  float weight[8], page_sum = 0.0f;
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    float score[8], local_max = -INFINITY;
+    bool live[8];
 #pragma unroll
-  for (uint32_t i = 0; i < 8; ++i) {
-    // The difference first, so the page's maximum gets exactly 1.
-    float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
-    if (MASKED) p = live[i] ? p : 0.0f;
-    page_sum += p;
-    const float w = p * r.vs[i >> 2][i & 3];
-    weight[i] = live[i] ? w : 0.0f;
-  }
-  st.row_sum = fmaf(st.row_sum, rescale, page_sum);
-  st.row_max = next_max;
-  // bf16 probabilities (round to nearest even): even tokens as they are, odd
-  // tokens negated (their value codes are expanded as 135 - c).
-  u32x4 pb;
-  float page_bias = 0.0f;
+    for (uint32_t i = 0; i < 8; ++i) {
+      const uint32_t tb = i >> 2, rr = i & 3;
+      float v = s[nb][tb][rr] * r.ks[tb][rr];
+      v *= score_scale;
+      live[i] = !MASKED || sight[nb].sees(first_token + 16 * tb + 4 * g + rr);
+      score[i] = live[i] ? v : -INFINITY;
+      local_max = fmaxf(local_max, score[i]);
+    }
+    local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
+    local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
+    const float next_max = fmaxf(st[nb].row_max, local_max);
+    // A row that has seen nothing yet keeps -inf; its rescale is 1, not exp(nan).
+    const float rescale = next_max == st[nb].row_max
+                              ? 1.0f
+                              : __builtin_amdgcn_exp2f((st[nb].row_max - next_max) * kLog2e);
+    float weight[8], page_sum = 0.0f;
 #pragma unroll
-  for (uint32_t p = 0; p < 4; ++p) {
-    const f32x2 pair = {weight[2 * p], weight[2 * p + 1]};
-    const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
-    page_bias = fmaf(136.0f, __uint_as_float(bits << 16), page_bias);
-    page_bias = fmaf(-135.0f, __uint_as_float(bits & 0xffff0000u), page_bias);
-    pb[p] = bits ^ 0x80000000u;
-  }
-  st.bias = fmaf(st.bias, rescale, page_bias);
-  if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
+    for (uint32_t i = 0; i < 8; ++i) {
+      // The difference first, so the page's maximum gets exactly 1.
+      float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
+      if (MASKED) p = live[i] ? p : 0.0f;
+      page_sum += p;
+      const float w = p * r.vs[i >> 2][i & 3];
+      weight[i] = live[i] ? w : 0.0f;
+    }
+    st[nb].row_sum = fmaf(st[nb].row_sum, rescale, page_sum);
+    st[nb].row_max = next_max;
+    // bf16 probabilities (round to nearest even): even tokens as they are, odd
+    // tokens negated (their value codes are expanded as 135 - c).
+    float page_bias = 0.0f;
 #pragma unroll
-    for (uint32_t m = 0; m < 16; ++m) st.acc[m] *= rescale;
+    for (uint32_t p = 0; p < 4; ++p) {
+      const f32x2 pair = {weight[2 * p], weight[2 * p + 1]};
+      const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+      page_bias = fmaf(136.0f, __uint_as_float(bits << 16), page_bias);
+      page_bias = fmaf(-135.0f, __uint_as_float(bits & 0xffff0000u), page_bias);
+      pb[nb][p] = bits ^ 0x80000000u;
+    }
+    st[nb].bias = fmaf(st[nb].bias, rescale, page_bias);
+    if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
+#pragma unroll
+      for (uint32_t m = 0; m < 16; ++m) st[nb].acc[m] *= rescale;
+    }
   }
   // ---- p.v ----
 #pragma unroll
@@ -191,7 +204,8 @@ __device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 *q_ld
 #pragma unroll
       for (uint32_t i = 0; i < 4; ++i) {
         const uint32_t m = 8 * half + 4 * part + i;
-        st.acc[m] = mfma_bf16(vop[i], pb, st.acc[m]);
+#pragma unroll
+        for (uint32_t nb = 0; nb < NB; ++nb) st[nb].acc[m] = mfma_bf16(vop[i], pb[nb], st[nb].acc[m]);
       }
     }
   }
@@ -200,15 +214,14 @@ __device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 *q_ld
 #ifndef KVX_DECODE_DEPTH
 #define KVX_DECODE_DEPTH 2
 #endif
-#ifndef KVX_DECODE_WAVES
-#define KVX_DECODE_WAVES 2
-#endif
 constexpr uint32_t kDepth = KVX_DECODE_DEPTH;
 
-__global__ __launch_bounds__(64)
-__attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void decode_int4_kernel(
-    const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
-    float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
+// The split kernel's body for NB blocks of 16 fused query rows per wave.
+template <uint32_t NB>
+__device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries,
+                                            uint16_t *__restrict__ output,
+                                            float *__restrict__ partials,
+                                            float *__restrict__ statistics, const DecodeArgs &a) {
   const uint32_t item = blockIdx.x, head = blockIdx.y;
   uint32_t li = 0;
   for (uint32_t i = 1; i < a.n_lanes; ++i)
@@ -226,16 +239,24 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
 
   const uint32_t lane = threadIdx.x, t = lane & 15, g = lane >> 4;
   const uint32_t H = a.kv_heads, G = a.group, M = a.fused_rows;
-  // This wave's MFMA columns are fused rows 16 z .. 16 z + 15 of the tile; a fused
-  // row is (query row, head in group) = (m / G, m % G).
-  const uint32_t m = 16 * blockIdx.z + t, query_row = m / G;
-  const bool in_tile = m < M, live_row = in_tile && query_row < l.active_rows;
-  Sight sight;
-  sight.committed = l.committed;
-  sight.visible = visible;
-  sight.limit = live_row ? min(visible, l.committed + min(query_row, l.active_rows - 1) + 1) : visible;
-  sight.tree = live_row && l.masks != nullptr;
-  sight.mask = sight.tree ? l.masks[query_row] : 0u;
+  // This wave's MFMA columns are fused rows 16 NB z .. of the tile, 16 per block;
+  // a fused row is (query row, head in group) = (m / G, m % G).
+  uint32_t m[NB];
+  bool in_tile[NB], live_row[NB];
+  Sight sight[NB];
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    m[nb] = 16 * (NB * blockIdx.z + nb) + t;
+    const uint32_t query_row = m[nb] / G;
+    in_tile[nb] = m[nb] < M;
+    live_row[nb] = in_tile[nb] && query_row < l.active_rows;
+    sight[nb].committed = l.committed;
+    sight[nb].visible = visible;
+    sight[nb].limit =
+        live_row[nb] ? min(visible, l.committed + min(query_row, l.active_rows - 1) + 1) : visible;
+    sight[nb].tree = live_row[nb] && l.masks != nullptr;
+    sight[nb].mask = sight[nb].tree ? l.masks[query_row] : 0u;
+  }
   const uint32_t db = kPage * H * kRowBytes, sb = kPage * H * 4;
   const RegionOffsets ro = region_offsets(a.kv.extent_pages, db, sb);
   const float score_scale = default_score_scale(kD, l.score_scale);
@@ -244,16 +265,20 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
   // first; everything behind them returns later, so the wait for the queries
   // leaves the page loads in flight.  Columns without a live row carry zeros.
   const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
-  const uint16_t *q_row = q_head + uint64_t(live_row ? m : 0) * kD;
-  u32x4 q_raw[8];
+  u32x4 q_raw[NB][8];
 #pragma unroll
-  for (uint32_t kb = 0; kb < 8; ++kb)
-    q_raw[kb] = load_global<u32x4>(q_row + 8 * (16 * (kb >> 2) + 4 * g + (kb & 3)));
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    const uint16_t *q_row = q_head + uint64_t(live_row[nb] ? m[nb] : 0) * kD;
+#pragma unroll
+    for (uint32_t kb = 0; kb < 8; ++kb)
+      q_raw[nb][kb] = load_global<u32x4>(q_row + 8 * (16 * (kb >> 2) + 4 * g + (kb & 3)));
+  }
 
   // The split's page entries (at most kTableSlots; the launcher declines longer
-  // splits) go through LDS and are read back with uniform LDS loads.  (Fetched from memory one by one they would be
-  // vector loads in the steady loop, and since loads return in order the wait for
-  // an entry would drain every page load in flight.)
+  // splits) go through LDS and are read back with uniform LDS loads.  (Fetched
+  // from memory one by one they would be vector loads in the steady loop, and
+  // since loads return in order the wait for an entry would drain every page
+  // load in flight.)
   __shared__ uint64_t table_lds[kTableSlots];
   for (uint32_t i = lane; i < end - begin; i += 64)
     table_lds[i] = load_global<uint64_t>(l.table + begin + i);
@@ -285,36 +310,43 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
   // Register kb of the staged queries holds the 8 dims of dword
   // w = 16*(kb>>2) + 4g + (kb&3) of a key row in expansion order; odd dims are
   // negated.  q_bias is the constant part of every score.
-  __shared__ u32x4 q_lds[8 * 64];
-  float q_bias = 0.0f;
+  __shared__ u32x4 q_lds[NB][8 * 64];
+  float q_bias[NB];
 #pragma unroll
-  for (uint32_t kb = 0; kb < 8; ++kb) {
-    // dims 8w .. 8w+7 as four bf16 pairs, regrouped to (p, p+4) pairs
-    const u32x4 raw = q_raw[kb];
-    u32x4 q_reg;
-    q_reg[0] = __builtin_amdgcn_perm(raw[2], raw[0], 0x05040100u);
-    q_reg[1] = __builtin_amdgcn_perm(raw[2], raw[0], 0x07060302u) ^ 0x80008000u;
-    q_reg[2] = __builtin_amdgcn_perm(raw[3], raw[1], 0x05040100u);
-    q_reg[3] = __builtin_amdgcn_perm(raw[3], raw[1], 0x07060302u) ^ 0x80008000u;
-    if (!live_row) q_reg = u32x4{0u, 0u, 0u, 0u};
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    q_bias[nb] = 0.0f;
 #pragma unroll
-    for (uint32_t p = 0; p < 4; ++p) {
-      // even dims carry +136 q, odd dims (stored negated) -135 q = +135 stored
-      const float pair_sum =
-          __uint_as_float(q_reg[p] << 16) + __uint_as_float(q_reg[p] & 0xffff0000u);
-      q_bias = fmaf((p & 1) ? 135.0f : 136.0f, pair_sum, q_bias);
+    for (uint32_t kb = 0; kb < 8; ++kb) {
+      // dims 8w .. 8w+7 as four bf16 pairs, regrouped to (p, p+4) pairs
+      const u32x4 raw = q_raw[nb][kb];
+      u32x4 q_reg;
+      q_reg[0] = __builtin_amdgcn_perm(raw[2], raw[0], 0x05040100u);
+      q_reg[1] = __builtin_amdgcn_perm(raw[2], raw[0], 0x07060302u) ^ 0x80008000u;
+      q_reg[2] = __builtin_amdgcn_perm(raw[3], raw[1], 0x05040100u);
+      q_reg[3] = __builtin_amdgcn_perm(raw[3], raw[1], 0x07060302u) ^ 0x80008000u;
+      if (!live_row[nb]) q_reg = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+      for (uint32_t p = 0; p < 4; ++p) {
+        // even dims carry +136 q, odd dims (stored negated) -135 q = +135 stored
+        const float pair_sum =
+            __uint_as_float(q_reg[p] << 16) + __uint_as_float(q_reg[p] & 0xffff0000u);
+        q_bias[nb] = fmaf((p & 1) ? 135.0f : 136.0f, pair_sum, q_bias[nb]);
+      }
+      q_lds[nb][kb * 64 + lane] = q_reg;
     }
-    q_lds[kb * 64 + lane] = q_reg;
+    q_bias[nb] += __shfl_xor(q_bias[nb], 16);
+    q_bias[nb] += __shfl_xor(q_bias[nb], 32);
   }
-  q_bias += __shfl_xor(q_bias, 16);
-  q_bias += __shfl_xor(q_bias, 32);
 
-  State st;
+  State st[NB];
 #pragma unroll
-  for (uint32_t m = 0; m < 16; ++m) st.acc[m] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-  st.row_max = -INFINITY;
-  st.row_sum = 0.0f;
-  st.bias = 0.0f;
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+#pragma unroll
+    for (uint32_t i = 0; i < 16; ++i) st[nb].acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    st[nb].row_max = -INFINITY;
+    st[nb].row_sum = 0.0f;
+    st[nb].bias = 0.0f;
+  }
 
   // Steady state: every refill is unconditional, so the loop body is straight
   // line code and the wait for a set counts exactly the loads issued after it;
@@ -324,8 +356,8 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
   for (; page + 2 * kDepth <= end; page += kDepth) {
 #pragma unroll
     for (uint32_t d = 0; d < kDepth; ++d) {
-      attend_page<false>(r[d], q_lds, q_bias, score_scale, (page + d) * kPage, sight, lane, g,
-                         st);
+      attend_page<false, NB>(r[d], q_lds, q_bias, score_scale, (page + d) * kPage, sight, lane, g,
+                             st);
       fill(r[d], page + d + kDepth - begin);
     }
   }
@@ -334,65 +366,83 @@ __attribute__((amdgpu_waves_per_eu(KVX_DECODE_WAVES, KVX_DECODE_WAVES))) void de
   for (uint32_t k = 0; k < 2 * kDepth - 1; ++k) {
     const uint32_t d = k % kDepth;
     if (page + k < end) {
-      attend_page<true>(r[d], q_lds, q_bias, score_scale, (page + k) * kPage, sight, lane, g,
-                        st);
+      attend_page<true, NB>(r[d], q_lds, q_bias, score_scale, (page + k) * kPage, sight, lane, g,
+                            st);
       if (k + kDepth < 2 * kDepth - 1 && page + k + kDepth < end)
         fill(r[d], page + k + kDepth - begin);
     }
   }
 
-  // Lanes of one q head hold disjoint tokens: combine their sums and the
-  // constant part, then take the constant part out of the accumulators.
-  float row_sum = st.row_sum, bias = st.bias;
-  row_sum += __shfl_xor(row_sum, 16);
-  row_sum += __shfl_xor(row_sum, 32);
-  bias += __shfl_xor(bias, 16);
-  bias += __shfl_xor(bias, 32);
   uint16_t *out_head = output + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
-
-  if (written == 1) {
-    // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
-    // Rows of the tile past the live ones read as zeros (row_sum is 0 there).
-    if (in_tile) {
-      const float denominator = live_row ? row_sum : 0.0f;
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    // Lanes of one column hold disjoint tokens: combine their sums and the
+    // constant part, then take the constant part out of the accumulators.
+    float row_sum = st[nb].row_sum, bias = st[nb].bias;
+    row_sum += __shfl_xor(row_sum, 16);
+    row_sum += __shfl_xor(row_sum, 32);
+    bias += __shfl_xor(bias, 16);
+    bias += __shfl_xor(bias, 32);
+    if (written == 1) {
+      // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
+      // Rows of the tile past the live ones read as zeros (row_sum is 0 there).
+      if (in_tile[nb]) {
+        const float denominator = live_row[nb] ? row_sum : 0.0f;
+#pragma unroll
+        for (uint32_t rr = 0; rr < 4; ++rr)
+#pragma unroll
+          for (uint32_t m4 = 0; m4 < 4; ++m4) {
+            u32x2 packed;
+#pragma unroll
+            for (uint32_t i = 0; i < 2; ++i) {
+              const float lo = st[nb].acc[4 * m4 + 2 * i][rr] - bias;
+              const float hi = st[nb].acc[4 * m4 + 2 * i + 1][rr] - bias;
+              const float qlo = denominator > 0.0f ? __fdiv_rn(lo, denominator) : 0.0f;
+              const float qhi = denominator > 0.0f ? __fdiv_rn(hi, denominator) : 0.0f;
+              packed[i] = uint32_t(f32_to_bf16(qlo)) | (uint32_t(f32_to_bf16(qhi)) << 16);
+            }
+            *reinterpret_cast<u32x2 *>(out_head + uint64_t(m[nb]) * kD + 16 * (4 * g + rr) +
+                                       4 * m4) = packed;
+          }
+      }
+      continue;
+    }
+    if (live_row[nb]) {
+      const uint64_t row =
+          l.row_base + uint64_t(head) * l.split_count * M + uint64_t(split) * M + m[nb];
+      float *out = partials + row * kD;
 #pragma unroll
       for (uint32_t rr = 0; rr < 4; ++rr)
 #pragma unroll
         for (uint32_t m4 = 0; m4 < 4; ++m4) {
-          u32x2 packed;
+          f32x4 v;
 #pragma unroll
-          for (uint32_t i = 0; i < 2; ++i) {
-            const float lo = st.acc[4 * m4 + 2 * i][rr] - bias;
-            const float hi = st.acc[4 * m4 + 2 * i + 1][rr] - bias;
-            const float qlo = denominator > 0.0f ? __fdiv_rn(lo, denominator) : 0.0f;
-            const float qhi = denominator > 0.0f ? __fdiv_rn(hi, denominator) : 0.0f;
-            packed[i] = uint32_t(f32_to_bf16(qlo)) | (uint32_t(f32_to_bf16(qhi)) << 16);
-          }
-          *reinterpret_cast<u32x2 *>(out_head + uint64_t(m) * kD + 16 * (4 * g + rr) + 4 * m4) =
-              packed;
+          for (uint32_t i = 0; i < 4; ++i) v[i] = st[nb].acc[4 * m4 + i][rr] - bias;
+          *reinterpret_cast<f32x4 *>(out + 16 * (4 * g + rr) + 4 * m4) = v;
         }
-    }
-    return;
-  }
-
-  const uint64_t head_row = l.row_base + uint64_t(head) * l.split_count * M;
-  if (live_row) {
-    const uint64_t row = head_row + uint64_t(split) * M + m;
-    float *out = partials + row * kD;
-#pragma unroll
-    for (uint32_t rr = 0; rr < 4; ++rr)
-#pragma unroll
-      for (uint32_t m4 = 0; m4 < 4; ++m4) {
-        f32x4 v;
-#pragma unroll
-        for (uint32_t i = 0; i < 4; ++i) v[i] = st.acc[4 * m4 + i][rr] - bias;
-        *reinterpret_cast<f32x4 *>(out + 16 * (4 * g + rr) + 4 * m4) = v;
+      if (g == 0) {
+        statistics[row * 2] = st[nb].row_max;
+        statistics[row * 2 + 1] = row_sum;
       }
-    if (g == 0) {
-      statistics[row * 2] = st.row_max;
-      statistics[row * 2 + 1] = row_sum;
     }
   }
+}
+
+// One block of 16 fused rows per wave, two waves per SIMD: one-row decode, where
+// the group's query heads are the only rows and memory latency is what to hide.
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_int4_kernel(
+    const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
+    float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
+  attend_int4<1>(queries, output, partials, statistics, a);
+}
+
+// Two blocks per wave share every expanded key and value operand (verify, tree
+// verify, prefill tiles); the accumulators of both take the register file of a
+// whole SIMD lane, so one wave per SIMD.
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void verify_int4_kernel(
+    const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
+    float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
+  attend_int4<2>(queries, output, partials, statistics, a);
 }
 
 }  // namespace
@@ -408,14 +458,26 @@ uint32_t kvx_attend_phases();  // bit 0 = split kernel, bit 1 = merge kernel
 // negative status.  Lane i reads its queries and writes its rows at element
 // offset i * lane_stride; the rows of one KV head lie row_stride * group * 256
 // elements apart.  row_masks: null, or one ancestor bitmask per (lane, row of
-// capacity).  Every lane has the row capacity of the first.
+// capacity).  Every lane has the row capacity of the first.  many_tiles: the
+// lanes are the 8-row tiles of a chunked prefill.
 int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_heads,
                            const void *queries, void *output, const uint64_t *const *page_tables,
                            const kvx_verify_params *lanes, uint32_t n_lanes,
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
-                           void *workspace, uint64_t workspace_bytes, hipStream_t stream) {
+                           void *workspace, uint64_t workspace_bytes, int many_tiles,
+                           hipStream_t stream) {
   if (s->layout.format != KVX_FMT_INT4 || !matrix_attention_covers(s, query_heads, lanes, n_lanes))
     return 1;
+  const uint32_t fused_rows = lanes[0].row_capacity * (query_heads / s->layout.kv_heads);
+  // Sharing the expanded operands between two blocks pays where the lanes are few
+  // and long (verify: 13% on 4 x 65536 tokens x 16 tree rows); chunked prefill has
+  // hundreds of tiles of 48 fused rows, where a half-empty second wave and one
+  // wave per SIMD cost more than the sharing saves.
+  if (fused_rows > 16 && !many_tiles)
+    return launch_matrix_attention(verify_int4_kernel, "verify_int4_kernel", 32, 64, s, kv,
+                                   query_heads, queries, output, page_tables, lanes, n_lanes,
+                                   row_masks, row_stride, lane_stride, workspace, workspace_bytes,
+                                   kvx_attend_phases(), stream);
   return launch_matrix_attention(decode_int4_kernel, "decode_int4_kernel", 16, 64, s, kv,
                                  query_heads, queries, output, page_tables, lanes, n_lanes,
                                  row_masks, row_stride, lane_stride, workspace, workspace_bytes,

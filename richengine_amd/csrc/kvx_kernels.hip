@@ -559,13 +559,15 @@ int kvx_attend_int4_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t
                            const void *queries, void *output, const uint64_t *const *page_tables,
                            const kvx_verify_params *lanes, uint32_t n_lanes,
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
-                           void *workspace, uint64_t workspace_bytes, hipStream_t stream);
+                           void *workspace, uint64_t workspace_bytes, int many_tiles,
+                           hipStream_t stream);
 
 int kvx_attend_wide_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t query_heads,
                            const void *queries, void *output, const uint64_t *const *page_tables,
                            const kvx_verify_params *lanes, uint32_t n_lanes,
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
-                           void *workspace, uint64_t workspace_bytes, hipStream_t stream);
+                           void *workspace, uint64_t workspace_bytes, int many_tiles,
+                           hipStream_t stream);
 
 // int4 pages go to their own kernels, bf16 and fp8 pages to the wide-element
 // ones; 1 = neither covers the shape.
@@ -573,14 +575,15 @@ static int attend_matrix(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_h
                          const void *queries, void *output, const uint64_t *const *page_tables,
                          const kvx_verify_params *lanes, uint32_t n_lanes,
                          const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
-                         void *workspace, uint64_t workspace_bytes, hipStream_t stream) {
+                         void *workspace, uint64_t workspace_bytes, int many_tiles,
+                         hipStream_t stream) {
   const int fast = kvx_attend_int4_launch(s, kv, query_heads, queries, output, page_tables, lanes,
                                           n_lanes, row_masks, row_stride, lane_stride, workspace,
-                                          workspace_bytes, stream);
+                                          workspace_bytes, many_tiles, stream);
   if (fast <= 0) return fast;
   return kvx_attend_wide_launch(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes,
                                 row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                stream);
+                                many_tiles, stream);
 }
 
 uint32_t kvx_attend_phases() { return kvx::g_attend_phases; }
@@ -759,7 +762,7 @@ int kv_attend_verify(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
   const int fast = took(attend_matrix(
       s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks, row_stride,
       uint64_t(s->layout.kv_heads) * row_stride * group * s->layout.head_dim, workspace,
-      workspace_bytes, static_cast<hipStream_t>(stream)));
+      workspace_bytes, 0, static_cast<hipStream_t>(stream)));
   if (fast <= 0) return fast;
   return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks,
                         row_stride, workspace, static_cast<hipStream_t>(stream), 3);
@@ -785,7 +788,7 @@ int kv_attend_decode(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
   const int fast = took(attend_matrix(
       s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, nullptr, row_stride,
       uint64_t(s->layout.kv_heads) * row_stride * group * s->layout.head_dim, workspace,
-      workspace_bytes, static_cast<hipStream_t>(stream)));
+      workspace_bytes, 0, static_cast<hipStream_t>(stream)));
   if (fast <= 0) return fast;
   return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, nullptr,
                         row_stride, workspace, static_cast<hipStream_t>(stream), 3);
@@ -836,7 +839,7 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
                        params->score_scale};
     const int fast = took(attend_matrix(
         s, kv, query_heads, queries, output, tile_tables.data(), tile_lanes.data(), tiles, nullptr,
-        params->chunk_stride, uint64_t(KVX_PREFILL_TILE_ROWS) * G * D, workspace, workspace_bytes, st));
+        params->chunk_stride, uint64_t(KVX_PREFILL_TILE_ROWS) * G * D, workspace, workspace_bytes, 1, st));
     if (fast <= 0) return fast;
   }
   float *partials = static_cast<float *>(workspace);
