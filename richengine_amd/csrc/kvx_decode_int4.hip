@@ -33,8 +33,7 @@ constexpr uint32_t kHeadSlabBytes = kPage * kRowBytes;  // 4 KiB per (head, page
 struct PageRegs {
   u32x4 k[4];   // [token block * 2 + half row]: 16 bytes of the lane's key token
   u32x2 v[8];   // [token slot]: 8 bytes (16 dims) of each of the lane's 8 tokens
-  f32x4 ks[2];  // key scales of the lane's score tokens, per token block
-  f32x4 vs[2];  // value scales, same tokens
+  float scale;  // lane i < 32: key scale of token i; lane 32 + i: value scale of token i
 };
 
 __device__ __forceinline__ f32x4 mfma_bf16(u32x4 a, u32x4 b, f32x4 c) {
@@ -49,6 +48,8 @@ __device__ __forceinline__ f32x4 mfma_bf16(u32x4 a, u32x4 b, f32x4 c) {
 //  p.v : A = values, row t = dims 16t..16t+15 (one MFMA per nibble position),
 //        k-slots = the lane group's 8 tokens 4g..4g+3, 16+4g..16+4g+3.
 //        B = probabilities, column t = q head: exactly the q.k output registers.
+// PARTS: bit 0 the keys, bit 1 values and both scale lines.
+template <uint32_t PARTS>
 __device__ __forceinline__ void load_page(PageRegs &r, uint64_t entry, uint32_t head,
                                           uint32_t kv_heads, uint32_t layer_offset,
                                           uint64_t key_scales_off, uint64_t values_off,
@@ -62,21 +63,25 @@ __device__ __forceinline__ void load_page(PageRegs &r, uint64_t entry, uint32_t 
   const float *key_scales = reinterpret_cast<const float *>(region + key_scales_off) + scale_index;
   const float *value_scales =
       reinterpret_cast<const float *>(region + value_scales_off) + scale_index;
+  if constexpr (PARTS & 1u) {
 #pragma unroll
-  for (uint32_t tb = 0; tb < 2; ++tb)
+    for (uint32_t tb = 0; tb < 2; ++tb)
 #pragma unroll
-    for (uint32_t half = 0; half < 2; ++half)
-      r.k[tb * 2 + half] =
-          load_streaming<u32x4>(keys + (16 * tb + t) * kRowBytes + 64 * half + 16 * g);
-#pragma unroll
-  for (uint32_t s = 0; s < 8; ++s) {
-    const uint32_t token = (s < 4 ? 0 : 16) + 4 * g + (s & 3);
-    r.v[s] = load_streaming<u32x2>(values + token * kRowBytes + 8 * t);
+      for (uint32_t half = 0; half < 2; ++half)
+        r.k[tb * 2 + half] =
+            load_streaming<u32x4>(keys + (16 * tb + t) * kRowBytes + 64 * half + 16 * g);
   }
+  if constexpr (PARTS & 2u) {
 #pragma unroll
-  for (uint32_t tb = 0; tb < 2; ++tb) {
-    r.ks[tb] = load_global<f32x4>(key_scales + 16 * tb + 4 * g);
-    r.vs[tb] = load_global<f32x4>(value_scales + 16 * tb + 4 * g);
+    for (uint32_t s = 0; s < 8; ++s) {
+      const uint32_t token = (s < 4 ? 0 : 16) + 4 * g + (s & 3);
+      r.v[s] = load_streaming<u32x2>(values + token * kRowBytes + 8 * t);
+    }
+    // One scale per lane instead of the sixteen a lane multiplies with: they
+    // are fetched from the owning lanes when the page is attended, which keeps
+    // a register set small enough for three of them.
+    const uint32_t lane = 16 * g + t;
+    r.scale = load_global<float>((lane < kPage ? key_scales : value_scales) + (lane & (kPage - 1)));
   }
 }
 
@@ -92,6 +97,10 @@ __device__ __forceinline__ u32x4 expand_key_dword(uint32_t x) {
   return out;
 }
 
+#ifdef KVX_PROBE_CLOCK
+__device__ uint64_t kvx_probe_log[16384][4];
+#endif
+
 // Softmax state and accumulators of one block of 16 fused query rows.
 struct State {
   f32x4 acc[16];  // [nibble position m]: dims 16*(4g + r) + m of column t
@@ -104,18 +113,21 @@ struct State {
 // operand is expanded once and used by all blocks.
 // MASKED: the page may hold tokens some row does not see (only the last two
 // pages of a sequence can); other pages skip the per-token test.
-template <bool MASKED, uint32_t NB>
-__device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 (*q_lds)[8 * 64],
+// keys_consumed() runs when the page's keys have been read for the last time:
+// the steady loop refills them from there, half a page ahead of the rest.
+template <bool MASKED, uint32_t NB, class KeysConsumed>
+__device__ __forceinline__ void attend_page(PageRegs &r, const u32x4 (*q_lds)[8 * 64],
                                             const float *q_bias, float score_scale,
                                             uint32_t first_token, const Sight *sight,
-                                            uint32_t lane, uint32_t g, State *st) {
+                                            uint32_t lane, uint32_t g, State *st,
+                                            KeysConsumed keys_consumed) {
 #ifdef KVX_PROBE_STREAM_ONLY
   // Measurement build: consume every loaded register with almost no arithmetic,
   // to see what the memory system delivers for this access pattern.
   uint32_t x = 0;
   for (uint32_t i = 0; i < 4; ++i) x ^= r.k[i][0] ^ r.k[i][1] ^ r.k[i][2] ^ r.k[i][3];
   for (uint32_t i = 0; i < 8; ++i) x ^= r.v[i][0] ^ r.v[i][1];
-  st[0].row_sum += r.ks[0][0] + r.ks[1][3] + r.vs[0][1] + r.vs[1][2] + __uint_as_float(x & 0xffu);
+  st[0].row_sum += r.scale + __uint_as_float(x & 0xffu);
   return;
 #endif
   // ---- q.k ----
@@ -135,6 +147,39 @@ __device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 (*q_l
       for (uint32_t nb = 0; nb < NB; ++nb) s[nb][tb] = mfma_bf16(k, q[nb], s[nb][tb]);
     }
   }
+  keys_consumed();
+  // The scales of the lane's eight score tokens, from the lanes that hold them
+  // (lane i: key scale of token i; lane 32 + i: value scale of token i).
+  // One base address per lane and the token's place as the instruction's
+  // constant offset; written out because the compiler would spend a register on
+  // every address.  The data comes back through the LDS return path, hence the
+  // wait inside the block.
+  float ks[8], vs[8];
+  {
+    const uint32_t own = 16 * g;
+    asm volatile(
+        "ds_bpermute_b32 %0, %16, %17\n\t"
+        "ds_bpermute_b32 %1, %16, %17 offset:4\n\t"
+        "ds_bpermute_b32 %2, %16, %17 offset:8\n\t"
+        "ds_bpermute_b32 %3, %16, %17 offset:12\n\t"
+        "ds_bpermute_b32 %4, %16, %17 offset:64\n\t"
+        "ds_bpermute_b32 %5, %16, %17 offset:68\n\t"
+        "ds_bpermute_b32 %6, %16, %17 offset:72\n\t"
+        "ds_bpermute_b32 %7, %16, %17 offset:76\n\t"
+        "ds_bpermute_b32 %8, %16, %17 offset:128\n\t"
+        "ds_bpermute_b32 %9, %16, %17 offset:132\n\t"
+        "ds_bpermute_b32 %10, %16, %17 offset:136\n\t"
+        "ds_bpermute_b32 %11, %16, %17 offset:140\n\t"
+        "ds_bpermute_b32 %12, %16, %17 offset:192\n\t"
+        "ds_bpermute_b32 %13, %16, %17 offset:196\n\t"
+        "ds_bpermute_b32 %14, %16, %17 offset:200\n\t"
+        "ds_bpermute_b32 %15, %16, %17 offset:204\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(ks[0]), "=&v"(ks[1]), "=&v"(ks[2]), "=&v"(ks[3]), "=&v"(ks[4]), "=&v"(ks[5]),
+          "=&v"(ks[6]), "=&v"(ks[7]), "=&v"(vs[0]), "=&v"(vs[1]), "=&v"(vs[2]), "=&v"(vs[3]),
+          "=&v"(vs[4]), "=&v"(vs[5]), "=&v"(vs[6]), "=&v"(vs[7])
+        : "v"(own), "v"(r.scale));
+  }
   // ---- page softmax, per block ----
   u32x4 pb[NB];
 #pragma unroll
@@ -144,7 +189,7 @@ __device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 (*q_l
 #pragma unroll
     for (uint32_t i = 0; i < 8; ++i) {
       const uint32_t tb = i >> 2, rr = i & 3;
-      float v = s[nb][tb][rr] * r.ks[tb][rr];
+      float v = s[nb][tb][rr] * ks[i];
       v *= score_scale;
       live[i] = !MASKED || sight[nb].sees(first_token + 16 * tb + 4 * g + rr);
       score[i] = live[i] ? v : -INFINITY;
@@ -164,7 +209,7 @@ __device__ __forceinline__ void attend_page(const PageRegs &r, const u32x4 (*q_l
       float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
       if (MASKED) p = live[i] ? p : 0.0f;
       page_sum += p;
-      const float w = p * r.vs[i >> 2][i & 3];
+      const float w = p * vs[i];
       weight[i] = live[i] ? w : 0.0f;
     }
     st[nb].row_sum = fmaf(st[nb].row_sum, rescale, page_sum);
@@ -223,6 +268,9 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
                                             float *__restrict__ partials,
                                             float *__restrict__ statistics, const DecodeArgs &a) {
   const uint32_t item = blockIdx.x, head = blockIdx.y;
+#ifdef KVX_PROBE_CLOCK
+  const uint64_t probe_cycles = __builtin_readcyclecounter(), probe_wall = wall_clock64();
+#endif
   uint32_t li = 0;
   for (uint32_t i = 1; i < a.n_lanes; ++i)
     if (item >= a.lane[i].first_item) li = i;
@@ -297,8 +345,28 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     // second copy of its registers, and interleaved with another fill's loads
     // they would make every wait cover both.
     asm volatile("");
-    load_page(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values,
-              ro.value_scales, t, g);
+    load_page<3>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values,
+                 ro.value_scales, t, g);
+    asm volatile("");
+  };
+  // The same in two steps for the steady loop: the keys as soon as the page that
+  // held the set has multiplied its last key, the rest when the page is done.
+  auto fill_keys = [&](PageRegs &set, uint32_t slot) {
+#ifdef KVX_PROBE_SAME_PAGE
+    slot = 0;
+#endif
+    asm volatile("");
+    load_page<1>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values,
+                 ro.value_scales, t, g);
+    asm volatile("");
+  };
+  auto fill_rest = [&](PageRegs &set, uint32_t slot) {
+#ifdef KVX_PROBE_SAME_PAGE
+    slot = 0;
+#endif
+    asm volatile("");
+    load_page<2>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values,
+                 ro.value_scales, t, g);
     asm volatile("");
   };
   // The first fills are unconditional too (a split shorter than kDepth pages
@@ -356,9 +424,10 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   for (; page + 2 * kDepth <= end; page += kDepth) {
 #pragma unroll
     for (uint32_t d = 0; d < kDepth; ++d) {
+      const uint32_t refill = page + d + kDepth - begin;
       attend_page<false, NB>(r[d], q_lds, q_bias, score_scale, (page + d) * kPage, sight, lane, g,
-                             st);
-      fill(r[d], page + d + kDepth - begin);
+                             st, [&] { fill_keys(r[d], refill); });
+      fill_rest(r[d], refill);
     }
   }
   // Tail: at most 2 * kDepth - 1 pages are left, the first kDepth of them loaded.
@@ -367,12 +436,25 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     const uint32_t d = k % kDepth;
     if (page + k < end) {
       attend_page<true, NB>(r[d], q_lds, q_bias, score_scale, (page + k) * kPage, sight, lane, g,
-                            st);
+                            st, [] {});
       if (k + kDepth < 2 * kDepth - 1 && page + k + kDepth < end)
         fill(r[d], page + k + kDepth - begin);
     }
   }
 
+#ifdef KVX_PROBE_CLOCK
+  // Measurement build: when and where every wave ran.
+  if (threadIdx.x == 0) {
+    const uint32_t slot = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    if (slot < 16384) {
+      kvx_probe_log[slot][0] = probe_wall;
+      kvx_probe_log[slot][1] = wall_clock64();
+      kvx_probe_log[slot][2] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11)) |
+                               (uint64_t(__builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11))) << 32);
+      kvx_probe_log[slot][3] = end - begin;
+    }
+  }
+#endif
   uint16_t *out_head = output + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
 #pragma unroll
   for (uint32_t nb = 0; nb < NB; ++nb) {
@@ -483,3 +565,9 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                                  row_masks, row_stride, lane_stride, workspace, workspace_bytes,
                                  kvx_attend_phases(), stream);
 }
+
+#ifdef KVX_PROBE_CLOCK
+extern "C" int kvx_probe_fetch(uint64_t *host, uint32_t slots) {
+  return hipMemcpyFromSymbol(host, HIP_SYMBOL(kvx::kvx_probe_log), uint64_t(slots) * 32) == hipSuccess ? 0 : -1;
+}
+#endif
