@@ -115,8 +115,9 @@ struct State {
 // pages of a sequence can); other pages skip the per-token test.
 // keys_consumed() runs when the page's keys have been read for the last time:
 // the steady loop refills them from there, half a page ahead of the rest.
-template <bool MASKED, uint32_t NB, class KeysConsumed>
-__device__ __forceinline__ void attend_page(PageRegs &r, const u32x4 (*q_lds)[8 * 64],
+// queries(nb, kb) yields the B operand of block nb for dims block kb.
+template <bool MASKED, uint32_t NB, class Queries, class KeysConsumed>
+__device__ __forceinline__ void attend_page(PageRegs &r, Queries queries,
                                             const float *q_bias, float score_scale,
                                             uint32_t first_token, const Sight *sight,
                                             uint32_t lane, uint32_t g, State *st,
@@ -139,7 +140,7 @@ __device__ __forceinline__ void attend_page(PageRegs &r, const u32x4 (*q_lds)[8 
   for (uint32_t kb = 0; kb < 8; ++kb) {
     u32x4 q[NB];
 #pragma unroll
-    for (uint32_t nb = 0; nb < NB; ++nb) q[nb] = q_lds[nb][kb * 64 + lane];
+    for (uint32_t nb = 0; nb < NB; ++nb) q[nb] = queries(nb, kb);
 #pragma unroll
     for (uint32_t tb = 0; tb < 2; ++tb) {
       const u32x4 k = expand_key_dword(r.k[tb * 2 + (kb >> 2)][kb & 3]);
@@ -260,6 +261,72 @@ __device__ __forceinline__ void attend_page(PageRegs &r, const u32x4 (*q_lds)[8 
 #define KVX_DECODE_DEPTH 2
 #endif
 constexpr uint32_t kDepth = KVX_DECODE_DEPTH;
+
+// Writes what a wave has accumulated for its NB blocks: the finished bf16 rows
+// when the lane has a single split, else fp32 partial rows and (max, sum).
+template <uint32_t NB>
+__device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m, const bool *in_tile,
+                                             const bool *live_row, const DecodeLane &l,
+                                             const DecodeArgs &a, uint32_t head, uint32_t split,
+                                             uint32_t written, uint32_t g,
+                                             uint16_t *__restrict__ output,
+                                             float *__restrict__ partials,
+                                             float *__restrict__ statistics) {
+  const uint32_t G = a.group, M = a.fused_rows;
+  uint16_t *out_head = output + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    // Lanes of one column hold disjoint tokens: combine their sums and the
+    // constant part, then take the constant part out of the accumulators.
+    float row_sum = st[nb].row_sum, bias = st[nb].bias;
+    row_sum += __shfl_xor(row_sum, 16);
+    row_sum += __shfl_xor(row_sum, 32);
+    bias += __shfl_xor(bias, 16);
+    bias += __shfl_xor(bias, 32);
+    if (written == 1) {
+      // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
+      // Rows of the tile past the live ones read as zeros (row_sum is 0 there).
+      if (in_tile[nb]) {
+        const float denominator = live_row[nb] ? row_sum : 0.0f;
+#pragma unroll
+        for (uint32_t rr = 0; rr < 4; ++rr)
+#pragma unroll
+          for (uint32_t m4 = 0; m4 < 4; ++m4) {
+            u32x2 packed;
+#pragma unroll
+            for (uint32_t i = 0; i < 2; ++i) {
+              const float lo = st[nb].acc[4 * m4 + 2 * i][rr] - bias;
+              const float hi = st[nb].acc[4 * m4 + 2 * i + 1][rr] - bias;
+              const float qlo = denominator > 0.0f ? __fdiv_rn(lo, denominator) : 0.0f;
+              const float qhi = denominator > 0.0f ? __fdiv_rn(hi, denominator) : 0.0f;
+              packed[i] = uint32_t(f32_to_bf16(qlo)) | (uint32_t(f32_to_bf16(qhi)) << 16);
+            }
+            *reinterpret_cast<u32x2 *>(out_head + uint64_t(m[nb]) * kD + 16 * (4 * g + rr) +
+                                       4 * m4) = packed;
+          }
+      }
+      continue;
+    }
+    if (live_row[nb]) {
+      const uint64_t row =
+          l.row_base + uint64_t(head) * l.split_count * M + uint64_t(split) * M + m[nb];
+      float *out = partials + row * kD;
+#pragma unroll
+      for (uint32_t rr = 0; rr < 4; ++rr)
+#pragma unroll
+        for (uint32_t m4 = 0; m4 < 4; ++m4) {
+          f32x4 v;
+#pragma unroll
+          for (uint32_t i = 0; i < 4; ++i) v[i] = st[nb].acc[4 * m4 + i][rr] - bias;
+          *reinterpret_cast<f32x4 *>(out + 16 * (4 * g + rr) + 4 * m4) = v;
+        }
+      if (g == 0) {
+        statistics[row * 2] = st[nb].row_max;
+        statistics[row * 2 + 1] = row_sum;
+      }
+    }
+  }
+}
 
 // The split kernel's body for NB blocks of 16 fused query rows per wave.
 template <uint32_t NB>
@@ -415,6 +482,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     st[nb].row_sum = 0.0f;
     st[nb].bias = 0.0f;
   }
+  auto staged_queries = [&](uint32_t nb, uint32_t kb) { return q_lds[nb][kb * 64 + lane]; };
 
   // Steady state: every refill is unconditional, so the loop body is straight
   // line code and the wait for a set counts exactly the loads issued after it;
@@ -425,7 +493,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
 #pragma unroll
     for (uint32_t d = 0; d < kDepth; ++d) {
       const uint32_t refill = page + d + kDepth - begin;
-      attend_page<false, NB>(r[d], q_lds, q_bias, score_scale, (page + d) * kPage, sight, lane, g,
+      attend_page<false, NB>(r[d], staged_queries, q_bias, score_scale, (page + d) * kPage, sight, lane, g,
                              st, [&] { fill_keys(r[d], refill); });
       fill_rest(r[d], refill);
     }
@@ -435,7 +503,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   for (uint32_t k = 0; k < 2 * kDepth - 1; ++k) {
     const uint32_t d = k % kDepth;
     if (page + k < end) {
-      attend_page<true, NB>(r[d], q_lds, q_bias, score_scale, (page + k) * kPage, sight, lane, g,
+      attend_page<true, NB>(r[d], staged_queries, q_bias, score_scale, (page + k) * kPage, sight, lane, g,
                             st, [] {});
       if (k + kDepth < 2 * kDepth - 1 && page + k + kDepth < end)
         fill(r[d], page + k + kDepth - begin);
@@ -455,59 +523,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     }
   }
 #endif
-  uint16_t *out_head = output + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
-#pragma unroll
-  for (uint32_t nb = 0; nb < NB; ++nb) {
-    // Lanes of one column hold disjoint tokens: combine their sums and the
-    // constant part, then take the constant part out of the accumulators.
-    float row_sum = st[nb].row_sum, bias = st[nb].bias;
-    row_sum += __shfl_xor(row_sum, 16);
-    row_sum += __shfl_xor(row_sum, 32);
-    bias += __shfl_xor(bias, 16);
-    bias += __shfl_xor(bias, 32);
-    if (written == 1) {
-      // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
-      // Rows of the tile past the live ones read as zeros (row_sum is 0 there).
-      if (in_tile[nb]) {
-        const float denominator = live_row[nb] ? row_sum : 0.0f;
-#pragma unroll
-        for (uint32_t rr = 0; rr < 4; ++rr)
-#pragma unroll
-          for (uint32_t m4 = 0; m4 < 4; ++m4) {
-            u32x2 packed;
-#pragma unroll
-            for (uint32_t i = 0; i < 2; ++i) {
-              const float lo = st[nb].acc[4 * m4 + 2 * i][rr] - bias;
-              const float hi = st[nb].acc[4 * m4 + 2 * i + 1][rr] - bias;
-              const float qlo = denominator > 0.0f ? __fdiv_rn(lo, denominator) : 0.0f;
-              const float qhi = denominator > 0.0f ? __fdiv_rn(hi, denominator) : 0.0f;
-              packed[i] = uint32_t(f32_to_bf16(qlo)) | (uint32_t(f32_to_bf16(qhi)) << 16);
-            }
-            *reinterpret_cast<u32x2 *>(out_head + uint64_t(m[nb]) * kD + 16 * (4 * g + rr) +
-                                       4 * m4) = packed;
-          }
-      }
-      continue;
-    }
-    if (live_row[nb]) {
-      const uint64_t row =
-          l.row_base + uint64_t(head) * l.split_count * M + uint64_t(split) * M + m[nb];
-      float *out = partials + row * kD;
-#pragma unroll
-      for (uint32_t rr = 0; rr < 4; ++rr)
-#pragma unroll
-        for (uint32_t m4 = 0; m4 < 4; ++m4) {
-          f32x4 v;
-#pragma unroll
-          for (uint32_t i = 0; i < 4; ++i) v[i] = st[nb].acc[4 * m4 + i][rr] - bias;
-          *reinterpret_cast<f32x4 *>(out + 16 * (4 * g + rr) + 4 * m4) = v;
-        }
-      if (g == 0) {
-        statistics[row * 2] = st[nb].row_max;
-        statistics[row * 2 + 1] = row_sum;
-      }
-    }
-  }
+  write_blocks<NB>(st, m, in_tile, live_row, l, a, head, split, written, g, output, partials, statistics);
 }
 
 // One block of 16 fused rows per wave, two waves per SIMD: one-row decode, where
