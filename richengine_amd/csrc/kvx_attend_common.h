@@ -92,16 +92,24 @@ struct MergeSums {
 };
 
 // Sums splits [first, last) of the row in split order; `maximum` is the row's
-// maximum over all splits.
+// maximum over all splits.  With PREFETCHED, `early` holds the partial rows of
+// the first eight splits (clamped to the last), loaded before the caller
+// waited for the statistics.
+template <bool PREFETCHED>
 __device__ __forceinline__ MergeSums merge_range(const float *__restrict__ partials,
                                                  const float *__restrict__ statistics,
                                                  uint64_t first_row, uint32_t first, uint32_t last,
-                                                 uint32_t M, float maximum, uint32_t lane) {
+                                                 uint32_t M, float maximum, uint32_t lane,
+                                                 const f32x4 (&early)[8], f32x2 early_stat) {
   MergeSums sums{{0.0f, 0.0f, 0.0f, 0.0f}, 0.0f};
   for (uint32_t base = first; base < last; base += 64) {
     const uint32_t mine = base + lane;
     f32x2 stat = {-INFINITY, 0.0f};
-    if (mine < last) stat = load_global<f32x2>(statistics + (first_row + uint64_t(mine) * M) * 2);
+    if (PREFETCHED && base == first) {
+      stat = early_stat;
+    } else if (mine < last) {
+      stat = load_global<f32x2>(statistics + (first_row + uint64_t(mine) * M) * 2);
+    }
     const float my_weight = expf(__fsub_rn(stat[0], maximum));
     const float my_term = __fmul_rn(my_weight, stat[1]);
     const uint32_t count = min(64u, last - base);
@@ -109,8 +117,12 @@ __device__ __forceinline__ MergeSums merge_range(const float *__restrict__ parti
       f32x4 part[8];
 #pragma unroll
       for (uint32_t u = 0; u < 8; ++u) {
-        const uint64_t row = first_row + uint64_t(base + min(i + u, count - 1)) * M;
-        part[u] = load_global<f32x4>(partials + row * kD + 4 * lane);
+        if (PREFETCHED && base == first && i == 0) {
+          part[u] = early[u];
+        } else {
+          const uint64_t row = first_row + uint64_t(base + min(i + u, count - 1)) * M;
+          part[u] = load_global<f32x4>(partials + row * kD + 4 * lane);
+        }
       }
 #pragma unroll
       for (uint32_t u = 0; u < 8; ++u) {
@@ -149,22 +161,38 @@ __global__ __launch_bounds__(64 * kMergeWaves) void matrix_merge_kernel(
   const uint64_t first_row = l.row_base + uint64_t(head) * l.split_count * M + j;
   const bool sequential = written <= kMergeSequential;
   if (sequential && wave) return;
+  // The sequential case (at most 64 splits) issues its statistics and the
+  // first eight partial rows together, before anything waits.
+  f32x4 early[8];
+  f32x2 early_stat = {-INFINITY, 0.0f};
   float maximum = -INFINITY;
-  for (uint32_t base = 0; base < written; base += 64) {
-    const uint32_t s = base + lane;
-    float m = s < written ? load_global<float>(statistics + (first_row + uint64_t(s) * M) * 2)
-                          : -INFINITY;
+  if (sequential) {
+    if (lane < written)
+      early_stat = load_global<f32x2>(statistics + (first_row + uint64_t(lane) * M) * 2);
 #pragma unroll
-    for (uint32_t step = 32; step > 0; step >>= 1) m = fmaxf(m, __shfl_xor(m, step));
-    maximum = fmaxf(maximum, m);
+    for (uint32_t u = 0; u < 8; ++u)
+      early[u] = load_global<f32x4>(partials + (first_row + uint64_t(min(u, written - 1)) * M) * kD +
+                                    4 * lane);
+    maximum = early_stat[0];
+    for (int offset = 32; offset; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset));
+  } else {
+    for (uint32_t base = 0; base < written; base += 64) {
+      const uint32_t s = base + lane;
+      float m = s < written ? load_global<float>(statistics + (first_row + uint64_t(s) * M) * 2)
+                            : -INFINITY;
+      for (int offset = 32; offset; offset >>= 1) m = fmaxf(m, __shfl_xor(m, offset));
+      maximum = fmaxf(maximum, m);
+    }
   }
   MergeSums sums;
   if (sequential) {
-    sums = merge_range(partials, statistics, first_row, 0, written, M, maximum, lane);
+    sums = merge_range<true>(partials, statistics, first_row, 0, written, M, maximum, lane, early,
+                             early_stat);
   } else {
     const uint32_t share = (written + kMergeWaves - 1) / kMergeWaves;
     const uint32_t first = min(written, wave * share), last = min(written, first + share);
-    const MergeSums mine = merge_range(partials, statistics, first_row, first, last, M, maximum, lane);
+    const MergeSums mine = merge_range<false>(partials, statistics, first_row, first, last, M,
+                                              maximum, lane, early, early_stat);
     __shared__ f32x4 numerators[kMergeWaves][64];
     __shared__ float denominators[kMergeWaves][64];
     numerators[wave][lane] = mine.numerator;

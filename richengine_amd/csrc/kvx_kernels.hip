@@ -26,6 +26,7 @@ struct AppendArgs {
   uint32_t n_lanes;
   uint32_t kv_heads, head_dim;
   uint32_t verify_max_rows;
+  uint32_t uniform_groups;  // workgroups per lane when every lane stores the same rows, else 0
   kvx_kv_layer kv;
   uint64_t lane_stride;
 };
@@ -55,8 +56,12 @@ __global__ __launch_bounds__(256) void append_kernel(const uint16_t *__restrict_
   __shared__ float wave_max[4];
   const uint32_t group = blockIdx.x;
   uint32_t li = 0;
-  for (uint32_t i = 1; i < a.n_lanes; ++i)
-    if (group >= a.lane[i].group_base) li = i;
+  if (a.uniform_groups) {
+    li = group / a.uniform_groups;
+  } else {
+    for (uint32_t i = 1; i < a.n_lanes; ++i)
+      if (group >= a.lane[i].group_base) li = i;
+  }
   const AppendLane &l = a.lane[li];
   if (!append_contract(l, a)) return;
   const uint32_t D = a.head_dim, H = a.kv_heads;
@@ -68,11 +73,12 @@ __global__ __launch_bounds__(256) void append_kernel(const uint16_t *__restrict_
   const uint32_t token = row % l.tokens, head = row / l.tokens;
   const uint32_t d = threadIdx.x;
   const uint32_t logical = l.committed + token;
-  const Slab s = slab_of(FMT, H, D, a.kv, head, l.table[logical / kPage]);
-  const uint32_t slot = logical % kPage;
+  // The row's source does not depend on the page entry: both loads are in flight together.
   const uint16_t source =
       value_tensor ? chunk_values[li * a.lane_stride + (uint64_t(head) * D + d) * l.stride + token]
                    : chunk_keys[li * a.lane_stride + (uint64_t(head) * l.stride + token) * D + d];
+  const Slab s = slab_of(FMT, H, D, a.kv, head, l.table[logical / kPage]);
+  const uint32_t slot = logical % kPage;
   uint8_t *data = value_tensor ? s.values : s.keys;
   // Element index inside the head's slab: keys token-major, values
   // dimension-major (packed int4: both token-major).
@@ -641,6 +647,9 @@ int kv_append(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
                    p.page_table_entries, groups, 0};
       groups += 2 * p.chunk_tokens * H;
     }
+    a.uniform_groups = 2 * lanes[first].chunk_tokens * H;
+    for (uint32_t i = 0; i < a.n_lanes; ++i)
+      if (lanes[first + i].chunk_tokens != lanes[first].chunk_tokens) a.uniform_groups = 0;
     const auto *keys = static_cast<const uint16_t *>(chunk_keys) + uint64_t(first) * lane_stride;
     const auto *values = static_cast<const uint16_t *>(chunk_values) + uint64_t(first) * lane_stride;
     const int rc = dispatch_format(s->layout.format, [&](auto fmt) {
