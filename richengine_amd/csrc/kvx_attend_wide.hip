@@ -1,11 +1,11 @@
-// bf16 and fp8-e4m3 paged attention for gfx950: the split kernel of
+// bf16, fp8-e4m3 and int8 paged attention for gfx950: the split kernel of
 // kv_attend_decode, kv_attend_verify and kv_attend_prefill for pages whose
-// elements are two bytes (bf16) or one byte (fp8) wide, head dimension 256.
+// elements are two bytes (bf16) or one byte (fp8, int8) wide, head dimension 256.
 //
 // One wave per (sequence or prefill tile, split, KV head, group of NB blocks of
 // 16 fused query rows).  The wave streams the split's pages once; keys and
 // values are the A operands of 16x16x32 MFMAs as they lie in the page (bf16) or
-// after an exact byte -> fp16 expansion (fp8), and all NB row blocks reuse
+// after an exact byte -> fp16 expansion (fp8, int8), and all NB row blocks reuse
 // them.  The arithmetic follows the reference tiles
 // (common/paged_attention_tile.h:85-349 for bf16,
 // common/paged_attention_fp8_tile.h:34-265 for fp8): page-granular online
@@ -18,6 +18,13 @@
 // subnormals included, because both formats then share mantissa alignment and
 // differ by the bias 15 - 7.  The factor 2^8 is applied in fp32, where it is
 // exact (to the scores with the key scale, to the accumulators at the end).
+//
+// int8 -> fp16 without a table: the code's byte with its top bit flipped is
+// u = c + 128 in 1..255, 0x6400 | u is the fp16 number 1024 + u exactly, and a
+// packed fp16 subtraction of 1152 leaves the code itself, exactly.  Queries and
+// probabilities meet the codes as fp16: a bf16 query, or a probability already
+// rounded to bf16 as the reference tile rounds it, converts without loss unless
+// its magnitude is below 2^-14, far under the tolerance.
 #include "kvx_attend_common.h"
 
 namespace kvx {
@@ -29,14 +36,16 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 template <uint32_t FMT>
 struct Wide {
   static constexpr bool kFp8 = FMT == KVX_FMT_FP8E4M3;
-  static constexpr uint32_t kBytes = kFp8 ? 1 : 2;                   // per element
+  static constexpr bool kInt8 = FMT == KVX_FMT_INT8;
+  static constexpr bool kByte = kFp8 || kInt8;                       // one byte per element, scaled
+  static constexpr uint32_t kBytes = kByte ? 1 : 2;                  // per element
   static constexpr uint32_t kSlab = kPage * kD * kBytes;             // per (head, page, tensor)
-  static constexpr uint32_t kDwords = kFp8 ? 2 : 4;                  // raw dwords per MFMA operand
+  static constexpr uint32_t kDwords = kByte ? 2 : 4;                 // raw dwords per MFMA operand
 };
 
 template <uint32_t FMT>
 __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
-  if constexpr (Wide<FMT>::kFp8)
+  if constexpr (Wide<FMT>::kByte)
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   else
@@ -54,6 +63,20 @@ __device__ __forceinline__ uint32_t fp8_pair(uint32_t x, uint32_t select) {
 __device__ __forceinline__ u32x4 fp8_operand(uint32_t first, uint32_t second) {
   return u32x4{fp8_pair(first, 0x0c010c00u), fp8_pair(first, 0x0c030c02u),
                fp8_pair(second, 0x0c010c00u), fp8_pair(second, 0x0c030c02u)};
+}
+
+// Two int8 codes (bytes of x flipped in the top bit, selected by the perm
+// pattern under the constant byte 0x64) to two fp16 halves holding the codes.
+__device__ __forceinline__ uint32_t int8_pair(uint32_t flipped, uint32_t select) {
+  const uint32_t biased = __builtin_amdgcn_perm(0x64646464u, flipped, select);  // 1024 + u each
+  const f16x2 codes = __builtin_bit_cast(f16x2, biased) - f16x2{_Float16(1152.0f), _Float16(1152.0f)};
+  return __builtin_bit_cast(uint32_t, codes);
+}
+// Eight consecutive int8 codes (two dwords) to eight fp16 in order.
+__device__ __forceinline__ u32x4 int8_operand(uint32_t first, uint32_t second) {
+  const uint32_t a = first ^ 0x80808080u, b = second ^ 0x80808080u;
+  return u32x4{int8_pair(a, 0x04010400u), int8_pair(a, 0x04030402u), int8_pair(b, 0x04010400u),
+               int8_pair(b, 0x04030402u)};
 }
 
 // What one lane holds of one page's keys / values.
@@ -100,7 +123,7 @@ __device__ __forceinline__ void load_keys(KeyRegs<FMT> &k, const PagePlace &p, u
 #pragma unroll
     for (uint32_t kb = 0; kb < 8; ++kb) {
       const uint8_t *at = p.keys + ((16 * tb + t) * kD + 32 * kb + 8 * g) * B;
-      if constexpr (Wide<FMT>::kFp8) {
+      if constexpr (Wide<FMT>::kByte) {
         const u32x2 v = load_streaming<u32x2>(at);
         k.raw[tb][kb][0] = v[0];
         k.raw[tb][kb][1] = v[1];
@@ -120,7 +143,7 @@ __device__ __forceinline__ void load_values(ValueRegs<FMT> &v, const PagePlace &
 #pragma unroll
     for (uint32_t half = 0; half < 2; ++half) {
       const uint8_t *at = p.values + ((16 * mb + t) * kPage + 16 * half + 4 * g) * B;
-      if constexpr (Wide<FMT>::kFp8) {
+      if constexpr (Wide<FMT>::kByte) {
         v.raw[mb][half] = load_streaming<uint32_t>(at);
       } else {
         const u32x2 x = load_streaming<u32x2>(at);
@@ -132,11 +155,13 @@ __device__ __forceinline__ void load_values(ValueRegs<FMT> &v, const PagePlace &
 template <uint32_t FMT>
 __device__ __forceinline__ u32x4 key_operand(const KeyRegs<FMT> &k, uint32_t tb, uint32_t kb) {
   if constexpr (Wide<FMT>::kFp8) return fp8_operand(k.raw[tb][kb][0], k.raw[tb][kb][1]);
+  else if constexpr (Wide<FMT>::kInt8) return int8_operand(k.raw[tb][kb][0], k.raw[tb][kb][1]);
   else return u32x4{k.raw[tb][kb][0], k.raw[tb][kb][1], k.raw[tb][kb][2], k.raw[tb][kb][3]};
 }
 template <uint32_t FMT>
 __device__ __forceinline__ u32x4 value_operand(const ValueRegs<FMT> &v, uint32_t mb) {
   if constexpr (Wide<FMT>::kFp8) return fp8_operand(v.raw[mb][0], v.raw[mb][1]);
+  else if constexpr (Wide<FMT>::kInt8) return int8_operand(v.raw[mb][0], v.raw[mb][1]);
   else return u32x4{v.raw[mb][0], v.raw[mb][1], v.raw[mb][2], v.raw[mb][3]};
 }
 
@@ -146,7 +171,7 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
                                                          float *__restrict__ partials,
                                                          float *__restrict__ statistics,
                                                          DecodeArgs a) {
-  constexpr bool kFp8 = Wide<FMT>::kFp8;
+  constexpr bool kFp8 = Wide<FMT>::kFp8, kInt8 = Wide<FMT>::kInt8, kByte = Wide<FMT>::kByte;
   const uint32_t item = blockIdx.x, head = blockIdx.y;
   uint32_t li = 0;
   for (uint32_t i = 1; i < a.n_lanes; ++i)
@@ -164,7 +189,7 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
 
   const uint32_t lane = threadIdx.x, t = lane & 15, g = lane >> 4;
   const uint32_t H = a.kv_heads, G = a.group, M = a.fused_rows;
-  const uint32_t db = Wide<FMT>::kSlab * H, sb = kFp8 ? kPage * H * 4 : 0;
+  const uint32_t db = Wide<FMT>::kSlab * H, sb = kByte ? kPage * H * 4 : 0;
   const RegionOffsets ro = region_offsets(a.kv.extent_pages, db, sb);
   const float score_scale = default_score_scale(kD, l.score_scale);
 
@@ -187,8 +212,8 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
   }
 
   // Queries: [row][g][D] bf16, fused row m; register kb of a column holds dims
-  // 32*kb + 8g .. + 7.  fp8 pages stage them as fp16.  Columns without a live row
-  // carry zeros.
+  // 32*kb + 8g .. + 7.  fp8 and int8 pages stage them as fp16.  Columns without a
+  // live row carry zeros.
   const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
   __shared__ u32x4 q_lds[NB][8][64];
   __shared__ uint64_t table_lds[kTableSlots];
@@ -198,7 +223,7 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
 #pragma unroll
     for (uint32_t kb = 0; kb < 8; ++kb) {
       u32x4 q = load_global<u32x4>(q_row + 32 * kb + 8 * g);
-      if constexpr (kFp8) {
+      if constexpr (kByte) {
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) {
           const f16x2 pair = {_Float16(__uint_as_float(q[i] << 16)),
@@ -218,12 +243,12 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
 
   KeyRegs<FMT> keys;
   ValueRegs<FMT> values;
-  f32x4 ks[2], vs[2];  // fp8: scales of the lane's score tokens, per token block
+  f32x4 ks[2], vs[2];  // fp8, int8: scales of the lane's score tokens, per token block
   auto fetch_keys = [&](uint32_t slot) {
     const PagePlace p = place_page<FMT>(table_lds[slot], head, H, a.kv.offset, ro);
     asm volatile("");  // the loads of one fetch stay together and in place
     load_keys<FMT>(keys, p, t, g);
-    if constexpr (kFp8) {
+    if constexpr (kByte) {
       ks[0] = load_global<f32x4>(p.key_scales + 4 * g);
       ks[1] = load_global<f32x4>(p.key_scales + 16 + 4 * g);
     }
@@ -233,7 +258,7 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
     const PagePlace p = place_page<FMT>(table_lds[slot], head, H, a.kv.offset, ro);
     asm volatile("");
     load_values<FMT>(values, p, t, g);
-    if constexpr (kFp8) {
+    if constexpr (kByte) {
       vs[0] = load_global<f32x4>(p.value_scales + 4 * g);
       vs[1] = load_global<f32x4>(p.value_scales + 16 + 4 * g);
     }
@@ -272,7 +297,7 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
         for (uint32_t nb = 0; nb < NB; ++nb) s[nb][tb] = mfma<FMT>(k, q_lds[nb][kb][lane], s[nb][tb]);
       }
     f32x4 page_ks[2];
-    if constexpr (kFp8) {
+    if constexpr (kByte) {
       page_ks[0] = ks[0];
       page_ks[1] = ks[1];
     }
@@ -281,7 +306,7 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
     const uint32_t first_token = page * kPage;
     u32x4 pb[NB];
     f32x4 page_vs[2];
-    if constexpr (kFp8) {
+    if constexpr (kByte) {
       page_vs[0] = vs[0];
       page_vs[1] = vs[1];
     }
@@ -293,7 +318,7 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
       for (uint32_t i = 0; i < 8; ++i) {
         const uint32_t tb = i >> 2, rr = i & 3;
         float v = s[nb][tb][rr] * kUnscale;
-        if constexpr (kFp8) v *= page_ks[tb][rr];
+        if constexpr (kByte) v *= page_ks[tb][rr];
         v *= score_scale;
         live[i] = sight[nb].sees(first_token + 16 * tb + 4 * g + rr);
         score[i] = live[i] ? v : -INFINITY;
@@ -313,7 +338,7 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
         float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
         p = live[i] ? p : 0.0f;
         page_sum += p;
-        weight[i] = kFp8 ? p * page_vs[i >> 2][i & 3] : p;
+        weight[i] = kByte ? p * page_vs[i >> 2][i & 3] : p;
       }
       row_sum[nb] = fmaf(row_sum[nb], rescale, page_sum);
       row_max[nb] = next_max;
@@ -321,6 +346,13 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
       for (uint32_t p = 0; p < 4; ++p) {
         if constexpr (kFp8) {
           const f16x2 pair = {_Float16(weight[2 * p]), _Float16(weight[2 * p + 1])};
+          pb[nb][p] = __builtin_bit_cast(uint32_t, pair);
+        } else if constexpr (kInt8) {
+          // Rounded to bf16 as the reference tile does, then carried as fp16.
+          const f32x2 wide = {weight[2 * p], weight[2 * p + 1]};
+          const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(wide, bf16x2));
+          const f16x2 pair = {_Float16(__uint_as_float(bits << 16)),
+                              _Float16(__uint_as_float(bits & 0xffff0000u))};
           pb[nb][p] = __builtin_bit_cast(uint32_t, pair);
         } else {
           const f32x2 pair = {weight[2 * p], weight[2 * p + 1]};
@@ -401,7 +433,7 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
                            hipStream_t stream) {
   const uint32_t format = s->layout.format;
-  if ((format != KVX_FMT_BF16 && format != KVX_FMT_FP8E4M3) ||
+  if ((format != KVX_FMT_BF16 && format != KVX_FMT_FP8E4M3 && format != KVX_FMT_INT8) ||
       !matrix_attention_covers(s, query_heads, lanes, n_lanes))
     return 1;
   const uint32_t M = lanes[0].row_capacity * (query_heads / s->layout.kv_heads);
@@ -417,6 +449,7 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   // layer with two blocks per wave against 10.1 with one; fp8, whose byte
   // expansion makes it VALU-bound at one wave per SIMD, 14.2 against 12.1.
   if (format == KVX_FMT_BF16) return M > 16 ? KVX_WIDE(KVX_FMT_BF16, 2) : KVX_WIDE(KVX_FMT_BF16, 1);
+  if (format == KVX_FMT_INT8) return M > 16 ? KVX_WIDE(KVX_FMT_INT8, 2) : KVX_WIDE(KVX_FMT_INT8, 1);
   return M > 16 && !many_tiles ? KVX_WIDE(KVX_FMT_FP8E4M3, 2) : KVX_WIDE(KVX_FMT_FP8E4M3, 1);
 #undef KVX_WIDE
 }

@@ -48,41 +48,82 @@ __device__ __forceinline__ f32x4 mfma_bf16(u32x4 a, u32x4 b, f32x4 c) {
 //  p.v : A = values, row t = dims 16t..16t+15 (one MFMA per nibble position),
 //        k-slots = the lane group's 8 tokens 4g..4g+3, 16+4g..16+4g+3.
 //        B = probabilities, column t = q head: exactly the q.k output registers.
+// Byte offsets of this lane inside a (head, page) slab and inside the page's
+// two scale rows; the same for every page, so the page's own part of an address
+// is uniform and the loads take a scalar base plus one of these.
+struct LaneOffsets {
+  uint32_t keys;    // token t, bytes 16g.. of the row's first half
+  uint32_t values;  // token 4g, bytes 8t..
+  uint32_t scale;   // lane i < 32: key scale i; lane 32 + i: value scale i (from the key scales)
+};
+__device__ __forceinline__ LaneOffsets lane_offsets(uint32_t t, uint32_t g, uint32_t scale_rows_apart) {
+  const uint32_t lane = 16 * g + t;
+  return {t * kRowBytes + 16 * g, 4 * g * kRowBytes + 8 * t,
+          (lane < kPage ? 0u : scale_rows_apart) + 4u * (lane & (kPage - 1))};
+}
+
 // PARTS: bit 0 the keys, bit 1 values and both scale lines.
 template <uint32_t PARTS>
 __device__ __forceinline__ void load_page(PageRegs &r, uint64_t entry, uint32_t head,
                                           uint32_t kv_heads, uint32_t layer_offset,
                                           uint64_t key_scales_off, uint64_t values_off,
-                                          uint64_t value_scales_off, uint32_t t, uint32_t g) {
-  const uint32_t index = uint32_t(entry) & KVX_PAGE_INDEX_MASK;
-  const uint8_t *region = reinterpret_cast<const uint8_t *>(entry - index) + layer_offset;
-  const uint64_t slab = (uint64_t(index) * kv_heads + head) * kHeadSlabBytes;
-  const uint8_t *keys = region + slab;
-  const uint8_t *values = region + values_off + slab;
-  const uint64_t scale_index = (uint64_t(index) * kv_heads + head) * kPage;
-  const float *key_scales = reinterpret_cast<const float *>(region + key_scales_off) + scale_index;
-  const float *value_scales =
-      reinterpret_cast<const float *>(region + value_scales_off) + scale_index;
+                                          const LaneOffsets &at) {
+  // The entry is the same in every lane; saying so keeps the address arithmetic
+  // on the scalar unit.
+  const uint32_t entry_lo = __builtin_amdgcn_readfirstlane(uint32_t(entry));
+  const uint32_t entry_hi = __builtin_amdgcn_readfirstlane(uint32_t(entry >> 32));
+  const uint32_t index = entry_lo & KVX_PAGE_INDEX_MASK;
+  const uint8_t *region =
+      reinterpret_cast<const uint8_t *>((uint64_t(entry_hi) << 32) | (entry_lo - index)) + layer_offset;
+  const uint64_t head_page = uint64_t(index) * kv_heads + head;
+  const uint8_t *keys = region + head_page * kHeadSlabBytes;
   if constexpr (PARTS & 1u) {
 #pragma unroll
     for (uint32_t tb = 0; tb < 2; ++tb)
 #pragma unroll
       for (uint32_t half = 0; half < 2; ++half)
         r.k[tb * 2 + half] =
-            load_streaming<u32x4>(keys + (16 * tb + t) * kRowBytes + 64 * half + 16 * g);
+            load_streaming<u32x4>(keys + at.keys + (16 * tb * kRowBytes + 64 * half));
   }
   if constexpr (PARTS & 2u) {
+    const uint8_t *values = keys + values_off;
 #pragma unroll
-    for (uint32_t s = 0; s < 8; ++s) {
-      const uint32_t token = (s < 4 ? 0 : 16) + 4 * g + (s & 3);
-      r.v[s] = load_streaming<u32x2>(values + token * kRowBytes + 8 * t);
-    }
+    for (uint32_t s = 0; s < 8; ++s)
+      r.v[s] = load_streaming<u32x2>(values + at.values + ((s < 4 ? 0 : 16) + (s & 3)) * kRowBytes);
     // One scale per lane instead of the sixteen a lane multiplies with: they
     // are fetched from the owning lanes when the page is attended, which keeps
     // a register set small enough for three of them.
-    const uint32_t lane = 16 * g + t;
-    r.scale = load_global<float>((lane < kPage ? key_scales : value_scales) + (lane & (kPage - 1)));
+    r.scale = load_global<float>(region + key_scales_off + head_page * (kPage * 4u) + at.scale);
   }
+}
+
+// x of this lane and x of the lane 16 (32) away, without the address register a
+// shuffle through the LDS crossbar needs: the swaps exchange the odd rows of 16
+// (the upper 32 lanes) of one operand with the even rows (lower lanes) of the
+// other, so the two results hold x[l] and x[l ^ 16] (x[l ^ 32]) in some order.
+struct LanePair {
+  float a, b;
+};
+__device__ __forceinline__ LanePair across16(float x) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return {__uint_as_float(r[0]), __uint_as_float(r[1])};
+}
+__device__ __forceinline__ LanePair across32(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return {__uint_as_float(r[0]), __uint_as_float(r[1])};
+}
+// Maximum / sum over the four lanes of a column (lanes l, l^16, l^32, l^48).
+__device__ __forceinline__ float column_max(float x) {
+  LanePair p = across16(x);
+  x = fmaxf(p.a, p.b);
+  p = across32(x);
+  return fmaxf(p.a, p.b);
+}
+__device__ __forceinline__ float column_sum(float x) {
+  LanePair p = across16(x);
+  x = p.a + p.b;
+  p = across32(x);
+  return p.a + p.b;
 }
 
 // Four bf16 pairs from one dword of eight nibbles: register p holds nibble p
@@ -196,8 +237,7 @@ __device__ __forceinline__ void attend_page(PageRegs &r, Queries queries,
       score[i] = live[i] ? v : -INFINITY;
       local_max = fmaxf(local_max, score[i]);
     }
-    local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
-    local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
+    local_max = column_max(local_max);
     const float next_max = fmaxf(st[nb].row_max, local_max);
     // A row that has seen nothing yet keeps -inf; its rescale is 1, not exp(nan).
     const float rescale = next_max == st[nb].row_max
@@ -279,10 +319,8 @@ __device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m,
     // Lanes of one column hold disjoint tokens: combine their sums and the
     // constant part, then take the constant part out of the accumulators.
     float row_sum = st[nb].row_sum, bias = st[nb].bias;
-    row_sum += __shfl_xor(row_sum, 16);
-    row_sum += __shfl_xor(row_sum, 32);
-    bias += __shfl_xor(bias, 16);
-    bias += __shfl_xor(bias, 32);
+    row_sum = column_sum(row_sum);
+    bias = column_sum(bias);
     if (written == 1) {
       // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
       // Rows of the tile past the live ones read as zeros (row_sum is 0 there).
@@ -401,6 +439,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   // kDepth register sets rotate: a set is refilled with the page kDepth ahead as
   // soon as its page has been consumed, so up to kDepth pages are in flight.
   PageRegs r[kDepth];
+  const LaneOffsets at = lane_offsets(t, g, uint32_t(ro.value_scales - ro.key_scales));
   auto fill = [&](PageRegs &set, uint32_t slot) {
 #ifdef KVX_PROBE_SAME_PAGE
     // Measurement build: every refill is the split's first page, so loads hit the
@@ -412,8 +451,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     // second copy of its registers, and interleaved with another fill's loads
     // they would make every wait cover both.
     asm volatile("");
-    load_page<3>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values,
-                 ro.value_scales, t, g);
+    load_page<3>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
   // The same in two steps for the steady loop: the keys as soon as the page that
@@ -423,8 +461,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     slot = 0;
 #endif
     asm volatile("");
-    load_page<1>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values,
-                 ro.value_scales, t, g);
+    load_page<1>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
   auto fill_rest = [&](PageRegs &set, uint32_t slot) {
@@ -432,8 +469,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     slot = 0;
 #endif
     asm volatile("");
-    load_page<2>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values,
-                 ro.value_scales, t, g);
+    load_page<2>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
   // The first fills are unconditional too (a split shorter than kDepth pages
@@ -469,8 +505,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
       }
       q_lds[nb][kb * 64 + lane] = q_reg;
     }
-    q_bias[nb] += __shfl_xor(q_bias[nb], 16);
-    q_bias[nb] += __shfl_xor(q_bias[nb], 32);
+    q_bias[nb] = column_sum(q_bias[nb]);
   }
 
   State st[NB];
