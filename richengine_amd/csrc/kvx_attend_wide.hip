@@ -79,20 +79,32 @@ __device__ __forceinline__ u32x4 int8_operand(uint32_t first, uint32_t second) {
                int8_pair(b, 0x04030402u)};
 }
 
-// What one lane holds of one page's keys / values.
-//  q.k : A = keys, row t = token 16*tb + t, k-slots = dims 32*kb + 8g .. + 7.
-//        B = queries, column t = fused query row, same dims.
-//        Output column t, rows 4g..4g+3 = tokens 16*tb + 4g + r.
+// What one lane holds of one page's keys / values.  Which token sits in which
+// MFMA row and which dims in which k-slots is free as long as both operands
+// agree; both are chosen so that every load instruction reads long contiguous
+// runs (a load that touches sixteen lines for 16 or 32 bytes each is bound by
+// the number of requests, not by bytes).
+//  q.k : A = keys, row t of token block tb = token 8*(t/4) + 4*tb + t%4; the
+//        k-slots of step kb are 8 dims at key_dims(kb, g).  B = queries, column
+//        t = fused query row, same dims.  Output column t, rows 4g..4g+3 =
+//        tokens 8g + 4*tb + r: a lane holds the scores of tokens 8g..8g+7.
 //  p.v : A = values (stored dimension-major), row t = dim 16*mb + t, k-slots =
-//        tokens 4g..4g+3 and 16+4g..16+4g+3: exactly the tokens whose scores the
-//        lane holds, so the probabilities are the B operand as they are.
+//        tokens 8g..8g+7, contiguous in the page: exactly the tokens whose scores
+//        the lane holds, so the probabilities are the B operand as they are.
+// First dim of the 8 dims lane group g multiplies in step kb: two-byte elements
+// take 16 bytes per step, one-byte elements take two steps out of one 16-byte load.
+template <uint32_t FMT>
+__device__ __forceinline__ uint32_t key_dims(uint32_t kb, uint32_t g) {
+  if constexpr (Wide<FMT>::kByte) return 64 * (kb >> 1) + 16 * g + 8 * (kb & 1);
+  else return 32 * kb + 8 * g;
+}
 template <uint32_t FMT>
 struct KeyRegs {
   uint32_t raw[2][8][Wide<FMT>::kDwords];  // [token block][dim block]
 };
 template <uint32_t FMT>
 struct ValueRegs {
-  uint32_t raw[16][Wide<FMT>::kDwords];  // [dim block]: tokens 4g.., then 16+4g..
+  uint32_t raw[16][Wide<FMT>::kDwords];  // [dim block]: tokens 8g .. 8g+7
 };
 
 struct PagePlace {
@@ -119,38 +131,44 @@ __device__ __forceinline__ void load_keys(KeyRegs<FMT> &k, const PagePlace &p, u
                                           uint32_t g) {
   constexpr uint32_t B = Wide<FMT>::kBytes;
 #pragma unroll
-  for (uint32_t tb = 0; tb < 2; ++tb)
+  for (uint32_t tb = 0; tb < 2; ++tb) {
+    const uint8_t *row = p.keys + (8 * (t >> 2) + 4 * tb + (t & 3)) * kD * B;
+    if constexpr (Wide<FMT>::kByte) {
 #pragma unroll
-    for (uint32_t kb = 0; kb < 8; ++kb) {
-      const uint8_t *at = p.keys + ((16 * tb + t) * kD + 32 * kb + 8 * g) * B;
-      if constexpr (Wide<FMT>::kByte) {
-        const u32x2 v = load_streaming<u32x2>(at);
-        k.raw[tb][kb][0] = v[0];
-        k.raw[tb][kb][1] = v[1];
-      } else {
-        const u32x4 v = load_streaming<u32x4>(at);
+      for (uint32_t j = 0; j < 4; ++j) {  // 16 tokens x 64 contiguous bytes per instruction
+        const u32x4 v = load_streaming<u32x4>(row + 64 * j + 16 * g);
+        k.raw[tb][2 * j][0] = v[0];
+        k.raw[tb][2 * j][1] = v[1];
+        k.raw[tb][2 * j + 1][0] = v[2];
+        k.raw[tb][2 * j + 1][1] = v[3];
+      }
+    } else {
+#pragma unroll
+      for (uint32_t kb = 0; kb < 8; ++kb) {
+        const u32x4 v = load_streaming<u32x4>(row + key_dims<FMT>(kb, g) * B);
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) k.raw[tb][kb][i] = v[i];
       }
     }
+  }
 }
 template <uint32_t FMT>
 __device__ __forceinline__ void load_values(ValueRegs<FMT> &v, const PagePlace &p, uint32_t t,
                                             uint32_t g) {
   constexpr uint32_t B = Wide<FMT>::kBytes;
 #pragma unroll
-  for (uint32_t mb = 0; mb < 16; ++mb)
+  for (uint32_t mb = 0; mb < 16; ++mb) {  // 16 dims x 32 tokens, contiguous, per instruction
+    const uint8_t *at = p.values + ((16 * mb + t) * kPage + 8 * g) * B;
+    if constexpr (Wide<FMT>::kByte) {
+      const u32x2 x = load_streaming<u32x2>(at);
+      v.raw[mb][0] = x[0];
+      v.raw[mb][1] = x[1];
+    } else {
+      const u32x4 x = load_streaming<u32x4>(at);
 #pragma unroll
-    for (uint32_t half = 0; half < 2; ++half) {
-      const uint8_t *at = p.values + ((16 * mb + t) * kPage + 16 * half + 4 * g) * B;
-      if constexpr (Wide<FMT>::kByte) {
-        v.raw[mb][half] = load_streaming<uint32_t>(at);
-      } else {
-        const u32x2 x = load_streaming<u32x2>(at);
-        v.raw[mb][2 * half] = x[0];
-        v.raw[mb][2 * half + 1] = x[1];
-      }
+      for (uint32_t i = 0; i < 4; ++i) v.raw[mb][i] = x[i];
     }
+  }
 }
 template <uint32_t FMT>
 __device__ __forceinline__ u32x4 key_operand(const KeyRegs<FMT> &k, uint32_t tb, uint32_t kb) {
@@ -166,7 +184,7 @@ __device__ __forceinline__ u32x4 value_operand(const ValueRegs<FMT> &v, uint32_t
 }
 
 template <uint32_t FMT, uint32_t NB>
-__global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restrict__ queries,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void attend_wide_kernel(const uint16_t *__restrict__ queries,
                                                          uint16_t *__restrict__ output,
                                                          float *__restrict__ partials,
                                                          float *__restrict__ statistics,
@@ -211,8 +229,8 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
     sight[nb].mask = sight[nb].tree ? l.masks[query_row] : 0u;
   }
 
-  // Queries: [row][g][D] bf16, fused row m; register kb of a column holds dims
-  // 32*kb + 8g .. + 7.  fp8 and int8 pages stage them as fp16.  Columns without a
+  // Queries: [row][g][D] bf16, fused row m; register kb of a column holds the 8
+  // dims from key_dims(kb, g).  fp8 and int8 pages stage them as fp16.  Columns without a
   // live row carry zeros.
   const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
   __shared__ u32x4 q_lds[NB][8][64];
@@ -222,7 +240,7 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
     const uint16_t *q_row = q_head + uint64_t(live_row[nb] ? m[nb] : 0) * kD;
 #pragma unroll
     for (uint32_t kb = 0; kb < 8; ++kb) {
-      u32x4 q = load_global<u32x4>(q_row + 32 * kb + 8 * g);
+      u32x4 q = load_global<u32x4>(q_row + key_dims<FMT>(kb, g));
       if constexpr (kByte) {
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) {
@@ -241,31 +259,47 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
     table_lds[i] = load_global<uint64_t>(l.table + begin + i);
   __syncthreads();
 
-  KeyRegs<FMT> keys;
-  ValueRegs<FMT> values;
-  f32x4 ks[2], vs[2];  // fp8, int8: scales of the lane's score tokens, per token block
-  auto fetch_keys = [&](uint32_t slot) {
+  // kSets register sets rotate: a set's keys are refilled with the page kSets
+  // ahead as soon as the page has multiplied its last key, its values when the
+  // page is done, so more than one page is always in flight.
+  // Two sets wherever the register file of a SIMD lane holds them next to the
+  // accumulators: not for two row blocks over two-byte elements.
+  constexpr uint32_t kSets = (!kByte && NB > 1) ? 1 : 2;
+  struct PageSet {
+    KeyRegs<FMT> keys;
+    ValueRegs<FMT> values;
+    f32x4 ks[2], vs[2];  // fp8, int8: scales of the lane's score tokens, per token block
+  };
+  PageSet set[kSets];
+  // The empty asm statements keep the loads of one fetch together and in place.
+  auto fetch_keys = [&](PageSet &r, uint32_t slot) {
     const PagePlace p = place_page<FMT>(table_lds[slot], head, H, a.kv.offset, ro);
-    asm volatile("");  // the loads of one fetch stay together and in place
-    load_keys<FMT>(keys, p, t, g);
+    asm volatile("");
+    load_keys<FMT>(r.keys, p, t, g);
     if constexpr (kByte) {
-      ks[0] = load_global<f32x4>(p.key_scales + 4 * g);
-      ks[1] = load_global<f32x4>(p.key_scales + 16 + 4 * g);
+      r.ks[0] = load_global<f32x4>(p.key_scales + 8 * g);
+      r.ks[1] = load_global<f32x4>(p.key_scales + 8 * g + 4);
     }
     asm volatile("");
   };
-  auto fetch_values = [&](uint32_t slot) {
+  auto fetch_values = [&](PageSet &r, uint32_t slot) {
     const PagePlace p = place_page<FMT>(table_lds[slot], head, H, a.kv.offset, ro);
     asm volatile("");
-    load_values<FMT>(values, p, t, g);
+    load_values<FMT>(r.values, p, t, g);
     if constexpr (kByte) {
-      vs[0] = load_global<f32x4>(p.value_scales + 4 * g);
-      vs[1] = load_global<f32x4>(p.value_scales + 16 + 4 * g);
+      r.vs[0] = load_global<f32x4>(p.value_scales + 8 * g);
+      r.vs[1] = load_global<f32x4>(p.value_scales + 8 * g + 4);
     }
     asm volatile("");
   };
-  fetch_keys(0);
-  fetch_values(0);
+  // The first fills are unconditional (a split shorter than kSets pages loads its
+  // last page again), so the steady loop is entered with the loads in flight that
+  // its own iterations leave behind.
+#pragma unroll
+  for (uint32_t d = 0; d < kSets; ++d) {
+    fetch_keys(set[d], min(d, end - begin - 1));
+    fetch_values(set[d], min(d, end - begin - 1));
+  }
 
   f32x4 acc[NB][16];  // [block][dim block]: dims 16*mb + 4g + r of column t
   float row_max[NB], row_sum[NB];
@@ -279,99 +313,120 @@ __global__ __launch_bounds__(64) void attend_wide_kernel(const uint16_t *__restr
   // fp8 operands are worth 2^-8 of their values; see the head of this file.
   constexpr float kUnscale = kFp8 ? 256.0f : 1.0f;
 
-  for (uint32_t page = begin; page < end; ++page) {
-    // Refills are unconditional (the last page is fetched once more) so the loop
-    // body is straight-line code and each wait counts exactly the loads issued
-    // after the ones it needs.
-    const uint32_t next = min(page + 1, end - 1) - begin;
-    // ---- q.k ----
-    f32x4 s[NB][2];
+  // One page out of set r; keys_consumed() runs when its keys have been read for
+  // the last time.
+  auto attend_page = [&](PageSet &r, uint32_t page, auto keys_consumed) {
+      // ---- q.k ----
+      f32x4 s[NB][2];
 #pragma unroll
-    for (uint32_t nb = 0; nb < NB; ++nb) s[nb][0] = s[nb][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      for (uint32_t nb = 0; nb < NB; ++nb) s[nb][0] = s[nb][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (uint32_t kb = 0; kb < 8; ++kb)
+      for (uint32_t kb = 0; kb < 8; ++kb)
 #pragma unroll
-      for (uint32_t tb = 0; tb < 2; ++tb) {
-        const u32x4 k = key_operand<FMT>(keys, tb, kb);
+        for (uint32_t tb = 0; tb < 2; ++tb) {
+          const u32x4 k = key_operand<FMT>(r.keys, tb, kb);
 #pragma unroll
-        for (uint32_t nb = 0; nb < NB; ++nb) s[nb][tb] = mfma<FMT>(k, q_lds[nb][kb][lane], s[nb][tb]);
+          for (uint32_t nb = 0; nb < NB; ++nb) s[nb][tb] = mfma<FMT>(k, q_lds[nb][kb][lane], s[nb][tb]);
+        }
+      f32x4 page_ks[2];
+      if constexpr (kByte) {
+        page_ks[0] = r.ks[0];
+        page_ks[1] = r.ks[1];
       }
-    f32x4 page_ks[2];
-    if constexpr (kByte) {
-      page_ks[0] = ks[0];
-      page_ks[1] = ks[1];
-    }
-    fetch_keys(next);
-    // ---- page softmax, per column block ----
-    const uint32_t first_token = page * kPage;
-    u32x4 pb[NB];
-    f32x4 page_vs[2];
-    if constexpr (kByte) {
-      page_vs[0] = vs[0];
-      page_vs[1] = vs[1];
-    }
-#pragma unroll
-    for (uint32_t nb = 0; nb < NB; ++nb) {
-      float score[8], local_max = -INFINITY;
-      bool live[8];
-#pragma unroll
-      for (uint32_t i = 0; i < 8; ++i) {
-        const uint32_t tb = i >> 2, rr = i & 3;
-        float v = s[nb][tb][rr] * kUnscale;
-        if constexpr (kByte) v *= page_ks[tb][rr];
-        v *= score_scale;
-        live[i] = sight[nb].sees(first_token + 16 * tb + 4 * g + rr);
-        score[i] = live[i] ? v : -INFINITY;
-        local_max = fmaxf(local_max, score[i]);
+      keys_consumed();
+      // ---- page softmax, per column block ----
+      const uint32_t first_token = page * kPage;
+      u32x4 pb[NB];
+      f32x4 page_vs[2];
+      if constexpr (kByte) {
+        page_vs[0] = r.vs[0];
+        page_vs[1] = r.vs[1];
       }
-      local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
-      local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
-      const float next_max = fmaxf(row_max[nb], local_max);
-      // A row that has seen nothing yet keeps -inf; its rescale is 1, not exp(nan).
-      const float rescale = next_max == row_max[nb]
-                                ? 1.0f
-                                : __builtin_amdgcn_exp2f((row_max[nb] - next_max) * kLog2e);
-      float weight[8], page_sum = 0.0f;
 #pragma unroll
-      for (uint32_t i = 0; i < 8; ++i) {
-        // The difference first, so the page's maximum gets exactly 1.
-        float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
-        p = live[i] ? p : 0.0f;
-        page_sum += p;
-        weight[i] = kByte ? p * page_vs[i >> 2][i & 3] : p;
-      }
-      row_sum[nb] = fmaf(row_sum[nb], rescale, page_sum);
-      row_max[nb] = next_max;
+      for (uint32_t nb = 0; nb < NB; ++nb) {
+        float score[8], local_max = -INFINITY;
+        bool live[8];
 #pragma unroll
-      for (uint32_t p = 0; p < 4; ++p) {
-        if constexpr (kFp8) {
-          const f16x2 pair = {_Float16(weight[2 * p]), _Float16(weight[2 * p + 1])};
-          pb[nb][p] = __builtin_bit_cast(uint32_t, pair);
-        } else if constexpr (kInt8) {
-          // Rounded to bf16 as the reference tile does, then carried as fp16.
-          const f32x2 wide = {weight[2 * p], weight[2 * p + 1]};
-          const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(wide, bf16x2));
-          const f16x2 pair = {_Float16(__uint_as_float(bits << 16)),
-                              _Float16(__uint_as_float(bits & 0xffff0000u))};
-          pb[nb][p] = __builtin_bit_cast(uint32_t, pair);
-        } else {
-          const f32x2 pair = {weight[2 * p], weight[2 * p + 1]};
-          pb[nb][p] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+        for (uint32_t i = 0; i < 8; ++i) {
+          const uint32_t tb = i >> 2, rr = i & 3;
+          float v = s[nb][tb][rr] * kUnscale;
+          if constexpr (kByte) v *= page_ks[tb][rr];
+          v *= score_scale;
+          live[i] = sight[nb].sees(first_token + 8 * g + 4 * tb + rr);
+          score[i] = live[i] ? v : -INFINITY;
+          local_max = fmaxf(local_max, score[i]);
+        }
+        local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
+        local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
+        const float next_max = fmaxf(row_max[nb], local_max);
+        // A row that has seen nothing yet keeps -inf; its rescale is 1, not exp(nan).
+        const float rescale = next_max == row_max[nb]
+                                  ? 1.0f
+                                  : __builtin_amdgcn_exp2f((row_max[nb] - next_max) * kLog2e);
+        float weight[8], page_sum = 0.0f;
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i) {
+          // The difference first, so the page's maximum gets exactly 1.
+          float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
+          p = live[i] ? p : 0.0f;
+          page_sum += p;
+          weight[i] = kByte ? p * page_vs[i >> 2][i & 3] : p;
+        }
+        row_sum[nb] = fmaf(row_sum[nb], rescale, page_sum);
+        row_max[nb] = next_max;
+#pragma unroll
+        for (uint32_t p = 0; p < 4; ++p) {
+          if constexpr (kFp8) {
+            const f16x2 pair = {_Float16(weight[2 * p]), _Float16(weight[2 * p + 1])};
+            pb[nb][p] = __builtin_bit_cast(uint32_t, pair);
+          } else if constexpr (kInt8) {
+            // Rounded to bf16 as the reference tile does, then carried as fp16.
+            const f32x2 wide = {weight[2 * p], weight[2 * p + 1]};
+            const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(wide, bf16x2));
+            const f16x2 pair = {_Float16(__uint_as_float(bits << 16)),
+                                _Float16(__uint_as_float(bits & 0xffff0000u))};
+            pb[nb][p] = __builtin_bit_cast(uint32_t, pair);
+          } else {
+            const f32x2 pair = {weight[2 * p], weight[2 * p + 1]};
+            pb[nb][p] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+          }
+        }
+        if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
+#pragma unroll
+          for (uint32_t mb = 0; mb < 16; ++mb) acc[nb][mb] *= rescale;
         }
       }
-      if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
+      // ---- p.v ----
 #pragma unroll
-        for (uint32_t mb = 0; mb < 16; ++mb) acc[nb][mb] *= rescale;
+      for (uint32_t mb = 0; mb < 16; ++mb) {
+        const u32x4 v = value_operand<FMT>(r.values, mb);
+#pragma unroll
+        for (uint32_t nb = 0; nb < NB; ++nb) acc[nb][mb] = mfma<FMT>(v, pb[nb], acc[nb][mb]);
+      }
+  };
+
+  // Steady state: every refill is unconditional, so the loop body is straight-line
+  // code and each wait counts exactly the loads issued after the ones it needs.
+  uint32_t page = begin;
+  for (; page + 2 * kSets <= end; page += kSets) {
+#pragma unroll
+    for (uint32_t d = 0; d < kSets; ++d) {
+      const uint32_t refill = page + d + kSets - begin;
+      attend_page(set[d], page + d, [&] { fetch_keys(set[d], refill); });
+      fetch_values(set[d], refill);
+    }
+  }
+  // Tail: at most 2 kSets - 1 pages are left, the first kSets of them loaded.
+#pragma unroll
+  for (uint32_t k = 0; k < 2 * kSets - 1; ++k) {
+    const uint32_t d = k % kSets;
+    if (page + k < end) {
+      attend_page(set[d], page + k, [] {});
+      if (k + kSets < 2 * kSets - 1 && page + k + kSets < end) {
+        fetch_keys(set[d], page + k + kSets - begin);
+        fetch_values(set[d], page + k + kSets - begin);
       }
     }
-    // ---- p.v ----
-#pragma unroll
-    for (uint32_t mb = 0; mb < 16; ++mb) {
-      const u32x4 v = value_operand<FMT>(values, mb);
-#pragma unroll
-      for (uint32_t nb = 0; nb < NB; ++nb) acc[nb][mb] = mfma<FMT>(v, pb[nb], acc[nb][mb]);
-    }
-    fetch_values(next);
   }
 
 #pragma unroll
