@@ -50,6 +50,9 @@ def parse():
                          "kv_page_copy: a plain copy of known size to scale HBM counters by")
     ap.add_argument("--pages-per-split", type=int, default=0,
                     help="override the library's decode split rule (experiments)")
+    ap.add_argument("--workload", choices=["decode", "tree-verify"], default="decode",
+                    help="decode = BASELINE configs[2], the headline metric (default); "
+                         "tree-verify = configs[4], the matrix-core verify path (profiling)")
     return ap.parse_args()
 
 
@@ -136,12 +139,143 @@ def profiled_traffic():
     return None
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def tree_verify(args):
+    """BASELINE configs[4]: int4, batch 4, contexts 65536, a 16-node draft tree per
+    sequence (branching <= 3).  A step = per layer, append the 16 draft rows and
+    run masked verify attention over history + rows; then compact a seeded
+    root-to-leaf path of every sequence, all layers in one call.  The dominant
+    kernel (verify_int4_kernel) runs on the matrix cores; its line carries the
+    MFMA roofline (flops = 4 x D x fused query rows x visible tokens per layer)."""
+    import numpy as np
+    import torch
+    from richengine_amd import kvx
+
+    L = kvx.lib()
+    torch.cuda.set_device(0)
+    rng = np.random.default_rng(args.seed)
+    lanes, context, nodes = 4, 65536, 16
+    n_pages = (context + nodes + 31) // 32
+    layout = kvx.Layout(LAYERS, H, D, kvx.INT4, 0.0)
+    extent_pages = L.kvx_layout_largest_extent_pages(C.byref(layout))
+    extents = -(-lanes * n_pages // extent_pages)
+    storage = kvx.Storage(LAYERS, H, D, kvx.INT4, extents * extent_pages, extent_pages, aligned=True)
+    storage.allocate_all()
+    ids = rng.permutation(extents * extent_pages)[:lanes * n_pages].astype(np.uint32)
+    tables = [storage.table(ids[i * n_pages:(i + 1) * n_pages]) for i in range(lanes)]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(args.seed)
+    for lane in range(lanes):
+        for done in range(0, context, 2048):
+            k = torch.randn((H, 2048, D), generator=gen, device="cuda").bfloat16()
+            v = torch.randn((H, D, 2048), generator=gen, device="cuda").bfloat16()
+            for layer in range(LAYERS):
+                kvx.append(storage, layer, k, v, [tables[lane]],
+                           [kvx.ChunkParams(done, 2048, 2048, n_pages)], H * 2048 * D)
+    none = 0xFFFFFFFF
+    masks = np.zeros((lanes, nodes), dtype=np.uint32)
+    paths = np.zeros((lanes, 16), dtype=np.uint32)
+    counts = np.zeros(lanes, dtype=np.uint32)
+    for lane in range(lanes):
+        parents, children = [none], {}
+        for row in range(1, nodes):
+            parent = int(rng.choice([c for c in range(row) if children.get(c, 0) < 3][-4:]))
+            children[parent] = children.get(parent, 0) + 1
+            parents.append(parent)
+        masks[lane] = kvx.tree_masks(parents)
+        leaf = int(rng.choice([c for c in range(nodes) if c not in children]))
+        walk = []
+        while leaf != none:
+            walk.append(leaf)
+            leaf = parents[leaf]
+        walk.reverse()
+        assert kvx.tree_path_valid(parents, walk)
+        paths[lane, :len(walk)], counts[lane] = walk, len(walk)
+    masks_d = torch.from_numpy(masks.view(np.int32)).cuda()
+    paths_d = torch.from_numpy(paths.view(np.int32)).cuda()
+    counts_d = torch.from_numpy(counts.view(np.int32)).cuda()
+    chunk_k = torch.randn((lanes, H, 32, D), generator=gen, device="cuda").bfloat16()
+    chunk_v = torch.randn((lanes, H, D, 32), generator=gen, device="cuda").bfloat16()
+    queries = torch.randn((lanes, H, 32, G, D), generator=gen, device="cuda").bfloat16()
+    output = torch.zeros_like(queries)
+    splits = L.kvx_verify_splits(context, nodes)
+    cp = [kvx.ChunkParams(context, nodes, 32, n_pages) for _ in range(lanes)]
+    vp = [kvx.VerifyParams(context, n_pages, kvx.KvLayer(), splits, splits, nodes, 16, 0.0)
+          for _ in range(lanes)]
+    workspace = torch.empty(kvx.attend_workspace_bytes(storage, vp, QH) + 4096, dtype=torch.uint8,
+                            device="cuda")
+    torch.cuda.synchronize()
+
+    def step():
+        for layer in range(LAYERS):
+            kvx.append(storage, layer, chunk_k, chunk_v, tables, cp, H * 32 * D, verify_max_rows=16)
+            kvx.attend_verify(storage, layer, QH, queries, output, tables, vp, masks_d, 32, workspace)
+        kvx.compact_path(storage, 0xFFFFFFFF, tables, cp, paths_d, counts_d, 16)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    def time_attend(phases):
+        L.kvx_debug_set_attend_phases(phases)
+        kvx.attend_verify(storage, 0, QH, queries, output, tables, vp, masks_d, 32, workspace)
+        torch.cuda.synchronize()
+        k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        k0.record()
+        for it in range(args.kernel_iters):
+            kvx.attend_verify(storage, it % LAYERS, QH, queries, output, tables, vp, masks_d, 32, workspace)
+        k1.record()
+        torch.cuda.synchronize()
+        L.kvx_debug_set_attend_phases(3)
+        return k0.elapsed_time(k1) / args.kernel_iters
+
+    kernel_ms = time_attend(1)
+    visible = lanes * (context + nodes)
+    flops = 4 * D * (nodes * QH) * visible  # q.k and p.v, multiply and add, every row over every token
+    kv_bytes = visible * BYTES_PER_TOKEN_LAYER
+    achieved = flops / (kernel_ms * 1e-3) / 1e12
+    result = {
+        "metric": "int4 tree verify (16-node trees, batch 4 x 65536 tokens): verified draft tokens/s",
+        "value": round(lanes * nodes * args.steps / wall, 1), "unit": "draft tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int4 pages, bf16 MFMA, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[4]: speculative tree verify on int4 KV, batch 4, "
+                               "contexts 65536, 16-node trees (branching <= 3), 16 layers: append 16 "
+                               "rows + masked verify per layer, then path compaction over all layers",
+                   "batch": lanes, "layers": LAYERS, "splits_per_sequence": int(splits),
+                   "seed": args.seed},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": None,
+                     "kernel": "verify_int4_kernel (split kernel of verify attention), one layer per launch",
+                     "flops_per_launch": flops, "ms_per_launch": round(kernel_ms, 4),
+                     "kv_gbs": round(kv_bytes / (kernel_ms * 1e-3) / 1e9, 1)},
+        "cpu_baseline": None,
+    }
+    storage.close()
+    print(json.dumps(result))
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the KV path of this build has no multi-GPU leg "
               "(run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "tree-verify":
+        from richengine_amd import kvx
+        if not os.path.exists(kvx.LIB_PATH):
+            from richengine_amd import build as kvx_build
+            kvx_build.build(verbose=False)
+        return tree_verify(args)
     import numpy as np
     import torch
     from richengine_amd import kvx
