@@ -6,7 +6,9 @@ Workload (BASELINE.json configs[2], the one the metric is quoted on): int4 KV,
 uniformly from [512, 32768]; pages come from a device-sized pool in a
 seed-shuffled order, reached through per-sequence page tables.  One step is one
 decode step of the whole batch: per layer, append one token per sequence
-(quantize + scatter) and run paged decode attention (split partials + merge).
+(quantize + scatter) and run paged decode attention (split partials + merge),
+through kv_append_attend_decode (or the two separate entries with
+--separate-append).
 
 Prints ONE JSON line: whole-step KV GB/s (algorithmic KV bytes read by attention
 / step time), decode tokens/s, the roofline of the dominant kernel measured
@@ -50,6 +52,8 @@ def parse():
                          "kv_page_copy: a plain copy of known size to scale HBM counters by")
     ap.add_argument("--pages-per-split", type=int, default=0,
                     help="override the library's decode split rule (experiments)")
+    ap.add_argument("--separate-append", action="store_true",
+                    help="call kv_append and kv_attend_decode instead of kv_append_attend_decode")
     ap.add_argument("--workload", choices=["decode", "tree-verify"], default="decode",
                     help="decode = BASELINE configs[2], the headline metric (default); "
                          "tree-verify = configs[4], the matrix-core verify path (profiling)")
@@ -359,6 +363,15 @@ def main():
         ap_arr = (kvx.ChunkParams * BATCH)(*ap)
         vp_arr = (kvx.VerifyParams * BATCH)(*vp)
         for layer in range(LAYERS):
+            if not args.separate_append:
+                # one call per layer: the token is stored by the attention kernel itself
+                rc = L.kv_append_attend_decode(storage.h, layer, chunk_k.data_ptr(), chunk_v.data_ptr(),
+                                               lane_stride, 32, QH, queries.data_ptr(),
+                                               output.data_ptr(), table_arr, vp_arr, BATCH, 1,
+                                               workspace.data_ptr(), ws_bytes, stream)
+                if rc:
+                    kvx.check(rc)
+                continue
             rc = L.kv_append(storage.h, layer, chunk_k.data_ptr(), chunk_v.data_ptr(), table_arr,
                              ap_arr, BATCH, lane_stride, 15, stream)
             if rc:

@@ -399,6 +399,21 @@ int kv_attend_decode(const kvx_storage *storage, uint32_t layer, uint32_t query_
                      const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
                      void *workspace, uint64_t workspace_bytes, void *stream);
 
+/* One decode step of a layer in one call: kv_append of one token per lane at
+   lanes[i].committed_tokens (chunk rows as for kv_append: keys [head][chunk_stride][D],
+   values [head][D][chunk_stride], token 0 of each lane's chunk, lanes chunk_lane_stride
+   elements apart) followed by kv_attend_decode over committed_tokens + 1 tokens.  The
+   reference stores and attends in one call the same way (ops::PagedAttention::addVerify,
+   runtime/ops/PagedAttention.cpp:467-544).  Same page bytes and same output as the two
+   calls; for int4 pages of head dimension 256 the wave that owns a sequence's last page
+   stores the token itself, which saves the append launch. */
+int kv_append_attend_decode(const kvx_storage *storage, uint32_t layer, const void *chunk_keys,
+                            const void *chunk_values, uint64_t chunk_lane_stride,
+                            uint32_t chunk_stride, uint32_t query_heads, const void *queries,
+                            void *output, const uint64_t *const *page_tables,
+                            const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                            void *workspace, uint64_t workspace_bytes, void *stream);
+
 /* Chunked prefill attention of one sequence: rows in tiles of 8, each tile
    causal over committed + its rows.  Replaces ops::PagedAttention::addPrefill
    (PagedAttention.cpp:442-465; kernels prefill/paged_attention.metal:7-206).

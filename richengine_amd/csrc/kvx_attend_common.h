@@ -54,6 +54,20 @@ struct DecodeArgs {
   uint32_t row_stride;
   uint32_t fused_rows;  // row capacity x group: fused query rows per (lane, KV head)
   kvx_kv_layer kv;
+  // One-row decode with the step's token appended by the kernel itself: the
+  // bf16 chunk rows of the launch's first lane ([head][stride][D] keys,
+  // [head][D][stride] values, token 0 of each lane's chunk); null = the rows are
+  // in the pages already.
+  const uint16_t *chunk_keys;
+  const uint16_t *chunk_values;
+  uint64_t chunk_lane_stride;
+  uint32_t chunk_stride;
+};
+// What a fused append brings to a launch (host side).
+struct FusedAppend {
+  const void *keys, *values;
+  uint64_t lane_stride;
+  uint32_t stride;
 };
 
 // Which tokens one fused query row (an MFMA column) may see
@@ -231,7 +245,8 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
                             const uint64_t *const *page_tables, const kvx_verify_params *lanes,
                             uint32_t n_lanes, const uint32_t *row_masks, uint32_t row_stride,
                             uint64_t lane_stride, void *workspace, uint64_t workspace_bytes,
-                            uint32_t phases, hipStream_t stream) {
+                            uint32_t phases, hipStream_t stream,
+                            const FusedAppend *fused = nullptr) {
   const kvx_layout &l = s->layout;
   const uint32_t H = l.kv_heads, G = query_heads / H;
   const uint32_t capacity = lanes[0].row_capacity, M = capacity * G;
@@ -250,6 +265,12 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
     a.row_stride = row_stride;
     a.fused_rows = M;
     a.kv = kv;
+    if (fused) {
+      a.chunk_keys = static_cast<const uint16_t *>(fused->keys) + uint64_t(first) * fused->lane_stride;
+      a.chunk_values = static_cast<const uint16_t *>(fused->values) + uint64_t(first) * fused->lane_stride;
+      a.chunk_lane_stride = fused->lane_stride;
+      a.chunk_stride = fused->stride;
+    }
     uint32_t items = 0, max_splits = 0;
     for (uint32_t i = 0; i < a.n_lanes; ++i) {
       const kvx_verify_params &p = lanes[first + i];

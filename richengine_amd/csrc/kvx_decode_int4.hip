@@ -297,6 +297,56 @@ __device__ __forceinline__ void attend_page(PageRegs &r, Queries queries,
   }
 }
 
+// One-token append done by the wave that owns the sequence's last page, for its
+// own KV head: quantizes the token's key row and value row (bf16 -> int4 codes and
+// one fp32 scale each, the arithmetic of append_kernel: reference
+// common/paged_store_row.h:47-147) and stores them at slot committed % 32 of the
+// page.  Each lane owns four consecutive dims.  The stores are complete before
+// the caller loads the page: the wave waits for them, and no cache of this CU can
+// hold the lines yet because only this wave reads this head of this page.
+__device__ __forceinline__ void append_decode_token(const DecodeArgs &a, const DecodeLane &l,
+                                                    uint32_t li, uint32_t head, uint32_t lane) {
+  const uint32_t H = a.kv_heads;
+  const uint32_t slot = l.committed % kPage;
+  const uint64_t entry = l.table[l.committed / kPage];
+  const Slab slab = slab_of(KVX_FMT_INT4, H, kD, a.kv, head, entry);
+  const uint16_t *key_row =
+      a.chunk_keys + li * a.chunk_lane_stride + uint64_t(head) * a.chunk_stride * kD + 4 * lane;
+  const uint16_t *value_column =
+      a.chunk_values + li * a.chunk_lane_stride + (uint64_t(head) * kD + 4 * lane) * a.chunk_stride;
+  const u32x2 key_bits = load_global<u32x2>(key_row);
+  float row[2][4];
+  row[0][0] = __uint_as_float(key_bits[0] << 16);
+  row[0][1] = __uint_as_float(key_bits[0] & 0xffff0000u);
+  row[0][2] = __uint_as_float(key_bits[1] << 16);
+  row[0][3] = __uint_as_float(key_bits[1] & 0xffff0000u);
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i)
+    row[1][i] = bf16_to_f32(load_global<uint16_t>(value_column + uint64_t(i) * a.chunk_stride));
+#pragma unroll
+  for (uint32_t tensor = 0; tensor < 2; ++tensor) {
+    float maximum = fmaxf(fmaxf(fabsf(row[tensor][0]), fabsf(row[tensor][1])),
+                          fmaxf(fabsf(row[tensor][2]), fabsf(row[tensor][3])));
+    for (int offset = 32; offset; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset));
+    uint32_t packed = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+      const float scaled =
+          maximum == 0.0f ? 0.0f : __fdiv_rn(__fmul_rn(row[tensor][i], 7.0f), maximum);
+      int code = int(rintf(scaled));
+      code = code < -7 ? -7 : code > 7 ? 7 : code;
+      if (maximum == 0.0f) code = 0;
+      packed |= (uint32_t(code) & 0xfu) << (4 * i);
+    }
+    uint8_t *data = tensor ? slab.values : slab.keys;
+    *reinterpret_cast<uint16_t *>(data + slot * kRowBytes + 2 * lane) = uint16_t(packed);
+    if (lane == 0)
+      (tensor ? slab.value_scales : slab.key_scales)[slot] =
+          maximum == 0.0f ? 0.0f : __fdiv_rn(maximum, 7.0f);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 #ifndef KVX_DECODE_DEPTH
 #define KVX_DECODE_DEPTH 2
 #endif
@@ -392,6 +442,12 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
 
   const uint32_t lane = threadIdx.x, t = lane & 15, g = lane >> 4;
   const uint32_t H = a.kv_heads, G = a.group, M = a.fused_rows;
+  // The wave that owns the sequence's last page stores the step's token: before
+  // anything else when that page is among the first fills, otherwise behind them,
+  // where its latency hides under the loads already in flight.
+  const bool appends = a.chunk_keys != nullptr && end == pages;
+  const bool appends_first = appends && end - begin <= kDepth;
+  if (appends_first) append_decode_token(a, l, li, head, lane);
   // This wave's MFMA columns are fused rows 16 NB z .. of the tile, 16 per block;
   // a fused row is (query row, head in group) = (m / G, m % G).
   uint32_t m[NB];
@@ -477,6 +533,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   // loads in flight, in the same order, as its own iterations leave behind.
 #pragma unroll
   for (uint32_t d = 0; d < kDepth; ++d) fill(r[d], min(d, end - begin - 1));
+  if (appends && !appends_first) append_decode_token(a, l, li, head, lane);
 
   // Register kb of the staged queries holds the 8 dims of dword
   // w = 16*(kb>>2) + 4g + (kb&3) of a key row in expansion order; odd dims are
@@ -598,10 +655,16 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                            const kvx_verify_params *lanes, uint32_t n_lanes,
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
-                           hipStream_t stream) {
+                           hipStream_t stream, const void *append_keys, const void *append_values,
+                           uint64_t append_lane_stride, uint32_t append_stride) {
   if (s->layout.format != KVX_FMT_INT4 || !matrix_attention_covers(s, query_heads, lanes, n_lanes))
     return 1;
+  const FusedAppend appended{append_keys, append_values, append_lane_stride, append_stride};
+  const FusedAppend *fused = append_keys ? &appended : nullptr;
   const uint32_t fused_rows = lanes[0].row_capacity * (query_heads / s->layout.kv_heads);
+  // The kernel appends the step's token itself only where one wave owns a
+  // (sequence, KV head, split): one-row decode.
+  if (fused && (fused_rows > 16 || lanes[0].row_capacity != 1)) return 1;
   // Sharing the expanded operands between two blocks pays where the lanes are few
   // and long (verify: 13% on 4 x 65536 tokens x 16 tree rows); chunked prefill has
   // hundreds of tiles of 48 fused rows, where a half-empty second wave and one
@@ -614,7 +677,7 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   return launch_matrix_attention(decode_int4_kernel, "decode_int4_kernel", 16, 64, s, kv,
                                  query_heads, queries, output, page_tables, lanes, n_lanes,
                                  row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                 kvx_attend_phases(), stream);
+                                 kvx_attend_phases(), stream, fused);
 }
 
 #ifdef KVX_PROBE_CLOCK

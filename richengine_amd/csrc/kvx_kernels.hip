@@ -560,13 +560,18 @@ int check_launch(const char *what) {
 using namespace kvx;
 
 // Implemented by the int4 MFMA kernels: enqueues the whole attention and
-// returns 0, or declines (returns 1) shapes it does not cover.
+// returns 0, or declines (returns 1) shapes it does not cover.  With
+// append_keys / append_values (bf16 chunk rows, one token per lane at
+// committed_tokens) the kernel also stores that token before it attends;
+// declined unless the lanes are one-row decode lanes.
 int kvx_attend_int4_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t query_heads,
                            const void *queries, void *output, const uint64_t *const *page_tables,
                            const kvx_verify_params *lanes, uint32_t n_lanes,
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
-                           hipStream_t stream);
+                           hipStream_t stream, const void *append_keys = nullptr,
+                           const void *append_values = nullptr, uint64_t append_lane_stride = 0,
+                           uint32_t append_stride = 0);
 
 int kvx_attend_wide_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t query_heads,
                            const void *queries, void *output, const uint64_t *const *page_tables,
@@ -801,6 +806,51 @@ int kv_attend_decode(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
   if (fast <= 0) return fast;
   return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, nullptr,
                         row_stride, workspace, static_cast<hipStream_t>(stream), 3);
+}
+
+int kv_append_attend_decode(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
+                            const void *chunk_values, uint64_t chunk_lane_stride,
+                            uint32_t chunk_stride, uint32_t query_heads, const void *queries,
+                            void *output, const uint64_t *const *page_tables,
+                            const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                            void *workspace, uint64_t workspace_bytes, void *stream) {
+  if (!s || !chunk_keys || !chunk_values || !queries || !output || !page_tables || !lanes ||
+      !n_lanes || !workspace)
+    return fail(KVX_EINVAL, "kv_append_attend_decode: null argument or no lanes");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
+  if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
+  kvx_kv_layer kv;
+  if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    if (lanes[i].active_rows != 1 || lanes[i].row_capacity != 1)
+      return fail(KVX_EINVAL, "decode attends exactly one row per lane");
+    if (!page_tables[i]) return fail(KVX_EINVAL, "kv_append_attend_decode: null page table");
+    const kvx_chunk_params chunk{lanes[i].committed_tokens, 1, chunk_stride,
+                                 lanes[i].page_table_entries, {}};
+    static const char *const names[] = {"", "chunk_tokens_out_of_range", "context_out_of_range",
+                                        "chunk_stride_invalid", "page_table_too_short"};
+    if (const int e = kvx_chunk_validation(&chunk)) return fail(KVX_EINVAL, names[e]);
+  }
+  if (int rc = validate_attend(s, query_heads, lanes, n_lanes, row_stride, page_tables,
+                               workspace_bytes))
+    return rc;
+  const uint32_t group = query_heads / s->layout.kv_heads;
+  const uint64_t lane_stride = uint64_t(s->layout.kv_heads) * row_stride * group * s->layout.head_dim;
+  // int4 pages: the wave that owns a sequence's last page stores the token itself.
+  const int fused = kvx_attend_int4_launch(s, kv, query_heads, queries, output, page_tables, lanes,
+                                           n_lanes, nullptr, row_stride, lane_stride, workspace,
+                                           workspace_bytes, 0, static_cast<hipStream_t>(stream),
+                                           chunk_keys, chunk_values, chunk_lane_stride, chunk_stride);
+  if (fused <= 0) return took(fused);
+  // Every other shape: the two entries one after the other.
+  std::vector<kvx_chunk_params> chunks(n_lanes);
+  for (uint32_t i = 0; i < n_lanes; ++i)
+    chunks[i] = {lanes[i].committed_tokens, 1, chunk_stride, lanes[i].page_table_entries, {}};
+  if (int rc = kv_append(s, layer, chunk_keys, chunk_values, page_tables, chunks.data(), n_lanes,
+                         chunk_lane_stride, 0, stream))
+    return rc;
+  return kv_attend_decode(s, layer, query_heads, queries, output, page_tables, lanes, n_lanes,
+                          row_stride, workspace, workspace_bytes, stream);
 }
 
 int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads,

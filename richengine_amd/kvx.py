@@ -35,7 +35,7 @@ SYMBOLS = [
     "kvx_pool_acquire", "kvx_pool_retain", "kvx_pool_release", "kvx_pool_page_active",
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
     "kvx_pool_snapshot_get", "kv_append", "kv_attend_verify", "kv_attend_decode",
-    "kv_attend_prefill", "kv_compact_path", "kvx_debug_set_attend_phases",
+    "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kvx_debug_set_attend_phases",
     "kvx_debug_attend_paths", "kvx_decode_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
     "kvx_prefix_chain", "kvx_prefix_retain_active", "kvx_prefix_release_active",
@@ -202,6 +202,8 @@ def _declare(L):
     L.kv_append.argtypes = [vp, u32, vp, vp, vp, vp, u32, u64, u32, vp]
     L.kv_attend_verify.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, vp, u32, vp, u64, vp]
     L.kv_attend_decode.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, u32, vp, u64, vp]
+    L.kv_append_attend_decode.argtypes = [vp, u32, vp, vp, u64, u32, u32, vp, vp, vp, vp, u32, u32, vp,
+                                          u64, vp]
     L.kv_attend_prefill.argtypes = [vp, u32, u32, vp, vp, vp, C.POINTER(PrefillParams), vp, u64, vp]
     L.kv_compact_path.argtypes = [vp, u32, vp, vp, u32, vp, vp, u32, vp]
     L.kvx_debug_set_attend_phases.argtypes, L.kvx_debug_set_attend_phases.restype = [u32], None
@@ -346,6 +348,16 @@ def attend_decode(storage, layer, query_heads, queries, output, tables, lanes, r
                                         _ptr(workspace),
                                         workspace.numel() * workspace.element_size(),
                                         _stream(stream)))
+
+
+def append_attend_decode(storage, layer, chunk_keys, chunk_values, chunk_lane_stride, chunk_stride,
+                         query_heads, queries, output, tables, lanes, row_stride, workspace,
+                         stream=None):
+    arr = (VerifyParams * len(lanes))(*lanes)
+    return check(lib().kv_append_attend_decode(
+        storage.h, layer, _ptr(chunk_keys), _ptr(chunk_values), chunk_lane_stride, chunk_stride,
+        query_heads, _ptr(queries), _ptr(output), _table_array(tables), arr, len(lanes), row_stride,
+        _ptr(workspace), workspace.numel() * workspace.element_size(), _stream(stream)))
 
 
 def prefill_workspace_bytes(storage, rows, query_heads):

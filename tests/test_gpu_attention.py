@@ -392,3 +392,54 @@ def test_generic_kernels_cover_other_shapes(fmt, heads, group, dim):
         Gp.check_attention(Gp.host_u16(out), want[:, :, :row_stride], want32[:, :, :row_stride], live,
                            tol(fmt), f"generic rows={active} fmt={fmt}")
     tw.close()
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+def test_append_attend_decode_is_the_two_calls(fmt):
+    """kv_append_attend_decode leaves the page bytes of kv_append (the oracle's,
+    bit for bit) and returns the output of kv_attend_decode; int4 pages take the
+    kernel that stores the token itself."""
+    committed = [0, 31, 32, 700, 4095, 1000, 63, 2047, 5000]
+    lanes = len(committed)
+    tw, counts, hts, dts = shared_pool_lanes(fmt, committed, 1, seed=61)
+    rng = np.random.default_rng(62)
+    k = rng.standard_normal((lanes, H, 1, D)).astype(np.float32)
+    v = rng.standard_normal((lanes, H, 1, D)).astype(np.float32)
+    k[:, :, :, [3, 77]] *= 20
+    k[2, 1] = 0  # a zero row: scale 0, codes 0
+    v[5, 3] *= 1e-20
+    ck = np.zeros((lanes, H, 32, D), dtype=np.uint16)
+    cv = np.zeros((lanes, H, D, 32), dtype=np.uint16)
+    for lane in range(lanes):
+        ck[lane], cv[lane] = T.chunk_buffers(k[lane], v[lane], 32)
+    q = queries((lanes, H, 1, G, D), 63)
+    splits = [max(kvx.lib().kvx_decode_splits(c, 1), 1 + (c > 600)) for c in committed]
+    dp = [kvx.VerifyParams(committed[i], counts[i], kvx.KvLayer(), splits[i], splits[i], 1, 1, 0.0)
+          for i in range(lanes)]
+    ws = torch.empty(kvx.attend_workspace_bytes(tw.dev, dp, QH), dtype=torch.uint8, device="cuda")
+    before = [tw.dev.extent_read(e).copy() for e in range(tw.extents)]
+    # the two calls
+    kvx.append(tw.dev, 1, Gp.dev(ck), Gp.dev(cv), dts,
+               [kvx.ChunkParams(committed[i], 1, 32, counts[i]) for i in range(lanes)], H * 32 * D)
+    out_two = torch.zeros((lanes, H, 1, G, D), dtype=torch.int16, device="cuda")
+    kvx.attend_decode(tw.dev, 1, QH, Gp.dev(q), out_two, dts, dp, 1, ws)
+    torch.cuda.synchronize()
+    for lane in range(lanes):
+        p = ko.ChunkParams(committed[lane], 1, 32, counts[lane], tw.host.layer(1))
+        assert ko.store_chunk(fmt, H, D, ck[lane], cv[lane], hts[lane], p) == 1
+    tw.assert_same_bytes()
+    # back to the state before the step, then the one call
+    for e in range(tw.extents):
+        tw.dev.extent_write(e, before[e])
+    out_one = torch.zeros_like(out_two)
+    ws.fill_(0xA5)
+    kvx.append_attend_decode(tw.dev, 1, Gp.dev(ck), Gp.dev(cv), H * 32 * D, 32, QH, Gp.dev(q), out_one,
+                             dts, dp, 1, ws)
+    torch.cuda.synchronize()
+    tw.assert_same_bytes()
+    assert torch.equal(out_one, out_two)
+    # and its parameter checks
+    with pytest.raises(kvx.KvxError):
+        kvx.append_attend_decode(tw.dev, 1, Gp.dev(ck), Gp.dev(cv), H * 32 * D, 31, QH, Gp.dev(q),
+                                 out_one, dts, dp, 1, ws)
+    tw.close()
