@@ -54,6 +54,8 @@ def parse():
                     help="override the library's decode split rule (experiments)")
     ap.add_argument("--separate-append", action="store_true",
                     help="call kv_append and kv_attend_decode instead of kv_append_attend_decode")
+    ap.add_argument("--verify-splits", type=int, default=0,
+                    help="tree-verify: splits per sequence instead of the library's plan (experiments)")
     ap.add_argument("--workload", choices=["decode", "tree-verify"], default="decode",
                     help="decode = BASELINE configs[2], the headline metric (default); "
                          "tree-verify = configs[4], the matrix-core verify path (profiling)")
@@ -204,7 +206,7 @@ def tree_verify(args):
     chunk_v = torch.randn((lanes, H, D, 32), generator=gen, device="cuda").bfloat16()
     queries = torch.randn((lanes, H, 32, G, D), generator=gen, device="cuda").bfloat16()
     output = torch.zeros_like(queries)
-    splits = L.kvx_verify_splits(context, nodes)
+    splits = args.verify_splits or kvx.verify_plan([context] * lanes, nodes, H, QH)[0]
     cp = [kvx.ChunkParams(context, nodes, 32, n_pages) for _ in range(lanes)]
     vp = [kvx.VerifyParams(context, n_pages, kvx.KvLayer(), splits, splits, nodes, 16, 0.0)
           for _ in range(lanes)]

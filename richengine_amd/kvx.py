@@ -36,7 +36,7 @@ SYMBOLS = [
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
     "kvx_pool_snapshot_get", "kv_append", "kv_attend_verify", "kv_attend_decode",
     "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kvx_debug_set_attend_phases",
-    "kvx_debug_attend_paths", "kvx_decode_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
+    "kvx_debug_attend_paths", "kvx_decode_plan", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
     "kvx_prefix_chain", "kvx_prefix_retain_active", "kvx_prefix_release_active",
     "kvx_prefix_touch", "kvx_prefix_eviction_candidate", "kvx_prefix_erase",
@@ -168,6 +168,7 @@ def _declare(L):
     L.kvx_sequences_compact_extent.argtypes = [vp, PU32, vp, PU32, vp]
     L.kvx_debug_attend_paths.argtypes, L.kvx_debug_attend_paths.restype = [PU64, PU64], None
     L.kvx_decode_plan.argtypes = [vp, u32, u32, vp]
+    L.kvx_verify_plan.argtypes = [vp, u32, u32, u32, u32, vp]
     L.kvx_tree_masks.argtypes = [vp, u32, vp]
     L.kvx_tree_path_valid.argtypes = [vp, u32, vp, u32]
     L.kvx_storage_destroy.argtypes = [vp]
@@ -572,6 +573,13 @@ def decode_plan(committed, kv_heads):
     """Split counts of a decode batch (kvx_decode_plan)."""
     out = (C.c_uint32 * len(committed))()
     check(lib().kvx_decode_plan(_u32(committed), len(committed), kv_heads, out))
+    return list(out)
+
+
+def verify_plan(committed, rows, kv_heads, query_heads):
+    """Split counts of a verify batch sized for the GPU (kvx_verify_plan)."""
+    out = (C.c_uint32 * len(committed))()
+    check(lib().kvx_verify_plan(_u32(committed), len(committed), rows, kv_heads, query_heads, out))
     return list(out)
 
 

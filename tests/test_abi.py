@@ -102,3 +102,35 @@ def test_planning_rules_agree_with_the_oracle():
     assert L.kvx_prefill_workspace(2049, 24, C.byref(layout_a), C.byref(pa), C.byref(pa)) == kvx.EINVAL
     assert L.kvx_prefill_workspace(8, 25, C.byref(layout_a), C.byref(pa), C.byref(pa)) == kvx.EINVAL
     assert L.kvx_last_error()
+
+
+def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
+    """kvx_decode_plan / kvx_verify_plan (no counterpart in the reference): every lane gets
+    between 1 and the maximum number of splits, the partition covers its pages, and the launch
+    has no more waves than the rule allows unless every split is already at its shortest."""
+    import numpy as np
+    rng = np.random.default_rng(3)
+    H, QH = 4, 24
+    pages = lambda tokens: (tokens + 31) // 32
+    for trial in range(40):
+        lanes = int(rng.integers(1, 40))
+        committed = [int(x) for x in rng.integers(0, 70000, lanes)]
+        plan = kvx.decode_plan(committed, H)
+        heads_pages = sum(pages(c + 1) for c in committed) * H
+        per = min(max(-(-heads_pages // 1024), 8), 32)
+        assert plan == [min(max(1, -(-pages(c + 1) // per)), 512) for c in committed]
+        for rows in (2, 8, 16):
+            plan = kvx.verify_plan(committed, rows, H, QH)
+            blocks = -(-rows * (QH // H) // 32) if rows * (QH // H) > 16 else 1
+            counts = [pages(c + rows) for c in committed]
+            per = max(-(-sum(counts) * H * blocks // 1024), 8)
+            while True:  # the rule, restated: the first length that fits one round of waves
+                want = [min(max(1, -(-n // per)), 128) for n in counts]
+                if sum(want) * H * blocks <= 1024 or all(s == 1 for s in want):
+                    break
+                per += 1
+            assert plan == want
+            assert all(1 <= s <= 128 and s <= max(n, 1) for s, n in zip(plan, counts))
+    assert kvx.verify_plan([65536] * 4, 16, H, QH) == [21] * 4
+    with pytest.raises(kvx.KvxError):
+        kvx.verify_plan([10], 8, 4, 6)
