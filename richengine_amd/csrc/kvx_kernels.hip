@@ -883,22 +883,43 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
     return fail(KVX_EINVAL, "prefill attention scratch is smaller than its bound");
   auto st = static_cast<hipStream_t>(stream);
   {
-    // The int4 MFMA kernels take the tiles as lanes: tile t attends rows 8t..8t+7
+    // The matrix-core kernels take the tiles as lanes: tile t attends rows 8t..8t+7
     // over committed + 8t tokens, its queries 8 rows further on in the chunk.
-    std::vector<kvx_verify_params> tile_lanes(tiles);
-    std::vector<const uint64_t *> tile_tables(tiles, page_table);
-    for (uint32_t t = 0; t < tiles; ++t)
-      tile_lanes[t] = {params->committed_tokens + KVX_PREFILL_TILE_ROWS * t,
+    // With a single split every tile walks its pages from the first, so two
+    // neighbouring tiles can share one walk as a lane of 16 rows: a row's softmax
+    // runs over the same pages in the same order (the page the second tile may
+    // add is invisible to the first tile's rows and changes nothing), and every
+    // key and value is fetched and expanded once for 16 rows instead of 8.
+    const uint32_t T = KVX_PREFILL_TILE_ROWS;
+    const uint32_t width = (params->split_count == 1 && tiles >= 2) ? 2 : 1;
+    const uint32_t wide_lanes = tiles / width, rest = tiles - wide_lanes * width;
+    std::vector<kvx_verify_params> tile_lanes(wide_lanes + rest);
+    std::vector<const uint64_t *> tile_tables(wide_lanes + rest, page_table);
+    for (uint32_t t = 0; t < wide_lanes + rest; ++t) {
+      const uint32_t first_row = t < wide_lanes ? T * width * t : T * (wide_lanes * width + (t - wide_lanes));
+      const uint32_t capacity = t < wide_lanes ? T * width : T;
+      tile_lanes[t] = {params->committed_tokens + first_row,
                        params->page_table_entries,
                        {},
                        params->split_count,
                        params->split_count,
-                       std::min(KVX_PREFILL_TILE_ROWS, params->rows - KVX_PREFILL_TILE_ROWS * t),
-                       KVX_PREFILL_TILE_ROWS,
+                       std::min(capacity, params->rows - first_row),
+                       capacity,
                        params->score_scale};
-    const int fast = took(attend_matrix(
-        s, kv, query_heads, queries, output, tile_tables.data(), tile_lanes.data(), tiles, nullptr,
-        params->chunk_stride, uint64_t(KVX_PREFILL_TILE_ROWS) * G * D, workspace, workspace_bytes, 1, st));
+    }
+    int fast = took(attend_matrix(s, kv, query_heads, queries, output, tile_tables.data(),
+                                  tile_lanes.data(), wide_lanes, nullptr, params->chunk_stride,
+                                  uint64_t(T) * width * G * D, workspace, workspace_bytes,
+                                  width == 1, st));
+    if (fast == 0 && rest) {
+      // The odd last tile on its own; lanes of one launch share a row capacity.
+      const uint64_t skip = uint64_t(T) * width * wide_lanes * G * D;
+      fast = attend_matrix(s, kv, query_heads, static_cast<const uint16_t *>(queries) + skip,
+                           static_cast<uint16_t *>(output) + skip, tile_tables.data(),
+                           tile_lanes.data() + wide_lanes, rest, nullptr, params->chunk_stride,
+                           uint64_t(T) * G * D, workspace, workspace_bytes, 1, st);
+      if (fast > 0) return fail(KVX_ESTATE, "the last prefill tile was declined after the others ran");
+    }
     if (fast <= 0) return fast;
   }
   float *partials = static_cast<float *>(workspace);
