@@ -339,10 +339,13 @@ public:
     return plan;
   }
   // decode = true selects the batched-decode split rule of this library
-  // (rows = 1 per lane, one split per 32 visible pages).
+  // (rows = 1 per lane, one split per 32 visible pages).  sizedForGpu = true
+  // takes the split counts from kvx_decode_plan / kvx_verify_plan, which look at
+  // the whole batch and give the launch one round of waves, instead of the
+  // reference's per-lane rules.
   static VerifyAttentionPlan verifyPlan(uint32_t lanes, uint32_t queryHeads, kv::Layout layout,
                                         const std::vector<uint32_t> &historyTokens, bool tree = false,
-                                        bool decode = false) {
+                                        bool decode = false, bool sizedForGpu = false) {
     requireShape(queryHeads, layout);
     if (!lanes || historyTokens.size() != lanes)
       throw std::invalid_argument("paged verify attention needs one history per lane");
@@ -350,10 +353,18 @@ public:
       throw std::invalid_argument("fp8 KV has no tree verify");
     const uint32_t rows = decode ? 1 : tree ? kv::kTreeVerifyNodes : kv::kVerifyRows;
     VerifyAttentionPlan plan{layout.format, lanes, {}, 0, {}, rows, queryHeads, layout.scoreScale};
-    for (uint32_t history : historyTokens) {
-      const uint32_t splits = decode ? kvx_decode_splits(history, 1) : kvx_verify_splits(history, rows);
-      plan.laneSplits.push_back(splits);
-      plan.splits = std::max(plan.splits, splits);
+    if (sizedForGpu) {
+      plan.laneSplits.resize(lanes);
+      check(decode ? kvx_decode_plan(historyTokens.data(), lanes, layout.kvHeads, plan.laneSplits.data())
+                   : kvx_verify_plan(historyTokens.data(), lanes, rows, layout.kvHeads, queryHeads,
+                                     plan.laneSplits.data()));
+      for (uint32_t splits : plan.laneSplits) plan.splits = std::max(plan.splits, splits);
+    } else {
+      for (uint32_t history : historyTokens) {
+        const uint32_t splits = decode ? kvx_decode_splits(history, 1) : kvx_verify_splits(history, rows);
+        plan.laneSplits.push_back(splits);
+        plan.splits = std::max(plan.splits, splits);
+      }
     }
     const uint32_t group = queryHeads / layout.kvHeads;
     uint64_t fusedRows = 0;
@@ -418,6 +429,20 @@ public:
     if (chunks.size() != plan.lanes) throw std::invalid_argument("one chunk per plan lane");
     const kv::Layout &layout = storage.layout();
     const uint64_t laneStride = uint64_t{layout.kvHeads} * kv::kVerifyChunkStride * layout.headDimension;
+    if (plan.rowCapacity == 1) {  // a decode step: one call stores the token and attends
+      std::vector<kv::VerifyAttentionParams> lanes(plan.lanes);
+      for (uint32_t i = 0; i < plan.lanes; ++i) {
+        if (chunks[i].chunk_tokens != 1 || chunks[i].chunk_stride != kv::kVerifyChunkStride)
+          throw std::invalid_argument("a decode lane stores one token in a 32-token chunk");
+        lanes[i] = {chunks[i].committed_tokens, chunks[i].page_table_entries, {}, plan.laneSplits[i],
+                    plan.splits, 1, 1, plan.scoreScale};
+      }
+      check(kv_append_attend_decode(storage.handle(), layer, buffers.chunkKeys, buffers.chunkValues,
+                                    laneStride, kv::kVerifyChunkStride, plan.queryHeads, buffers.queries,
+                                    buffers.output, buffers.pageTables, lanes.data(), plan.lanes, 1,
+                                    buffers.workspace, buffers.workspaceBytes, stream));
+      return;
+    }
     check(kv_append(storage.handle(), layer, buffers.chunkKeys, buffers.chunkValues, buffers.pageTables,
                     chunks.data(), plan.lanes, laneStride, kv::kTreeVerifyNodes, stream));
     attend(stream, storage, layer, buffers, chunks, plan);

@@ -292,6 +292,44 @@ void testAppendDecodeSingleToken() {
     EXPECT(wrong == 0);
     hip(hipFree(workspace));
   }
+  // A second token: addVerify with a decode plan stores it and attends in one
+  // call (layer 0); the store and the attention as two calls on layer 1, which
+  // holds the same first token, must give the same bits.
+  {
+    for (uint32_t h = 0; h < H; ++h)
+      for (uint32_t d = 0; d < D; ++d) {
+        keys[(h * 32 + 0) * D + d] = bf16(std::cos(0.21f * d - h));
+        values[(h * D + d) * 32 + 0] = bf16(std::sin(0.05f * d + 0.3f * h));
+      }
+    hip(hipMemcpy(keysDevice, keys.data(), keys.size() * 2, hipMemcpyHostToDevice));
+    hip(hipMemcpy(valuesDevice, values.data(), values.size() * 2, hipMemcpyHostToDevice));
+    const auto chunk = ops::PagedAttention::verifyParams(1, 2, 1);
+    const auto plan = ops::PagedAttention::verifyPlan(1, QH, layout, {1}, false, true, /*sizedForGpu=*/true);
+    EXPECT(plan.laneSplits.size() == 1 && plan.laneSplits[0] == 1);
+    void *workspace = nullptr;
+    hip(hipMalloc(&workspace, plan.workspace.bytes() + 256));
+    ops::PagedVerifyBuffers buffers;
+    buffers.chunkKeys = keysDevice;
+    buffers.chunkValues = valuesDevice;
+    buffers.queries = queriesDevice;
+    buffers.output = outputDevice;
+    buffers.workspace = workspace;
+    buffers.workspaceBytes = plan.workspace.bytes() + 256;
+    buffers.pageTables = tables;
+    std::vector<uint16_t> one(queries.size()), two(queries.size());
+    ops::PagedAttention::addVerify(nullptr, storage, 0, buffers, {chunk}, plan);
+    hip(hipDeviceSynchronize());
+    hip(hipMemcpy(one.data(), outputDevice, one.size() * 2, hipMemcpyDeviceToHost));
+    ops::PagedAttention::addPrefillStore(nullptr, storage, 1, keysDevice, valuesDevice, tableDevice, chunk);
+    ops::PagedAttention::attend(nullptr, storage, 1, buffers, {chunk}, plan);
+    hip(hipDeviceSynchronize());
+    hip(hipMemcpy(two.data(), outputDevice, two.size() * 2, hipMemcpyDeviceToHost));
+    EXPECT(one == two);
+    bool moved = false;  // and the second token did change the result
+    for (size_t i = 0; i < one.size(); ++i) moved = moved || f32(one[i]) != 0.5f * (i / (G * D) + 1) * (float(i % D % 15) - 7.0f);
+    EXPECT(moved);
+    hip(hipFree(workspace));
+  }
   // an invalid chunk is refused before anything is enqueued
   kv::ChunkedPrefillParams bad{0, 1, 32, 0, {}};
   EXPECT(throws<std::invalid_argument>(
