@@ -56,9 +56,12 @@ def parse():
                     help="call kv_append and kv_attend_decode instead of kv_append_attend_decode")
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
-    ap.add_argument("--workload", choices=["decode", "tree-verify"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "tree-verify", "prefill"], default="decode",
                     help="decode = BASELINE configs[2], the headline metric (default); "
-                         "tree-verify = configs[4], the matrix-core verify path (profiling)")
+                         "tree-verify = configs[4] and prefill = configs[3], the matrix-core paths "
+                         "(profiling)")
+    ap.add_argument("--format", choices=["bf16", "fp8", "int8", "int4"], default="bf16",
+                    help="page format of the prefill workload")
     return ap.parse_args()
 
 
@@ -270,18 +273,122 @@ def tree_verify(args):
     print(json.dumps(result))
 
 
+def chunked_prefill(args):
+    """BASELINE configs[3]: batch 4, a 2048-token chunk per sequence appended onto a
+    shared 16384-token prefix (the prefix pages are the same physical pages in every
+    sequence's table), bf16 or fp8 pages.  A step = per layer and sequence, quantize +
+    scatter of the chunk, then causal attention of its 2048 rows over prefix + chunk.
+    The attention kernel's line carries the MFMA roofline (useful flops = 4 x D x
+    query heads x sum over rows of the tokens the row sees)."""
+    import numpy as np
+    import torch
+    from richengine_amd import kvx
+
+    L = kvx.lib()
+    torch.cuda.set_device(0)
+    rng = np.random.default_rng(args.seed)
+    fmt = {"bf16": kvx.BF16, "fp8": kvx.FP8, "int8": kvx.INT8, "int4": kvx.INT4}[args.format]
+    peak = 2500.0  # bf16 and fp16 MFMA (the one-byte formats multiply as fp16)
+    sequences, prefix, chunk = 4, 16384, 2048
+    prefix_pages, chunk_pages = prefix // 32, chunk // 32
+    total = prefix_pages + sequences * chunk_pages
+    layout = kvx.Layout(LAYERS, H, D, fmt, 0.0)
+    extent_pages = L.kvx_layout_largest_extent_pages(C.byref(layout))
+    extents = -(-total // extent_pages)
+    storage = kvx.Storage(LAYERS, H, D, fmt, extents * extent_pages, extent_pages, aligned=True)
+    storage.allocate_all()
+    ids = rng.permutation(extents * extent_pages)[:total].astype(np.uint32)
+    shared = ids[:prefix_pages]
+    tables = [storage.table(np.concatenate([shared, ids[prefix_pages + s * chunk_pages:
+                                                        prefix_pages + (s + 1) * chunk_pages]]))
+              for s in range(sequences)]
+    entries = prefix_pages + chunk_pages
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(args.seed)
+
+    def rows(shape):  # N(0,1); fp8 pages take values clipped to the e4m3 range of the scaled codes
+        return torch.randn(shape, generator=gen, device="cuda").clamp_(-6, 6).bfloat16()
+
+    for done in range(0, prefix, 2048):
+        k, v = rows((H, 2048, D)), rows((H, D, 2048))
+        for layer in range(LAYERS):
+            kvx.append(storage, layer, k, v, [tables[0]], [kvx.ChunkParams(done, 2048, 2048, entries)],
+                       H * 2048 * D)
+    chunk_k = [rows((H, chunk, D)) for _ in range(sequences)]
+    chunk_v = [rows((H, D, chunk)) for _ in range(sequences)]
+    queries = [rows((H, chunk, G, D)) for _ in range(sequences)]
+    output = torch.zeros_like(queries[0])
+    splits = L.kvx_prefill_splits(chunk)
+    cp = kvx.ChunkParams(prefix, chunk, chunk, entries)
+    pp = kvx.PrefillParams(prefix, chunk, chunk, entries, kvx.KvLayer(), splits, 0.0)
+    workspace = torch.empty(kvx.prefill_workspace_bytes(storage, chunk, QH) + 4096, dtype=torch.uint8,
+                            device="cuda")
+    torch.cuda.synchronize()
+
+    def step():
+        for layer in range(LAYERS):
+            for s in range(sequences):
+                kvx.append(storage, layer, chunk_k[s], chunk_v[s], [tables[s]], [cp], H * chunk * D)
+                kvx.attend_prefill(storage, layer, QH, queries[s], output, tables[s], pp, workspace)
+
+    steps, warmup = min(args.steps, 5), min(args.warmup, 1)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    iters = max(2, args.kernel_iters // 4)
+    k0.record()
+    for it in range(iters):
+        kvx.attend_prefill(storage, it % LAYERS, QH, queries[it % sequences], output,
+                           tables[it % sequences], pp, workspace)
+    k1.record()
+    torch.cuda.synchronize()
+    kernel_ms = k0.elapsed_time(k1) / iters
+    flops = 4 * D * QH * sum(prefix + r + 1 for r in range(chunk))
+    achieved = flops / (kernel_ms * 1e-3) / 1e12
+    result = {
+        "metric": f"{args.format} chunked prefill (2048-token chunks onto a shared 16384-token prefix, "
+                  "batch 4): prefill tokens/s",
+        "value": round(sequences * chunk * steps / wall, 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": round(wall * 1e3 / steps, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {"bf16": "bf16 pages, bf16 MFMA", "fp8": "fp8e4m3 pages, fp16 MFMA",
+                  "int8": "int8 pages, fp16 MFMA", "int4": "int4 pages, bf16 MFMA"}[args.format] +
+                 ", fp32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs[3]: chunked prefill with a shared prefix, batch 4, "
+                               "2048-row chunks over 16384 + 2048 tokens, 16 layers: quantize + scatter "
+                               "of the chunk, then causal attention per layer and sequence",
+                   "batch": sequences, "layers": LAYERS, "format": args.format, "splits": int(splits),
+                   "seed": args.seed},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "kernel": "split kernel of kv_attend_prefill (verify_int4_kernel or "
+                               "attend_wide_kernel), one sequence and layer per launch",
+                     "flops_per_launch": flops, "ms_per_launch": round(kernel_ms, 4)},
+        "cpu_baseline": None,
+    }
+    storage.close()
+    print(json.dumps(result))
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the KV path of this build has no multi-GPU leg "
               "(run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
-    if args.workload == "tree-verify":
+    if args.workload != "decode":
         from richengine_amd import kvx
         if not os.path.exists(kvx.LIB_PATH):
             from richengine_amd import build as kvx_build
             kvx_build.build(verbose=False)
-        return tree_verify(args)
+        return tree_verify(args) if args.workload == "tree-verify" else chunked_prefill(args)
     import numpy as np
     import torch
     from richengine_amd import kvx

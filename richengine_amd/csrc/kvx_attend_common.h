@@ -62,7 +62,40 @@ struct DecodeArgs {
   const uint16_t *chunk_values;
   uint64_t chunk_lane_stride;
   uint32_t chunk_stride;
+  // Regular lanes (the tiles of a chunked prefill): tile_lanes > 0 means lane[0]
+  // describes the first of that many lanes over one page table, each tile_rows
+  // query rows and committed tokens after the one before, its queries
+  // tile_lane_stride elements further on; the last holds tile_last_rows rows.
+  // Any number of them fits one launch.
+  uint32_t tile_lanes;
+  uint32_t tile_rows;
+  uint32_t tile_last_rows;
+  uint64_t tile_lane_stride;
 };
+
+// The lane with this index of a launch: read from the arguments, or derived
+// from the first for regular lanes.
+__device__ __forceinline__ DecodeLane lane_at(const DecodeArgs &a, uint32_t index) {
+  if (!a.tile_lanes) return a.lane[index];
+  DecodeLane l = a.lane[0];
+  l.committed += index * a.tile_rows;
+  if (index + 1 == a.tile_lanes) l.active_rows = a.tile_last_rows;
+  l.first_item = index * l.split_count;
+  l.row_base += uint64_t(index) * l.split_count * a.kv_heads * a.fused_rows;
+  l.q_offset += index * a.tile_lane_stride;
+  return l;
+}
+// The lane that owns work item `item` (a lane's items are its splits), and its index.
+__device__ __forceinline__ DecodeLane lane_of_item(const DecodeArgs &a, uint32_t item, uint32_t &index) {
+  index = 0;
+  if (a.tile_lanes) {
+    index = item / a.lane[0].split_count;
+  } else {
+    for (uint32_t i = 1; i < a.n_lanes; ++i)
+      if (item >= a.lane[i].first_item) index = i;
+  }
+  return lane_at(a, index);
+}
 // What a fused append brings to a launch (host side).
 struct FusedAppend {
   const void *keys, *values;
@@ -160,7 +193,7 @@ __global__ __launch_bounds__(64 * kMergeWaves) void matrix_merge_kernel(
     const float *__restrict__ statistics, DecodeArgs a) {
   const uint32_t j = blockIdx.x, head = blockIdx.y;
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-  const DecodeLane &l = a.lane[blockIdx.z];
+  const DecodeLane l = lane_at(a, blockIdx.z);
   const uint32_t pages = (l.committed + l.active_rows + kPage - 1) / kPage;
   const uint32_t per = (pages + l.split_count - 1) / l.split_count;
   const uint32_t written = (pages + per - 1) / per;
@@ -246,7 +279,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
                             uint32_t n_lanes, const uint32_t *row_masks, uint32_t row_stride,
                             uint64_t lane_stride, void *workspace, uint64_t workspace_bytes,
                             uint32_t phases, hipStream_t stream,
-                            const FusedAppend *fused = nullptr) {
+                            const FusedAppend *fused = nullptr, uint32_t tile_rows = 0) {
   const kvx_layout &l = s->layout;
   const uint32_t H = l.kv_heads, G = query_heads / H;
   const uint32_t capacity = lanes[0].row_capacity, M = capacity * G;
@@ -257,9 +290,19 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
   float *partials = static_cast<float *>(workspace);
   float *statistics = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + statistics_offset);
   uint64_t row_base = 0;
-  for (uint32_t first = 0; first < n_lanes; first += kLanes) {
+  // Regular lanes (tile_rows > 0: lane i is lane 0 moved on by i x tile_rows rows
+  // and tokens, all full but perhaps the last) go out in one launch whatever
+  // their number; others 32 to a launch.
+  const uint32_t lanes_per_launch = tile_rows ? n_lanes : kLanes;
+  for (uint32_t first = 0; first < n_lanes; first += lanes_per_launch) {
     DecodeArgs a{};
-    a.n_lanes = std::min(kLanes, n_lanes - first);
+    a.n_lanes = std::min(lanes_per_launch, n_lanes - first);
+    if (tile_rows) {
+      a.tile_lanes = n_lanes;
+      a.tile_rows = tile_rows;
+      a.tile_last_rows = lanes[n_lanes - 1].active_rows;
+      a.tile_lane_stride = lane_stride;
+    }
     a.kv_heads = H;
     a.group = G;
     a.row_stride = row_stride;
@@ -272,7 +315,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       a.chunk_stride = fused->stride;
     }
     uint32_t items = 0, max_splits = 0;
-    for (uint32_t i = 0; i < a.n_lanes; ++i) {
+    for (uint32_t i = 0; i < (tile_rows ? 1u : a.n_lanes); ++i) {
       const kvx_verify_params &p = lanes[first + i];
       DecodeLane &dl = a.lane[i];
       dl.table = page_tables[first + i];
@@ -288,6 +331,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       max_splits = std::max(max_splits, p.split_count);
       row_base += uint64_t(p.split_count) * H * M;
     }
+    if (tile_rows) items = n_lanes * lanes[0].split_count;
     if (phases & 1u) {
       hipLaunchKernelGGL(split_kernel, dim3(items, H, (M + columns - 1) / columns), dim3(threads), 0,
                          stream, static_cast<const uint16_t *>(queries),

@@ -191,10 +191,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
                                                          DecodeArgs a) {
   constexpr bool kFp8 = Wide<FMT>::kFp8, kInt8 = Wide<FMT>::kInt8, kByte = Wide<FMT>::kByte;
   const uint32_t item = blockIdx.x, head = blockIdx.y;
-  uint32_t li = 0;
-  for (uint32_t i = 1; i < a.n_lanes; ++i)
-    if (item >= a.lane[i].first_item) li = i;
-  const DecodeLane &l = a.lane[li];
+  uint32_t li;
+  const DecodeLane l = lane_of_item(a, item, li);
   const uint32_t split = item - l.first_item;
   if (split >= l.split_count) return;
   const uint32_t visible = l.committed + l.active_rows;
@@ -486,7 +484,7 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                            const kvx_verify_params *lanes, uint32_t n_lanes,
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
-                           hipStream_t stream) {
+                           hipStream_t stream, uint32_t tile_rows) {
   const uint32_t format = s->layout.format;
   if ((format != KVX_FMT_BF16 && format != KVX_FMT_FP8E4M3 && format != KVX_FMT_INT8) ||
       !matrix_attention_covers(s, query_heads, lanes, n_lanes))
@@ -496,7 +494,8 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
 #define KVX_WIDE(FMT, NB)                                                                        \
   launch_matrix_attention(attend_wide_kernel<FMT, NB>, "attend_wide_kernel", 16 * NB, 64, s, kv, \
                           query_heads, queries, output, page_tables, lanes, n_lanes, row_masks,  \
-                          row_stride, lane_stride, workspace, workspace_bytes, phases, stream)
+                          row_stride, lane_stride, workspace, workspace_bytes, phases, stream,    \
+                          nullptr, tile_rows)
   // Two blocks of 16 fused rows per wave share every key and value operand; a
   // third would not fit the register file next to a page of bf16 keys and values.
   // many_tiles: the lanes are the 8-row tiles of a chunked prefill.

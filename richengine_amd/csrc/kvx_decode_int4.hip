@@ -426,10 +426,8 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
 #ifdef KVX_PROBE_CLOCK
   const uint64_t probe_cycles = __builtin_readcyclecounter(), probe_wall = wall_clock64();
 #endif
-  uint32_t li = 0;
-  for (uint32_t i = 1; i < a.n_lanes; ++i)
-    if (item >= a.lane[i].first_item) li = i;
-  const DecodeLane &l = a.lane[li];
+  uint32_t li;
+  const DecodeLane l = lane_of_item(a, item, li);
   const uint32_t split = item - l.first_item;
   if (split >= l.split_count) return;
   const uint32_t visible = l.committed + l.active_rows;
@@ -656,7 +654,7 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
                            hipStream_t stream, const void *append_keys, const void *append_values,
-                           uint64_t append_lane_stride, uint32_t append_stride) {
+                           uint64_t append_lane_stride, uint32_t append_stride, uint32_t tile_rows) {
   if (s->layout.format != KVX_FMT_INT4 || !matrix_attention_covers(s, query_heads, lanes, n_lanes))
     return 1;
   const FusedAppend appended{append_keys, append_values, append_lane_stride, append_stride};
@@ -673,11 +671,11 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
     return launch_matrix_attention(verify_int4_kernel, "verify_int4_kernel", 32, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                   kvx_attend_phases(), stream);
+                                   kvx_attend_phases(), stream, nullptr, tile_rows);
   return launch_matrix_attention(decode_int4_kernel, "decode_int4_kernel", 16, 64, s, kv,
                                  query_heads, queries, output, page_tables, lanes, n_lanes,
                                  row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                 kvx_attend_phases(), stream, fused);
+                                 kvx_attend_phases(), stream, fused, tile_rows);
 }
 
 #ifdef KVX_PROBE_CLOCK

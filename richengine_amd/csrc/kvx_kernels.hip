@@ -571,14 +571,14 @@ int kvx_attend_int4_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
                            hipStream_t stream, const void *append_keys = nullptr,
                            const void *append_values = nullptr, uint64_t append_lane_stride = 0,
-                           uint32_t append_stride = 0);
+                           uint32_t append_stride = 0, uint32_t tile_rows = 0);
 
 int kvx_attend_wide_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t query_heads,
                            const void *queries, void *output, const uint64_t *const *page_tables,
                            const kvx_verify_params *lanes, uint32_t n_lanes,
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
-                           hipStream_t stream);
+                           hipStream_t stream, uint32_t tile_rows = 0);
 
 // int4 pages go to their own kernels, bf16 and fp8 pages to the wide-element
 // ones; 1 = neither covers the shape.
@@ -587,14 +587,18 @@ static int attend_matrix(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_h
                          const kvx_verify_params *lanes, uint32_t n_lanes,
                          const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                          void *workspace, uint64_t workspace_bytes, int many_tiles,
-                         hipStream_t stream) {
+                         hipStream_t stream, uint32_t tile_rows = 0) {
+  // tile_rows > 0: the lanes are regular (lane i = lane 0 moved on by i x tile_rows
+  // rows and tokens over one table, all full but perhaps the last), which lets
+  // any number of them share a launch.
   const int fast = kvx_attend_int4_launch(s, kv, query_heads, queries, output, page_tables, lanes,
                                           n_lanes, row_masks, row_stride, lane_stride, workspace,
-                                          workspace_bytes, many_tiles, stream);
+                                          workspace_bytes, many_tiles, stream, nullptr, nullptr, 0, 0,
+                                          tile_rows);
   if (fast <= 0) return fast;
   return kvx_attend_wide_launch(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes,
                                 row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                many_tiles, stream);
+                                many_tiles, stream, tile_rows);
 }
 
 uint32_t kvx_attend_phases() { return kvx::g_attend_phases; }
@@ -910,7 +914,7 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
     int fast = took(attend_matrix(s, kv, query_heads, queries, output, tile_tables.data(),
                                   tile_lanes.data(), wide_lanes, nullptr, params->chunk_stride,
                                   uint64_t(T) * width * G * D, workspace, workspace_bytes,
-                                  width == 1, st));
+                                  width == 1, st, T * width));
     if (fast == 0 && rest) {
       // The odd last tile on its own; lanes of one launch share a row capacity.
       const uint64_t skip = uint64_t(T) * width * wide_lanes * G * D;
