@@ -76,13 +76,21 @@ struct DecodeArgs {
 // The lane with this index of a launch: read from the arguments, or derived
 // from the first for regular lanes.
 __device__ __forceinline__ DecodeLane lane_at(const DecodeArgs &a, uint32_t index) {
-  if (!a.tile_lanes) return a.lane[index];
-  DecodeLane l = a.lane[0];
-  l.committed += index * a.tile_rows;
-  if (index + 1 == a.tile_lanes) l.active_rows = a.tile_last_rows;
-  l.first_item = index * l.split_count;
-  l.row_base += uint64_t(index) * l.split_count * a.kv_heads * a.fused_rows;
-  l.q_offset += index * a.tile_lane_stride;
+  // Field by field from a reference into the kernel arguments: a copy of a whole
+  // lane record picked by a run-time index would make the compiler move the
+  // argument block to scratch memory.
+  const uint32_t tile = a.tile_lanes ? index : 0u;
+  const DecodeLane &from = a.lane[a.tile_lanes ? 0u : index];
+  DecodeLane l;
+  l.table = from.table;
+  l.masks = from.masks;
+  l.committed = from.committed + tile * a.tile_rows;
+  l.active_rows = (a.tile_lanes && index + 1 == a.tile_lanes) ? a.tile_last_rows : from.active_rows;
+  l.split_count = from.split_count;
+  l.first_item = a.tile_lanes ? index * from.split_count : from.first_item;
+  l.score_scale = from.score_scale;
+  l.row_base = from.row_base + uint64_t(tile) * from.split_count * a.kv_heads * a.fused_rows;
+  l.q_offset = from.q_offset + tile * a.tile_lane_stride;
   return l;
 }
 // The lane that owns work item `item` (a lane's items are its splits), and its index.
