@@ -260,9 +260,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
   // kSets register sets rotate: a set's keys are refilled with the page kSets
   // ahead as soon as the page has multiplied its last key, its values when the
   // page is done, so more than one page is always in flight.
-  // Two sets wherever the register file of a SIMD lane holds them next to the
-  // accumulators: not for two row blocks over two-byte elements.
-  constexpr uint32_t kSets = (!kByte && NB > 1) ? 1 : 2;
+  // Two sets for the one-byte formats.  A page of two-byte elements is 128
+  // registers per lane: with two of them the compiler spills (and a spill reload
+  // waits behind every page load in flight), and one set already streams bf16
+  // decode at 5.5 TB/s (two sets with spills: 4.7).
+  constexpr uint32_t kSets = kByte ? 2 : 1;
   struct PageSet {
     KeyRegs<FMT> keys;
     ValueRegs<FMT> values;
