@@ -184,7 +184,7 @@ __device__ __forceinline__ u32x4 value_operand(const ValueRegs<FMT> &v, uint32_t
 }
 
 template <uint32_t FMT, uint32_t NB>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void attend_wide_kernel(const uint16_t *__restrict__ queries,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu((Wide<FMT>::kByte && NB == 1) ? 2 : 1, (Wide<FMT>::kByte && NB == 1) ? 2 : 1))) void attend_wide_kernel(const uint16_t *__restrict__ queries,
                                                          uint16_t *__restrict__ output,
                                                          float *__restrict__ partials,
                                                          float *__restrict__ statistics,
@@ -260,11 +260,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
   // kSets register sets rotate: a set's keys are refilled with the page kSets
   // ahead as soon as the page has multiplied its last key, its values when the
   // page is done, so more than one page is always in flight.
-  // Two sets for the one-byte formats.  A page of two-byte elements is 128
-  // registers per lane: with two of them the compiler spills (and a spill reload
-  // waits behind every page load in flight), and one set already streams bf16
-  // decode at 5.5 TB/s (two sets with spills: 4.7).
-  constexpr uint32_t kSets = kByte ? 2 : 1;
+  // Two sets for the one-byte formats with two row blocks (one wave per SIMD).
+  // With one row block those run two waves per SIMD with one set each, which
+  // overlaps one wave's expansion arithmetic with the other's loads better than
+  // one wave with two sets (int8 decode 262 -> 246 us).  A page of two-byte
+  // elements is 128 registers per lane: with two of them the compiler spills (and
+  // a spill reload waits behind every page load in flight), and one set already
+  // streams bf16 decode at 5.5 TB/s (two sets with spills: 4.7).
+  constexpr uint32_t kSets = (kByte && NB > 1) ? 2 : 1;
   struct PageSet {
     KeyRegs<FMT> keys;
     ValueRegs<FMT> values;
