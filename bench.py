@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the paged-KV decode path on one MI355X.
 
-Workload (BASELINE.json configs[2], the one the metric is quoted on): int4 KV,
+Workload (the configuration the headline metric is quoted on): int4 KV,
 16 layers, 4 KV heads x 256, 24 query heads, batch 32 with contexts drawn
 uniformly from [512, 32768]; pages come from a device-sized pool in a
 seed-shuffled order, reached through per-sequence page tables.  One step is one
@@ -57,9 +57,9 @@ def parse():
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
     ap.add_argument("--workload", choices=["decode", "tree-verify", "prefill"], default="decode",
-                    help="decode = BASELINE configs[2], the headline metric (default); "
-                         "tree-verify = configs[4] and prefill = configs[3], the matrix-core paths "
-                         "(profiling)")
+                    help="decode = batch-32 mixed-length int4 decode, the headline metric (default); "
+                         "tree-verify = 16-node tree verify and prefill = chunked prefill with a shared "
+                         "prefix, the matrix-core paths (profiling)")
     ap.add_argument("--format", choices=["bf16", "fp8", "int8", "int4"], default="bf16",
                     help="page format of the prefill workload")
     return ap.parse_args()
@@ -152,7 +152,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
 def tree_verify(args):
-    """BASELINE configs[4]: int4, batch 4, contexts 65536, a 16-node draft tree per
+    """Speculative tree verify: int4, batch 4, contexts 65536, a 16-node draft tree per
     sequence (branching <= 3).  A step = per layer, append the 16 draft rows and
     run masked verify attention over history + rows; then compact a seeded
     root-to-leaf path of every sequence, all layers in one call.  The dominant
@@ -274,7 +274,7 @@ def tree_verify(args):
 
 
 def chunked_prefill(args):
-    """BASELINE configs[3]: batch 4, a 2048-token chunk per sequence appended onto a
+    """Chunked prefill with prefix reuse: batch 4, a 2048-token chunk per sequence appended onto a
     shared 16384-token prefix (the prefix pages are the same physical pages in every
     sequence's table), bf16 or fp8 pages.  A step = per layer and sequence, quantize +
     scatter of the chunk, then causal attention of its 2048 rows over prefix + chunk.

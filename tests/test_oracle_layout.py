@@ -51,7 +51,7 @@ def test_byte_accounting_known_answers():
     assert (pf(ci8, 255), pf(ci8, 511), pf(ci8, 10_240), pf(ci8, 10_496)) == (0, 256, 512, 256)
     assert (pf(bf16, 31), pf(bf16, 448), pf(bf16, 97)) == (0, 64, 48)
     assert not L.ko_layout_valid(C.byref(ko.Layout(16, 4, 256, 0, 0.0)))
-    # BASELINE geometry: int4 = 1056 B/token/layer, fp8 = int8 geometry.
+    # benchmark geometry: int4 = 1056 B/token/layer, fp8 = int8 geometry.
     i4 = layout(16, 4, 256, ko.INT4)
     assert geo(i4)["model"] == 540_672 == 16 * 32 * 1056 and geo(i4)["align"] == 128
     assert geo(layout(16, 4, 256, ko.FP8))["model"] == 1_064_960
