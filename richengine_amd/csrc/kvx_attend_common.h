@@ -348,7 +348,10 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       if (e != hipSuccess) return hip_fail(e, name);
     }
     if (max_splits > 1 && (phases & 2u)) {
-      hipLaunchKernelGGL(matrix_merge_kernel, dim3(M, H, a.n_lanes), dim3(64 * kMergeWaves), 0,
+      // One wave per row is all the sequential merge uses; the other three only
+      // join in for lists longer than kMergeSequential.
+      const uint32_t merge_threads = max_splits <= kMergeSequential ? 64 : 64 * kMergeWaves;
+      hipLaunchKernelGGL(matrix_merge_kernel, dim3(M, H, a.n_lanes), dim3(merge_threads), 0,
                          stream, static_cast<uint16_t *>(output), partials, statistics, a);
       const hipError_t e = hipGetLastError();
       if (e != hipSuccess) return hip_fail(e, "matrix_merge_kernel");
