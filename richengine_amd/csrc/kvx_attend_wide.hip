@@ -183,8 +183,9 @@ __device__ __forceinline__ u32x4 value_operand(const ValueRegs<FMT> &v, uint32_t
   else return u32x4{v.raw[mb][0], v.raw[mb][1], v.raw[mb][2], v.raw[mb][3]};
 }
 
-template <uint32_t FMT, uint32_t NB>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu((Wide<FMT>::kByte && NB == 1) ? 2 : 1, (Wide<FMT>::kByte && NB == 1) ? 2 : 1))) void attend_wide_kernel(const uint16_t *__restrict__ queries,
+// WAVES: waves per SIMD the kernel is compiled for (1 or 2).
+template <uint32_t FMT, uint32_t NB, uint32_t WAVES>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) void attend_wide_kernel(const uint16_t *__restrict__ queries,
                                                          uint16_t *__restrict__ output,
                                                          float *__restrict__ partials,
                                                          float *__restrict__ statistics,
@@ -260,14 +261,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu((Wide<FMT>::
   // kSets register sets rotate: a set's keys are refilled with the page kSets
   // ahead as soon as the page has multiplied its last key, its values when the
   // page is done, so more than one page is always in flight.
-  // Two sets for the one-byte formats with two row blocks (one wave per SIMD).
-  // With one row block those run two waves per SIMD with one set each, which
-  // overlaps one wave's expansion arithmetic with the other's loads better than
-  // one wave with two sets (int8 decode 262 -> 246 us).  A page of two-byte
-  // elements is 128 registers per lane: with two of them the compiler spills (and
-  // a spill reload waits behind every page load in flight), and one set already
-  // streams bf16 decode at 5.5 TB/s (two sets with spills: 4.7).
-  constexpr uint32_t kSets = (kByte && NB > 1) ? 2 : 1;
+  // Two sets when the wave has a SIMD's registers to itself and the elements are
+  // one byte wide.  With two waves per SIMD each has one set, which overlaps one
+  // wave's expansion arithmetic with the other's loads better than one wave with
+  // two sets (int8 decode 262 -> 246 us).  A page of two-byte elements is 128 registers per lane:
+  // with two of them the compiler spills (and a spill reload waits behind every
+  // page load in flight), and one set already streams bf16 decode at 5.5 TB/s
+  // (two sets with spills: 4.7).
+  constexpr uint32_t kSets = (kByte && WAVES == 1) ? 2 : 1;
   struct PageSet {
     KeyRegs<FMT> keys;
     ValueRegs<FMT> values;
@@ -496,19 +497,21 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
     return 1;
   const uint32_t M = lanes[0].row_capacity * (query_heads / s->layout.kv_heads);
   const uint32_t phases = kvx_attend_phases();
-#define KVX_WIDE(FMT, NB)                                                                        \
-  launch_matrix_attention(attend_wide_kernel<FMT, NB>, "attend_wide_kernel", 16 * NB, 64, s, kv, \
-                          query_heads, queries, output, page_tables, lanes, n_lanes, row_masks,  \
-                          row_stride, lane_stride, workspace, workspace_bytes, phases, stream,    \
+#define KVX_WIDE(FMT, NB, WAVES)                                                                 \
+  launch_matrix_attention(attend_wide_kernel<FMT, NB, WAVES>, "attend_wide_kernel", 16 * NB, 64, s, \
+                          kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks, \
+                          row_stride, lane_stride, workspace, workspace_bytes, phases, stream,      \
                           nullptr, tile_rows)
   // Two blocks of 16 fused rows per wave share every key and value operand; a
   // third would not fit the register file next to a page of bf16 keys and values.
-  // many_tiles: the lanes are the 8-row tiles of a chunked prefill.
-  // Measured on 2048-row prefill over 16384 tokens: bf16 8.1 ms per sequence and
-  // layer with two blocks per wave against 10.1 with one; fp8, whose byte
-  // expansion makes it VALU-bound at one wave per SIMD, 14.2 against 12.1.
-  if (format == KVX_FMT_BF16) return M > 16 ? KVX_WIDE(KVX_FMT_BF16, 2) : KVX_WIDE(KVX_FMT_BF16, 1);
-  if (format == KVX_FMT_INT8) return M > 16 ? KVX_WIDE(KVX_FMT_INT8, 2) : KVX_WIDE(KVX_FMT_INT8, 1);
-  return M > 16 && !many_tiles ? KVX_WIDE(KVX_FMT_FP8E4M3, 2) : KVX_WIDE(KVX_FMT_FP8E4M3, 1);
+  // One-byte formats run two waves per SIMD with one block (decode, the 8-row
+  // tiles of a prefill with several splits); with two blocks the accumulators
+  // leave too little room for that (the compiler spills inside the page loop:
+  // int8 prefill 2.9 -> 4.5 ms), so those keep the SIMD to themselves.
+  if (format == KVX_FMT_BF16)
+    return M > 16 ? KVX_WIDE(KVX_FMT_BF16, 2, 1) : KVX_WIDE(KVX_FMT_BF16, 1, 1);
+  const bool two_blocks = M > 16 && !many_tiles;
+  if (format == KVX_FMT_INT8) return two_blocks ? KVX_WIDE(KVX_FMT_INT8, 2, 1) : KVX_WIDE(KVX_FMT_INT8, 1, 2);
+  return two_blocks ? KVX_WIDE(KVX_FMT_FP8E4M3, 2, 1) : KVX_WIDE(KVX_FMT_FP8E4M3, 1, 2);
 #undef KVX_WIDE
 }

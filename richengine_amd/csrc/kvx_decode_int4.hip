@@ -350,7 +350,7 @@ __device__ __forceinline__ void append_decode_token(const DecodeArgs &a, const D
 #ifndef KVX_DECODE_DEPTH
 #define KVX_DECODE_DEPTH 2
 #endif
-constexpr uint32_t kDepth = KVX_DECODE_DEPTH;
+constexpr uint32_t kDecodeDepth = KVX_DECODE_DEPTH;
 
 // Writes what a wave has accumulated for its NB blocks: the finished bf16 rows
 // when the lane has a single split, else fp32 partial rows and (max, sum).
@@ -416,8 +416,9 @@ __device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m,
   }
 }
 
-// The split kernel's body for NB blocks of 16 fused query rows per wave.
-template <uint32_t NB>
+// The split kernel's body for NB blocks of 16 fused query rows per wave, with
+// kDepth register sets of pages.
+template <uint32_t NB, uint32_t kDepth>
 __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries,
                                             uint16_t *__restrict__ output,
                                             float *__restrict__ partials,
@@ -621,7 +622,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_int4_kernel(
     const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
     float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
-  attend_int4<1>(queries, output, partials, statistics, a);
+  attend_int4<1, kDecodeDepth>(queries, output, partials, statistics, a);
 }
 
 // Two blocks per wave share every expanded key and value operand (verify, tree
@@ -630,7 +631,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void verify_int4_kernel(
     const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
     float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
-  attend_int4<2>(queries, output, partials, statistics, a);
+  attend_int4<2, 2>(queries, output, partials, statistics, a);
+}
+
+// The same two blocks with one register set of pages, which fits two waves per
+// SIMD: for the paired tiles of a chunked prefill, whose 1536 waves per 2048-row
+// chunk then all run at once instead of in a full round and a half-empty one
+// (2.0 -> 1.5 ms on 2048 rows over 16K tokens).  Verify batches, sized to one
+// wave per SIMD by their plan, are faster with two sets and the SIMD to
+// themselves.
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_int4_kernel(
+    const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
+    float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
+  attend_int4<2, 1>(queries, output, partials, statistics, a);
 }
 
 }  // namespace
@@ -667,6 +680,11 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   // and long (verify: 13% on 4 x 65536 tokens x 16 tree rows); chunked prefill has
   // hundreds of tiles of 48 fused rows, where a half-empty second wave and one
   // wave per SIMD cost more than the sharing saves.
+  if (fused_rows > 16 && !many_tiles && tile_rows)
+    return launch_matrix_attention(prefill_int4_kernel, "prefill_int4_kernel", 32, 64, s, kv,
+                                   query_heads, queries, output, page_tables, lanes, n_lanes,
+                                   row_masks, row_stride, lane_stride, workspace, workspace_bytes,
+                                   kvx_attend_phases(), stream, nullptr, tile_rows);
   if (fused_rows > 16 && !many_tiles)
     return launch_matrix_attention(verify_int4_kernel, "verify_int4_kernel", 32, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
