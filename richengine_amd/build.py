@@ -1,5 +1,7 @@
 """Builds libkvx.so (HIP kernels + C ABI) for gfx950, in-tree."""
+import json
 import os
+import re
 import subprocess
 import sys
 
@@ -14,23 +16,59 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
          # packed fp32 instructions stay off for every kernel of this library
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-I", os.path.join(ROOT, "include"), "-I", CSRC]
+# What the compiler reports per kernel (registers, scratch bytes per lane, spills,
+# waves per SIMD) goes to this file next to the library, so that a change that
+# sends a hot kernel to scratch memory shows up without a GPU.
+RESOURCES = os.path.join(HERE, "kernel_resources.json")
+REMARK = re.compile(r"remark:\s+(Function Name|VGPRs|AGPRs|ScratchSize \[bytes/lane\]|"
+                    r"Occupancy \[waves/SIMD\]|VGPRs Spill|LDS Size \[bytes/block\]): (\S+)")
+
+
+def kernel_resources(compiler_stderr):
+    """{kernel name: {field: value}} from -Rpass-analysis=kernel-resource-usage remarks."""
+    kernels, current = {}, None
+    for line in compiler_stderr.splitlines():
+        m = REMARK.search(line)
+        if not m:
+            continue
+        field, value = m.groups()
+        if field == "Function Name":
+            current = kernels.setdefault(value, {})
+        elif current is not None:
+            current[field.split(" [")[0].replace(" ", "_").lower()] = int(value)
+    return kernels
 
 
 def build(verbose=True, lib=LIB, extra_flags=(), tag=""):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    objects = []
+    objects, resources = [], {}
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
     for src in SOURCES:
         obj = os.path.join(HERE, "build", src + tag + ".o")
         cmd = [hipcc, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + FLAGS + list(extra_flags)
+        if src.endswith(".hip"):
+            cmd.append("-Rpass-analysis=kernel-resource-usage")
         if verbose:
             print(" ".join(cmd), flush=True)
-        subprocess.check_call(cmd)
+        done = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+        # the remarks and the host pass's note about the packed-fp32 feature are not warnings
+        for line in done.stderr.splitlines():
+            if "kernel-resource-usage" in line or "packed-fp32-ops" in line:
+                continue
+            if re.match(r"\s*\d* *\||\s*\^|In file included from", line) and "warning" not in done.stderr:
+                continue
+            print(line, file=sys.stderr)
+        if done.returncode:
+            raise subprocess.CalledProcessError(done.returncode, cmd)
+        resources.update(kernel_resources(done.stderr))
         objects.append(obj)
     cmd = [hipcc, "-shared", "-o", lib] + objects + ["--offload-arch=gfx950"]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    if lib == LIB:
+        with open(RESOURCES, "w") as out:
+            json.dump(resources, out, indent=1, sort_keys=True)
     return lib
 
 

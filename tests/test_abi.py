@@ -134,3 +134,34 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
     assert kvx.verify_plan([65536] * 4, 16, H, QH) == [21] * 4
     with pytest.raises(kvx.KvxError):
         kvx.verify_plan([10], 8, 4, 6)
+
+
+def test_hot_kernels_stay_out_of_scratch_memory():
+    """What the compiler reported when the library was built (written next to it by
+    richengine_amd/build.py): the kernels of the decode path and the verify kernel must
+    not touch scratch memory -- a spill reload or an argument block moved to scratch waits
+    behind every page load in flight -- and the int4 decode kernel must fit two waves per
+    SIMD."""
+    import json
+    import os
+    from richengine_amd import build as kvx_build
+    if not os.path.exists(kvx_build.RESOURCES):
+        pytest.skip("the library was built without the compiler's resource report")
+    report = json.load(open(kvx_build.RESOURCES))
+
+    def one(fragment):
+        names = [n for n in report if fragment in n]
+        assert len(names) == 1, (fragment, names)
+        return report[names[0]]
+
+    for fragment in ("decode_int4_kernel", "verify_int4_kernel", "matrix_merge_kernel",
+                     "attend_wide_kernelILj1ELj1ELj2E",    # int8, one block, two waves per SIMD
+                     "attend_wide_kernelILj4ELj1ELj2E",    # fp8
+                     "attend_wide_kernelILj2ELj1ELj1E",    # bf16 decode
+                     "attend_wide_kernelILj1ELj2ELj1E", "attend_wide_kernelILj4ELj2ELj1E"):
+        r = one(fragment)
+        assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, (fragment, r)
+    assert one("decode_int4_kernel")["occupancy"] == 2
+    assert one("attend_wide_kernelILj1ELj1ELj2E")["occupancy"] == 2
+    for fmt in (1, 2, 3, 4):
+        assert one(f"append_kernelILj{fmt}E")["scratchsize"] == 0
