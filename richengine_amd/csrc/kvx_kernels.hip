@@ -118,6 +118,114 @@ __global__ __launch_bounds__(256) void append_kernel(const uint16_t *__restrict_
   }
 }
 
+// The same store for chunks of many tokens: one workgroup per (lane, logical page
+// the chunk touches, head, tensor) stages the page's share of the chunk in LDS,
+// so that the value rows, which the chunk holds dimension-major, are read as
+// runs of consecutive tokens instead of one element per 2 x stride bytes, and so
+// that dimension-major value pages are written as runs too.  Each wave then
+// quantizes whole token rows; the arithmetic and the bytes are those of
+// append_kernel.
+constexpr uint32_t kAppendMaxD = 256;
+template <uint32_t FMT>
+__global__ __launch_bounds__(256) void append_page_kernel(const uint16_t *__restrict__ chunk_keys,
+                                                          const uint16_t *__restrict__ chunk_values,
+                                                          AppendArgs a) {
+  __shared__ uint16_t tile[kPage][kAppendMaxD + 2];
+  __shared__ uint8_t codes[kPage][kAppendMaxD + 4];
+  const uint32_t group = blockIdx.x;
+  uint32_t li = 0;
+  for (uint32_t i = 1; i < a.n_lanes; ++i)
+    if (group >= a.lane[i].group_base) li = i;
+  const AppendLane &l = a.lane[li];
+  if (!append_contract(l, a)) return;
+  const uint32_t D = a.head_dim, H = a.kv_heads;
+  const uint32_t first_page = l.committed / kPage;
+  const uint32_t touched = (l.committed + l.tokens - 1) / kPage - first_page + 1;
+  const uint32_t local = group - l.group_base;
+  if (local >= touched * 2 * H) return;
+  const uint32_t page = first_page + local / (2 * H);
+  const bool value_tensor = local % (2 * H) >= H;
+  const uint32_t head = local % H;
+  // Chunk tokens [begin, begin + n) live in this page, from slot0 on.
+  const uint32_t begin = max(l.committed, page * kPage) - l.committed;
+  const uint32_t n = min(l.committed + l.tokens, (page + 1) * kPage) - l.committed - begin;
+  const uint32_t slot0 = (l.committed + begin) % kPage;
+  const Slab s = slab_of(FMT, H, D, a.kv, head, l.table[page]);
+  const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+  if (!value_tensor) {
+    const uint16_t *rows = chunk_keys + li * a.lane_stride + (uint64_t(head) * l.stride + begin) * D;
+    for (uint32_t i = tid; i < n * D; i += 256) tile[i / D][i % D] = rows[i];
+  } else {
+    const uint16_t *columns = chunk_values + li * a.lane_stride + uint64_t(head) * D * l.stride + begin;
+    for (uint32_t i = tid; i < D * kPage; i += 256) {
+      const uint32_t d = i / kPage, t = i % kPage;
+      if (t < n) tile[t][d] = columns[uint64_t(d) * l.stride + t];
+    }
+  }
+  __syncthreads();
+  // Element index inside the head's slab: keys token-major, values
+  // dimension-major (packed int4: both token-major).
+  const bool dimension_major = value_tensor && FMT != KVX_FMT_INT4;
+  uint8_t *data = value_tensor ? s.values : s.keys;
+  if constexpr (FMT == KVX_FMT_BF16) {
+    uint16_t *out = reinterpret_cast<uint16_t *>(data);
+    if (!dimension_major) {
+      for (uint32_t i = tid; i < n * D; i += 256) out[(slot0 + i / D) * D + i % D] = tile[i / D][i % D];
+    } else {
+      for (uint32_t i = tid; i < D * kPage; i += 256) {
+        const uint32_t d = i / kPage, t = i % kPage;
+        if (t < n) out[d * kPage + slot0 + t] = tile[t][d];
+      }
+    }
+    return;
+  } else {
+    constexpr float qmax = FMT == KVX_FMT_INT4 ? 7.0f : FMT == KVX_FMT_INT8 ? 127.0f : 448.0f;
+    for (uint32_t t = wave; t < n; t += 4) {
+      const uint32_t slot = slot0 + t;
+      float v[kAppendMaxD / 64], maximum = 0.0f;
+#pragma unroll
+      for (uint32_t k = 0; k < kAppendMaxD / 64; ++k) {
+        const uint32_t d = lane + 64 * k;
+        v[k] = d < D ? bf16_to_f32(tile[t][d]) : 0.0f;
+        maximum = fmaxf(maximum, fabsf(v[k]));
+      }
+      for (int offset = 32; offset; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset));
+      const float scale = maximum == 0.0f ? 0.0f : __fdiv_rn(maximum, qmax);
+      if (lane == 0) (value_tensor ? s.value_scales : s.key_scales)[slot] = scale;
+#pragma unroll
+      for (uint32_t k = 0; k < kAppendMaxD / 64; ++k) {
+        const uint32_t d = lane + 64 * k;
+        const float scaled = maximum == 0.0f ? 0.0f : __fdiv_rn(__fmul_rn(v[k], qmax), maximum);
+        uint32_t byte;
+        if constexpr (FMT == KVX_FMT_FP8E4M3) {
+          byte = maximum == 0.0f ? 0u : f32_to_e4m3(scaled);
+        } else {
+          constexpr int limit = FMT == KVX_FMT_INT4 ? 7 : 127;
+          int code = int(rintf(scaled));
+          code = code < -limit ? -limit : code > limit ? limit : code;
+          if (maximum == 0.0f) code = 0;
+          byte = uint32_t(code) & (FMT == KVX_FMT_INT4 ? 0xfu : 0xffu);
+        }
+        if constexpr (FMT == KVX_FMT_INT4) {
+          // Even dimension in the low nibble; the even lane writes the byte.
+          const uint32_t partner = __shfl_xor(byte, 1);
+          if (d < D && (d & 1) == 0) data[(slot * D + d) >> 1] = uint8_t(byte | (partner << 4));
+        } else if (d < D) {
+          if (dimension_major) codes[t][d] = uint8_t(byte);
+          else data[slot * D + d] = uint8_t(byte);
+        }
+      }
+    }
+    if (dimension_major) {
+      __syncthreads();
+      for (uint32_t i = tid; i < D * kPage; i += 256) {
+        const uint32_t d = i / kPage, t = i % kPage;
+        if (t < n) data[d * kPage + slot0 + t] = codes[t][d];
+      }
+    }
+  }
+}
+
 // ===================================================== generic attention ====
 // One tile = row_capacity query rows x `group` query heads of one KV head
 // (M fused rows) over the pages of one split.
@@ -661,7 +769,27 @@ int kv_append(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
       if (lanes[first + i].chunk_tokens != lanes[first].chunk_tokens) a.uniform_groups = 0;
     const auto *keys = static_cast<const uint16_t *>(chunk_keys) + uint64_t(first) * lane_stride;
     const auto *values = static_cast<const uint16_t *>(chunk_values) + uint64_t(first) * lane_stride;
+    // Chunks of many tokens go page by page through LDS; a few rows per lane
+    // (decode, verify) keep one workgroup per row, which has the shorter latency.
+    bool by_page = !verify_max_rows && D <= kAppendMaxD;
+    uint32_t most = 0;
+    for (uint32_t i = 0; i < a.n_lanes; ++i) most = std::max(most, lanes[first + i].chunk_tokens);
+    by_page = by_page && most > KVX_TREE_NODES;
+    if (by_page) {
+      groups = 0;
+      for (uint32_t i = 0; i < a.n_lanes; ++i) {
+        const kvx_chunk_params &p = lanes[first + i];
+        a.lane[i].group_base = groups;
+        groups += ((p.committed_tokens + p.chunk_tokens - 1) / kPage - p.committed_tokens / kPage + 1) * 2 * H;
+      }
+      a.uniform_groups = 0;
+    }
     const int rc = dispatch_format(s->layout.format, [&](auto fmt) {
+      if (by_page) {
+        hipLaunchKernelGGL((append_page_kernel<decltype(fmt)::value>), dim3(groups), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), keys, values, a);
+        return check_launch("append_page_kernel");
+      }
       hipLaunchKernelGGL((append_kernel<decltype(fmt)::value>), dim3(groups), dim3(D), 0,
                          static_cast<hipStream_t>(stream), keys, values, a);
       return check_launch("append_kernel");
