@@ -625,8 +625,20 @@ __global__ __launch_bounds__(256) void page_copy_kernel(CopyArgs a) {
   const uint64_t start = tensor == 0 ? 0 : tensor == 1 ? r.key_scales : tensor == 2 ? r.values : r.value_scales;
   const uint8_t *src = reinterpret_cast<const uint8_t *>(from - fi) + region + start + uint64_t(fi) * bytes;
   uint8_t *dst = reinterpret_cast<uint8_t *>(to - ti) + region + start + uint64_t(ti) * bytes;
-  for (uint32_t o = begin + threadIdx.x * 16; o < end; o += 256 * 16)
-    *reinterpret_cast<uint4 *>(dst + o) = *reinterpret_cast<const uint4 *>(src + o);
+  // A chunk is four steps of the workgroup: all four loads go out before the
+  // first store, so a thread has 64 bytes in flight instead of 16.
+  static_assert(kCopyChunk == 4 * 256 * 16, "a chunk is four 16-byte steps of 256 threads");
+  const uint32_t o = begin + threadIdx.x * 16;
+  typedef uint32_t word4 __attribute__((ext_vector_type(4)));
+  word4 v[4];
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i)
+    if (o + i * 4096 < end)
+      v[i] = __builtin_nontemporal_load(reinterpret_cast<const word4 *>(src + o + i * 4096));
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i)
+    if (o + i * 4096 < end)
+      __builtin_nontemporal_store(v[i], reinterpret_cast<word4 *>(dst + o + i * 4096));
 }
 
 // ============================================================= launchers ====
