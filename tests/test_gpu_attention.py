@@ -400,6 +400,8 @@ def test_append_attend_decode_is_the_two_calls(fmt):
     bit for bit) and returns the output of kv_attend_decode; int4 pages take the
     kernel that stores the token itself."""
     committed = [0, 31, 32, 700, 4095, 1000, 63, 2047, 5000]
+    if fmt == ko.INT4:  # more lanes than one launch holds
+        committed += [int(x) for x in np.random.default_rng(60).integers(0, 1500, 31)]
     lanes = len(committed)
     tw, counts, hts, dts = shared_pool_lanes(fmt, committed, 1, seed=61)
     rng = np.random.default_rng(62)
