@@ -92,7 +92,7 @@ __device__ __forceinline__ void load_page(PageRegs &r, uint64_t entry, uint32_t 
       r.v[s] = load_streaming<u32x2>(values + at.values + ((s < 4 ? 0 : 16) + (s & 3)) * kRowBytes);
     // One scale per lane instead of the sixteen a lane multiplies with: they
     // are fetched from the owning lanes when the page is attended, which keeps
-    // a register set small enough for three of them.
+    // a register set at 33 registers.
     r.scale = load_global<float>(region + key_scales_off + head_page * (kPage * 4u) + at.scale);
   }
 }

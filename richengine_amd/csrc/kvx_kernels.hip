@@ -700,7 +700,7 @@ int kvx_attend_wide_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
                            hipStream_t stream, uint32_t tile_rows = 0);
 
-// int4 pages go to their own kernels, bf16 and fp8 pages to the wide-element
+// int4 pages go to their own kernels, bf16, fp8 and int8 pages to the wide-element
 // ones; 1 = neither covers the shape.
 static int attend_matrix(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_heads,
                          const void *queries, void *output, const uint64_t *const *page_tables,
