@@ -151,14 +151,19 @@ uint32_t kvx_prefill_splits(uint32_t rows);
    floor would only add partial traffic. */
 #define KVX_DECODE_PAGES_PER_SPLIT 32u
 uint32_t kvx_decode_splits(uint32_t committed_tokens, uint32_t rows);
-/* The same rule for a whole decode batch, which also fills the GPU when the batch is small:
-   pages per split = clamp(ceil(total page-heads / 1024 waves), 8, 32), and each lane gets
-   clamp(ceil(its pages / that), 1, KVX_DECODE_MAX_SPLITS) splits.  One-row decode lanes may
-   use up to KVX_DECODE_MAX_SPLITS splits; every other attend entry keeps the reference's
-   KVX_VERIFY_MAX_SPLITS. */
+/* The split counts of a whole decode batch of pages of `format`.  A launch runs (sum of splits) x
+   KV heads waves; the plan is a split length in pages, each lane getting
+   clamp(ceil(its pages / that), 1, KVX_DECODE_MAX_SPLITS) splits.  The length starts at
+   max(ceil(total page-heads / 1024), 8) (at most 32 for int4, whose kernel holds two waves per
+   SIMD and is fastest at 32), which fills the GPU when the batch is small, and grows until the
+   launch has no more waves than the kernel has wave slots (2048 for int4, 1024 for the other
+   formats), because waves beyond that run as a second round on a nearly empty GPU.  One-row
+   decode lanes may use up to KVX_DECODE_MAX_SPLITS splits; every other attend entry keeps the
+   reference's KVX_VERIFY_MAX_SPLITS.  No counterpart in the reference, whose decode shares the
+   verify plan (runtime/ops/PagedAttention.cpp:232-262). */
 #define KVX_DECODE_MAX_SPLITS 512u
 int kvx_decode_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t kv_heads,
-                    uint32_t *split_counts);
+                    uint32_t format, uint32_t *split_counts);
 /* Split counts of a verify batch (`rows` live rows per lane) sized for this GPU instead of
    the reference's clamp(ceil(pages/16), 32, 128): the longest split length (at least 8 pages)
    for which the launch has no more waves than the GPU has SIMDs (1024), each lane getting

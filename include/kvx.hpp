@@ -355,7 +355,8 @@ public:
     VerifyAttentionPlan plan{layout.format, lanes, {}, 0, {}, rows, queryHeads, layout.scoreScale};
     if (sizedForGpu) {
       plan.laneSplits.resize(lanes);
-      check(decode ? kvx_decode_plan(historyTokens.data(), lanes, layout.kvHeads, plan.laneSplits.data())
+      check(decode ? kvx_decode_plan(historyTokens.data(), lanes, layout.kvHeads,
+                                     static_cast<uint32_t>(layout.format), plan.laneSplits.data())
                    : kvx_verify_plan(historyTokens.data(), lanes, rows, layout.kvHeads, queryHeads,
                                      plan.laneSplits.data()));
       for (uint32_t splits : plan.laneSplits) plan.splits = std::max(plan.splits, splits);

@@ -164,21 +164,34 @@ uint32_t kvx_decode_splits(uint32_t committed, uint32_t rows) {
   const uint32_t wanted = (pages + KVX_DECODE_PAGES_PER_SPLIT - 1) / KVX_DECODE_PAGES_PER_SPLIT;
   return std::min(std::max(1u, wanted), KVX_VERIFY_MAX_SPLITS);
 }
-int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_heads,
+int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_heads, uint32_t format,
                     uint32_t *split_counts) {
   if (!committed || !split_counts || !n_lanes || !kv_heads)
     return fail(KVX_EINVAL, "kvx_decode_plan: null argument or empty batch");
-  // One wave per SIMD of 256 CUs x 4 SIMDs is the least that fills the GPU;
-  // shorter splits than 8 pages cost more in set-up and partial rows than they
-  // win, and once the batch is large 32 pages per split measure best.
-  constexpr uint64_t kWaves = 1024;
+  // A launch runs (sum of splits) x KV heads waves.  One per SIMD of 256 CUs x 4
+  // is the least that fills the GPU; shorter splits than 8 pages cost more in
+  // set-up and partial rows than they win.  What must not happen is a launch
+  // with more waves than the kernel has wave slots: the overflow runs as a second
+  // round on a nearly empty GPU (measured on 530 K tokens: int4 146 -> 115 us,
+  // bf16 397 -> 350 us once the waves fit).  The int4 kernel holds two waves per
+  // SIMD and is fastest with 32 pages per split as long as those fit; the other
+  // formats' kernels are fastest with one wave per SIMD.
+  constexpr uint64_t kSimds = 1024;
+  const uint64_t slots = format == KVX_FMT_INT4 ? 2 * kSimds : kSimds;
   uint64_t page_heads = 0;
   for (uint32_t i = 0; i < n_lanes; ++i) page_heads += uint64_t(pages_of(uint64_t(committed[i]) + 1)) * kv_heads;
-  const uint32_t per = uint32_t(std::min<uint64_t>(
-      std::max<uint64_t>((page_heads + kWaves - 1) / kWaves, 8), KVX_DECODE_PAGES_PER_SPLIT));
-  for (uint32_t i = 0; i < n_lanes; ++i) {
-    const uint32_t pages = pages_of(uint64_t(committed[i]) + 1);
-    split_counts[i] = std::min(std::max(1u, (pages + per - 1) / per), KVX_DECODE_MAX_SPLITS);
+  uint32_t per = uint32_t(std::max<uint64_t>((page_heads + kSimds - 1) / kSimds, 8));
+  if (format == KVX_FMT_INT4) per = std::min(per, KVX_DECODE_PAGES_PER_SPLIT);
+  for (;; ++per) {
+    uint64_t waves = 0;
+    bool single = true;
+    for (uint32_t i = 0; i < n_lanes; ++i) {
+      const uint32_t pages = pages_of(uint64_t(committed[i]) + 1);
+      split_counts[i] = std::min(std::max(1u, (pages + per - 1) / per), KVX_DECODE_MAX_SPLITS);
+      waves += uint64_t(split_counts[i]) * kv_heads;
+      single = single && split_counts[i] == 1;
+    }
+    if (waves <= slots || single) break;  // one split per lane is the fewest waves there can be
   }
   return KVX_OK;
 }

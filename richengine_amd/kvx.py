@@ -167,7 +167,7 @@ def _declare(L):
     L.kvx_sequence_view.argtypes = [vp, u64, C.POINTER(SequencePages)]
     L.kvx_sequences_compact_extent.argtypes = [vp, PU32, vp, PU32, vp]
     L.kvx_debug_attend_paths.argtypes, L.kvx_debug_attend_paths.restype = [PU64, PU64], None
-    L.kvx_decode_plan.argtypes = [vp, u32, u32, vp]
+    L.kvx_decode_plan.argtypes = [vp, u32, u32, u32, vp]
     L.kvx_verify_plan.argtypes = [vp, u32, u32, u32, u32, vp]
     L.kvx_tree_masks.argtypes = [vp, u32, vp]
     L.kvx_tree_path_valid.argtypes = [vp, u32, vp, u32]
@@ -569,10 +569,10 @@ class Sequences:
         return {"first": first.value, "dest": list(dest), "moved": moved.value}
 
 
-def decode_plan(committed, kv_heads):
-    """Split counts of a decode batch (kvx_decode_plan)."""
+def decode_plan(committed, kv_heads, fmt=INT4):
+    """Split counts of a decode batch of pages of format `fmt` (kvx_decode_plan)."""
     out = (C.c_uint32 * len(committed))()
-    check(lib().kvx_decode_plan(_u32(committed), len(committed), kv_heads, out))
+    check(lib().kvx_decode_plan(_u32(committed), len(committed), kv_heads, fmt, out))
     return list(out)
 
 

@@ -115,10 +115,18 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
     for trial in range(40):
         lanes = int(rng.integers(1, 40))
         committed = [int(x) for x in rng.integers(0, 70000, lanes)]
-        plan = kvx.decode_plan(committed, H)
         heads_pages = sum(pages(c + 1) for c in committed) * H
-        per = min(max(-(-heads_pages // 1024), 8), 32)
-        assert plan == [min(max(1, -(-pages(c + 1) // per)), 512) for c in committed]
+        for fmt, slots in ((kvx.INT4, 2048), (kvx.INT8, 1024), (kvx.BF16, 1024), (kvx.FP8, 1024)):
+            plan = kvx.decode_plan(committed, H, fmt)
+            per = max(-(-heads_pages // 1024), 8)
+            if fmt == kvx.INT4:
+                per = min(per, 32)
+            while True:  # the rule, restated: the first length whose waves fit the kernel's slots
+                want = [min(max(1, -(-pages(c + 1) // per)), 512) for c in committed]
+                if sum(want) * H <= slots or all(s == 1 for s in want):
+                    break
+                per += 1
+            assert plan == want
         for rows in (2, 8, 16):
             plan = kvx.verify_plan(committed, rows, H, QH)
             blocks = -(-rows * (QH // H) // 32) if rows * (QH // H) > 16 else 1
