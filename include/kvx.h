@@ -237,6 +237,17 @@ int kvx_storage_write_entries(const kvx_storage *storage, const uint32_t *pages,
    (bytes_per_page long), copied to / from host memory.  Synchronous. */
 int kvx_storage_page_read(const kvx_storage *storage, uint32_t page, void *host_bytes);
 int kvx_storage_page_write(kvx_storage *storage, uint32_t page, const void *host_bytes);
+/* The same wire form for many pages at once and without a host round trip per span: page i of
+   the list occupies bytes [i, i + 1) x bytes_per_page of `buffer`, which is device memory or
+   pinned host memory the device can reach (hipHostMalloc), so that a host or disk tier can
+   demote and restore pages byte for byte (engine::KvPageTier::demote / restore,
+   runtime/engine/cache/KvPageTier.hpp:13-21, which moves PageStorage::spans to and from a slot
+   file).  Enqueued on `stream`; nothing is enqueued when a page id is invalid, its extent is not
+   allocated, or two imported pages share a destination. */
+int kv_page_export(const kvx_storage *storage, const uint32_t *pages, uint32_t n, void *buffer,
+                   void *stream);
+int kv_page_import(kvx_storage *storage, const uint32_t *pages, uint32_t n, const void *buffer,
+                   void *stream);
 /* Raw extent bytes, for tests that compare whole extents.  Synchronous. */
 int kvx_storage_extent_read(const kvx_storage *storage, uint32_t extent, uint64_t offset,
                             uint64_t bytes, void *host_bytes);

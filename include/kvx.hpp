@@ -159,6 +159,15 @@ public:
     check(kv_page_copy(storage_, copies, static_cast<uint32_t>(count), stream_));
   }
   void copyPages(const std::vector<PageCopy> &copies) { copyPages(copies.data(), copies.size()); }
+  // The pages' spans (PageStorage::spans, PageStorage.mm:143-167) as one linear
+  // buffer, page after page: what a host or disk tier demotes and restores
+  // (engine::KvPageTier).  `buffer` is device memory or pinned host memory.
+  void exportPages(const std::vector<uint32_t> &pages, void *buffer) const {
+    check(kv_page_export(storage_, pages.data(), static_cast<uint32_t>(pages.size()), buffer, stream_));
+  }
+  void importPages(const std::vector<uint32_t> &pages, const void *buffer) {
+    check(kv_page_import(storage_, pages.data(), static_cast<uint32_t>(pages.size()), buffer, stream_));
+  }
 
   KvLayer layer(uint32_t index) const {
     KvLayer out{};

@@ -641,6 +641,49 @@ __global__ __launch_bounds__(256) void page_copy_kernel(CopyArgs a) {
       __builtin_nontemporal_store(v[i], reinterpret_cast<word4 *>(dst + o + i * 4096));
 }
 
+// Pages to and from their wire form: a page's spans in the order the reference's
+// storage hands them to its disk tier (PageStorage::spans,
+// runtime/ops/PageStorage.mm:143-167: layer by layer, keys, key scales, values,
+// value scales), bytes_per_page per page, page after page in one linear buffer.
+// Same grid as page_copy_kernel: blockIdx = (chunk of the span, layer * 4 +
+// tensor, page of the launch).
+struct WireArgs {
+  uint64_t page[kCopiesPerLaunch];  // page entries (extent address | index)
+  uint8_t *buffer;                  // wire bytes of the launch's first page
+  uint32_t extent_pages, data_bytes, scale_bytes, layers;
+};
+template <bool EXPORT>
+__global__ __launch_bounds__(256) void page_wire_kernel(WireArgs a) {
+  const uint32_t tensor = blockIdx.y & 3, layer = blockIdx.y >> 2;
+  const uint32_t bytes = (tensor & 1) ? a.scale_bytes : a.data_bytes;
+  const uint32_t begin = blockIdx.x * kCopyChunk;
+  if (begin >= bytes) return;
+  const uint32_t end = min(bytes, begin + kCopyChunk);
+  const uint64_t entry = a.page[blockIdx.z];
+  const uint32_t index = uint32_t(entry) & KVX_PAGE_INDEX_MASK;
+  const RegionOffsets r = region_offsets(a.extent_pages, a.data_bytes, a.scale_bytes);
+  const uint64_t layer_bytes = 2 * (uint64_t(a.data_bytes) + a.scale_bytes);
+  const uint64_t start = tensor == 0 ? 0 : tensor == 1 ? r.key_scales : tensor == 2 ? r.values : r.value_scales;
+  uint8_t *paged = reinterpret_cast<uint8_t *>(entry - index) + uint64_t(layer) * a.extent_pages * layer_bytes +
+                   start + uint64_t(index) * bytes;
+  const uint64_t wire_start = tensor == 0   ? 0
+                              : tensor == 1 ? a.data_bytes
+                              : tensor == 2 ? uint64_t(a.data_bytes) + a.scale_bytes
+                                            : 2 * uint64_t(a.data_bytes) + a.scale_bytes;
+  uint8_t *wire = a.buffer + (uint64_t(blockIdx.z) * a.layers + layer) * layer_bytes + wire_start;
+  const uint8_t *src = EXPORT ? paged : wire;
+  uint8_t *dst = EXPORT ? wire : paged;
+  typedef uint32_t word4 __attribute__((ext_vector_type(4)));
+  const uint32_t o = begin + threadIdx.x * 16;
+  word4 v[4];
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i)
+    if (o + i * 4096 < end) v[i] = *reinterpret_cast<const word4 *>(src + o + i * 4096);
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i)
+    if (o + i * 4096 < end) *reinterpret_cast<word4 *>(dst + o + i * 4096) = v[i];
+}
+
 // ============================================================= launchers ====
 namespace {
 
@@ -1174,6 +1217,57 @@ int kv_page_copy(kvx_storage *s, const kvx_page_copy *copies, uint32_t n, void *
     if (int rc = check_launch("page_copy_kernel")) return rc;
   }
   return KVX_OK;
+}
+
+
+static int page_wire(const kvx_storage *s, const uint32_t *pages, uint32_t n, void *buffer,
+                     bool to_wire, void *stream) {
+  if (!s || (n && (!pages || !buffer))) return fail(KVX_EINVAL, "page export / import: null argument");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
+  // All-or-nothing: validate every page before anything is enqueued.
+  for (uint32_t i = 0; i < n; ++i) {
+    if (pages[i] >= s->page_count) return fail(KVX_ERANGE, "invalid KV page id");
+    if (!s->extents[pages[i] / s->extent_pages])
+      return fail(KVX_ESTATE, "KV page of an extent that is not allocated");
+  }
+  if (!to_wire) {
+    std::vector<uint32_t> sorted(pages, pages + n);
+    std::sort(sorted.begin(), sorted.end());
+    if (std::adjacent_find(sorted.begin(), sorted.end()) != sorted.end())
+      return fail(KVX_EINVAL, "two imported pages share a destination");
+  }
+  const uint32_t span = std::max(s->data_bytes, s->scale_bytes);
+  const uint32_t chunks = (span + kCopyChunk - 1) / kCopyChunk;
+  const uint64_t page_bytes = kvx_storage_bytes_per_page(s);
+  for (uint32_t first = 0; first < n; first += kCopiesPerLaunch) {
+    WireArgs a{};
+    const uint32_t count = std::min(kCopiesPerLaunch, n - first);
+    a.buffer = static_cast<uint8_t *>(buffer) + uint64_t(first) * page_bytes;
+    a.extent_pages = s->extent_pages;
+    a.data_bytes = s->data_bytes;
+    a.scale_bytes = s->scale_bytes;
+    a.layers = s->layout.layers;
+    for (uint32_t i = 0; i < count; ++i) {
+      const uint32_t page = pages[first + i];
+      a.page[i] = reinterpret_cast<uint64_t>(s->extents[page / s->extent_pages]) | (page % s->extent_pages);
+    }
+    const dim3 grid(chunks, s->layout.layers * 4, count);
+    if (to_wire)
+      hipLaunchKernelGGL(page_wire_kernel<true>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a);
+    else
+      hipLaunchKernelGGL(page_wire_kernel<false>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a);
+    if (int rc = check_launch("page_wire_kernel")) return rc;
+  }
+  return KVX_OK;
+}
+
+int kv_page_export(const kvx_storage *s, const uint32_t *pages, uint32_t n, void *buffer,
+                   void *stream) {
+  return page_wire(s, pages, n, buffer, true, stream);
+}
+int kv_page_import(kvx_storage *s, const uint32_t *pages, uint32_t n, const void *buffer,
+                   void *stream) {
+  return page_wire(s, pages, n, const_cast<void *>(buffer), false, stream);
 }
 
 }  // extern "C"

@@ -35,7 +35,7 @@ SYMBOLS = [
     "kvx_pool_acquire", "kvx_pool_retain", "kvx_pool_release", "kvx_pool_page_active",
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
     "kvx_pool_snapshot_get", "kv_append", "kv_attend_verify", "kv_attend_decode",
-    "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kvx_debug_set_attend_phases",
+    "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kv_page_export", "kv_page_import", "kvx_debug_set_attend_phases",
     "kvx_debug_attend_paths", "kvx_decode_plan", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
     "kvx_prefix_chain", "kvx_prefix_retain_active", "kvx_prefix_release_active",
@@ -190,6 +190,8 @@ def _declare(L):
     L.kvx_storage_extent_read.argtypes = [vp, u32, u64, u64, vp]
     L.kvx_storage_extent_write.argtypes = [vp, u32, u64, u64, vp]
     L.kv_page_copy.argtypes = [vp, vp, u32, vp]
+    L.kv_page_export.argtypes = [vp, vp, u32, vp, vp]
+    L.kv_page_import.argtypes = [vp, vp, u32, vp, vp]
     L.kvx_pool_create.argtypes = [vp, u32, C.POINTER(vp)]
     L.kvx_pool_destroy.argtypes, L.kvx_pool_destroy.restype = [vp], None
     L.kvx_pool_acquire.argtypes = [vp, u32, vp]
@@ -312,6 +314,13 @@ class Storage:
         data = np.ascontiguousarray(data, dtype=np.uint8)
         return check(lib().kvx_storage_extent_write(self.h, extent, offset, data.size,
                                                     data.ctypes.data))
+
+    def export_pages(self, pages, buffer, stream=None):
+        """Wire bytes of `pages` into `buffer` (device or pinned host tensor)."""
+        return check(lib().kv_page_export(self.h, _u32(pages), len(pages), _ptr(buffer), _stream(stream)))
+
+    def import_pages(self, pages, buffer, stream=None):
+        return check(lib().kv_page_import(self.h, _u32(pages), len(pages), _ptr(buffer), _stream(stream)))
 
     def copy_pages(self, copies, stream=None):
         arr = (PageCopy * len(copies))(*[PageCopy(a, b) for a, b in copies])

@@ -293,3 +293,50 @@ def test_pool_compaction_moves_page_bytes_on_the_device():
         st.entries_host([0])  # the released extent's pages have no entries
     pool.close()
     st.close()
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("pinned", [False, True])
+def test_page_export_and_import_are_the_wire_bytes(fmt, pinned):
+    """kv_page_export writes exactly the bytes PageStorage::spans lists for each page
+    (the oracle's page_read, pinned by its own tests), into device memory or pinned host
+    memory; kv_import puts them back into other pages byte for byte; invalid lists
+    enqueue nothing."""
+    rng = np.random.default_rng(70 + fmt)
+    tokens, layers = 200 * 32, 3          # 200 pages: more than one launch of 128
+    n_pages = tokens // 32
+    tw = Gp.Twin(fmt, H, D, layers, 2 * n_pages + 4)
+    pages = tw.pages(2 * n_pages, 71)
+    source, target = pages[:n_pages], pages[n_pages:]
+    _, td = tw.tables(source)
+    for layer in range(layers):
+        for done in range(0, tokens, 1600):
+            k, v = random_rows(rng, 1600)
+            ck, cv = T.chunk_buffers(k, v, 1600)
+            kvx.append(tw.dev, layer, Gp.dev(ck), Gp.dev(cv), [td],
+                       [kvx.ChunkParams(done, 1600, 1600, n_pages)], H * 1600 * D)
+    torch.cuda.synchronize()
+    tw.download()
+    page_bytes = tw.dev.bytes_per_page
+    want = np.concatenate([tw.host.page_read(int(p)) for p in source])
+    buffer = torch.zeros(n_pages * page_bytes, dtype=torch.uint8, pin_memory=pinned,
+                         device="cpu" if pinned else "cuda")
+    tw.dev.export_pages(source, buffer)
+    torch.cuda.synchronize()
+    assert np.array_equal(buffer.cpu().numpy(), want)
+    before = [tw.dev.page_read(int(p)) for p in source[::37]]
+    tw.dev.import_pages(target, buffer)
+    torch.cuda.synchronize()
+    for a, b in list(zip(source, target))[::17]:
+        assert np.array_equal(tw.dev.page_read(int(b)), tw.host.page_read(int(a)))
+    assert all(np.array_equal(x, tw.dev.page_read(int(p))) for x, p in zip(before, source[::37]))
+    # an invalid page, an unallocated extent's page or a repeated destination: nothing enqueued
+    probe = tw.dev.page_read(int(target[0]))
+    for bad in ([int(target[0]), tw.dev.page_count], [int(target[0]), int(target[0])]):
+        with pytest.raises(kvx.KvxError):
+            tw.dev.import_pages(bad, buffer)
+    with pytest.raises(kvx.KvxError):
+        tw.dev.export_pages([tw.dev.page_count + 5], buffer)
+    torch.cuda.synchronize()
+    assert np.array_equal(probe, tw.dev.page_read(int(target[0])))
+    tw.close()
