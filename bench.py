@@ -56,6 +56,10 @@ def parse():
                     help="override the library's decode split rule (experiments)")
     ap.add_argument("--separate-append", action="store_true",
                     help="call kv_append and kv_attend_decode instead of kv_append_attend_decode")
+    ap.add_argument("--hidden", choices=["none", "gate", "gather"], default="none",
+                    help="decode: the merge also writes the out-projection's operand "
+                         "(kv_attend_verify_hidden), gated by packed projection rows or plainly "
+                         "gathered; implies --separate-append")
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
     ap.add_argument("--workload", choices=["decode", "tree-verify", "prefill"], default="decode",
@@ -468,6 +472,21 @@ def main():
     table_arr = (C.c_void_p * BATCH)(*[t.data_ptr() for t in tables])
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     lane_stride = H * 32 * D
+    hidden = packed = None
+    if args.hidden != "none":
+        args.separate_append = True
+        hidden = torch.zeros((BATCH, 1, QH, D), dtype=torch.bfloat16, device="cuda")
+        if args.hidden == "gate":
+            packed = torch.randn((BATCH, 1, (2 * QH + 2 * H) * D), generator=gen, device="cuda").bfloat16()
+
+    def attend(layer, vp_arr):
+        if hidden is None:
+            return L.kv_attend_decode(storage.h, layer, QH, queries.data_ptr(), output.data_ptr(),
+                                      table_arr, vp_arr, BATCH, 1, workspace.data_ptr(), ws_bytes, stream)
+        return L.kv_attend_verify_hidden(storage.h, layer, QH, queries.data_ptr(), output.data_ptr(),
+                                         table_arr, vp_arr, BATCH, None, 1, workspace.data_ptr(),
+                                         ws_bytes, packed.data_ptr() if packed is not None else None,
+                                         hidden.data_ptr(), stream)
 
     def step():
         ap, vp = lane_params()
@@ -487,8 +506,7 @@ def main():
                              ap_arr, BATCH, lane_stride, 15, stream)
             if rc:
                 kvx.check(rc)
-            rc = L.kv_attend_decode(storage.h, layer, QH, queries.data_ptr(), output.data_ptr(),
-                                    table_arr, vp_arr, BATCH, 1, workspace.data_ptr(), ws_bytes, stream)
+            rc = attend(layer, vp_arr)
             if rc:
                 kvx.check(rc)
         for i in range(BATCH):
@@ -530,14 +548,12 @@ def main():
     def time_attend(phases):
         L.kvx_debug_set_attend_phases(phases)
         for layer in range(2):
-            L.kv_attend_decode(storage.h, layer, QH, queries.data_ptr(), output.data_ptr(), table_arr,
-                               vp_arr, BATCH, 1, workspace.data_ptr(), ws_bytes, stream)
+            attend(layer, vp_arr)
         torch.cuda.synchronize()
         k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         k0.record()
         for it in range(args.kernel_iters):
-            L.kv_attend_decode(storage.h, it % LAYERS, QH, queries.data_ptr(), output.data_ptr(),
-                               table_arr, vp_arr, BATCH, 1, workspace.data_ptr(), ws_bytes, stream)
+            attend(it % LAYERS, vp_arr)
         k1.record()
         torch.cuda.synchronize()
         L.kvx_debug_set_attend_phases(3)
@@ -563,6 +579,8 @@ def main():
             "pool_gb": round(extents * extent_bytes / 1e9, 1), "extents": extents,
             "page_order": "contiguous" if args.contiguous else "seed-shuffled",
             "seed": args.seed,
+            **({"entries": "kv_append + kv_attend_verify_hidden", "hidden": args.hidden}
+               if args.hidden != "none" else {}),
         },
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "decode_tokens_per_s": round(BATCH * args.steps / wall, 1),

@@ -415,6 +415,30 @@ int kv_attend_verify(const kvx_storage *storage, uint32_t layer, uint32_t query_
                      const uint32_t *row_masks, uint32_t row_stride, void *workspace,
                      uint64_t workspace_bytes, void *stream);
 
+/* kv_attend_verify whose merge also hands the out-projection its operand, so that no
+   elementwise gate or gather dispatch has to read the attention rows back.  Replaces
+   ops::PagedAttention::addVerify with gateHidden bound (runtime/ops/PagedAttention.hpp:299-311,
+   PagedAttention.cpp:514-541; kernels verify_attention_reduce_gate* and
+   verify_tree_attention_reduce_gate*, decode/paged_attention.metal:266-330, 466-530, and
+   verify_attention_reduce_gather*, :356-413).
+   hidden: bf16 [lane][row_capacity][query head][D], query head = kv head x group + head in group.
+   packed_qkv: NULL, or the lanes' packed projection rows, bf16 [lane][row_capacity][stride] with
+   stride = (2 x query heads + 2 x KV heads) x D: per query head its D query values then its D gate
+   values, then keys and values.
+   packed_qkv given: hidden = bf16(value x sigmoid(gate)), value being the bf16 attention element
+   and sigmoid(x) = 1 / (1 + 2^(-x log2 e)) (common/activation.h:14-16), what
+   verify_attention_gate computes from the staged rows (decode/attention_qkv.metal:121-164).
+   packed_qkv NULL: hidden = value (verify_attention_gather).
+   output may be NULL; when given it receives the staged rows exactly as kv_attend_verify writes
+   them.  Rows >= active_rows of hidden are zeros.  The reference has no fused gather for tree
+   rows; this entry takes row_masks in both modes. */
+int kv_attend_verify_hidden(const kvx_storage *storage, uint32_t layer, uint32_t query_heads,
+                            const void *queries, void *output, const uint64_t *const *page_tables,
+                            const kvx_verify_params *lanes, uint32_t n_lanes,
+                            const uint32_t *row_masks, uint32_t row_stride, void *workspace,
+                            uint64_t workspace_bytes, const void *packed_qkv, void *hidden,
+                            void *stream);
+
 /* One-row decode attention per lane: kv_attend_verify with active_rows =
    row_capacity = 1 on the bandwidth-tuned kernels (the reference reaches decode
    through its prefill entries with rows = 1, prefill/paged_attention.metal:7-67,

@@ -433,13 +433,21 @@ public:
                             workspace, workspaceBytes, stream));
   }
   // Stores each lane's chunk and attends its rows with the plan's split counts.
+  // With gateHidden the merge also writes the out-projection's operand
+  // ([lane][row capacity][query head][D]): scaled by the sigmoid of the gates in
+  // gatePacked, the lanes' packed projection rows, or plainly gathered when
+  // gatePacked is null, which the reference has for chain plans only
+  // (ops::PagedAttention::addVerify, runtime/ops/PagedAttention.cpp:514-541).
   static void addVerify(void *stream, const kv::PageStorage &storage, uint32_t layer,
                         const PagedVerifyBuffers &buffers,
-                        const std::vector<kv::ChunkedPrefillParams> &chunks, const VerifyAttentionPlan &plan) {
+                        const std::vector<kv::ChunkedPrefillParams> &chunks, const VerifyAttentionPlan &plan,
+                        const void *gatePacked = nullptr, void *gateHidden = nullptr) {
     if (chunks.size() != plan.lanes) throw std::invalid_argument("one chunk per plan lane");
+    if (gateHidden && !gatePacked && buffers.treeMasks)
+      throw std::invalid_argument("tree verify has no fused gather");
     const kv::Layout &layout = storage.layout();
     const uint64_t laneStride = uint64_t{layout.kvHeads} * kv::kVerifyChunkStride * layout.headDimension;
-    if (plan.rowCapacity == 1) {  // a decode step: one call stores the token and attends
+    if (plan.rowCapacity == 1 && !gateHidden) {  // a decode step: one call stores the token and attends
       std::vector<kv::VerifyAttentionParams> lanes(plan.lanes);
       for (uint32_t i = 0; i < plan.lanes; ++i) {
         if (chunks[i].chunk_tokens != 1 || chunks[i].chunk_stride != kv::kVerifyChunkStride)
@@ -455,18 +463,25 @@ public:
     }
     check(kv_append(storage.handle(), layer, buffers.chunkKeys, buffers.chunkValues, buffers.pageTables,
                     chunks.data(), plan.lanes, laneStride, kv::kTreeVerifyNodes, stream));
-    attend(stream, storage, layer, buffers, chunks, plan);
+    attend(stream, storage, layer, buffers, chunks, plan, gatePacked, gateHidden);
   }
   // The attention half of addVerify alone (rows already stored); decode plans
   // take the bandwidth-tuned one-row kernels with rows packed (row stride 1).
   static void attend(void *stream, const kv::PageStorage &storage, uint32_t layer,
                      const PagedVerifyBuffers &buffers, const std::vector<kv::ChunkedPrefillParams> &chunks,
-                     const VerifyAttentionPlan &plan) {
+                     const VerifyAttentionPlan &plan, const void *gatePacked = nullptr,
+                     void *gateHidden = nullptr) {
     std::vector<kv::VerifyAttentionParams> lanes(plan.lanes);
     for (uint32_t i = 0; i < plan.lanes; ++i)
       lanes[i] = {chunks[i].committed_tokens, chunks[i].page_table_entries, {}, plan.laneSplits[i],
                   plan.splits, chunks[i].chunk_tokens, plan.rowCapacity, plan.scoreScale};
-    if (plan.rowCapacity == 1)
+    if (gateHidden)
+      check(kv_attend_verify_hidden(storage.handle(), layer, plan.queryHeads, buffers.queries,
+                                    buffers.output, buffers.pageTables, lanes.data(), plan.lanes,
+                                    buffers.treeMasks, plan.rowCapacity == 1 ? 1 : kv::kVerifyChunkStride,
+                                    buffers.workspace, buffers.workspaceBytes, gatePacked, gateHidden,
+                                    stream));
+    else if (plan.rowCapacity == 1)
       check(kv_attend_decode(storage.handle(), layer, plan.queryHeads, buffers.queries, buffers.output,
                              buffers.pageTables, lanes.data(), plan.lanes, 1, buffers.workspace,
                              buffers.workspaceBytes, stream));

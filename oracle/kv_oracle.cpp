@@ -776,6 +776,34 @@ int ko_attend_verify(uint32_t format, uint32_t kv_heads, uint32_t group, uint32_
   return attended;
 }
 
+float ko_sigmoid(float x) {
+  // common/activation.h:14-16
+  return 1.0f / (1.0f + exp2f(-1.44269504089f * x));
+}
+
+void ko_attention_hidden(uint32_t kv_heads, uint32_t group, uint32_t head_dim, uint32_t lanes,
+                         uint32_t rows, uint32_t row_stride, const uint16_t *attention,
+                         const uint16_t *packed_qkv, uint16_t *hidden) {
+  // decode/attention_qkv.metal:121-164 (full_attention_gate_value and its loop)
+  const uint32_t D = head_dim, q_heads = kv_heads * group;
+  const uint64_t q_stride = packed_qkv ? 2ull * D : D;
+  const uint64_t packed_stride = q_heads * q_stride + 2ull * kv_heads * D;
+  const uint64_t per_lane = uint64_t{rows} * q_heads * D;
+  for (uint64_t element = 0; element < per_lane * lanes; ++element) {
+    const uint64_t batch = element / per_lane, lane_element = element % per_lane;
+    const uint64_t row = lane_element / (uint64_t{q_heads} * D);
+    const uint64_t remainder = lane_element % (uint64_t{q_heads} * D);
+    const uint64_t query_head = remainder / D, dim = remainder % D;
+    float gate_scale = 1.0f;
+    if (packed_qkv)
+      gate_scale = ko_sigmoid(ko_bf16_to_float(
+          packed_qkv[(batch * rows + row) * packed_stride + query_head * q_stride + D + dim]));
+    const uint64_t kv_head = query_head / group, local_head = query_head % group;
+    const uint64_t at = (((batch * kv_heads + kv_head) * row_stride + row) * group + local_head) * D + dim;
+    hidden[element] = ko_float_to_bf16(ko_bf16_to_float(attention[at]) * gate_scale);
+  }
+}
+
 // ------------------------------------------------------------ compaction ---
 int ko_compact_tree(uint32_t format, uint32_t kv_heads, uint32_t head_dim,
                     const uint64_t *const *page_tables, const ko_chunk_params *params,

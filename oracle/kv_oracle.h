@@ -20,6 +20,10 @@
  *                          Metal runtime, which cannot run here
  *   tree verify/compact  : pinned by brute force only (the reference holds no
  *                          test of them) -- parity unpinned against reference
+ *   gate / gather        : pinned by mathematics (sigmoid identities and fp64
+ *                          values; the index map against an independent
+ *                          transpose/reshape statement); the reference's only
+ *                          check is a Metal fused-vs-unfused comparison
  *   pool                 : pinned (reference pool tests' exact page ids/moves)
  */
 #pragma once
@@ -221,6 +225,18 @@ int ko_attend_verify(uint32_t format, uint32_t kv_heads, uint32_t group, uint32_
                      const uint16_t *queries, uint16_t *output, float *out_f32,
                      const uint64_t *const *page_tables, const ko_verify_params *params,
                      uint32_t lanes, const uint32_t *row_masks);
+
+/* common/activation.h:14-16: 1 / (1 + 2^(-x log2 e)). */
+float ko_sigmoid(float x);
+/* The out-projection's operand from staged attention rows: verify_attention_gate /
+   verify_attention_gather (decode/attention_qkv.metal:121-164), which the fused reduces
+   (decode/paged_attention.metal:266-309, 356-393, 466-510) reproduce bit for bit.
+   attention is [lane][kv head][row_stride][g][D] bf16, hidden [lane][rows][query head][D];
+   packed_qkv (NULL = gather) is [lane][rows][(2 x query heads + 2 x kv heads) x D] with each
+   query head's gate D elements after its query.  One flat element at a time, as the kernel. */
+void ko_attention_hidden(uint32_t kv_heads, uint32_t group, uint32_t head_dim, uint32_t lanes,
+                         uint32_t rows, uint32_t row_stride, const uint16_t *attention,
+                         const uint16_t *packed_qkv, uint16_t *hidden);
 
 /* ---- tree path compaction: decode/paged_attention_store.metal:198-278 ---- */
 int ko_compact_tree(uint32_t format, uint32_t kv_heads, uint32_t head_dim,

@@ -205,6 +205,10 @@ def _declare(L):
     L.ko_attend_prefill.argtypes = [u32, u32, u32, u32, vp, vp, vp, vp, C.POINTER(PrefillParams)]
     L.ko_attend_verify.argtypes = [u32, u32, u32, u32, vp, vp, vp, vp, vp, u32, vp]
     L.ko_compact_tree.argtypes = [u32, u32, u32, vp, vp, vp, vp, u32, u32]
+    L.ko_sigmoid.argtypes = [C.c_float]
+    L.ko_sigmoid.restype = C.c_float
+    L.ko_attention_hidden.argtypes = [u32, u32, u32, u32, u32, u32, vp, vp, vp]
+    L.ko_attention_hidden.restype = None
     L.ko_pool_create.argtypes = [u32, u64, u32, u32, u32]
     L.ko_pool_create.restype = vp
     L.ko_pool_destroy.argtypes = [vp]
@@ -341,6 +345,15 @@ def attend_verify(fmt, kv_heads, group, head_dim, queries, tables, params, row_m
     n = lib().ko_attend_verify(fmt, kv_heads, group, head_dim, ptr(queries), ptr(out), ptr(f32),
                                _table_ptrs(tables), arr, len(params), ptr(row_masks))
     return n, out, f32
+
+
+def attention_hidden(kv_heads, group, head_dim, rows, attention, packed_qkv=None):
+    """hidden [lane][rows][query head][D] from staged rows [lane][kv head][stride][g][D]."""
+    lanes, _, row_stride = attention.shape[:3]
+    hidden = np.zeros((lanes, rows, kv_heads * group, head_dim), dtype=np.uint16)
+    lib().ko_attention_hidden(kv_heads, group, head_dim, lanes, rows, row_stride, ptr(attention),
+                              ptr(packed_qkv), ptr(hidden))
+    return hidden
 
 
 def compact_tree(fmt, kv_heads, head_dim, tables, params, retained_path, retained_count,

@@ -71,6 +71,13 @@ struct DecodeArgs {
   uint32_t tile_rows;
   uint32_t tile_last_rows;
   uint64_t tile_lane_stride;
+  // The merge's second output (see Epilogue): hidden rows of the launch's first
+  // lane onwards, and the packed rows their gates come from (null = no gate).
+  // With `hidden` every split writes partials, the only split of a short lane
+  // too, so that the merge produces every row.
+  uint16_t *hidden;
+  const uint16_t *packed_qkv;
+  uint32_t all_partials;
 };
 
 // The lane with this index of a launch: read from the arguments, or derived
@@ -205,18 +212,33 @@ __global__ __launch_bounds__(64 * kMergeWaves) void matrix_merge_kernel(
   const uint32_t pages = (l.committed + l.active_rows + kPage - 1) / kPage;
   const uint32_t per = (pages + l.split_count - 1) / l.split_count;
   const uint32_t written = (pages + per - 1) / per;
-  if (written <= 1) return;
+  if (written <= 1 && !a.all_partials) return;
   const uint32_t G = a.group, M = a.fused_rows;
   uint16_t *out_row =
-      output + l.q_offset + uint64_t(head) * a.row_stride * G * kD + uint64_t(j) * kD;
+      output ? output + l.q_offset + uint64_t(head) * a.row_stride * G * kD + uint64_t(j) * kD
+             : nullptr;
+  // The row's place in the out-projection's operand and in the packed rows:
+  // [lane][row][query head], the gate D elements after the head's query.
+  const uint64_t hidden_row = uint64_t(blockIdx.z) * (M / G) + j / G;
+  const uint32_t query_head = head * G + j % G;
+  uint16_t *hidden_out =
+      a.hidden ? a.hidden + (hidden_row * a.kv_heads * G + query_head) * kD + 4 * lane : nullptr;
   if (j / G >= l.active_rows) {  // rows past the live ones read as zeros
-    if (wave == 0) *reinterpret_cast<u32x2 *>(out_row + 4 * lane) = u32x2{0u, 0u};
+    if (wave == 0) {
+      if (out_row) *reinterpret_cast<u32x2 *>(out_row + 4 * lane) = u32x2{0u, 0u};
+      if (hidden_out) *reinterpret_cast<u32x2 *>(hidden_out) = u32x2{0u, 0u};
+    }
     return;
   }
+  u32x2 gates = {0u, 0u};
+  if (a.packed_qkv && wave == 0)
+    gates = load_global<u32x2>(a.packed_qkv +
+                               hidden_row * (2ull * a.kv_heads * G + 2ull * a.kv_heads) * kD +
+                               uint64_t(query_head) * 2 * kD + kD + 4 * lane);
   const uint64_t first_row = l.row_base + uint64_t(head) * l.split_count * M + j;
   const bool sequential = written <= kMergeSequential;
   if (sequential && wave) return;
-  // The sequential case (at most 64 splits) issues its statistics and the
+  // The sequential case (at most kMergeSequential splits) issues its statistics and the
   // first eight partial rows together, before anything waits.
   f32x4 early[8];
   f32x2 early_stat = {-INFINITY, 0.0f};
@@ -271,7 +293,20 @@ __global__ __launch_bounds__(64 * kMergeWaves) void matrix_merge_kernel(
         sums.denominator > 0.0f ? __fdiv_rn(sums.numerator[2 * i + 1], sums.denominator) : 0.0f;
     packed[i] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
   }
-  *reinterpret_cast<u32x2 *>(out_row + 4 * lane) = packed;
+  if (out_row) *reinterpret_cast<u32x2 *>(out_row + 4 * lane) = packed;
+  if (!hidden_out) return;
+  if (a.packed_qkv) {
+    // hidden = bf16(value x sigmoid(gate)) with the bf16 value just written
+    // (reference: decode/paged_attention.metal:302-308, common/activation.h:14-16).
+#pragma unroll
+    for (uint32_t i = 0; i < 2; ++i) {
+      const float lo = __fmul_rn(bf16_to_f32(uint16_t(packed[i])), sigmoid(bf16_to_f32(uint16_t(gates[i]))));
+      const float hi = __fmul_rn(bf16_to_f32(uint16_t(packed[i] >> 16)),
+                                 sigmoid(bf16_to_f32(uint16_t(gates[i] >> 16))));
+      packed[i] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
+    }
+  }
+  *reinterpret_cast<u32x2 *>(hidden_out) = packed;
 }
 
 // Launches a split kernel over (work items, KV heads, column blocks) and then
@@ -287,7 +322,8 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
                             uint32_t n_lanes, const uint32_t *row_masks, uint32_t row_stride,
                             uint64_t lane_stride, void *workspace, uint64_t workspace_bytes,
                             uint32_t phases, hipStream_t stream,
-                            const FusedAppend *fused = nullptr, uint32_t tile_rows = 0) {
+                            const FusedAppend *fused = nullptr, uint32_t tile_rows = 0,
+                            const Epilogue *epilogue = nullptr) {
   const kvx_layout &l = s->layout;
   const uint32_t H = l.kv_heads, G = query_heads / H;
   const uint32_t capacity = lanes[0].row_capacity, M = capacity * G;
@@ -340,6 +376,14 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       row_base += uint64_t(p.split_count) * H * M;
     }
     if (tile_rows) items = n_lanes * lanes[0].split_count;
+    if (epilogue) {
+      a.hidden = epilogue->hidden + uint64_t(first) * capacity * query_heads * kD;
+      a.packed_qkv = epilogue->packed_qkv
+                         ? epilogue->packed_qkv +
+                               uint64_t(first) * capacity * (2ull * query_heads + 2ull * H) * kD
+                         : nullptr;
+      a.all_partials = 1;
+    }
     if (phases & 1u) {
       hipLaunchKernelGGL(split_kernel, dim3(items, H, (M + columns - 1) / columns), dim3(threads), 0,
                          stream, static_cast<const uint16_t *>(queries),
@@ -347,7 +391,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       const hipError_t e = hipGetLastError();
       if (e != hipSuccess) return hip_fail(e, name);
     }
-    if (max_splits > 1 && (phases & 2u)) {
+    if ((max_splits > 1 || epilogue) && (phases & 2u)) {
       // One wave per row is all the sequential merge uses; the other three only
       // join in for lists longer than kMergeSequential.
       const uint32_t merge_threads = max_splits <= kMergeSequential ? 64 : 64 * kMergeWaves;

@@ -440,7 +440,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
     sum += __shfl_xor(sum, 16);
     sum += __shfl_xor(sum, 32);
     uint16_t *out_head = output + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
-    if (written == 1) {
+    if (written == 1 && !a.all_partials) {
       // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
       // Rows of the tile past the live ones read as zeros.
       if (in_tile[nb]) {
@@ -490,7 +490,7 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                            const kvx_verify_params *lanes, uint32_t n_lanes,
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
-                           hipStream_t stream, uint32_t tile_rows) {
+                           hipStream_t stream, uint32_t tile_rows, const Epilogue *epilogue) {
   const uint32_t format = s->layout.format;
   if ((format != KVX_FMT_BF16 && format != KVX_FMT_FP8E4M3 && format != KVX_FMT_INT8) ||
       !matrix_attention_covers(s, query_heads, lanes, n_lanes))
@@ -501,7 +501,7 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   launch_matrix_attention(attend_wide_kernel<FMT, NB, WAVES>, "attend_wide_kernel", 16 * NB, 64, s, \
                           kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks, \
                           row_stride, lane_stride, workspace, workspace_bytes, phases, stream,      \
-                          nullptr, tile_rows)
+                          nullptr, tile_rows, epilogue)
   // Two blocks of 16 fused rows per wave share every key and value operand; a
   // third would not fit the register file next to a page of bf16 keys and values.
   // One-byte formats run two waves per SIMD with one block (decode, the 8-row

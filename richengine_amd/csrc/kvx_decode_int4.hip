@@ -614,7 +614,8 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     }
   }
 #endif
-  write_blocks<NB>(st, m, in_tile, live_row, l, a, head, split, written, g, output, partials, statistics);
+  write_blocks<NB>(st, m, in_tile, live_row, l, a, head, split, a.all_partials ? 2u : written, g, output,
+                   partials, statistics);
 }
 
 // One block of 16 fused rows per wave, two waves per SIMD: one-row decode, where
@@ -667,7 +668,8 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
                            hipStream_t stream, const void *append_keys, const void *append_values,
-                           uint64_t append_lane_stride, uint32_t append_stride, uint32_t tile_rows) {
+                           uint64_t append_lane_stride, uint32_t append_stride, uint32_t tile_rows,
+                           const Epilogue *epilogue) {
   if (s->layout.format != KVX_FMT_INT4 || !matrix_attention_covers(s, query_heads, lanes, n_lanes))
     return 1;
   const FusedAppend appended{append_keys, append_values, append_lane_stride, append_stride};
@@ -684,16 +686,16 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
     return launch_matrix_attention(prefill_int4_kernel, "prefill_int4_kernel", 32, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                   kvx_attend_phases(), stream, nullptr, tile_rows);
+                                   kvx_attend_phases(), stream, nullptr, tile_rows, epilogue);
   if (fused_rows > 16 && !many_tiles)
     return launch_matrix_attention(verify_int4_kernel, "verify_int4_kernel", 32, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                   kvx_attend_phases(), stream, nullptr, tile_rows);
+                                   kvx_attend_phases(), stream, nullptr, tile_rows, epilogue);
   return launch_matrix_attention(decode_int4_kernel, "decode_int4_kernel", 16, 64, s, kv,
                                  query_heads, queries, output, page_tables, lanes, n_lanes,
                                  row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                 kvx_attend_phases(), stream, fused, tile_rows);
+                                 kvx_attend_phases(), stream, fused, tile_rows, epilogue);
 }
 
 #ifdef KVX_PROBE_CLOCK

@@ -26,6 +26,11 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
   return uint16_t((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
 }
 __device__ __forceinline__ float round_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+// The logistic sigmoid as the reference's kernels take it, 1 / (1 + 2^(-x log2 e))
+// (reference: common/activation.h:14-16).
+__device__ __forceinline__ float sigmoid(float x) {
+  return __fdiv_rn(1.0f, __fadd_rn(1.0f, exp2f(__fmul_rn(-1.44269504089f, x))));
+}
 __device__ __forceinline__ float round_f16(float f) { return float(_Float16(f)); }
 
 // OCP e4m3 (bias 7, no infinities, 0x7f NaN): round to nearest even, saturate

@@ -73,6 +73,19 @@ __device__ inline Slab slab_of(uint32_t format, uint32_t kv_heads, uint32_t head
   return s;
 }
 
+// ---- attention epilogue -----------------------------------------------------
+// What an attend call writes beside (or instead of) its staging rows: `hidden`,
+// the out-projection's operand, bf16 [lane][row capacity][query head][D]
+// (reference: the reduce/gather fusion, decode/paged_attention.metal:356-393).
+// With `packed_qkv`, the lanes' packed projection rows, bf16 [lane][row capacity]
+// [(query | gate) x query heads, (key | value) x KV heads][D], each element is
+// first scaled by the sigmoid of its gate (the reduce/gate fusion,
+// decode/paged_attention.metal:266-309, 466-510).
+struct Epilogue {
+  const uint16_t *packed_qkv;
+  uint16_t *hidden;
+};
+
 // ---- storage ----------------------------------------------------------------
 struct Storage {
   kvx_layout layout;

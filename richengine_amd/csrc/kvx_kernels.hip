@@ -244,6 +244,9 @@ struct AttendArgs {
   uint32_t row_capacity;
   uint32_t row_stride;  // rows between KV heads in queries / output
   kvx_kv_layer kv;
+  // The merge's second output (see Epilogue), from the launch's first lane on.
+  uint16_t *hidden;
+  const uint16_t *packed_qkv;
 };
 struct PrefillArgs {
   const uint64_t *table;
@@ -463,16 +466,14 @@ __global__ __launch_bounds__(kTileThreads) void prefill_split_kernel(
 }
 
 // Fixed-order merge of one fused row's splits (reference:
-// common/paged_attention_tile.h:362-417).  head_dim threads, one per dimension.
-__device__ void reduce_row(const float *__restrict__ partials, const float *__restrict__ statistics,
-                           uint16_t *__restrict__ out_row, uint32_t G, uint32_t D, uint32_t M,
-                           uint32_t committed, uint32_t active_rows, uint32_t splits,
-                           uint64_t head_row, uint32_t fused_row) {
+// common/paged_attention_tile.h:362-417).  head_dim threads, one per dimension;
+// returns the thread's bf16 element, zero for rows past the live ones.
+__device__ uint16_t reduce_row(const float *__restrict__ partials,
+                               const float *__restrict__ statistics, uint32_t G, uint32_t D,
+                               uint32_t M, uint32_t committed, uint32_t active_rows,
+                               uint32_t splits, uint64_t head_row, uint32_t fused_row) {
   const uint32_t d = threadIdx.x;
-  if (fused_row / G >= active_rows) {
-    out_row[d] = 0;
-    return;
-  }
+  if (fused_row / G >= active_rows) return 0;
   const uint32_t pages = (committed + active_rows + kPage - 1) / kPage;
   const uint32_t per = (pages + splits - 1) / splits;
   const uint32_t written = (pages + per - 1) / per;
@@ -486,7 +487,7 @@ __device__ void reduce_row(const float *__restrict__ partials, const float *__re
     numerator = __fadd_rn(numerator, __fmul_rn(weight, partials[row * D + d]));
     denominator = __fadd_rn(denominator, __fmul_rn(weight, statistics[row * 2 + 1]));
   }
-  out_row[d] = f32_to_bf16(denominator > 0.0f ? __fdiv_rn(numerator, denominator) : 0.0f);
+  return f32_to_bf16(denominator > 0.0f ? __fdiv_rn(numerator, denominator) : 0.0f);
 }
 
 __global__ __launch_bounds__(256) void attend_reduce_kernel(const float *__restrict__ partials,
@@ -496,11 +497,27 @@ __global__ __launch_bounds__(256) void attend_reduce_kernel(const float *__restr
   const uint32_t fused_row = blockIdx.x, head = blockIdx.y, li = blockIdx.z;
   const AttendLane &l = a.lane[li];
   if (!attend_contract(l, a)) return;
-  const uint32_t M = a.row_capacity * a.group, D = a.head_dim;
-  uint16_t *out = output + l.q_offset + uint64_t(head) * a.row_stride * a.group * D +
-                  uint64_t(fused_row) * D;
-  reduce_row(partials, statistics, out, a.group, D, M, l.committed, l.active_rows, l.split_count,
-             l.row_base + uint64_t(head) * l.split_count * M, fused_row);
+  const uint32_t M = a.row_capacity * a.group, D = a.head_dim, d = threadIdx.x;
+  const uint16_t value =
+      reduce_row(partials, statistics, a.group, D, M, l.committed, l.active_rows, l.split_count,
+                 l.row_base + uint64_t(head) * l.split_count * M, fused_row);
+  if (output)
+    output[l.q_offset + uint64_t(head) * a.row_stride * a.group * D + uint64_t(fused_row) * D + d] =
+        value;
+  if (!a.hidden) return;
+  // The out-projection's operand, [lane][row][query head][D], scaled by the
+  // sigmoid of the element's gate where packed rows are given (reference:
+  // decode/paged_attention.metal:302-308, 389-393).
+  const uint64_t hidden_row = uint64_t(li) * a.row_capacity + fused_row / a.group;
+  const uint32_t query_heads = a.kv_heads * a.group;
+  const uint32_t query_head = head * a.group + fused_row % a.group;
+  uint16_t hidden = value;
+  if (a.packed_qkv) {
+    const uint16_t gate = a.packed_qkv[hidden_row * (2ull * query_heads + 2ull * a.kv_heads) * D +
+                                       uint64_t(query_head) * 2 * D + D + d];
+    hidden = f32_to_bf16(__fmul_rn(bf16_to_f32(value), sigmoid(bf16_to_f32(gate))));
+  }
+  a.hidden[(hidden_row * query_heads + query_head) * D + d] = hidden;
 }
 
 __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float *__restrict__ partials,
@@ -513,9 +530,9 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float *__rest
   const uint32_t active = min(KVX_PREFILL_TILE_ROWS, p.rows - tile_start);
   const uint32_t M = KVX_PREFILL_TILE_ROWS * p.group, D = p.head_dim;
   const uint64_t tile_offset = (uint64_t(head) * p.stride + tile_start) * p.group * D;
-  reduce_row(partials, statistics, output + tile_offset + uint64_t(fused_row) * D, p.group, D, M,
-             p.committed + tile_start, active, p.splits,
-             (uint64_t(tile) * p.kv_heads + head) * p.splits * M, fused_row);
+  output[tile_offset + uint64_t(fused_row) * D + threadIdx.x] =
+      reduce_row(partials, statistics, p.group, D, M, p.committed + tile_start, active, p.splits,
+                 (uint64_t(tile) * p.kv_heads + head) * p.splits * M, fused_row);
 }
 
 // =========================================================== compaction ====
@@ -734,14 +751,16 @@ int kvx_attend_int4_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
                            hipStream_t stream, const void *append_keys = nullptr,
                            const void *append_values = nullptr, uint64_t append_lane_stride = 0,
-                           uint32_t append_stride = 0, uint32_t tile_rows = 0);
+                           uint32_t append_stride = 0, uint32_t tile_rows = 0,
+                           const Epilogue *epilogue = nullptr);
 
 int kvx_attend_wide_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t query_heads,
                            const void *queries, void *output, const uint64_t *const *page_tables,
                            const kvx_verify_params *lanes, uint32_t n_lanes,
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
-                           hipStream_t stream, uint32_t tile_rows = 0);
+                           hipStream_t stream, uint32_t tile_rows = 0,
+                           const Epilogue *epilogue = nullptr);
 
 // int4 pages go to their own kernels, bf16, fp8 and int8 pages to the wide-element
 // ones; 1 = neither covers the shape.
@@ -750,18 +769,19 @@ static int attend_matrix(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_h
                          const kvx_verify_params *lanes, uint32_t n_lanes,
                          const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                          void *workspace, uint64_t workspace_bytes, int many_tiles,
-                         hipStream_t stream, uint32_t tile_rows = 0) {
+                         hipStream_t stream, uint32_t tile_rows = 0,
+                         const Epilogue *epilogue = nullptr) {
   // tile_rows > 0: the lanes are regular (lane i = lane 0 moved on by i x tile_rows
   // rows and tokens over one table, all full but perhaps the last), which lets
   // any number of them share a launch.
   const int fast = kvx_attend_int4_launch(s, kv, query_heads, queries, output, page_tables, lanes,
                                           n_lanes, row_masks, row_stride, lane_stride, workspace,
                                           workspace_bytes, many_tiles, stream, nullptr, nullptr, 0, 0,
-                                          tile_rows);
+                                          tile_rows, epilogue);
   if (fast <= 0) return fast;
   return kvx_attend_wide_launch(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes,
                                 row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                many_tiles, stream, tile_rows);
+                                many_tiles, stream, tile_rows, epilogue);
 }
 
 uint32_t kvx_attend_phases() { return kvx::g_attend_phases; }
@@ -887,7 +907,8 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
                           const void *queries, void *output, const uint64_t *const *page_tables,
                           const kvx_verify_params *lanes, uint32_t n_lanes,
                           const uint32_t *row_masks, uint32_t row_stride, void *workspace,
-                          hipStream_t stream, uint32_t phases) {
+                          hipStream_t stream, uint32_t phases,
+                          const Epilogue *epilogue = nullptr) {
   const kvx_layout &l = s->layout;
   const uint32_t H = l.kv_heads, G = query_heads / H, D = l.head_dim;
   const uint32_t capacity = lanes[0].row_capacity, M = capacity * G;
@@ -907,6 +928,13 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
     a.row_capacity = capacity;
     a.row_stride = row_stride;
     a.kv = kv;
+    if (epilogue) {
+      a.hidden = epilogue->hidden + uint64_t(first) * capacity * query_heads * D;
+      a.packed_qkv = epilogue->packed_qkv
+                         ? epilogue->packed_qkv +
+                               uint64_t(first) * capacity * (2ull * query_heads + 2ull * H) * D
+                         : nullptr;
+    }
     uint32_t max_splits = 0;
     for (uint32_t i = 0; i < a.n_lanes; ++i) {
       const kvx_verify_params &p = lanes[first + i];
@@ -944,12 +972,14 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
   return KVX_OK;
 }
 
-int kv_attend_verify(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
-                     const void *queries, void *output, const uint64_t *const *page_tables,
-                     const kvx_verify_params *lanes, uint32_t n_lanes, const uint32_t *row_masks,
-                     uint32_t row_stride, void *workspace, uint64_t workspace_bytes, void *stream) {
-  if (!s || !queries || !output || !page_tables || !lanes || !n_lanes || !workspace)
-    return fail(KVX_EINVAL, "kv_attend_verify: null argument or no lanes");
+static int attend_verify(const char *entry, const kvx_storage *s, uint32_t layer,
+                         uint32_t query_heads, const void *queries, void *output,
+                         const uint64_t *const *page_tables, const kvx_verify_params *lanes,
+                         uint32_t n_lanes, const uint32_t *row_masks, uint32_t row_stride,
+                         void *workspace, uint64_t workspace_bytes, const Epilogue *epilogue,
+                         void *stream) {
+  if (!s || !queries || (!output && !epilogue) || !page_tables || !lanes || !n_lanes || !workspace)
+    return fail(KVX_EINVAL, std::string(entry) + ": null argument or no lanes");
   if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
   if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
   kvx_kv_layer kv;
@@ -963,10 +993,34 @@ int kv_attend_verify(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
   const int fast = took(attend_matrix(
       s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks, row_stride,
       uint64_t(s->layout.kv_heads) * row_stride * group * s->layout.head_dim, workspace,
-      workspace_bytes, 0, static_cast<hipStream_t>(stream)));
+      workspace_bytes, 0, static_cast<hipStream_t>(stream), 0, epilogue));
   if (fast <= 0) return fast;
   return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks,
-                        row_stride, workspace, static_cast<hipStream_t>(stream), 3);
+                        row_stride, workspace, static_cast<hipStream_t>(stream), 3, epilogue);
+}
+
+int kv_attend_verify(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
+                     const void *queries, void *output, const uint64_t *const *page_tables,
+                     const kvx_verify_params *lanes, uint32_t n_lanes, const uint32_t *row_masks,
+                     uint32_t row_stride, void *workspace, uint64_t workspace_bytes, void *stream) {
+  return attend_verify("kv_attend_verify", s, layer, query_heads, queries, output, page_tables,
+                       lanes, n_lanes, row_masks, row_stride, workspace, workspace_bytes, nullptr,
+                       stream);
+}
+
+int kv_attend_verify_hidden(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
+                            const void *queries, void *output, const uint64_t *const *page_tables,
+                            const kvx_verify_params *lanes, uint32_t n_lanes,
+                            const uint32_t *row_masks, uint32_t row_stride, void *workspace,
+                            uint64_t workspace_bytes, const void *packed_qkv, void *hidden,
+                            void *stream) {
+  if (!hidden) return fail(KVX_EINVAL, "kv_attend_verify_hidden: null hidden rows");
+  if (hidden == queries || hidden == output || hidden == packed_qkv)
+    return fail(KVX_EINVAL, "hidden rows must not alias another argument");
+  const Epilogue epilogue{static_cast<const uint16_t *>(packed_qkv), static_cast<uint16_t *>(hidden)};
+  return attend_verify("kv_attend_verify_hidden", s, layer, query_heads, queries, output,
+                       page_tables, lanes, n_lanes, row_masks, row_stride, workspace,
+                       workspace_bytes, &epilogue, stream);
 }
 
 int kv_attend_decode(const kvx_storage *s, uint32_t layer, uint32_t query_heads,

@@ -34,7 +34,7 @@ SYMBOLS = [
     "kvx_storage_extent_write", "kv_page_copy", "kvx_pool_create", "kvx_pool_destroy",
     "kvx_pool_acquire", "kvx_pool_retain", "kvx_pool_release", "kvx_pool_page_active",
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
-    "kvx_pool_snapshot_get", "kv_append", "kv_attend_verify", "kv_attend_decode",
+    "kvx_pool_snapshot_get", "kv_append", "kv_attend_verify", "kv_attend_verify_hidden", "kv_attend_decode",
     "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kv_page_export", "kv_page_import", "kvx_debug_set_attend_phases",
     "kvx_debug_attend_paths", "kvx_decode_plan", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
@@ -204,6 +204,8 @@ def _declare(L):
     L.kvx_pool_snapshot_get.argtypes = [vp, C.POINTER(PoolSnapshot)]
     L.kv_append.argtypes = [vp, u32, vp, vp, vp, vp, u32, u64, u32, vp]
     L.kv_attend_verify.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, vp, u32, vp, u64, vp]
+    L.kv_attend_verify_hidden.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, vp, u32, vp, u64, vp, vp,
+                                          vp]
     L.kv_attend_decode.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, u32, vp, u64, vp]
     L.kv_append_attend_decode.argtypes = [vp, u32, vp, vp, u64, u32, u32, vp, vp, vp, vp, u32, u32, vp,
                                           u64, vp]
@@ -348,6 +350,19 @@ def attend_verify(storage, layer, query_heads, queries, output, tables, lanes, r
                                         row_stride, _ptr(workspace),
                                         workspace.numel() * workspace.element_size(),
                                         _stream(stream)))
+
+
+def attend_verify_hidden(storage, layer, query_heads, queries, output, tables, lanes, row_masks,
+                         row_stride, workspace, packed_qkv, hidden, stream=None):
+    """attend_verify whose merge also writes the out-projection's operand `hidden`
+    ([lane][row capacity][query head][D]), gated by `packed_qkv` when that is given; `output`
+    may be None."""
+    arr = (VerifyParams * len(lanes))(*lanes)
+    return check(lib().kv_attend_verify_hidden(
+        storage.h, layer, query_heads, _ptr(queries), _ptr(output), _table_array(tables), arr,
+        len(lanes), _ptr(row_masks), row_stride, _ptr(workspace),
+        workspace.numel() * workspace.element_size(), _ptr(packed_qkv), _ptr(hidden),
+        _stream(stream)))
 
 
 def attend_decode(storage, layer, query_heads, queries, output, tables, lanes, row_stride,

@@ -328,6 +328,31 @@ void testAppendDecodeSingleToken() {
     bool moved = false;  // and the second token did change the result
     for (size_t i = 0; i < one.size(); ++i) moved = moved || f32(one[i]) != 0.5f * (i / (G * D) + 1) * (float(i % D % 15) - 7.0f);
     EXPECT(moved);
+    // The merge's second output.  One-row lanes with packed rows: the gathered
+    // operand [lane][row][query head][D] has the staged rows' order, and a zero
+    // gate halves every element exactly.
+    void *hiddenDevice = nullptr, *packedDevice = nullptr;
+    hip(hipMalloc(&hiddenDevice, two.size() * 2));
+    hip(hipMalloc(&packedDevice, size_t{2 * QH + 2 * H} * D * 2));
+    hip(hipMemset(packedDevice, 0, size_t{2 * QH + 2 * H} * D * 2));
+    std::vector<uint16_t> hidden(two.size());
+    ops::PagedAttention::attend(nullptr, storage, 1, buffers, {chunk}, plan, nullptr, hiddenDevice);
+    hip(hipDeviceSynchronize());
+    hip(hipMemcpy(hidden.data(), hiddenDevice, hidden.size() * 2, hipMemcpyDeviceToHost));
+    EXPECT(hidden == two);
+    ops::PagedAttention::attend(nullptr, storage, 1, buffers, {chunk}, plan, packedDevice, hiddenDevice);
+    hip(hipDeviceSynchronize());
+    hip(hipMemcpy(hidden.data(), hiddenDevice, hidden.size() * 2, hipMemcpyDeviceToHost));
+    uint32_t unhalved = 0;
+    for (size_t i = 0; i < hidden.size(); ++i) unhalved += f32(hidden[i]) != 0.5f * f32(two[i]);
+    EXPECT(unhalved == 0);
+    buffers.treeMasks = static_cast<const uint32_t *>(packedDevice);  // any non-null masks: a tree plan
+    EXPECT(throws<std::invalid_argument>([&] {
+      ops::PagedAttention::addVerify(nullptr, storage, 1, buffers, {chunk}, plan, nullptr, hiddenDevice);
+    }));
+    buffers.treeMasks = nullptr;
+    hip(hipFree(hiddenDevice));
+    hip(hipFree(packedDevice));
     hip(hipFree(workspace));
   }
   // an invalid chunk is refused before anything is enqueued
