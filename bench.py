@@ -62,7 +62,7 @@ def parse():
                          "gathered; implies --separate-append")
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
-    ap.add_argument("--workload", choices=["decode", "tree-verify", "prefill"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "tree-verify", "prefill", "qkv-prepare"], default="decode",
                     help="decode = batch-32 mixed-length int4 decode, the headline metric (default); "
                          "tree-verify = 16-node tree verify and prefill = chunked prefill with a shared "
                          "prefix, the matrix-core paths (profiling)")
@@ -279,6 +279,88 @@ def tree_verify(args):
     print(json.dumps(result))
 
 
+def qkv_prepare(args):
+    """QKV prepare fused with quantize-on-append (kv_prepare_append), int4 pages, the
+    reference's 24 query heads with gates, bf16 norms, 32 rotary pairs: a 2048-token prefill
+    chunk per launch (the roofline line: packed rows and rotation tables read, queries and
+    pages written), and the one-row step of a batch of 32.  kv_append of ready bf16 chunk
+    rows, which the fused kernel replaces together with the prepare kernel in front of it, is
+    timed beside both."""
+    import numpy as np
+    import torch
+    from richengine_amd import kvx
+
+    L = kvx.lib()
+    torch.cuda.set_device(0)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(args.seed)
+    rng = np.random.default_rng(args.seed)
+    layout = kvx.Layout(LAYERS, H, D, kvx.INT4, 0.0)
+    extent_pages = L.kvx_layout_largest_extent_pages(C.byref(layout))
+    storage = kvx.Storage(LAYERS, H, D, kvx.INT4, extent_pages, extent_pages, aligned=True)
+    storage.allocate_all()
+    ids = rng.permutation(extent_pages).astype(np.uint32)
+    pairs, width = 32, (2 * QH + 2 * H) * D
+    shape = kvx.QkvShape(QH, pairs, 1, 1, 0.0)
+    wq = torch.randn(D, generator=gen, device="cuda").bfloat16()
+    wk = torch.randn(D, generator=gen, device="cuda").bfloat16()
+
+    def timed(call):
+        call(0)
+        torch.cuda.synchronize()
+        k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        k0.record()
+        for it in range(args.kernel_iters):
+            call(it % LAYERS)
+        k1.record()
+        torch.cuda.synchronize()
+        return k0.elapsed_time(k1) / args.kernel_iters
+
+    def case(lanes, committed, tokens):
+        rows = tokens
+        stride = (tokens + 31) // 32 * 32
+        n_pages = (committed + tokens + 31) // 32
+        tables = [storage.table(ids[i * n_pages:(i + 1) * n_pages]) for i in range(lanes)]
+        packed = torch.randn((lanes, rows, width), generator=gen, device="cuda").bfloat16()
+        cos = torch.rand((lanes, rows, pairs), generator=gen, device="cuda")
+        sin = torch.rand((lanes, rows, pairs), generator=gen, device="cuda")
+        queries = torch.zeros((lanes, H, stride, G, D), dtype=torch.bfloat16, device="cuda")
+        chunk_k = torch.randn((lanes, H, stride, D), generator=gen, device="cuda").bfloat16()
+        chunk_v = torch.randn((lanes, H, D, stride), generator=gen, device="cuda").bfloat16()
+        cp = [kvx.ChunkParams(committed, tokens, stride, n_pages) for _ in range(lanes)]
+        fused = timed(lambda layer: kvx.prepare_append(storage, layer, shape, packed, wq, wk, cos, sin,
+                                                       queries, stride, tables, cp, rows))
+        store = timed(lambda layer: kvx.append(storage, layer, chunk_k, chunk_v, tables, cp,
+                                               H * stride * D))
+        moved = lanes * tokens * (width * 2 + 2 * pairs * 4 + QH * D * 2 + BYTES_PER_TOKEN_LAYER)
+        return fused, store, moved
+
+    chunk_ms, chunk_store_ms, chunk_bytes = case(1, 16384, 2048)
+    step_ms, step_store_ms, _ = case(BATCH, 4096, 1)
+    achieved = chunk_bytes / (chunk_ms * 1e-3) / 1e9
+    result = {
+        "metric": "qkv prepare + int4 quantize-on-append, 2048-token chunk: tokens/s per layer launch",
+        "value": round(2048 / (chunk_ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.kernel_iters, "warmup": 1, "ms_per_step": round(chunk_ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 rows, fp32 norm and rotation, int4 pages", "data": "synthetic",
+        "config": {"workload": "kv_prepare_append: 24 query heads with gates, 4 KV heads x 256, bf16 "
+                               "norms, 32 rotary pairs; one 2048-token chunk after 16384 committed "
+                               "tokens per launch",
+                   "seed": args.seed},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "prepare_append_wave_kernel<int4, 4> (one wave per row and head)", "bytes_per_launch": chunk_bytes,
+                     "ms_per_launch": round(chunk_ms, 4)},
+        "kv_append_alone_ms": round(chunk_store_ms, 4),
+        "decode_batch32_one_row": {"prepare_append_ms": round(step_ms, 4),
+                                   "kv_append_alone_ms": round(step_store_ms, 4)},
+        "cpu_baseline": None,
+    }
+    storage.close()
+    print(json.dumps(result))
+
+
 def chunked_prefill(args):
     """Chunked prefill with prefix reuse: batch 4, a 2048-token chunk per sequence appended onto a
     shared 16384-token prefix (the prefix pages are the same physical pages in every
@@ -394,6 +476,8 @@ def main():
         if not os.path.exists(kvx.LIB_PATH):
             from richengine_amd import build as kvx_build
             kvx_build.build(verbose=False)
+        if args.workload == "qkv-prepare":
+            return qkv_prepare(args)
         return tree_verify(args) if args.workload == "tree-verify" else chunked_prefill(args)
     import numpy as np
     import torch

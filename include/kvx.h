@@ -397,6 +397,41 @@ int kv_append(const kvx_storage *storage, uint32_t layer, const void *chunk_keys
               const kvx_chunk_params *lanes, uint32_t n_lanes, uint64_t lane_stride,
               uint32_t verify_max_rows, void *stream);
 
+/* QKV prepare fused with quantize-on-append: what prefill_attention_qkv* / verify_attention_qkv*
+   followed by the store kernels do (ops::PagedAttention::addPrefillQkv / addVerifyQkv,
+   runtime/ops/PagedAttention.cpp:299-320, 351-371; kernels prefill/attention_qkv.metal:6-33,
+   decode/attention_qkv.metal:6-118, common/attention_qkv_prepare.h:12-83, common/rms_inverse.h:14-31;
+   then the stores kv_append replaces), without the bf16 chunk between them: the reference's own
+   open item (TODO.md, item 10).
+   Per live row and head: RMS norm over the head dimension with the head-type's weights, rotation
+   of the first rotary_pairs dimension pairs (d, d + rotary_pairs) by the row's cos / sin, bf16
+   rounding after the norm and after the rotation; queries go to `queries` in the attention
+   layout, keys are quantized from the rotated bf16 row and values from the packed row as
+   kv_append quantizes them, into the slots of tokens committed_tokens + row.
+   packed_qkv: bf16 [lane][rows][query heads x (query_gate ? 2 : 1) x D | KV heads x D keys |
+   KV heads x D values] (with query_gate each query head is its D query values, then D gate
+   values, which kv_attend_verify_hidden reads later).
+   q_norm / k_norm: [D] weights, bf16 (norm_type 1) or float (2); norm_type 0 runs no norm.
+   rope_cos / rope_sin: float [lane][rows][rotary_pairs].
+   queries: bf16 [lane][kv head][row_stride][group][D]; rows >= a lane's chunk_tokens are not
+   written.  lanes[i]: committed_tokens, chunk_tokens (live rows <= rows), page_table_entries;
+   chunk_stride must be a valid chunk stride (32 does) and is otherwise unused.
+   verify_max_rows > 0 bounds chunk_tokens as in kv_append.  Every buffer is 16-byte aligned.
+   Results depend on the inputs alone (fixed summation order, no fused multiply-add). */
+typedef struct kvx_qkv_shape {
+  uint32_t query_heads;
+  uint32_t rotary_pairs; /* 32 for the 256-wide heads of the reference, D / 2 for full rotary */
+  uint32_t query_gate;   /* 1: packed query heads are [query | gate] pairs */
+  uint32_t norm_type;    /* 0 none, 1 bf16 weights, 2 float weights */
+  float eps;             /* 0 selects 1e-6 (kRmsEpsilon) */
+} kvx_qkv_shape;
+int kv_prepare_append(const kvx_storage *storage, uint32_t layer, const kvx_qkv_shape *shape,
+                      const void *packed_qkv, const void *q_norm, const void *k_norm,
+                      const float *rope_cos, const float *rope_sin, void *queries,
+                      uint32_t row_stride, const uint64_t *const *page_tables,
+                      const kvx_chunk_params *lanes, uint32_t n_lanes, uint32_t rows,
+                      uint32_t verify_max_rows, void *stream);
+
 /* Paged attention of `active_rows` query rows per lane over committed history
    plus those rows (chain: causal; tree: row_masks).  Replaces the split and
    reduce dispatches of ops::PagedAttention::addVerify (PagedAttention.cpp:506-544;

@@ -424,6 +424,35 @@ public:
     const uint64_t *tables[1] = {pageTable};
     check(kv_append(storage.handle(), layer, chunkKeys, chunkValues, tables, &params, 1, 0, 0, stream));
   }
+  // addPrefillQkv / addVerifyQkv followed by the store (runtime/ops/PagedAttention.cpp:299-320,
+  // 351-371, then 424-440 / 467-500) as one dispatch: norms, rotation and layout of the packed
+  // projection rows, queries out, keys and values quantized straight into their page slots.
+  // `rows` rows per lane lie in packed / ropeCos / ropeSin; each lane's chunk_tokens of them are
+  // live.  Norm weights: both null (none), bf16, or float with normsAreFloat (the reference's
+  // NormWeights of a GGUF's F32 norms).
+  struct QkvBuffers final {
+    const void *packed = nullptr;
+    const void *queryNorm = nullptr;
+    const void *keyNorm = nullptr;
+    bool normsAreFloat = false;
+    const float *ropeCos = nullptr;
+    const float *ropeSin = nullptr;
+    void *queries = nullptr;
+    const uint64_t *const *pageTables = nullptr;
+  };
+  static void addQkvStore(void *stream, const kv::PageStorage &storage, uint32_t layer,
+                          const QkvBuffers &buffers, const std::vector<kv::ChunkedPrefillParams> &chunks,
+                          uint32_t queryHeads, uint32_t rows, uint32_t rowStride, uint32_t rotaryPairs,
+                          bool queryGate, float eps = 0.0f, uint32_t verifyMaxRows = 0) {
+    if ((buffers.queryNorm == nullptr) != (buffers.keyNorm == nullptr))
+      throw std::invalid_argument("query and key norms come together");
+    const kvx_qkv_shape shape{queryHeads, rotaryPairs, queryGate ? 1u : 0u,
+                              !buffers.queryNorm ? 0u : buffers.normsAreFloat ? 2u : 1u, eps};
+    check(kv_prepare_append(storage.handle(), layer, &shape, buffers.packed, buffers.queryNorm,
+                            buffers.keyNorm, buffers.ropeCos, buffers.ropeSin, buffers.queries, rowStride,
+                            buffers.pageTables, chunks.data(), static_cast<uint32_t>(chunks.size()), rows,
+                            verifyMaxRows, stream));
+  }
   static void addPrefill(void *stream, const kv::PageStorage &storage, uint32_t layer, const void *queries,
                          void *output, void *workspace, uint64_t workspaceBytes, const uint64_t *pageTable,
                          const kv::ChunkedPrefillParams &chunk, const PrefillAttentionPlan &plan) {

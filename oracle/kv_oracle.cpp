@@ -804,6 +804,83 @@ void ko_attention_hidden(uint32_t kv_heads, uint32_t group, uint32_t head_dim, u
   }
 }
 
+// ----------------------------------------------------------- QKV prepare ---
+namespace {
+// common/rms_inverse.h:14-31: simd_sum per 32 lanes (the xor butterfly), the
+// simdgroups' sums added in order by thread 0, rsqrt(total / width + eps).
+float rms_inverse_of_sums(const float *squares, uint32_t width, float eps) {
+  float total = 0.0f;
+  for (uint32_t base = 0; base < width; base += 32) {
+    float lane[32];
+    for (uint32_t i = 0; i < 32; ++i) lane[i] = squares[base + i];
+    for (uint32_t offset = 16; offset; offset >>= 1) {
+      float next[32];
+      for (uint32_t i = 0; i < 32; ++i) next[i] = lane[i] + lane[i ^ offset];
+      std::memcpy(lane, next, sizeof lane);
+    }
+    total += lane[0];
+  }
+  return 1.0f / std::sqrt(total / float(width) + eps);
+}
+}  // namespace
+
+void ko_qkv_prepare(uint32_t kv_heads, uint32_t group, uint32_t head_dim, uint32_t rotary_pairs,
+                    int query_gate, int norm_f32, float eps, uint32_t tokens, uint32_t stride,
+                    const uint16_t *packed, const void *q_norm, const void *k_norm,
+                    const float *rope_cos, const float *rope_sin, uint16_t *queries,
+                    uint16_t *chunk_keys, uint16_t *chunk_values) {
+  // common/attention_qkv_prepare.h:12-83, one task per (row, head), D threads
+  const uint32_t D = head_dim, q_heads = kv_heads * group;
+  const uint32_t q_stride = query_gate ? 2 * D : D;
+  const uint64_t packed_stride = uint64_t{q_heads} * q_stride + 2ull * kv_heads * D;
+  const uint32_t q_width = q_heads * q_stride, k_width = kv_heads * D;
+  const bool norms = q_norm && k_norm;
+  std::vector<float> element(D), squares(D);
+  std::vector<uint16_t> normalized(D);
+  const uint32_t tasks = tokens * (q_heads + kv_heads);
+  for (uint32_t task = 0; task < tasks; ++task) {
+    const bool query = task < tokens * q_heads;
+    const uint32_t local_task = query ? task : task - tokens * q_heads;
+    const uint32_t heads = query ? q_heads : kv_heads;
+    const uint32_t row = local_task / heads, head_index = local_task % heads;
+    const uint16_t *source = query ? packed + row * packed_stride + uint64_t{head_index} * q_stride
+                                   : packed + row * packed_stride + q_width + uint64_t{head_index} * D;
+    const void *weight = query ? q_norm : k_norm;
+    uint16_t *destination;
+    if (query) {
+      const uint32_t kv_head = head_index / group, local_head = head_index % group;
+      destination = queries + ((uint64_t{kv_head} * stride + row) * group + local_head) * D;
+    } else {
+      destination = chunk_keys + (uint64_t{head_index} * stride + row) * D;
+    }
+    for (uint32_t d = 0; d < D; ++d) {
+      element[d] = ko_bf16_to_float(source[d]);
+      squares[d] = element[d] * element[d];
+    }
+    const float inverse = norms ? rms_inverse_of_sums(squares.data(), D, eps) : 1.0f;
+    for (uint32_t d = 0; d < D; ++d) {
+      float scale = 1.0f;
+      if (norms)
+        scale = norm_f32 ? static_cast<const float *>(weight)[d]
+                         : ko_bf16_to_float(static_cast<const uint16_t *>(weight)[d]);
+      normalized[d] = ko_float_to_bf16(element[d] * inverse * scale);
+      if (!query) chunk_values[(uint64_t{head_index} * D + d) * stride + row] = source[k_width + d];
+    }
+    for (uint32_t d = 0; d < D; ++d) {
+      if (d < rotary_pairs) {
+        const float first = ko_bf16_to_float(normalized[d]);
+        const float second = ko_bf16_to_float(normalized[d + rotary_pairs]);
+        const float cosine = rope_cos[uint64_t{row} * rotary_pairs + d];
+        const float sine = rope_sin[uint64_t{row} * rotary_pairs + d];
+        destination[d] = ko_float_to_bf16(first * cosine - second * sine);
+        destination[d + rotary_pairs] = ko_float_to_bf16(second * cosine + first * sine);
+      } else if (d >= 2 * rotary_pairs) {
+        destination[d] = normalized[d];
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------ compaction ---
 int ko_compact_tree(uint32_t format, uint32_t kv_heads, uint32_t head_dim,
                     const uint64_t *const *page_tables, const ko_chunk_params *params,

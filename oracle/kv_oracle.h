@@ -24,6 +24,11 @@
  *                          values; the index map against an independent
  *                          transpose/reshape statement); the reference's only
  *                          check is a Metal fused-vs-unfused comparison
+ *   QKV prepare          : pinned by mathematics (float64 RMS norm and rotation,
+ *                          exact special cases); the simdgroup sum order and
+ *                          rsqrt of the reference are Metal's -- parity of
+ *                          those two unpinned (one float ulp before the bf16
+ *                          rounding)
  *   pool                 : pinned (reference pool tests' exact page ids/moves)
  */
 #pragma once
@@ -237,6 +242,25 @@ float ko_sigmoid(float x);
 void ko_attention_hidden(uint32_t kv_heads, uint32_t group, uint32_t head_dim, uint32_t lanes,
                          uint32_t rows, uint32_t row_stride, const uint16_t *attention,
                          const uint16_t *packed_qkv, uint16_t *hidden);
+
+/* QKV prepare of one lane: per-head RMS norm, partial rotary embedding and the layout
+   change from packed projection rows to attention queries and bf16 chunk rows
+   (common/attention_qkv_prepare.h:12-83, common/rms_inverse.h:14-31; entries
+   prefill_attention_qkv*, prefill/attention_qkv.metal:6-33, and verify_attention_qkv*,
+   decode/attention_qkv.metal:6-118, which call it per lane).
+   packed: bf16 [tokens][query heads x (query_gate ? 2 : 1) x D, kv heads x D keys, kv heads x D
+   values]; norms: NULL (none), bf16 (norm_f32 = 0) or float (norm_f32 = 1) [D]; rope_cos /
+   rope_sin: float [tokens][rotary_pairs]; queries: bf16 [kv head][stride][g][D]; chunk_keys
+   [kv head][stride][D], chunk_values [kv head][D][stride].
+   Two operations are implementation-defined in Metal and fixed here: simd_sum over a
+   simdgroup of 32 is the xor butterfly (offsets 16, 8, 4, 2, 1), and rsqrt(x) is the
+   correctly rounded 1 / sqrt(x).  Every other operation is a single rounded fp32 product,
+   sum or quotient in the source's order. */
+void ko_qkv_prepare(uint32_t kv_heads, uint32_t group, uint32_t head_dim, uint32_t rotary_pairs,
+                    int query_gate, int norm_f32, float eps, uint32_t tokens, uint32_t stride,
+                    const uint16_t *packed, const void *q_norm, const void *k_norm,
+                    const float *rope_cos, const float *rope_sin, uint16_t *queries,
+                    uint16_t *chunk_keys, uint16_t *chunk_values);
 
 /* ---- tree path compaction: decode/paged_attention_store.metal:198-278 ---- */
 int ko_compact_tree(uint32_t format, uint32_t kv_heads, uint32_t head_dim,

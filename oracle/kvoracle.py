@@ -205,6 +205,9 @@ def _declare(L):
     L.ko_attend_prefill.argtypes = [u32, u32, u32, u32, vp, vp, vp, vp, C.POINTER(PrefillParams)]
     L.ko_attend_verify.argtypes = [u32, u32, u32, u32, vp, vp, vp, vp, vp, u32, vp]
     L.ko_compact_tree.argtypes = [u32, u32, u32, vp, vp, vp, vp, u32, u32]
+    L.ko_qkv_prepare.argtypes = [u32, u32, u32, u32, C.c_int, C.c_int, C.c_float, u32, u32, vp, vp, vp,
+                                 vp, vp, vp, vp, vp]
+    L.ko_qkv_prepare.restype = None
     L.ko_sigmoid.argtypes = [C.c_float]
     L.ko_sigmoid.restype = C.c_float
     L.ko_attention_hidden.argtypes = [u32, u32, u32, u32, u32, u32, vp, vp, vp]
@@ -345,6 +348,21 @@ def attend_verify(fmt, kv_heads, group, head_dim, queries, tables, params, row_m
     n = lib().ko_attend_verify(fmt, kv_heads, group, head_dim, ptr(queries), ptr(out), ptr(f32),
                                _table_ptrs(tables), arr, len(params), ptr(row_masks))
     return n, out, f32
+
+
+def qkv_prepare(kv_heads, group, head_dim, rotary_pairs, query_gate, eps, tokens, stride, packed,
+                q_norm, k_norm, rope_cos, rope_sin):
+    """One lane: (queries [kv head][stride][g][D], chunk_keys [kv head][stride][D],
+    chunk_values [kv head][D][stride]) as bf16 bit patterns.  Norm weights: None, uint16 (bf16
+    bits) or float32 arrays."""
+    queries = np.zeros((kv_heads, stride, group, head_dim), dtype=np.uint16)
+    keys = np.zeros((kv_heads, stride, head_dim), dtype=np.uint16)
+    values = np.zeros((kv_heads, head_dim, stride), dtype=np.uint16)
+    norm_f32 = int(q_norm is not None and q_norm.dtype == np.float32)
+    lib().ko_qkv_prepare(kv_heads, group, head_dim, rotary_pairs, int(query_gate), norm_f32, eps,
+                         tokens, stride, ptr(packed), ptr(q_norm), ptr(k_norm), ptr(rope_cos),
+                         ptr(rope_sin), ptr(queries), ptr(keys), ptr(values))
+    return queries, keys, values
 
 
 def attention_hidden(kv_heads, group, head_dim, rows, attention, packed_qkv=None):

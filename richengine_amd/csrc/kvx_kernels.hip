@@ -46,39 +46,14 @@ __device__ inline bool append_contract(const AppendLane &l, const AppendArgs &a)
   return ok;
 }
 
-// One workgroup stores one row (one tensor, one head, one token) of one lane:
-// head_dim threads, one per dimension (reference:
-// common/paged_store_row.h:47-147, paged_store_row_fp8.h:28-78).
+// One thread's share of storing a row (one tensor, one head, one token): the
+// row's maximum over the workgroup's D threads, its scale, this dimension's code
+// (reference: common/paged_store_row.h:47-147, paged_store_row_fp8.h:28-78).
+// Every thread of the workgroup calls it; `wave_max` is four floats of LDS.
 template <uint32_t FMT>
-__global__ __launch_bounds__(256) void append_kernel(const uint16_t *__restrict__ chunk_keys,
-                                                     const uint16_t *__restrict__ chunk_values,
-                                                     AppendArgs a) {
-  __shared__ float wave_max[4];
-  const uint32_t group = blockIdx.x;
-  uint32_t li = 0;
-  if (a.uniform_groups) {
-    li = group / a.uniform_groups;
-  } else {
-    for (uint32_t i = 1; i < a.n_lanes; ++i)
-      if (group >= a.lane[i].group_base) li = i;
-  }
-  const AppendLane &l = a.lane[li];
-  if (!append_contract(l, a)) return;
-  const uint32_t D = a.head_dim, H = a.kv_heads;
-  const uint32_t local = group - l.group_base;
-  const uint32_t rows = l.tokens * H;
-  if (local >= 2 * rows) return;
-  const bool value_tensor = local >= rows;
-  const uint32_t row = value_tensor ? local - rows : local;
-  const uint32_t token = row % l.tokens, head = row / l.tokens;
-  const uint32_t d = threadIdx.x;
-  const uint32_t logical = l.committed + token;
-  // The row's source does not depend on the page entry: both loads are in flight together.
-  const uint16_t source =
-      value_tensor ? chunk_values[li * a.lane_stride + (uint64_t(head) * D + d) * l.stride + token]
-                   : chunk_keys[li * a.lane_stride + (uint64_t(head) * l.stride + token) * D + d];
-  const Slab s = slab_of(FMT, H, D, a.kv, head, l.table[logical / kPage]);
-  const uint32_t slot = logical % kPage;
+__device__ __forceinline__ void store_row_element(uint16_t source, bool value_tensor, const Slab &s,
+                                                  uint32_t slot, uint32_t d, uint32_t D,
+                                                  float *wave_max) {
   uint8_t *data = value_tensor ? s.values : s.keys;
   // Element index inside the head's slab: keys token-major, values
   // dimension-major (packed int4: both token-major).
@@ -116,6 +91,351 @@ __global__ __launch_bounds__(256) void append_kernel(const uint16_t *__restrict_
       }
     }
   }
+}
+
+// One workgroup stores one row (one tensor, one head, one token) of one lane:
+// head_dim threads, one per dimension (reference:
+// common/paged_store_row.h:47-147, paged_store_row_fp8.h:28-78).
+template <uint32_t FMT>
+__global__ __launch_bounds__(256) void append_kernel(const uint16_t *__restrict__ chunk_keys,
+                                                     const uint16_t *__restrict__ chunk_values,
+                                                     AppendArgs a) {
+  __shared__ float wave_max[4];
+  const uint32_t group = blockIdx.x;
+  uint32_t li = 0;
+  if (a.uniform_groups) {
+    li = group / a.uniform_groups;
+  } else {
+    for (uint32_t i = 1; i < a.n_lanes; ++i)
+      if (group >= a.lane[i].group_base) li = i;
+  }
+  const AppendLane &l = a.lane[li];
+  if (!append_contract(l, a)) return;
+  const uint32_t D = a.head_dim, H = a.kv_heads;
+  const uint32_t local = group - l.group_base;
+  const uint32_t rows = l.tokens * H;
+  if (local >= 2 * rows) return;
+  const bool value_tensor = local >= rows;
+  const uint32_t row = value_tensor ? local - rows : local;
+  const uint32_t token = row % l.tokens, head = row / l.tokens;
+  const uint32_t d = threadIdx.x;
+  const uint32_t logical = l.committed + token;
+  // The row's source does not depend on the page entry: both loads are in flight together.
+  const uint16_t source =
+      value_tensor ? chunk_values[li * a.lane_stride + (uint64_t(head) * D + d) * l.stride + token]
+                   : chunk_keys[li * a.lane_stride + (uint64_t(head) * l.stride + token) * D + d];
+  const Slab s = slab_of(FMT, H, D, a.kv, head, l.table[logical / kPage]);
+  store_row_element<FMT>(source, value_tensor, s, logical % kPage, d, D, wave_max);
+}
+
+// QKV prepare fused with the store: per-head RMS norm, partial rotary embedding
+// and the layout change from packed projection rows to attention queries
+// (reference: common/attention_qkv_prepare.h:12-83, common/rms_inverse.h:14-31),
+// with the key and value rows quantized straight into their page slots instead
+// of a bf16 chunk that the store kernel reads back.  One workgroup per (row,
+// head) task, query tasks first, head_dim threads.  The sums keep one fixed
+// order (32-lane xor butterflies, then the groups in order) and every product,
+// sum and quotient is rounded on its own, so results do not depend on the
+// launch.
+struct PrepareArgs {
+  AppendArgs append;  // lanes: table, committed tokens, live rows
+  const uint16_t *packed;
+  const void *q_norm, *k_norm;
+  const float *rope_cos, *rope_sin;
+  uint16_t *queries;
+  uint32_t query_heads, rotary_pairs, query_gate, norm_f32;
+  uint32_t rows;        // rows per lane in packed / rope_cos / rope_sin
+  uint32_t row_stride;  // rows between KV heads in the queries
+  float eps;
+};
+
+template <uint32_t FMT>
+__global__ __launch_bounds__(256) void prepare_append_kernel(PrepareArgs p) {
+  // Every product and sum below is rounded on its own: no fused multiply-add may
+  // be formed from them (the rounding intrinsics of the HIP headers are plain
+  // operators, which the default contraction mode would still fuse).
+#pragma clang fp contract(off)
+  __shared__ float reductions[8];
+  __shared__ float key_max[4], value_max[4];
+  __shared__ uint16_t normalized[256], rotated[256];
+  const AppendArgs &a = p.append;
+  const uint32_t group = blockIdx.x;
+  uint32_t li = 0;
+  for (uint32_t i = 1; i < a.n_lanes; ++i)
+    if (group >= a.lane[i].group_base) li = i;
+  const AppendLane &l = a.lane[li];
+  if (!append_contract(l, a)) return;
+  const uint32_t D = a.head_dim, H = a.kv_heads, QH = p.query_heads, G = QH / H;
+  const uint32_t local = group - l.group_base;
+  if (local >= l.tokens * (QH + H)) return;
+  const bool query = local < l.tokens * QH;
+  const uint32_t local_task = query ? local : local - l.tokens * QH;
+  const uint32_t heads = query ? QH : H;
+  const uint32_t row = local_task / heads, head = local_task % heads;
+  const uint32_t d = threadIdx.x;
+  const uint32_t q_stride = p.query_gate ? 2 * D : D;
+  const uint64_t packed_stride = uint64_t(QH) * q_stride + 2ull * H * D;
+  const uint16_t *source = p.packed + (uint64_t(li) * p.rows + row) * packed_stride +
+                           (query ? uint64_t(head) * q_stride : uint64_t(QH) * q_stride + uint64_t(head) * D);
+  const uint16_t raw = source[d];
+  const uint16_t raw_value = query ? uint16_t(0) : source[uint64_t(H) * D + d];
+  const float element = bf16_to_f32(raw);
+  float inverse = 1.0f, scale = 1.0f;
+  if (p.q_norm) {
+    float sum = element * element;
+    for (int offset = 16; offset; offset >>= 1) sum = sum + __shfl_xor(sum, offset);
+    if ((d & 31u) == 0) reductions[d >> 5] = sum;
+    __syncthreads();
+    float total = 0.0f;
+    for (uint32_t i = 0; i < D / 32; ++i) total = total + reductions[i];
+    // sqrtf and the quotients are correctly rounded (__fsqrt_rn is the hardware's
+    // approximate root)
+    const float mean = total / float(D);
+    inverse = 1.0f / sqrtf(mean + p.eps);
+    const void *weight = query ? p.q_norm : p.k_norm;
+    scale = p.norm_f32 ? static_cast<const float *>(weight)[d]
+                       : bf16_to_f32(static_cast<const uint16_t *>(weight)[d]);
+  }
+  const float unit = element * inverse;
+  normalized[d] = f32_to_bf16(unit * scale);
+  __syncthreads();
+  const uint32_t RP = p.rotary_pairs;
+  if (d < RP) {
+    const float first = bf16_to_f32(normalized[d]), second = bf16_to_f32(normalized[d + RP]);
+    const uint64_t at = (uint64_t(li) * p.rows + row) * RP + d;
+    const float cosine = p.rope_cos[at], sine = p.rope_sin[at];
+    const float fc = first * cosine, ss = second * sine, sc = second * cosine, fs = first * sine;
+    rotated[d] = f32_to_bf16(fc - ss);
+    rotated[d + RP] = f32_to_bf16(sc + fs);
+  } else if (d >= 2 * RP) {
+    rotated[d] = normalized[d];
+  }
+  __syncthreads();
+  const uint16_t prepared = rotated[d];
+  if (query) {
+    const uint32_t kv_head = head / G, local_head = head % G;
+    p.queries[uint64_t(li) * H * p.row_stride * G * D +
+              ((uint64_t(kv_head) * p.row_stride + row) * G + local_head) * D + d] = prepared;
+    return;
+  }
+  const uint32_t logical = l.committed + row;
+  const Slab s = slab_of(FMT, H, D, a.kv, head, l.table[logical / kPage]);
+  store_row_element<FMT>(prepared, false, s, logical % kPage, d, D, key_max);
+  store_row_element<FMT>(raw_value, true, s, logical % kPage, d, D, value_max);
+}
+
+// E consecutive bf16 values (E x 2 bytes, aligned to that) as one load / store.
+template <uint32_t E>
+__device__ __forceinline__ void load_bf16s(const uint16_t *from, uint16_t (&out)[E]) {
+  if constexpr (E == 4) {
+    const uint2 v = *reinterpret_cast<const uint2 *>(from);
+    out[0] = uint16_t(v.x), out[1] = uint16_t(v.x >> 16), out[2] = uint16_t(v.y), out[3] = uint16_t(v.y >> 16);
+  } else if constexpr (E == 2) {
+    const uint32_t v = *reinterpret_cast<const uint32_t *>(from);
+    out[0] = uint16_t(v), out[1] = uint16_t(v >> 16);
+  } else {
+    out[0] = *from;
+  }
+}
+template <uint32_t E>
+__device__ __forceinline__ void store_bf16s(uint16_t *to, const uint16_t (&v)[E]) {
+  if constexpr (E == 4) {
+    *reinterpret_cast<uint2 *>(to) = uint2{uint32_t(v[0]) | (uint32_t(v[1]) << 16), uint32_t(v[2]) | (uint32_t(v[3]) << 16)};
+  } else if constexpr (E == 2) {
+    *reinterpret_cast<uint32_t *>(to) = uint32_t(v[0]) | (uint32_t(v[1]) << 16);
+  } else {
+    *to = v[0];
+  }
+}
+template <uint32_t E>
+__device__ __forceinline__ void load_floats(const float *from, float (&out)[E]) {
+  if constexpr (E == 4) {
+    const float4 v = *reinterpret_cast<const float4 *>(from);
+    out[0] = v.x, out[1] = v.y, out[2] = v.z, out[3] = v.w;
+  } else if constexpr (E == 2) {
+    const float2 v = *reinterpret_cast<const float2 *>(from);
+    out[0] = v.x, out[1] = v.y;
+  } else {
+    out[0] = *from;
+  }
+}
+
+// The same work with one wave per (row, head) task for head dimensions 64, 128
+// and 256: each lane owns E = D / 64 consecutive dimensions, the sums and the
+// row maxima travel by lane exchange, and nothing goes through LDS.  The sum of
+// squares keeps the order of the kernel above: within each 32 dimensions the
+// xor butterfly over dimension offsets 16, 8, 4, 2, 1 (offsets of E and more are
+// lane exchanges, smaller ones pair a lane's own elements), then the groups in
+// order; the results are the same bits.  Needs rotary_pairs / E to be a power
+// of two, so that a pair's two dimensions sit rotary_pairs / E lanes apart.
+template <uint32_t FMT, uint32_t E>
+__device__ __forceinline__ void store_row_wave(const uint16_t (&source)[E], bool value_tensor,
+                                               const Slab &s, uint32_t slot, uint32_t lane,
+                                               uint32_t D) {
+  uint8_t *data = value_tensor ? s.values : s.keys;
+  const uint32_t d0 = E * lane;
+  const bool token_major = !value_tensor || FMT == KVX_FMT_INT4;
+  if constexpr (FMT == KVX_FMT_BF16) {
+    uint16_t *out = reinterpret_cast<uint16_t *>(data);
+    if (token_major) {
+      store_bf16s<E>(out + slot * D + d0, source);
+    } else {
+#pragma unroll
+      for (uint32_t e = 0; e < E; ++e) out[(d0 + e) * kPage + slot] = source[e];
+    }
+    return;
+  } else {
+    float v[E];
+    float m = 0.0f;
+#pragma unroll
+    for (uint32_t e = 0; e < E; ++e) {
+      v[e] = bf16_to_f32(source[e]);
+      m = fmaxf(m, fabsf(v[e]));
+    }
+    for (int offset = 32; offset; offset >>= 1) m = fmaxf(m, __shfl_xor(m, offset));
+    const float maximum = m;
+    constexpr float qmax = FMT == KVX_FMT_INT4 ? 7.0f : FMT == KVX_FMT_INT8 ? 127.0f : 448.0f;
+    const float scale = maximum == 0.0f ? 0.0f : __fdiv_rn(maximum, qmax);
+    if (lane == 0) (value_tensor ? s.value_scales : s.key_scales)[slot] = scale;
+    uint32_t code[E];
+#pragma unroll
+    for (uint32_t e = 0; e < E; ++e) {
+      const float scaled = maximum == 0.0f ? 0.0f : __fdiv_rn(__fmul_rn(v[e], qmax), maximum);
+      if constexpr (FMT == KVX_FMT_FP8E4M3) {
+        code[e] = maximum == 0.0f ? 0u : uint32_t(f32_to_e4m3(scaled));
+      } else {
+        constexpr int limit = FMT == KVX_FMT_INT4 ? 7 : 127;
+        int c = int(rintf(scaled));
+        c = c < -limit ? -limit : c > limit ? limit : c;
+        if (maximum == 0.0f) c = 0;
+        code[e] = uint32_t(c) & (FMT == KVX_FMT_INT4 ? 0xfu : 0xffu);
+      }
+    }
+    if constexpr (FMT == KVX_FMT_INT4) {
+      // Even dimension in the low nibble; both tensors token-major.
+      uint8_t *out = data + (slot * D + d0) / 2;
+      if constexpr (E == 1) {
+        const uint32_t partner = __shfl_xor(code[0], 1);
+        if ((lane & 1) == 0) *out = uint8_t(code[0] | (partner << 4));
+      } else if constexpr (E == 2) {
+        *out = uint8_t(code[0] | (code[1] << 4));
+      } else {
+        *reinterpret_cast<uint16_t *>(out) =
+            uint16_t(code[0] | (code[1] << 4) | (code[2] << 8) | (code[3] << 12));
+      }
+    } else if (token_major) {
+      uint8_t *out = data + slot * D + d0;
+      if constexpr (E == 4) {
+        *reinterpret_cast<uint32_t *>(out) = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
+      } else if constexpr (E == 2) {
+        *reinterpret_cast<uint16_t *>(out) = uint16_t(code[0] | (code[1] << 8));
+      } else {
+        *out = uint8_t(code[0]);
+      }
+    } else {
+#pragma unroll
+      for (uint32_t e = 0; e < E; ++e) data[(d0 + e) * kPage + slot] = uint8_t(code[e]);
+    }
+  }
+}
+
+template <uint32_t FMT, uint32_t E>
+__global__ __launch_bounds__(256) void prepare_append_wave_kernel(PrepareArgs p) {
+#pragma clang fp contract(off)
+  constexpr uint32_t D = 64 * E;
+  const AppendArgs &a = p.append;
+  const uint32_t task_id = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
+  uint32_t li = 0;
+  for (uint32_t i = 1; i < a.n_lanes; ++i)
+    if (task_id >= a.lane[i].group_base) li = i;
+  const AppendLane &l = a.lane[li];
+  if (!append_contract(l, a)) return;
+  const uint32_t H = a.kv_heads, QH = p.query_heads, G = QH / H;
+  const uint32_t local = task_id - l.group_base;
+  if (local >= l.tokens * (QH + H)) return;
+  const bool query = local < l.tokens * QH;
+  const uint32_t local_task = query ? local : local - l.tokens * QH;
+  const uint32_t heads = query ? QH : H;
+  const uint32_t row = local_task / heads, head = local_task % heads;
+  const uint32_t d0 = E * lane;
+  const uint32_t q_stride = p.query_gate ? 2 * D : D;
+  const uint64_t packed_stride = uint64_t(QH) * q_stride + 2ull * H * D;
+  const uint16_t *source = p.packed + (uint64_t(li) * p.rows + row) * packed_stride +
+                           (query ? uint64_t(head) * q_stride : uint64_t(QH) * q_stride + uint64_t(head) * D);
+  // Everything the task reads is requested before anything waits: the row, the
+  // value row (a query task reads its own row twice), the norm weights (any
+  // readable address when there are none), the rotation of the lane's
+  // dimensions (entry 0 for dimensions past the rotated ones) and the page entry.
+  const bool norms = p.q_norm != nullptr;
+  const uint32_t RP = p.rotary_pairs, pair_lanes = RP / E;
+  const bool rotated = d0 < 2 * RP, is_first = d0 < RP;
+  uint16_t raw[E], raw_value[E], weight_bf16[E];
+  float weight_f32[E], cosine[E], sine[E];
+  load_bf16s<E>(source + d0, raw);
+  load_bf16s<E>(source + (query ? 0u : H * D) + d0, raw_value);
+  const void *weight = norms ? (query ? p.q_norm : p.k_norm) : static_cast<const void *>(p.packed);
+  if (p.norm_f32) load_floats<E>(static_cast<const float *>(weight) + d0, weight_f32);
+  else load_bf16s<E>(static_cast<const uint16_t *>(weight) + d0, weight_bf16);
+  const uint64_t rope_at = (uint64_t(li) * p.rows + row) * RP + (rotated ? (is_first ? d0 : d0 - RP) : 0u);
+  load_floats<E>(p.rope_cos + rope_at, cosine);
+  load_floats<E>(p.rope_sin + rope_at, sine);
+  const uint32_t logical = l.committed + row;
+  const uint64_t entry = l.table[logical / kPage];
+
+  float element[E], scale[E];
+  float inverse = 1.0f;
+#pragma unroll
+  for (uint32_t e = 0; e < E; ++e) {
+    element[e] = bf16_to_f32(raw[e]);
+    scale[e] = !norms ? 1.0f : p.norm_f32 ? weight_f32[e] : bf16_to_f32(weight_bf16[e]);
+  }
+  if (norms) {
+    float sum[E];
+#pragma unroll
+    for (uint32_t e = 0; e < E; ++e) sum[e] = element[e] * element[e];
+    // dimension offsets 16 .. E: the partner sits offset / E lanes away
+#pragma unroll
+    for (uint32_t offset = 16; offset >= E; offset >>= 1) {
+#pragma unroll
+      for (uint32_t e = 0; e < E; ++e) sum[e] = sum[e] + __shfl_xor(sum[e], int(offset / E));
+    }
+    // dimension offsets below E pair the lane's own elements
+    float group_sum;
+    if constexpr (E == 4) {
+      const float a02 = sum[0] + sum[2], a13 = sum[1] + sum[3];
+      group_sum = a02 + a13;
+    } else if constexpr (E == 2) {
+      group_sum = sum[0] + sum[1];
+    } else {
+      group_sum = sum[0];
+    }
+    // the groups of 32 dimensions in order; a group spans 32 / E lanes
+    float total = 0.0f;
+#pragma unroll
+    for (uint32_t g = 0; g < D / 32; ++g) total = total + __shfl(group_sum, int(g * (32 / E)));
+    const float mean = total / float(D);
+    inverse = 1.0f / sqrtf(mean + p.eps);
+  }
+  uint16_t prepared[E];
+#pragma unroll
+  for (uint32_t e = 0; e < E; ++e) {
+    const float unit = element[e] * inverse;
+    const uint16_t normal = f32_to_bf16(unit * scale[e]);
+    const float mine = bf16_to_f32(normal);
+    const float other = __shfl_xor(mine, int(pair_lanes));
+    const float mc = mine * cosine[e], os = other * sine[e];
+    prepared[e] = rotated ? f32_to_bf16(is_first ? mc - os : mc + os) : normal;
+  }
+  if (query) {
+    const uint32_t kv_head = head / G, local_head = head % G;
+    store_bf16s<E>(p.queries + uint64_t(li) * H * p.row_stride * G * D +
+                       ((uint64_t(kv_head) * p.row_stride + row) * G + local_head) * D + d0,
+                   prepared);
+    return;
+  }
+  const Slab s = slab_of(FMT, H, D, a.kv, head, entry);
+  store_row_wave<FMT, E>(prepared, false, s, logical % kPage, lane, D);
+  store_row_wave<FMT, E>(raw_value, true, s, logical % kPage, lane, D);
 }
 
 // The same store for chunks of many tokens: one workgroup per (lane, logical page
@@ -868,6 +1188,96 @@ int kv_append(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
       hipLaunchKernelGGL((append_kernel<decltype(fmt)::value>), dim3(groups), dim3(D), 0,
                          static_cast<hipStream_t>(stream), keys, values, a);
       return check_launch("append_kernel");
+    });
+    if (rc) return rc;
+  }
+  return KVX_OK;
+}
+
+int kv_prepare_append(const kvx_storage *s, uint32_t layer, const kvx_qkv_shape *shape,
+                      const void *packed_qkv, const void *q_norm, const void *k_norm,
+                      const float *rope_cos, const float *rope_sin, void *queries,
+                      uint32_t row_stride, const uint64_t *const *page_tables,
+                      const kvx_chunk_params *lanes, uint32_t n_lanes, uint32_t rows,
+                      uint32_t verify_max_rows, void *stream) {
+  if (!s || !shape || !packed_qkv || !rope_cos || !rope_sin || !queries || !page_tables || !lanes ||
+      !n_lanes)
+    return fail(KVX_EINVAL, "kv_prepare_append: null argument or no lanes");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
+  kvx_kv_layer kv;
+  if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
+  const uint32_t H = s->layout.kv_heads, D = s->layout.head_dim;
+  if (!shape->query_heads || shape->query_heads % H)
+    return fail(KVX_EINVAL, "query heads are not a multiple of the KV heads");
+  if (D % 32 || D > 256) return fail(KVX_EINVAL, "QKV prepare covers head dimensions 32..256 in steps of 32");
+  if (!shape->rotary_pairs || 2 * shape->rotary_pairs > D)
+    return fail(KVX_EINVAL, "rotary pairs do not fit the head dimension");
+  if (shape->norm_type > 2 || (shape->norm_type && (!q_norm || !k_norm)))
+    return fail(KVX_EINVAL, "norm weights are missing or of an unknown type");
+  if (packed_qkv == queries) return fail(KVX_EINVAL, "packed rows and queries must not alias");
+  for (const void *buffer : {packed_qkv, q_norm, k_norm, static_cast<const void *>(rope_cos),
+                             static_cast<const void *>(rope_sin), static_cast<const void *>(queries)})
+    if (reinterpret_cast<uintptr_t>(buffer) % 16)
+      return fail(KVX_EINVAL, "kv_prepare_append: buffers must be 16-byte aligned");
+  if (verify_max_rows > KVX_TREE_NODES)
+    return fail(KVX_EINVAL, "verify stores hold at most 16 rows per lane");
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    static const char *const names[] = {"", "chunk_tokens_out_of_range", "context_out_of_range",
+                                        "chunk_stride_invalid", "page_table_too_short"};
+    if (const int e = kvx_chunk_validation(&lanes[i])) return fail(KVX_EINVAL, names[e]);
+    if (lanes[i].chunk_tokens > rows || rows > row_stride)
+      return fail(KVX_EINVAL, "a lane's rows exceed the packed rows or the row stride");
+    if (verify_max_rows && lanes[i].chunk_tokens > verify_max_rows)
+      return fail(KVX_EINVAL, "verify store rows are out of range");
+    if (!page_tables[i]) return fail(KVX_EINVAL, "kv_prepare_append: null page table");
+  }
+  const uint32_t QH = shape->query_heads;
+  const uint64_t packed_lane = uint64_t(rows) * (uint64_t(QH) * (shape->query_gate ? 2 : 1) + 2ull * H) * D;
+  for (uint32_t first = 0; first < n_lanes; first += kLanes) {
+    PrepareArgs p{};
+    AppendArgs &a = p.append;
+    a.n_lanes = std::min(kLanes, n_lanes - first);
+    a.kv_heads = H;
+    a.head_dim = D;
+    a.verify_max_rows = 0;  // the rows bound was checked above; there is no chunk stride here
+    a.kv = kv;
+    uint32_t groups = 0;
+    for (uint32_t i = 0; i < a.n_lanes; ++i) {
+      const kvx_chunk_params &c = lanes[first + i];
+      a.lane[i] = {page_tables[first + i], c.committed_tokens, c.chunk_tokens, c.chunk_stride,
+                   c.page_table_entries, groups, 0};
+      groups += c.chunk_tokens * (QH + H);
+    }
+    p.packed = static_cast<const uint16_t *>(packed_qkv) + uint64_t(first) * packed_lane;
+    p.q_norm = shape->norm_type ? q_norm : nullptr;
+    p.k_norm = shape->norm_type ? k_norm : nullptr;
+    p.rope_cos = rope_cos + uint64_t(first) * rows * shape->rotary_pairs;
+    p.rope_sin = rope_sin + uint64_t(first) * rows * shape->rotary_pairs;
+    p.queries = static_cast<uint16_t *>(queries) + uint64_t(first) * H * row_stride * (QH / H) * D;
+    p.query_heads = QH;
+    p.rotary_pairs = shape->rotary_pairs;
+    p.query_gate = shape->query_gate ? 1 : 0;
+    p.norm_f32 = shape->norm_type == 2;
+    p.rows = rows;
+    p.row_stride = row_stride;
+    p.eps = shape->eps != 0.0f ? shape->eps : 1e-6f;
+    // One wave per task where the head dimension is 64, 128 or 256 and a rotary pair's
+    // dimensions are a power-of-two number of lanes apart; else one workgroup per task.
+    const uint32_t E = D / 64, pair_lanes = E ? shape->rotary_pairs / E : 0;
+    const bool by_wave = (D == 64 || D == 128 || D == 256) && shape->rotary_pairs % E == 0 &&
+                         pair_lanes && !(pair_lanes & (pair_lanes - 1));
+    const int rc = dispatch_format(s->layout.format, [&](auto fmt) {
+      constexpr uint32_t F = decltype(fmt)::value;
+      const hipStream_t st = static_cast<hipStream_t>(stream);
+      if (by_wave) {
+        const dim3 grid((groups + 3) / 4), block(256);
+        if (E == 4) hipLaunchKernelGGL((prepare_append_wave_kernel<F, 4>), grid, block, 0, st, p);
+        else if (E == 2) hipLaunchKernelGGL((prepare_append_wave_kernel<F, 2>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((prepare_append_wave_kernel<F, 1>), grid, block, 0, st, p);
+        return check_launch("prepare_append_wave_kernel");
+      }
+      hipLaunchKernelGGL((prepare_append_kernel<F>), dim3(groups), dim3(D), 0, st, p);
+      return check_launch("prepare_append_kernel");
     });
     if (rc) return rc;
   }

@@ -34,7 +34,7 @@ SYMBOLS = [
     "kvx_storage_extent_write", "kv_page_copy", "kvx_pool_create", "kvx_pool_destroy",
     "kvx_pool_acquire", "kvx_pool_retain", "kvx_pool_release", "kvx_pool_page_active",
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
-    "kvx_pool_snapshot_get", "kv_append", "kv_attend_verify", "kv_attend_verify_hidden", "kv_attend_decode",
+    "kvx_pool_snapshot_get", "kv_append", "kv_prepare_append", "kv_attend_verify", "kv_attend_verify_hidden", "kv_attend_decode",
     "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kv_page_export", "kv_page_import", "kvx_debug_set_attend_phases",
     "kvx_debug_attend_paths", "kvx_decode_plan", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
@@ -54,6 +54,11 @@ class Layout(C.Structure):
 
 class KvLayer(C.Structure):
     _fields_ = [("extent_pages", C.c_uint32), ("offset", C.c_uint32)]
+
+
+class QkvShape(C.Structure):
+    _fields_ = [("query_heads", C.c_uint32), ("rotary_pairs", C.c_uint32), ("query_gate", C.c_uint32),
+                ("norm_type", C.c_uint32), ("eps", C.c_float)]
 
 
 class ChunkParams(C.Structure):
@@ -203,6 +208,8 @@ def _declare(L):
     L.kvx_pool_compact_extent.argtypes = [vp, vp, u32, C.POINTER(u32), vp, C.POINTER(u32), vp]
     L.kvx_pool_snapshot_get.argtypes = [vp, C.POINTER(PoolSnapshot)]
     L.kv_append.argtypes = [vp, u32, vp, vp, vp, vp, u32, u64, u32, vp]
+    L.kv_prepare_append.argtypes = [vp, u32, C.POINTER(QkvShape), vp, vp, vp, vp, vp, vp, u32, vp, vp,
+                                    u32, u32, u32, vp]
     L.kv_attend_verify.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, vp, u32, vp, u64, vp]
     L.kv_attend_verify_hidden.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, vp, u32, vp, u64, vp, vp,
                                           vp]
@@ -340,6 +347,16 @@ def append(storage, layer, chunk_keys, chunk_values, tables, lanes, lane_stride,
 def attend_workspace_bytes(storage, lanes, query_heads):
     arr = (VerifyParams * len(lanes))(*lanes)
     return lib().kvx_attend_workspace_bytes(arr, len(lanes), query_heads, C.byref(storage.layout))
+
+
+def prepare_append(storage, layer, shape, packed_qkv, q_norm, k_norm, rope_cos, rope_sin, queries,
+                   row_stride, tables, lanes, rows, verify_max_rows=0, stream=None):
+    """QKV prepare fused with quantize-on-append (kv_prepare_append)."""
+    arr = (ChunkParams * len(lanes))(*lanes)
+    return check(lib().kv_prepare_append(storage.h, layer, C.byref(shape), _ptr(packed_qkv),
+                                         _ptr(q_norm), _ptr(k_norm), _ptr(rope_cos), _ptr(rope_sin),
+                                         _ptr(queries), row_stride, _table_array(tables), arr,
+                                         len(lanes), rows, verify_max_rows, _stream(stream)))
 
 
 def attend_verify(storage, layer, query_heads, queries, output, tables, lanes, row_masks,

@@ -370,6 +370,64 @@ void testAppendDecodeSingleToken() {
   hip(hipFree(outputDevice));
 }
 
+// The fused QKV prepare + store without norms and with an identity rotation is the
+// layout change alone: the pages must hold what addPrefillStore writes from the same
+// rows, and the queries the packed query values.
+void testQkvStoreIsPrepareThenStore() {
+  const Layout layout{1, 4, 256, Format::Int8};
+  const uint32_t H = 4, G = 6, D = 256, QH = H * G, T = 5, packedStride = (2 * QH + 2 * H) * D;
+  kv::PageStorage plain(layout, 4, 4, /*aligned=*/false), fused(layout, 4, 4, /*aligned=*/false);
+  plain.allocateExtent(0);
+  fused.allocateExtent(0);
+  const std::vector<uint32_t> pages{2, 1};
+  std::vector<uint64_t> plainTable(2), fusedTable(2);
+  plain.entries(pages, 0, plainTable.data());
+  fused.entries(pages, 0, fusedTable.data());
+  uint64_t *plainDevice = toDevice(plainTable), *fusedDevice = toDevice(fusedTable);
+  std::vector<uint16_t> packed(T * packedStride), keys(H * 32 * D, 0), values(H * D * 32, 0);
+  for (size_t i = 0; i < packed.size(); ++i) packed[i] = bf16(std::sin(0.013f * float(i % 7919)));
+  for (uint32_t t = 0; t < T; ++t)
+    for (uint32_t h = 0; h < H; ++h)
+      for (uint32_t d = 0; d < D; ++d) {
+        keys[(h * 32 + t) * D + d] = packed[t * packedStride + 2 * QH * D + h * D + d];
+        values[(h * D + d) * 32 + t] = packed[t * packedStride + 2 * QH * D + H * D + h * D + d];
+      }
+  std::vector<float> ones(T * 32, 1.0f), zeros(T * 32, 0.0f);
+  uint16_t *packedDevice = toDevice(packed), *keysDevice = toDevice(keys), *valuesDevice = toDevice(values);
+  float *cosDevice = toDevice(ones), *sinDevice = toDevice(zeros);
+  uint16_t *queriesDevice = nullptr;
+  hip(hipMalloc(&queriesDevice, size_t{H} * 32 * G * D * 2));
+  hip(hipMemset(queriesDevice, 0, size_t{H} * 32 * G * D * 2));
+  const auto chunk = ops::PagedAttention::prefillParams(30, T, 32, 2);  // crosses a page boundary
+  ops::PagedAttention::addPrefillStore(nullptr, plain, 0, keysDevice, valuesDevice, plainDevice, chunk);
+  const uint64_t *tables[1] = {fusedDevice};
+  ops::PagedAttention::QkvBuffers buffers;
+  buffers.packed = packedDevice;
+  buffers.ropeCos = cosDevice;
+  buffers.ropeSin = sinDevice;
+  buffers.queries = queriesDevice;
+  buffers.pageTables = tables;
+  ops::PagedAttention::addQkvStore(nullptr, fused, 0, buffers, {chunk}, QH, T, 32, 32, /*queryGate=*/true);
+  hip(hipDeviceSynchronize());
+  EXPECT(plain.readPage(2) == fused.readPage(2) && plain.readPage(1) == fused.readPage(1));
+  std::vector<uint16_t> queries(size_t{H} * 32 * G * D);
+  hip(hipMemcpy(queries.data(), queriesDevice, queries.size() * 2, hipMemcpyDeviceToHost));
+  uint32_t wrong = 0;
+  for (uint32_t t = 0; t < T; ++t)
+    for (uint32_t q = 0; q < QH; ++q)
+      for (uint32_t d = 0; d < D; ++d)
+        wrong += queries[(((q / G) * 32 + t) * G + q % G) * D + d] != packed[t * packedStride + q * 2 * D + d];
+  EXPECT(wrong == 0);
+  buffers.keyNorm = packedDevice;  // one norm without the other
+  EXPECT(throws<std::invalid_argument>([&] {
+    ops::PagedAttention::addQkvStore(nullptr, fused, 0, buffers, {chunk}, QH, T, 32, 32, true);
+  }));
+  for (void *p : {static_cast<void *>(plainDevice), static_cast<void *>(fusedDevice), static_cast<void *>(packedDevice),
+                  static_cast<void *>(keysDevice), static_cast<void *>(valuesDevice), static_cast<void *>(cosDevice),
+                  static_cast<void *>(sinDevice), static_cast<void *>(queriesDevice)})
+    hip(hipFree(p));
+}
+
 }  // namespace
 
 int main(int argc, char **argv) {
@@ -381,6 +439,7 @@ int main(int argc, char **argv) {
     testStorageLifecycle();
     testPoolCompaction();
     testAppendDecodeSingleToken();
+    testQkvStoreIsPrepareThenStore();
   }
   if (failures) {
     std::printf("kvx_host_test (%s): %d failure(s)\n", mode.c_str(), failures);

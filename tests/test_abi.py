@@ -172,4 +172,5 @@ def test_hot_kernels_stay_out_of_scratch_memory():
     assert one("decode_int4_kernel")["occupancy"] == 2
     assert one("attend_wide_kernelILj1ELj1ELj2E")["occupancy"] == 2
     for fmt in (1, 2, 3, 4):
-        assert one(f"append_kernelILj{fmt}E")["scratchsize"] == 0
+        assert one(f"13append_kernelILj{fmt}E")["scratchsize"] == 0
+        assert one(f"prepare_append_kernelILj{fmt}E")["scratchsize"] == 0
