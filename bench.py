@@ -60,6 +60,10 @@ def parse():
                     help="decode: the merge also writes the out-projection's operand "
                          "(kv_attend_verify_hidden), gated by packed projection rows or plainly "
                          "gathered; implies --separate-append")
+    ap.add_argument("--prepare", action="store_true",
+                    help="decode: the step's queries, keys and values come from packed projection rows "
+                         "through kv_prepare_append (norm, rotation, quantize, store) instead of "
+                         "ready chunk rows through kv_append; implies --separate-append")
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
     ap.add_argument("--workload", choices=["decode", "tree-verify", "prefill", "qkv-prepare"], default="decode",
@@ -563,6 +567,17 @@ def main():
         if args.hidden == "gate":
             packed = torch.randn((BATCH, 1, (2 * QH + 2 * H) * D), generator=gen, device="cuda").bfloat16()
 
+    qkv_shape = qkv_packed = None
+    if args.prepare:
+        args.separate_append = True
+        qkv_shape = kvx.QkvShape(QH, 32, 1, 1, 0.0)
+        qkv_packed = packed if packed is not None else torch.randn(
+            (BATCH, 1, (2 * QH + 2 * H) * D), generator=gen, device="cuda").bfloat16()
+        norm_q = torch.randn(D, generator=gen, device="cuda").bfloat16()
+        norm_k = torch.randn(D, generator=gen, device="cuda").bfloat16()
+        rope_cos = torch.rand((BATCH, 1, 32), generator=gen, device="cuda")
+        rope_sin = torch.rand((BATCH, 1, 32), generator=gen, device="cuda")
+
     def attend(layer, vp_arr):
         if hidden is None:
             return L.kv_attend_decode(storage.h, layer, QH, queries.data_ptr(), output.data_ptr(),
@@ -586,8 +601,14 @@ def main():
                 if rc:
                     kvx.check(rc)
                 continue
-            rc = L.kv_append(storage.h, layer, chunk_k.data_ptr(), chunk_v.data_ptr(), table_arr,
-                             ap_arr, BATCH, lane_stride, 15, stream)
+            if args.prepare:
+                rc = L.kv_prepare_append(storage.h, layer, C.byref(qkv_shape), qkv_packed.data_ptr(),
+                                         norm_q.data_ptr(), norm_k.data_ptr(), rope_cos.data_ptr(),
+                                         rope_sin.data_ptr(), queries.data_ptr(), 1, table_arr, ap_arr,
+                                         BATCH, 1, 15, stream)
+            else:
+                rc = L.kv_append(storage.h, layer, chunk_k.data_ptr(), chunk_v.data_ptr(), table_arr,
+                                 ap_arr, BATCH, lane_stride, 15, stream)
             if rc:
                 kvx.check(rc)
             rc = attend(layer, vp_arr)
@@ -663,8 +684,10 @@ def main():
             "pool_gb": round(extents * extent_bytes / 1e9, 1), "extents": extents,
             "page_order": "contiguous" if args.contiguous else "seed-shuffled",
             "seed": args.seed,
-            **({"entries": "kv_append + kv_attend_verify_hidden", "hidden": args.hidden}
-               if args.hidden != "none" else {}),
+            **({"entries": ("kv_prepare_append" if args.prepare else "kv_append") + " + " +
+                           ("kv_attend_verify_hidden" if args.hidden != "none" else "kv_attend_decode"),
+                "hidden": args.hidden}
+               if args.hidden != "none" or args.prepare else {}),
         },
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "decode_tokens_per_s": round(BATCH * args.steps / wall, 1),

@@ -47,6 +47,10 @@ struct DecodeLane {
   uint64_t q_offset;    // element offset of the lane's queries
 };
 struct DecodeArgs {
+  // First work item of every lane again, side by side (unused lanes hold the largest
+  // value): a wave finds its lane from these with a few wide scalar loads instead of
+  // walking the lane records, whose loads would follow one another.
+  uint32_t item_base[kLanes];
   DecodeLane lane[kLanes];
   uint32_t n_lanes;
   uint32_t kv_heads;
@@ -106,8 +110,10 @@ __device__ __forceinline__ DecodeLane lane_of_item(const DecodeArgs &a, uint32_t
   if (a.tile_lanes) {
     index = item / a.lane[0].split_count;
   } else {
-    for (uint32_t i = 1; i < a.n_lanes; ++i)
-      if (item >= a.lane[i].first_item) index = i;
+    // item_base is non-decreasing: the lane is the number of later lanes that
+    // start at or before the item.
+#pragma unroll
+    for (uint32_t i = 1; i < kLanes; ++i) index += item >= a.item_base[i] ? 1u : 0u;
   }
   return lane_at(a, index);
 }
@@ -359,6 +365,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       a.chunk_stride = fused->stride;
     }
     uint32_t items = 0, max_splits = 0;
+    for (uint32_t i = 0; i < kLanes; ++i) a.item_base[i] = UINT32_MAX;
     for (uint32_t i = 0; i < (tile_rows ? 1u : a.n_lanes); ++i) {
       const kvx_verify_params &p = lanes[first + i];
       DecodeLane &dl = a.lane[i];
@@ -368,6 +375,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       dl.active_rows = p.active_rows;
       dl.split_count = p.split_count;
       dl.first_item = items;
+      a.item_base[i] = items;
       dl.score_scale = p.score_scale != 0.0f ? p.score_scale : l.score_scale;
       dl.row_base = row_base;
       dl.q_offset = uint64_t(first + i) * lane_stride;

@@ -346,8 +346,12 @@ __global__ __launch_bounds__(256) void prepare_append_wave_kernel(PrepareArgs p)
   const AppendArgs &a = p.append;
   const uint32_t task_id = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
   uint32_t li = 0;
-  for (uint32_t i = 1; i < a.n_lanes; ++i)
-    if (task_id >= a.lane[i].group_base) li = i;
+  if (a.uniform_groups) {  // every lane has as many tasks: no walk over the lane records
+    li = min(task_id / a.uniform_groups, a.n_lanes - 1);
+  } else {
+    for (uint32_t i = 1; i < a.n_lanes; ++i)
+      if (task_id >= a.lane[i].group_base) li = i;
+  }
   const AppendLane &l = a.lane[li];
   if (!append_contract(l, a)) return;
   const uint32_t H = a.kv_heads, QH = p.query_heads, G = QH / H;
@@ -1248,6 +1252,9 @@ int kv_prepare_append(const kvx_storage *s, uint32_t layer, const kvx_qkv_shape 
                    c.page_table_entries, groups, 0};
       groups += c.chunk_tokens * (QH + H);
     }
+    a.uniform_groups = lanes[first].chunk_tokens * (QH + H);
+    for (uint32_t i = 0; i < a.n_lanes; ++i)
+      if (lanes[first + i].chunk_tokens != lanes[first].chunk_tokens) a.uniform_groups = 0;
     p.packed = static_cast<const uint16_t *>(packed_qkv) + uint64_t(first) * packed_lane;
     p.q_norm = shape->norm_type ? q_norm : nullptr;
     p.k_norm = shape->norm_type ? k_norm : nullptr;
