@@ -66,13 +66,17 @@ def parse():
                          "ready chunk rows through kv_append; implies --separate-append")
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
-    ap.add_argument("--workload", choices=["decode", "tree-verify", "prefill", "qkv-prepare"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "tree-verify", "prefill", "qkv-prepare", "shared-prefix"], default="decode",
                     help="decode = batch-32 mixed-length int4 decode, the headline metric (default); "
                          "tree-verify = 16-node tree verify and prefill = chunked prefill with a shared "
                          "prefix, the matrix-core paths (profiling)")
-    ap.add_argument("--format", choices=["bf16", "fp8", "int8", "int4"], default="bf16",
-                    help="page format of the prefill workload")
-    return ap.parse_args()
+    ap.add_argument("--format", choices=["bf16", "fp8", "int8", "int4"], default=None,
+                    help="page format of the prefill workload (default bf16) and of the shared-prefix "
+                         "workload (default int4; no fp8)")
+    args = ap.parse_args()
+    if args.format is None:
+        args.format = "int4" if args.workload == "shared-prefix" else "bf16"
+    return args
 
 
 def cpu_lane(ctx, seed):
@@ -365,6 +369,110 @@ def qkv_prepare(args):
     print(json.dumps(result))
 
 
+def shared_prefix(args):
+    """Decode attention of 16 sequences that share a 30 016-token prompt prefix (938 pages) and
+    hold 64..1024 tokens of their own, int4 pages, one layer per launch: kv_attend_decode_shared
+    (the prefix read once for all sequences) beside kv_attend_decode on the same page tables (the
+    prefix read once per sequence).  `value` is sequence-steps per second of one layer's
+    attention with the shared entry; the KV bytes counted are those of the whole sequences,
+    which is what the unshared entry has to read."""
+    import numpy as np
+    import torch
+    from richengine_amd import kvx
+
+    L = kvx.lib()
+    torch.cuda.set_device(0)
+    rng = np.random.default_rng(args.seed)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(args.seed)
+    fmt = {"bf16": kvx.BF16, "int8": kvx.INT8, "int4": kvx.INT4}[args.format]
+    bytes_per_token = {"bf16": 4096, "int8": 2080, "int4": BYTES_PER_TOKEN_LAYER}[args.format]
+    lanes, shared_pages = 16, 938
+    own = [int(t) for t in rng.integers(64, 1025, lanes)]
+    own_pages = [(t + 1 + 31) // 32 for t in own]
+    layout = kvx.Layout(LAYERS, H, D, fmt, 0.0)
+    extent_pages = L.kvx_layout_largest_extent_pages(C.byref(layout))
+    storage = kvx.Storage(LAYERS, H, D, fmt, extent_pages, extent_pages, aligned=True)
+    storage.allocate_all()
+    ids = rng.permutation(extent_pages).astype(np.uint32)
+    prefix, first, tables = ids[:shared_pages], shared_pages, []
+    for n in own_pages:
+        tables.append(storage.table(np.concatenate([prefix, ids[first:first + n]])))
+        first += n
+    entries = [shared_pages + n for n in own_pages]
+
+    def fill(lane, start, count):
+        done = 0
+        while done < count:
+            n = min(2048, count - done)
+            stride = (n + 31) // 32 * 32
+            k = torch.randn((H, stride, D), generator=gen, device="cuda").bfloat16()
+            v = torch.randn((H, D, stride), generator=gen, device="cuda").bfloat16()
+            for layer in range(LAYERS):
+                kvx.append(storage, layer, k, v, [tables[lane]],
+                           [kvx.ChunkParams(start + done, n, stride, entries[lane])], H * stride * D)
+            done += n
+
+    fill(0, 0, shared_pages * 32)
+    for lane in range(lanes):
+        fill(lane, shared_pages * 32, own[lane] + 1)
+    committed = [shared_pages * 32 + t for t in own]
+    queries = torch.randn((lanes, H, 1, G, D), generator=gen, device="cuda").bfloat16()
+    output = torch.zeros_like(queries)
+    prefix_splits = args.verify_splits or kvx.verify_plan([shared_pages * 32], lanes, H, QH)[0]
+    own_splits = kvx.decode_plan(own, H, fmt)
+    sp = [kvx.VerifyParams(committed[i], entries[i], kvx.KvLayer(), own_splits[i], own_splits[i], 1, 1, 0.0)
+          for i in range(lanes)]
+    plain_splits = kvx.decode_plan(committed, H, fmt)
+    pp = [kvx.VerifyParams(committed[i], entries[i], kvx.KvLayer(), plain_splits[i], plain_splits[i], 1, 1,
+                           0.0) for i in range(lanes)]
+    ws = torch.empty(max(kvx.attend_shared_workspace_bytes(storage, sp, prefix_splits, QH),
+                         kvx.attend_workspace_bytes(storage, pp, QH)) + 4096, dtype=torch.uint8, device="cuda")
+
+    def timed(call):
+        call(0)
+        torch.cuda.synchronize()
+        k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        k0.record()
+        for it in range(args.kernel_iters):
+            call(it % LAYERS)
+        k1.record()
+        torch.cuda.synchronize()
+        return k0.elapsed_time(k1) / args.kernel_iters
+
+    shared_ms = timed(lambda layer: kvx.attend_decode_shared(storage, layer, QH, queries, output, tables, sp,
+                                                             shared_pages, prefix_splits, 1, ws))
+    plain_ms = timed(lambda layer: kvx.attend_decode(storage, layer, QH, queries, output, tables, pp, 1, ws))
+    logical = sum(c + 1 for c in committed) * bytes_per_token
+    physical = (shared_pages * 32 + sum(t + 1 for t in own)) * bytes_per_token
+    result = {
+        "metric": args.format + " decode attention over a shared prefix, 16 sequences x 30 016 shared tokens: "
+                  "sequence-steps/s of one layer",
+        "value": round(lanes / (shared_ms * 1e-3), 1), "unit": "sequence-steps/s", "n_gpus": 1,
+        "steps": args.kernel_iters, "warmup": 1, "ms_per_step": round(shared_ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.format + " pages, bf16 / fp16 MFMA, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "kv_attend_decode_shared: 16 sequences, 938 shared pages, 64..1024 own "
+                               "tokens each, 4 KV heads x 256, 24 query heads, one layer per call",
+                   "format": args.format, "prefix_splits": int(prefix_splits), "seed": args.seed},
+        "roofline": {"bound": "mfma", "achieved": round(4 * D * QH * sum(c + 1 for c in committed) /
+                                                        (shared_ms * 1e-3) / 1e12, 1),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(4 * D * QH * sum(c + 1 for c in committed) / (shared_ms * 1e-3) / 1e12 /
+                                   MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": None, "kernel": "split kernels over the shared pages (stacked rows) and over the "
+                                                "sequences' own pages + shared_merge_kernel",
+                     "ms_per_launch": round(shared_ms, 4)},
+        "unshared_ms": round(plain_ms, 4),
+        "kv_bytes_logical": logical, "kv_bytes_physical": physical,
+        "logical_kv_gbs_shared": round(logical / (shared_ms * 1e-3) / 1e9, 1),
+        "logical_kv_gbs_unshared": round(logical / (plain_ms * 1e-3) / 1e9, 1),
+        "cpu_baseline": None,
+    }
+    storage.close()
+    print(json.dumps(result))
+
+
 def chunked_prefill(args):
     """Chunked prefill with prefix reuse: batch 4, a 2048-token chunk per sequence appended onto a
     shared 16384-token prefix (the prefix pages are the same physical pages in every
@@ -482,6 +590,8 @@ def main():
             kvx_build.build(verbose=False)
         if args.workload == "qkv-prepare":
             return qkv_prepare(args)
+        if args.workload == "shared-prefix":
+            return shared_prefix(args)
         return tree_verify(args) if args.workload == "tree-verify" else chunked_prefill(args)
     import numpy as np
     import torch

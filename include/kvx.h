@@ -474,6 +474,27 @@ int kv_attend_verify_hidden(const kvx_storage *storage, uint32_t layer, uint32_t
                             uint64_t workspace_bytes, const void *packed_qkv, void *hidden,
                             void *stream);
 
+/* One-row decode attention of up to 16 sequences whose page tables begin with the same
+   `shared_pages` pages (a cached prompt prefix, engine::KvCache chains restored by
+   Cache::restoreRequest): the shared pages are read once for all of them instead of once per
+   sequence.  The reference lists this as a gap (docs/PERF_REPORT.md:250, :259) and has no
+   counterpart; the result is kv_attend_decode's within its tolerance (the partition into splits
+   differs, so the fp32 sums are taken in another order).
+   The sequences' query rows are attended together over the prefix as the rows of one lane with
+   `prefix_splits` splits, each sequence's remaining pages as a decode lane of its own with
+   lanes[i].split_count splits, and one merge combines both per sequence.  lanes[i] describe the
+   whole sequences (committed_tokens >= shared_pages x 32; tables of all their pages).
+   queries / output as kv_attend_decode.  Head dimension 256, int4 / int8 / bf16 pages.
+   workspace: at least kvx_attend_shared_workspace_bytes(). */
+uint64_t kvx_attend_shared_workspace_bytes(const kvx_verify_params *lanes, uint32_t n_lanes,
+                                           uint32_t prefix_splits, uint32_t query_heads,
+                                           const kvx_layout *layout);
+int kv_attend_decode_shared(const kvx_storage *storage, uint32_t layer, uint32_t query_heads,
+                            const void *queries, void *output, const uint64_t *const *page_tables,
+                            const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t shared_pages,
+                            uint32_t prefix_splits, uint32_t row_stride, void *workspace,
+                            uint64_t workspace_bytes, void *stream);
+
 /* One-row decode attention per lane: kv_attend_verify with active_rows =
    row_capacity = 1 on the bandwidth-tuned kernels (the reference reaches decode
    through its prefill entries with rows = 1, prefill/paged_attention.metal:7-67,

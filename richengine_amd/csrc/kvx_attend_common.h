@@ -384,7 +384,9 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       row_base += uint64_t(p.split_count) * H * M;
     }
     if (tile_rows) items = n_lanes * lanes[0].split_count;
-    if (epilogue) {
+    if (epilogue && epilogue->partials_only) {
+      a.all_partials = 1;
+    } else if (epilogue) {
       a.hidden = epilogue->hidden + uint64_t(first) * capacity * query_heads * kD;
       a.packed_qkv = epilogue->packed_qkv
                          ? epilogue->packed_qkv +
@@ -399,7 +401,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       const hipError_t e = hipGetLastError();
       if (e != hipSuccess) return hip_fail(e, name);
     }
-    if ((max_splits > 1 || epilogue) && (phases & 2u)) {
+    if ((max_splits > 1 || epilogue) && (phases & 2u) && !(epilogue && epilogue->partials_only)) {
       // One wave per row is all the sequential merge uses; the other three only
       // join in for lists longer than kMergeSequential.
       const uint32_t merge_threads = max_splits <= kMergeSequential ? 64 : 64 * kMergeWaves;

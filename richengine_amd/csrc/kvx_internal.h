@@ -81,9 +81,13 @@ __device__ inline Slab slab_of(uint32_t format, uint32_t kv_heads, uint32_t head
 // [(query | gate) x query heads, (key | value) x KV heads][D], each element is
 // first scaled by the sigmoid of its gate (the reduce/gate fusion,
 // decode/paged_attention.metal:266-309, 466-510).
+// With `partials_only` nothing is merged at all: every split writes its partial rows and
+// statistics, and the caller combines them (attention over a shared prefix merges the
+// prefix's splits with each sequence's own).
 struct Epilogue {
   const uint16_t *packed_qkv;
   uint16_t *hidden;
+  bool partials_only = false;
 };
 
 // ---- storage ----------------------------------------------------------------

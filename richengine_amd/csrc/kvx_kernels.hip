@@ -1025,6 +1025,147 @@ __global__ __launch_bounds__(256) void page_wire_kernel(WireArgs a) {
     if (o + i * 4096 < end) *reinterpret_cast<word4 *>(dst + o + i * 4096) = v[i];
 }
 
+// ============================================ attention over a shared prefix ====
+// Sequences whose page tables begin with the same pages: the prefix is attended
+// once, the sequences' one-row queries stacked as the rows of one lane, and each
+// sequence's own pages as a decode lane of its own; this merge then combines, per
+// sequence, KV head and query head, the partial rows of the prefix's splits and of
+// the sequence's splits: the maximum over all of them, then the weighted sums in
+// a fixed order (prefix splits in split order, then the sequence's), as
+// reduce_row does for one list.
+constexpr uint32_t kSharedLanes = KVX_TREE_NODES;
+constexpr uint32_t kSharedD = 256;  // the matrix-core kernels' head dimension
+typedef float vec4f __attribute__((ext_vector_type(4)));
+typedef uint32_t vec2u __attribute__((ext_vector_type(2)));
+struct SharedLane {
+  uint64_t base;     // first fused row of the sequence's own slots
+  uint32_t splits;   // its split count (the slot stride) and how many of them own a page
+  uint32_t written;
+};
+struct SharedArgs {
+  SharedLane lane[kSharedLanes];
+  const float *prefix_partials, *prefix_statistics;
+  const float *own_partials, *own_statistics;
+  uint32_t prefix_splits, prefix_written, prefix_rows;  // rows: fused rows of the prefix lane
+  uint32_t kv_heads, group, row_stride;
+};
+
+// Stacks the sequences' query rows as the rows of one lane, [kv head][sequence][g][D],
+// and clears the row masks of that lane (a row sees the committed prefix only).
+__global__ __launch_bounds__(256) void shared_stage_kernel(const uint16_t *__restrict__ queries,
+                                                           uint16_t *__restrict__ staged,
+                                                           uint32_t *__restrict__ masks, uint32_t lanes,
+                                                           uint32_t kv_heads, uint32_t group,
+                                                           uint32_t row_stride) {
+  const uint32_t lane = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
+  if (head == 0 && d == 0) masks[lane] = 0;
+  const uint64_t from = (uint64_t(lane) * kv_heads + head) * row_stride * group * kSharedD;
+  const uint64_t to = (uint64_t(head) * lanes + lane) * group * kSharedD;
+  for (uint32_t g = 0; g < group; ++g) staged[to + g * kSharedD + d] = queries[from + g * kSharedD + d];
+}
+
+// grid (query head in group, KV head, sequence), four waves, each lane four dimensions.
+// The two lists are walked as one: entry t is prefix split t, or the sequence's own
+// split t - prefix_written.  The entries are cut into four consecutive ranges, one per
+// wave; a wave fetches its statistics 64 entries at a time, one per lane, and its
+// partial rows eight at a time, so that the loads of a batch are in flight together,
+// and sums its range in entry order; the ranges are then added in range order, which
+// keeps the result a function of the inputs and the split counts alone.
+constexpr uint32_t kSharedWaves = 4;
+__global__ __launch_bounds__(64 * kSharedWaves) void shared_merge_kernel(uint16_t *__restrict__ output,
+                                                                         SharedArgs a) {
+  const uint32_t g = blockIdx.x, head = blockIdx.y, li = blockIdx.z;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const SharedLane l = a.lane[li];
+  const uint32_t G = a.group;
+  const uint64_t prefix_row = uint64_t(head) * a.prefix_splits * a.prefix_rows + li * G + g;
+  const uint64_t own_row = l.base + uint64_t(head) * l.splits * G + g;
+  const uint32_t entries = a.prefix_written + l.written;
+  const auto statistics_of = [&](uint32_t t) {
+    return t < a.prefix_written
+               ? a.prefix_statistics + (prefix_row + uint64_t(t) * a.prefix_rows) * 2
+               : a.own_statistics + (own_row + uint64_t(t - a.prefix_written) * G) * 2;
+  };
+  const auto partials_of = [&](uint32_t t) {
+    return t < a.prefix_written
+               ? a.prefix_partials + (prefix_row + uint64_t(t) * a.prefix_rows) * kSharedD
+               : a.own_partials + (own_row + uint64_t(t - a.prefix_written) * G) * kSharedD;
+  };
+  const uint32_t share = (entries + kSharedWaves - 1) / kSharedWaves;
+  const uint32_t first = min(entries, wave * share), last = min(entries, first + share);
+  // The statistics of all entries (for the maximum) and the wave's first sixteen partial
+  // rows are requested before anything waits; loads return in order, so the wait for
+  // the statistics leaves the rows in flight.
+  constexpr uint32_t kEarly = 16;
+  float early_max[2];
+#pragma unroll
+  for (uint32_t b = 0; b < 2; ++b)
+    early_max[b] = 64 * b + lane < entries ? statistics_of(64 * b + lane)[0] : -INFINITY;
+  vec4f early[kEarly];
+#pragma unroll
+  for (uint32_t u = 0; u < kEarly; ++u)
+    early[u] = *reinterpret_cast<const vec4f *>(partials_of(min(first + u, entries - 1)) + 4 * lane);
+  float maximum = fmaxf(early_max[0], early_max[1]);  // over all entries, by every wave
+  for (uint32_t base = 128; base < entries; base += 64)
+    maximum = fmaxf(maximum, base + lane < entries ? statistics_of(base + lane)[0] : -INFINITY);
+  for (int offset = 32; offset; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset));
+  vec4f numerator = {0.0f, 0.0f, 0.0f, 0.0f};
+  float denominator = 0.0f;
+  for (uint32_t base = first; base < last; base += 64) {
+    const uint32_t mine = base + lane, count = min(64u, last - base);
+    float my_max = -INFINITY, my_sum = 0.0f;
+    if (mine < last) {
+      const float *stat = statistics_of(mine);
+      my_max = stat[0];
+      my_sum = stat[1];
+    }
+    const float my_weight = expf(__fsub_rn(my_max, maximum));
+    const float my_term = __fmul_rn(my_weight, my_sum);
+    for (uint32_t i = 0; i < count; i += kEarly) {
+      vec4f part[kEarly];
+#pragma unroll
+      for (uint32_t u = 0; u < kEarly; ++u) {
+        if (base == first && i == 0)
+          part[u] = early[u];
+        else
+          part[u] = *reinterpret_cast<const vec4f *>(partials_of(base + min(i + u, count - 1)) + 4 * lane);
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < kEarly; ++u) {
+        if (i + u < count) {
+          const float weight = __shfl(my_weight, int(i + u));
+#pragma unroll
+          for (uint32_t c = 0; c < 4; ++c)
+            numerator[c] = __fadd_rn(numerator[c], __fmul_rn(weight, part[u][c]));
+          denominator = __fadd_rn(denominator, __shfl(my_term, int(i + u)));
+        }
+      }
+    }
+  }
+  __shared__ vec4f numerators[kSharedWaves][64];
+  __shared__ float denominators[kSharedWaves][64];
+  numerators[wave][lane] = numerator;
+  denominators[wave][lane] = denominator;
+  __syncthreads();
+  if (wave) return;
+#pragma unroll
+  for (uint32_t w = 1; w < kSharedWaves; ++w) {
+    const vec4f other = numerators[w][lane];
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) numerator[c] = __fadd_rn(numerator[c], other[c]);
+    denominator = __fadd_rn(denominator, denominators[w][lane]);
+  }
+  vec2u packed;
+#pragma unroll
+  for (uint32_t i = 0; i < 2; ++i) {
+    const float lo = denominator > 0.0f ? __fdiv_rn(numerator[2 * i], denominator) : 0.0f;
+    const float hi = denominator > 0.0f ? __fdiv_rn(numerator[2 * i + 1], denominator) : 0.0f;
+    packed[i] = uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
+  }
+  *reinterpret_cast<vec2u *>(output + (uint64_t(li) * a.kv_heads + head) * a.row_stride * G * kSharedD +
+                             uint64_t(g) * kSharedD + 4 * lane) = packed;
+}
+
 // ============================================================= launchers ====
 namespace {
 
@@ -1438,6 +1579,150 @@ int kv_attend_verify_hidden(const kvx_storage *s, uint32_t layer, uint32_t query
   return attend_verify("kv_attend_verify_hidden", s, layer, query_heads, queries, output,
                        page_tables, lanes, n_lanes, row_masks, row_stride, workspace,
                        workspace_bytes, &epilogue, stream);
+}
+
+namespace {
+uint64_t align256(uint64_t bytes) { return (bytes + 255) / 256 * 256; }
+// Bytes of one attend call's partials and statistics over `rows` slot rows.
+uint64_t slot_bytes(uint64_t rows, uint32_t head_dim) {
+  return align256(rows * head_dim * sizeof(float)) + rows * 2 * sizeof(float);
+}
+}  // namespace
+
+uint64_t kvx_attend_shared_workspace_bytes(const kvx_verify_params *lanes, uint32_t n_lanes,
+                                           uint32_t prefix_splits, uint32_t query_heads,
+                                           const kvx_layout *layout) {
+  if (!lanes || !layout || !n_lanes) return 0;
+  const uint64_t staged = align256(uint64_t(n_lanes) * query_heads * layout->head_dim * 2);
+  const uint64_t masks = 256;
+  const uint64_t prefix = align256(slot_bytes(uint64_t(prefix_splits) * n_lanes * query_heads, layout->head_dim));
+  uint64_t own_rows = 0;
+  for (uint32_t i = 0; i < n_lanes; ++i) own_rows += uint64_t(lanes[i].split_count) * query_heads;
+  return staged + masks + prefix + slot_bytes(own_rows, layout->head_dim);
+}
+
+int kv_attend_decode_shared(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
+                            const void *queries, void *output, const uint64_t *const *page_tables,
+                            const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t shared_pages,
+                            uint32_t prefix_splits, uint32_t row_stride, void *workspace,
+                            uint64_t workspace_bytes, void *stream) {
+  if (!s || !queries || !output || !page_tables || !lanes || !n_lanes || !workspace)
+    return fail(KVX_EINVAL, "kv_attend_decode_shared: null argument or no lanes");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
+  if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
+  kvx_kv_layer kv;
+  if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
+  const kvx_layout &l = s->layout;
+  const uint32_t H = l.kv_heads, D = l.head_dim;
+  if (!query_heads || query_heads % H)
+    return fail(KVX_EINVAL, "query heads are not a multiple of the KV heads");
+  const uint32_t G = query_heads / H;
+  if (D != 256 || G > 16 || l.format == KVX_FMT_FP8E4M3)
+    return fail(KVX_EINVAL, "shared-prefix attention covers head dimension 256, groups of at most "
+                            "16 query heads and int4, int8 or bf16 pages");
+  if (n_lanes > kSharedLanes || n_lanes * G > 128)
+    return fail(KVX_EINVAL, "too many sequences share the prefix for one call (16, and 128 fused rows)");
+  if (!shared_pages || !prefix_splits || prefix_splits > KVX_VERIFY_MAX_SPLITS || !row_stride)
+    return fail(KVX_EINVAL, "shared pages, prefix splits or row stride are out of range");
+  const uint64_t shared_tokens = uint64_t(shared_pages) * kPage;
+  std::vector<kvx_verify_params> own(n_lanes);
+  std::vector<const uint64_t *> own_tables(n_lanes);
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    const kvx_verify_params &p = lanes[i];
+    if (p.active_rows != 1 || p.row_capacity != 1)
+      return fail(KVX_EINVAL, "decode attends exactly one row per lane");
+    if (!page_tables[i]) return fail(KVX_EINVAL, "null page table");
+    if (p.committed_tokens < shared_tokens)
+      return fail(KVX_EINVAL, "a sequence's row lies inside the shared pages");
+    if (uint64_t(p.committed_tokens) + 1 > KVX_MAX_PHYSICAL_TOKENS)
+      return fail(KVX_EINVAL, "verify attention history exceeds physical context");
+    if (p.page_table_entries < (uint64_t(p.committed_tokens) + 1 + kPage - 1) / kPage)
+      return fail(KVX_EINVAL, "page_table_too_short");
+    if (!p.split_count || p.split_count > KVX_DECODE_MAX_SPLITS)
+      return fail(KVX_EINVAL, "verify split count is out of range");
+    if (p.score_scale != lanes[0].score_scale)
+      return fail(KVX_EINVAL, "sequences that share a prefix share the score scale");
+    own[i] = p;
+    own[i].committed_tokens = uint32_t(p.committed_tokens - shared_tokens);
+    own[i].page_table_entries = p.page_table_entries - shared_pages;
+    own_tables[i] = page_tables[i] + shared_pages;
+  }
+  if (workspace_bytes < kvx_attend_shared_workspace_bytes(lanes, n_lanes, prefix_splits, query_heads, &l))
+    return fail(KVX_EINVAL, "verify attention scratch is smaller than its bound");
+  // The prefix as one lane of n rows over the first sequence's table; its rows see
+  // the committed prefix only (masks of zero), so the one page past it, which the
+  // row slots would occupy, is read but never attended.
+  kvx_verify_params prefix{};
+  prefix.committed_tokens = uint32_t(shared_tokens);
+  prefix.page_table_entries = lanes[0].page_table_entries;
+  prefix.split_count = prefix.slot_splits = prefix_splits;
+  prefix.active_rows = prefix.row_capacity = n_lanes;
+  prefix.score_scale = lanes[0].score_scale;
+  // The matrix-core kernels stage one split's page entries in LDS, 1024 at most.
+  const auto split_fits = [](const kvx_verify_params &p) {
+    const uint32_t pages = (p.committed_tokens + p.active_rows + kPage - 1) / kPage;
+    return (pages + p.split_count - 1) / p.split_count <= 1024;
+  };
+  bool fits = split_fits(prefix);
+  for (uint32_t i = 0; i < n_lanes; ++i) fits = fits && split_fits(own[i]);
+  if (!fits) return fail(KVX_EINVAL, "a split is longer than 1024 pages: use more splits");
+
+  uint8_t *base = static_cast<uint8_t *>(workspace);
+  uint16_t *staged = reinterpret_cast<uint16_t *>(base);
+  base += align256(uint64_t(n_lanes) * query_heads * D * 2);
+  uint32_t *masks = reinterpret_cast<uint32_t *>(base);
+  base += 256;
+  void *prefix_space = base;
+  const uint64_t prefix_rows_total = uint64_t(prefix_splits) * H * n_lanes * G;
+  const uint64_t prefix_bytes = align256(slot_bytes(prefix_rows_total, D));
+  base += prefix_bytes;
+  void *own_space = base;
+  uint64_t own_rows_total = 0;
+  for (uint32_t i = 0; i < n_lanes; ++i) own_rows_total += uint64_t(own[i].split_count) * H * G;
+  const uint64_t own_bytes = slot_bytes(own_rows_total, D);
+
+  const hipStream_t st = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(shared_stage_kernel, dim3(n_lanes, H), dim3(D), 0, st,
+                     static_cast<const uint16_t *>(queries), staged, masks, n_lanes, H, G, row_stride);
+  if (int rc = check_launch("shared_stage_kernel")) return rc;
+  Epilogue partials{nullptr, nullptr, true};
+  const uint64_t *prefix_table[1] = {page_tables[0]};
+  int rc = took(attend_matrix(s, kv, query_heads, staged, nullptr, prefix_table, &prefix, 1, masks,
+                              n_lanes, uint64_t(H) * n_lanes * G * D, prefix_space, prefix_bytes, 0, st, 0,
+                              &partials));
+  if (rc) return rc < 0 ? rc : fail(KVX_EINVAL, "no matrix-core kernel covers the shared prefix");
+  rc = took(attend_matrix(s, kv, query_heads, queries, nullptr, own_tables.data(), own.data(), n_lanes,
+                          nullptr, row_stride, uint64_t(H) * row_stride * G * D, own_space, own_bytes, 0,
+                          st, 0, &partials));
+  if (rc) return rc < 0 ? rc : fail(KVX_EINVAL, "no matrix-core kernel covers the sequences' own pages");
+
+  SharedArgs a{};
+  a.prefix_partials = static_cast<const float *>(prefix_space);
+  a.prefix_statistics = reinterpret_cast<const float *>(static_cast<uint8_t *>(prefix_space) +
+                                                        align256(prefix_rows_total * D * sizeof(float)));
+  a.own_partials = static_cast<const float *>(own_space);
+  a.own_statistics = reinterpret_cast<const float *>(static_cast<uint8_t *>(own_space) +
+                                                     align256(own_rows_total * D * sizeof(float)));
+  const auto written_of = [](uint64_t tokens, uint32_t splits) {
+    const uint32_t pages = uint32_t((tokens + kPage - 1) / kPage);
+    const uint32_t per = (pages + splits - 1) / splits;
+    return (pages + per - 1) / per;
+  };
+  a.prefix_splits = prefix_splits;
+  a.prefix_written = written_of(shared_tokens + n_lanes, prefix_splits);
+  a.prefix_rows = n_lanes * G;
+  a.kv_heads = H;
+  a.group = G;
+  a.row_stride = row_stride;
+  uint64_t row_base = 0;
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    a.lane[i] = {row_base, own[i].split_count,
+                 written_of(uint64_t(own[i].committed_tokens) + 1, own[i].split_count)};
+    row_base += uint64_t(own[i].split_count) * H * G;
+  }
+  hipLaunchKernelGGL(shared_merge_kernel, dim3(G, H, n_lanes), dim3(64 * kSharedWaves), 0, st,
+                     static_cast<uint16_t *>(output), a);
+  return check_launch("shared_merge_kernel");
 }
 
 int kv_attend_decode(const kvx_storage *s, uint32_t layer, uint32_t query_heads,

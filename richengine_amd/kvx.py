@@ -34,7 +34,7 @@ SYMBOLS = [
     "kvx_storage_extent_write", "kv_page_copy", "kvx_pool_create", "kvx_pool_destroy",
     "kvx_pool_acquire", "kvx_pool_retain", "kvx_pool_release", "kvx_pool_page_active",
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
-    "kvx_pool_snapshot_get", "kv_append", "kv_prepare_append", "kv_attend_verify", "kv_attend_verify_hidden", "kv_attend_decode",
+    "kvx_pool_snapshot_get", "kv_append", "kv_prepare_append", "kv_attend_decode_shared", "kvx_attend_shared_workspace_bytes", "kv_attend_verify", "kv_attend_verify_hidden", "kv_attend_decode",
     "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kv_page_export", "kv_page_import", "kvx_debug_set_attend_phases",
     "kvx_debug_attend_paths", "kvx_decode_plan", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
@@ -214,6 +214,9 @@ def _declare(L):
     L.kv_attend_verify_hidden.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, vp, u32, vp, u64, vp, vp,
                                           vp]
     L.kv_attend_decode.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, u32, vp, u64, vp]
+    L.kv_attend_decode_shared.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, u32, u32, u32, vp, u64, vp]
+    L.kvx_attend_shared_workspace_bytes.argtypes = [vp, u32, u32, u32, C.POINTER(Layout)]
+    L.kvx_attend_shared_workspace_bytes.restype = u64
     L.kv_append_attend_decode.argtypes = [vp, u32, vp, vp, u64, u32, u32, vp, vp, vp, vp, u32, u32, vp,
                                           u64, vp]
     L.kv_attend_prefill.argtypes = [vp, u32, u32, vp, vp, vp, C.POINTER(PrefillParams), vp, u64, vp]
@@ -390,6 +393,22 @@ def attend_decode(storage, layer, query_heads, queries, output, tables, lanes, r
                                         _ptr(workspace),
                                         workspace.numel() * workspace.element_size(),
                                         _stream(stream)))
+
+
+def attend_shared_workspace_bytes(storage, lanes, prefix_splits, query_heads):
+    arr = (VerifyParams * len(lanes))(*lanes)
+    return lib().kvx_attend_shared_workspace_bytes(arr, len(lanes), prefix_splits, query_heads,
+                                                   C.byref(storage.layout))
+
+
+def attend_decode_shared(storage, layer, query_heads, queries, output, tables, lanes, shared_pages,
+                         prefix_splits, row_stride, workspace, stream=None):
+    """One-row decode of sequences whose tables begin with the same `shared_pages` pages."""
+    arr = (VerifyParams * len(lanes))(*lanes)
+    return check(lib().kv_attend_decode_shared(
+        storage.h, layer, query_heads, _ptr(queries), _ptr(output), _table_array(tables), arr,
+        len(lanes), shared_pages, prefix_splits, row_stride, _ptr(workspace),
+        workspace.numel() * workspace.element_size(), _stream(stream)))
 
 
 def append_attend_decode(storage, layer, chunk_keys, chunk_values, chunk_lane_stride, chunk_stride,
