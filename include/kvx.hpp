@@ -519,6 +519,24 @@ public:
                              buffers.pageTables, lanes.data(), plan.lanes, buffers.treeMasks,
                              kv::kVerifyChunkStride, buffers.workspace, buffers.workspaceBytes, stream));
   }
+  // One-row decode of up to 16 lanes whose page tables begin with the same sharedPages pages:
+  // those pages are attended once for all of them (no counterpart in the reference, which lists
+  // the case as a gap, docs/PERF_REPORT.md:250).  plan: a decode plan over the lanes' own tokens
+  // (history minus the shared tokens); prefixSplits: the verify plan of one lane of plan.lanes
+  // rows over the shared tokens.
+  static void attendShared(void *stream, const kv::PageStorage &storage, uint32_t layer,
+                           const PagedVerifyBuffers &buffers, const std::vector<kv::ChunkedPrefillParams> &chunks,
+                           const VerifyAttentionPlan &plan, uint32_t sharedPages, uint32_t prefixSplits) {
+    if (plan.rowCapacity != 1 || chunks.size() != plan.lanes)
+      throw std::invalid_argument("shared-prefix attention takes a decode plan, one chunk per lane");
+    std::vector<kv::VerifyAttentionParams> lanes(plan.lanes);
+    for (uint32_t i = 0; i < plan.lanes; ++i)
+      lanes[i] = {chunks[i].committed_tokens, chunks[i].page_table_entries, {}, plan.laneSplits[i],
+                  plan.splits, 1, 1, plan.scoreScale};
+    check(kv_attend_decode_shared(storage.handle(), layer, plan.queryHeads, buffers.queries, buffers.output,
+                                  buffers.pageTables, lanes.data(), plan.lanes, sharedPages, prefixSplits, 1,
+                                  buffers.workspace, buffers.workspaceBytes, stream));
+  }
   static void addVerifyTreeCompact(void *stream, const kv::PageStorage &storage, uint32_t layer,
                                    const uint64_t *const *pageTables, const uint32_t *retainedPath,
                                    const uint32_t *retained,
