@@ -170,7 +170,7 @@ def tree_verify(args):
     sequence (branching <= 3).  A step = per layer, append the 16 draft rows and
     run masked verify attention over history + rows; then compact a seeded
     root-to-leaf path of every sequence, all layers in one call.  The dominant
-    kernel (verify_int4_kernel) runs on the matrix cores; its line carries the
+    kernel (verify48_int4_kernel) runs on the matrix cores; its line carries the
     MFMA roofline (flops = 4 x D x fused query rows x visible tokens per layer)."""
     import numpy as np
     import torch
@@ -278,7 +278,7 @@ def tree_verify(args):
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": None,
-                     "kernel": "verify_int4_kernel (split kernel of verify attention), one layer per launch",
+                     "kernel": "verify48_int4_kernel (split kernel of verify attention, 48 fused rows per wave), one layer per launch",
                      "flops_per_launch": flops, "ms_per_launch": round(kernel_ms, 4),
                      "kv_gbs": round(kv_bytes / (kernel_ms * 1e-3) / 1e9, 1)},
         "cpu_baseline": None,
@@ -419,7 +419,7 @@ def shared_prefix(args):
     committed = [shared_pages * 32 + t for t in own]
     queries = torch.randn((lanes, H, 1, G, D), generator=gen, device="cuda").bfloat16()
     output = torch.zeros_like(queries)
-    prefix_splits = args.verify_splits or kvx.verify_plan([shared_pages * 32], lanes, H, QH)[0]
+    prefix_splits = args.verify_splits or kvx.verify_plan([shared_pages * 32], lanes, H, QH, fmt)[0]
     own_splits = kvx.decode_plan(own, H, fmt)
     sp = [kvx.VerifyParams(committed[i], entries[i], kvx.KvLayer(), own_splits[i], own_splits[i], 1, 1, 0.0)
           for i in range(lanes)]

@@ -168,11 +168,13 @@ int kvx_decode_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t
    the reference's clamp(ceil(pages/16), 32, 128): the longest split length (at least 8 pages)
    for which the launch has no more waves than the GPU has SIMDs (1024), each lane getting
    clamp(ceil(its pages / that), 1, KVX_VERIFY_MAX_SPLITS).  A launch runs (sum of splits) x
-   KV heads x ceil(rows x group / 32) waves, one per SIMD.  No counterpart in the reference
+   KV heads x ceil(rows x group / 32) waves, one per SIMD; on int4 pages ceil(rows x group / 48)
+   where that is fewer by more than two fifths (33 .. 48 and 65 .. 96 fused rows among others).  No counterpart in the reference
    (its rule is kvx_verify_splits); any split count either rule gives is valid for
    kv_attend_verify. */
 int kvx_verify_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t rows,
-                    uint32_t kv_heads, uint32_t query_heads, uint32_t *split_counts);
+                    uint32_t kv_heads, uint32_t query_heads, uint32_t format,
+                    uint32_t *split_counts);
 /* kv::chunkedPrefillValidationError: 0 ok, 1 chunk_tokens_out_of_range,
    2 context_out_of_range, 3 chunk_stride_invalid, 4 page_table_too_short */
 int kvx_chunk_validation(const kvx_chunk_params *params);

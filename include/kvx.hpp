@@ -367,7 +367,7 @@ public:
       check(decode ? kvx_decode_plan(historyTokens.data(), lanes, layout.kvHeads,
                                      static_cast<uint32_t>(layout.format), plan.laneSplits.data())
                    : kvx_verify_plan(historyTokens.data(), lanes, rows, layout.kvHeads, queryHeads,
-                                     plan.laneSplits.data()));
+                                     static_cast<uint32_t>(layout.format), plan.laneSplits.data()));
       for (uint32_t splits : plan.laneSplits) plan.splits = std::max(plan.splits, splits);
     } else {
       for (uint32_t history : historyTokens) {

@@ -347,6 +347,9 @@ __device__ __forceinline__ void append_decode_token(const DecodeArgs &a, const D
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+#ifndef KVX_V48_DEPTH
+#define KVX_V48_DEPTH 1
+#endif
 #ifndef KVX_DECODE_DEPTH
 #define KVX_DECODE_DEPTH 2
 #endif
@@ -647,6 +650,15 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   attend_int4<2, 1>(queries, output, partials, statistics, a);
 }
 
+// Three blocks (48 fused rows: a chain of 8 rows for a group of 6 query heads, half
+// of a 16-node tree) read and expand every page once for all of them; one register set of pages,
+// one wave per SIMD.
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void verify48_int4_kernel(
+    const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
+    float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
+  attend_int4<3, KVX_V48_DEPTH>(queries, output, partials, statistics, a);
+}
+
 }  // namespace
 }  // namespace kvx
 
@@ -687,6 +699,15 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
                                    kvx_attend_phases(), stream, nullptr, tile_rows, epilogue);
+#ifndef KVX_NO_V48
+  // 48 fused rows per wave where that leaves clearly fewer waves: the pages are
+  // read and expanded once per 48 rows instead of once per 32.
+  if (verify_block_rows(KVX_FMT_INT4, fused_rows) == 48 && !many_tiles)
+    return launch_matrix_attention(verify48_int4_kernel, "verify48_int4_kernel", 48, 64, s, kv,
+                                   query_heads, queries, output, page_tables, lanes, n_lanes,
+                                   row_masks, row_stride, lane_stride, workspace, workspace_bytes,
+                                   kvx_attend_phases(), stream, nullptr, tile_rows, epilogue);
+#endif
   if (fused_rows > 16 && !many_tiles)
     return launch_matrix_attention(verify_int4_kernel, "verify_int4_kernel", 32, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,

@@ -196,19 +196,19 @@ int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_hea
   return KVX_OK;
 }
 int kvx_verify_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t rows, uint32_t kv_heads,
-                    uint32_t query_heads, uint32_t *split_counts) {
+                    uint32_t query_heads, uint32_t format, uint32_t *split_counts) {
   if (!committed || !split_counts || !n_lanes || !kv_heads || !rows || !query_heads ||
       query_heads % kv_heads)
     return fail(KVX_EINVAL, "kvx_verify_plan: null argument, empty batch or bad head counts");
-  // The verify kernels keep 32 fused rows (16 when there are no more) per wave and
-  // run one wave per SIMD, so a launch is (sum of splits) x KV heads x row blocks
+  // The verify kernels keep 32 fused rows (16 when there are no more; all of 33 .. 48
+  // on int4 pages) per wave and run one wave per SIMD, so a launch is (sum of splits) x KV heads x row blocks
   // waves: the plan is the longest split length that still gives every SIMD of
   // 256 CUs x 4 a wave, but no more waves than SIMDs, so that no second round of
   // waves starts on a nearly empty GPU; splits shorter than 8 pages cost more in
   // set-up and partial rows than they win.
   constexpr uint64_t kSimds = 1024;
   const uint32_t fused = rows * (query_heads / kv_heads);
-  const uint32_t blocks = fused > 16 ? (fused + 31) / 32 : 1;
+  const uint32_t blocks = kvx::verify_row_blocks(format, fused);
   uint64_t page_waves = 0;
   for (uint32_t i = 0; i < n_lanes; ++i)
     page_waves += uint64_t(pages_of(uint64_t(committed[i]) + rows)) * kv_heads * blocks;

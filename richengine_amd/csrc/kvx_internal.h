@@ -107,6 +107,25 @@ struct Storage {
   uint32_t allocated_extents() const;
 };
 
+// Fused query rows one wave of a verify launch covers: the matrix-core kernels
+// hold 32 per wave (16 when there are no more); the int4 kernels also have a
+// 48-row form, which reads and expands every page once for all three blocks of
+// 16 and costs about 1.4 waves of the 32-row form.  It is used where it leaves
+// fewer waves by more than that.
+inline uint32_t verify_block_rows(uint32_t format, uint32_t fused_rows) {
+  if (fused_rows <= 16) return 16;
+#ifndef KVX_NO_V48
+  const uint32_t by32 = (fused_rows + 31) / 32, by48 = (fused_rows + 47) / 48;
+  if (format == KVX_FMT_INT4 && 7 * by48 < 5 * by32) return 48;
+#endif
+  return 32;
+}
+// Waves (row blocks) per (lane, split, KV head) of a verify launch.
+inline uint32_t verify_row_blocks(uint32_t format, uint32_t fused_rows) {
+  const uint32_t rows = verify_block_rows(format, fused_rows);
+  return (fused_rows + rows - 1) / rows;
+}
+
 }  // namespace kvx
 
 struct kvx_storage : kvx::Storage {};

@@ -173,7 +173,7 @@ def _declare(L):
     L.kvx_sequences_compact_extent.argtypes = [vp, PU32, vp, PU32, vp]
     L.kvx_debug_attend_paths.argtypes, L.kvx_debug_attend_paths.restype = [PU64, PU64], None
     L.kvx_decode_plan.argtypes = [vp, u32, u32, u32, vp]
-    L.kvx_verify_plan.argtypes = [vp, u32, u32, u32, u32, vp]
+    L.kvx_verify_plan.argtypes = [vp, u32, u32, u32, u32, u32, vp]
     L.kvx_tree_masks.argtypes = [vp, u32, vp]
     L.kvx_tree_path_valid.argtypes = [vp, u32, vp, u32]
     L.kvx_storage_destroy.argtypes = [vp]
@@ -636,10 +636,10 @@ def decode_plan(committed, kv_heads, fmt=INT4):
     return list(out)
 
 
-def verify_plan(committed, rows, kv_heads, query_heads):
+def verify_plan(committed, rows, kv_heads, query_heads, fmt=INT4):
     """Split counts of a verify batch sized for the GPU (kvx_verify_plan)."""
     out = (C.c_uint32 * len(committed))()
-    check(lib().kvx_verify_plan(_u32(committed), len(committed), rows, kv_heads, query_heads, out))
+    check(lib().kvx_verify_plan(_u32(committed), len(committed), rows, kv_heads, query_heads, fmt, out))
     return list(out)
 
 

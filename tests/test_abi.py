@@ -127,9 +127,12 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
                     break
                 per += 1
             assert plan == want
-        for rows in (2, 8, 16):
-            plan = kvx.verify_plan(committed, rows, H, QH)
-            blocks = -(-rows * (QH // H) // 32) if rows * (QH // H) > 16 else 1
+        for rows, fmt in ((2, kvx.INT4), (8, kvx.INT4), (8, kvx.INT8), (16, kvx.INT4), (16, kvx.BF16)):
+            plan = kvx.verify_plan(committed, rows, H, QH, fmt)
+            fused = rows * (QH // H)
+            blocks = -(-fused // 32) if fused > 16 else 1
+            if fmt == kvx.INT4 and fused > 16 and 7 * -(-fused // 48) < 5 * -(-fused // 32):
+                blocks = -(-fused // 48)  # the int4 kernel for 48 fused rows per wave
             counts = [pages(c + rows) for c in committed]
             per = max(-(-sum(counts) * H * blocks // 1024), 8)
             while True:  # the rule, restated: the first length that fits one round of waves
@@ -139,7 +142,8 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
                 per += 1
             assert plan == want
             assert all(1 <= s <= 128 and s <= max(n, 1) for s, n in zip(plan, counts))
-    assert kvx.verify_plan([65536] * 4, 16, H, QH) == [21] * 4
+    assert kvx.verify_plan([65536] * 4, 16, H, QH) == [32] * 4          # two waves of 48 fused rows
+    assert kvx.verify_plan([65536] * 4, 16, H, QH, kvx.BF16) == [21] * 4  # three of 32
     with pytest.raises(kvx.KvxError):
         kvx.verify_plan([10], 8, 4, 6)
 

@@ -246,6 +246,45 @@ def test_tree_verify_matches_oracle(fmt, nodes):
     tw.close()
 
 
+@pytest.mark.parametrize("nodes,capacity", [(7, 7), (5, 8)])
+def test_int4_small_tree_verify_in_one_wave(nodes, capacity):
+    # capacity x group = 42 or 48 fused rows: the int4 kernel that keeps three
+    # blocks of 16 fused rows in one wave, with ancestor masks and, for capacity 7,
+    # a last block that is only partly in the tile
+    fmt = ko.INT4
+    committed = [260, 31, 4000, 0]
+    lanes = len(committed)
+    tw, counts, hts, dts = shared_pool_lanes(fmt, committed, nodes, seed=90 + nodes)
+    rng = np.random.default_rng(nodes)
+    masks = np.zeros((lanes, capacity), dtype=np.uint32)
+    for lane in range(lanes):
+        parents = [-1] + [int(rng.integers(max(0, i - 3), i)) for i in range(1, nodes)]
+        masks[lane, :nodes] = tree_masks(parents)
+    q = np.zeros((lanes, H, 32, G, D), dtype=np.uint16)
+    q[:, :, :capacity] = queries((lanes, H, capacity, G, D), 9)
+    splits = kvx.verify_plan(committed, nodes, H, QH, fmt)
+    splits = [max(s, 2) if c > 64 else s for s, c in zip(splits, committed)]  # merged and single-split lanes
+    hp = [ko.VerifyParams(committed[i], counts[i], tw.host.layer(1), splits[i], 128, nodes, capacity, 0.0)
+          for i in range(lanes)]
+    n, want, want32 = ko.attend_verify(fmt, H, G, D, q, hts, hp, masks)
+    assert n == lanes
+    dp = [kvx.VerifyParams(committed[i], counts[i], kvx.KvLayer(), splits[i], 128, nodes, capacity, 0.0)
+          for i in range(lanes)]
+    out = torch.full((lanes, H, 32, G, D), 0x5A5A, dtype=torch.int16, device="cuda")
+    ws = torch.empty(kvx.attend_workspace_bytes(tw.dev, dp, QH), dtype=torch.uint8, device="cuda")
+    before = kvx.attend_paths()
+    kvx.attend_verify(tw.dev, 1, QH, Gp.dev(q), out, dts, dp, Gp.dev(masks), 32, ws)
+    torch.cuda.synchronize()
+    after = kvx.attend_paths()
+    assert after[1] == before[1] + 1 and after[0] == before[0]  # a matrix-core launch
+    got = Gp.host_u16(out)
+    live = np.zeros((lanes, H, 32), dtype=bool)
+    live[:, :, :nodes] = True
+    Gp.check_attention(got, want, want32, live, tol(fmt), "small tree verify", matrix_core=True)
+    assert not got[:, :, nodes:capacity].any() and (got[:, :, capacity:] == 0x5A5A).all()
+    tw.close()
+
+
 def decode_case(fmt, committed, seed, row_stride=1, layers=2, layer=1):
     lanes = len(committed)
     tw, counts, hts, dts = shared_pool_lanes(fmt, committed, 1, seed=seed, layers=layers, layer=layer)
