@@ -64,6 +64,9 @@ def parse():
                     help="decode: the step's queries, keys and values come from packed projection rows "
                          "through kv_prepare_append (norm, rotation, quantize, store) instead of "
                          "ready chunk rows through kv_append; implies --separate-append")
+    ap.add_argument("--prefill-streams", type=int, default=4,
+                    help="prefill: HIP streams the batch's sequences are spread over (1 = all on the "
+                         "current stream); a sequence's layers stay in order on its stream")
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
     ap.add_argument("--workload", choices=["decode", "tree-verify", "prefill", "qkv-prepare", "shared-prefix"], default="decode",
@@ -517,19 +520,32 @@ def chunked_prefill(args):
     chunk_k = [rows((H, chunk, D)) for _ in range(sequences)]
     chunk_v = [rows((H, D, chunk)) for _ in range(sequences)]
     queries = [rows((H, chunk, G, D)) for _ in range(sequences)]
-    output = torch.zeros_like(queries[0])
+    # One stream, output and workspace per sequence: the sequences of a batch are
+    # independent, and the 1536 waves of one sequence's launch leave half of the
+    # SIMDs idle in their second round on the formats that run one wave per SIMD.
+    # Launches of other sequences on other streams fill that round.
+    n_streams = max(1, min(args.prefill_streams, sequences))
+    streams = [torch.cuda.Stream() for _ in range(n_streams)] if n_streams > 1 else [None]
+    outputs = [torch.zeros_like(queries[0]) for _ in range(n_streams)]
+    output = outputs[0]
     splits = L.kvx_prefill_splits(chunk)
     cp = kvx.ChunkParams(prefix, chunk, chunk, entries)
     pp = kvx.PrefillParams(prefix, chunk, chunk, entries, kvx.KvLayer(), splits, 0.0)
-    workspace = torch.empty(kvx.prefill_workspace_bytes(storage, chunk, QH) + 4096, dtype=torch.uint8,
-                            device="cuda")
+    workspaces = [torch.empty(kvx.prefill_workspace_bytes(storage, chunk, QH) + 4096, dtype=torch.uint8,
+                              device="cuda") for _ in range(n_streams)]
+    workspace = workspaces[0]
     torch.cuda.synchronize()
 
     def step():
+        # a sequence's layers follow one another on its stream, as they do in a model
         for layer in range(LAYERS):
             for s in range(sequences):
-                kvx.append(storage, layer, chunk_k[s], chunk_v[s], [tables[s]], [cp], H * chunk * D)
-                kvx.attend_prefill(storage, layer, QH, queries[s], output, tables[s], pp, workspace)
+                lane = s % n_streams
+                handle = streams[lane].cuda_stream if streams[lane] is not None else None
+                kvx.append(storage, layer, chunk_k[s], chunk_v[s], [tables[s]], [cp], H * chunk * D,
+                           stream=handle)
+                kvx.attend_prefill(storage, layer, QH, queries[s], outputs[lane], tables[s], pp,
+                                   workspaces[lane], stream=handle)
 
     steps, warmup = min(args.steps, 5), min(args.warmup, 1)
     for _ in range(warmup):
@@ -565,10 +581,10 @@ def chunked_prefill(args):
                                "2048-row chunks over 16384 + 2048 tokens, 16 layers: quantize + scatter "
                                "of the chunk, then causal attention per layer and sequence",
                    "batch": sequences, "layers": LAYERS, "format": args.format, "splits": int(splits),
-                   "seed": args.seed},
+                   "streams": n_streams, "seed": args.seed},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": None,
-                     "kernel": "split kernel of kv_attend_prefill (verify_int4_kernel or "
+                     "kernel": "split kernel of kv_attend_prefill (prefill_int4_kernel or "
                                "attend_wide_kernel), one sequence and layer per launch",
                      "flops_per_launch": flops, "ms_per_launch": round(kernel_ms, 4)},
         "cpu_baseline": None,

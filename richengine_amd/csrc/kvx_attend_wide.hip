@@ -126,7 +126,7 @@ __device__ __forceinline__ PagePlace place_page(uint64_t entry, uint32_t head, u
   return p;
 }
 
-template <uint32_t FMT>
+template <uint32_t FMT, bool REUSED>
 __device__ __forceinline__ void load_keys(KeyRegs<FMT> &k, const PagePlace &p, uint32_t t,
                                           uint32_t g) {
   constexpr uint32_t B = Wide<FMT>::kBytes;
@@ -136,7 +136,7 @@ __device__ __forceinline__ void load_keys(KeyRegs<FMT> &k, const PagePlace &p, u
     if constexpr (Wide<FMT>::kByte) {
 #pragma unroll
       for (uint32_t j = 0; j < 4; ++j) {  // 16 tokens x 64 contiguous bytes per instruction
-        const u32x4 v = load_streaming<u32x4>(row + 64 * j + 16 * g);
+        const u32x4 v = load_streaming<u32x4, REUSED>(row + 64 * j + 16 * g);
         k.raw[tb][2 * j][0] = v[0];
         k.raw[tb][2 * j][1] = v[1];
         k.raw[tb][2 * j + 1][0] = v[2];
@@ -145,14 +145,14 @@ __device__ __forceinline__ void load_keys(KeyRegs<FMT> &k, const PagePlace &p, u
     } else {
 #pragma unroll
       for (uint32_t kb = 0; kb < 8; ++kb) {
-        const u32x4 v = load_streaming<u32x4>(row + key_dims<FMT>(kb, g) * B);
+        const u32x4 v = load_streaming<u32x4, REUSED>(row + key_dims<FMT>(kb, g) * B);
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) k.raw[tb][kb][i] = v[i];
       }
     }
   }
 }
-template <uint32_t FMT>
+template <uint32_t FMT, bool REUSED>
 __device__ __forceinline__ void load_values(ValueRegs<FMT> &v, const PagePlace &p, uint32_t t,
                                             uint32_t g) {
   constexpr uint32_t B = Wide<FMT>::kBytes;
@@ -160,11 +160,11 @@ __device__ __forceinline__ void load_values(ValueRegs<FMT> &v, const PagePlace &
   for (uint32_t mb = 0; mb < 16; ++mb) {  // 16 dims x 32 tokens, contiguous, per instruction
     const uint8_t *at = p.values + ((16 * mb + t) * kPage + 8 * g) * B;
     if constexpr (Wide<FMT>::kByte) {
-      const u32x2 x = load_streaming<u32x2>(at);
+      const u32x2 x = load_streaming<u32x2, REUSED>(at);
       v.raw[mb][0] = x[0];
       v.raw[mb][1] = x[1];
     } else {
-      const u32x4 x = load_streaming<u32x4>(at);
+      const u32x4 x = load_streaming<u32x4, REUSED>(at);
 #pragma unroll
       for (uint32_t i = 0; i < 4; ++i) v.raw[mb][i] = x[i];
     }
@@ -184,7 +184,7 @@ __device__ __forceinline__ u32x4 value_operand(const ValueRegs<FMT> &v, uint32_t
 }
 
 // WAVES: waves per SIMD the kernel is compiled for (1 or 2).
-template <uint32_t FMT, uint32_t NB, uint32_t WAVES>
+template <uint32_t FMT, uint32_t NB, uint32_t WAVES, bool REUSED>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) void attend_wide_kernel(const uint16_t *__restrict__ queries,
                                                          uint16_t *__restrict__ output,
                                                          float *__restrict__ partials,
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
   auto fetch_keys = [&](PageSet &r, uint32_t slot) {
     const PagePlace p = place_page<FMT>(table_lds[slot], head, H, a.kv.offset, ro);
     asm volatile("");
-    load_keys<FMT>(r.keys, p, t, g);
+    load_keys<FMT, REUSED>(r.keys, p, t, g);
     if constexpr (kByte) {
       r.ks[0] = load_global<f32x4>(p.key_scales + 8 * g);
       r.ks[1] = load_global<f32x4>(p.key_scales + 8 * g + 4);
@@ -289,7 +289,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
   auto fetch_values = [&](PageSet &r, uint32_t slot) {
     const PagePlace p = place_page<FMT>(table_lds[slot], head, H, a.kv.offset, ro);
     asm volatile("");
-    load_values<FMT>(r.values, p, t, g);
+    load_values<FMT, REUSED>(r.values, p, t, g);
     if constexpr (kByte) {
       r.vs[0] = load_global<f32x4>(p.value_scales + 8 * g);
       r.vs[1] = load_global<f32x4>(p.value_scales + 8 * g + 4);
@@ -497,8 +497,8 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
     return 1;
   const uint32_t M = lanes[0].row_capacity * (query_heads / s->layout.kv_heads);
   const uint32_t phases = kvx_attend_phases();
-#define KVX_WIDE(FMT, NB, WAVES)                                                                 \
-  launch_matrix_attention(attend_wide_kernel<FMT, NB, WAVES>, "attend_wide_kernel", 16 * NB, 64, s, \
+#define KVX_WIDE(FMT, NB, WAVES, REUSED)                                                         \
+  launch_matrix_attention(attend_wide_kernel<FMT, NB, WAVES, REUSED>, "attend_wide_kernel", 16 * NB, 64, s, \
                           kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks, \
                           row_stride, lane_stride, workspace, workspace_bytes, phases, stream,      \
                           nullptr, tile_rows, epilogue)
@@ -508,10 +508,19 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   // tiles of a prefill with several splits); with two blocks the accumulators
   // leave too little room for that (the compiler spills inside the page loop:
   // int8 prefill 2.9 -> 4.5 ms), so those keep the SIMD to themselves.
-  if (format == KVX_FMT_BF16)
-    return M > 16 ? KVX_WIDE(KVX_FMT_BF16, 2, 1) : KVX_WIDE(KVX_FMT_BF16, 1, 1);
+  // The regular tiles of a chunked prefill (tile_rows > 0) walk the same pages
+  // over and over: their loads may stay in the caches.
+  const bool reused = tile_rows > 0;
+  if (format == KVX_FMT_BF16) {
+    if (M > 16) return reused ? KVX_WIDE(KVX_FMT_BF16, 2, 1, true) : KVX_WIDE(KVX_FMT_BF16, 2, 1, false);
+    return KVX_WIDE(KVX_FMT_BF16, 1, 1, false);
+  }
   const bool two_blocks = M > 16 && !many_tiles;
-  if (format == KVX_FMT_INT8) return two_blocks ? KVX_WIDE(KVX_FMT_INT8, 2, 1) : KVX_WIDE(KVX_FMT_INT8, 1, 2);
-  return two_blocks ? KVX_WIDE(KVX_FMT_FP8E4M3, 2, 1) : KVX_WIDE(KVX_FMT_FP8E4M3, 1, 2);
+  if (format == KVX_FMT_INT8) {
+    if (two_blocks) return reused ? KVX_WIDE(KVX_FMT_INT8, 2, 1, true) : KVX_WIDE(KVX_FMT_INT8, 2, 1, false);
+    return KVX_WIDE(KVX_FMT_INT8, 1, 2, false);
+  }
+  if (two_blocks) return reused ? KVX_WIDE(KVX_FMT_FP8E4M3, 2, 1, true) : KVX_WIDE(KVX_FMT_FP8E4M3, 2, 1, false);
+  return KVX_WIDE(KVX_FMT_FP8E4M3, 1, 2, false);
 #undef KVX_WIDE
 }

@@ -63,7 +63,7 @@ __device__ __forceinline__ LaneOffsets lane_offsets(uint32_t t, uint32_t g, uint
 }
 
 // PARTS: bit 0 the keys, bit 1 values and both scale lines.
-template <uint32_t PARTS>
+template <uint32_t PARTS, bool REUSED>
 __device__ __forceinline__ void load_page(PageRegs &r, uint64_t entry, uint32_t head,
                                           uint32_t kv_heads, uint32_t layer_offset,
                                           uint64_t key_scales_off, uint64_t values_off,
@@ -83,13 +83,13 @@ __device__ __forceinline__ void load_page(PageRegs &r, uint64_t entry, uint32_t 
 #pragma unroll
       for (uint32_t half = 0; half < 2; ++half)
         r.k[tb * 2 + half] =
-            load_streaming<u32x4>(keys + at.keys + (16 * tb * kRowBytes + 64 * half));
+            load_streaming<u32x4, REUSED>(keys + at.keys + (16 * tb * kRowBytes + 64 * half));
   }
   if constexpr (PARTS & 2u) {
     const uint8_t *values = keys + values_off;
 #pragma unroll
     for (uint32_t s = 0; s < 8; ++s)
-      r.v[s] = load_streaming<u32x2>(values + at.values + ((s < 4 ? 0 : 16) + (s & 3)) * kRowBytes);
+      r.v[s] = load_streaming<u32x2, REUSED>(values + at.values + ((s < 4 ? 0 : 16) + (s & 3)) * kRowBytes);
     // One scale per lane instead of the sixteen a lane multiplies with: they
     // are fetched from the owning lanes when the page is attended, which keeps
     // a register set at 33 registers.
@@ -421,7 +421,7 @@ __device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m,
 
 // The split kernel's body for NB blocks of 16 fused query rows per wave, with
 // kDepth register sets of pages.
-template <uint32_t NB, uint32_t kDepth>
+template <uint32_t NB, uint32_t kDepth, bool kReused = false>
 __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries,
                                             uint16_t *__restrict__ output,
                                             float *__restrict__ partials,
@@ -509,7 +509,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     // second copy of its registers, and interleaved with another fill's loads
     // they would make every wait cover both.
     asm volatile("");
-    load_page<3>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
+    load_page<3, kReused>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
   // The same in two steps for the steady loop: the keys as soon as the page that
@@ -519,7 +519,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     slot = 0;
 #endif
     asm volatile("");
-    load_page<1>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
+    load_page<1, kReused>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
   auto fill_rest = [&](PageRegs &set, uint32_t slot) {
@@ -527,7 +527,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     slot = 0;
 #endif
     asm volatile("");
-    load_page<2>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
+    load_page<2, kReused>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
   // The first fills are unconditional too (a split shorter than kDepth pages
@@ -641,13 +641,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
 // The same two blocks with one register set of pages, which fits two waves per
 // SIMD: for the paired tiles of a chunked prefill, whose 1536 waves per 2048-row
 // chunk then all run at once instead of in a full round and a half-empty one
-// (2.0 -> 1.5 ms on 2048 rows over 16K tokens).  Verify batches, sized to one
+// (2.0 -> 1.5 ms on 2048 rows over 16K tokens); its page loads may stay in the
+// caches, because every tile of the chunk walks the same pages.  Verify batches, sized to one
 // wave per SIMD by their plan, are faster with two sets and the SIMD to
 // themselves.
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_int4_kernel(
     const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
     float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
-  attend_int4<2, 1>(queries, output, partials, statistics, a);
+  attend_int4<2, 1, true>(queries, output, partials, statistics, a);
 }
 
 // Three blocks (48 fused rows: a chain of 8 rows for a group of 6 query heads, half

@@ -167,10 +167,12 @@ def test_hot_kernels_stay_out_of_scratch_memory():
         return report[names[0]]
 
     for fragment in ("decode_int4_kernel", "verify_int4_kernel", "matrix_merge_kernel",
-                     "attend_wide_kernelILj1ELj1ELj2E",    # int8, one block, two waves per SIMD
-                     "attend_wide_kernelILj4ELj1ELj2E",    # fp8
-                     "attend_wide_kernelILj2ELj1ELj1E",    # bf16 decode
-                     "attend_wide_kernelILj1ELj2ELj1E", "attend_wide_kernelILj4ELj2ELj1E"):
+                     "attend_wide_kernelILj1ELj1ELj2ELb0E",    # int8, one block, two waves per SIMD
+                     "attend_wide_kernelILj4ELj1ELj2ELb0E",    # fp8
+                     "attend_wide_kernelILj2ELj1ELj1ELb0E",    # bf16 decode
+                     "attend_wide_kernelILj1ELj2ELj1ELb0E", "attend_wide_kernelILj4ELj2ELj1ELb0E",
+                     # the same two with page loads that may stay in the caches (prefill tiles)
+                     "attend_wide_kernelILj1ELj2ELj1ELb1E", "attend_wide_kernelILj4ELj2ELj1ELb1E"):
         r = one(fragment)
         assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, (fragment, r)
     assert one("decode_int4_kernel")["occupancy"] == 2
