@@ -13,11 +13,10 @@
 // scale rounded to bf16 (bf16 pages) or fp16 (fp8 pages, whose queries are
 // staged as fp16) before they meet the values.
 //
-// fp8 -> fp16 without a table: an e4m3 byte s.eeee.mmm placed at bits 14..7 of a
-// half (sign moved to bit 15) is the fp16 number 2^-8 times the e4m3 value,
-// subnormals included, because both formats then share mantissa alignment and
-// differ by the bias 15 - 7.  The factor 2^8 is applied in fp32, where it is
-// exact (to the scores with the key scale, to the accumulators at the end).
+// fp8 -> fp16: gfx950 converts two e4m3 (OCP) bytes to two halves in one
+// instruction (v_cvt_scalef32_pk_f16_fp8); every e4m3 value, subnormals included,
+// is a normal fp16 number, so the conversion is exact (half a VALU instruction per
+// byte; a shift-and-mask construction of the same halves took 2.5).
 //
 // int8 -> fp16 without a table: the code's byte with its top bit flipped is
 // u = c + 128 in 1..255, 0x6400 | u is the fp16 number 1024 + u exactly, and a
@@ -53,16 +52,16 @@ __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-// Two e4m3 bytes (bytes `lo` and `hi` of x, selected by the perm pattern) to
-// two fp16 halves worth 2^-8 of their values.
-__device__ __forceinline__ uint32_t fp8_pair(uint32_t x, uint32_t select) {
-  const uint32_t y = __builtin_amdgcn_perm(0u, x, select);  // 0x00bb00aa
-  return ((y << 8) & 0x80008000u) | ((y << 7) & 0x3F803F80u);
+// Two e4m3 bytes (the low or the high half of x) to two fp16 halves holding their
+// values: one v_cvt_scalef32_pk_f16_fp8 with scale 1.
+template <bool HIGH>
+__device__ __forceinline__ uint32_t fp8_pair(uint32_t x) {
+  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(x, 1.0f, HIGH));
 }
 // Eight consecutive bytes (two dwords) to eight fp16 in order.
 __device__ __forceinline__ u32x4 fp8_operand(uint32_t first, uint32_t second) {
-  return u32x4{fp8_pair(first, 0x0c010c00u), fp8_pair(first, 0x0c030c02u),
-               fp8_pair(second, 0x0c010c00u), fp8_pair(second, 0x0c030c02u)};
+  return u32x4{fp8_pair<false>(first), fp8_pair<true>(first), fp8_pair<false>(second),
+               fp8_pair<true>(second)};
 }
 
 // Two int8 codes (bytes of x flipped in the top bit, selected by the perm
@@ -314,8 +313,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
     row_max[nb] = -INFINITY;
     row_sum[nb] = 0.0f;
   }
-  // fp8 operands are worth 2^-8 of their values; see the head of this file.
-  constexpr float kUnscale = kFp8 ? 256.0f : 1.0f;
+  constexpr float kUnscale = 1.0f;  // every format's MFMA operands hold the values themselves
 
   // One page out of set r; keys_consumed() runs when its keys have been read for
   // the last time.
