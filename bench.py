@@ -25,6 +25,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# Kernel arguments in device memory rather than in host memory (HIP reads this when
+# its runtime starts, which is after this line): every wave of the attention
+# kernels finds its sequence in a 1.9 KB argument block, and fetching that from
+# the host costs the merge kernel 2 us and a decode step 3 % (1.96 -> 1.89 ms).
+# A caller's own setting wins.
+os.environ.setdefault("HIP_FORCE_DEV_KERNARG", "1")
+
 HBM_PEAK_GBS = 8000.0
 H, G, D, LAYERS = 4, 6, 256, 16
 QH = H * G
