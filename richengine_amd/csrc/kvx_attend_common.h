@@ -161,6 +161,9 @@ struct Sight {
 // order.
 constexpr uint32_t kMergeSequential = 32;
 constexpr uint32_t kMergeWaves = 4;
+// Partial rows a wave has in flight at a time: a list of up to 16 splits (the
+// average of a mixed batch at 32 pages per split) costs one load latency.
+constexpr uint32_t kMergeAhead = 16;
 
 struct MergeSums {
   f32x4 numerator;
@@ -169,14 +172,14 @@ struct MergeSums {
 
 // Sums splits [first, last) of the row in split order; `maximum` is the row's
 // maximum over all splits.  With PREFETCHED, `early` holds the partial rows of
-// the first eight splits (clamped to the last), loaded before the caller
+// the first kMergeAhead splits (clamped to the last), loaded before the caller
 // waited for the statistics.
 template <bool PREFETCHED>
 __device__ __forceinline__ MergeSums merge_range(const float *__restrict__ partials,
                                                  const float *__restrict__ statistics,
                                                  uint64_t first_row, uint32_t first, uint32_t last,
                                                  uint32_t M, float maximum, uint32_t lane,
-                                                 const f32x4 (&early)[8], f32x2 early_stat) {
+                                                 const f32x4 (&early)[kMergeAhead], f32x2 early_stat) {
   MergeSums sums{{0.0f, 0.0f, 0.0f, 0.0f}, 0.0f};
   for (uint32_t base = first; base < last; base += 64) {
     const uint32_t mine = base + lane;
@@ -189,10 +192,10 @@ __device__ __forceinline__ MergeSums merge_range(const float *__restrict__ parti
     const float my_weight = expf(__fsub_rn(stat[0], maximum));
     const float my_term = __fmul_rn(my_weight, stat[1]);
     const uint32_t count = min(64u, last - base);
-    for (uint32_t i = 0; i < count; i += 8) {
-      f32x4 part[8];
+    for (uint32_t i = 0; i < count; i += kMergeAhead) {
+      f32x4 part[kMergeAhead];
 #pragma unroll
-      for (uint32_t u = 0; u < 8; ++u) {
+      for (uint32_t u = 0; u < kMergeAhead; ++u) {
         if (PREFETCHED && base == first && i == 0) {
           part[u] = early[u];
         } else {
@@ -201,7 +204,7 @@ __device__ __forceinline__ MergeSums merge_range(const float *__restrict__ parti
         }
       }
 #pragma unroll
-      for (uint32_t u = 0; u < 8; ++u) {
+      for (uint32_t u = 0; u < kMergeAhead; ++u) {
         if (i + u < count) {
           const float weight = __shfl(my_weight, i + u);
 #pragma unroll
@@ -253,15 +256,15 @@ __global__ __launch_bounds__(64 * kMergeWaves) void matrix_merge_kernel(
   const bool sequential = written <= kMergeSequential;
   if (sequential && wave) return;
   // The sequential case (at most kMergeSequential splits) issues its statistics and the
-  // first eight partial rows together, before anything waits.
-  f32x4 early[8];
+  // first kMergeAhead partial rows together, before anything waits.
+  f32x4 early[kMergeAhead];
   f32x2 early_stat = {-INFINITY, 0.0f};
   float maximum = -INFINITY;
   if (sequential) {
     if (lane < written)
       early_stat = load_global<f32x2>(statistics + (first_row + uint64_t(lane) * M) * 2);
 #pragma unroll
-    for (uint32_t u = 0; u < 8; ++u)
+    for (uint32_t u = 0; u < kMergeAhead; ++u)
       early[u] = load_global<f32x4>(partials + (first_row + uint64_t(min(u, written - 1)) * M) * kD +
                                     4 * lane);
     maximum = early_stat[0];
