@@ -178,11 +178,26 @@ int kvx_verify_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t
 /* kv::chunkedPrefillValidationError: 0 ok, 1 chunk_tokens_out_of_range,
    2 context_out_of_range, 3 chunk_stride_invalid, 4 page_table_too_short */
 int kvx_chunk_validation(const kvx_chunk_params *params);
+/* Split count of one sequence's chunked prefill sized for this GPU instead of the reference's
+   clamp(32 / tiles, 1, 32).  That rule gives chunks of 256 rows and more a single split, which
+   is one wave per (pair of tiles, KV head, block of 32 fused rows): 192 waves for 256 rows of
+   24 query heads on 4 KV heads, on a GPU with 1024 SIMDs, each walking the whole context
+   alone.  The plan keeps one split while those waves fill at least half of the kernel's wave
+   slots and otherwise takes the largest count (at most 32, at least 8 pages per split) whose
+   launch of tiles x splits x KV heads x ceil(8 x group / 16) waves still fits one round of
+   slots.  Returns 0 for bad head counts.  No counterpart in the reference (its rule is
+   kvx_prefill_splits); any count in 1..32 is valid for kv_attend_prefill. */
+uint32_t kvx_prefill_plan(uint32_t committed_tokens, uint32_t rows, uint32_t kv_heads,
+                          uint32_t query_heads, uint32_t format);
 /* ops::PagedAttention::prefillPlan(...).workspace / prefillWorkspace / verifyWorkspace.
    Bytes of partials and statistics; a workspace buffer holds partials first,
    then statistics at the next 256-byte boundary. */
 int kvx_prefill_workspace(uint32_t rows, uint32_t query_heads, const kvx_layout *layout,
                           uint64_t *partials_bytes, uint64_t *statistics_bytes);
+/* The same for a given split count (kvx_prefill_plan's, or any in 1..32). */
+int kvx_prefill_workspace_for(uint32_t rows, uint32_t split_count, uint32_t query_heads,
+                              const kvx_layout *layout, uint64_t *partials_bytes,
+                              uint64_t *statistics_bytes);
 int kvx_prefill_workspace_bound(uint32_t maximum_rows, uint32_t query_heads,
                                 const kvx_layout *layout, uint64_t *partials_bytes,
                                 uint64_t *statistics_bytes);

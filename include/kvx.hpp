@@ -347,6 +347,19 @@ public:
                                 &plan.workspace.statisticsBytes));
     return plan;
   }
+  // The same with the split count sized for the GPU (kvx_prefill_plan): the
+  // reference rule gives chunks of 256 rows and more one split, which leaves
+  // most of 1024 SIMDs idle until the chunk has about 2048 rows.
+  static PrefillAttentionPlan prefillPlan(uint32_t historyTokens, uint32_t rows, uint32_t queryHeads,
+                                          kv::Layout layout) {
+    PrefillAttentionPlan plan = prefillPlan(rows, queryHeads, layout);
+    plan.splits = kvx_prefill_plan(historyTokens, rows, layout.kvHeads, queryHeads,
+                                   static_cast<uint32_t>(layout.format));
+    const kvx_layout l = layout.c();
+    check(kvx_prefill_workspace_for(rows, plan.splits, queryHeads, &l, &plan.workspace.partialsBytes,
+                                    &plan.workspace.statisticsBytes));
+    return plan;
+  }
   // decode = true selects the batched-decode split rule of this library
   // (rows = 1 per lane, one split per 32 visible pages).  sizedForGpu = true
   // takes the split counts from kvx_decode_plan / kvx_verify_plan, which look at

@@ -511,14 +511,14 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   const bool reused = tile_rows > 0;
   if (format == KVX_FMT_BF16) {
     if (M > 16) return reused ? KVX_WIDE(KVX_FMT_BF16, 2, 1, true) : KVX_WIDE(KVX_FMT_BF16, 2, 1, false);
-    return KVX_WIDE(KVX_FMT_BF16, 1, 1, false);
+    return reused ? KVX_WIDE(KVX_FMT_BF16, 1, 1, true) : KVX_WIDE(KVX_FMT_BF16, 1, 1, false);
   }
   const bool two_blocks = M > 16 && !many_tiles;
   if (format == KVX_FMT_INT8) {
     if (two_blocks) return reused ? KVX_WIDE(KVX_FMT_INT8, 2, 1, true) : KVX_WIDE(KVX_FMT_INT8, 2, 1, false);
-    return KVX_WIDE(KVX_FMT_INT8, 1, 2, false);
+    return reused ? KVX_WIDE(KVX_FMT_INT8, 1, 2, true) : KVX_WIDE(KVX_FMT_INT8, 1, 2, false);
   }
   if (two_blocks) return reused ? KVX_WIDE(KVX_FMT_FP8E4M3, 2, 1, true) : KVX_WIDE(KVX_FMT_FP8E4M3, 2, 1, false);
-  return KVX_WIDE(KVX_FMT_FP8E4M3, 1, 2, false);
+  return reused ? KVX_WIDE(KVX_FMT_FP8E4M3, 1, 2, true) : KVX_WIDE(KVX_FMT_FP8E4M3, 1, 2, false);
 #undef KVX_WIDE
 }

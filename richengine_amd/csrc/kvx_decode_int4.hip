@@ -629,6 +629,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   attend_int4<1, kDecodeDepth>(queries, output, partials, statistics, a);
 }
 
+// The same for the 8-row tiles of a chunked prefill with several splits: every
+// tile of the chunk walks the same pages, so the loads may stay in the caches.
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_int4_tiles_kernel(
+    const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
+    float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
+  attend_int4<1, kDecodeDepth, true>(queries, output, partials, statistics, a);
+}
+
 // Two blocks per wave share every expanded key and value operand (verify, tree
 // verify, prefill tiles); the accumulators of both take the register file of a
 // whole SIMD lane, so one wave per SIMD.
@@ -712,6 +720,11 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   if (fused_rows > 16 && !many_tiles)
     return launch_matrix_attention(verify_int4_kernel, "verify_int4_kernel", 32, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
+                                   row_masks, row_stride, lane_stride, workspace, workspace_bytes,
+                                   kvx_attend_phases(), stream, nullptr, tile_rows, epilogue);
+  if (tile_rows && !fused)
+    return launch_matrix_attention(decode_int4_tiles_kernel, "decode_int4_tiles_kernel", 16, 64, s,
+                                   kv, query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
                                    kvx_attend_phases(), stream, nullptr, tile_rows, epilogue);
   return launch_matrix_attention(decode_int4_kernel, "decode_int4_kernel", 16, 64, s, kv,

@@ -159,6 +159,27 @@ uint32_t kvx_prefill_splits(uint32_t rows) {
   if (!tiles) return KVX_PREFILL_MAX_SPLITS;
   return std::min(std::max(KVX_PREFILL_MAX_SPLITS / tiles, 1u), KVX_PREFILL_MAX_SPLITS);
 }
+uint32_t kvx_prefill_plan(uint32_t committed, uint32_t rows, uint32_t kv_heads, uint32_t query_heads,
+                          uint32_t format) {
+  if (!kv_heads || !query_heads || query_heads % kv_heads) return 0;
+  const uint32_t tiles = (rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+  if (!tiles) return 1;
+  const uint32_t group = query_heads / kv_heads, tile_fused = KVX_PREFILL_TILE_ROWS * group;
+  const uint32_t pages = pages_of(uint64_t(committed) + rows);
+  constexpr uint32_t kSimds = 1024;
+  // One split: neighbouring tiles share a walk as lanes of 16 rows on the kernels
+  // with two blocks of 16 fused rows per wave (int4: two waves per SIMD).
+  const uint32_t paired_waves = (tiles + 1) / 2 * kv_heads * ((2 * tile_fused + 31) / 32);
+  const uint32_t paired_slots = format == KVX_FMT_INT4 ? 2 * kSimds : kSimds;
+  if (tile_fused <= 16 || 2 * paired_waves >= paired_slots) return 1;
+  // Several splits: one lane per tile on the kernels with one block per wave
+  // (two waves per SIMD except for bf16 pages).
+  const uint32_t slots = format == KVX_FMT_BF16 ? kSimds : 2 * kSimds;
+  const uint32_t per_split = tiles * kv_heads * ((tile_fused + 15) / 16);
+  const uint32_t fit = slots / per_split, by_pages = std::max(1u, pages / 8);
+  const uint32_t splits = std::min({fit, by_pages, KVX_PREFILL_MAX_SPLITS});
+  return splits >= 2 ? splits : 1;
+}
 uint32_t kvx_decode_splits(uint32_t committed, uint32_t rows) {
   const uint32_t pages = pages_of(uint64_t(committed) + rows);
   const uint32_t wanted = (pages + KVX_DECODE_PAGES_PER_SPLIT - 1) / KVX_DECODE_PAGES_PER_SPLIT;
@@ -254,6 +275,16 @@ int kvx_prefill_workspace(uint32_t rows, uint32_t query_heads, const kvx_layout 
   const uint64_t tiles = (rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
   workspace_rows(tiles * kvx_prefill_splits(rows) * KVX_PREFILL_TILE_ROWS * query_heads,
                  l->head_dim, pb, sb);
+  return KVX_OK;
+}
+int kvx_prefill_workspace_for(uint32_t rows, uint32_t split_count, uint32_t query_heads,
+                              const kvx_layout *l, uint64_t *pb, uint64_t *sb) {
+  if (int rc = geometry_ok(query_heads, l)) return rc;
+  if (!rows || rows > KVX_PREFILL_TOKEN_BUDGET || !split_count ||
+      split_count > KVX_PREFILL_MAX_SPLITS)
+    return fail(KVX_EINVAL, "invalid paged prefill attention geometry");
+  const uint64_t tiles = (rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+  workspace_rows(tiles * split_count * KVX_PREFILL_TILE_ROWS * query_heads, l->head_dim, pb, sb);
   return KVX_OK;
 }
 int kvx_prefill_workspace_bound(uint32_t maximum_rows, uint32_t query_heads, const kvx_layout *l,

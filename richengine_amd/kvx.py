@@ -23,8 +23,8 @@ SYMBOLS = [
     "kvx_layout_bytes_per_model_page", "kvx_layout_extent_alignment_pages",
     "kvx_layout_minimum_extent_pages", "kvx_layout_maximum_extent_pages",
     "kvx_layout_extent_pages_for", "kvx_layout_largest_extent_pages", "kvx_kv_offset",
-    "kvx_verify_splits", "kvx_prefill_splits", "kvx_decode_splits", "kvx_chunk_validation",
-    "kvx_prefill_workspace", "kvx_prefill_workspace_bound", "kvx_verify_workspace",
+    "kvx_verify_splits", "kvx_prefill_splits", "kvx_prefill_plan", "kvx_decode_splits", "kvx_chunk_validation",
+    "kvx_prefill_workspace", "kvx_prefill_workspace_for", "kvx_prefill_workspace_bound", "kvx_verify_workspace",
     "kvx_attend_workspace_bytes", "kvx_storage_create", "kvx_storage_destroy",
     "kvx_storage_page_count", "kvx_storage_extent_pages", "kvx_storage_bytes_per_page",
     "kvx_storage_extent_bytes", "kvx_storage_allocated_bytes", "kvx_storage_is_allocated",
@@ -138,6 +138,7 @@ def _declare(L):
     for n in ("kvx_verify_splits", "kvx_decode_splits"):
         getattr(L, n).argtypes, getattr(L, n).restype = [u32, u32], u32
     L.kvx_prefill_splits.argtypes, L.kvx_prefill_splits.restype = [u32], u32
+    L.kvx_prefill_plan.argtypes, L.kvx_prefill_plan.restype = [u32, u32, u32, u32, u32], u32
     L.kvx_chunk_validation.argtypes = [C.POINTER(ChunkParams)]
     P64 = C.POINTER(u64)
     L.kvx_prefill_workspace.argtypes = [u32, u32, LP, P64, P64]
@@ -421,10 +422,15 @@ def append_attend_decode(storage, layer, chunk_keys, chunk_values, chunk_lane_st
         _ptr(workspace), workspace.numel() * workspace.element_size(), _stream(stream)))
 
 
-def prefill_workspace_bytes(storage, rows, query_heads):
+def prefill_workspace_bytes(storage, rows, query_heads, splits=None):
+    """Workspace of kv_attend_prefill: for the reference's split rule, or for `splits`."""
     pb, sb = C.c_uint64(), C.c_uint64()
-    check(lib().kvx_prefill_workspace(rows, query_heads, C.byref(storage.layout), C.byref(pb),
-                                      C.byref(sb)))
+    if splits is None:
+        check(lib().kvx_prefill_workspace(rows, query_heads, C.byref(storage.layout), C.byref(pb),
+                                          C.byref(sb)))
+    else:
+        check(lib().kvx_prefill_workspace_for(rows, splits, query_heads, C.byref(storage.layout),
+                                              C.byref(pb), C.byref(sb)))
     return pb.value + sb.value
 
 
@@ -634,6 +640,14 @@ def decode_plan(committed, kv_heads, fmt=INT4):
     out = (C.c_uint32 * len(committed))()
     check(lib().kvx_decode_plan(_u32(committed), len(committed), kv_heads, fmt, out))
     return list(out)
+
+
+def prefill_plan(committed, rows, kv_heads, query_heads, fmt=INT4):
+    """Split count of a chunked prefill sized for the GPU (kvx_prefill_plan)."""
+    splits = lib().kvx_prefill_plan(committed, rows, kv_heads, query_heads, fmt)
+    if not splits:
+        raise KvxError(-1, "kvx_prefill_plan: bad head counts")
+    return splits
 
 
 def verify_plan(committed, rows, kv_heads, query_heads, fmt=INT4):

@@ -115,6 +115,9 @@ void testPlans() {
   // rows per slot = 8 * group.
   EXPECT(full.workspace.partialsBytes == uint64_t{256} * 4 * 1 * 48 * 256 * 4);
   EXPECT(full.workspace.statisticsBytes == uint64_t{256} * 4 * 1 * 48 * 2 * 4);
+  const auto sized = ops::PagedAttention::prefillPlan(16384, 256, 24, layout);
+  EXPECT(sized.splits > 1 && sized.splits <= 32);
+  EXPECT(sized.workspace.partialsBytes == uint64_t(32) * sized.splits * 8 * 24 * 256 * 4);
   const auto bound = ops::PagedAttention::prefillWorkspace(2048, 24, layout);
   EXPECT(bound.partialsBytes >= full.workspace.partialsBytes);
   const auto verify = ops::PagedAttention::verifyPlan(2, 24, layout, {0, 131072});

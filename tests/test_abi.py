@@ -142,6 +142,25 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
                 per += 1
             assert plan == want
             assert all(1 <= s <= 128 and s <= max(n, 1) for s, n in zip(plan, counts))
+    # chunked prefill: one split while the paired tiles fill half of the wave slots, else the
+    # largest count whose one-tile lanes fit one round (and leave 8 pages per split)
+    for fmt in (kvx.INT4, kvx.INT8, kvx.FP8, kvx.BF16):
+        single_slots = 2048 if fmt == kvx.INT4 else 1024
+        slots = 1024 if fmt == kvx.BF16 else 2048
+        for committed, rows in ((16384, 64), (16384, 256), (16384, 512), (16384, 2048), (0, 256),
+                                (100, 7), (3000, 264)):
+            tiles = -(-rows // 8)
+            paired = -(-tiles // 2) * H * -(-(16 * (QH // H)) // 32)
+            want = 1
+            if 2 * paired < single_slots:
+                want = min(slots // (tiles * H * -(-(8 * (QH // H)) // 16)),
+                           max(1, pages(committed + rows) // 8), 32)
+                want = want if want >= 2 else 1
+            assert kvx.prefill_plan(committed, rows, H, QH, fmt) == want
+    assert kvx.prefill_plan(16384, 256, H, QH, kvx.INT4) == 5
+    assert kvx.prefill_plan(16384, 2048, H, QH, kvx.INT4) == 1
+    with pytest.raises(kvx.KvxError):
+        kvx.prefill_plan(16384, 256, 4, 6)
     assert kvx.verify_plan([65536] * 4, 16, H, QH) == [32] * 4          # two waves of 48 fused rows
     assert kvx.verify_plan([65536] * 4, 16, H, QH, kvx.BF16) == [21] * 4  # three of 32
     with pytest.raises(kvx.KvxError):
@@ -166,20 +185,22 @@ def test_hot_kernels_stay_out_of_scratch_memory():
         assert len(names) == 1, (fragment, names)
         return report[names[0]]
 
-    for fragment in ("decode_int4_kernel", "verify_int4_kernel", "matrix_merge_kernel",
+    for fragment in ("decode_int4_kernelE", "decode_int4_tiles_kernel", "verify_int4_kernel", "matrix_merge_kernel",
                      "attend_wide_kernelILj1ELj1ELj2ELb0E",    # int8, one block, two waves per SIMD
                      "attend_wide_kernelILj4ELj1ELj2ELb0E",    # fp8
                      "attend_wide_kernelILj2ELj1ELj1ELb0E",    # bf16 decode
+                     "attend_wide_kernelILj1ELj1ELj2ELb1E", "attend_wide_kernelILj4ELj1ELj2ELb1E",
+                     "attend_wide_kernelILj2ELj1ELj1ELb1E",    # the same three for prefill tiles
                      "attend_wide_kernelILj1ELj2ELj1ELb0E", "attend_wide_kernelILj4ELj2ELj1ELb0E",
                      # the same two with page loads that may stay in the caches (prefill tiles)
                      "attend_wide_kernelILj1ELj2ELj1ELb1E", "attend_wide_kernelILj4ELj2ELj1ELb1E"):
         r = one(fragment)
         assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, (fragment, r)
-    assert one("decode_int4_kernel")["occupancy"] == 2
+    assert one("decode_int4_kernelE")["occupancy"] == 2
     # the 48-row verify kernel keeps a few set-up values in scratch memory, none of
     # them touched inside its page loop; more than that would be accumulators or pages
     assert one("verify48_int4_kernel")["vgprs_spill"] <= 20
-    assert one("attend_wide_kernelILj1ELj1ELj2E")["occupancy"] == 2
+    assert one("attend_wide_kernelILj1ELj1ELj2ELb0E")["occupancy"] == 2
     for fmt in (1, 2, 3, 4):
         assert one(f"13append_kernelILj{fmt}E")["scratchsize"] == 0
         assert one(f"prepare_append_kernelILj{fmt}E")["scratchsize"] == 0

@@ -78,8 +78,11 @@ def queries(shape_rows, seed):
 
 @pytest.mark.parametrize("fmt", FORMATS)
 @pytest.mark.parametrize("committed,rows", [(0, 1), (33, 7), (255, 17), (1023, 8), (100, 77),
-                                            (2000, 130)])
+                                            (2000, 130), (1500, -264)])
 def test_prefill_matches_oracle(fmt, committed, rows):
+    # rows < 0: that many rows with kvx_prefill_plan's split count in place of the
+    # reference rule's (which gives 264 rows a single split)
+    planned, rows = rows < 0, abs(rows)
     tw = Gp.Twin(fmt, H, D, 2, (committed + rows + 31) // 32)
     pages, th, td = fill(tw, committed + rows, seed=committed + rows)
     tw.assert_same_bytes()
@@ -87,11 +90,15 @@ def test_prefill_matches_oracle(fmt, committed, rows):
     q = np.zeros((H, stride, G, D), dtype=np.uint16)
     q[:, :rows] = queries((H, rows, G, D), committed)
     splits = kvx.lib().kvx_prefill_splits(rows)
+    if planned:
+        splits = kvx.prefill_plan(committed, rows, H, QH, fmt)
+        assert splits > 1
     hp = ko.PrefillParams(committed, rows, stride, len(pages), tw.host.layer(1), splits, 0.0)
     ok, want, want32 = ko.attend_prefill(fmt, H, G, D, q, th, hp)
     assert ok == 1
     out = torch.full((H, stride, G, D), 0x5A5A, dtype=torch.int16, device="cuda")
-    ws = torch.empty(kvx.prefill_workspace_bytes(tw.dev, rows, QH), dtype=torch.uint8, device="cuda")
+    ws = torch.empty(kvx.prefill_workspace_bytes(tw.dev, rows, QH, splits), dtype=torch.uint8,
+                     device="cuda")
     kvx.attend_prefill(tw.dev, 1, QH, Gp.dev(q), out, td,
                        kvx.PrefillParams(committed, rows, stride, len(pages), kvx.KvLayer(), splits, 0.0), ws)
     torch.cuda.synchronize()
