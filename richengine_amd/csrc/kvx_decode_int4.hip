@@ -582,8 +582,12 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   // line code and the wait for a set counts exactly the loads issued after it;
   // a refill under a branch would make each wait cover the newest loads too.
   // The last page of the split is never consumed here, so no token test.
+  // Nor is the page before it: the rows of a lane may see different parts of the
+  // last two pages of a sequence (a chain of 8 rows or a pair of prefill tiles
+  // that begins shortly before a page boundary), so both take the masked path.
+  constexpr uint32_t kUnmaskedStop = 2 * kDepth > kDepth + 2 ? 2 * kDepth : kDepth + 2;
   uint32_t page = begin;
-  for (; page + 2 * kDepth <= end; page += kDepth) {
+  for (; page + kUnmaskedStop <= end; page += kDepth) {
 #pragma unroll
     for (uint32_t d = 0; d < kDepth; ++d) {
       const uint32_t refill = page + d + kDepth - begin;
@@ -592,14 +596,14 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
       fill_rest(r[d], refill);
     }
   }
-  // Tail: at most 2 * kDepth - 1 pages are left, the first kDepth of them loaded.
+  // Tail: at most kUnmaskedStop - 1 pages are left, the first kDepth of them loaded.
 #pragma unroll
-  for (uint32_t k = 0; k < 2 * kDepth - 1; ++k) {
+  for (uint32_t k = 0; k < kUnmaskedStop - 1; ++k) {
     const uint32_t d = k % kDepth;
     if (page + k < end) {
       attend_page<true, NB>(r[d], staged_queries, q_bias, score_scale, (page + k) * kPage, sight, lane, g,
                             st, [] {});
-      if (k + kDepth < 2 * kDepth - 1 && page + k + kDepth < end)
+      if (k + kDepth < kUnmaskedStop - 1 && page + k + kDepth < end)
         fill(r[d], page + k + kDepth - begin);
     }
   }

@@ -172,11 +172,16 @@ uint32_t kvx_prefill_plan(uint32_t committed, uint32_t rows, uint32_t kv_heads, 
   const uint32_t paired_waves = (tiles + 1) / 2 * kv_heads * ((2 * tile_fused + 31) / 32);
   const uint32_t paired_slots = format == KVX_FMT_INT4 ? 2 * kSimds : kSimds;
   if (tile_fused <= 16 || 2 * paired_waves >= paired_slots) return 1;
+  const uint32_t by_pages = std::max(1u, pages / 8);
+  // Tiles that pair under any split count keep their shared walks: as many
+  // splits as fit one round of the paired kernels' slots.
+  if (kvx::prefill_tiles_pair(committed) && tiles >= 2)
+    return std::max(1u, std::min({paired_slots / paired_waves, by_pages, KVX_PREFILL_MAX_SPLITS}));
   // Several splits: one lane per tile on the kernels with one block per wave
   // (two waves per SIMD except for bf16 pages).
   const uint32_t slots = format == KVX_FMT_BF16 ? kSimds : 2 * kSimds;
   const uint32_t per_split = tiles * kv_heads * ((tile_fused + 15) / 16);
-  const uint32_t fit = slots / per_split, by_pages = std::max(1u, pages / 8);
+  const uint32_t fit = slots / per_split;
   const uint32_t splits = std::min({fit, by_pages, KVX_PREFILL_MAX_SPLITS});
   return splits >= 2 ? splits : 1;
 }

@@ -120,6 +120,15 @@ inline uint32_t verify_block_rows(uint32_t format, uint32_t fused_rows) {
 #endif
   return 32;
 }
+// Whether tiles 2i and 2i + 1 of a chunked prefill that starts after `committed`
+// tokens see the same number of pages, for every i: tile 2i sees committed + 16 i
+// + 8 tokens, its neighbour 8 more, and no page boundary lies in between exactly
+// when committed mod 16 is 0 or at least 9 (page-aligned chunk starts among them).
+// Such pairs cut their pages into the same splits, whatever the split count.
+inline bool prefill_tiles_pair(uint32_t committed) {
+  const uint32_t r = committed % 16;
+  return r == 0 || r >= 9;
+}
 // Waves (row blocks) per (lane, split, KV head) of a verify launch.
 inline uint32_t verify_row_blocks(uint32_t format, uint32_t fused_rows) {
   const uint32_t rows = verify_block_rows(format, fused_rows);

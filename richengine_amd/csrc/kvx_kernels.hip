@@ -1833,8 +1833,14 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
     // runs over the same pages in the same order (the page the second tile may
     // add is invisible to the first tile's rows and changes nothing), and every
     // key and value is fetched and expanded once for 16 rows instead of 8.
+    // With several splits the two tiles must also cut their pages into the same
+    // splits, which they do when they see the same number of pages
+    // (prefill_tiles_pair: true for every pair of the chunk, or for none).
     const uint32_t T = KVX_PREFILL_TILE_ROWS;
-    const uint32_t width = (params->split_count == 1 && tiles >= 2) ? 2 : 1;
+    const uint32_t width =
+        (tiles >= 2 && (params->split_count == 1 || prefill_tiles_pair(params->committed_tokens)))
+            ? 2
+            : 1;
     const uint32_t wide_lanes = tiles / width, rest = tiles - wide_lanes * width;
     std::vector<kvx_verify_params> tile_lanes(wide_lanes + rest);
     std::vector<const uint64_t *> tile_tables(wide_lanes + rest, page_table);

@@ -148,16 +148,20 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
         single_slots = 2048 if fmt == kvx.INT4 else 1024
         slots = 1024 if fmt == kvx.BF16 else 2048
         for committed, rows in ((16384, 64), (16384, 256), (16384, 512), (16384, 2048), (0, 256),
-                                (100, 7), (3000, 264)):
+                                (100, 7), (3000, 264), (3004, 264), (16388, 512)):
             tiles = -(-rows // 8)
             paired = -(-tiles // 2) * H * -(-(16 * (QH // H)) // 32)
             want = 1
             if 2 * paired < single_slots:
-                want = min(slots // (tiles * H * -(-(8 * (QH // H)) // 16)),
-                           max(1, pages(committed + rows) // 8), 32)
-                want = want if want >= 2 else 1
+                by_pages = max(1, pages(committed + rows) // 8)
+                if tiles >= 2 and (committed % 16 == 0 or committed % 16 >= 9):
+                    want = max(1, min(single_slots // paired, by_pages, 32))   # tiles stay paired
+                else:
+                    want = min(slots // (tiles * H * -(-(8 * (QH // H)) // 16)), by_pages, 32)
+                    want = want if want >= 2 else 1
             assert kvx.prefill_plan(committed, rows, H, QH, fmt) == want
-    assert kvx.prefill_plan(16384, 256, H, QH, kvx.INT4) == 5
+    assert kvx.prefill_plan(16384, 256, H, QH, kvx.INT4) == 10     # 192 waves of paired tiles per split
+    assert kvx.prefill_plan(16388, 256, H, QH, kvx.INT4) == 5      # 384 of single tiles
     assert kvx.prefill_plan(16384, 2048, H, QH, kvx.INT4) == 1
     with pytest.raises(kvx.KvxError):
         kvx.prefill_plan(16384, 256, 4, 6)

@@ -78,10 +78,13 @@ def queries(shape_rows, seed):
 
 @pytest.mark.parametrize("fmt", FORMATS)
 @pytest.mark.parametrize("committed,rows", [(0, 1), (33, 7), (255, 17), (1023, 8), (100, 77),
-                                            (2000, 130), (1500, -264)])
+                                            (2000, 130), (1500, 264), (1500, -136), (1508, -136)])
 def test_prefill_matches_oracle(fmt, committed, rows):
     # rows < 0: that many rows with kvx_prefill_plan's split count in place of the
-    # reference rule's (which gives 264 rows a single split)
+    # reference rule's (2 for 136 rows; 264 rows get a single split); after 1500 tokens the
+    # tiles stay paired under several splits, after 1508 they run one by one.  1500
+    # is 4 tokens before a page boundary, so the rows of the first pair of tiles see
+    # different parts of two pages
     planned, rows = rows < 0, abs(rows)
     tw = Gp.Twin(fmt, H, D, 2, (committed + rows + 31) // 32)
     pages, th, td = fill(tw, committed + rows, seed=committed + rows)
@@ -119,7 +122,9 @@ def test_prefill_matches_oracle(fmt, committed, rows):
 
 @pytest.mark.parametrize("fmt", FORMATS)
 def test_verify_chain_matches_oracle(fmt):
-    committed = [0, 1023, 1023 + 649, 40]
+    # 348 and 1980 tokens end 4 tokens before a page boundary: the chain's rows see
+    # different parts of the last two pages
+    committed = [0, 1023, 1023 + 649, 40, 348, 1980]
     lanes = len(committed)
     counts = [(c + 8 + 31) // 32 for c in committed]
     tws, hts, dts = [], [], []
@@ -185,7 +190,7 @@ def shared_pool_lanes(fmt, committed, rows, seed, layers=2, layer=1):
 
 @pytest.mark.parametrize("fmt", [ko.INT4, ko.INT8, ko.BF16])
 def test_batched_verify_chain_matches_oracle(fmt):
-    committed = [0, 1023, 1672, 31]
+    committed = [0, 1023, 1672, 31, 1980]
     tw, counts, hts, dts = shared_pool_lanes(fmt, committed, 8, seed=41)
     lanes = len(committed)
     q = np.zeros((lanes, H, 32, G, D), dtype=np.uint16)
