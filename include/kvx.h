@@ -186,7 +186,7 @@ int kvx_chunk_validation(const kvx_chunk_params *params);
    slots and otherwise takes the largest count (at most 32, at least 8 pages per split) whose
    launch still fits one round of slots: of the paired tiles' waves where the two tiles of
    every pair see the same number of pages (committed_tokens mod 16 is 0 or at least 9, so
-   every page-aligned chunk start), else of tiles x splits x KV heads x ceil(8 x group / 16)
+   every page-aligned chunk start; int4 pages: from 512 rows on), else of tiles x splits x KV heads x ceil(8 x group / 16)
    waves of single tiles.  Returns 0 for bad head counts.  No counterpart in the reference (its rule is
    kvx_prefill_splits); any count in 1..32 is valid for kv_attend_prefill. */
 uint32_t kvx_prefill_plan(uint32_t committed_tokens, uint32_t rows, uint32_t kv_heads,

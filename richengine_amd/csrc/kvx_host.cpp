@@ -169,14 +169,17 @@ uint32_t kvx_prefill_plan(uint32_t committed, uint32_t rows, uint32_t kv_heads, 
   constexpr uint32_t kSimds = 1024;
   // One split: neighbouring tiles share a walk as lanes of 16 rows on the kernels
   // with two blocks of 16 fused rows per wave (int4: two waves per SIMD).
-  const uint32_t paired_waves = (tiles + 1) / 2 * kv_heads * ((2 * tile_fused + 31) / 32);
-  const uint32_t paired_slots = format == KVX_FMT_INT4 ? 2 * kSimds : kSimds;
+  const uint32_t paired_waves = kvx::prefill_paired_waves(tiles, kv_heads, group);
+  const uint32_t paired_slots = kvx::prefill_paired_slots(format);
   if (tile_fused <= 16 || 2 * paired_waves >= paired_slots) return 1;
   const uint32_t by_pages = std::max(1u, pages / 8);
   // Tiles that pair under any split count keep their shared walks: as many
   // splits as fit one round of the paired kernels' slots.
-  if (kvx::prefill_tiles_pair(committed) && tiles >= 2)
-    return std::max(1u, std::min({paired_slots / paired_waves, by_pages, KVX_PREFILL_MAX_SPLITS}));
+  const uint32_t paired_splits =
+      std::max(1u, std::min({paired_slots / paired_waves, by_pages, KVX_PREFILL_MAX_SPLITS}));
+  if (paired_splits >= 2 &&
+      kvx::prefill_pairs_with_splits(format, committed, tiles, paired_splits, kv_heads, group))
+    return paired_splits;
   // Several splits: one lane per tile on the kernels with one block per wave
   // (two waves per SIMD except for bf16 pages).
   const uint32_t slots = format == KVX_FMT_BF16 ? kSimds : 2 * kSimds;

@@ -129,6 +129,24 @@ inline bool prefill_tiles_pair(uint32_t committed) {
   const uint32_t r = committed % 16;
   return r == 0 || r >= 9;
 }
+// Waves of a chunked prefill whose tiles run in pairs (lanes of 16 rows on the
+// kernels with two blocks of 16 fused rows per wave), per split, and the wave
+// slots those kernels have (int4: two waves per SIMD).
+inline uint32_t prefill_paired_waves(uint32_t tiles, uint32_t kv_heads, uint32_t group) {
+  return (tiles + 1) / 2 * kv_heads * ((2 * KVX_PREFILL_TILE_ROWS * group + 31) / 32);
+}
+inline uint32_t prefill_paired_slots(uint32_t format) { return format == KVX_FMT_INT4 ? 2048 : 1024; }
+// Whether a prefill with several splits runs its tiles in pairs: the pairs must
+// cut their pages alike, and the paired launch must fill at least half of its
+// wave slots (half as many waves, each twice as long, lose on an emptier GPU).
+// int4 pages: only from 64 tiles on; below, the one-tile kernel with its two
+// register sets of pages is faster per page than sharing saves.
+inline bool prefill_pairs_with_splits(uint32_t format, uint32_t committed, uint32_t tiles,
+                                      uint32_t splits, uint32_t kv_heads, uint32_t group) {
+  if (tiles < 2 || !prefill_tiles_pair(committed)) return false;
+  if (format == KVX_FMT_INT4 && tiles < 64) return false;
+  return 2ull * prefill_paired_waves(tiles, kv_heads, group) * splits >= prefill_paired_slots(format);
+}
 // Waves (row blocks) per (lane, split, KV head) of a verify launch.
 inline uint32_t verify_row_blocks(uint32_t format, uint32_t fused_rows) {
   const uint32_t rows = verify_block_rows(format, fused_rows);

@@ -1835,10 +1835,13 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
     // key and value is fetched and expanded once for 16 rows instead of 8.
     // With several splits the two tiles must also cut their pages into the same
     // splits, which they do when they see the same number of pages
-    // (prefill_tiles_pair: true for every pair of the chunk, or for none).
+    // (prefill_tiles_pair: true for every pair of the chunk, or for none), and pay
+    // only where the paired launch fills the GPU (prefill_pairs_with_splits).
     const uint32_t T = KVX_PREFILL_TILE_ROWS;
     const uint32_t width =
-        (tiles >= 2 && (params->split_count == 1 || prefill_tiles_pair(params->committed_tokens)))
+        (tiles >= 2 && (params->split_count == 1 ||
+                        prefill_pairs_with_splits(l.format, params->committed_tokens, tiles,
+                                                  params->split_count, H, G)))
             ? 2
             : 1;
     const uint32_t wide_lanes = tiles / width, rest = tiles - wide_lanes * width;

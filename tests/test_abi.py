@@ -154,14 +154,20 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
             want = 1
             if 2 * paired < single_slots:
                 by_pages = max(1, pages(committed + rows) // 8)
-                if tiles >= 2 and (committed % 16 == 0 or committed % 16 >= 9):
-                    want = max(1, min(single_slots // paired, by_pages, 32))   # tiles stay paired
+                pairable = tiles >= 2 and (committed % 16 == 0 or committed % 16 >= 9)
+                if fmt == kvx.INT4 and tiles < 64:
+                    pairable = False
+                together = max(1, min(single_slots // paired, by_pages, 32))
+                if pairable and together >= 2 and 2 * paired * together >= single_slots:
+                    want = together                                            # tiles stay paired
                 else:
                     want = min(slots // (tiles * H * -(-(8 * (QH // H)) // 16)), by_pages, 32)
                     want = want if want >= 2 else 1
             assert kvx.prefill_plan(committed, rows, H, QH, fmt) == want
-    assert kvx.prefill_plan(16384, 256, H, QH, kvx.INT4) == 10     # 192 waves of paired tiles per split
-    assert kvx.prefill_plan(16388, 256, H, QH, kvx.INT4) == 5      # 384 of single tiles
+    assert kvx.prefill_plan(16384, 256, H, QH, kvx.INT4) == 5      # 384 waves of single tiles per split
+    assert kvx.prefill_plan(16384, 256, H, QH, kvx.BF16) == 5      # 192 of paired tiles
+    assert kvx.prefill_plan(16384, 1024, H, QH, kvx.INT4) == 2     # 768 of paired tiles
+    assert kvx.prefill_plan(16388, 256, H, QH, kvx.BF16) == 2      # 384 of single tiles
     assert kvx.prefill_plan(16384, 2048, H, QH, kvx.INT4) == 1
     with pytest.raises(kvx.KvxError):
         kvx.prefill_plan(16384, 256, 4, 6)

@@ -81,10 +81,21 @@ def queries(shape_rows, seed):
                                             (2000, 130), (1500, 264), (1500, -136), (1508, -136)])
 def test_prefill_matches_oracle(fmt, committed, rows):
     # rows < 0: that many rows with kvx_prefill_plan's split count in place of the
-    # reference rule's (2 for 136 rows; 264 rows get a single split); after 1500 tokens the
+    # reference rule's (which gives 136 and 264 rows a single split); after 1500 tokens the
     # tiles stay paired under several splits, after 1508 they run one by one.  1500
     # is 4 tokens before a page boundary, so the rows of the first pair of tiles see
     # different parts of two pages
+    prefill_case(fmt, committed, rows)
+
+
+def test_int4_prefill_pairs_tiles_under_several_splits():
+    # int4 tiles pair under several splits only from 64 tiles on: 512 rows after 284
+    # tokens (4 before a page boundary), three splits by kvx_prefill_plan
+    assert kvx.prefill_plan(284, 512, H, QH, ko.INT4) == 3
+    prefill_case(ko.INT4, 284, -512)
+
+
+def prefill_case(fmt, committed, rows):
     planned, rows = rows < 0, abs(rows)
     tw = Gp.Twin(fmt, H, D, 2, (committed + rows + 31) // 32)
     pages, th, td = fill(tw, committed + rows, seed=committed + rows)
