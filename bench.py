@@ -71,6 +71,9 @@ def parse():
                     help="decode: the step's queries, keys and values come from packed projection rows "
                          "through kv_prepare_append (norm, rotation, quantize, store) instead of "
                          "ready chunk rows through kv_append; implies --separate-append")
+    ap.add_argument("--prefill-chunk", type=int, default=2048, choices=[64, 128, 256, 512, 1024, 2048],
+                    help="prefill: rows per chunk (BASELINE configs[3] has 2048); smaller chunks show "
+                         "what kvx_prefill_plan's split counts do")
     ap.add_argument("--prefill-streams", type=int, default=4,
                     help="prefill: HIP streams the batch's sequences are spread over (1 = all on the "
                          "current stream); a sequence's layers stay in order on its stream")
@@ -499,7 +502,7 @@ def chunked_prefill(args):
     rng = np.random.default_rng(args.seed)
     fmt = {"bf16": kvx.BF16, "fp8": kvx.FP8, "int8": kvx.INT8, "int4": kvx.INT4}[args.format]
     peak = 2500.0  # bf16 and fp16 MFMA (the one-byte formats multiply as fp16)
-    sequences, prefix, chunk = 4, 16384, 2048
+    sequences, prefix, chunk = 4, 16384, args.prefill_chunk
     prefix_pages, chunk_pages = prefix // 32, chunk // 32
     total = prefix_pages + sequences * chunk_pages
     layout = kvx.Layout(LAYERS, H, D, fmt, 0.0)
@@ -535,10 +538,10 @@ def chunked_prefill(args):
     streams = [torch.cuda.Stream() for _ in range(n_streams)] if n_streams > 1 else [None]
     outputs = [torch.zeros_like(queries[0]) for _ in range(n_streams)]
     output = outputs[0]
-    splits = L.kvx_prefill_splits(chunk)
+    splits = kvx.prefill_plan(prefix, chunk, H, QH, fmt)  # 1 for 2048 rows; chunks of 64 .. 1024 rows get more
     cp = kvx.ChunkParams(prefix, chunk, chunk, entries)
     pp = kvx.PrefillParams(prefix, chunk, chunk, entries, kvx.KvLayer(), splits, 0.0)
-    workspaces = [torch.empty(kvx.prefill_workspace_bytes(storage, chunk, QH) + 4096, dtype=torch.uint8,
+    workspaces = [torch.empty(kvx.prefill_workspace_bytes(storage, chunk, QH, splits) + 4096, dtype=torch.uint8,
                               device="cuda") for _ in range(n_streams)]
     workspace = workspaces[0]
     torch.cuda.synchronize()
@@ -575,7 +578,7 @@ def chunked_prefill(args):
     flops = 4 * D * QH * sum(prefix + r + 1 for r in range(chunk))
     achieved = flops / (kernel_ms * 1e-3) / 1e12
     result = {
-        "metric": f"{args.format} chunked prefill (2048-token chunks onto a shared 16384-token prefix, "
+        "metric": f"{args.format} chunked prefill ({chunk}-token chunks onto a shared 16384-token prefix, "
                   "batch 4): prefill tokens/s",
         "value": round(sequences * chunk * steps / wall, 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": steps, "warmup": warmup, "ms_per_step": round(wall * 1e3 / steps, 3),
@@ -585,7 +588,7 @@ def chunked_prefill(args):
                  ", fp32 accumulate",
         "data": "synthetic",
         "config": {"workload": "BASELINE configs[3]: chunked prefill with a shared prefix, batch 4, "
-                               "2048-row chunks over 16384 + 2048 tokens, 16 layers: quantize + scatter "
+                               f"{chunk}-row chunks over 16384 + {chunk} tokens, 16 layers: quantize + scatter "
                                "of the chunk, then causal attention per layer and sequence",
                    "batch": sequences, "layers": LAYERS, "format": args.format, "splits": int(splits),
                    "streams": n_streams, "seed": args.seed},
