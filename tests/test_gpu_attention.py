@@ -78,7 +78,7 @@ def queries(shape_rows, seed):
 
 @pytest.mark.parametrize("fmt", FORMATS)
 @pytest.mark.parametrize("committed,rows", [(0, 1), (33, 7), (255, 17), (1023, 8), (100, 77),
-                                            (2000, 130), (1500, 264), (1500, -136), (1508, -136)])
+                                            (2000, 130), (1500, -136), (1508, -136)])
 def test_prefill_matches_oracle(fmt, committed, rows):
     # rows < 0: that many rows with kvx_prefill_plan's split count in place of the
     # reference rule's (which gives 136 and 264 rows a single split); after 1500 tokens the
@@ -93,6 +93,9 @@ def test_int4_prefill_pairs_tiles_under_several_splits():
     # tokens (4 before a page boundary), three splits by kvx_prefill_plan
     assert kvx.prefill_plan(284, 512, H, QH, ko.INT4) == 3
     prefill_case(ko.INT4, 284, -512)
+    # and under the reference rule's single split for 264 rows, after 1500 tokens
+    # (also 4 before a page boundary): the kernel with one register set of pages
+    prefill_case(ko.INT4, 1500, 264)
 
 
 def prefill_case(fmt, committed, rows):
