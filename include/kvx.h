@@ -353,6 +353,19 @@ void kvx_prefix_follow_pages(kvx_prefix *prefix, uint32_t first_page, const uint
 uint64_t kvx_prefix_match(const kvx_prefix *prefix, const uint32_t *prompt, uint64_t n_tokens,
                           uint64_t *blocks, uint32_t capacity, uint32_t *matched);
 
+/* engine::blockImageIdentity (runtime/engine/cache/KvCache.hpp:22-32, KvCache.cpp:29-52): the
+   128-bit identity that the images overlapping tokens [block_begin, block_begin + block_tokens)
+   of a prompt add to that block's key; both halves 0 for a text-only block.  `spans` are the
+   prompt's images sorted by offset (model::ImageSpan, runtime/model/Model.hpp:130-138). */
+typedef struct kvx_image_span {
+  uint32_t offset, tokens;
+  uint32_t grid_height, grid_width;
+  uint64_t digest_lo, digest_hi;
+} kvx_image_span;
+void kvx_block_image_identity(uint64_t block_begin, uint32_t block_tokens,
+                              const kvx_image_span *spans, uint32_t n_spans, uint64_t *lo,
+                              uint64_t *hi);
+
 /* ---- per-sequence page lists: the Request records of engine::Cache
         (runtime/engine/cache/Cache.cpp:143-166, 284-333, 381-413, 700-731, 748-785) ---- */
 typedef struct kvx_sequences kvx_sequences;
@@ -373,6 +386,23 @@ int kvx_sequence_end(kvx_sequences *sequences, uint64_t id);   /* Cache::endRequ
 int kvx_sequence_restore(kvx_sequences *sequences, uint64_t id, uint64_t last_block);
 /* Cache::ensureTokens: pages for `tokens` tokens, or KVX_ENOMEM with nothing taken. */
 int kvx_sequence_ensure_tokens(kvx_sequences *sequences, uint64_t id, uint64_t tokens);
+/* Copy-on-write sharing of a prefix that does not end on a page boundary.  No counterpart in
+   the reference, which shares whole published pages only (Cache.cpp:183-184, :774).
+   kvx_sequence_fork: the empty sequence `id` takes the pages that hold the first `tokens`
+   tokens of `source` by reference (one more active reference each, the partly filled last
+   page included) and the source's blocks over them.
+   kvx_sequence_ensure_writable: call before rows are stored at `token` and after.  When
+   another sequence or the prefix cache also holds the page of `token`, the sequence gets a
+   fresh page, kv_page_copy copies every layer of the shared page into it on `stream`, the
+   sequence's list points at the copy (revision / first_changed say so) and its reference to
+   the shared page is given back; *copied = 1 with the two page ids.  A page held by nobody
+   else is written in place (*copied = 0).  KVX_ESTATE for a published page (its rows are
+   final), KVX_EINVAL when the sequence holds no page for `token`, KVX_ENOMEM with nothing
+   changed when no page is to be had.  Stores into the copy go on `stream` or after it. */
+int kvx_sequence_fork(kvx_sequences *sequences, uint64_t id, uint64_t source, uint64_t tokens);
+int kvx_sequence_ensure_writable(kvx_sequences *sequences, uint64_t id, uint64_t token,
+                                 uint32_t *copied, uint32_t *from_page, uint32_t *to_page,
+                                 void *stream);
 /* Cache::publishCommittedBlocks: every newly full page becomes a block; where the content is
    cached already the sequence moves to the canonical page (copy-free dedup) and the view's
    revision / first_changed say so. */

@@ -1058,6 +1058,7 @@ ko_pool *ko_pool_create(uint32_t page_count, uint64_t bytes_per_page, uint32_t e
 void ko_pool_destroy(ko_pool *p) { delete p; }
 void ko_pool_set_growth_blocked(ko_pool *p, int blocked) { p->growth_blocked = blocked != 0; }
 void ko_pool_set_refused_extent(ko_pool *p, int64_t extent) { p->refused_extent = extent; }
+void ko_pool_set_budget_pages(ko_pool *p, uint32_t pages) { p->budget_pages = pages; }
 
 int ko_pool_acquire(ko_pool *p, uint32_t count, uint32_t *out) {
   // KvPool.cpp:35-72

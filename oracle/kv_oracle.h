@@ -278,6 +278,7 @@ ko_pool *ko_pool_create(uint32_t page_count, uint64_t bytes_per_page, uint32_t e
 void ko_pool_destroy(ko_pool *p);
 void ko_pool_set_growth_blocked(ko_pool *p, int blocked);
 void ko_pool_set_refused_extent(ko_pool *p, int64_t extent); /* -1 = none */
+void ko_pool_set_budget_pages(ko_pool *p, uint32_t pages);  /* the storage's budget moves */
 /* returns count granted (== count) or -1 denied, -2 ids ran out */
 int ko_pool_acquire(ko_pool *p, uint32_t count, uint32_t *pages);
 int ko_pool_retain(ko_pool *p, uint32_t page, int prefix_owner);   /* 0 ok, -1 logic error */

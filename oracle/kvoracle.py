@@ -217,6 +217,7 @@ def _declare(L):
     L.ko_pool_destroy.argtypes = [vp]
     L.ko_pool_set_growth_blocked.argtypes = [vp, C.c_int]
     L.ko_pool_set_refused_extent.argtypes = [vp, C.c_int64]
+    L.ko_pool_set_budget_pages.argtypes = [vp, u32]
     L.ko_pool_acquire.argtypes = [vp, u32, vp]
     L.ko_pool_retain.argtypes = [vp, u32, C.c_int]
     L.ko_pool_release.argtypes = [vp, u32, C.c_int]

@@ -302,3 +302,33 @@ def tree_masks(parents, none=0xFFFFFFFF):
             parent = parents[parent]
         masks.append(mask)
     return masks
+
+
+def block_image_identity(block_begin, block_tokens, spans):
+    """Restates blockImageIdentity (runtime/engine/cache/KvCache.cpp:29-52): (lo, hi) of a block
+    of `block_tokens` tokens at `block_begin`; spans are (offset, tokens, grid height, grid
+    width, digest lo, digest hi) sorted by offset.  Only spans that overlap the block count;
+    a block without any has identity (0, 0).
+
+    The reference holds no golden value of this function, only the properties of
+    dev/tests/engine/kv_page_cache_test.cpp:44-69 (zero for text, zero after the image,
+    dependence on digest and alignment, spans outside the block ignored): PARITY UNPINNED at
+    the bit level, pinned to those properties in tests/test_prefix_cache.py."""
+    mask = (1 << 64) - 1
+
+    def mix(h, v):
+        return h ^ ((v + 0x9E3779B97F4A7C15 + ((h << 6) & mask) + (h >> 2)) & mask)
+
+    lo = hi = 0
+    end = block_begin + block_tokens
+    for offset, tokens, height, width, digest_lo, digest_hi in spans:
+        if offset >= end:
+            break
+        if ((offset + tokens) & 0xFFFFFFFF) <= block_begin:
+            continue
+        lo = lo or 0x243F6A8885A308D3
+        hi = hi or 0x13198A2E03707344
+        for value in (digest_lo, digest_hi, (height << 32) | width, (offset << 32) | tokens, block_begin):
+            lo = mix(lo, value)
+            hi = mix(hi, ~value & mask)
+    return lo, hi

@@ -1,298 +1,306 @@
+// The page pool; the header describes its bookkeeping.
 #include "kvx_pool.h"
 
 #include <algorithm>
 #include <chrono>
-#include <numeric>
 
 namespace kvx {
 
 namespace {
-using Clock = std::chrono::steady_clock;
-double ms_since(Clock::time_point start) {
-  return std::chrono::duration<double, std::milli>(Clock::now() - start).count();
+double elapsed_ms(std::chrono::steady_clock::time_point since) {
+  return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - since).count();
 }
 }  // namespace
 
 KvPool::KvPool(ExtentStorage &storage, uint32_t runway_pages)
-    : storage_(storage), extent_pages_(storage.extent_pages()), pages_(storage.page_count()) {
-  if (pages_.empty() || !storage.bytes_per_page() || !extent_pages_ ||
-      pages_.size() % extent_pages_ || runway_pages > pages_.size()) {
+    : storage_(storage), span_(storage.extent_pages()) {
+  const uint32_t pages = storage.page_count();
+  if (!pages || !span_ || pages % span_ || !storage.bytes_per_page() || runway_pages > pages) {
     status_ = KVX_EINVAL;
     return;
   }
-  extents_.resize(pages_.size() / extent_pages_);
-  for (uint32_t extent = 0; extent * extent_pages_ < runway_pages; ++extent) {
-    if (int rc = allocate_extent(extent)) {
-      status_ = rc;
-      return;
-    }
-  }
+  page_.resize(pages);
+  extent_.resize(pages / span_);
+  const uint32_t runway_extents = (runway_pages + span_ - 1) / span_;
+  for (uint32_t x = 0; x < runway_extents && status_ == KVX_OK; ++x) status_ = bring_in(x);
 }
 
 uint64_t KvPool::allocated_bytes() const {
-  return uint64_t(allocated_extents_) * extent_pages_ * storage_.bytes_per_page();
+  return uint64_t(resident_) * span_ * storage_.bytes_per_page();
 }
 
-// A freed page goes to the head of its extent's list, so the page released
-// last is handed out first.
-void KvPool::list_insert(uint32_t page) {
-  Page &p = pages_[page];
-  Extent &e = extents_[extent_of(page)];
-  p.prev = kNone;
-  p.next = e.free_head;
-  p.listed = true;
-  if (e.free_head != kNone) pages_[e.free_head].prev = page;
-  e.free_head = page;
-  ++e.free_count;
-  ++free_pages_;
-  packing_ = kNone;
-}
+// ---- free stacks ---------------------------------------------------------------
 
-void KvPool::list_remove(uint32_t page) {
-  Page &p = pages_[page];
-  Extent &e = extents_[extent_of(page)];
-  if (p.prev == kNone) e.free_head = p.next;
-  else pages_[p.prev].next = p.next;
-  if (p.next != kNone) pages_[p.next].prev = p.prev;
-  p.prev = p.next = kNone;
-  p.listed = false;
-  --e.free_count;
-  --free_pages_;
-}
-
-// The allocated extent with the most held pages that still has a free one;
-// ties go to the lowest index and an empty extent loses to any used one.
-uint32_t KvPool::packing_extent() {
-  if (packing_ != kNone && extents_[packing_].free_count) return packing_;
-  uint32_t best = kNone;
-  for (uint32_t i = 0; i < extents_.size(); ++i)
-    if (extents_[i].free_count && (best == kNone || extents_[i].used > extents_[best].used))
-      best = i;
-  packing_ = best;
-  return best;
-}
-
-void KvPool::mark_used(uint32_t page) {
-  const uint32_t x = extent_of(page);
-  if (pages_[page].listed) {
-    list_remove(page);
-    if (x != packing_) packing_ = kNone;
+void KvPool::stack_push(uint32_t page) {
+  ExtentBook &x = extent_[extent_of(page)];
+  page_[page].ticket = ++next_ticket_;  // never 0, which means "not on a stack"
+  x.stack.push_back({next_ticket_, page});
+  ++x.free;
+  ++free_total_;
+  if (x.stack.size() > 2u * span_) {  // squeeze the stale entries out, order kept
+    size_t kept = 0;
+    for (const FreeEntry &e : x.stack)
+      if (live(e)) x.stack[kept++] = e;
+    x.stack.resize(kept);
   }
-  if (!extents_[x].used) set_reclaimable(x, false);
-  ++extents_[x].used;
 }
 
-void KvPool::mark_free(uint32_t page) {
-  const uint32_t x = extent_of(page);
-  --extents_[x].used;
-  list_insert(page);
-  if (!extents_[x].used) set_reclaimable(x, true);
+uint32_t KvPool::stack_pop(uint32_t extent) {
+  ExtentBook &x = extent_[extent];
+  while (!live(x.stack.back())) x.stack.pop_back();
+  const uint32_t page = x.stack.back().page;
+  x.stack.pop_back();
+  page_[page].ticket = 0;
+  --x.free;
+  --free_total_;
+  return page;
 }
 
-void KvPool::set_reclaimable(uint32_t x, bool on) {
-  Extent &e = extents_[x];
-  if (e.reclaimable == on) return;
-  if (on) {  // newest at the head
-    e.prev_reclaimable = kNone;
-    e.next_reclaimable = reclaimable_head_;
-    if (reclaimable_head_ != kNone) extents_[reclaimable_head_].prev_reclaimable = x;
-    reclaimable_head_ = x;
-    ++reclaimable_count_;
-  } else {
-    if (e.prev_reclaimable == kNone) reclaimable_head_ = e.next_reclaimable;
-    else extents_[e.prev_reclaimable].next_reclaimable = e.next_reclaimable;
-    if (e.next_reclaimable != kNone)
-      extents_[e.next_reclaimable].prev_reclaimable = e.prev_reclaimable;
-    e.prev_reclaimable = e.next_reclaimable = kNone;
-    --reclaimable_count_;
+void KvPool::stack_forget(uint32_t page) {
+  page_[page].ticket = 0;
+  --extent_[extent_of(page)].free;
+  --free_total_;
+}
+
+void KvPool::stack_peek(uint32_t extent, uint32_t count, std::vector<uint32_t> *out) const {
+  const ExtentBook &x = extent_[extent];
+  for (size_t i = x.stack.size(); i > 0 && count; --i)
+    if (live(x.stack[i - 1])) {
+      out->push_back(x.stack[i - 1].page);
+      --count;
+    }
+}
+
+// ---- the fill order -------------------------------------------------------------
+
+// Moves an extent to its place in the fill order after `held` or `free` changed;
+// the arguments are what they were when it was last filed.
+void KvPool::refile(uint32_t extent, uint32_t held_before, uint32_t free_before) {
+  const ExtentBook &x = extent_[extent];
+  if (free_before) fill_order_.erase(FillKey(span_ - held_before, extent));
+  if (x.resident && x.free) fill_order_.insert(FillKey(span_ - x.held, extent));
+}
+
+void KvPool::hold(uint32_t page) {
+  const uint32_t e = extent_of(page);
+  ExtentBook &x = extent_[e];
+  const uint32_t held = x.held, free = x.free;
+  if (page_[page].ticket) stack_forget(page);
+  if (!x.held++) {
+    x.idle_since = 0;
+    --idle_;
   }
-  e.reclaimable = on;
+  refile(e, held, free);
 }
 
-void KvPool::set_allocated(uint32_t x, bool on) {
-  Extent &e = extents_[x];
-  const uint32_t first = x * extent_pages_;
-  if (on) {
-    e.allocated = true;
-    ++allocated_extents_;
-    // Inserted highest first so the lowest page ends at the head.
-    for (uint32_t page = first + extent_pages_; page > first;) list_insert(--page);
-    set_reclaimable(x, true);
-    return;
+void KvPool::unhold(uint32_t page) {
+  const uint32_t e = extent_of(page);
+  ExtentBook &x = extent_[e];
+  const uint32_t held = x.held, free = x.free;
+  stack_push(page);
+  if (!--x.held) {
+    x.idle_since = ++idle_clock_;
+    ++idle_;
   }
-  set_reclaimable(x, false);
-  for (uint32_t page = first; page < first + extent_pages_; ++page) list_remove(page);
-  e.allocated = false;
-  --allocated_extents_;
+  refile(e, held, free);
 }
 
-int KvPool::allocate_extent(uint32_t x) {
-  const auto start = Clock::now();
-  if (int rc = storage_.allocate_extent(x)) return rc;
+// ---- extents --------------------------------------------------------------------
+
+int KvPool::bring_in(uint32_t extent) {
+  const auto start = std::chrono::steady_clock::now();
+  if (const int rc = storage_.allocate_extent(extent)) return rc;
+  allocate_max_ms_ = std::max(allocate_max_ms_, elapsed_ms(start));
   ++allocations_;
-  allocate_max_ms_ = std::max(allocate_max_ms_, ms_since(start));
-  set_allocated(x, true);
+  ExtentBook &x = extent_[extent];
+  x.resident = true;
+  ++resident_;
+  x.idle_since = ++idle_clock_;
+  ++idle_;
+  // Highest page first, so that the lowest ends on top.
+  for (uint32_t i = span_; i > 0; --i) stack_push(extent * span_ + i - 1);
+  refile(extent, 0, 0);
   return KVX_OK;
 }
 
-int KvPool::release_extent(uint32_t x) {
-  const auto start = Clock::now();
-  if (int rc = storage_.release_extent(x)) return rc;  // a refusal changes nothing
+int KvPool::give_up(uint32_t extent) {
+  const auto start = std::chrono::steady_clock::now();
+  if (const int rc = storage_.release_extent(extent)) return rc;  // a refusal changes nothing
+  release_max_ms_ = std::max(release_max_ms_, elapsed_ms(start));
   ++releases_;
-  release_max_ms_ = std::max(release_max_ms_, ms_since(start));
-  set_allocated(x, false);
+  ExtentBook &x = extent_[extent];
+  const uint32_t free = x.free;
+  for (uint32_t i = 0; i < span_; ++i) page_[extent * span_ + i].ticket = 0;
+  free_total_ -= x.free;
+  x.free = 0;
+  x.stack.clear();
+  x.resident = false;
+  --resident_;
+  x.idle_since = 0;
+  --idle_;
+  refile(extent, 0, free);
   return KVX_OK;
 }
+
+// ---- references -------------------------------------------------------------------
 
 int KvPool::acquire(uint32_t count, uint32_t *out) {
-  if (!count) return KVX_OK;
-  std::vector<uint32_t> selected;
-  selected.reserve(count);
-  auto give_back = [&] {
-    for (auto it = selected.rbegin(); it != selected.rend(); ++it) list_insert(*it);
-  };
-  while (selected.size() < count) {
-    if (free_pages_) {
-      const uint32_t page = extents_[packing_extent()].free_head;
-      list_remove(page);
-      selected.push_back(page);
+  // Pages are only taken off their stacks here and get their reference once all
+  // of them are found: a refused growth puts them back in reverse, which leaves
+  // every stack, the fill order and the idle order as they were.
+  std::vector<uint32_t> taken;
+  taken.reserve(count);
+  int rc = KVX_OK;
+  while (taken.size() < count) {
+    if (!fill_order_.empty()) {
+      const uint32_t e = fill_order_.begin()->second;
+      const uint32_t held = extent_[e].held, free = extent_[e].free;
+      taken.push_back(stack_pop(e));
+      refile(e, held, free);
       continue;
     }
-    uint32_t x = kNone;
-    for (uint32_t i = 0; i < extents_.size(); ++i)
-      if (!extents_[i].allocated) {
-        x = i;
-        break;
-      }
-    if (x == kNone) {  // page ids ran out before the budget did
-      give_back();
-      return KVX_ESTATE;
-    }
-    if (int rc = allocate_extent(x)) {
-      // Extents this call did allocate stay, reclaimable, for the retry.
-      give_back();
-      return rc;
-    }
+    uint32_t absent = 0;
+    while (absent < extent_.size() && extent_[absent].resident) ++absent;
+    rc = absent == extent_.size() ? KVX_ESTATE  // page ids ran out before the budget did
+                                  : bring_in(absent);
+    if (rc) break;
   }
-  for (uint32_t page : selected) {
-    mark_used(page);
-    pages_[page].active = 1;
-    ++active_pages_;
+  if (rc) {
+    // Extents this call did bring in stay, idle, for the retry.
+    for (size_t i = taken.size(); i > 0; --i) {
+      const uint32_t e = extent_of(taken[i - 1]);
+      const uint32_t held = extent_[e].held, free = extent_[e].free;
+      stack_push(taken[i - 1]);
+      refile(e, held, free);
+    }
+    return rc;
   }
-  std::copy(selected.begin(), selected.end(), out);
+  for (uint32_t i = 0; i < count; ++i) {
+    hold(taken[i]);
+    page_[taken[i]].holders = 1;
+    out[i] = taken[i];
+  }
+  active_total_ += count;
   return KVX_OK;
 }
 
 int KvPool::retain(uint32_t page, bool prefix_owner) {
-  if (page >= pages_.size()) return KVX_ERANGE;
-  if (!extents_[extent_of(page)].allocated) return KVX_ESTATE;
-  Page &p = pages_[page];
-  if (prefix_owner && p.prefix) return KVX_ESTATE;
-  if (!prefix_owner && p.active == 0xffffffffu) return KVX_ESTATE;
-  if (is_free(page)) mark_used(page);
+  if (page >= page_.size()) return KVX_ERANGE;
+  if (!extent_[extent_of(page)].resident) return KVX_ESTATE;
+  PageBook &p = page_[page];
+  if (prefix_owner ? p.cached : p.holders == UINT32_MAX) return KVX_ESTATE;
+  if (!p.held()) hold(page);
   if (prefix_owner) {
-    p.prefix = true;
-    ++prefix_pages_;
-  } else if (!p.active++) {
-    ++active_pages_;
+    p.cached = true;
+    ++cached_total_;
+  } else if (!p.holders++) {
+    ++active_total_;
   }
   return KVX_OK;
 }
 
 int KvPool::release(uint32_t page, bool prefix_owner) {
-  if (page >= pages_.size()) return KVX_ERANGE;
-  Page &p = pages_[page];
-  if (prefix_owner ? !p.prefix : !p.active) return KVX_ESTATE;
+  if (page >= page_.size()) return KVX_ERANGE;
+  PageBook &p = page_[page];
+  if (prefix_owner ? !p.cached : !p.holders) return KVX_ESTATE;
   if (prefix_owner) {
-    p.prefix = false;
-    --prefix_pages_;
-  } else if (!--p.active) {
-    --active_pages_;
+    p.cached = false;
+    --cached_total_;
+  } else if (!--p.holders) {
+    --active_total_;
   }
-  if (is_free(page)) mark_free(page);
+  if (!p.held()) unhold(page);
   return KVX_OK;
 }
 
+// ---- giving memory back -----------------------------------------------------------
+
 int KvPool::reclaim_empty(bool keep_runway, uint32_t limit, uint64_t *released) {
-  uint32_t reclaimed = 0;
-  bool kept = false;
+  std::vector<std::pair<uint64_t, uint32_t>> idle;  // (idle since, extent)
+  for (uint32_t e = 0; e < extent_.size(); ++e)
+    if (extent_[e].resident && !extent_[e].held) idle.emplace_back(extent_[e].idle_since, e);
+  std::sort(idle.begin(), idle.end(), std::greater<>());  // latest first
+  uint32_t given = 0;
   int rc = KVX_OK;
-  for (uint32_t x = reclaimable_head_; x != kNone && reclaimed < limit;) {
-    const uint32_t next = extents_[x].next_reclaimable;
-    if (keep_runway && !kept) {
-      kept = true;
-    } else {
-      if ((rc = release_extent(x))) break;
-      ++reclaimed;
-    }
-    x = next;
+  // The extent that fell idle last stays as the runway when asked to.
+  for (size_t i = keep_runway ? 1 : 0; i < idle.size() && given < limit; ++i) {
+    if ((rc = give_up(idle[i].second))) break;
+    ++given;
   }
-  if (released) *released = uint64_t(reclaimed) * extent_pages_ * storage_.bytes_per_page();
+  if (released) *released = uint64_t(given) * span_ * storage_.bytes_per_page();
   return rc;
 }
 
 int KvPool::compact_extent(const uint32_t *fixed, uint32_t n_fixed, PageMoves *moves) {
   *moves = {};
-  // Pages move only into extents that already hold pages.
-  uint32_t free_in_use = 0;
-  for (const Extent &e : extents_)
-    if (e.allocated && e.used) free_in_use += e.free_count;
-  uint32_t emptied = kNone;
-  for (uint32_t i = 0; i < extents_.size(); ++i) {
-    const Extent &e = extents_[i];
-    if (!e.allocated || !e.used || e.used > free_in_use - e.free_count) continue;
-    if (emptied != kNone && e.used >= extents_[emptied].used) continue;
-    bool pinned = false;
-    for (uint32_t f = 0; f < n_fixed && !pinned; ++f) pinned = extent_of(fixed[f]) == i;
-    if (!pinned) emptied = i;
+  // Pages only move into extents that hold pages already, so what counts is the
+  // free room of those.
+  uint32_t room = 0;
+  for (const ExtentBook &x : extent_)
+    if (x.resident && x.held) room += x.free;
+  std::vector<bool> pinned(extent_.size(), false);
+  for (uint32_t i = 0; i < n_fixed; ++i)
+    if (fixed[i] < page_.size()) pinned[extent_of(fixed[i])] = true;
+  // The extent to empty: the one with the fewest held pages that the others can
+  // take in, the lowest index among equals.
+  uint32_t victim = UINT32_MAX;
+  for (uint32_t e = 0; e < extent_.size(); ++e) {
+    const ExtentBook &x = extent_[e];
+    if (!x.resident || !x.held || pinned[e] || x.held > room - x.free) continue;
+    if (victim == UINT32_MAX || x.held < extent_[victim].held) victim = e;
   }
-  if (emptied == kNone) return KVX_OK;
+  if (victim == UINT32_MAX) return KVX_OK;
 
-  std::vector<uint32_t> receivers;
-  for (uint32_t i = 0; i < extents_.size(); ++i) {
-    const Extent &e = extents_[i];
-    if (i != emptied && e.allocated && e.used && e.free_count) receivers.push_back(i);
+  // Receivers fullest first (lowest index among equals); each gives its free
+  // pages in the order an acquisition would.
+  std::vector<std::pair<uint32_t, uint32_t>> receivers;  // (unheld pages, extent)
+  for (uint32_t e = 0; e < extent_.size(); ++e) {
+    const ExtentBook &x = extent_[e];
+    if (e != victim && x.resident && x.held && x.free) receivers.emplace_back(span_ - x.held, e);
   }
-  std::stable_sort(receivers.begin(), receivers.end(), [&](uint32_t a, uint32_t b) {
-    return extents_[a].used > extents_[b].used;
-  });
-  const uint32_t first = emptied * extent_pages_;
+  std::sort(receivers.begin(), receivers.end());
+  std::vector<uint32_t> landing;
+  uint32_t wanted = extent_[victim].held;
+  for (size_t r = 0; r < receivers.size() && wanted; ++r) {
+    const uint32_t take = std::min(wanted, extent_[receivers[r].second].free);
+    stack_peek(receivers[r].second, take, &landing);
+    wanted -= take;
+  }
+  // One sweep over the victim, lowest page first, pairs every held page with the
+  // next landing place.
   std::vector<kvx_page_copy> copies;
-  size_t r = 0;
-  uint32_t to = extents_[receivers[r]].free_head;
-  for (uint32_t page = first; page < first + extent_pages_; ++page) {
-    if (is_free(page)) continue;
-    while (to == kNone) to = extents_[receivers[++r]].free_head;
-    copies.push_back({page, to});
-    to = pages_[to].next;
-  }
-  if (int rc = storage_.copy_pages(copies.data(), uint32_t(copies.size()))) return rc;
+  copies.reserve(landing.size());
+  const uint32_t first = victim * span_;
+  for (uint32_t page = first; page < first + span_; ++page)
+    if (page_[page].held()) copies.push_back({page, landing[copies.size()]});
+  if (const int rc = storage_.copy_pages(copies.data(), uint32_t(copies.size()))) return rc;
 
   moves->first_page = first;
-  moves->destinations.resize(extent_pages_);
-  std::iota(moves->destinations.begin(), moves->destinations.end(), first);
+  moves->destinations.resize(span_);
+  for (uint32_t i = 0; i < span_; ++i) moves->destinations[i] = first + i;
   for (const kvx_page_copy &c : copies) {
-    mark_used(c.to);
-    pages_[c.to].active = pages_[c.from].active;
-    pages_[c.from].active = 0;
-    pages_[c.to].prefix = pages_[c.from].prefix;
-    pages_[c.from].prefix = false;
-    mark_free(c.from);
+    hold(c.to);
+    page_[c.to].holders = page_[c.from].holders;
+    page_[c.to].cached = page_[c.from].cached;
+    page_[c.from].holders = 0;
+    page_[c.from].cached = false;
+    unhold(c.from);
     moves->destinations[c.from - first] = c.to;
   }
   moves->moved = uint32_t(copies.size());
-  ++compactions_;
   moved_ += copies.size();
+  ++compactions_;
   return KVX_OK;
 }
 
 void KvPool::snapshot(kvx_pool_snapshot *out) const {
-  out->pages_allocated = allocated_extents_ * extent_pages_;
-  out->pages_free = free_pages_;
-  out->pages_active = active_pages_;
-  out->pages_prefix = prefix_pages_;
-  out->allocated_bytes = allocated_bytes();
-  out->reclaimable_bytes = uint64_t(reclaimable_count_) * extent_pages_ * storage_.bytes_per_page();
+  const uint64_t extent_bytes = uint64_t(span_) * storage_.bytes_per_page();
+  out->pages_allocated = resident_ * span_;
+  out->pages_free = free_total_;
+  out->pages_active = active_total_;
+  out->pages_prefix = cached_total_;
+  out->allocated_bytes = resident_ * extent_bytes;
+  out->reclaimable_bytes = idle_ * extent_bytes;
   out->extent_allocations = allocations_;
   out->extent_releases = releases_;
   out->extent_allocate_max_ms = allocate_max_ms_;

@@ -4,21 +4,32 @@
 #include <algorithm>
 
 namespace kvx {
-namespace {
 
-// runtime/engine/cache/KvCache.cpp:12-25
-uint64_t mix(uint64_t hash, uint64_t value) {
-  hash ^= value + 0x9e3779b97f4a7c15ULL + (hash << 6) + (hash >> 2);
-  return hash;
-}
-uint64_t index_hash(uint64_t parent_hash, const uint32_t *tokens, uint64_t lo, uint64_t hi) {
-  uint64_t hash = mix(0x6a09e667f3bcc909ULL, parent_hash);
-  for (uint32_t i = 0; i < KVX_PAGE_TOKENS; ++i) hash = mix(hash, tokens[i]);
-  hash = mix(hash, lo);
-  return mix(hash, hi);
+// A 64-bit FNV-1a over the key's words.  The hash only spreads keys over the
+// map's buckets; equality is the map's comparison of whole keys.
+size_t PrefixCache::ContentKeyHash::operator()(const ContentKey &key) const {
+  uint64_t h = 0xcbf29ce484222325ull;
+  auto fold = [&h](uint64_t word) {
+    h ^= word;
+    h *= 0x100000001b3ull;
+  };
+  fold(key.parent);
+  for (uint32_t i = 0; i < KVX_PAGE_TOKENS; i += 2)
+    fold(uint64_t(key.tokens[i]) | uint64_t(key.tokens[i + 1]) << 32);
+  fold(key.image_lo);
+  fold(key.image_hi);
+  return size_t(h ^ (h >> 29));
 }
 
-}  // namespace
+PrefixCache::ContentKey PrefixCache::key_of(uint64_t parent, const uint32_t *tokens,
+                                            uint64_t image_lo, uint64_t image_hi) {
+  ContentKey key;
+  key.parent = parent;
+  key.image_lo = image_lo;
+  key.image_hi = image_hi;
+  std::copy(tokens, tokens + KVX_PAGE_TOKENS, key.tokens.begin());
+  return key;
+}
 
 PrefixCache::~PrefixCache() {
   for (const auto &entry : blocks_)
@@ -47,24 +58,16 @@ void PrefixCache::reindex(Block &b) {
   b.listed_at = b.last_used;
 }
 
+// A block id is never reused, so a key under a parent that no longer exists
+// cannot be in the map: an unknown parent simply finds nothing.
 bool PrefixCache::find(uint64_t parent, const uint32_t *tokens, uint32_t n_tokens, uint64_t image_lo,
                        uint64_t image_hi, uint64_t *block, uint32_t *page) const {
   if (n_tokens != KVX_PAGE_TOKENS) return false;
-  const Block *above = parent ? get(parent) : nullptr;
-  if (parent && !above) return false;
-  const uint64_t hash = index_hash(above ? above->index_hash : 0, tokens, image_lo, image_hi);
-  const auto range = index_.equal_range(hash);
-  for (auto candidate = range.first; candidate != range.second; ++candidate) {
-    const Block &entry = *get(candidate->second);
-    // Hashes filter candidates; equality needs the complete key.
-    if (entry.parent == parent && entry.image_lo == image_lo && entry.image_hi == image_hi &&
-        std::equal(entry.tokens.begin(), entry.tokens.end(), tokens)) {
-      if (block) *block = entry.id;
-      if (page) *page = entry.page;
-      return true;
-    }
-  }
-  return false;
+  const auto hit = by_content_.find(key_of(parent, tokens, image_lo, image_hi));
+  if (hit == by_content_.end()) return false;
+  if (block) *block = hit->second;
+  if (page) *page = get(hit->second)->page;
+  return true;
 }
 
 int PrefixCache::insert(uint64_t parent, const uint32_t *tokens, uint32_t n_tokens, uint32_t page,
@@ -72,38 +75,36 @@ int PrefixCache::insert(uint64_t parent, const uint32_t *tokens, uint32_t n_toke
                         uint32_t *canonical_page) {
   if (n_tokens != KVX_PAGE_TOKENS) return KVX_EINVAL;  // one full page
   if (page >= pool_.page_count()) return KVX_ERANGE;
-  uint64_t existing = 0;
-  uint32_t existing_page = kNoPage;
-  if (find(parent, tokens, n_tokens, image_lo, image_hi, &existing, &existing_page)) {
-    if (block) *block = existing;
-    if (canonical_page) *canonical_page = existing_page;
+  // One probe either finds the content or reserves its place.
+  const auto placed = by_content_.try_emplace(key_of(parent, tokens, image_lo, image_hi), 0);
+  if (!placed.second) {  // cached already: the caller gets the canonical block and page
+    if (block) *block = placed.first->second;
+    if (canonical_page) *canonical_page = get(placed.first->second)->page;
     return KVX_OK;
   }
   Block *above = parent ? get(parent) : nullptr;
-  if (parent && !above) return KVX_EINVAL;  // unknown parent
-  if (block_on_page_[page]) return KVX_ESTATE;  // the page already holds a block
-  if (const int rc = pool_.retain(page, true)) return rc;
-  Block entry;
-  entry.id = next_id_++;
-  entry.parent = parent;
-  entry.index_hash = index_hash(above ? above->index_hash : 0, tokens, image_lo, image_hi);
-  std::copy(tokens, tokens + KVX_PAGE_TOKENS, entry.tokens.begin());
-  entry.image_lo = image_lo;
-  entry.image_hi = image_hi;
-  entry.page = page;
-  entry.depth = above ? above->depth + 1 : 1;
-  const uint64_t id = entry.id;
-  index_.emplace(entry.index_hash, id);
-  blocks_.emplace(id, entry);
-  block_on_page_[page] = id;
-  if (parent) {
-    Block &p = *get(parent);
-    ++p.children;
-    reindex(p);
+  int rc = KVX_OK;
+  if (parent && !above) rc = KVX_EINVAL;           // unknown parent
+  else if (block_on_page_[page]) rc = KVX_ESTATE;  // the page already holds a block
+  else rc = pool_.retain(page, true);
+  if (rc) {
+    by_content_.erase(placed.first);
+    return rc;
   }
-  Block &placed = *get(id);
-  placed.last_used = ++clock_;
-  reindex(placed);
+  const uint64_t id = next_id_++;
+  placed.first->second = id;
+  Block &fresh = blocks_[id];
+  fresh.id = id;
+  fresh.key = placed.first->first;
+  fresh.page = page;
+  fresh.depth = above ? above->depth + 1 : 1;
+  fresh.last_used = ++clock_;
+  block_on_page_[page] = id;
+  if (above) {  // no longer a leaf
+    ++above->children;
+    reindex(*above);
+  }
+  reindex(fresh);
   ++generation_;
   if (block) *block = id;
   if (canonical_page) *canonical_page = page;
@@ -127,7 +128,7 @@ int PrefixCache::chain(uint64_t block, std::vector<uint64_t> *blocks,
     if (!b) return KVX_ESTATE;
     (*blocks)[index - 1] = b->id;
     (*pages)[index - 1] = b->page;
-    b = b->parent ? get(b->parent) : nullptr;
+    b = b->key.parent ? get(b->key.parent) : nullptr;
   }
   return b ? KVX_ESTATE : KVX_OK;
 }
@@ -186,15 +187,10 @@ int PrefixCache::erase(uint64_t block) {
   Block *b = get(block);
   if (!b) return KVX_ERANGE;
   if (b->children || b->active_users) return KVX_ESTATE;  // a referenced block stays
-  const uint64_t parent = b->parent, hash = b->index_hash, last_used = b->last_used;
+  const uint64_t parent = b->key.parent, last_used = b->last_used;
   const uint32_t page = b->page;
   if (b->listed) leaves_.erase(std::make_pair(b->listed_at, b->id));
-  const auto range = index_.equal_range(hash);
-  for (auto it = range.first; it != range.second; ++it)
-    if (it->second == block) {
-      index_.erase(it);
-      break;
-    }
+  by_content_.erase(b->key);
   blocks_.erase(block);
   ++generation_;
   block_on_page_[page] = 0;
@@ -288,6 +284,57 @@ int SequenceCache::ensure_tokens(uint64_t id, uint64_t tokens) {
   if (const int rc = pool_.acquire(uint32_t(acquired.size()), acquired.data())) return rc;
   s.pages.insert(s.pages.end(), acquired.begin(), acquired.end());
   changed(s, previous);
+  return KVX_OK;
+}
+
+int SequenceCache::fork(uint64_t id, uint64_t source, uint64_t tokens) {
+  const auto found = sequences_.find(id), origin = sequences_.find(source);
+  if (found == sequences_.end() || origin == sequences_.end()) return KVX_ERANGE;
+  Sequence &s = found->second;
+  const Sequence &from = origin->second;
+  if (id == source || !s.pages.empty() || !s.blocks.empty()) return KVX_ESTATE;
+  const uint64_t pages = (tokens + KVX_PAGE_TOKENS - 1) / KVX_PAGE_TOKENS;
+  if (pages > from.pages.size()) return KVX_EINVAL;  // more than the source holds
+  if (!pages) return KVX_OK;
+  for (uint64_t i = 0; i < pages; ++i)
+    if (const int rc = pool_.retain(from.pages[i], false)) {
+      while (i > 0) pool_.release(from.pages[--i], false);
+      return rc;
+    }
+  s.pages.assign(from.pages.begin(), from.pages.begin() + pages);
+  // Blocks exist for published whole pages only.
+  const uint64_t blocks = std::min<uint64_t>(tokens / KVX_PAGE_TOKENS, from.blocks.size());
+  s.blocks.assign(from.blocks.begin(), from.blocks.begin() + blocks);
+  if (blocks) prefix_.retain_active(s.blocks.back());
+  changed(s, 0);
+  return KVX_OK;
+}
+
+int SequenceCache::ensure_writable(uint64_t id, uint64_t token, bool *copied, uint32_t *from,
+                                   uint32_t *to) {
+  *copied = false;
+  const auto found = sequences_.find(id);
+  if (found == sequences_.end()) return KVX_ERANGE;
+  Sequence &s = found->second;
+  const uint64_t logical = token / KVX_PAGE_TOKENS;
+  if (logical >= s.pages.size()) return KVX_EINVAL;  // ensure_tokens comes first
+  // A published page never changes again: rows stored at or after `token` lie past it.
+  if (logical < s.blocks.size()) return KVX_ESTATE;
+  const uint32_t shared = s.pages[logical];
+  if (!pool_.page_shared(shared)) return KVX_OK;
+  uint32_t mine = 0;
+  if (pool_.acquire(1, &mine)) return KVX_ENOMEM;  // refused growth, or no page id left
+  const kvx_page_copy copy{shared, mine};
+  if (const int rc = pool_.copy_pages(&copy, 1)) {
+    pool_.release(mine, false);
+    return rc;
+  }
+  s.pages[logical] = mine;
+  changed(s, uint32_t(logical));
+  pool_.release(shared, false);
+  *copied = true;
+  *from = shared;
+  *to = mine;
   return KVX_OK;
 }
 

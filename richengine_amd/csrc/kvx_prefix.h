@@ -6,6 +6,11 @@
 // identity); a block owns one prefix reference of its page in the pool.  The
 // disk tier, recurrent states and poisoning of the reference are not part of
 // the KV data path and have no counterpart here.
+//
+// Blocks are found through one hash map whose key is the whole content key
+// (parent block id, the 32 tokens, both halves of the image identity), so a
+// lookup is a single probe that compares complete keys, and a block's place in
+// the tree is its parent's id, not a hash chained down from the root.
 #pragma once
 
 #include <array>
@@ -53,10 +58,22 @@ public:
   uint64_t block_count() const { return blocks_.size(); }
 
 private:
-  struct Block {
-    uint64_t id = 0, parent = 0, index_hash = 0;
+  struct ContentKey {
+    uint64_t parent = 0, image_lo = 0, image_hi = 0;
     std::array<uint32_t, KVX_PAGE_TOKENS> tokens{};
-    uint64_t image_lo = 0, image_hi = 0;
+    bool operator==(const ContentKey &o) const {
+      return parent == o.parent && image_lo == o.image_lo && image_hi == o.image_hi &&
+             tokens == o.tokens;
+    }
+  };
+  struct ContentKeyHash {
+    size_t operator()(const ContentKey &key) const;
+  };
+  static ContentKey key_of(uint64_t parent, const uint32_t *tokens, uint64_t image_lo,
+                           uint64_t image_hi);
+  struct Block {
+    uint64_t id = 0;
+    ContentKey key;
     uint32_t page = kNoPage, depth = 0, children = 0, active_users = 0;
     uint64_t last_used = 0, listed_at = 0;
     bool listed = false;
@@ -67,7 +84,7 @@ private:
 
   KvPool &pool_;
   std::unordered_map<uint64_t, Block> blocks_;
-  std::unordered_multimap<uint64_t, uint64_t> index_;
+  std::unordered_map<ContentKey, uint64_t, ContentKeyHash> by_content_;  // key -> block id
   std::map<std::pair<uint64_t, uint64_t>, uint64_t> leaves_;  // (last used, id) -> id
   std::vector<uint64_t> block_on_page_;
   uint64_t next_id_ = 1, clock_ = 0, generation_ = 0;
@@ -82,6 +99,15 @@ public:
   int end(uint64_t id);                                     // Cache::endRequest
   int restore(uint64_t id, uint64_t last_block);            // Cache::restoreRequest, resident chain
   int ensure_tokens(uint64_t id, uint64_t tokens);          // Cache::ensureTokens
+  // Copy-on-write sharing, which the reference does not have (it shares whole
+  // published pages only, Cache.cpp:183-184, :774).  fork: the empty sequence `id`
+  // takes the pages that hold the first `tokens` tokens of `source` by reference,
+  // the partly filled last one included, and the source's blocks over those pages.
+  // ensure_writable: before rows are stored at `token` and after, the page that
+  // holds it is replaced by a private copy (all layers, on the pool's copy stream)
+  // when anyone else holds it too; *copied says whether, *from / *to which pages.
+  int fork(uint64_t id, uint64_t source, uint64_t tokens);
+  int ensure_writable(uint64_t id, uint64_t token, bool *copied, uint32_t *from, uint32_t *to);
   int publish(uint64_t id, const uint32_t *tokens, uint64_t n_tokens, uint32_t committed);
   struct View {                                             // Cache::pageTable
     const uint32_t *pages;

@@ -110,6 +110,37 @@ uint64_t kvx_prefix_match(const kvx_prefix *prefix, const uint32_t *prompt, uint
   return hashed;
 }
 
+// The identity is a value that travels with a block's key (and would be persisted
+// with it), so its bits are the reference's: two chains with their own seeds fold,
+// for every span that overlaps the block, the span's content digest, its grid, its
+// place in the prompt and the block's start.  `a ^= v + golden + (a << 6) + (a >> 2)`
+// is the fold of both chains; the second takes the complement of every value.
+void kvx_block_image_identity(uint64_t block_begin, uint32_t block_tokens,
+                              const kvx_image_span *spans, uint32_t n_spans, uint64_t *lo,
+                              uint64_t *hi) {
+  const auto fold = [](uint64_t a, uint64_t v) {
+    return a ^ (v + 0x9e3779b97f4a7c15ull + (a << 6) + (a >> 2));
+  };
+  uint64_t chain_lo = 0, chain_hi = 0;
+  const uint64_t block_end = block_begin + block_tokens;
+  for (uint32_t i = 0; i < n_spans; ++i) {
+    const kvx_image_span &span = spans[i];
+    if (span.offset >= block_end) break;  // spans are sorted by offset
+    if (uint32_t(span.offset + span.tokens) <= block_begin) continue;  // 32-bit end, as ImageSpan::end()
+    const uint64_t words[5] = {span.digest_lo, span.digest_hi,
+                               uint64_t(span.grid_height) << 32 | span.grid_width,
+                               uint64_t(span.offset) << 32 | span.tokens, block_begin};
+    if (!chain_lo) chain_lo = 0x243f6a8885a308d3ull;
+    if (!chain_hi) chain_hi = 0x13198a2e03707344ull;
+    for (const uint64_t word : words) {
+      chain_lo = fold(chain_lo, word);
+      chain_hi = fold(chain_hi, ~word);
+    }
+  }
+  *lo = chain_lo;
+  *hi = chain_hi;
+}
+
 int kvx_sequences_create(kvx_pool *pool, kvx_prefix *prefix, kvx_sequences **out) {
   if (!pool || !prefix || !out) return kvx::fail(KVX_EINVAL, "kvx_sequences_create: null argument");
   *out = new kvx_sequences(pool, prefix);
@@ -128,6 +159,38 @@ int kvx_sequence_restore(kvx_sequences *s, uint64_t id, uint64_t last_block) {
 int kvx_sequence_ensure_tokens(kvx_sequences *s, uint64_t id, uint64_t tokens) {
   const int rc = s->sequences.ensure_tokens(id, tokens);
   return rc == KVX_ENOMEM ? rc : report(rc, "unknown sequence, or KV target past the page id range");
+}
+int kvx_sequence_fork(kvx_sequences *s, uint64_t id, uint64_t source, uint64_t tokens) {
+  const int rc = s->sequences.fork(id, source, tokens);
+  switch (rc) {
+  case KVX_ESTATE:
+    return kvx::fail(rc, "fork target already owns KV pages, or is its own source");
+  case KVX_EINVAL:
+    return kvx::fail(rc, "fork point past the pages the source holds");
+  default:
+    return report(rc, "unknown sequence");
+  }
+}
+int kvx_sequence_ensure_writable(kvx_sequences *s, uint64_t id, uint64_t token, uint32_t *copied,
+                                 uint32_t *from_page, uint32_t *to_page, void *stream) {
+  bool did = false;
+  uint32_t from = KVX_NO_PAGE, to = KVX_NO_PAGE;
+  kvx_pool_set_stream(s->pool, stream);
+  const int rc = s->sequences.ensure_writable(id, token, &did, &from, &to);
+  kvx_pool_set_stream(s->pool, nullptr);
+  if (copied) *copied = did ? 1u : 0u;
+  if (from_page) *from_page = from;
+  if (to_page) *to_page = to;
+  switch (rc) {
+  case KVX_ESTATE:
+    return kvx::fail(rc, "the page is published: rows before the token's page boundary are final");
+  case KVX_EINVAL:
+    return kvx::fail(rc, "the sequence holds no page for this token");
+  case KVX_ENOMEM:
+    return rc;
+  default:
+    return report(rc, "unknown sequence");
+  }
 }
 int kvx_sequence_publish(kvx_sequences *s, uint64_t id, const uint32_t *tokens, uint64_t n_tokens,
                          uint32_t committed_tokens) {

@@ -44,6 +44,7 @@ SYMBOLS = [
     "kvx_sequences_destroy", "kvx_sequence_begin", "kvx_sequence_end", "kvx_sequence_restore",
     "kvx_sequence_ensure_tokens", "kvx_sequence_publish", "kvx_sequence_view",
     "kvx_sequences_compact_extent", "kvx_tree_masks", "kvx_tree_path_valid",
+    "kvx_sequence_fork", "kvx_sequence_ensure_writable", "kvx_block_image_identity",
 ]
 
 
@@ -97,6 +98,19 @@ class PoolSnapshot(C.Structure):
                 ("extent_allocations", C.c_uint64), ("extent_releases", C.c_uint64),
                 ("extent_allocate_max_ms", C.c_double), ("extent_release_max_ms", C.c_double),
                 ("extent_compactions", C.c_uint64), ("pages_moved", C.c_uint64)]
+
+
+def _depends_on(child, parent):
+    """The library objects behind `child` use those behind `parent` until they are destroyed,
+    their destructors included, and the garbage collector may finalize a group of objects in
+    any order: a parent closes the children that registered here before it closes itself.
+    (Strong references: the collector clears weak ones before it runs any finalizer.)"""
+    parent.__dict__.setdefault("_dependents", []).append(child)
+
+
+def _close_dependents(parent):
+    for child in reversed(parent.__dict__.pop("_dependents", [])):
+        child.close()
 
 
 class KvxError(RuntimeError):
@@ -172,6 +186,10 @@ def _declare(L):
     L.kvx_sequence_publish.argtypes = [vp, u64, vp, u64, u32]
     L.kvx_sequence_view.argtypes = [vp, u64, C.POINTER(SequencePages)]
     L.kvx_sequences_compact_extent.argtypes = [vp, PU32, vp, PU32, vp]
+    L.kvx_sequence_fork.argtypes = [vp, u64, u64, u64]
+    L.kvx_sequence_ensure_writable.argtypes = [vp, u64, u64, PU32, PU32, PU32, vp]
+    L.kvx_block_image_identity.argtypes = [u64, u32, vp, u32, PU64, PU64]
+    L.kvx_block_image_identity.restype = None
     L.kvx_debug_attend_paths.argtypes, L.kvx_debug_attend_paths.restype = [PU64, PU64], None
     L.kvx_decode_plan.argtypes = [vp, u32, u32, u32, vp]
     L.kvx_verify_plan.argtypes = [vp, u32, u32, u32, u32, u32, vp]
@@ -266,6 +284,7 @@ class Storage:
         self.bytes_per_page = lib().kvx_storage_bytes_per_page(h)
 
     def close(self):
+        _close_dependents(self)
         if getattr(self, "h", None):
             lib().kvx_storage_destroy(self.h)
             self.h = None
@@ -458,8 +477,10 @@ class Pool:
         h = C.c_void_p()
         check(lib().kvx_pool_create(storage.h, runway_pages, C.byref(h)))
         self.h, self.storage = h, storage
+        _depends_on(self, storage)
 
     def close(self):
+        _close_dependents(self)
         if getattr(self, "h", None):
             lib().kvx_pool_destroy(self.h)
             self.h = None
@@ -515,8 +536,10 @@ class Prefix:
         h = C.c_void_p()
         check(lib().kvx_prefix_create(pool.h, C.byref(h)))
         self.h, self.pool = h, pool
+        _depends_on(self, pool)
 
     def close(self):
+        _close_dependents(self)
         if getattr(self, "h", None):
             lib().kvx_prefix_destroy(self.h)
             self.h = None
@@ -591,6 +614,7 @@ class Sequences:
         h = C.c_void_p()
         check(lib().kvx_sequences_create(pool.h, prefix.h, C.byref(h)))
         self.h, self.pool, self.prefix = h, pool, prefix
+        _depends_on(self, prefix)
 
     def close(self):
         if getattr(self, "h", None):
@@ -616,6 +640,20 @@ class Sequences:
         return check(lib().kvx_sequence_publish(self.h, sequence, _u32(tokens), len(tokens),
                                                 committed))
 
+    def fork(self, sequence, source, tokens):
+        """`sequence` (empty) shares the pages of the first `tokens` tokens of `source`."""
+        return check(lib().kvx_sequence_fork(self.h, sequence, source, tokens))
+
+    def ensure_writable(self, sequence, token, stream=None):
+        """Copy-on-write of the page that holds `token`: None when the page is written in
+        place, else (shared page, the sequence's new copy)."""
+        if stream is None and self.pool.storage.accounting:
+            stream = 0
+        copied, source, copy = C.c_uint32(), C.c_uint32(), C.c_uint32()
+        check(lib().kvx_sequence_ensure_writable(self.h, sequence, token, C.byref(copied),
+                                                 C.byref(source), C.byref(copy), _stream(stream)))
+        return (source.value, copy.value) if copied.value else None
+
     def view(self, sequence):
         out = SequencePages()
         check(lib().kvx_sequence_view(self.h, sequence, C.byref(out)))
@@ -633,6 +671,20 @@ class Sequences:
         if not moved.value:
             return None
         return {"first": first.value, "dest": list(dest), "moved": moved.value}
+
+
+class ImageSpan(C.Structure):
+    _fields_ = [("offset", C.c_uint32), ("tokens", C.c_uint32), ("grid_height", C.c_uint32),
+                ("grid_width", C.c_uint32), ("digest_lo", C.c_uint64), ("digest_hi", C.c_uint64)]
+
+
+def block_image_identity(block_begin, block_tokens, spans):
+    """(lo, hi) of the images overlapping a block; spans = (offset, tokens, grid height, grid
+    width, digest lo, digest hi) tuples sorted by offset (kvx_block_image_identity)."""
+    arr = (ImageSpan * max(len(spans), 1))(*[ImageSpan(*s) for s in spans])
+    lo, hi = C.c_uint64(), C.c_uint64()
+    lib().kvx_block_image_identity(block_begin, block_tokens, arr, len(spans), C.byref(lo), C.byref(hi))
+    return lo.value, hi.value
 
 
 def decode_plan(committed, kv_heads, fmt=INT4):

@@ -230,3 +230,89 @@ def test_compaction_leaves_fixed_pages_in_place():
     moves = pool.compact([9])
     assert moves["first"] == 12 and follow(moves, 12) == 3 and follow(moves, 13) == 7
     assert follow(moves, 9) == 9 and pool.active(9)
+
+
+def test_random_walk_in_lockstep_with_the_oracle_pool():
+    """Page ids, refusals, reclaimed bytes and compaction moves of the product's pool against
+    the oracle's restatement of the reference pool over a long random walk: acquisitions of
+    random sizes (some refused by a budget that moves), releases in random order, references
+    to pages that are free, prefix references, reclaims with and without a runway and a limit,
+    compactions with and without fixed pages."""
+    import numpy as np
+    from oracle import kvoracle as ko
+    KO = ko.lib()
+    rng = np.random.default_rng(20260)
+    for extent_pages, extents in ((4, 6), (5, 9), (16, 5)):
+        pages = extent_pages * extents
+        runway = int(rng.integers(0, pages + 1))
+        mine = Pool(pages, runway, extent_pages)
+        theirs = KO.ko_pool_create(pages, mine.page_bytes, extent_pages, runway, NO_LIMIT)
+        assert theirs
+        held_active, held_prefix = [], []
+
+        def same_books():
+            a, b = mine.snap(), ko.PoolSnapshot()
+            KO.ko_pool_snapshot_get(theirs, C.byref(b))
+            for field in ("pages_allocated", "pages_free", "pages_active", "pages_prefix",
+                          "allocated_bytes", "reclaimable_bytes", "extent_allocations",
+                          "extent_releases", "extent_compactions", "pages_moved"):
+                assert getattr(a, field) == getattr(b, field), field
+
+        for step in range(3000):
+            op = rng.integers(0, 100)
+            if op < 30:
+                count = int(rng.integers(0, extent_pages * 2 + 1))
+                out = np.zeros(max(count, 1), dtype=np.uint32)
+                rc_theirs = KO.ko_pool_acquire(theirs, count, ko.ptr(out))
+                rc_mine, got = mine.acquire(count)
+                assert rc_mine == rc_theirs, (step, count)
+                if rc_mine == count:
+                    assert got == list(out[:count]), (step, got, list(out[:count]))
+                    held_active += got
+            elif op < 55 and held_active:
+                page = held_active.pop(int(rng.integers(0, len(held_active))))
+                assert KO.ko_pool_release(theirs, page, 0) == 0
+                mine.release([page])
+            elif op < 62 and held_prefix:
+                page = held_prefix.pop(int(rng.integers(0, len(held_prefix))))
+                assert KO.ko_pool_release(theirs, page, 1) == 0
+                mine.release([page], True)
+            elif op < 72:
+                # a reference to any page of the pool: held, free in the middle of a stack,
+                # or without memory (refused by both)
+                page, prefix = int(rng.integers(0, pages)), bool(rng.integers(0, 2))
+                rc_theirs = KO.ko_pool_retain(theirs, page, int(prefix))
+                rc_mine = mine.retain(page, prefix)
+                assert rc_mine == rc_theirs, (step, page, prefix)
+                if rc_mine == 0:
+                    (held_prefix if prefix else held_active).append(page)
+            elif op < 80:
+                keep, limit = bool(rng.integers(0, 2)), int(rng.choice([0, 1, 2, NO_LIMIT]))
+                assert mine.reclaim(keep, limit) == KO.ko_pool_reclaim_empty(theirs, int(keep), limit)
+            elif op < 84:
+                # the budget moves: between nothing and the whole pool
+                budget = int(rng.integers(0, extents + 1))
+                mine.budget(None if budget == extents else budget * extent_pages)
+                KO.ko_pool_set_budget_pages(theirs, NO_LIMIT if budget == extents
+                                            else budget * extent_pages)
+            else:
+                fixed = [int(p) for p in rng.choice(pages, size=int(rng.integers(0, 3)), replace=False)]
+                arr = np.array(fixed, dtype=np.uint32)
+                first, n = C.c_uint32(), C.c_uint32()
+                dest = np.zeros(extent_pages, dtype=np.uint32)
+                copies = (ko.PageCopy * extent_pages)()
+                moved = KO.ko_pool_compact_extent(theirs, ko.ptr(arr) if fixed else None, len(fixed),
+                                                  C.byref(first), ko.ptr(dest), copies, C.byref(n))
+                moves = mine.compact(fixed)
+                assert (moves is not None) == bool(moved), (step, fixed)
+                if moves:
+                    assert moves["first"] == first.value and moves["dest"] == list(dest), step
+                    assert moves["moved"] == n.value
+                    held_active = [follow(moves, p) for p in held_active]
+                    held_prefix = [follow(moves, p) for p in held_prefix]
+            if step % 50 == 0:
+                same_books()
+                for page in range(pages):
+                    assert mine.active(page) == bool(KO.ko_pool_page_active(theirs, page))
+        same_books()
+        KO.ko_pool_destroy(theirs)

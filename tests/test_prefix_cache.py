@@ -400,3 +400,122 @@ def test_tree_masks_and_paths():
     assert not kvx.tree_path_valid(parents, [0, 2])        # not a child of the row before
     assert not kvx.tree_path_valid(parents, [1, 2])        # must start at the anchor
     assert not kvx.tree_path_valid(parents, [0, 1, 1])     # rows strictly increase
+
+
+# ---- image identity ---------------------------------------------------------------
+
+def test_block_image_identity_properties_of_the_reference():
+    """dev/tests/engine/kv_page_cache_test.cpp:44-69, for the product and the oracle."""
+    red, blue = (8, 16, 8, 8, 0x1111, 0x2222), (8, 16, 8, 8, 0x3333, 0x4444)
+    red_later, first = (40, 16, 8, 8, 0x1111, 0x2222), (0, 8, 4, 8, 0x5555, 0x6666)
+    for identity in (kvx.block_image_identity, po.block_image_identity):
+        assert identity(0, 32, []) == (0, 0)                    # text only
+        assert identity(32, 32, [red]) == (0, 0)                # a block after the image
+        r, b = identity(0, 32, [red]), identity(0, 32, [blue])
+        assert r != (0, 0) and r != b                           # the content digest counts
+        assert identity(32, 32, [red_later]) != r               # so does the block's alignment
+        three = [first, blue, red_later]                        # only overlapping spans count
+        assert identity(32, 32, three) == identity(32, 32, [red_later])
+        assert identity(0, 8, three) == identity(0, 8, [first])
+        assert identity(0, 32, three) != identity(0, 32, [first])   # two spans in one block
+    rng = random.Random(11)
+    for _ in range(300):
+        spans, at = [], 0
+        for _ in range(rng.randrange(0, 5)):
+            at += rng.randrange(0, 40)
+            tokens = rng.randrange(1, 70)
+            spans.append((at, tokens, rng.randrange(1, 64), rng.randrange(1, 64),
+                          rng.getrandbits(64), rng.getrandbits(64)))
+            at += tokens
+        begin = 32 * rng.randrange(0, 8)
+        assert kvx.block_image_identity(begin, 32, spans) == po.block_image_identity(begin, 32, spans)
+
+
+# ---- copy-on-write of a shared, partly filled page (no counterpart in the reference) ----
+
+def test_fork_shares_pages_and_a_write_copies_the_partial_one():
+    s = ProductStack(16, extent_pages=4)
+    prompt = [3 * i % 997 for i in range(200)]
+    ok(s.begin(1))
+    ok(s.ensure(1, 80))                              # 2 full pages + 16 tokens of a third
+    ok(s.publish(1, prompt, 80))
+    one = s.view(1)
+    assert len(one["pages"]) == 3 and len(one["blocks"]) == 2
+    ok(s.begin(2))
+    s.sequences.fork(2, 1, 80)
+    two = s.view(2)
+    assert two["pages"] == one["pages"] and two["blocks"] == one["blocks"]
+    assert two["revision"] == 1 and two["first_changed"] == 0
+    counts = s.pool_counts()
+    assert counts[2] == 3                            # three pages, each held twice
+    # the fork's first write: the shared partial page is copied, the whole pages stay shared
+    moved = s.sequences.ensure_writable(2, 80)
+    assert moved is not None and moved[0] == one["pages"][2] and moved[1] not in one["pages"]
+    two = s.view(2)
+    assert two["pages"] == one["pages"][:2] + [moved[1]]
+    assert two["revision"] == 2 and two["first_changed"] == 2
+    assert s.view(1) == one                          # the source is untouched
+    assert s.pool_counts()[2] == 4
+    # now both hold their last page alone: further writes go in place
+    assert s.sequences.ensure_writable(2, 81) is None
+    assert s.sequences.ensure_writable(1, 80) is None
+    assert s.view(1) == one and s.view(2) == two
+    # published pages are final; a token without a page is refused
+    with pytest.raises(kvx.KvxError) as final:
+        s.sequences.ensure_writable(2, 63)
+    assert final.value.code == kvx.ESTATE
+    with pytest.raises(kvx.KvxError) as absent:
+        s.sequences.ensure_writable(2, 96)
+    assert absent.value.code == kvx.EINVAL
+    # the fork goes on: its own pages, published blocks continue the shared chain
+    ok(s.ensure(2, 130))
+    other = prompt[:80] + [5000 + i for i in range(50)]
+    ok(s.publish(2, other, 128))
+    two = s.view(2)
+    assert two["blocks"][:2] == one["blocks"] and len(two["blocks"]) == 4
+    assert two["pages"][2] == moved[1]
+    # the source publishes its own third page: different tokens, a different block
+    ok(s.ensure(1, 96))
+    ok(s.publish(1, prompt, 96))
+    assert s.view(1)["blocks"][2] != two["blocks"][2] and s.view(1)["pages"] == one["pages"]
+    ok(s.end(1))
+    ok(s.end(2))
+    assert s.pool_counts()[2] == 0
+
+
+def test_fork_errors_and_the_source_writing_first():
+    s = ProductStack(8, extent_pages=4, runway=8)
+    ok(s.begin(1))
+    ok(s.ensure(1, 40))
+    ok(s.begin(2))
+    with pytest.raises(kvx.KvxError) as too_far:
+        s.sequences.fork(2, 1, 65)
+    assert too_far.value.code == kvx.EINVAL
+    with pytest.raises(kvx.KvxError):
+        s.sequences.fork(2, 9, 8)                     # unknown source
+    with pytest.raises(kvx.KvxError) as itself:
+        s.sequences.fork(1, 1, 8)
+    assert itself.value.code == kvx.ESTATE
+    s.sequences.fork(2, 1, 40)
+    with pytest.raises(kvx.KvxError) as twice:
+        s.sequences.fork(2, 1, 40)
+    assert twice.value.code == kvx.ESTATE
+    before = s.view(1)
+    # the source writes first: it is the one that moves to a copy, the fork keeps the page
+    moved = s.sequences.ensure_writable(1, 40)
+    assert moved and moved[0] == before["pages"][1]
+    assert s.view(1)["pages"] == [before["pages"][0], moved[1]]
+    assert s.view(2)["pages"] == before["pages"]
+    assert s.sequences.ensure_writable(2, 40) is None      # sole holder now
+    # no page to be had: nothing changes
+    ok(s.begin(3))
+    s.sequences.fork(3, 2, 40)
+    ok(s.begin(4))
+    ok(s.ensure(4, 32 * 5))                          # takes the five free pages
+    held = s.view(3)
+    with pytest.raises(kvx.KvxError) as full:
+        s.sequences.ensure_writable(3, 40)
+    assert full.value.code == kvx.ENOMEM and s.view(3) == held
+    for q in (1, 2, 3, 4):
+        ok(s.end(q))
+    assert s.pool_counts()[2] == 0 and s.pool_counts()[1] == 8
