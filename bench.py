@@ -259,20 +259,19 @@ def tree_verify(args):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
 
-    def time_attend(phases):
-        L.kvx_debug_set_attend_phases(phases)
-        kvx.attend_verify(storage, 0, QH, queries, output, tables, vp, masks_d, 32, workspace)
+    def time_split():
+        # the split dispatch alone (kv_attend_split), events on the launch stream
+        kvx.attend_split(storage, 0, QH, queries, tables, vp, masks_d, 32, workspace)
         torch.cuda.synchronize()
         k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         k0.record()
         for it in range(args.kernel_iters):
-            kvx.attend_verify(storage, it % LAYERS, QH, queries, output, tables, vp, masks_d, 32, workspace)
+            kvx.attend_split(storage, it % LAYERS, QH, queries, tables, vp, masks_d, 32, workspace)
         k1.record()
         torch.cuda.synchronize()
-        L.kvx_debug_set_attend_phases(3)
         return k0.elapsed_time(k1) / args.kernel_iters
 
-    kernel_ms = time_attend(1)
+    kernel_ms = time_split()
     visible = lanes * (context + nodes)
     flops = 4 * D * (nodes * QH) * visible  # q.k and p.v, multiply and add, every row over every token
     kv_bytes = visible * BYTES_PER_TOKEN_LAYER
@@ -786,23 +785,31 @@ def main():
     vp_arr = (kvx.VerifyParams * BATCH)(*vp)
     launch_bytes = sum(c + 1 for c in committed) * BYTES_PER_TOKEN_LAYER
 
-    def time_attend(phases):
-        L.kvx_debug_set_attend_phases(phases)
+    def time_attend(which):
+        # "both": the attend call as a step issues it; "split" / "merge": the two dispatches
+        # as calls of their own (kv_attend_split, kv_attend_merge) over the same lanes
+        def call(layer):
+            if which == "both":
+                return attend(layer, vp_arr)
+            if which == "split":
+                return L.kv_attend_split(storage.h, layer, QH, queries.data_ptr(), table_arr, vp_arr,
+                                         BATCH, None, 1, workspace.data_ptr(), ws_bytes, stream)
+            return L.kv_attend_merge(storage.h, QH, output.data_ptr(), vp_arr, BATCH, 1,
+                                     workspace.data_ptr(), ws_bytes, stream)
         for layer in range(2):
-            attend(layer, vp_arr)
+            kvx.check(call(layer))
         torch.cuda.synchronize()
         k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         k0.record()
         for it in range(args.kernel_iters):
-            attend(it % LAYERS, vp_arr)
+            call(it % LAYERS)
         k1.record()
         torch.cuda.synchronize()
-        L.kvx_debug_set_attend_phases(3)
         return k0.elapsed_time(k1) / args.kernel_iters
 
-    both_ms = time_attend(3)
-    merge_ms = time_attend(2)
-    kernel_ms = time_attend(1)
+    both_ms = time_attend("both")
+    kernel_ms = time_attend("split")
+    merge_ms = time_attend("merge")
     achieved = launch_bytes / (kernel_ms * 1e-3) / 1e9
     traffic = profiled_traffic()
 

@@ -207,7 +207,7 @@ int kvx_verify_workspace(uint32_t lanes, uint32_t row_capacity, uint32_t query_h
                          const kvx_layout *layout, uint64_t *partials_bytes,
                          uint64_t *statistics_bytes);
 /* Total bytes of one workspace buffer for an attend call over these lanes
-   (sum over lanes of slot_splits * kv_heads * row_capacity * group fused rows). */
+   (sum over lanes of split_count * kv_heads * row_capacity * group fused rows). */
 uint64_t kvx_attend_workspace_bytes(const kvx_verify_params *lanes, uint32_t n_lanes,
                                     uint32_t query_heads, const kvx_layout *layout);
 
@@ -489,8 +489,10 @@ int kv_prepare_append(const kvx_storage *storage, uint32_t layer, const kvx_qkv_
    (dev/tuning/AttentionFixture.hpp:167-173; row_stride = 32 in the reference).
    row_masks: NULL, or u32 [lane][row_capacity] ancestor bitmasks
    (shared/embedding.metal:248-281).  Each lane's split_count partitions its
-   pages as ceil(pages / split_count) per split; slot_splits is ignored (slots
-   are packed per lane).  Output rows >= active_rows up to row_capacity are
+   pages as ceil(pages / split_count) per split.  The reference strides a lane's
+   slots by slot_splits (common/paged_attention_tile.h:57-58); here slots are packed
+   by split_count, and slot_splits is only checked: 0, or split_count <= slot_splits
+   <= the maximum, else KVX_EINVAL.  Output rows >= active_rows up to row_capacity are
    written as zeros.  workspace: device memory of at least
    kvx_attend_workspace_bytes(). */
 int kv_attend_verify(const kvx_storage *storage, uint32_t layer, uint32_t query_heads,
@@ -498,6 +500,27 @@ int kv_attend_verify(const kvx_storage *storage, uint32_t layer, uint32_t query_
                      const kvx_verify_params *lanes, uint32_t n_lanes,
                      const uint32_t *row_masks, uint32_t row_stride, void *workspace,
                      uint64_t workspace_bytes, void *stream);
+
+/* The two dispatches of kv_attend_verify as calls of their own, as the reference encodes them
+   (ops::PagedAttention::addVerify: the *_split dispatch, runtime/ops/PagedAttention.cpp:506-513,
+   then the *_reduce dispatch, :517-544).
+   kv_attend_split: every split of every lane writes its fp32 partial rows and (max, sum) to the
+   workspace and nothing is merged, also for a lane with one split.  The workspace holds the
+   partial rows first, [fused row slot][D] floats, then, at the next 256-byte boundary, the
+   statistics, [fused row slot][2]; lane i's slots start after those of lanes 0 .. i-1 (split_count x
+   KV heads x row_capacity x group each) and are ordered [KV head][split][fused row], fused row =
+   query row x group + head in group.
+   kv_attend_merge: the fixed-order merge over a workspace filled that way, by kv_attend_split or
+   by the caller (the reference pins its reduce kernels with synthetic partial rows,
+   dev/tests/engine/q8_flash_attention_metal_test.mm:648-725); `lanes` as for the split (their
+   committed_tokens, active_rows and split_count say which slots were written). */
+int kv_attend_split(const kvx_storage *storage, uint32_t layer, uint32_t query_heads,
+                    const void *queries, const uint64_t *const *page_tables,
+                    const kvx_verify_params *lanes, uint32_t n_lanes, const uint32_t *row_masks,
+                    uint32_t row_stride, void *workspace, uint64_t workspace_bytes, void *stream);
+int kv_attend_merge(const kvx_storage *storage, uint32_t query_heads, void *output,
+                    const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                    void *workspace, uint64_t workspace_bytes, void *stream);
 
 /* kv_attend_verify whose merge also hands the out-projection its operand, so that no
    elementwise gate or gather dispatch has to read the attention rows back.  Replaces
@@ -590,11 +613,6 @@ int kv_compact_path(const kvx_storage *storage, uint32_t layer,
                     uint32_t n_lanes, const uint32_t *retained_path,
                     const uint32_t *retained_count, uint32_t path_stride, void *stream);
 
-/* Profiling aid with no counterpart in the reference: selects which phases the
-   attend entries launch (bit 0 = split kernel, bit 1 = merge kernel; default 3)
-   so a harness can time one kernel alone with events on its stream.  Outputs
-   are only meaningful with both bits set. */
-void kvx_debug_set_attend_phases(uint32_t phases);
 /* Also no counterpart in the reference: how many attend calls of this process went to the
    format-generic kernels and how many to the matrix-core (MFMA) kernels, so tests can tell
    which path they measured. */

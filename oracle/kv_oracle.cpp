@@ -586,6 +586,88 @@ int ko_store_verify(uint32_t format, uint32_t kv_heads, uint32_t head_dim,
 }
 
 // ------------------------------------------------------------- attention ---
+namespace {
+// A test's question to the oracle: "had the rounding of this one probability
+// fallen the other way, what would the row be?"  While set, the tile moves the
+// rounded weight of (fused row, token) by `steps` places of its format (bf16, or
+// fp16 on the fp8 path) and, with only_row, computes that fused row alone.
+struct Nudge {
+  int64_t fused_row = -1;
+  uint32_t token = 0;
+  int steps = 0;
+  bool only_row = false;
+};
+thread_local Nudge g_nudge;
+
+float step_bf16(float w, int steps) {
+  // weights are finite and not negative: neighbours in the format are neighbours as integers
+  const int bits = int(ko_float_to_bf16(w)) + steps;
+  return ko_bf16_to_float(uint16_t(bits < 0 ? 0 : bits));
+}
+float step_f16(float w, int steps) {
+  // w is a non-negative binary16 value: its neighbours lie one step of its binade away
+  // (2^-24 below 2^-14), and going down from a power of two the step halves.
+  for (int i = 0; i < (steps < 0 ? -steps : steps); ++i) {
+    const int e = w < 6.103515625e-05f ? -14 : std::ilogb(w);
+    float step = std::ldexp(1.0f, e - 10);
+    if (steps < 0) {
+      if (w == 0.0f) break;
+      if (e > -14 && w == std::ldexp(1.0f, e)) step *= 0.5f;
+      w -= step;
+    } else {
+      w += step;
+    }
+  }
+  return w;
+}
+}  // namespace
+
+void ko_attention_nudge(int64_t fused_row, uint32_t token, int steps, int only_row) {
+  g_nudge.fused_row = fused_row;
+  g_nudge.token = token;
+  g_nudge.steps = steps;
+  g_nudge.only_row = only_row != 0;
+}
+
+void ko_attention_row_weights(uint32_t format, uint32_t kv_heads, uint32_t head_dim,
+                              const uint16_t *query_row, const uint64_t *page_table, ko_kv_layer kv,
+                              uint32_t kv_head, uint32_t committed, uint32_t active_rows,
+                              uint32_t row, const uint32_t *row_masks, float score_scale_param,
+                              float *weights) {
+  // softmax weight x value scale of every token the row sees, against the row's
+  // maximum over all pages; tokens it does not see get 0.
+  const uint32_t D = head_dim, visible = committed + active_rows;
+  const bool fp8 = format == KO_FP8E4M3, quant = quantized(format);
+  const float score_scale = default_score_scale(D, score_scale_param);
+  const uint32_t limit = std::min(visible, committed + std::min(row, active_rows - 1) + 1);
+  const uint32_t mask = row_masks ? row_masks[row] : 0u;
+  std::vector<float> q(D), score(visible, -kInf);
+  for (uint32_t d = 0; d < D; ++d) {
+    const float v = ko_bf16_to_float(query_row[d]);
+    q[d] = fp8 ? ko_round_to_f16(v) : v;
+  }
+  float maximum = -kInf;
+  for (uint32_t t = 0; t < visible; ++t) {
+    const bool admitted = !row_masks ? t < limit
+                                     : (t < committed) || ((mask >> (t - committed)) & 1u);
+    if (!admitted) continue;
+    const Slab s = slab_of(format, kv_heads, D, kv, kv_head, page_table[t / kPage]);
+    float dot = 0.0f;
+    for (uint32_t d = 0; d < D; ++d) dot += q[d] * key_code(format, s, D, t % kPage, d);
+    if (quant) dot *= s.key_scales[t % kPage];
+    score[t] = dot * score_scale;
+    maximum = std::max(maximum, score[t]);
+  }
+  for (uint32_t t = 0; t < visible; ++t) {
+    if (score[t] == -kInf) {
+      weights[t] = 0.0f;
+      continue;
+    }
+    const Slab s = slab_of(format, kv_heads, D, kv, kv_head, page_table[t / kPage]);
+    weights[t] = std::exp(score[t] - maximum) * (quant ? s.value_scales[t % kPage] : 1.0f);
+  }
+}
+
 int ko_attention_tile(uint32_t format, uint32_t kv_heads, uint32_t group, uint32_t head_dim,
                       uint32_t row_capacity, const uint16_t *tile_queries,
                       const uint64_t *page_table, ko_kv_layer kv, uint32_t kv_head,
@@ -611,6 +693,7 @@ int ko_attention_tile(uint32_t format, uint32_t kv_heads, uint32_t group, uint32
     // Rows past the live ones are never read by the merge (it writes zeros
     // for them), so the oracle leaves their partials untouched.
     if (query_row >= active_rows) continue;
+    if (g_nudge.only_row && g_nudge.fused_row >= 0 && int64_t(r) != g_nudge.fused_row) continue;
     for (uint32_t d = 0; d < D; ++d) {
       const float v = ko_bf16_to_float(tile_queries[uint64_t{r} * D + d]);
       q[d] = fp8 ? ko_round_to_f16(v) : v;  // fp8 tile stages queries as fp16
@@ -662,6 +745,8 @@ int ko_attention_tile(uint32_t format, uint32_t kv_heads, uint32_t group, uint32
         float w = 0.0f;
         if (admitted[j] && score[j] > -kInf) w = prob[j] * (quant ? s.value_scales[j] : 1.0f);
         weight[j] = fp8 ? ko_round_to_f16(w) : ko_bf16_to_float(ko_float_to_bf16(w));
+        if (g_nudge.fused_row == int64_t(r) && g_nudge.token == token_start + j && g_nudge.steps)
+          weight[j] = fp8 ? step_f16(weight[j], g_nudge.steps) : step_bf16(weight[j], g_nudge.steps);
       }
       for (uint32_t d = 0; d < D; ++d) {
         float sum = 0.0f;

@@ -202,6 +202,11 @@ def _declare(L):
                                     u32, vp, vp, u64, vp, f32]
     L.ko_attention_reduce_row.argtypes = [u32, u32, u32, vp, vp, u32, u32, u32, u64, u32, vp, vp]
     L.ko_attention_reduce_row.restype = None
+    L.ko_attention_nudge.argtypes = [C.c_int64, u32, C.c_int, C.c_int]
+    L.ko_attention_nudge.restype = None
+    L.ko_attention_row_weights.argtypes = [u32, u32, u32, vp, vp, KvLayer, u32, u32, u32, u32, vp,
+                                           C.c_float, vp]
+    L.ko_attention_row_weights.restype = None
     L.ko_attend_prefill.argtypes = [u32, u32, u32, u32, vp, vp, vp, vp, C.POINTER(PrefillParams)]
     L.ko_attend_verify.argtypes = [u32, u32, u32, u32, vp, vp, vp, vp, vp, u32, vp]
     L.ko_compact_tree.argtypes = [u32, u32, u32, vp, vp, vp, vp, u32, u32]
@@ -380,3 +385,64 @@ def compact_tree(fmt, kv_heads, head_dim, tables, params, retained_path, retaine
     arr = (ChunkParams * len(params))(*params)
     return lib().ko_compact_tree(fmt, kv_heads, head_dim, _table_ptrs(tables), arr,
                                  ptr(retained_path), ptr(retained_count), len(params), path_stride)
+
+
+# ------------------------------------------------ one tile, and "what if" rows ---
+def attention_tile_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv, head, committed,
+                        active, splits, capacity, masks=None, score_scale=0.0, only_row=None):
+    """The oracle's attention of one tile (capacity rows x group fused rows) of one KV head: every
+    split's partial tile, then the fixed-order merge of each live fused row.  tile_queries: bf16
+    [capacity * group, D].  Returns (bf16, fp32) outputs of that shape; rows past `active` are
+    zeros.  only_row: merge that fused row alone (the others stay zero)."""
+    L = lib()
+    M, D = capacity * group, head_dim
+    tile_queries = np.ascontiguousarray(tile_queries, dtype=np.uint16).reshape(M, D)
+    partials = np.zeros((splits, M, D), dtype=np.float32)
+    statistics = np.zeros((splits, M, 2), dtype=np.float32)
+    mask_ptr = ptr(np.ascontiguousarray(masks, dtype=np.uint32)) if masks is not None else None
+    for split in range(splits):
+        L.ko_attention_tile(fmt, kv_heads, group, D, capacity, ptr(tile_queries), ptr(table), kv,
+                            head, committed, active, splits, split, ptr(partials),
+                            ptr(statistics), split, mask_ptr, score_scale)
+    out = np.zeros((M, D), dtype=np.uint16)
+    out32 = np.zeros((M, D), dtype=np.float32)
+    for row in (range(M) if only_row is None else [only_row]):
+        L.ko_attention_reduce_row(group, D, capacity, ptr(partials), ptr(statistics), committed,
+                                  active, splits, 0, row, ptr(out[row]), ptr(out32[row]))
+    return out, out32
+
+
+def rounding_flip_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv, head, committed,
+                       active, splits, capacity, fused_row, masks=None, score_scale=0.0, top=4):
+    """What one fused row of a tile would be had the rounding of one probability fallen the other
+    way: for each of the row's `top` heaviest tokens (softmax weight x value scale) and each
+    direction, the row recomputed with that token's rounded weight moved one place of its format
+    (bf16; fp16 on fp8 pages).  Yields (token, steps, bf16 row bits).
+
+    A kernel that sums q.k in another order than this oracle can differ from it in the last bits
+    of a score, and so in the rounding of a probability that sits on a rounding boundary; when
+    that token carries most of the row, the whole row moves by up to half a place.  A row that is
+    farther from the oracle than the tolerance, but within it of one of these rows, is explained by
+    exactly that; any other difference is not."""
+    L = lib()
+    M, D = capacity * group, head_dim
+    tile_queries = np.ascontiguousarray(tile_queries, dtype=np.uint16).reshape(M, D)
+    row = fused_row // group
+    visible = committed + active
+    weights = np.zeros(visible, dtype=np.float32)
+    mask_ptr = ptr(np.ascontiguousarray(masks, dtype=np.uint32)) if masks is not None else None
+    L.ko_attention_row_weights(fmt, kv_heads, D, ptr(tile_queries[fused_row]), ptr(table), kv, head,
+                               committed, active, row, mask_ptr, score_scale, ptr(weights))
+    heaviest = np.argsort(-weights, kind="stable")[:top]
+    try:
+        for token in heaviest:
+            if weights[token] <= 0:
+                continue
+            for steps in (1, -1):
+                L.ko_attention_nudge(fused_row, int(token), steps, 1)
+                bits, _ = attention_tile_rows(fmt, kv_heads, group, D, tile_queries, table, kv, head,
+                                              committed, active, splits, capacity, masks, score_scale,
+                                              only_row=fused_row)
+                yield int(token), steps, bits[fused_row]
+    finally:
+        L.ko_attention_nudge(-1, 0, 0, 0)

@@ -338,9 +338,10 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
                             const uint64_t *const *page_tables, const kvx_verify_params *lanes,
                             uint32_t n_lanes, const uint32_t *row_masks, uint32_t row_stride,
                             uint64_t lane_stride, void *workspace, uint64_t workspace_bytes,
-                            uint32_t phases, hipStream_t stream,
-                            const FusedAppend *fused = nullptr, uint32_t tile_rows = 0,
-                            const Epilogue *epilogue = nullptr) {
+                            hipStream_t stream, const FusedAppend *fused = nullptr,
+                            uint32_t tile_rows = 0, const Epilogue *epilogue = nullptr) {
+  const bool run_split = !(epilogue && epilogue->merge_only);
+  const bool run_merge = !(epilogue && epilogue->partials_only);
   const kvx_layout &l = s->layout;
   const uint32_t H = l.kv_heads, G = query_heads / H;
   const uint32_t capacity = lanes[0].row_capacity, M = capacity * G;
@@ -380,7 +381,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
     for (uint32_t i = 0; i < (tile_rows ? 1u : a.n_lanes); ++i) {
       const kvx_verify_params &p = lanes[first + i];
       DecodeLane &dl = a.lane[i];
-      dl.table = page_tables[first + i];
+      dl.table = page_tables ? page_tables[first + i] : nullptr;
       dl.masks = row_masks ? row_masks + uint64_t(first + i) * capacity : nullptr;
       dl.committed = p.committed_tokens;
       dl.active_rows = p.active_rows;
@@ -395,7 +396,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       row_base += uint64_t(p.split_count) * H * M;
     }
     if (tile_rows) items = n_lanes * lanes[0].split_count;
-    if (epilogue && epilogue->partials_only) {
+    if (epilogue && !epilogue->hidden) {
       a.all_partials = 1;
     } else if (epilogue) {
       a.hidden = epilogue->hidden + uint64_t(first) * capacity * query_heads * kD;
@@ -405,14 +406,14 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
                          : nullptr;
       a.all_partials = 1;
     }
-    if (phases & 1u) {
+    if (run_split) {
       hipLaunchKernelGGL(split_kernel, dim3(items, H, (M + columns - 1) / columns), dim3(threads), 0,
                          stream, static_cast<const uint16_t *>(queries),
                          static_cast<uint16_t *>(output), partials, statistics, a);
       const hipError_t e = hipGetLastError();
       if (e != hipSuccess) return hip_fail(e, name);
     }
-    if ((max_splits > 1 || epilogue) && (phases & 2u) && !(epilogue && epilogue->partials_only)) {
+    if ((max_splits > 1 || epilogue) && run_merge) {
       // One wave per row is all the sequential merge uses; the other three only
       // join in for lists longer than kMergeSequential.
       const uint32_t merge_threads = max_splits <= kMergeSequential ? 64 : 64 * kMergeWaves;

@@ -478,8 +478,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
 
 using namespace kvx;
 
-uint32_t kvx_attend_phases();  // bit 0 = split kernel, bit 1 = merge kernel
-
 // Runs paged attention for bf16 or fp8 pages of head dimension 256 on the
 // matrix cores; returns 1 (declined) for shapes it does not cover, 0 when
 // enqueued, or a negative status.  Arguments as kvx_attend_int4_launch.
@@ -494,11 +492,10 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
       !matrix_attention_covers(s, query_heads, lanes, n_lanes))
     return 1;
   const uint32_t M = lanes[0].row_capacity * (query_heads / s->layout.kv_heads);
-  const uint32_t phases = kvx_attend_phases();
 #define KVX_WIDE(FMT, NB, WAVES, REUSED)                                                         \
   launch_matrix_attention(attend_wide_kernel<FMT, NB, WAVES, REUSED>, "attend_wide_kernel", 16 * NB, 64, s, \
                           kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks, \
-                          row_stride, lane_stride, workspace, workspace_bytes, phases, stream,      \
+                          row_stride, lane_stride, workspace, workspace_bytes, stream,              \
                           nullptr, tile_rows, epilogue)
   // Two blocks of 16 fused rows per wave share every key and value operand; a
   // third would not fit the register file next to a page of bf16 keys and values.

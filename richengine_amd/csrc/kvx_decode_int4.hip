@@ -138,10 +138,6 @@ __device__ __forceinline__ u32x4 expand_key_dword(uint32_t x) {
   return out;
 }
 
-#ifdef KVX_PROBE_CLOCK
-__device__ uint64_t kvx_probe_log[16384][4];
-#endif
-
 // Softmax state and accumulators of one block of 16 fused query rows.
 struct State {
   f32x4 acc[16];  // [nibble position m]: dims 16*(4g + r) + m of column t
@@ -163,15 +159,6 @@ __device__ __forceinline__ void attend_page(PageRegs &r, Queries queries,
                                             uint32_t first_token, const Sight *sight,
                                             uint32_t lane, uint32_t g, State *st,
                                             KeysConsumed keys_consumed) {
-#ifdef KVX_PROBE_STREAM_ONLY
-  // Measurement build: consume every loaded register with almost no arithmetic,
-  // to see what the memory system delivers for this access pattern.
-  uint32_t x = 0;
-  for (uint32_t i = 0; i < 4; ++i) x ^= r.k[i][0] ^ r.k[i][1] ^ r.k[i][2] ^ r.k[i][3];
-  for (uint32_t i = 0; i < 8; ++i) x ^= r.v[i][0] ^ r.v[i][1];
-  st[0].row_sum += r.scale + __uint_as_float(x & 0xffu);
-  return;
-#endif
   // ---- q.k ----
   f32x4 s[NB][2];
 #pragma unroll
@@ -347,13 +334,10 @@ __device__ __forceinline__ void append_decode_token(const DecodeArgs &a, const D
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-#ifndef KVX_V48_DEPTH
-#define KVX_V48_DEPTH 1
-#endif
-#ifndef KVX_DECODE_DEPTH
-#define KVX_DECODE_DEPTH 2
-#endif
-constexpr uint32_t kDecodeDepth = KVX_DECODE_DEPTH;
+// Register sets of pages per wave: two rotate in the one-block decode kernel
+// (two waves per SIMD), one in the three-block verify kernel.
+constexpr uint32_t kDecodeDepth = 2;
+constexpr uint32_t kVerify48Depth = 1;
 
 // Writes what a wave has accumulated for its NB blocks: the finished bf16 rows
 // when the lane has a single split, else fp32 partial rows and (max, sum).
@@ -427,9 +411,6 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
                                             float *__restrict__ partials,
                                             float *__restrict__ statistics, const DecodeArgs &a) {
   const uint32_t item = blockIdx.x, head = blockIdx.y;
-#ifdef KVX_PROBE_CLOCK
-  const uint64_t probe_cycles = __builtin_readcyclecounter(), probe_wall = wall_clock64();
-#endif
   uint32_t li;
   const DecodeLane l = lane_of_item(a, item, li);
   const uint32_t split = item - l.first_item;
@@ -499,11 +480,6 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   PageRegs r[kDepth];
   const LaneOffsets at = lane_offsets(t, g, uint32_t(ro.value_scales - ro.key_scales));
   auto fill = [&](PageRegs &set, uint32_t slot) {
-#ifdef KVX_PROBE_SAME_PAGE
-    // Measurement build: every refill is the split's first page, so loads hit the
-    // caches and the time left is the kernel's own arithmetic.
-    slot = 0;
-#endif
     // The empty asm statements pin the loads of one fill together and in place:
     // moved up into the arithmetic that still reads the set they would need a
     // second copy of its registers, and interleaved with another fill's loads
@@ -515,17 +491,11 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   // The same in two steps for the steady loop: the keys as soon as the page that
   // held the set has multiplied its last key, the rest when the page is done.
   auto fill_keys = [&](PageRegs &set, uint32_t slot) {
-#ifdef KVX_PROBE_SAME_PAGE
-    slot = 0;
-#endif
     asm volatile("");
     load_page<1, kReused>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
   auto fill_rest = [&](PageRegs &set, uint32_t slot) {
-#ifdef KVX_PROBE_SAME_PAGE
-    slot = 0;
-#endif
     asm volatile("");
     load_page<2, kReused>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
@@ -608,19 +578,6 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     }
   }
 
-#ifdef KVX_PROBE_CLOCK
-  // Measurement build: when and where every wave ran.
-  if (threadIdx.x == 0) {
-    const uint32_t slot = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
-    if (slot < 16384) {
-      kvx_probe_log[slot][0] = probe_wall;
-      kvx_probe_log[slot][1] = wall_clock64();
-      kvx_probe_log[slot][2] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11)) |
-                               (uint64_t(__builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11))) << 32);
-      kvx_probe_log[slot][3] = end - begin;
-    }
-  }
-#endif
   write_blocks<NB>(st, m, in_tile, live_row, l, a, head, split, a.all_partials ? 2u : written, g, output,
                    partials, statistics);
 }
@@ -669,15 +626,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void verify48_int4_kernel(
     const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
     float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
-  attend_int4<3, KVX_V48_DEPTH>(queries, output, partials, statistics, a);
+  attend_int4<3, kVerify48Depth>(queries, output, partials, statistics, a);
 }
 
 }  // namespace
 }  // namespace kvx
 
 using namespace kvx;
-
-uint32_t kvx_attend_phases();  // bit 0 = split kernel, bit 1 = merge kernel
 
 // Runs paged attention (split kernel, then the merge of multi-split lanes) for
 // int4 pages of head dimension 256; returns 1 (declined) for shapes it does not
@@ -711,34 +666,26 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
     return launch_matrix_attention(prefill_int4_kernel, "prefill_int4_kernel", 32, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                   kvx_attend_phases(), stream, nullptr, tile_rows, epilogue);
-#ifndef KVX_NO_V48
+                                   stream, nullptr, tile_rows, epilogue);
   // 48 fused rows per wave where that leaves clearly fewer waves: the pages are
   // read and expanded once per 48 rows instead of once per 32.
   if (verify_block_rows(KVX_FMT_INT4, fused_rows) == 48 && !many_tiles)
     return launch_matrix_attention(verify48_int4_kernel, "verify48_int4_kernel", 48, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                   kvx_attend_phases(), stream, nullptr, tile_rows, epilogue);
-#endif
+                                   stream, nullptr, tile_rows, epilogue);
   if (fused_rows > 16 && !many_tiles)
     return launch_matrix_attention(verify_int4_kernel, "verify_int4_kernel", 32, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                   kvx_attend_phases(), stream, nullptr, tile_rows, epilogue);
+                                   stream, nullptr, tile_rows, epilogue);
   if (tile_rows && !fused)
     return launch_matrix_attention(decode_int4_tiles_kernel, "decode_int4_tiles_kernel", 16, 64, s,
                                    kv, query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                   kvx_attend_phases(), stream, nullptr, tile_rows, epilogue);
+                                   stream, nullptr, tile_rows, epilogue);
   return launch_matrix_attention(decode_int4_kernel, "decode_int4_kernel", 16, 64, s, kv,
                                  query_heads, queries, output, page_tables, lanes, n_lanes,
                                  row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                 kvx_attend_phases(), stream, fused, tile_rows, epilogue);
+                                 stream, fused, tile_rows, epilogue);
 }
-
-#ifdef KVX_PROBE_CLOCK
-extern "C" int kvx_probe_fetch(uint64_t *host, uint32_t slots) {
-  return hipMemcpyFromSymbol(host, HIP_SYMBOL(kvx::kvx_probe_log), uint64_t(slots) * 32) == hipSuccess ? 0 : -1;
-}
-#endif

@@ -82,12 +82,14 @@ __device__ inline Slab slab_of(uint32_t format, uint32_t kv_heads, uint32_t head
 // first scaled by the sigmoid of its gate (the reduce/gate fusion,
 // decode/paged_attention.metal:266-309, 466-510).
 // With `partials_only` nothing is merged at all: every split writes its partial rows and
-// statistics, and the caller combines them (attention over a shared prefix merges the
-// prefix's splits with each sequence's own).
+// statistics, and the caller combines them (kv_attend_split; attention over a shared
+// prefix merges the prefix's splits with each sequence's own).  With `merge_only` no
+// split kernel runs: the workspace holds every split's rows already (kv_attend_merge).
 struct Epilogue {
   const uint16_t *packed_qkv;
   uint16_t *hidden;
   bool partials_only = false;
+  bool merge_only = false;
 };
 
 // ---- storage ----------------------------------------------------------------
@@ -114,10 +116,8 @@ struct Storage {
 // fewer waves by more than that.
 inline uint32_t verify_block_rows(uint32_t format, uint32_t fused_rows) {
   if (fused_rows <= 16) return 16;
-#ifndef KVX_NO_V48
   const uint32_t by32 = (fused_rows + 31) / 32, by48 = (fused_rows + 47) / 48;
   if (format == KVX_FMT_INT4 && 7 * by48 < 5 * by32) return 48;
-#endif
   return 32;
 }
 // Whether tiles 2i and 2i + 1 of a chunked prefill that starts after `committed`

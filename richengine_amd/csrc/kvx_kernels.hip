@@ -1190,10 +1190,6 @@ int dispatch_rows(uint32_t M, F &&f) {
   return fail(KVX_EINVAL, "tile holds more than 128 fused rows");
 }
 
-// Which attention phases the attend entries launch: bit 0 the split kernel,
-// bit 1 the merge.  Profiling harnesses clear a bit to time one kernel alone.
-uint32_t g_attend_phases = 3;
-
 int check_launch(const char *what) {
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? KVX_OK : hip_fail(e, what);
@@ -1249,8 +1245,6 @@ static int attend_matrix(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_h
                                 many_tiles, stream, tile_rows, epilogue);
 }
 
-uint32_t kvx_attend_phases() { return kvx::g_attend_phases; }
-
 namespace {
 uint64_t g_generic_attends = 0, g_matrix_attends = 0;
 int took(int fast) {  // counts which kernels an attend call went to
@@ -1262,7 +1256,6 @@ int took(int fast) {  // counts which kernels an attend call went to
 
 extern "C" {
 
-void kvx_debug_set_attend_phases(uint32_t phases) { kvx::g_attend_phases = phases & 3u; }
 void kvx_debug_attend_paths(uint64_t *generic_calls, uint64_t *matrix_core_calls) {
   if (generic_calls) *generic_calls = g_generic_attends;
   if (matrix_core_calls) *matrix_core_calls = g_matrix_attends;
@@ -1432,6 +1425,7 @@ int kv_prepare_append(const kvx_storage *s, uint32_t layer, const kvx_qkv_shape 
   return KVX_OK;
 }
 
+// page_tables may be null where no pages are read (the merge alone).
 static int validate_attend(const kvx_storage *s, uint32_t query_heads,
                            const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
                            const uint64_t *const *page_tables, uint64_t workspace_bytes) {
@@ -1452,7 +1446,13 @@ static int validate_attend(const kvx_storage *s, uint32_t query_heads,
       return fail(KVX_EINVAL, "page_table_too_short");
     if (!p.split_count || p.split_count > max_splits)
       return fail(KVX_EINVAL, "verify split count is out of range");
-    if (!page_tables[i]) return fail(KVX_EINVAL, "null page table");
+    // The reference strides a lane's slots by slot_splits and requires
+    // split_count <= slot_splits <= the maximum (common/paged_attention_tile.h:57-58).
+    // Slots are packed by split_count here, so the field only has to be consistent;
+    // 0 stands for "the split count".
+    if (p.slot_splits && (p.slot_splits < p.split_count || p.slot_splits > max_splits))
+      return fail(KVX_EINVAL, "verify slot splits are out of range");
+    if (page_tables && !page_tables[i]) return fail(KVX_EINVAL, "null page table");
   }
   if (capacity * (query_heads / l.kv_heads) > 128)
     return fail(KVX_EINVAL, "tile holds more than 128 fused rows");
@@ -1465,12 +1465,13 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
                           const void *queries, void *output, const uint64_t *const *page_tables,
                           const kvx_verify_params *lanes, uint32_t n_lanes,
                           const uint32_t *row_masks, uint32_t row_stride, void *workspace,
-                          hipStream_t stream, uint32_t phases,
-                          const Epilogue *epilogue = nullptr) {
+                          hipStream_t stream, const Epilogue *epilogue = nullptr) {
+  // The generic split kernel always writes partial rows; the phases are its two launches.
+  const uint32_t phases = (epilogue && epilogue->merge_only ? 0u : 1u) |
+                          (epilogue && epilogue->partials_only ? 0u : 2u);
   const kvx_layout &l = s->layout;
   const uint32_t H = l.kv_heads, G = query_heads / H, D = l.head_dim;
   const uint32_t capacity = lanes[0].row_capacity, M = capacity * G;
-  phases &= g_attend_phases;
   uint64_t total_rows = 0;
   for (uint32_t i = 0; i < n_lanes; ++i) total_rows += uint64_t(lanes[i].split_count) * H * M;
   float *partials = static_cast<float *>(workspace);
@@ -1486,7 +1487,7 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
     a.row_capacity = capacity;
     a.row_stride = row_stride;
     a.kv = kv;
-    if (epilogue) {
+    if (epilogue && epilogue->hidden) {
       a.hidden = epilogue->hidden + uint64_t(first) * capacity * query_heads * D;
       a.packed_qkv = epilogue->packed_qkv
                          ? epilogue->packed_qkv +
@@ -1497,7 +1498,7 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
     for (uint32_t i = 0; i < a.n_lanes; ++i) {
       const kvx_verify_params &p = lanes[first + i];
       AttendLane &al = a.lane[i];
-      al.table = page_tables[first + i];
+      al.table = page_tables ? page_tables[first + i] : nullptr;
       al.committed = p.committed_tokens;
       al.entries = p.page_table_entries;
       al.split_count = p.split_count;
@@ -1536,10 +1537,13 @@ static int attend_verify(const char *entry, const kvx_storage *s, uint32_t layer
                          uint32_t n_lanes, const uint32_t *row_masks, uint32_t row_stride,
                          void *workspace, uint64_t workspace_bytes, const Epilogue *epilogue,
                          void *stream) {
-  if (!s || !queries || (!output && !epilogue) || !page_tables || !lanes || !n_lanes || !workspace)
+  const bool merges = !(epilogue && epilogue->partials_only);
+  const bool splits = !(epilogue && epilogue->merge_only);
+  if (!s || !lanes || !n_lanes || !workspace || (splits && (!queries || !page_tables)) ||
+      (merges && !output && !(epilogue && epilogue->hidden)))
     return fail(KVX_EINVAL, std::string(entry) + ": null argument or no lanes");
   if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
-  if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
+  if (queries && queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
   kvx_kv_layer kv;
   if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
   if (row_masks && s->layout.format == KVX_FMT_FP8E4M3)
@@ -1554,7 +1558,27 @@ static int attend_verify(const char *entry, const kvx_storage *s, uint32_t layer
       workspace_bytes, 0, static_cast<hipStream_t>(stream), 0, epilogue));
   if (fast <= 0) return fast;
   return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks,
-                        row_stride, workspace, static_cast<hipStream_t>(stream), 3, epilogue);
+                        row_stride, workspace, static_cast<hipStream_t>(stream), epilogue);
+}
+
+int kv_attend_split(const kvx_storage *s, uint32_t layer, uint32_t query_heads, const void *queries,
+                    const uint64_t *const *page_tables, const kvx_verify_params *lanes,
+                    uint32_t n_lanes, const uint32_t *row_masks, uint32_t row_stride,
+                    void *workspace, uint64_t workspace_bytes, void *stream) {
+  Epilogue epilogue{nullptr, nullptr};
+  epilogue.partials_only = true;
+  return attend_verify("kv_attend_split", s, layer, query_heads, queries, nullptr, page_tables,
+                       lanes, n_lanes, row_masks, row_stride, workspace, workspace_bytes, &epilogue,
+                       stream);
+}
+
+int kv_attend_merge(const kvx_storage *s, uint32_t query_heads, void *output,
+                    const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                    void *workspace, uint64_t workspace_bytes, void *stream) {
+  Epilogue epilogue{nullptr, nullptr};
+  epilogue.merge_only = true;
+  return attend_verify("kv_attend_merge", s, 0, query_heads, nullptr, output, nullptr, lanes,
+                       n_lanes, nullptr, row_stride, workspace, workspace_bytes, &epilogue, stream);
 }
 
 int kv_attend_verify(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
@@ -1748,7 +1772,7 @@ int kv_attend_decode(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
       workspace_bytes, 0, static_cast<hipStream_t>(stream)));
   if (fast <= 0) return fast;
   return attend_generic(s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, nullptr,
-                        row_stride, workspace, static_cast<hipStream_t>(stream), 3);
+                        row_stride, workspace, static_cast<hipStream_t>(stream));
 }
 
 int kv_append_attend_decode(const kvx_storage *s, uint32_t layer, const void *chunk_keys,

@@ -35,7 +35,7 @@ SYMBOLS = [
     "kvx_pool_acquire", "kvx_pool_retain", "kvx_pool_release", "kvx_pool_page_active",
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
     "kvx_pool_snapshot_get", "kv_append", "kv_prepare_append", "kv_attend_decode_shared", "kvx_attend_shared_workspace_bytes", "kv_attend_verify", "kv_attend_verify_hidden", "kv_attend_decode",
-    "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kv_page_export", "kv_page_import", "kvx_debug_set_attend_phases",
+    "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kv_page_export", "kv_page_import", "kv_attend_split", "kv_attend_merge",
     "kvx_debug_attend_paths", "kvx_decode_plan", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
     "kvx_prefix_chain", "kvx_prefix_retain_active", "kvx_prefix_release_active",
@@ -233,6 +233,8 @@ def _declare(L):
     L.kv_attend_verify_hidden.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, vp, u32, vp, u64, vp, vp,
                                           vp]
     L.kv_attend_decode.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, u32, vp, u64, vp]
+    L.kv_attend_split.argtypes = [vp, u32, u32, vp, vp, vp, u32, vp, u32, vp, u64, vp]
+    L.kv_attend_merge.argtypes = [vp, u32, vp, vp, u32, u32, vp, u64, vp]
     L.kv_attend_decode_shared.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, u32, u32, u32, vp, u64, vp]
     L.kvx_attend_shared_workspace_bytes.argtypes = [vp, u32, u32, u32, C.POINTER(Layout)]
     L.kvx_attend_shared_workspace_bytes.restype = u64
@@ -240,7 +242,6 @@ def _declare(L):
                                           u64, vp]
     L.kv_attend_prefill.argtypes = [vp, u32, u32, vp, vp, vp, C.POINTER(PrefillParams), vp, u64, vp]
     L.kv_compact_path.argtypes = [vp, u32, vp, vp, u32, vp, vp, u32, vp]
-    L.kvx_debug_set_attend_phases.argtypes, L.kvx_debug_set_attend_phases.restype = [u32], None
 
 
 def check(rc):
@@ -390,6 +391,24 @@ def attend_verify(storage, layer, query_heads, queries, output, tables, lanes, r
                                         row_stride, _ptr(workspace),
                                         workspace.numel() * workspace.element_size(),
                                         _stream(stream)))
+
+
+def attend_split(storage, layer, query_heads, queries, tables, lanes, row_masks, row_stride,
+                 workspace, stream=None):
+    """The split dispatch alone: partial rows and statistics of every split into `workspace`."""
+    arr = lanes if isinstance(lanes, C.Array) else (VerifyParams * len(lanes))(*lanes)
+    return check(lib().kv_attend_split(storage.h, layer, query_heads, _ptr(queries),
+                                       _table_array(tables), arr, len(arr), _ptr(row_masks),
+                                       row_stride, _ptr(workspace),
+                                       workspace.numel() * workspace.element_size(), _stream(stream)))
+
+
+def attend_merge(storage, query_heads, output, lanes, row_stride, workspace, stream=None):
+    """The merge dispatch alone over a workspace in kv_attend_split's layout."""
+    arr = lanes if isinstance(lanes, C.Array) else (VerifyParams * len(lanes))(*lanes)
+    return check(lib().kv_attend_merge(storage.h, query_heads, _ptr(output), arr, len(arr),
+                                       row_stride, _ptr(workspace),
+                                       workspace.numel() * workspace.element_size(), _stream(stream)))
 
 
 def attend_verify_hidden(storage, layer, query_heads, queries, output, tables, lanes, row_masks,

@@ -85,7 +85,12 @@ def bf16_ulp_diff(a_bits, b_bits):
     return np.abs(key(a_bits) - key(b_bits))
 
 
-def check_attention(out_bits, want_bits, want_f32, rows_mask, tol, label="", matrix_core=False):
+# Rows that were farther from the oracle than the tolerance and were shown to be one
+# rounding flip away from it, per check: (label, rows explained, rows checked).
+ALLOWANCE_LOG = []
+
+
+def check_attention(out_bits, want_bits, want_f32, rows_mask, tol, label="", explain=None):
     """out_bits / want_bits: bf16 outputs (GPU, oracle); want_f32: the oracle's
     value before its final rounding.  rows_mask selects live rows (last axis D).
 
@@ -95,54 +100,101 @@ def check_attention(out_bits, want_bits, want_f32, rows_mask, tol, label="", mat
     2.0e-3 in this norm (the oracle's own bf16 output is that far from its
     fp32 value), which would leave no room for anything else.
 
-    matrix_core: kernels that sum q.k on the matrix cores cannot keep the
-    oracle's summation order, so a score can differ in its last bits and the
-    bf16 rounding of one probability can fall the other way.  When that
-    probability dominates its row, the row moves by up to half a bf16 step
-    (2e-3) on top of everything else.  For those kernels at least 99% of the
-    rows must meet tol and every row tol + 2e-3."""
+    explain: for kernels that sum q.k on the matrix cores, which cannot keep the
+    oracle's summation order: a score can differ in its last bits, so the rounding
+    of one probability (to bf16; fp16 on fp8 pages) can fall the other way, and when
+    that token carries most of its row the row moves by up to half a place.  A row
+    above tol is accepted only if that is shown to be what happened: explain(index)
+    describes the row's tile (keyword arguments of ko.rounding_flip_rows, or {"rows": ...}
+    with such rows from an arrangement of the caller's own), the oracle
+    recomputes the row with the rounded weight of one of its heaviest tokens moved
+    one place up or down, and one of those rows must be within tol of the GPU's.
+    At most 1% of the rows (one where there are fewer than a hundred) may need it and
+    none may be more than tol + 2e-3 away; every such row is counted in ALLOWANCE_LOG."""
     got = ko.bf16_to_f32(out_bits).reshape(out_bits.shape)
     want = ko.bf16_to_f32(want_bits).reshape(want_bits.shape)
     assert np.isfinite(got).all(), f"{label}: non-finite attention output"
     rel = T.rel_l2(got[rows_mask], want[rows_mask])
-    flat = np.unravel_index(int(np.argmax(rel)), rel.shape)
-    worst = tuple(int(x) for x in np.argwhere(rows_mask)[flat[0]]) + tuple(int(x) for x in flat[1:])
-    hard = tol + 2e-3 if matrix_core else tol
-    assert rel.max() <= hard, (f"{label}: relative L2 vs oracle bf16 {rel.max():.3e} > {hard} "
-                               f"at row {worst}")
-    within = float((rel <= tol).mean())
-    # 1% of the rows, and at least one where there are fewer than a hundred
-    allowed = max(1, int(0.01 * rel.size)) if matrix_core else 0
-    assert int((rel > tol).sum()) <= allowed, (
-        f"{label}: only {within:.4f} of the {rel.size} rows are within {tol}")
+    coords = np.argwhere(rows_mask)
+
+    def index_of(flat):
+        at = np.unravel_index(int(flat), rel.shape)
+        return tuple(int(x) for x in coords[at[0]]) + tuple(int(x) for x in at[1:])
+
+    over = np.flatnonzero(rel.ravel() > tol)
+    within = 1.0 - over.size / rel.size
+    if over.size:
+        worst = index_of(np.argmax(rel))
+        assert explain is not None, (f"{label}: relative L2 vs oracle bf16 {rel.max():.3e} > {tol} "
+                                     f"at row {worst}")
+        assert rel.max() <= tol + 2e-3, (f"{label}: relative L2 vs oracle bf16 {rel.max():.3e} > "
+                                         f"{tol + 2e-3} at row {worst}")
+        assert over.size <= max(1, int(0.01 * rel.size)), (
+            f"{label}: only {within:.4f} of the {rel.size} rows are within {tol}")
+        for flat in over:
+            index = index_of(flat)
+            mine = got[index]
+            flipped = None
+            described = explain(index)
+            candidates = described["rows"] if "rows" in described else ko.rounding_flip_rows(**described)
+            for token, steps, bits in candidates:
+                other = ko.bf16_to_f32(bits).reshape(mine.shape)
+                if T.rel_l2(mine[None], other[None])[0] <= tol:
+                    flipped = (token, steps)
+                    break
+            assert flipped, (f"{label}: row {index} is {rel.ravel()[flat]:.3e} from the oracle and no "
+                             f"single rounding flip of its heaviest tokens explains it")
+    if explain is not None:
+        ALLOWANCE_LOG.append((label, int(over.size), int(rel.size)))
     rel32 = T.rel_l2(got[rows_mask], want_f32[rows_mask])
-    assert rel32.max() <= tol + 2e-3, f"{label}: relative L2 vs oracle fp32 {rel32.max():.3e}"
+    bound32 = np.full(rel32.shape, tol + 2e-3)
+    bound32.ravel()[over] += 2e-3  # an explained row: half a place more
+    assert (rel32 <= bound32).all(), f"{label}: relative L2 vs oracle fp32 {rel32.max():.3e}"
     ulps = bf16_ulp_diff(out_bits[rows_mask], want_bits[rows_mask])
     return dict(rel_l2=float(rel.max()), rel_l2_mean=float(rel.mean()), rows_within_tol=within,
-                rel_l2_fp32=float(rel32.max()),
+                rel_l2_fp32=float(rel32.max()), explained_rows=int(over.size),
                 max_abs=float(np.abs(got[rows_mask] - want_f32[rows_mask]).max()),
                 exact=float((ulps == 0).mean()), max_ulp=int(ulps.max()))
 
 
+def lanes_explainer(fmt, kv_heads, group, head_dim, queries, tables, kv, committed, active, splits,
+                    capacity, masks=None, one_row=False):
+    """explain() for outputs indexed (lane, KV head, row, head in group) over verify-shaped
+    queries [lane][KV head][row stride][group][D]; committed / active / splits per lane.
+    one_row: outputs indexed (lane, KV head, head in group), row 0 (decode)."""
+    def explain(index):
+        if one_row:
+            lane, head, g = index
+            row = 0
+        else:
+            lane, head, row, g = index
+        return dict(fmt=fmt, kv_heads=kv_heads, group=group, head_dim=head_dim,
+                    tile_queries=queries[lane, head, :capacity].reshape(capacity * group, head_dim),
+                    table=tables[lane], kv=kv, head=head, committed=int(committed[lane]),
+                    active=int(active[lane] if np.ndim(active) else active), splits=int(splits[lane]),
+                    capacity=capacity, fused_row=row * group + g,
+                    masks=None if masks is None else masks[lane])
+    return explain
+
+
+def prefill_explainer(fmt, kv_heads, group, head_dim, queries, table, kv, committed, rows, splits):
+    """explain() for outputs indexed (KV head, chunk row, head in group) of a chunked prefill
+    over queries [KV head][chunk stride][group][D]: the row's 8-row tile."""
+    def explain(index):
+        head, row, g = index
+        tile = row // 8
+        tile_queries = np.zeros((8, group, head_dim), dtype=np.uint16)
+        live = queries[head, 8 * tile:8 * tile + 8]
+        tile_queries[:live.shape[0]] = live
+        return dict(fmt=fmt, kv_heads=kv_heads, group=group, head_dim=head_dim,
+                    tile_queries=tile_queries.reshape(8 * group, head_dim), table=table, kv=kv,
+                    head=head, committed=committed + 8 * tile, active=min(8, rows - 8 * tile),
+                    splits=splits, capacity=8, fused_row=(row % 8) * group + g)
+    return explain
+
+
 def oracle_tile(fmt, kv_heads, group, head_dim, tile_queries, table, kv, head, committed, active,
                 splits, capacity, masks=None, score_scale=0.0):
-    """The oracle's attention of one tile (capacity rows x group fused rows) of one
-    KV head: every split's partial tile, then the fixed-order merge of each live
-    fused row.  tile_queries: bf16 [capacity * group, D].  Returns (bf16, fp32)
-    outputs of that shape; rows past `active` are zeros."""
-    L = ko.lib()
-    M, D = capacity * group, head_dim
-    tile_queries = np.ascontiguousarray(tile_queries, dtype=np.uint16).reshape(M, D)
-    partials = np.zeros((splits, M, D), dtype=np.float32)
-    statistics = np.zeros((splits, M, 2), dtype=np.float32)
-    mask_ptr = ko.ptr(np.ascontiguousarray(masks, dtype=np.uint32)) if masks is not None else None
-    for split in range(splits):
-        L.ko_attention_tile(fmt, kv_heads, group, D, capacity, ko.ptr(tile_queries), ko.ptr(table), kv,
-                            head, committed, active, splits, split, ko.ptr(partials),
-                            ko.ptr(statistics), split, mask_ptr, score_scale)
-    out = np.zeros((M, D), dtype=np.uint16)
-    out32 = np.zeros((M, D), dtype=np.float32)
-    for row in range(M):
-        L.ko_attention_reduce_row(group, D, capacity, ko.ptr(partials), ko.ptr(statistics), committed,
-                                  active, splits, 0, row, ko.ptr(out[row]), ko.ptr(out32[row]))
-    return out, out32
+    """The oracle's attention of one tile of one KV head (ko.attention_tile_rows)."""
+    return ko.attention_tile_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv, head,
+                                  committed, active, splits, capacity, masks, score_scale)

@@ -122,8 +122,10 @@ def prefill_case(fmt, committed, rows):
     got = Gp.host_u16(out)
     live = np.zeros((H, stride), dtype=bool)
     live[:, :rows] = True
-    stats = Gp.check_attention(got, want, want32, live, tol(fmt), f"prefill fmt={fmt}",
-                               matrix_core=fmt in MATRIX)
+    stats = Gp.check_attention(got, want, want32, live, tol(fmt),
+                               f"prefill fmt={fmt} H={H} G={G} committed={committed} rows={rows}",
+                               explain=Gp.prefill_explainer(fmt, H, G, D, q, th, tw.host.layer(1),
+                                                            committed, rows, splits))
     # the matrix cores sum in another order than the oracle; the mean stays far
     # below the per-row bar
     assert stats["rel_l2_mean"] < 5e-4
@@ -166,8 +168,10 @@ def test_verify_chain_matches_oracle(fmt):
         got = Gp.host_u16(out)
         live = np.zeros((1, H, 32), dtype=bool)
         live[:, :, :8] = True
-        Gp.check_attention(got, want, want32, live, tol(fmt), f"verify lane {lane}",
-                           matrix_core=fmt in MATRIX)
+        Gp.check_attention(got, want, want32, live, tol(fmt),
+                           f"verify chain fmt={fmt} H={H} G={G} committed={committed[lane]}",
+                           explain=Gp.lanes_explainer(fmt, H, G, D, q, [hts[lane]], tw.host.layer(1),
+                                                      [committed[lane]], 8, [splits], 8))
         assert (got[:, :, 8:] == 0x5A5A).all()
     for tw in tws:
         tw.close()
@@ -222,8 +226,10 @@ def test_batched_verify_chain_matches_oracle(fmt):
     torch.cuda.synchronize()
     live = np.zeros((lanes, H, 32), dtype=bool)
     live[:, :, :8] = True
-    Gp.check_attention(Gp.host_u16(out), want, want32, live, tol(fmt), "batched verify",
-                       matrix_core=fmt in MATRIX)
+    Gp.check_attention(Gp.host_u16(out), want, want32, live, tol(fmt),
+                       f"batched verify chain fmt={fmt} H={H} G={G}",
+                       explain=Gp.lanes_explainer(fmt, H, G, D, q, hts, tw.host.layer(1), committed, 8,
+                                                  splits, 8))
     # a repeat submission gives the same bits
     out2 = torch.zeros_like(out)
     kvx.attend_verify(tw.dev, 1, QH, Gp.dev(q), out2, dts, dp, None, 32, ws)
@@ -266,8 +272,10 @@ def test_tree_verify_matches_oracle(fmt, nodes):
     got = Gp.host_u16(out)
     live = np.zeros((lanes, H, 32), dtype=bool)
     live[:, :, :nodes] = True
-    Gp.check_attention(got, want, want32, live, tol(fmt), "tree verify",
-                       matrix_core=fmt in MATRIX)
+    Gp.check_attention(got, want, want32, live, tol(fmt),
+                       f"tree verify fmt={fmt} H={H} G={G} nodes={nodes}",
+                       explain=Gp.lanes_explainer(fmt, H, G, D, q, hts, tw.host.layer(1), committed,
+                                                  nodes, splits, 16, masks))
     assert not got[:, :, nodes:16].any() and (got[:, :, 16:] == 0x5A5A).all()
     tw.close()
 
@@ -306,7 +314,9 @@ def test_int4_small_tree_verify_in_one_wave(nodes, capacity):
     got = Gp.host_u16(out)
     live = np.zeros((lanes, H, 32), dtype=bool)
     live[:, :, :nodes] = True
-    Gp.check_attention(got, want, want32, live, tol(fmt), "small tree verify", matrix_core=True)
+    Gp.check_attention(got, want, want32, live, tol(fmt), f"small tree verify nodes={nodes}",
+                       explain=Gp.lanes_explainer(fmt, H, G, D, q, hts, tw.host.layer(1), committed,
+                                                  nodes, splits, capacity, masks))
     assert not got[:, :, nodes:capacity].any() and (got[:, :, capacity:] == 0x5A5A).all()
     tw.close()
 
@@ -336,7 +346,9 @@ def decode_case(fmt, committed, seed, row_stride=1, layers=2, layer=1):
     torch.cuda.synchronize()
     got = Gp.host_u16(out)
     stats = Gp.check_attention(got[:, :, 0], want, want32, np.ones((lanes, H), dtype=bool), tol(fmt),
-                               f"decode fmt={fmt} committed={committed}", matrix_core=fmt in MATRIX)
+                               f"decode fmt={fmt} H={H} G={G} committed={committed}",
+                               explain=Gp.lanes_explainer(fmt, H, G, D, q, hts, tw.host.layer(layer),
+                                                          committed, 1, splits, 1, one_row=True))
     assert stats["rel_l2_mean"] < 5e-4
     if row_stride > 1:
         assert (got[:, :, 1:] == 0x5A5A).all()
@@ -383,7 +395,9 @@ def test_invalid_attention_parameters_enqueue_nothing():
     ws = torch.full((kvx.attend_workspace_bytes(tw.dev, [good], QH),), 0xA5, dtype=torch.uint8, device="cuda")
     cases = []
     for field, value in (("page_table_entries", 1), ("split_count", 0), ("split_count", 129),
-                         ("active_rows", 0), ("active_rows", 9), ("committed_tokens", 262159)):
+                         ("active_rows", 0), ("active_rows", 9), ("committed_tokens", 262159),
+                         # common/paged_attention_tile.h:57-58: split_count <= slot_splits <= maximum
+                         ("slot_splits", 31), ("slot_splits", 129)):
         p = kvx.VerifyParams(40, counts[0], kvx.KvLayer(), 32, 32, 8, 8, 0.0)
         setattr(p, field, value)
         cases.append(p)

@@ -119,7 +119,9 @@ def test_config2_int4_long_context_batch1():
     got = decode_on_device(tw, 1, q, [td], [committed], [n_pages], splits)
     want, want32 = decode_on_oracle(tw, 1, q, [th], [committed], [n_pages], splits)
     stats = Gp.check_attention(got, want, want32, np.ones((1, H), dtype=bool), tol(ko.INT4),
-                               "config 2", matrix_core=True)
+                               "config 2",
+                               explain=Gp.lanes_explainer(ko.INT4, H, G, D, q, [th], tw.host.layer(1),
+                                                          [committed], 1, splits, 1, one_row=True))
     assert stats["rel_l2_mean"] < 1e-3
     # placement invariance: move every page to a shuffled id, attend again
     shuffled = (n_pages + np.random.default_rng(4).permutation(n_pages)).astype(np.uint32)
@@ -153,7 +155,9 @@ def test_config3_int4_mixed_batch32():
     got = decode_on_device(tw, 0, q, dts, contexts, counts, splits)
     want, want32 = decode_on_oracle(tw, 0, q, hts, contexts, counts, splits)
     stats = Gp.check_attention(got, want, want32, np.ones((32, H), dtype=bool), tol(ko.INT4),
-                               "config 3", matrix_core=True)
+                               "config 3",
+                               explain=Gp.lanes_explainer(ko.INT4, H, G, D, q, hts, tw.host.layer(0),
+                                                          contexts, 1, splits, 1, one_row=True))
     assert stats["rel_l2_mean"] < 5e-4
     tw.close()
 
@@ -240,8 +244,13 @@ def test_config4_shared_prefix_chunked_prefill(fmt):
             want, want32 = Gp.oracle_tile(fmt, H, G, D, tile_q, table_host, tw.host.layer(0), head,
                                           prefix + 8 * tile, 8, splits, 8)
             mine = got[head, 8 * tile:8 * tile + 8].reshape(8 * G, D)
-            stats = Gp.check_attention(mine, want, want32, np.ones(8 * G, dtype=bool), tol(fmt),
-                                       f"config 4 tile {tile} head {head}", matrix_core=True)
+            stats = Gp.check_attention(
+                mine, want, want32, np.ones(8 * G, dtype=bool), tol(fmt),
+                f"config 4 fmt={fmt} tile {tile} head {head}",
+                explain=lambda index: dict(fmt=fmt, kv_heads=H, group=G, head_dim=D, tile_queries=tile_q,
+                                           table=table_host, kv=tw.host.layer(0), head=head,
+                                           committed=prefix + 8 * tile, active=8, splits=splits,
+                                           capacity=8, fused_row=index[0]))
             rels.append(stats["rel_l2_mean"])
     assert np.mean(rels) < (4e-3 if fmt == ko.FP8 else 1e-3)
     for s in range(1, sequences + 1):
@@ -249,6 +258,114 @@ def test_config4_shared_prefix_chunked_prefill(fmt):
     for p in spare:
         pool.release(p)
     assert pool.snapshot().pages_active == 0 and pool.snapshot().pages_prefix == prefix_pages
+    seqs.close()
+    cache.close()
+    pool.close()
+    tw.close()
+
+
+@pytest.mark.parametrize("fmt", [ko.BF16, ko.FP8, ko.INT4])
+def test_config4_copy_on_write_of_the_partial_last_page(fmt):
+    """configs[3] with a prefix that does not end on a page boundary: 16 400 tokens = 512 whole
+    pages and 16 tokens of a 513th.  The second sequence forks the first at 16 400 tokens (every
+    page shared by reference, the partial one included), and its first store triggers the copy:
+    kv_page_copy of the partial page, every layer, into a page of its own, then the chunk's rows
+    from slot 16 on.  The reference shares whole pages only (runtime/engine/cache/Cache.cpp:183-184,
+    :774), so the pins are invariants: the copy is the source's bytes, the source is untouched,
+    the references add up, and after the store every byte equals the oracle's page copy + store."""
+    prefix, chunk, layers = 16400, 2048, 2
+    whole = prefix // 32
+    prefix_pages, total_pages = whole + 1, whole + 1 + 2 * ((prefix % 32 + chunk + 31) // 32) + 8
+    tw = Gp.Twin(fmt, H, D, layers, total_pages, one_extent=True)
+    tw.dev.release(0)                      # the pool allocates the device extent itself
+    pool = kvx.Pool(tw.dev, tw.dev.page_count)
+    cache = kvx.Prefix(pool)
+    seqs = kvx.Sequences(pool, cache)
+    gen = torch.Generator(device="cuda").manual_seed(44)
+    tokens = [(11 * i) % 50021 for i in range(prefix + chunk)]
+    # the first sequence computes the prefix and publishes its whole pages
+    seqs.begin(1)
+    seqs.ensure_tokens(1, prefix)
+    one = seqs.view(1)
+    assert len(one["pages"]) == prefix_pages
+    table1 = tw.dev.table(np.array(one["pages"], dtype=np.uint32))
+    for layer in range(layers):
+        device_history(tw, layer, table1, prefix_pages, 0, prefix, gen, outliers=True)
+    torch.cuda.synchronize()
+    seqs.publish(1, tokens, prefix)
+    assert len(seqs.view(1)["blocks"]) == whole
+    # the fork: all 513 pages by reference, no copy yet
+    seqs.begin(2)
+    seqs.fork(2, 1, prefix)
+    two = seqs.view(2)
+    assert two["pages"] == one["pages"] and two["blocks"] == seqs.view(1)["blocks"]
+    snap = pool.snapshot()
+    assert snap.pages_active == prefix_pages and snap.pages_prefix == whole
+    partial = one["pages"][whole]
+    source_bytes = tw.dev.page_read(partial)
+    assert source_bytes.any()
+    tw.download()                          # the oracle's store takes over the history so far
+    # the fork's first store: copy-on-write of the partial page, then pages for the chunk
+    moved = seqs.ensure_writable(2, prefix)
+    assert moved is not None and moved[0] == partial and moved[1] not in one["pages"]
+    copy = moved[1]
+    torch.cuda.synchronize()
+    assert np.array_equal(tw.dev.page_read(copy), source_bytes)        # every layer, every tensor
+    seqs.ensure_tokens(2, prefix + chunk)
+    two = seqs.view(2)
+    assert two["pages"][:whole] == one["pages"][:whole] and two["pages"][whole] == copy
+    assert not set(two["pages"][whole:]) & set(one["pages"])
+    assert two["first_changed"] == prefix_pages and two["revision"] == 3
+    n_entries = len(two["pages"])
+    snap = pool.snapshot()
+    assert snap.pages_active == prefix_pages + (n_entries - whole) and snap.pages_prefix == whole
+    assert all(pool.page_active(p) for p in one["pages"] + two["pages"])
+    # the oracle's side: its own whole-page copy, after which both stores hold the same bytes
+    assert tw.host.copy_pages([(partial, copy)]) == 0
+    tw.assert_same_bytes()
+    table2 = tw.dev.table(np.array(two["pages"], dtype=np.uint32))
+    table2_host = tw.host.entries(np.array(two["pages"], dtype=np.uint32))
+    k = torch.randn((H, chunk, D), generator=gen, device="cuda").bfloat16()
+    v = torch.randn((H, D, chunk), generator=gen, device="cuda").bfloat16()
+    for layer in range(layers):
+        kvx.append(tw.dev, layer, k, v, [table2], [kvx.ChunkParams(prefix, chunk, chunk, n_entries)],
+                   H * chunk * D)
+        p = ko.ChunkParams(prefix, chunk, chunk, n_entries, tw.host.layer(layer))
+        assert ko.store_chunk(fmt, H, D, Gp.host_u16(k.view(torch.int16)),
+                              Gp.host_u16(v.view(torch.int16)), table2_host, p) == 1
+    torch.cuda.synchronize()
+    tw.assert_same_bytes()                                             # copy + store, bit for bit
+    assert np.array_equal(tw.dev.page_read(partial), source_bytes)     # the shared page is untouched
+    # the copy: slots 0..15 are the source's rows, slots 16..31 the chunk's first rows
+    assert not np.array_equal(tw.dev.page_read(copy), source_bytes)
+    # attention of the chunk over prefix + chunk through the fork's table, sampled tiles
+    q = torch.randn((H, chunk, G, D), generator=gen, device="cuda").bfloat16()
+    splits = kvx.lib().kvx_prefill_splits(chunk)
+    ws = torch.empty(kvx.prefill_workspace_bytes(tw.dev, chunk, QH) + 256, dtype=torch.uint8, device="cuda")
+    out = torch.zeros((H, chunk, G, D), dtype=torch.int16, device="cuda")
+    kvx.attend_prefill(tw.dev, 1, QH, q, out, table2,
+                       kvx.PrefillParams(prefix, chunk, chunk, n_entries, kvx.KvLayer(), splits, 0.0), ws)
+    torch.cuda.synchronize()
+    q_host, got = Gp.host_u16(q.view(torch.int16)), Gp.host_u16(out)
+    for tile, head in ((0, 0), (1, 2), (255, 3)):
+        tile_q = q_host[head, 8 * tile:8 * tile + 8].reshape(8 * G, D)
+        want, want32 = Gp.oracle_tile(fmt, H, G, D, tile_q, table2_host, tw.host.layer(1), head,
+                                      prefix + 8 * tile, 8, splits, 8)
+        mine = got[head, 8 * tile:8 * tile + 8].reshape(8 * G, D)
+        Gp.check_attention(
+            mine, want, want32, np.ones(8 * G, dtype=bool), tol(fmt),
+            f"config 4 copy-on-write fmt={fmt} tile {tile} head {head}",
+            explain=lambda index: dict(fmt=fmt, kv_heads=H, group=G, head_dim=D, tile_queries=tile_q,
+                                       table=table2_host, kv=tw.host.layer(1), head=head,
+                                       committed=prefix + 8 * tile, active=8, splits=splits,
+                                       capacity=8, fused_row=index[0]))
+    # the source goes on writing its own page in place; the references unwind
+    assert seqs.ensure_writable(1, prefix) is None
+    seqs.end(1)
+    assert all(pool.page_active(p) for p in two["pages"]) and not pool.page_active(partial)
+    seqs.end(2)
+    snap = pool.snapshot()
+    assert snap.pages_active == 0 and snap.pages_prefix == whole
     seqs.close()
     cache.close()
     pool.close()
@@ -313,8 +430,13 @@ def test_config5_int4_tree_verify_and_rollback():
         want, want32 = Gp.oracle_tile(ko.INT4, H, G, D, tile_q, hts[lane], tw.host.layer(0), head,
                                       committed, nodes, splits[lane], 16, masks=masks[lane])
         mine = got[lane, head, :16].reshape(16 * G, D)
-        Gp.check_attention(mine, want, want32, np.ones(16 * G, dtype=bool), tol(ko.INT4),
-                           f"config 5 lane {lane} head {head}", matrix_core=True)
+        Gp.check_attention(
+            mine, want, want32, np.ones(16 * G, dtype=bool), tol(ko.INT4),
+            f"config 5 lane {lane} head {head}",
+            explain=lambda index: dict(fmt=ko.INT4, kv_heads=H, group=G, head_dim=D, tile_queries=tile_q,
+                                       table=hts[lane], kv=tw.host.layer(0), head=head,
+                                       committed=committed, active=nodes, splits=splits[lane],
+                                       capacity=16, fused_row=index[0], masks=masks[lane]))
     # a tree that is a path must see exactly what the chain sees
     chain_masks = np.zeros((lanes, nodes), dtype=np.uint32)
     chain_masks[:] = kvx.tree_masks([none] + list(range(nodes - 1)))

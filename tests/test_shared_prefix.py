@@ -103,7 +103,10 @@ def test_shared_prefix_decode_matches_oracle(fmt, shared_pages, own_tokens, pref
     got = Gp.host_u16(out)[:, :, 0]
     same, same32 = oracle_shared(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_splits, own_splits)
     Gp.check_attention(got, same, same32, np.ones((lanes, H), dtype=bool), A.tol(fmt),
-                       f"shared prefix fmt={fmt}", matrix_core=True)
+                       f"shared prefix fmt={fmt} pages={shared_pages}",
+                       explain=lambda index: dict(rows=flipped_rows(
+                           fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_splits, own_splits,
+                           committed, index)))
     # the ordinary decode of every sequence, another partition: see the module's note
     value = lambda bits: ko.bf16_to_f32(bits).reshape(bits.shape).astype(np.float64)
     apart = np.linalg.norm(value(got) - value(want), axis=-1) / np.linalg.norm(value(want), axis=-1)
@@ -127,8 +130,28 @@ def test_shared_prefix_decode_matches_oracle(fmt, shared_pages, own_tokens, pref
     tw.close()
 
 
-def oracle_shared(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_splits, own_splits, layer=1):
-    """The oracle's tiles in the shared arrangement, merged in the library's order."""
+def flipped_rows(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_splits, own_splits,
+                 committed, index, layer=1, top=4):
+    """For check_attention's allowance: output row (lane, head, head in group) in the shared
+    arrangement with the rounded weight of one of its heaviest tokens moved one place, the token
+    being in the prefix tile or in the sequence's own."""
+    lane, head, g = index
+    weights = np.zeros(committed[lane] + 1, dtype=np.float32)
+    ko.lib().ko_attention_row_weights(fmt, H, D, ko.ptr(np.ascontiguousarray(q[lane, head, 0, g])),
+                                      ko.ptr(hts[lane]), tw.host.layer(layer), head, committed[lane], 1,
+                                      0, None, 0.0, ko.ptr(weights))
+    for token in np.argsort(-weights, kind="stable")[:top]:
+        for steps in (1, -1):
+            bits, _ = oracle_shared(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_splits,
+                                    own_splits, layer, only=index, nudge=(int(token), steps))
+            yield int(token), steps, bits[lane, head, g]
+
+
+def oracle_shared(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_splits, own_splits, layer=1,
+                  only=None, nudge=None):
+    """The oracle's tiles in the shared arrangement, merged in the library's order.  only =
+    (lane, head, head in group): that output row alone; nudge = (token of the sequence, steps):
+    with the rounded weight of that token moved (see ko_attention_nudge)."""
     L = ko.lib()
     lanes = len(own_tokens)
     kv = tw.host.layer(layer)
@@ -139,27 +162,43 @@ def oracle_shared(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_spl
         per = -(-pages // splits)
         return -(-pages // per)
 
-    def tiles(queries, table, committed, active, capacity, splits, masks, head):
+    def tiles(queries, table, committed, active, capacity, splits, masks, head, moved=None):
         M = capacity * G
         partials = np.zeros((splits, M, D), dtype=np.float32)
         statistics = np.zeros((splits, M, 2), dtype=np.float32)
         tile_q = np.ascontiguousarray(queries, dtype=np.uint16).reshape(M, D)
-        for split in range(splits):
-            L.ko_attention_tile(fmt, H, G, D, capacity, ko.ptr(tile_q), ko.ptr(table), kv, head, committed,
-                                active, splits, split, ko.ptr(partials), ko.ptr(statistics), split,
-                                ko.ptr(masks) if masks is not None else None, 0.0)
+        if moved:
+            L.ko_attention_nudge(moved[0], moved[1], moved[2], 1)
+        try:
+            for split in range(splits):
+                L.ko_attention_tile(fmt, H, G, D, capacity, ko.ptr(tile_q), ko.ptr(table), kv, head,
+                                    committed, active, splits, split, ko.ptr(partials),
+                                    ko.ptr(statistics), split,
+                                    ko.ptr(masks) if masks is not None else None, 0.0)
+        finally:
+            L.ko_attention_nudge(-1, 0, 0, 0)
         return partials, statistics
 
     out = np.zeros((lanes, H, G, D), dtype=np.float32)
     zero_masks = np.zeros(lanes, dtype=np.uint32)
-    for head in range(H):
-        pp, ps = tiles(q[:, head, 0], hts[0], shared_pages * 32, lanes, lanes, prefix_splits, zero_masks, head)
-        pw = written(shared_pages * 32 + lanes, prefix_splits)
-        for i in range(lanes):
+    shared_tokens = shared_pages * 32
+    for head in range(H) if only is None else [only[1]]:
+        # a moved weight sits in one of the two tiles; with `only`, each tile computes one row
+        in_prefix = in_own = None
+        if only is not None:
+            in_prefix, in_own = (only[0] * G + only[2], 0, 0), (only[2], 0, 0)
+            if nudge and nudge[0] < shared_tokens:
+                in_prefix = (only[0] * G + only[2], nudge[0], nudge[1])
+            elif nudge:
+                in_own = (only[2], nudge[0] - shared_tokens, nudge[1])
+        pp, ps = tiles(q[:, head, 0], hts[0], shared_tokens, lanes, lanes, prefix_splits, zero_masks, head,
+                       in_prefix)
+        pw = written(shared_tokens + lanes, prefix_splits)
+        for i in range(lanes) if only is None else [only[0]]:
             own_table = np.ascontiguousarray(hts[i][shared_pages:])
-            op, os_ = tiles(q[i, head, 0], own_table, own_tokens[i], 1, 1, own_splits[i], None, head)
+            op, os_ = tiles(q[i, head, 0], own_table, own_tokens[i], 1, 1, own_splits[i], None, head, in_own)
             ow = written(own_tokens[i] + 1, own_splits[i])
-            for g in range(G):
+            for g in range(G) if only is None else [only[2]]:
                 rows = [(pp[k, i * G + g], ps[k, i * G + g]) for k in range(pw)]
                 rows += [(op[k, g], os_[k, g]) for k in range(ow)]
                 maximum = max(st[0] for _, st in rows)
