@@ -576,6 +576,21 @@ int kv_attend_decode(const kvx_storage *storage, uint32_t layer, uint32_t query_
                      const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
                      void *workspace, uint64_t workspace_bytes, void *stream);
 
+/* kv_attend_decode for callers that cannot allocate device memory or bring a workspace: code
+   under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart
+   in the reference.  The partial rows and statistics go to a static device array of the library
+   (KVX_STATIC_WORKSPACE_BYTES, held by every GPU the library runs on until the process ends)
+   instead of a workspace argument; the call allocates nothing, on the host or on the device.
+   KVX_EINVAL when kvx_attend_workspace_bytes() of the lanes exceeds the array (the headline batch
+   of 32 sequences at 507 splits needs 12.6 MB), KVX_ESTATE when the storage's device is not the
+   current device.  All calls on one GPU share the array: calls that overlap there (two streams,
+   two threads) race on it; calls on one stream, or ordered by events, do not. */
+#define KVX_STATIC_WORKSPACE_BYTES (32u << 20)
+int kv_attend_decode_static(const kvx_storage *storage, uint32_t layer, uint32_t query_heads,
+                            const void *queries, void *output, const uint64_t *const *page_tables,
+                            const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                            void *stream);
+
 /* One decode step of a layer in one call: kv_append of one token per lane at
    lanes[i].committed_tokens (chunk rows as for kv_append: keys [head][chunk_stride][D],
    values [head][D][chunk_stride], token 0 of each lane's chunk, lanes chunk_lane_stride

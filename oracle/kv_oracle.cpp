@@ -587,47 +587,59 @@ int ko_store_verify(uint32_t format, uint32_t kv_heads, uint32_t head_dim,
 
 // ------------------------------------------------------------- attention ---
 namespace {
-// A test's question to the oracle: "had the rounding of this one probability
-// fallen the other way, what would the row be?"  While set, the tile moves the
-// rounded weight of (fused row, token) by `steps` places of its format (bf16, or
-// fp16 on the fp8 path) and, with only_row, computes that fused row alone.
-struct Nudge {
+// A test's question to the oracle: "had the rounding of these probabilities fallen the
+// other way, what would the row be?"  While set, the tile looks at the weight
+// (probability x value scale) of each listed token of one fused row before it is rounded
+// to its format (bf16; fp16 on the fp8 path): where that value lies within `slack`
+// (relative) of the boundary between two neighbours of the format, the tile takes the
+// neighbour on the other side.  A weight that is not that close to a boundary is left
+// alone, so only roundings that a perturbation of `slack` in the score could have turned
+// are turned.  With only_row the tile computes that fused row alone.
+struct Flips {
   int64_t fused_row = -1;
-  uint32_t token = 0;
-  int steps = 0;
   bool only_row = false;
+  float slack = 0.0f;
+  uint32_t count = 0;
+  uint32_t tokens[32] = {};
+  uint32_t applied = 0;  // bit i: token i was close to a boundary and was turned
 };
-thread_local Nudge g_nudge;
+thread_local Flips g_flips;
 
-float step_bf16(float w, int steps) {
-  // weights are finite and not negative: neighbours in the format are neighbours as integers
-  const int bits = int(ko_float_to_bf16(w)) + steps;
-  return ko_bf16_to_float(uint16_t(bits < 0 ? 0 : bits));
+float next_up(float r, bool f16) {
+  // the neighbour above a non-negative value of the format
+  if (!f16) return ko_bf16_to_float(uint16_t(ko_float_to_bf16(r) + 1));
+  const int e = r < 6.103515625e-05f ? -14 : std::ilogb(r);
+  return r + std::ldexp(1.0f, e - 10);
 }
-float step_f16(float w, int steps) {
-  // w is a non-negative binary16 value: its neighbours lie one step of its binade away
-  // (2^-24 below 2^-14), and going down from a power of two the step halves.
-  for (int i = 0; i < (steps < 0 ? -steps : steps); ++i) {
-    const int e = w < 6.103515625e-05f ? -14 : std::ilogb(w);
-    float step = std::ldexp(1.0f, e - 10);
-    if (steps < 0) {
-      if (w == 0.0f) break;
-      if (e > -14 && w == std::ldexp(1.0f, e)) step *= 0.5f;
-      w -= step;
-    } else {
-      w += step;
-    }
-  }
-  return w;
+float next_down(float r, bool f16) {
+  if (r == 0.0f) return 0.0f;
+  if (!f16) return ko_bf16_to_float(uint16_t(ko_float_to_bf16(r) - 1));
+  const int e = r < 6.103515625e-05f ? -14 : std::ilogb(r);
+  const float step = std::ldexp(1.0f, e - 10);
+  return r - ((e > -14 && r == std::ldexp(1.0f, e)) ? 0.5f * step : step);
+}
+// `rounded` is `w` rounded to the format; the value on the other side of the nearest
+// rounding boundary if w is within slack * w of it, else `rounded`.
+float turned(float w, float rounded, bool f16, float slack, bool *did) {
+  const float lo = rounded <= w ? rounded : next_down(rounded, f16);
+  const float hi = rounded <= w ? next_up(rounded, f16) : rounded;
+  const float boundary = 0.5f * (lo + hi);
+  if (!(std::fabs(w - boundary) <= slack * w)) return rounded;
+  *did = true;
+  return rounded == lo ? hi : lo;
 }
 }  // namespace
 
-void ko_attention_nudge(int64_t fused_row, uint32_t token, int steps, int only_row) {
-  g_nudge.fused_row = fused_row;
-  g_nudge.token = token;
-  g_nudge.steps = steps;
-  g_nudge.only_row = only_row != 0;
+void ko_attention_flips(int64_t fused_row, const uint32_t *tokens, uint32_t count, float slack,
+                        int only_row) {
+  g_flips = Flips{};
+  g_flips.fused_row = fused_row;
+  g_flips.only_row = only_row != 0;
+  g_flips.slack = slack;
+  g_flips.count = std::min<uint32_t>(count, 32);
+  for (uint32_t i = 0; i < g_flips.count; ++i) g_flips.tokens[i] = tokens[i];
 }
+uint32_t ko_attention_flips_applied(void) { return g_flips.applied; }
 
 void ko_attention_row_weights(uint32_t format, uint32_t kv_heads, uint32_t head_dim,
                               const uint16_t *query_row, const uint64_t *page_table, ko_kv_layer kv,
@@ -693,7 +705,7 @@ int ko_attention_tile(uint32_t format, uint32_t kv_heads, uint32_t group, uint32
     // Rows past the live ones are never read by the merge (it writes zeros
     // for them), so the oracle leaves their partials untouched.
     if (query_row >= active_rows) continue;
-    if (g_nudge.only_row && g_nudge.fused_row >= 0 && int64_t(r) != g_nudge.fused_row) continue;
+    if (g_flips.only_row && g_flips.fused_row >= 0 && int64_t(r) != g_flips.fused_row) continue;
     for (uint32_t d = 0; d < D; ++d) {
       const float v = ko_bf16_to_float(tile_queries[uint64_t{r} * D + d]);
       q[d] = fp8 ? ko_round_to_f16(v) : v;  // fp8 tile stages queries as fp16
@@ -745,8 +757,13 @@ int ko_attention_tile(uint32_t format, uint32_t kv_heads, uint32_t group, uint32
         float w = 0.0f;
         if (admitted[j] && score[j] > -kInf) w = prob[j] * (quant ? s.value_scales[j] : 1.0f);
         weight[j] = fp8 ? ko_round_to_f16(w) : ko_bf16_to_float(ko_float_to_bf16(w));
-        if (g_nudge.fused_row == int64_t(r) && g_nudge.token == token_start + j && g_nudge.steps)
-          weight[j] = fp8 ? step_f16(weight[j], g_nudge.steps) : step_bf16(weight[j], g_nudge.steps);
+        if (g_flips.fused_row == int64_t(r))
+          for (uint32_t f = 0; f < g_flips.count; ++f)
+            if (g_flips.tokens[f] == token_start + j) {
+              bool did = false;
+              weight[j] = turned(w, weight[j], fp8, g_flips.slack, &did);
+              if (did) g_flips.applied |= 1u << f;
+            }
       }
       for (uint32_t d = 0; d < D; ++d) {
         float sum = 0.0f;

@@ -210,12 +210,18 @@ int ko_attention_tile(uint32_t format, uint32_t kv_heads, uint32_t group, uint32
                       const uint32_t *row_masks, float score_scale);
 /* common/paged_attention_tile.h:362-417: merges one fused row. out_bf16 and
    out_f32 (either may be NULL) receive D values. */
-/* Test aids.  ko_attention_nudge: while fused_row >= 0, ko_attention_tile moves the rounded
-   weight (probability x value scale) of (fused_row, token) by `steps` places of its format and,
-   with only_row, computes that fused row alone; fused_row = -1 switches it off.  State is per
-   thread.  ko_attention_row_weights: softmax weight x value scale of every token a query row
-   sees (against the row's maximum over all pages), weights[committed + active_rows]. */
-void ko_attention_nudge(int64_t fused_row, uint32_t token, int steps, int only_row);
+/* Test aids.  ko_attention_flips: while fused_row >= 0, ko_attention_tile looks at the weight
+   (probability x value scale) of each listed token of that fused row before it rounds it to its
+   format (bf16; fp16 on fp8 pages); where the unrounded value lies within slack (relative) of the
+   boundary between two neighbours of the format it takes the neighbour on the other side, and
+   leaves the weight alone otherwise.  With only_row it computes that fused row alone;
+   fused_row = -1 switches everything off.  ko_attention_flips_applied: bit i set when token i was
+   turned since the last ko_attention_flips.  State is per thread.
+   ko_attention_row_weights: softmax weight x value scale of every token a query row sees (against
+   the row's maximum over all pages), weights[committed + active_rows]. */
+void ko_attention_flips(int64_t fused_row, const uint32_t *tokens, uint32_t count, float slack,
+                        int only_row);
+uint32_t ko_attention_flips_applied(void);
 void ko_attention_row_weights(uint32_t format, uint32_t kv_heads, uint32_t head_dim,
                               const uint16_t *query_row, const uint64_t *page_table, ko_kv_layer kv,
                               uint32_t kv_head, uint32_t committed, uint32_t active_rows,

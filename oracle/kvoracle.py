@@ -202,8 +202,10 @@ def _declare(L):
                                     u32, vp, vp, u64, vp, f32]
     L.ko_attention_reduce_row.argtypes = [u32, u32, u32, vp, vp, u32, u32, u32, u64, u32, vp, vp]
     L.ko_attention_reduce_row.restype = None
-    L.ko_attention_nudge.argtypes = [C.c_int64, u32, C.c_int, C.c_int]
-    L.ko_attention_nudge.restype = None
+    L.ko_attention_flips.argtypes = [C.c_int64, vp, u32, C.c_float, C.c_int]
+    L.ko_attention_flips.restype = None
+    L.ko_attention_flips_applied.argtypes = []
+    L.ko_attention_flips_applied.restype = u32
     L.ko_attention_row_weights.argtypes = [u32, u32, u32, vp, vp, KvLayer, u32, u32, u32, u32, vp,
                                            C.c_float, vp]
     L.ko_attention_row_weights.restype = None
@@ -412,37 +414,56 @@ def attention_tile_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv,
     return out, out32
 
 
-def rounding_flip_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv, head, committed,
-                       active, splits, capacity, fused_row, masks=None, score_scale=0.0, top=4):
-    """What one fused row of a tile would be had the rounding of one probability fallen the other
-    way: for each of the row's `top` heaviest tokens (softmax weight x value scale) and each
-    direction, the row recomputed with that token's rounded weight moved one place of its format
-    (bf16; fp16 on fp8 pages).  Yields (token, steps, bf16 row bits).
+# How far (relative) the unrounded weight of a token may lie from a rounding boundary for the
+# other rounding to count as explained.  The matrix-core kernels carry a constant of 128 + 8 per
+# int4 code (1024 + 128 per int8 code) through the fp32 accumulator of q.k, so a raw dot product
+# whose partial sums reach a few thousand is summed with an absolute error of up to 2^-11 or so;
+# times key scale and score scale (0.5 for keys with 20x outlier channels) that is a few 1e-4 in a
+# score, and the same, relative, in its probability.  A bf16 place is 3.9e-3 to 7.8e-3 relative,
+# so about one weight in ten lies this close to a boundary.
+FLIP_SLACK = 5e-4
 
-    A kernel that sums q.k in another order than this oracle can differ from it in the last bits
-    of a score, and so in the rounding of a probability that sits on a rounding boundary; when
-    that token carries most of the row, the whole row moves by up to half a place.  A row that is
-    farther from the oracle than the tolerance, but within it of one of these rows, is explained by
-    exactly that; any other difference is not."""
+
+def rounding_flip_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv, head, committed,
+                       active, splits, capacity, fused_row, masks=None, score_scale=0.0, top=6,
+                       slack=FLIP_SLACK):
+    """What one fused row of a tile would be had the rounding of some of its heaviest
+    probabilities fallen the other way.  Of the row's `top` heaviest tokens (softmax weight x
+    value scale) only those count whose unrounded weight lies within `slack` (relative) of a
+    rounding boundary of its format (bf16; fp16 on fp8 pages): for every non-empty set of them
+    the oracle recomputes the row with those weights on the other side of their boundaries.
+    Yields (tokens, len(tokens), bf16 row bits).
+
+    A kernel that sums q.k in another order than this oracle differs from it in the last bits of
+    a score, and so in the rounding of a probability that sits on a rounding boundary; a token
+    that carries much of the row then moves the whole row by up to half a place.  A row that is
+    farther from the oracle than the tolerance, but within it of one of these rows, is explained
+    by exactly that; any other difference is not."""
+    import itertools
     L = lib()
     M, D = capacity * group, head_dim
     tile_queries = np.ascontiguousarray(tile_queries, dtype=np.uint16).reshape(M, D)
     row = fused_row // group
-    visible = committed + active
-    weights = np.zeros(visible, dtype=np.float32)
+    weights = np.zeros(committed + active, dtype=np.float32)
     mask_ptr = ptr(np.ascontiguousarray(masks, dtype=np.uint32)) if masks is not None else None
     L.ko_attention_row_weights(fmt, kv_heads, D, ptr(tile_queries[fused_row]), ptr(table), kv, head,
                                committed, active, row, mask_ptr, score_scale, ptr(weights))
-    heaviest = np.argsort(-weights, kind="stable")[:top]
-    try:
-        for token in heaviest:
-            if weights[token] <= 0:
-                continue
-            for steps in (1, -1):
-                L.ko_attention_nudge(fused_row, int(token), steps, 1)
-                bits, _ = attention_tile_rows(fmt, kv_heads, group, D, tile_queries, table, kv, head,
-                                              committed, active, splits, capacity, masks, score_scale,
-                                              only_row=fused_row)
-                yield int(token), steps, bits[fused_row]
-    finally:
-        L.ko_attention_nudge(-1, 0, 0, 0)
+    heaviest = [int(t) for t in np.argsort(-weights, kind="stable")[:top] if weights[t] > 0]
+
+    def recompute(tokens):
+        arr = np.array(tokens, dtype=np.uint32)
+        L.ko_attention_flips(fused_row, ptr(arr), len(arr), slack, 1)
+        try:
+            bits, _ = attention_tile_rows(fmt, kv_heads, group, D, tile_queries, table, kv, head,
+                                          committed, active, splits, capacity, masks, score_scale,
+                                          only_row=fused_row)
+            return bits[fused_row], L.ko_attention_flips_applied()
+        finally:
+            L.ko_attention_flips(-1, None, 0, 0.0, 0)
+
+    _, applied = recompute(heaviest)          # which of them sit on a boundary at all
+    near = [t for i, t in enumerate(heaviest) if applied >> i & 1]
+    for size in range(1, len(near) + 1):
+        for tokens in itertools.combinations(near, size):
+            bits, _ = recompute(list(tokens))
+            yield tokens, size, bits

@@ -1775,6 +1775,57 @@ int kv_attend_decode(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
                         row_stride, workspace, static_cast<hipStream_t>(stream));
 }
 
+// ---- decode attention without a caller's workspace ------------------------------
+// The split kernels' partial rows and statistics live in this array instead: device
+// memory of the library's code object, one copy per GPU, held until the process ends.
+// In host code the array's name is only a stand-in for the symbol; its address on a
+// device comes from hipGetSymbolAddress, asked once per device with that device current,
+// and that pointer is what every launch is given.
+constexpr uint64_t kStaticScratchBytes = KVX_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char kvx_static_scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void *g_static_scratch[kMaxDevices] = {};  // the array's address on each device, once known
+
+// The address of the scratch array on the current device, which must be the storage's.
+int static_scratch(const kvx_storage *s, void **out) {
+  int device = -1;
+  KVX_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) return fail(KVX_EDEVICE, "device index out of range");
+  if (device != s->device)
+    return fail(KVX_ESTATE, "the storage's device is not the current device");
+  if (!g_static_scratch[device]) {
+    void *address = nullptr;
+    KVX_HIP(hipGetSymbolAddress(&address, HIP_SYMBOL(kvx_static_scratch)));
+    if (!address) return fail(KVX_EDEVICE, "the static workspace has no address on this device");
+    g_static_scratch[device] = address;
+  }
+  *out = g_static_scratch[device];
+  return KVX_OK;
+}
+}  // namespace
+
+int kv_attend_decode_static(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
+                            const void *queries, void *output, const uint64_t *const *page_tables,
+                            const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                            void *stream) {
+  if (!s || !lanes || !n_lanes) return fail(KVX_EINVAL, "kv_attend_decode_static: null argument or no lanes");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
+  const uint64_t needed = kvx_attend_workspace_bytes(lanes, n_lanes, query_heads, &s->layout);
+  if (needed > kStaticScratchBytes)
+    return fail(KVX_EINVAL, "kv_attend_decode_static: the lanes' partial rows need " +
+                                std::to_string(needed) + " bytes, the static workspace holds " +
+                                std::to_string(kStaticScratchBytes) +
+                                "; use kv_attend_decode with a workspace of the caller's");
+  void *scratch = nullptr;
+  if (const int rc = static_scratch(s, &scratch)) return rc;
+  // Every partial row and statistic a merge reads is written by the split kernel of the
+  // same call first, so nothing of the previous call's contents has to be cleared.
+  return kv_attend_decode(s, layer, query_heads, queries, output, page_tables, lanes, n_lanes,
+                          row_stride, scratch, kStaticScratchBytes, stream);
+}
+
 int kv_append_attend_decode(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
                             const void *chunk_values, uint64_t chunk_lane_stride,
                             uint32_t chunk_stride, uint32_t query_heads, const void *queries,

@@ -35,7 +35,7 @@ SYMBOLS = [
     "kvx_pool_acquire", "kvx_pool_retain", "kvx_pool_release", "kvx_pool_page_active",
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
     "kvx_pool_snapshot_get", "kv_append", "kv_prepare_append", "kv_attend_decode_shared", "kvx_attend_shared_workspace_bytes", "kv_attend_verify", "kv_attend_verify_hidden", "kv_attend_decode",
-    "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kv_page_export", "kv_page_import", "kv_attend_split", "kv_attend_merge",
+    "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kv_page_export", "kv_page_import", "kv_attend_split", "kv_attend_merge", "kv_attend_decode_static",
     "kvx_debug_attend_paths", "kvx_decode_plan", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
     "kvx_prefix_chain", "kvx_prefix_retain_active", "kvx_prefix_release_active",
@@ -233,6 +233,7 @@ def _declare(L):
     L.kv_attend_verify_hidden.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, vp, u32, vp, u64, vp, vp,
                                           vp]
     L.kv_attend_decode.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, u32, vp, u64, vp]
+    L.kv_attend_decode_static.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, u32, vp]
     L.kv_attend_split.argtypes = [vp, u32, u32, vp, vp, vp, u32, vp, u32, vp, u64, vp]
     L.kv_attend_merge.argtypes = [vp, u32, vp, vp, u32, u32, vp, u64, vp]
     L.kv_attend_decode_shared.argtypes = [vp, u32, u32, vp, vp, vp, vp, u32, u32, u32, u32, vp, u64, vp]
@@ -432,6 +433,15 @@ def attend_decode(storage, layer, query_heads, queries, output, tables, lanes, r
                                         _ptr(workspace),
                                         workspace.numel() * workspace.element_size(),
                                         _stream(stream)))
+
+
+def attend_decode_static(storage, layer, query_heads, queries, output, tables, lanes, row_stride,
+                         stream=None):
+    """kv_attend_decode over the library's static workspace (kv_attend_decode_static)."""
+    arr = (VerifyParams * len(lanes))(*lanes)
+    return check(lib().kv_attend_decode_static(storage.h, layer, query_heads, _ptr(queries),
+                                               _ptr(output), _table_array(tables), arr, len(lanes),
+                                               row_stride, _stream(stream)))
 
 
 def attend_shared_workspace_bytes(storage, lanes, prefix_splits, query_heads):

@@ -22,12 +22,12 @@ FMT = ko.INT4
 def one_row(fmt, tile_queries, table, kv, head, committed, active, splits, capacity, fused_row):
     """One fused row of a tile by the oracle, the other rows skipped."""
     L = ko.lib()
-    L.ko_attention_nudge(fused_row, 0, 0, 1)
+    L.ko_attention_flips(fused_row, None, 0, 0.0, 1)   # no flips: that fused row alone
     try:
         bits, f32 = ko.attention_tile_rows(fmt, H, G, D, tile_queries, table, kv, head, committed,
                                            active, splits, capacity, only_row=fused_row)
     finally:
-        L.ko_attention_nudge(-1, 0, 0, 0)
+        L.ko_attention_flips(-1, None, 0, 0.0, 0)
     return bits[fused_row], f32[fused_row]
 
 

@@ -340,3 +340,38 @@ def test_merge_against_fp64_reference_pattern(splits, active):
         want = (w[:, None] * part[:, row]).sum(0) / (w * sm[:, row]).sum()
         got = ko.bf16_to_f32(ob).astype(np.float64)
         assert np.all(np.abs(got - want) <= np.abs(want) * 0.004 + 2e-6)
+
+
+@pytest.mark.parametrize("fmt", [ko.INT4, ko.FP8])
+def test_rounding_flips_turn_only_weights_on_a_boundary(fmt):
+    """The GPU checks' allowance machinery (ko.rounding_flip_rows): with no slack nothing is
+    turned; with a slack of a whole place every one of the heaviest tokens is, one at a time
+    and together; a turned rounding moves the row by that token's share of a place, no more;
+    and the untouched call still gives the plain tile."""
+    committed, active, capacity, splits, head = 300, 8, 8, 3, 2
+    store, pages, table = build_history(fmt, committed, active, seed=77)
+    q = random_queries(capacity, 32, 78)
+    tile_q = q[head, :capacity].reshape(capacity * G, D)
+    kv = store.layer(1)
+    base, base32 = ko.attention_tile_rows(fmt, H, G, D, tile_q, table, kv, head, committed, active,
+                                          splits, capacity)
+    fused_row = 3 * G + 1
+    args = (fmt, H, G, D, tile_q, table, kv, head, committed, active, splits, capacity, fused_row)
+    assert list(ko.rounding_flip_rows(*args, slack=0.0)) == []
+    rows = list(ko.rounding_flip_rows(*args, top=3, slack=1.0))
+    assert len(rows) == 7 and sorted(size for _, size, _ in rows) == [1, 1, 1, 2, 2, 2, 3]
+    value = lambda bits: ko.bf16_to_f32(bits).astype(np.float64)
+    for tokens, size, bits in rows:
+        moved = np.linalg.norm(value(bits) - value(base[fused_row])) / np.linalg.norm(value(base[fused_row]))
+        # one place of the weight's format, times at most the whole row
+        assert 0 < moved <= size * (2.0 ** -7 if fmt != ko.FP8 else 2.0 ** -9) + 2e-3
+    # at the real slack a minority of the weights is that close to a boundary (about a quarter:
+    # the window is 1e-3 wide, a place 3.9e-3 to 7.8e-3); at a hundredth of it hardly any
+    def near(slack):
+        return sum(sum(1 for _, size, _ in ko.rounding_flip_rows(*args[:-1], r, top=6, slack=slack)
+                       if size == 1) for r in range(0, 8 * G, 2))
+    assert near(ko.FLIP_SLACK) <= 6 * 4 * G * 0.4 and near(ko.FLIP_SLACK / 100) <= 2
+    again, _ = ko.attention_tile_rows(fmt, H, G, D, tile_q, table, kv, head, committed, active,
+                                      splits, capacity)
+    assert np.array_equal(again, base)
+    store.close()

@@ -131,27 +131,37 @@ def test_shared_prefix_decode_matches_oracle(fmt, shared_pages, own_tokens, pref
 
 
 def flipped_rows(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_splits, own_splits,
-                 committed, index, layer=1, top=4):
+                 committed, index, layer=1, top=6):
     """For check_attention's allowance: output row (lane, head, head in group) in the shared
-    arrangement with the rounded weight of one of its heaviest tokens moved one place, the token
-    being in the prefix tile or in the sequence's own."""
+    arrangement with the roundings turned of those of its heaviest tokens whose weights sit on a
+    rounding boundary (ko.rounding_flip_rows says how close), the tokens being in the prefix tile
+    or in the sequence's own."""
+    import itertools
     lane, head, g = index
     weights = np.zeros(committed[lane] + 1, dtype=np.float32)
     ko.lib().ko_attention_row_weights(fmt, H, D, ko.ptr(np.ascontiguousarray(q[lane, head, 0, g])),
                                       ko.ptr(hts[lane]), tw.host.layer(layer), head, committed[lane], 1,
                                       0, None, 0.0, ko.ptr(weights))
-    for token in np.argsort(-weights, kind="stable")[:top]:
-        for steps in (1, -1):
-            bits, _ = oracle_shared(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_splits,
-                                    own_splits, layer, only=index, nudge=(int(token), steps))
-            yield int(token), steps, bits[lane, head, g]
+    heaviest = [int(t) for t in np.argsort(-weights, kind="stable")[:top]]
+
+    def recompute(tokens):
+        return oracle_shared(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_splits,
+                             own_splits, layer, only=index, flips=tokens)
+
+    _, _, applied = recompute(heaviest)
+    near = [t for t in heaviest if t in applied]
+    for size in range(1, len(near) + 1):
+        for tokens in itertools.combinations(near, size):
+            bits, _, _ = recompute(list(tokens))
+            yield tokens, size, bits[lane, head, g]
 
 
 def oracle_shared(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_splits, own_splits, layer=1,
-                  only=None, nudge=None):
+                  only=None, flips=None):
     """The oracle's tiles in the shared arrangement, merged in the library's order.  only =
-    (lane, head, head in group): that output row alone; nudge = (token of the sequence, steps):
-    with the rounded weight of that token moved (see ko_attention_nudge)."""
+    (lane, head, head in group): that output row alone; flips = tokens of that sequence whose
+    roundings are turned where they sit on a boundary (ko_attention_flips), in which case the
+    tokens that were turned are returned as a third value."""
     L = ko.lib()
     lanes = len(own_tokens)
     kv = tw.host.layer(layer)
@@ -168,29 +178,33 @@ def oracle_shared(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_spl
         statistics = np.zeros((splits, M, 2), dtype=np.float32)
         tile_q = np.ascontiguousarray(queries, dtype=np.uint16).reshape(M, D)
         if moved:
-            L.ko_attention_nudge(moved[0], moved[1], moved[2], 1)
+            arr = np.array(moved[1], dtype=np.uint32)
+            L.ko_attention_flips(moved[0], ko.ptr(arr) if len(arr) else None, len(arr), ko.FLIP_SLACK, 1)
         try:
             for split in range(splits):
                 L.ko_attention_tile(fmt, H, G, D, capacity, ko.ptr(tile_q), ko.ptr(table), kv, head,
                                     committed, active, splits, split, ko.ptr(partials),
                                     ko.ptr(statistics), split,
                                     ko.ptr(masks) if masks is not None else None, 0.0)
+            if moved:
+                mask = L.ko_attention_flips_applied()
+                turned.update(moved[2] + t for i, t in enumerate(moved[1]) if mask >> i & 1)
         finally:
-            L.ko_attention_nudge(-1, 0, 0, 0)
+            L.ko_attention_flips(-1, None, 0, 0.0, 0)
         return partials, statistics
 
     out = np.zeros((lanes, H, G, D), dtype=np.float32)
+    turned = set()
     zero_masks = np.zeros(lanes, dtype=np.uint32)
     shared_tokens = shared_pages * 32
     for head in range(H) if only is None else [only[1]]:
         # a moved weight sits in one of the two tiles; with `only`, each tile computes one row
+        # (fused row, tokens of the tile, what to add to name them as tokens of the sequence)
         in_prefix = in_own = None
         if only is not None:
-            in_prefix, in_own = (only[0] * G + only[2], 0, 0), (only[2], 0, 0)
-            if nudge and nudge[0] < shared_tokens:
-                in_prefix = (only[0] * G + only[2], nudge[0], nudge[1])
-            elif nudge:
-                in_own = (only[2], nudge[0] - shared_tokens, nudge[1])
+            mine = flips or []
+            in_prefix = (only[0] * G + only[2], [t for t in mine if t < shared_tokens], 0)
+            in_own = (only[2], [t - shared_tokens for t in mine if t >= shared_tokens], shared_tokens)
         pp, ps = tiles(q[:, head, 0], hts[0], shared_tokens, lanes, lanes, prefix_splits, zero_masks, head,
                        in_prefix)
         pw = written(shared_tokens + lanes, prefix_splits)
@@ -208,6 +222,8 @@ def oracle_shared(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_spl
                     numerator = numerator + weight * part
                     denominator = f32(denominator + weight * f32(st[1]))
                 out[i, head, g] = numerator / denominator
+    if flips is not None:
+        return ko.f32_to_bf16(out).reshape(out.shape), out, turned
     return ko.f32_to_bf16(out).reshape(out.shape), out
 
 
