@@ -424,15 +424,26 @@ def attention_tile_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv,
 FLIP_SLACK = 5e-4
 
 
+def flip_slack(fmt):
+    """FLIP_SLACK in terms of the weights' format: an eighth to a sixteenth of a bf16 place, and
+    the same part of an fp16 place (8 times finer) on fp8 pages, whose weights are fp16."""
+    return FLIP_SLACK / 8 if fmt == FP8 else FLIP_SLACK
+
+
 def rounding_flip_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv, head, committed,
-                       active, splits, capacity, fused_row, masks=None, score_scale=0.0, top=6,
-                       slack=FLIP_SLACK):
+                       active, splits, capacity, fused_row, masks=None, score_scale=0.0, top=32,
+                       slack=None, together=2):
     """What one fused row of a tile would be had the rounding of some of its heaviest
     probabilities fallen the other way.  Of the row's `top` heaviest tokens (softmax weight x
     value scale) only those count whose unrounded weight lies within `slack` (relative) of a
-    rounding boundary of its format (bf16; fp16 on fp8 pages): for every non-empty set of them
-    the oracle recomputes the row with those weights on the other side of their boundaries.
-    Yields (tokens, len(tokens), bf16 row bits).
+    rounding boundary of its format (bf16; fp16 on fp8 pages): for every set of at most
+    `together` of them the oracle recomputes the row with those weights on the other side of
+    their boundaries.  Yields (tokens, len(tokens), bf16 row bits).
+
+    How much one turned rounding moves a row: a place of a weight in [0.25, 0.5) is 2^-9, and
+    the row is a sum of value rows with weights w, so it moves by about 2^-9 / sqrt(sum w^2) --
+    1e-3 to 3e-3 when the attention is spread over some ten heavy tokens, each of which can be
+    the one.  Hence `top` reaches well past the few heaviest.
 
     A kernel that sums q.k in another order than this oracle differs from it in the last bits of
     a score, and so in the rounding of a probability that sits on a rounding boundary; a token
@@ -441,6 +452,8 @@ def rounding_flip_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv, 
     by exactly that; any other difference is not."""
     import itertools
     L = lib()
+    if slack is None:
+        slack = flip_slack(fmt)
     M, D = capacity * group, head_dim
     tile_queries = np.ascontiguousarray(tile_queries, dtype=np.uint16).reshape(M, D)
     row = fused_row // group
@@ -463,7 +476,7 @@ def rounding_flip_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv, 
 
     _, applied = recompute(heaviest)          # which of them sit on a boundary at all
     near = [t for i, t in enumerate(heaviest) if applied >> i & 1]
-    for size in range(1, len(near) + 1):
+    for size in range(1, min(together, len(near)) + 1):
         for tokens in itertools.combinations(near, size):
             bits, _ = recompute(list(tokens))
             yield tokens, size, bits

@@ -37,11 +37,29 @@ __device__ __forceinline__ T load_global(const void *p) {
   return *reinterpret_cast<const KVX_GLOBAL T *>(reinterpret_cast<uintptr_t>(p));
 }
 
+// A page-table entry through the scalar unit: the table pointer and the slot are the
+// same in every lane, and a table is not written while a launch reads it, so the entry
+// can come through the constant path (s_load) into scalar registers.  A vector load
+// would return in order behind every page load in flight, and the wait for it would
+// drain them; a scalar load waits on its own counter.
+__device__ __forceinline__ uint64_t scalar_entry(const uint64_t *table, uint32_t slot) {
+  typedef __attribute__((address_space(4))) const uint64_t ConstantEntry;
+  return *reinterpret_cast<ConstantEntry *>(reinterpret_cast<uintptr_t>(table + slot));
+}
+
+// Stores through pointers rebuilt from page entries, as global memory.  A flat
+// store would do, but while one is pending the compiler has to assume that memory
+// operations complete out of order, and every wait for a page load after it, the
+// ones in the page loop included, becomes a wait for all loads in flight.
+template <class T>
+__device__ __forceinline__ void store_global(void *p, T value) {
+  *reinterpret_cast<KVX_GLOBAL T *>(reinterpret_cast<uintptr_t>(p)) = value;
+}
+
 constexpr uint32_t kPage = KVX_PAGE_TOKENS;
 constexpr uint32_t kLanes = KVX_LANES_PER_LAUNCH;
 constexpr uint32_t kD = 256;
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr uint32_t kTableSlots = 1024;  // page entries of one split staged in LDS
 
 struct DecodeLane {
   const uint64_t *table;
@@ -428,8 +446,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
 
 // The shapes every matrix-core kernel of this library covers: head dimension
 // 256, a group of at most 16 query heads, at most KVX_TREE_NODES rows per lane,
-// every lane with the row capacity of the first, splits of at most kTableSlots
-// pages.
+// every lane with the row capacity of the first.
 inline bool matrix_attention_covers(const kvx_storage *s, uint32_t query_heads,
                                     const kvx_verify_params *lanes, uint32_t n_lanes) {
   const kvx_layout &l = s->layout;
@@ -439,9 +456,6 @@ inline bool matrix_attention_covers(const kvx_storage *s, uint32_t query_heads,
   for (uint32_t i = 0; i < n_lanes; ++i) {
     const kvx_verify_params &p = lanes[i];
     if (p.row_capacity != capacity || !p.active_rows || p.active_rows > capacity) return false;
-    const uint32_t pages = (p.committed_tokens + p.active_rows + kPage - 1) / kPage;
-    const uint32_t splits = std::max(1u, p.split_count);
-    if ((pages + splits - 1) / splits > kTableSlots) return false;
   }
   return true;
 }

@@ -232,7 +232,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
   // live row carry zeros.
   const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
   __shared__ u32x4 q_lds[NB][8][64];
-  __shared__ uint64_t table_lds[kTableSlots];
 #pragma unroll
   for (uint32_t nb = 0; nb < NB; ++nb) {
     const uint16_t *q_row = q_head + uint64_t(live_row[nb] ? m[nb] : 0) * kD;
@@ -251,11 +250,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
       q_lds[nb][kb][lane] = q;
     }
   }
-  // The split's page entries (at most kTableSlots; the launcher declines longer
-  // splits) go through LDS and are read back with uniform LDS loads.
-  for (uint32_t i = lane; i < end - begin; i += 64)
-    table_lds[i] = load_global<uint64_t>(l.table + begin + i);
-  __syncthreads();
+  __syncthreads();  // the staged queries
+  // The split's page entries come through the scalar unit, each set's next entry
+  // fetched a whole page period before the refill that uses it.
+  const uint64_t *const entries = l.table + begin;
+  const uint32_t last_slot = end - begin - 1;
 
   // kSets register sets rotate: a set's keys are refilled with the page kSets
   // ahead as soon as the page has multiplied its last key, its values when the
@@ -275,8 +274,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
   };
   PageSet set[kSets];
   // The empty asm statements keep the loads of one fetch together and in place.
-  auto fetch_keys = [&](PageSet &r, uint32_t slot) {
-    const PagePlace p = place_page<FMT>(table_lds[slot], head, H, a.kv.offset, ro);
+  auto fetch_keys = [&](PageSet &r, uint64_t entry) {
+    const PagePlace p = place_page<FMT>(entry, head, H, a.kv.offset, ro);
     asm volatile("");
     load_keys<FMT, REUSED>(r.keys, p, t, g);
     if constexpr (kByte) {
@@ -285,8 +284,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
     }
     asm volatile("");
   };
-  auto fetch_values = [&](PageSet &r, uint32_t slot) {
-    const PagePlace p = place_page<FMT>(table_lds[slot], head, H, a.kv.offset, ro);
+  auto fetch_values = [&](PageSet &r, uint64_t entry) {
+    const PagePlace p = place_page<FMT>(entry, head, H, a.kv.offset, ro);
     asm volatile("");
     load_values<FMT, REUSED>(r.values, p, t, g);
     if constexpr (kByte) {
@@ -298,10 +297,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
   // The first fills are unconditional (a split shorter than kSets pages loads its
   // last page again), so the steady loop is entered with the loads in flight that
   // its own iterations leave behind.
+  uint64_t upcoming[kSets];  // upcoming[d]: the entry of set d's next refill
+#pragma unroll
+  for (uint32_t d = 0; d < kSets; ++d) upcoming[d] = scalar_entry(entries, min(d, last_slot));
 #pragma unroll
   for (uint32_t d = 0; d < kSets; ++d) {
-    fetch_keys(set[d], min(d, end - begin - 1));
-    fetch_values(set[d], min(d, end - begin - 1));
+    fetch_keys(set[d], upcoming[d]);
+    fetch_values(set[d], upcoming[d]);
+    upcoming[d] = scalar_entry(entries, min(d + kSets, last_slot));
   }
 
   f32x4 acc[NB][16];  // [block][dim block]: dims 16*mb + 4g + r of column t
@@ -413,9 +416,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
   for (; page + 2 * kSets <= end; page += kSets) {
 #pragma unroll
     for (uint32_t d = 0; d < kSets; ++d) {
-      const uint32_t refill = page + d + kSets - begin;
-      attend_page(set[d], page + d, [&] { fetch_keys(set[d], refill); });
-      fetch_values(set[d], refill);
+      // upcoming[d] is the entry of slot page + d + kSets - begin, this set's refill
+      attend_page(set[d], page + d, [&] { fetch_keys(set[d], upcoming[d]); });
+      fetch_values(set[d], upcoming[d]);
+      upcoming[d] = scalar_entry(entries, min(page + d + 2 * kSets - begin, last_slot));
     }
   }
   // Tail: at most 2 kSets - 1 pages are left, the first kSets of them loaded.
@@ -425,8 +429,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
     if (page + k < end) {
       attend_page(set[d], page + k, [] {});
       if (k + kSets < 2 * kSets - 1 && page + k + kSets < end) {
-        fetch_keys(set[d], page + k + kSets - begin);
-        fetch_values(set[d], page + k + kSets - begin);
+        fetch_keys(set[d], upcoming[d]);  // slot page + k + kSets - begin, and d = k here
+        fetch_values(set[d], upcoming[d]);
+        upcoming[d] = scalar_entry(entries, min(page + k + 2 * kSets - begin, last_slot));
       }
     }
   }

@@ -326,12 +326,15 @@ __device__ __forceinline__ void append_decode_token(const DecodeArgs &a, const D
       packed |= (uint32_t(code) & 0xfu) << (4 * i);
     }
     uint8_t *data = tensor ? slab.values : slab.keys;
-    *reinterpret_cast<uint16_t *>(data + slot * kRowBytes + 2 * lane) = uint16_t(packed);
+    store_global<uint16_t>(data + slot * kRowBytes + 2 * lane, uint16_t(packed));
     if (lane == 0)
-      (tensor ? slab.value_scales : slab.key_scales)[slot] =
-          maximum == 0.0f ? 0.0f : __fdiv_rn(maximum, 7.0f);
+      store_global<float>((tensor ? slab.value_scales : slab.key_scales) + slot,
+                          maximum == 0.0f ? 0.0f : __fdiv_rn(maximum, 7.0f));
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // The stores are complete before the page is loaded: vmcnt(0), with the other
+  // counters left alone.  The builtin, so that the compiler's own count of what is
+  // in flight sees the wait.
+  __builtin_amdgcn_s_waitcnt(0x0F70);
 }
 
 // Register sets of pages per wave: two rotate in the one-block decode kernel
@@ -466,45 +469,46 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
       q_raw[nb][kb] = load_global<u32x4>(q_row + 8 * (16 * (kb >> 2) + 4 * g + (kb & 3)));
   }
 
-  // The split's page entries (at most kTableSlots; the launcher declines longer
-  // splits) go through LDS and are read back with uniform LDS loads.  (Fetched
-  // from memory one by one they would be vector loads in the steady loop, and
-  // since loads return in order the wait for an entry would drain every page
-  // load in flight.)
-  __shared__ uint64_t table_lds[kTableSlots];
-  for (uint32_t i = lane; i < end - begin; i += 64)
-    table_lds[i] = load_global<uint64_t>(l.table + begin + i);
-  __syncthreads();
+  // The split's page entries come through the scalar unit, each set's next entry
+  // fetched a whole page period before the refill that uses it.
   // kDepth register sets rotate: a set is refilled with the page kDepth ahead as
   // soon as its page has been consumed, so up to kDepth pages are in flight.
   PageRegs r[kDepth];
+  const uint64_t *const entries = l.table + begin;
+  const uint32_t last_slot = end - begin - 1;
+  uint64_t upcoming[kDepth];  // upcoming[d]: the entry of set d's next refill
   const LaneOffsets at = lane_offsets(t, g, uint32_t(ro.value_scales - ro.key_scales));
-  auto fill = [&](PageRegs &set, uint32_t slot) {
-    // The empty asm statements pin the loads of one fill together and in place:
-    // moved up into the arithmetic that still reads the set they would need a
-    // second copy of its registers, and interleaved with another fill's loads
-    // they would make every wait cover both.
+  // The empty asm statements pin the loads of one fill together and in place:
+  // moved up into the arithmetic that still reads the set they would need a
+  // second copy of its registers, and interleaved with another fill's loads
+  // they would make every wait cover both.
+  auto fill = [&](PageRegs &set, uint64_t entry) {
     asm volatile("");
-    load_page<3, kReused>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
+    load_page<3, kReused>(set, entry, head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
   // The same in two steps for the steady loop: the keys as soon as the page that
   // held the set has multiplied its last key, the rest when the page is done.
-  auto fill_keys = [&](PageRegs &set, uint32_t slot) {
+  auto fill_keys = [&](PageRegs &set, uint64_t entry) {
     asm volatile("");
-    load_page<1, kReused>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
+    load_page<1, kReused>(set, entry, head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
-  auto fill_rest = [&](PageRegs &set, uint32_t slot) {
+  auto fill_rest = [&](PageRegs &set, uint64_t entry) {
     asm volatile("");
-    load_page<2, kReused>(set, table_lds[slot], head, H, a.kv.offset, ro.key_scales, ro.values, at);
+    load_page<2, kReused>(set, entry, head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
   // The first fills are unconditional too (a split shorter than kDepth pages
   // loads its last page again): the steady loop must be entered with the same
   // loads in flight, in the same order, as its own iterations leave behind.
 #pragma unroll
-  for (uint32_t d = 0; d < kDepth; ++d) fill(r[d], min(d, end - begin - 1));
+  for (uint32_t d = 0; d < kDepth; ++d) upcoming[d] = scalar_entry(entries, min(d, last_slot));
+#pragma unroll
+  for (uint32_t d = 0; d < kDepth; ++d) {
+    fill(r[d], upcoming[d]);
+    upcoming[d] = scalar_entry(entries, min(d + kDepth, last_slot));
+  }
   if (appends && !appends_first) append_decode_token(a, l, li, head, lane);
 
   // Register kb of the staged queries holds the 8 dims of dword
@@ -560,10 +564,11 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   for (; page + kUnmaskedStop <= end; page += kDepth) {
 #pragma unroll
     for (uint32_t d = 0; d < kDepth; ++d) {
-      const uint32_t refill = page + d + kDepth - begin;
+      // upcoming[d] is the entry of slot page + d + kDepth - begin, this set's refill
       attend_page<false, NB>(r[d], staged_queries, q_bias, score_scale, (page + d) * kPage, sight, lane, g,
-                             st, [&] { fill_keys(r[d], refill); });
-      fill_rest(r[d], refill);
+                             st, [&] { fill_keys(r[d], upcoming[d]); });
+      fill_rest(r[d], upcoming[d]);
+      upcoming[d] = scalar_entry(entries, min(page + d + 2 * kDepth - begin, last_slot));
     }
   }
   // Tail: at most kUnmaskedStop - 1 pages are left, the first kDepth of them loaded.
@@ -573,8 +578,10 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     if (page + k < end) {
       attend_page<true, NB>(r[d], staged_queries, q_bias, score_scale, (page + k) * kPage, sight, lane, g,
                             st, [] {});
-      if (k + kDepth < kUnmaskedStop - 1 && page + k + kDepth < end)
-        fill(r[d], page + k + kDepth - begin);
+      if (k + kDepth < kUnmaskedStop - 1 && page + k + kDepth < end) {
+        fill(r[d], upcoming[d]);  // slot page + k + kDepth - begin, and d = k here
+        upcoming[d] = scalar_entry(entries, min(page + k + 2 * kDepth - begin, last_slot));
+      }
     }
   }
 

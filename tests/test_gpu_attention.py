@@ -488,7 +488,7 @@ def test_append_attend_decode_is_the_two_calls(fmt):
     v = rng.standard_normal((lanes, H, 1, D)).astype(np.float32)
     k[:, :, :, [3, 77]] *= 20
     k[2, 1] = 0  # a zero row: scale 0, codes 0
-    v[5, 3] *= 1e-20
+    v[5, H - 1] *= 1e-20
     ck = np.zeros((lanes, H, 32, D), dtype=np.uint16)
     cv = np.zeros((lanes, H, D, 32), dtype=np.uint16)
     for lane in range(lanes):

@@ -358,7 +358,7 @@ def test_rounding_flips_turn_only_weights_on_a_boundary(fmt):
     fused_row = 3 * G + 1
     args = (fmt, H, G, D, tile_q, table, kv, head, committed, active, splits, capacity, fused_row)
     assert list(ko.rounding_flip_rows(*args, slack=0.0)) == []
-    rows = list(ko.rounding_flip_rows(*args, top=3, slack=1.0))
+    rows = list(ko.rounding_flip_rows(*args, top=3, slack=1.0, together=3))
     assert len(rows) == 7 and sorted(size for _, size, _ in rows) == [1, 1, 1, 2, 2, 2, 3]
     value = lambda bits: ko.bf16_to_f32(bits).astype(np.float64)
     for tokens, size, bits in rows:
@@ -370,7 +370,7 @@ def test_rounding_flips_turn_only_weights_on_a_boundary(fmt):
     def near(slack):
         return sum(sum(1 for _, size, _ in ko.rounding_flip_rows(*args[:-1], r, top=6, slack=slack)
                        if size == 1) for r in range(0, 8 * G, 2))
-    assert near(ko.FLIP_SLACK) <= 6 * 4 * G * 0.4 and near(ko.FLIP_SLACK / 100) <= 2
+    assert near(ko.flip_slack(fmt)) <= 6 * 4 * G * 0.4 and near(ko.flip_slack(fmt) / 100) <= 2
     again, _ = ko.attention_tile_rows(fmt, H, G, D, tile_q, table, kv, head, committed, active,
                                       splits, capacity)
     assert np.array_equal(again, base)

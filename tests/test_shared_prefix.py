@@ -131,7 +131,7 @@ def test_shared_prefix_decode_matches_oracle(fmt, shared_pages, own_tokens, pref
 
 
 def flipped_rows(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_splits, own_splits,
-                 committed, index, layer=1, top=6):
+                 committed, index, layer=1, top=32, together=2):
     """For check_attention's allowance: output row (lane, head, head in group) in the shared
     arrangement with the roundings turned of those of its heaviest tokens whose weights sit on a
     rounding boundary (ko.rounding_flip_rows says how close), the tokens being in the prefix tile
@@ -150,7 +150,7 @@ def flipped_rows(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_spli
 
     _, _, applied = recompute(heaviest)
     near = [t for t in heaviest if t in applied]
-    for size in range(1, len(near) + 1):
+    for size in range(1, min(together, len(near)) + 1):
         for tokens in itertools.combinations(near, size):
             bits, _, _ = recompute(list(tokens))
             yield tokens, size, bits[lane, head, g]
@@ -179,7 +179,7 @@ def oracle_shared(fmt, tw, hts, entries, q, shared_pages, own_tokens, prefix_spl
         tile_q = np.ascontiguousarray(queries, dtype=np.uint16).reshape(M, D)
         if moved:
             arr = np.array(moved[1], dtype=np.uint32)
-            L.ko_attention_flips(moved[0], ko.ptr(arr) if len(arr) else None, len(arr), ko.FLIP_SLACK, 1)
+            L.ko_attention_flips(moved[0], ko.ptr(arr) if len(arr) else None, len(arr), ko.flip_slack(fmt), 1)
         try:
             for split in range(splits):
                 L.ko_attention_tile(fmt, H, G, D, capacity, ko.ptr(tile_q), ko.ptr(table), kv, head,
