@@ -12,15 +12,20 @@
 // maximum moves once per 32-token page, and probability x value scale is
 // rounded to bf16 before it meets the value codes.
 //
-// Nibble -> bf16 without a table: OR-ing a 4-bit field into the mantissa of
-// 0x4300 gives 128 + field exactly.  With the stored two's-complement code c,
-// field = (c & 15) ^ 8 = c + 8 gives 136 + c and field = (c & 15) ^ 7 = 7 - c
-// gives 135 - c.  Even positions use the first form, odd positions the second
-// with the other operand negated, so the products are q.c + 136 q and
-// q.c - 135 q: the constant parts largely cancel pairwise and what is left is
-// tracked in fp32 and subtracted (keys: once per q row; values: per page,
-// rescaled with the accumulator).  Positions are dimensions for q.k and tokens
-// for p.v.
+// Nibble -> bf16 without a table: a 4-bit field OR-ed into the mantissa of a
+// power of two 2^e, at the place whose weight is 1, gives 2^e + field exactly:
+// 0x4300 | field = 128 + field, 0x4180 | field << 3 = 16 + field.  With the stored
+// two's-complement code c, field = (c & 15) ^ 8 = c + 8 and field = (c & 15) ^ 7 =
+// 7 - c.  Even positions use the first form, odd positions the second with the other
+// operand negated, so the products are q.c plus a constant times q; the constant
+// parts are tracked in fp32 and subtracted (keys: once per q row; values: per page,
+// rescaled with the accumulator).  Positions are dimensions for q.k and tokens for p.v.
+// Keys use 16 + field (24 + c, 23 - c): what the fp32 accumulator of q.k carries
+// beside q.c decides how exact a score is, and a score that is off in its fifth
+// digit turns the bf16 rounding of a probability now and then; with 128 + field that
+// happened to one output row in two hundred, each then up to a bf16 place from the
+// scalar result.  The field's place costs one shift per dword.  Values use 128 +
+// field (136 + c, 135 - c): nothing is rounded after p.v but the result.
 #include "kvx_attend_common.h"
 
 namespace kvx {
@@ -127,14 +132,14 @@ __device__ __forceinline__ float column_sum(float x) {
 }
 
 // Four bf16 pairs from one dword of eight nibbles: register p holds nibble p
-// (low half) and nibble p + 4 (high half).  Even nibbles become 136 + c, odd
-// ones 135 - c.
+// (low half) and nibble p + 4 (high half).  Even nibbles become 24 + c, odd
+// ones 23 - c: the field sits at mantissa bits 3..6 of 16.0 (0x4180).
 __device__ __forceinline__ u32x4 expand_key_dword(uint32_t x) {
   u32x4 out;
-  out[0] = (x & 0x000F000Fu) ^ 0x43084308u;
-  out[1] = ((x >> 4) & 0x000F000Fu) ^ 0x43074307u;
-  out[2] = ((x >> 8) & 0x000F000Fu) ^ 0x43084308u;
-  out[3] = ((x >> 12) & 0x000F000Fu) ^ 0x43074307u;
+  out[0] = ((x << 3) & 0x00780078u) ^ 0x41C041C0u;
+  out[1] = ((x >> 1) & 0x00780078u) ^ 0x41B841B8u;
+  out[2] = ((x >> 5) & 0x00780078u) ^ 0x41C041C0u;
+  out[3] = ((x >> 9) & 0x00780078u) ^ 0x41B841B8u;
   return out;
 }
 
@@ -531,10 +536,10 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
       if (!live_row[nb]) q_reg = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
       for (uint32_t p = 0; p < 4; ++p) {
-        // even dims carry +136 q, odd dims (stored negated) -135 q = +135 stored
+        // even dims carry +24 q, odd dims (stored negated) -23 q = +23 stored
         const float pair_sum =
             __uint_as_float(q_reg[p] << 16) + __uint_as_float(q_reg[p] & 0xffff0000u);
-        q_bias[nb] = fmaf((p & 1) ? 135.0f : 136.0f, pair_sum, q_bias[nb]);
+        q_bias[nb] = fmaf((p & 1) ? 23.0f : 24.0f, pair_sum, q_bias[nb]);
       }
       q_lds[nb][kb * 64 + lane] = q_reg;
     }

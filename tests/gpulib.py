@@ -109,7 +109,7 @@ def check_attention(out_bits, want_bits, want_f32, rows_mask, tol, label="", exp
     with such rows from an arrangement of the caller's own), the oracle
     recomputes the row with the rounded weight of one of its heaviest tokens moved
     one place up or down, and one of those rows must be within tol of the GPU's.
-    At most 1% of the rows (one where there are fewer than a hundred) may need it and
+    At most 1% of the rows (two where there are fewer than two hundred) may need it and
     none may be more than tol + 2^-7 away (one place of a weight just above a power of
     two, were the row that one token); every such row is counted in ALLOWANCE_LOG."""
     got = ko.bf16_to_f32(out_bits).reshape(out_bits.shape)
@@ -130,7 +130,7 @@ def check_attention(out_bits, want_bits, want_f32, rows_mask, tol, label="", exp
                                      f"at row {worst}")
         assert rel.max() <= tol + 2.0 ** -7, (f"{label}: relative L2 vs oracle bf16 {rel.max():.3e} > "
                                               f"{tol + 2.0 ** -7} at row {worst}")
-        assert over.size <= max(1, int(0.01 * rel.size)), (
+        assert over.size <= max(2, int(0.01 * rel.size)), (
             f"{label}: only {within:.4f} of the {rel.size} rows are within {tol}")
         for flat in over:
             index = index_of(flat)

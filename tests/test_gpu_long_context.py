@@ -136,9 +136,10 @@ def test_long_history_verify_decode_and_prefill(history):
     tw.close()
 
 
-def test_a_split_too_long_for_the_matrix_kernels_is_still_right():
-    """A split of more pages than the matrix-core kernels stage (1024) goes to the format-generic
-    kernels: one split over 40 000 tokens (1251 pages), one-row decode."""
+def test_one_split_over_a_long_history():
+    """The matrix-core kernels take a split of any length (their page entries come through the
+    scalar unit as they go, not from a staged table): one split over 40 000 tokens (1251 pages),
+    one-row decode."""
     history = 40000
     n_pages = (history + 1 + 31) // 32
     tw = Gp.Twin(FMT, H, D, 1, n_pages)
@@ -165,11 +166,13 @@ def test_a_split_too_long_for_the_matrix_kernels_is_still_right():
     kvx.attend_decode(tw.dev, 0, QH, Gp.dev(q1), out, [td], dp, 1, ws)
     torch.cuda.synchronize()
     after = kvx.attend_paths()
-    assert after[0] == before[0] + 1 and after[1] == before[1]
+    assert after[1] == before[1] + 1 and after[0] == before[0]
     got = Gp.host_u16(out)
     for head, g in [(0, 0), (3, 5)]:
         want, want32 = one_row(FMT, q1[0, head, 0].reshape(G, D), th, tw.host.layer(0), head, history,
                                1, 1, 1, g)
-        Gp.check_attention(got[0, head, 0, g].reshape(1, D), want.reshape(1, D), want32.reshape(1, D),
-                           np.ones(1, dtype=bool), 2e-3, "one long split on the generic kernels")
+        args = dict(fmt=FMT, tile_queries=q1[0, head, 0].reshape(G, D), table=th, kv=tw.host.layer(0),
+                    head=head, committed=history, active=1, splits=1, capacity=1, fused_row=g)
+        check_row(got[0, head, 0, g], want, want32, "one split over 1251 pages",
+                  dict(kv_heads=H, group=G, head_dim=D, **args))
     tw.close()
