@@ -452,7 +452,8 @@ inline bool matrix_attention_covers(const kvx_storage *s, uint32_t query_heads,
   const kvx_layout &l = s->layout;
   if (l.head_dim != kD) return false;
   const uint32_t G = query_heads / l.kv_heads, capacity = lanes[0].row_capacity;
-  if (G > 16 || !capacity || capacity > KVX_TREE_NODES) return false;
+  // up to 16 rows per lane (a verify tree), or the 32 rows of four prefill tiles
+  if (G > 16 || !capacity || capacity > 2 * KVX_TREE_NODES) return false;
   for (uint32_t i = 0; i < n_lanes; ++i) {
     const kvx_verify_params &p = lanes[i];
     if (p.row_capacity != capacity || !p.active_rows || p.active_rows > capacity) return false;
