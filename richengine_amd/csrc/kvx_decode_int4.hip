@@ -204,35 +204,6 @@ struct RegisterPage {
   }
 };
 
-// A page that the waves of a workgroup expanded together into LDS, every operand
-// already in the layout its MFMA wants: a wave reads what RegisterPage computes.
-struct GroupPage {
-  u32x4 keys[2][8][64];    // [token block][dims block][lane]
-  u32x4 values[16][64];    // [nibble position][lane]
-  float scales[2][kPage];  // key scales, value scales, by token
-};
-struct SharedPage {
-  const GroupPage *page;
-  uint32_t lane, g;
-  __device__ __forceinline__ u32x4 key(uint32_t tb, uint32_t kb) const { return page->keys[tb][kb][lane]; }
-  __device__ __forceinline__ void scales(float (&ks)[8], float (&vs)[8]) const {
-#pragma unroll
-    for (uint32_t tb = 0; tb < 2; ++tb) {
-      const f32x4 k = *reinterpret_cast<const f32x4 *>(&page->scales[0][16 * tb + 4 * g]);
-      const f32x4 v = *reinterpret_cast<const f32x4 *>(&page->scales[1][16 * tb + 4 * g]);
-#pragma unroll
-      for (uint32_t rr = 0; rr < 4; ++rr) {
-        ks[4 * tb + rr] = k[rr];
-        vs[4 * tb + rr] = v[rr];
-      }
-    }
-  }
-  __device__ __forceinline__ void values(uint32_t half, uint32_t part, u32x4 (&vop)[4]) const {
-#pragma unroll
-    for (uint32_t i = 0; i < 4; ++i) vop[i] = page->values[8 * half + 4 * part + i][lane];
-  }
-};
-
 // One page against NB blocks of 16 fused query rows; every key and value
 // operand is made once and used by all blocks.
 // MASKED: the page may hold tokens some row does not see (only the last pages of a
@@ -637,234 +608,6 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
                    partials, statistics);
 }
 
-// ---- pages shared by the waves of a workgroup: verify, tree verify, chunked prefill ----
-//
-// With many query rows the cost of a page is not fetching it but turning its nibbles into
-// MFMA operands, and a wave that does so for its own 32 or 48 fused rows repeats what the
-// wave next to it does for the same page.  Here W waves (2 or 4) form a workgroup per
-// (lane, split, KV head): each fetches and expands 1/W of the page into LDS, in the
-// operands' final layout, and all of them multiply their own 48 fused rows with the shared
-// copy.  Two LDS copies alternate: while a page is multiplied the next one is expanded, one
-// barrier per page.  Raw pages are small per wave (9 or 17 registers), so each wave keeps the
-// pages two and three ahead in flight.
-constexpr uint32_t kGroupBlocks = 3;  // blocks of 16 fused rows per wave
-
-template <uint32_t W>
-struct GroupRaw {  // one wave's share of a page as loaded
-  static constexpr uint32_t kPieces = 4 / W;  // pieces of 8 tokens
-  u32x4 k[kPieces];                  // 16 bytes of token 8 piece + lane / 8
-  u32x2 v_even[kPieces], v_odd[kPieces];  // 8 bytes of tokens 8 piece + 2 (lane / 16), + 1
-  float scale;                       // wave 0: as PageRegs::scale
-};
-
-template <uint32_t W, bool REUSED>
-__device__ __forceinline__ void load_group_raw(GroupRaw<W> &r, uint64_t entry, uint32_t head,
-                                               uint32_t kv_heads, uint32_t layer_offset,
-                                               uint64_t key_scales_off, uint64_t values_off,
-                                               uint32_t scale_rows_apart, uint32_t wave,
-                                               uint32_t lane) {
-  const uint32_t entry_lo = __builtin_amdgcn_readfirstlane(uint32_t(entry));
-  const uint32_t entry_hi = __builtin_amdgcn_readfirstlane(uint32_t(entry >> 32));
-  const uint32_t index = entry_lo & KVX_PAGE_INDEX_MASK;
-  const uint8_t *region =
-      reinterpret_cast<const uint8_t *>((uint64_t(entry_hi) << 32) | (entry_lo - index)) + layer_offset;
-  const uint64_t head_page = uint64_t(index) * kv_heads + head;
-  const uint8_t *keys = region + head_page * kHeadSlabBytes;
-  const uint8_t *values = keys + values_off;
-#pragma unroll
-  for (uint32_t s = 0; s < GroupRaw<W>::kPieces; ++s) {
-    const uint32_t piece = GroupRaw<W>::kPieces * wave + s;
-    r.k[s] = load_streaming<u32x4, REUSED>(keys + (8 * piece + (lane >> 3)) * kRowBytes + 16 * (lane & 7));
-    const uint8_t *pair = values + (8 * piece + 2 * (lane >> 4)) * kRowBytes + 8 * (lane & 15);
-    r.v_even[s] = load_streaming<u32x2, REUSED>(pair);
-    r.v_odd[s] = load_streaming<u32x2, REUSED>(pair + kRowBytes);
-  }
-  if (wave == 0)
-    r.scale = load_global<float>(region + key_scales_off + head_page * (kPage * 4u) +
-                                 (lane < kPage ? 0u : scale_rows_apart) + 4u * (lane & (kPage - 1)));
-}
-
-// Expands a wave's share into the workgroup's copy.  Which lane of which MFMA an
-// element belongs to follows from its token and dims exactly as in RegisterPage:
-// keys: token 16 tb + t, dword 16 (kb >> 2) + 4 g + (kb & 3) of its row is lane (t, g) of
-// operand (tb, kb); values: the pair of tokens 16 tb + 4 g + rr, + 1 (rr even) at dims
-// 16 t + m is element 2 tb + rr / 2 of lane (t, g) of operand m.
-template <uint32_t W>
-__device__ __forceinline__ void expand_group_raw(GroupPage &page, const GroupRaw<W> &r, uint32_t wave,
-                                                 uint32_t lane) {
-#pragma unroll
-  for (uint32_t s = 0; s < GroupRaw<W>::kPieces; ++s) {
-    const uint32_t piece = GroupRaw<W>::kPieces * wave + s;
-    {
-      const uint32_t token = 8 * piece + (lane >> 3), quad = lane & 7;
-      const uint32_t tb = token >> 4, t = token & 15, g = quad & 3, kb = 4 * (quad >> 2);
-#pragma unroll
-      for (uint32_t c = 0; c < 4; ++c) page.keys[tb][kb + c][16 * g + t] = expand_key_dword(r.k[s][c]);
-    }
-    {
-      const uint32_t token = 8 * piece + 2 * (lane >> 4), t = lane & 15;
-      const uint32_t tb = token >> 4, g = (token & 15) >> 2, element = 2 * tb + ((token & 3) >> 1);
-#pragma unroll
-      for (uint32_t half = 0; half < 2; ++half)
-#pragma unroll
-        for (uint32_t part = 0; part < 2; ++part) {
-          const uint32_t both = __builtin_amdgcn_perm(r.v_odd[s][half], r.v_even[s][half],
-                                                      part ? 0x07060302u : 0x05040100u);
-#pragma unroll
-          for (uint32_t i = 0; i < 4; ++i)
-            reinterpret_cast<uint32_t *>(&page.values[8 * half + 4 * part + i][16 * g + t])[element] =
-                ((both >> (4 * i)) & 0x000F000Fu) ^ 0x43074308u;
-        }
-    }
-  }
-  if (wave == 0) (&page.scales[0][0])[lane] = r.scale;
-}
-
-template <uint32_t W, bool kReused>
-__device__ __forceinline__ void attend_group_int4(const uint16_t *__restrict__ queries,
-                                                  uint16_t *__restrict__ output,
-                                                  float *__restrict__ partials,
-                                                  float *__restrict__ statistics,
-                                                  const DecodeArgs &a) {
-  constexpr uint32_t NB = kGroupBlocks;
-  __shared__ GroupPage shared_page[2];
-  const uint32_t item = blockIdx.x, head = blockIdx.y;
-  uint32_t li;
-  const DecodeLane l = lane_of_item(a, item, li);
-  const uint32_t split = item - l.first_item;
-  // Every wave of the workgroup takes the same way out: the barriers below are
-  // reached by all of them or by none.
-  if (split >= l.split_count) return;
-  const uint32_t visible = l.committed + l.active_rows;
-  const uint32_t pages = (visible + kPage - 1) / kPage;
-  const uint32_t per = (pages + l.split_count - 1) / l.split_count;
-  const uint32_t written = (pages + per - 1) / per;
-  const uint32_t begin = split * per;
-  if (begin >= pages) return;
-  const uint32_t end = min(pages, begin + per);
-
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t lane = threadIdx.x & 63u, t = lane & 15, g = lane >> 4;
-  const uint32_t H = a.kv_heads, G = a.group, M = a.fused_rows;
-  uint32_t m[NB];
-  bool in_tile[NB], live_row[NB];
-  Sight sight[NB];
-#pragma unroll
-  for (uint32_t nb = 0; nb < NB; ++nb) {
-    m[nb] = 16 * (NB * wave + nb) + t;
-    const uint32_t query_row = m[nb] / G;
-    in_tile[nb] = m[nb] < M;
-    live_row[nb] = in_tile[nb] && query_row < l.active_rows;
-    sight[nb].committed = l.committed;
-    sight[nb].visible = visible;
-    sight[nb].limit =
-        live_row[nb] ? min(visible, l.committed + min(query_row, l.active_rows - 1) + 1) : visible;
-    sight[nb].tree = live_row[nb] && l.masks != nullptr;
-    sight[nb].mask = sight[nb].tree ? l.masks[query_row] : 0u;
-  }
-  // A wave none of whose rows is in the tile still fetches and expands its share.
-  const bool computes = 16 * NB * wave < M;
-  const uint32_t db = kPage * H * kRowBytes, sb = kPage * H * 4;
-  const RegionOffsets ro = region_offsets(a.kv.extent_pages, db, sb);
-  const float score_scale = default_score_scale(kD, l.score_scale);
-
-  // The wave's raw shares of the pages two and three ahead are in flight while the
-  // page one ahead is expanded; set i % 2 holds page i.
-  const uint64_t *const entries = l.table + begin;
-  const uint32_t count = end - begin, last_slot = count - 1;
-  GroupRaw<W> raw[2];
-  auto fetch = [&](GroupRaw<W> &set, uint32_t slot) {
-    const uint64_t entry = scalar_entry(entries, min(slot, last_slot));
-    asm volatile("");
-    load_group_raw<W, kReused>(set, entry, head, H, a.kv.offset, ro.key_scales, ro.values,
-                               uint32_t(ro.value_scales - ro.key_scales), wave, lane);
-    asm volatile("");
-  };
-  fetch(raw[0], 0);
-  fetch(raw[1], 1);
-
-  // Queries in expansion order (see attend_int4): two blocks stay in registers, the
-  // third is read from LDS page by page (three would leave too few registers for the
-  // operands in flight, and the compiler would spill inside the page loop).
-  const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
-  constexpr uint32_t kHeldBlocks = 2;
-  __shared__ u32x4 q_lds[W][NB - kHeldBlocks][8 * 64];
-  u32x4 q_reg[kHeldBlocks][8];
-  float q_bias[NB];
-#pragma unroll
-  for (uint32_t nb = 0; nb < NB; ++nb) {
-    const uint16_t *q_row = q_head + uint64_t(live_row[nb] ? m[nb] : 0) * kD;
-    q_bias[nb] = 0.0f;
-#pragma unroll
-    for (uint32_t kb = 0; kb < 8; ++kb) {
-      const u32x4 raw_q = load_global<u32x4>(q_row + 8 * (16 * (kb >> 2) + 4 * g + (kb & 3)));
-      u32x4 q;
-      q[0] = __builtin_amdgcn_perm(raw_q[2], raw_q[0], 0x05040100u);
-      q[1] = __builtin_amdgcn_perm(raw_q[2], raw_q[0], 0x07060302u) ^ 0x80008000u;
-      q[2] = __builtin_amdgcn_perm(raw_q[3], raw_q[1], 0x05040100u);
-      q[3] = __builtin_amdgcn_perm(raw_q[3], raw_q[1], 0x07060302u) ^ 0x80008000u;
-      if (!live_row[nb]) q = u32x4{0u, 0u, 0u, 0u};
-#pragma unroll
-      for (uint32_t p = 0; p < 4; ++p) {
-        const float pair_sum = __uint_as_float(q[p] << 16) + __uint_as_float(q[p] & 0xffff0000u);
-        q_bias[nb] = fmaf((p & 1) ? 23.0f : 24.0f, pair_sum, q_bias[nb]);
-      }
-      if (nb < kHeldBlocks) q_reg[nb][kb] = q;
-      else q_lds[wave][nb - kHeldBlocks][kb * 64 + lane] = q;
-    }
-    q_bias[nb] = column_sum(q_bias[nb]);
-  }
-  State st[NB];
-#pragma unroll
-  for (uint32_t nb = 0; nb < NB; ++nb) {
-#pragma unroll
-    for (uint32_t i = 0; i < 16; ++i) st[nb].acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    st[nb].row_max = -INFINITY;
-    st[nb].row_sum = 0.0f;
-    st[nb].bias = 0.0f;
-  }
-  auto held_queries = [&](uint32_t nb, uint32_t kb) {
-    return nb < kHeldBlocks ? q_reg[nb][kb] : q_lds[wave][nb - kHeldBlocks][kb * 64 + lane];
-  };
-
-  // The first page into the first copy.
-  expand_group_raw<W>(shared_page[0], raw[0], wave, lane);
-  fetch(raw[0], 2);
-  __syncthreads();
-  // Slot i of the split: copy i % 2 holds it expanded when its turn comes; while it is
-  // multiplied, slot i + 1 goes from raw set (i + 1) % 2 into the other copy and that set
-  // is sent for slot i + 3.  Pages from the one that holds token `committed` on take the
-  // masked path: before it every row sees every token.
-  const uint32_t first_masked_page = l.committed / kPage;
-  for (uint32_t slot = 0; slot < count; ++slot) {
-    const GroupPage &now = shared_page[slot & 1];
-    const uint32_t first_token = (begin + slot) * kPage;
-    if (slot & 1) {
-      if (slot + 1 < count) {
-        expand_group_raw<W>(shared_page[0], raw[0], wave, lane);
-        fetch(raw[0], slot + 3);
-      }
-    } else {
-      if (slot + 1 < count) {
-        expand_group_raw<W>(shared_page[1], raw[1], wave, lane);
-        fetch(raw[1], slot + 3);
-      }
-    }
-    if (computes) {
-      if (begin + slot >= first_masked_page)
-        attend_page<true, NB>(SharedPage{&now, lane, g}, held_queries, q_bias, score_scale, first_token,
-                              sight, g, st, [] {});
-      else
-        attend_page<false, NB>(SharedPage{&now, lane, g}, held_queries, q_bias, score_scale, first_token,
-                               sight, g, st, [] {});
-    }
-    __syncthreads();
-  }
-  if (computes)
-    write_blocks<NB>(st, m, in_tile, live_row, l, a, head, split, a.all_partials ? 2u : written, g, output,
-                     partials, statistics);
-}
-
 // One block of 16 fused rows per wave, two waves per SIMD: one-row decode, where
 // the group's query heads are the only rows and memory latency is what to hide.
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_int4_kernel(
@@ -912,29 +655,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
   attend_int4<3, kVerify48Depth>(queries, output, partials, statistics, a);
 }
 
-// Workgroups of two and of four waves over shared pages (96 and 192 fused rows), for lanes
-// read once (verify) and for the lanes of a chunked prefill, which walk the same pages.
-template <uint32_t W, bool kReused>
-__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 1))) void group_int4_kernel(
-    const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
-    float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
-  attend_group_int4<W, kReused>(queries, output, partials, statistics, a);
-}
-
 }  // namespace
 }  // namespace kvx
 
 using namespace kvx;
-
-// While the workgroup kernels are being brought up: KVX_INT4_GROUPS=1 in the environment
-// selects them for more than 16 fused rows.
-static bool kvx_int4_groups_off() {
-  static const bool off = [] {
-    const char *v = getenv("KVX_INT4_GROUPS");
-    return !(v && v[0] == '1');
-  }();
-  return off;
-}
 
 // Runs paged attention (split kernel, then the merge of multi-split lanes) for
 // int4 pages of head dimension 256; returns 1 (declined) for shapes it does not
@@ -964,29 +688,6 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   // and long (verify: 13% on 4 x 65536 tokens x 16 tree rows); chunked prefill has
   // hundreds of tiles of 48 fused rows, where a half-empty second wave and one
   // wave per SIMD cost more than the sharing saves.
-  // More than 16 fused rows: the waves of a workgroup share every expanded page.
-  // Lanes of up to 96 fused rows take two waves, up to 192 four; the tiles of a
-  // chunked prefill walk the same pages, so their loads may stay in the caches.
-  if (fused_rows > 16 && !many_tiles && !kvx_int4_groups_off()) {
-    if (fused_rows > 48 * 4) return 1;
-    if (fused_rows <= 96)
-      return tile_rows ? launch_matrix_attention(group_int4_kernel<2, true>, "group_int4_kernel", 96, 128, s,
-                                                 kv, query_heads, queries, output, page_tables, lanes,
-                                                 n_lanes, row_masks, row_stride, lane_stride, workspace,
-                                                 workspace_bytes, stream, nullptr, tile_rows, epilogue)
-                       : launch_matrix_attention(group_int4_kernel<2, false>, "group_int4_kernel", 96, 128, s,
-                                                 kv, query_heads, queries, output, page_tables, lanes,
-                                                 n_lanes, row_masks, row_stride, lane_stride, workspace,
-                                                 workspace_bytes, stream, nullptr, tile_rows, epilogue);
-    return tile_rows ? launch_matrix_attention(group_int4_kernel<4, true>, "group_int4_kernel", 192, 256, s,
-                                               kv, query_heads, queries, output, page_tables, lanes,
-                                               n_lanes, row_masks, row_stride, lane_stride, workspace,
-                                               workspace_bytes, stream, nullptr, tile_rows, epilogue)
-                     : launch_matrix_attention(group_int4_kernel<4, false>, "group_int4_kernel", 192, 256, s,
-                                               kv, query_heads, queries, output, page_tables, lanes,
-                                               n_lanes, row_masks, row_stride, lane_stride, workspace,
-                                               workspace_bytes, stream, nullptr, tile_rows, epilogue);
-  }
   if (fused_rows > 16 && !many_tiles && tile_rows)
     return launch_matrix_attention(prefill_int4_kernel, "prefill_int4_kernel", 32, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
