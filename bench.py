@@ -79,9 +79,10 @@ def parse():
                          "current stream); a sequence's layers stay in order on its stream")
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
-    ap.add_argument("--workload", choices=["decode", "tree-verify", "prefill", "qkv-prepare", "shared-prefix"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "decode-single", "tree-verify", "prefill", "qkv-prepare", "shared-prefix"], default="decode",
                     help="decode = batch-32 mixed-length int4 decode, the headline metric (default); "
-                         "tree-verify = 16-node tree verify and prefill = chunked prefill with a shared "
+                         "decode-single = one sequence of 32768 tokens, the 16 per-layer calls replayed "
+                         "as one HIP graph; tree-verify = 16-node tree verify and prefill = chunked prefill with a shared "
                          "prefix, the matrix-core paths (profiling)")
     ap.add_argument("--format", choices=["bf16", "fp8", "int8", "int4"], default=None,
                     help="page format of the prefill workload (default bf16) and of the shared-prefix "
@@ -158,6 +159,92 @@ def cpu_baseline(contexts, seed, budget_s):
                       "note": "same sequences, one per thread; rate = bytes / (summed attention "
                               "seconds / threads), history fills excluded"},
     }
+
+
+def cpu_history(ko, rng, fmt, tokens):
+    """An oracle store of one layer holding `tokens` tokens of N(0,1) rows (untimed fill);
+    returns (store, table, pages)."""
+    import numpy as np
+    n_pages = (tokens + 31) // 32 + 1
+    store = ko.Store(1, H, D, fmt, n_pages, n_pages)
+    store.allocate(0)
+    table = store.entries(np.arange(n_pages, dtype=np.uint32))
+    done = 0
+    while done < tokens:
+        n = min(2048, tokens - done)
+        stride = (n + 31) // 32 * 32
+        k = ko.f32_to_bf16(rng.standard_normal((H, stride, D)).astype(np.float32)).reshape(H, stride, D)
+        v = ko.f32_to_bf16(rng.standard_normal((H, D, stride)).astype(np.float32)).reshape(H, D, stride)
+        ko.store_chunk(fmt, H, D, k, v, table, ko.ChunkParams(done, n, stride, n_pages, store.layer(0)))
+        done += n
+    return store, table, n_pages
+
+
+def cpu_tree_verify(seed, context, nodes, masks, budget_s):
+    """The oracle on a bounded sample of the tree-verify workload: one sequence, one layer,
+    the append of the tree's rows and the masked verify over a history cut to what the budget
+    allows (cost is linear in the history); the rate is scaled back to the full history and to
+    16 layers."""
+    import numpy as np
+    from oracle import kvoracle as ko
+    rng = np.random.default_rng(seed)
+    # ~1 GFLOP/s for the scalar port: rows x heads x D x 4 flops per visible token
+    per_token = 4.0 * D * nodes * QH / 1.0e9
+    history = int(min(context, max(2048, (budget_s / per_token) // 2048 * 2048)))
+    store, table, n_pages = cpu_history(ko, rng, ko.INT4, history)
+    k = ko.f32_to_bf16(rng.standard_normal((H, 32, D)).astype(np.float32)).reshape(H, 32, D)
+    v = ko.f32_to_bf16(rng.standard_normal((H, D, 32)).astype(np.float32)).reshape(H, D, 32)
+    q = ko.f32_to_bf16(rng.standard_normal((1, H, 32, G, D)).astype(np.float32)).reshape(1, H, 32, G, D)
+    splits = min(max(1, n_pages // 64), 128)
+    t0 = time.perf_counter()
+    stored = ko.store_verify(ko.INT4, H, D, k[None], v[None], [table],
+                             [ko.ChunkParams(history, nodes, 32, n_pages, store.layer(0))], 16)
+    attended = ko.attend_verify(ko.INT4, H, G, D, q, [table],
+                                [ko.VerifyParams(history, n_pages, store.layer(0), splits, 128, nodes, 16,
+                                                 0.0)],
+                                row_masks=np.ascontiguousarray(masks[:1]), want_f32=False)[0]
+    spent = time.perf_counter() - t0
+    store.close()
+    assert stored == 1 and attended == 1, "the oracle refused the tree-verify sample"
+    full = spent * (context + nodes) / (history + nodes) * LAYERS  # one sequence, all layers, full history
+    return {"value": nodes / full, "unit": "draft tokens/s", "cores": 1, "kind": "port",
+            "sample": f"one sequence of the batch, one layer, history cut to {history} of {context} tokens: "
+                      f"append {nodes} tree rows + masked verify, {spent:.1f} s of scalar C++ oracle; "
+                      f"scaled linearly to the full history and {LAYERS} layers",
+            "seconds": spent, "history_tokens": history}
+
+
+def cpu_prefill(seed, fmt_name, prefix, chunk, budget_s):
+    """The oracle on a bounded sample of the chunked-prefill workload: one sequence, one layer,
+    the first rows of one chunk (append + causal attention over the prefix and those rows), as
+    many rows as the budget allows; the rate is per 16 layers."""
+    import numpy as np
+    from oracle import kvoracle as ko
+    fmt = {"bf16": ko.BF16, "fp8": ko.FP8, "int8": ko.INT8, "int4": ko.INT4}[fmt_name]
+    rng = np.random.default_rng(seed)
+    per_row = 4.0 * D * QH * prefix / 1.0e9  # seconds per chunk row at ~1 GFLOP/s
+    rows = int(min(chunk, max(8, (budget_s / per_row) // 8 * 8)))
+    store, table, n_pages = cpu_history(ko, rng, fmt, prefix + rows)
+    # cpu_history filled prefix + rows tokens; the chunk's rows are stored again by the timed append
+    stride = (rows + 31) // 32 * 32
+    k = ko.f32_to_bf16(rng.standard_normal((H, stride, D)).astype(np.float32)).reshape(H, stride, D)
+    v = ko.f32_to_bf16(rng.standard_normal((H, D, stride)).astype(np.float32)).reshape(H, D, stride)
+    q = ko.f32_to_bf16(rng.standard_normal((H, stride, G, D)).astype(np.float32)).reshape(H, stride, G, D)
+    t0 = time.perf_counter()
+    stored = ko.store_chunk(fmt, H, D, k, v, table,
+                            ko.ChunkParams(prefix, rows, stride, n_pages, store.layer(0)))
+    attended = ko.attend_prefill(fmt, H, G, D, q, table,
+                                 ko.PrefillParams(prefix, rows, stride, n_pages, store.layer(0), 1, 0.0),
+                                 want_f32=False)[0]
+    spent = time.perf_counter() - t0
+    store.close()
+    assert stored == 1 and attended == 1, "the oracle refused the prefill sample"
+    return {"value": rows / (spent * LAYERS), "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"one sequence, one layer, the first {rows} rows of a {chunk}-row chunk over the "
+                      f"{prefix}-token prefix: append + causal attention, {spent:.1f} s of scalar C++ "
+                      f"oracle; rate = rows / (seconds x {LAYERS} layers)",
+            "seconds": spent, "rows": rows}
+
 
 
 def profiled_traffic():
@@ -296,6 +383,8 @@ def tree_verify(args):
         "cpu_baseline": None,
     }
     storage.close()
+    if args.cpu_seconds > 0:
+        result["cpu_baseline"] = cpu_tree_verify(args.seed, context, nodes, masks, args.cpu_seconds)
     print(json.dumps(result))
 
 
@@ -599,6 +688,146 @@ def chunked_prefill(args):
         "cpu_baseline": None,
     }
     storage.close()
+    if args.cpu_seconds > 0:
+        result["cpu_baseline"] = cpu_prefill(args.seed, args.format, prefix, chunk, args.cpu_seconds)
+    print(json.dumps(result))
+
+
+def single_decode(args):
+    """One sequence, context 32768, int4, 16 layers, contiguous page table: a step appends one
+    token and runs decode attention in every layer (kv_append_attend_decode, one call per
+    layer).  The 16 calls are captured once in a HIP graph and a step is one replay: a lone
+    sequence leaves the GPU nothing to overlap the launches with, so the gaps between them
+    are what a graph removes.  Every replay stores the same token and attends the same
+    32769 tokens.  Eager steps (the same calls issued one by one) are timed beside it."""
+    import numpy as np
+    import torch
+    from richengine_amd import kvx
+
+    L = kvx.lib()
+    torch.cuda.set_device(0)
+    context = args.uniform_context or 32768
+    n_pages = (context + 1 + 31) // 32
+    layout = kvx.Layout(LAYERS, H, D, kvx.INT4, 0.0)
+    extent_pages = L.kvx_layout_largest_extent_pages(C.byref(layout))
+    extents = -(-n_pages // extent_pages)
+    storage = kvx.Storage(LAYERS, H, D, kvx.INT4, extents * extent_pages, extent_pages, aligned=True)
+    storage.allocate_all()
+    table = storage.table(np.arange(n_pages, dtype=np.uint32))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(args.seed)
+    for done in range(0, context, 2048):
+        n = min(2048, context - done)
+        stride = (n + 31) // 32 * 32
+        k = torch.randn((H, stride, D), generator=gen, device="cuda").bfloat16()
+        v = torch.randn((H, D, stride), generator=gen, device="cuda").bfloat16()
+        for layer in range(LAYERS):
+            kvx.append(storage, layer, k, v, [table], [kvx.ChunkParams(done, n, stride, n_pages)],
+                       H * stride * D)
+    chunk_k = torch.randn((1, H, 32, D), generator=gen, device="cuda").bfloat16()
+    chunk_v = torch.randn((1, H, D, 32), generator=gen, device="cuda").bfloat16()
+    queries = torch.randn((1, H, 1, G, D), generator=gen, device="cuda").bfloat16()
+    output = torch.zeros_like(queries)
+    splits = kvx.decode_plan([context], H)[0]
+    if args.pages_per_split:
+        splits = min(max(1, -(-n_pages // args.pages_per_split)), 512)
+    vp = [kvx.VerifyParams(context, n_pages, kvx.KvLayer(), splits, splits, 1, 1, 0.0)]
+    vp_arr = (kvx.VerifyParams * 1)(*vp)
+    ws_bytes = kvx.attend_workspace_bytes(storage, vp, QH) + (1 << 20)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    table_arr = (C.c_void_p * 1)(table.data_ptr())
+
+    def layers(stream):
+        for layer in range(LAYERS):
+            rc = L.kv_append_attend_decode(storage.h, layer, chunk_k.data_ptr(), chunk_v.data_ptr(),
+                                           H * 32 * D, 32, QH, queries.data_ptr(), output.data_ptr(),
+                                           table_arr, vp_arr, 1, 1, workspace.data_ptr(), ws_bytes, stream)
+            if rc:
+                kvx.check(rc)
+
+    def timed(run, count):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(count):
+            run()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / count
+
+    eager_stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for _ in range(max(args.warmup, 1)):
+        layers(eager_stream)
+    eager_s = timed(lambda: layers(eager_stream), args.steps)
+    eager_out = output.clone()
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layers(C.c_void_p(side.cuda_stream))  # every kernel loaded before the capture
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            layers(C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(max(args.warmup, 1)):
+        graph.replay()
+    # Replays between eager work and synchronisations, each checked against the eager result.
+    for _ in range(3):
+        output.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(output, eager_out), "a graph replay differs from the eager step"
+        layers(eager_stream)
+    step_s = timed(graph.replay, args.steps)
+
+    def time_kernel(call):
+        call(0)
+        torch.cuda.synchronize()
+        k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        k0.record()
+        for it in range(args.kernel_iters):
+            call(it % LAYERS)
+        k1.record()
+        torch.cuda.synchronize()
+        return k0.elapsed_time(k1) / args.kernel_iters
+
+    split_ms = time_kernel(lambda layer: L.kv_attend_split(
+        storage.h, layer, QH, queries.data_ptr(), table_arr, vp_arr, 1, None, 1, workspace.data_ptr(),
+        ws_bytes, eager_stream))
+    merge_ms = time_kernel(lambda layer: L.kv_attend_merge(
+        storage.h, QH, output.data_ptr(), vp_arr, 1, 1, workspace.data_ptr(), ws_bytes, eager_stream))
+    layer_bytes = (context + 1) * BYTES_PER_TOKEN_LAYER
+    value = layer_bytes * LAYERS / step_s / 1e9
+    achieved = layer_bytes / (split_ms * 1e-3) / 1e9
+    result = {
+        "metric": "int4 paged decode attn, one sequence of 32768 tokens: KV GB/s per step",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int4 pages, bf16 MFMA, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: single-sequence int4 decode, batch 1, context "
+                               f"{context}, 16 layers, contiguous page table: 1-token append + split-K "
+                               "paged attention per layer; a step = one replay of the HIP graph of the "
+                               "16 per-layer calls",
+                   "batch": 1, "layers": LAYERS, "context": context, "splits": int(splits),
+                   "pages_per_split": -(-n_pages // int(splits)), "seed": args.seed},
+        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "decode_tokens_per_s": round(1 / step_s, 1),
+        "us_per_layer": round(step_s * 1e6 / LAYERS, 2),
+        "eager_ms_per_step": round(eager_s * 1e3, 4),
+        "eager_us_per_layer": round(eager_s * 1e6 / LAYERS, 2),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "decode_int4_kernel (split kernel of paged decode attention), one layer per launch",
+                     "bytes_per_launch": layer_bytes, "ms_per_launch": round(split_ms, 4),
+                     "merge_ms_per_launch": round(merge_ms, 4)},
+        "cpu_baseline": None,
+    }
+    storage.close()
+    if args.cpu_seconds > 0:
+        spent = cpu_lane(context, args.seed)
+        result["cpu_baseline"] = {
+            "value": layer_bytes / spent / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"the sequence itself, one layer of the 16: append 1 token + decode attention over "
+                      f"{context + 1} tokens, {spent:.1f} s of scalar C++ oracle"}
     print(json.dumps(result))
 
 
@@ -615,6 +844,8 @@ def main():
             kvx_build.build(verbose=False)
         if args.workload == "qkv-prepare":
             return qkv_prepare(args)
+        if args.workload == "decode-single":
+            return single_decode(args)
         if args.workload == "shared-prefix":
             return shared_prefix(args)
         return tree_verify(args) if args.workload == "tree-verify" else chunked_prefill(args)
@@ -813,6 +1044,32 @@ def main():
     achieved = launch_bytes / (kernel_ms * 1e-3) / 1e9
     traffic = profiled_traffic()
 
+    # ---- what the access pattern streams at: the same pages through the split kernel's
+    # own loads with no arithmetic behind them (kvx_calibrate_stream), 32 pages per wave
+    # as the plan gives the long lanes.
+    live = [(c + 1 + 31) // 32 for c in committed]
+    all_entries = torch.cat([tables[i][:live[i]] for i in range(BATCH)]).contiguous()
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+    def time_stream(per, heads):
+        def call(layer):
+            return L.kvx_calibrate_stream(storage.h, layer, all_entries.data_ptr(), all_entries.numel(),
+                                          per, heads, sink.data_ptr(), stream)
+        for layer in range(2):
+            kvx.check(call(layer))
+        torch.cuda.synchronize()
+        k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        k0.record()
+        for it in range(args.kernel_iters):
+            call(it % LAYERS)
+        k1.record()
+        torch.cuda.synchronize()
+        return k0.elapsed_time(k1) / args.kernel_iters
+
+    stream_bytes = all_entries.numel() * 32 * BYTES_PER_TOKEN_LAYER
+    stream_ms = {per: time_stream(per, 1) for per in (16, 32, 64)}
+    stream4_ms = {per: time_stream(per, 4) for per in (16, 32, 64)}
+
     result = {
         "metric": "int4 paged decode attn: KV GB/s (% HBM peak) + decode tokens/s, bs=32",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -842,6 +1099,16 @@ def main():
             "bytes_per_launch": launch_bytes, "ms_per_launch": round(kernel_ms, 4),
             "merge_ms_per_launch": round(merge_ms, 4), "split_plus_merge_ms": round(both_ms, 4),
             "split_plus_merge_gbs": round(launch_bytes / (both_ms * 1e-3) / 1e9, 1),
+            "stream_ceiling": {
+                "what": "the split kernel's page loads alone (kvx_calibrate_stream) over the same pages, "
+                        "whole pages counted",
+                "bytes_per_launch": stream_bytes,
+                "gbs_by_pages_per_wave": {str(per): round(stream_bytes / (ms * 1e-3) / 1e9, 1)
+                                          for per, ms in stream_ms.items()},
+                "ms_by_pages_per_wave": {str(per): round(ms, 4) for per, ms in stream_ms.items()},
+                "gbs_four_heads_per_workgroup": {str(per): round(stream_bytes / (ms * 1e-3) / 1e9, 1)
+                                                 for per, ms in stream4_ms.items()},
+            },
         },
     }
     storage.close()

@@ -36,7 +36,7 @@ SYMBOLS = [
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
     "kvx_pool_snapshot_get", "kv_append", "kv_prepare_append", "kv_attend_decode_shared", "kvx_attend_shared_workspace_bytes", "kv_attend_verify", "kv_attend_verify_hidden", "kv_attend_decode",
     "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kv_page_export", "kv_page_import", "kv_attend_split", "kv_attend_merge", "kv_attend_decode_static",
-    "kvx_debug_attend_paths", "kvx_decode_plan", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
+    "kvx_debug_attend_paths", "kvx_calibrate_stream", "kvx_decode_plan", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
     "kvx_prefix_chain", "kvx_prefix_retain_active", "kvx_prefix_release_active",
     "kvx_prefix_touch", "kvx_prefix_eviction_candidate", "kvx_prefix_erase",
@@ -191,6 +191,7 @@ def _declare(L):
     L.kvx_block_image_identity.argtypes = [u64, u32, vp, u32, PU64, PU64]
     L.kvx_block_image_identity.restype = None
     L.kvx_debug_attend_paths.argtypes, L.kvx_debug_attend_paths.restype = [PU64, PU64], None
+    L.kvx_calibrate_stream.argtypes = [vp, u32, vp, u32, u32, u32, vp, vp]
     L.kvx_decode_plan.argtypes = [vp, u32, u32, u32, vp]
     L.kvx_verify_plan.argtypes = [vp, u32, u32, u32, u32, u32, vp]
     L.kvx_tree_masks.argtypes = [vp, u32, vp]

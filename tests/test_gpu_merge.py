@@ -96,3 +96,36 @@ def test_split_then_merge_is_the_verify_call(fmt):
     torch.cuda.synchronize()
     assert torch.equal(one, two)
     tw.close()
+
+
+@pytest.mark.gpu
+def test_calibration_stream_runs_and_rejects_what_it_does_not_cover():
+    """kvx_calibrate_stream: the int4 decode kernel's loads alone.  It has no output to compare;
+    the test is that it runs to completion over a shuffled table with every grouping of heads,
+    leaves its sink word alone, and refuses other formats and head groupings."""
+    L = kvx.lib()
+    twin = Gp.Twin(kvx.INT4, 4, 256, 2, 40)
+    try:
+        pages = twin.pages(37, seed=5)
+        _, table = twin.tables(pages)
+        sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+        for heads in (1, 2, 4):
+            for per in (1, 5, 64):
+                assert L.kvx_calibrate_stream(twin.dev.h, 1, table.data_ptr(), len(pages), per, heads,
+                                              sink.data_ptr(), None) == 0
+        torch.cuda.synchronize()
+        assert int(sink.item()) == 0
+        assert L.kvx_calibrate_stream(twin.dev.h, 1, table.data_ptr(), len(pages), 4, 3,
+                                      sink.data_ptr(), None) == -1
+        assert L.kvx_calibrate_stream(twin.dev.h, 2, table.data_ptr(), len(pages), 4, 1,
+                                      sink.data_ptr(), None) != 0
+    finally:
+        twin.close()
+    other = Gp.Twin(kvx.BF16, 4, 256, 1, 8)
+    try:
+        _, table = other.tables(other.pages(4, seed=1))
+        sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+        assert L.kvx_calibrate_stream(other.dev.h, 0, table.data_ptr(), 4, 2, 1, sink.data_ptr(),
+                                      None) == -1
+    finally:
+        other.close()
