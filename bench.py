@@ -441,7 +441,10 @@ def qkv_prepare(args):
                                                        queries, stride, tables, cp, rows))
         store = timed(lambda layer: kvx.append(storage, layer, chunk_k, chunk_v, tables, cp,
                                                H * stride * D))
-        moved = lanes * tokens * (width * 2 + 2 * pairs * 4 + QH * D * 2 + BYTES_PER_TOKEN_LAYER)
+        # what the kernel has to move per row: the query, key and value parts of the packed
+        # row (the gate halves belong to the attention epilogue and are not read here), the
+        # rotation, the prepared queries and the page bytes
+        moved = lanes * tokens * ((QH + 2 * H) * D * 2 + 2 * pairs * 4 + QH * D * 2 + BYTES_PER_TOKEN_LAYER)
         return fused, store, moved
 
     chunk_ms, chunk_store_ms, chunk_bytes = case(1, 16384, 2048)

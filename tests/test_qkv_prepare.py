@@ -231,6 +231,20 @@ def test_prefill_chunk_prepared_and_stored(fmt):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("fmt", FORMATS)
+def test_long_chunks_of_unequal_lanes(fmt):
+    """More than 32 768 (row, head) tasks in one call, lanes of very different length (so
+    the kernel finds a task's lane by walking the lane records), a task count that is no
+    multiple of a workgroup's four."""
+    fused_case(fmt, 4, 6, 256, 32, True, 1, [77, 1000], [1230, 37], 1230, 1248, seed=211)
+
+
+@pytest.mark.gpu
+def test_long_chunk_of_a_narrower_head():
+    fused_case(ko.INT4, 8, 4, 128, 64, False, 2, [5], [1030], 1030, 1056, seed=213)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("fmt", [ko.INT4, ko.BF16])
 @pytest.mark.parametrize("heads,group,dim,pairs,norm", [(2, 8, 128, 64, 0), (8, 4, 64, 32, 2)])
 def test_other_head_dimensions(fmt, heads, group, dim, pairs, norm):
