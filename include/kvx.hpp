@@ -288,6 +288,21 @@ private:
   kvx_pool *pool_ = nullptr;
 };
 
+// runtime/engine/cache/KvCache.hpp:25-32, KvCache.cpp:29-52: what the images that overlap
+// tokens [blockBegin, blockBegin + blockTokens) add to that block's cache key.
+using ImageSpan = kvx_image_span;
+struct ImageIdentity final {
+  uint64_t lo = 0, hi = 0;
+  bool operator==(const ImageIdentity &o) const noexcept { return lo == o.lo && hi == o.hi; }
+};
+inline ImageIdentity blockImageIdentity(uint64_t blockBegin, uint32_t blockTokens,
+                                        const std::vector<ImageSpan> &spans) noexcept {
+  ImageIdentity identity;
+  kvx_block_image_identity(blockBegin, blockTokens, spans.data(), static_cast<uint32_t>(spans.size()),
+                           &identity.lo, &identity.hi);
+  return identity;
+}
+
 }  // namespace engine
 
 namespace ops {
@@ -531,6 +546,23 @@ public:
       check(kv_attend_verify(storage.handle(), layer, plan.queryHeads, buffers.queries, buffers.output,
                              buffers.pageTables, lanes.data(), plan.lanes, buffers.treeMasks,
                              kv::kVerifyChunkStride, buffers.workspace, buffers.workspaceBytes, stream));
+  }
+  // attend() of a decode plan for callers that cannot bring a workspace or allocate one (graph
+  // capture, tight serving loops): partial rows go to the library's static device array
+  // (kv_attend_decode_static, at most KVX_STATIC_WORKSPACE_BYTES; no counterpart in the
+  // reference).  Calls that overlap on one GPU race on that array.
+  static void attendStatic(void *stream, const kv::PageStorage &storage, uint32_t layer,
+                           const PagedVerifyBuffers &buffers,
+                           const std::vector<kv::ChunkedPrefillParams> &chunks,
+                           const VerifyAttentionPlan &plan) {
+    if (plan.rowCapacity != 1 || chunks.size() != plan.lanes)
+      throw std::invalid_argument("the static workspace serves decode plans, one chunk per lane");
+    std::vector<kv::VerifyAttentionParams> lanes(plan.lanes);
+    for (uint32_t i = 0; i < plan.lanes; ++i)
+      lanes[i] = {chunks[i].committed_tokens, chunks[i].page_table_entries, {}, plan.laneSplits[i],
+                  plan.splits, 1, 1, plan.scoreScale};
+    check(kv_attend_decode_static(storage.handle(), layer, plan.queryHeads, buffers.queries,
+                                  buffers.output, buffers.pageTables, lanes.data(), plan.lanes, 1, stream));
   }
   // One-row decode of up to 16 lanes whose page tables begin with the same sharedPages pages:
   // those pages are attended once for all of them (no counterpart in the reference, which lists

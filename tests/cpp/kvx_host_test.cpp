@@ -132,6 +132,23 @@ void testPlans() {
       [&] { (void)ops::PagedAttention::verifyPlan(1, 24, {16, 4, 256, Format::Float8E4M3}, {0}, true); }));
 }
 
+// dev/tests/engine/kv_page_cache_test.cpp:44-69: what images add to a block's key.
+void testImageIdentity() {
+  using engine::ImageSpan;
+  const ImageSpan red{8, 16, 8, 8, 0x1111, 0x2222}, blue{8, 16, 8, 8, 0x3333, 0x4444};
+  const ImageSpan redLater{40, 16, 8, 8, 0x1111, 0x2222}, first{0, 8, 4, 8, 0x5555, 0x6666};
+  const engine::ImageIdentity none;
+  EXPECT(engine::blockImageIdentity(0, 32, {}) == none);              // text only
+  EXPECT(engine::blockImageIdentity(32, 32, {red}) == none);          // a block after the image
+  const auto r = engine::blockImageIdentity(0, 32, {red}), b = engine::blockImageIdentity(0, 32, {blue});
+  EXPECT(!(r == none) && !(r == b));                                  // the content digest counts
+  EXPECT(!(engine::blockImageIdentity(32, 32, {redLater}) == r));     // so does the block's alignment
+  const std::vector<ImageSpan> three{first, blue, redLater};          // only overlapping spans count
+  EXPECT(engine::blockImageIdentity(32, 32, three) == engine::blockImageIdentity(32, 32, {redLater}));
+  EXPECT(engine::blockImageIdentity(0, 8, three) == engine::blockImageIdentity(0, 8, {first}));
+  EXPECT(!(engine::blockImageIdentity(0, 32, three) == engine::blockImageIdentity(0, 32, {first})));
+}
+
 void testParams() {
   const auto p = ops::PagedAttention::prefillParams(4093, 77, 96, 131);
   EXPECT(p.committed_tokens == 4093 && p.chunk_tokens == 77 && p.chunk_stride == 96);
@@ -328,6 +345,18 @@ void testAppendDecodeSingleToken() {
     hip(hipDeviceSynchronize());
     hip(hipMemcpy(two.data(), outputDevice, two.size() * 2, hipMemcpyDeviceToHost));
     EXPECT(one == two);
+    // the same attention over the library's static workspace, no buffer of the caller's
+    {
+      std::vector<uint16_t> three(queries.size());
+      ops::PagedVerifyBuffers bare = buffers;
+      bare.workspace = nullptr;
+      bare.workspaceBytes = 0;
+      hip(hipMemset(outputDevice, 0x5A, three.size() * 2));
+      ops::PagedAttention::attendStatic(nullptr, storage, 1, bare, {chunk}, plan);
+      hip(hipDeviceSynchronize());
+      hip(hipMemcpy(three.data(), outputDevice, three.size() * 2, hipMemcpyDeviceToHost));
+      EXPECT(three == two);
+    }
     bool moved = false;  // and the second token did change the result
     for (size_t i = 0; i < one.size(); ++i) moved = moved || f32(one[i]) != 0.5f * (i / (G * D) + 1) * (float(i % D % 15) - 7.0f);
     EXPECT(moved);
@@ -438,6 +467,7 @@ int main(int argc, char **argv) {
   testByteAccounting();
   testPlans();
   testParams();
+  testImageIdentity();
   if (mode == "device") {
     testStorageLifecycle();
     testPoolCompaction();

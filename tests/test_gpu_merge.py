@@ -98,6 +98,46 @@ def test_split_then_merge_is_the_verify_call(fmt):
     tw.close()
 
 
+def test_decode_call_is_split_then_merge():
+    """kv_attend_decode over a mixed batch gives the bits of kv_attend_split followed by
+    kv_attend_merge: lanes of one split (written by the split call), of two to 32, more than 32
+    lanes (several launches), repeated calls over a dirty workspace, and three streams at
+    once."""
+    H, G = A.H, A.G
+    rng = np.random.default_rng(7)
+    committed = [int(c) for c in rng.integers(1, 3000, 40)] + [0, 31, 32, 1023, 1024, 2047]
+    tw, counts, hts, dts = A.shared_pool_lanes(ko.INT4, committed, 1, seed=143)
+    lanes = len(committed)
+    q = A.queries((lanes, H, 1, G, D), 17)
+    splits = [min(max(1, counts[i] // (1 + i % 5)), 40) for i in range(lanes)]
+    dp = [kvx.VerifyParams(committed[i], counts[i], kvx.KvLayer(), splits[i], splits[i], 1, 1, 0.0)
+          for i in range(lanes)]
+    ws_bytes = kvx.attend_workspace_bytes(tw.dev, dp, H * G)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    want = torch.full((lanes, H, 1, G, D), 0x5A5A, dtype=torch.int16, device="cuda")
+    kvx.attend_split(tw.dev, 1, H * G, Gp.dev(q), dts, dp, None, 1, ws)
+    kvx.attend_merge(tw.dev, H * G, want, dp, 1, ws)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        ws.fill_(0xA5)
+        got = torch.full_like(want, 0x5A5A)
+        kvx.attend_decode(tw.dev, 1, H * G, Gp.dev(q), got, dts, dp, 1, ws)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    spaces = [torch.empty(ws_bytes, dtype=torch.uint8, device="cuda") for _ in streams]
+    outs = [torch.full_like(want, 0x5A5A) for _ in streams]
+    qd = Gp.dev(q)
+    torch.cuda.synchronize()
+    for turn in range(4):
+        for s, space, out in zip(streams, spaces, outs):
+            kvx.attend_decode(tw.dev, 1, H * G, qd, out, dts, dp, 1, space, stream=s.cuda_stream)
+    torch.cuda.synchronize()
+    for out in outs:
+        assert torch.equal(out, want)
+    tw.close()
+
+
 @pytest.mark.gpu
 def test_calibration_stream_runs_and_rejects_what_it_does_not_cover():
     """kvx_calibrate_stream: the int4 decode kernel's loads alone.  It has no output to compare;
