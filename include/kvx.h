@@ -305,7 +305,14 @@ int kvx_pool_reclaim_empty(kvx_pool *pool, int keep_runway, uint32_t limit, uint
 /* KvPool::compactExtent (KvPool.cpp:165-230): empties the sparsest extent into
    the fullest others through kv_page_copy on `stream`.  *moved_pages = 0 when
    nothing moved; otherwise *first_page and destinations[extent_pages] say where
-   each page of the emptied extent went (KvPageMoves, KvPool.hpp:39-52). */
+   each page of the emptied extent went (KvPageMoves, KvPool.hpp:39-52).
+   The reference copies on the host before it returns; here the copies are only
+   enqueued when the call returns, while the emptied extent's pages are already free
+   and the receiving pages already held.  Whatever may write a page of the emptied
+   extent (an append into a page acquired after this call) or read a receiving page
+   must therefore be ordered after `stream` has passed this point: the same stream, or
+   an event recorded on it.  kvx_pool_reclaim_empty frees memory with hipFree, which
+   waits for the device. */
 int kvx_pool_compact_extent(kvx_pool *pool, const uint32_t *fixed, uint32_t n_fixed,
                             uint32_t *first_page, uint32_t *destinations,
                             uint32_t *moved_pages, void *stream);
@@ -409,7 +416,8 @@ int kvx_sequence_ensure_writable(kvx_sequences *sequences, uint64_t id, uint64_t
 int kvx_sequence_publish(kvx_sequences *sequences, uint64_t id, const uint32_t *tokens,
                          uint64_t n_tokens, uint32_t committed_tokens);
 int kvx_sequence_view(const kvx_sequences *sequences, uint64_t id, kvx_sequence_pages *out);
-/* Cache::compactExtent: kvx_pool_compact_extent, then blocks and sequences follow their pages. */
+/* Cache::compactExtent: kvx_pool_compact_extent (with its ordering rule for `stream`), then
+   blocks and sequences follow their pages. */
 int kvx_sequences_compact_extent(kvx_sequences *sequences, uint32_t *first_page,
                                  uint32_t *destinations, uint32_t *moved_pages, void *stream);
 
