@@ -176,12 +176,17 @@ struct Sight {
 // in split order by one wave, as the reference does; longer lists (small
 // batches over long contexts) are cut into kMergeWaves consecutive ranges, one
 // per wave, each summed in split order, and the ranges are then added in range
-// order.
+// order.  Eight ranges (two waves per SIMD, so a wave may hold 20 partial rows in
+// registers): a range of a list of up to 160 splits is requested at once, statistics
+// and partial rows together, and the merge costs little more than one round trip to
+// memory; longer lists take one more per 20 splits of a range.
 constexpr uint32_t kMergeSequential = 32;
-constexpr uint32_t kMergeWaves = 4;
-// Partial rows a wave has in flight at a time: a list of up to 16 splits (the
-// average of a mixed batch at 32 pages per split) costs one load latency.
+constexpr uint32_t kMergeWaves = 8;
+// Partial rows a wave has in flight at a time.  One wave per row (lists of up to
+// kMergeSequential splits): 16, the average list of a mixed batch at 32 pages per split.
+// A wave of the ranged form: 20, which is what two waves per SIMD leave registers for.
 constexpr uint32_t kMergeAhead = 16;
+constexpr uint32_t kMergeAheadRanged = 20;
 
 struct MergeSums {
   f32x4 numerator;
@@ -189,20 +194,35 @@ struct MergeSums {
 };
 
 // Sums splits [first, last) of the row in split order; `maximum` is the row's
-// maximum over all splits.  With PREFETCHED, `early` holds the partial rows of
-// the first kMergeAhead splits (clamped to the last), loaded before the caller
-// waited for the statistics.
-template <bool PREFETCHED>
+// maximum over all splits.  `early` holds the partial rows of the range's first
+// kMergeAhead splits (clamped to the last) and `early_stat` the statistics of split
+// first + lane, loaded before the caller waited for anything.
+template <uint32_t AHEAD>
 __device__ __forceinline__ MergeSums merge_range(const float *__restrict__ partials,
                                                  const float *__restrict__ statistics,
                                                  uint64_t first_row, uint32_t first, uint32_t last,
                                                  uint32_t M, float maximum, uint32_t lane,
-                                                 const f32x4 (&early)[kMergeAhead], f32x2 early_stat) {
+                                                 const f32x4 (&early)[AHEAD], f32x2 early_stat) {
   MergeSums sums{{0.0f, 0.0f, 0.0f, 0.0f}, 0.0f};
+  // One batch of up to AHEAD splits from `base + i` on, in split order; the weights
+  // and terms of the 64 splits from `base` on sit one per lane.
+  const auto add_batch = [&](const f32x4 (&part)[AHEAD], uint32_t i, uint32_t count,
+                             float my_weight, float my_term) {
+#pragma unroll
+    for (uint32_t u = 0; u < AHEAD; ++u) {
+      if (i + u < count) {
+        const float weight = __shfl(my_weight, i + u);
+#pragma unroll
+        for (uint32_t c = 0; c < 4; ++c)
+          sums.numerator[c] = __fadd_rn(sums.numerator[c], __fmul_rn(weight, part[u][c]));
+        sums.denominator = __fadd_rn(sums.denominator, __shfl(my_term, i + u));
+      }
+    }
+  };
   for (uint32_t base = first; base < last; base += 64) {
     const uint32_t mine = base + lane;
     f32x2 stat = {-INFINITY, 0.0f};
-    if (PREFETCHED && base == first) {
+    if (base == first) {
       stat = early_stat;
     } else if (mine < last) {
       stat = load_global<f32x2>(statistics + (first_row + uint64_t(mine) * M) * 2);
@@ -210,35 +230,29 @@ __device__ __forceinline__ MergeSums merge_range(const float *__restrict__ parti
     const float my_weight = expf(__fsub_rn(stat[0], maximum));
     const float my_term = __fmul_rn(my_weight, stat[1]);
     const uint32_t count = min(64u, last - base);
-    for (uint32_t i = 0; i < count; i += kMergeAhead) {
-      f32x4 part[kMergeAhead];
+    uint32_t i = 0;
+    if (base == first) {  // the batch that was requested ahead
+      add_batch(early, 0, count, my_weight, my_term);
+      i = AHEAD;
+    }
+    for (; i < count; i += AHEAD) {
+      f32x4 part[AHEAD];
 #pragma unroll
-      for (uint32_t u = 0; u < kMergeAhead; ++u) {
-        if (PREFETCHED && base == first && i == 0) {
-          part[u] = early[u];
-        } else {
-          const uint64_t row = first_row + uint64_t(base + min(i + u, count - 1)) * M;
-          part[u] = load_global<f32x4>(partials + row * kD + 4 * lane);
-        }
+      for (uint32_t u = 0; u < AHEAD; ++u) {
+        const uint64_t row = first_row + uint64_t(base + min(i + u, count - 1)) * M;
+        part[u] = load_global<f32x4>(partials + row * kD + 4 * lane);
       }
-#pragma unroll
-      for (uint32_t u = 0; u < kMergeAhead; ++u) {
-        if (i + u < count) {
-          const float weight = __shfl(my_weight, i + u);
-#pragma unroll
-          for (uint32_t c = 0; c < 4; ++c)
-            sums.numerator[c] = __fadd_rn(sums.numerator[c], __fmul_rn(weight, part[u][c]));
-          sums.denominator = __fadd_rn(sums.denominator, __shfl(my_term, i + u));
-        }
-      }
+      add_batch(part, i, count, my_weight, my_term);
     }
   }
   return sums;
 }
 
-// grid (fused query row, KV head, lane), kMergeWaves waves per row.  Lanes whose
-// pages fit one split were written by the split kernel itself.
-__global__ __launch_bounds__(64 * kMergeWaves) void matrix_merge_kernel(
+// grid (fused query row, KV head, lane), WAVES waves per row: one for launches whose
+// longest list has at most kMergeSequential splits, else kMergeWaves.  Lanes whose pages
+// fit one split were written by the split kernel itself.
+template <uint32_t WAVES, uint32_t AHEAD>
+__global__ __launch_bounds__(64 * WAVES) void matrix_merge_kernel(
     uint16_t *__restrict__ output, const float *__restrict__ partials,
     const float *__restrict__ statistics, DecodeArgs a) {
   const uint32_t j = blockIdx.x, head = blockIdx.y;
@@ -271,49 +285,47 @@ __global__ __launch_bounds__(64 * kMergeWaves) void matrix_merge_kernel(
                                hidden_row * (2ull * a.kv_heads * G + 2ull * a.kv_heads) * kD +
                                uint64_t(query_head) * 2 * kD + kD + 4 * lane);
   const uint64_t first_row = l.row_base + uint64_t(head) * l.split_count * M + j;
-  const bool sequential = written <= kMergeSequential;
+  const bool sequential = WAVES == 1 || written <= kMergeSequential;
   if (sequential && wave) return;
-  // The sequential case (at most kMergeSequential splits) issues its statistics and the
-  // first kMergeAhead partial rows together, before anything waits.
-  f32x4 early[kMergeAhead];
+  // A wave's range of the list: all of it for the sequential case (at most kMergeSequential
+  // splits), else one of kMergeWaves consecutive shares (at most 32 splits of 512).  Its
+  // statistics and its first kMergeAhead partial rows are requested together, before
+  // anything waits.
+  const uint32_t share = sequential ? written : (written + WAVES - 1) / WAVES;
+  const uint32_t first = min(written, wave * share), last = min(written, first + share);
+  const uint32_t count = last - first;
+  f32x4 early[AHEAD];
   f32x2 early_stat = {-INFINITY, 0.0f};
-  float maximum = -INFINITY;
-  if (sequential) {
-    if (lane < written)
-      early_stat = load_global<f32x2>(statistics + (first_row + uint64_t(lane) * M) * 2);
+  if (lane < count)
+    early_stat = load_global<f32x2>(statistics + (first_row + uint64_t(first + lane) * M) * 2);
 #pragma unroll
-    for (uint32_t u = 0; u < kMergeAhead; ++u)
-      early[u] = load_global<f32x4>(partials + (first_row + uint64_t(min(u, written - 1)) * M) * kD +
-                                    4 * lane);
-    maximum = early_stat[0];
-    for (int offset = 32; offset; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset));
-  } else {
-    for (uint32_t base = 0; base < written; base += 64) {
-      const uint32_t s = base + lane;
-      float m = s < written ? load_global<float>(statistics + (first_row + uint64_t(s) * M) * 2)
-                            : -INFINITY;
-      for (int offset = 32; offset; offset >>= 1) m = fmaxf(m, __shfl_xor(m, offset));
-      maximum = fmaxf(maximum, m);
-    }
+  for (uint32_t u = 0; u < AHEAD; ++u)
+    early[u] = count ? load_global<f32x4>(partials +
+                                          (first_row + uint64_t(first + min(u, count - 1)) * M) * kD +
+                                          4 * lane)
+                     : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  float maximum = early_stat[0];
+  for (int offset = 32; offset; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset));
+  __shared__ float maxima[WAVES];
+  __shared__ f32x4 numerators[WAVES][64];
+  __shared__ float denominators[WAVES][64];
+  if (!sequential) {  // the row's maximum is the largest of the ranges' maxima
+    if (lane == 0) maxima[wave] = maximum;
+    __syncthreads();
+#pragma unroll
+    for (uint32_t w = 0; w < WAVES; ++w) maximum = fmaxf(maximum, maxima[w]);
   }
-  MergeSums sums;
-  if (sequential) {
-    sums = merge_range<true>(partials, statistics, first_row, 0, written, M, maximum, lane, early,
-                             early_stat);
-  } else {
-    const uint32_t share = (written + kMergeWaves - 1) / kMergeWaves;
-    const uint32_t first = min(written, wave * share), last = min(written, first + share);
-    const MergeSums mine = merge_range<false>(partials, statistics, first_row, first, last, M,
-                                              maximum, lane, early, early_stat);
-    __shared__ f32x4 numerators[kMergeWaves][64];
-    __shared__ float denominators[kMergeWaves][64];
-    numerators[wave][lane] = mine.numerator;
-    denominators[wave][lane] = mine.denominator;
+  MergeSums sums{{0.0f, 0.0f, 0.0f, 0.0f}, 0.0f};
+  if (count)
+    sums = merge_range<AHEAD>(partials, statistics, first_row, first, last, M, maximum, lane, early,
+                              early_stat);
+  if (!sequential) {
+    numerators[wave][lane] = sums.numerator;
+    denominators[wave][lane] = sums.denominator;
     __syncthreads();
     if (wave) return;
-    sums = mine;
 #pragma unroll
-    for (uint32_t w = 1; w < kMergeWaves; ++w) {
+    for (uint32_t w = 1; w < WAVES; ++w) {
       const f32x4 other = numerators[w][lane];
 #pragma unroll
       for (uint32_t c = 0; c < 4; ++c) sums.numerator[c] = __fadd_rn(sums.numerator[c], other[c]);
@@ -432,11 +444,15 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       if (e != hipSuccess) return hip_fail(e, name);
     }
     if ((max_splits > 1 || epilogue) && run_merge) {
-      // One wave per row is all the sequential merge uses; the other three only
-      // join in for lists longer than kMergeSequential.
-      const uint32_t merge_threads = max_splits <= kMergeSequential ? 64 : 64 * kMergeWaves;
-      hipLaunchKernelGGL(matrix_merge_kernel, dim3(M, H, a.n_lanes), dim3(merge_threads), 0,
-                         stream, static_cast<uint16_t *>(output), partials, statistics, a);
+      // One wave per row where every list of the launch is short; else the ranged form,
+      // whose first wave alone sums the short lists among them.
+      if (max_splits <= kMergeSequential)
+        hipLaunchKernelGGL((matrix_merge_kernel<1, kMergeAhead>), dim3(M, H, a.n_lanes), dim3(64), 0,
+                           stream, static_cast<uint16_t *>(output), partials, statistics, a);
+      else
+        hipLaunchKernelGGL((matrix_merge_kernel<kMergeWaves, kMergeAheadRanged>), dim3(M, H, a.n_lanes),
+                           dim3(64 * kMergeWaves), 0, stream, static_cast<uint16_t *>(output), partials,
+                           statistics, a);
       const hipError_t e = hipGetLastError();
       if (e != hipSuccess) return hip_fail(e, "matrix_merge_kernel");
     }

@@ -195,7 +195,8 @@ def test_hot_kernels_stay_out_of_scratch_memory():
         assert len(names) == 1, (fragment, names)
         return report[names[0]]
 
-    for fragment in ("decode_int4_kernelE", "decode_int4_tiles_kernel", "verify_int4_kernel", "matrix_merge_kernel",
+    for fragment in ("decode_int4_kernelE", "decode_int4_tiles_kernel", "verify_int4_kernel",
+                     "matrix_merge_kernelILj1E", "matrix_merge_kernelILj8E",   # one wave per row; ranged
                      "attend_wide_kernelILj1ELj1ELj2ELb0E",    # int8, one block, two waves per SIMD
                      "attend_wide_kernelILj4ELj1ELj2ELb0E",    # fp8
                      "attend_wide_kernelILj2ELj1ELj1ELb0E",    # bf16 decode

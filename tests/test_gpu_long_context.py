@@ -85,7 +85,7 @@ def test_long_history_verify_decode_and_prefill(history):
         check_row(got[lane, head, row, g], want, want32, f"long verify {history} {lane, head, row, g}",
                   dict(kv_heads=H, group=G, head_dim=D, **args))
 
-    # ---- decode: one row, the decode plan (hundreds of splits, merged in four ranges) ----
+    # ---- decode: one row, the decode plan (hundreds of splits, merged in eight ranges) ----
     q1 = np.zeros((1, H, 1, G, D), dtype=np.uint16)
     q1[0, :, 0] = q[2, :, 0]
     splits = kvx.decode_plan([history], H, FMT)[0]

@@ -2,7 +2,7 @@
 statistics -- maxima up to 2000 apart, so that weights underflow, next to fractional ones,
 ragged sums, inactive rows -- and compared with the fp64 merge at the reference's bound
 |got - want| <= 0.004 |want| + 2e-6 (dev/tests/engine/q8_flash_attention_metal_test.mm:648-725).
-One to 512 splits: up to 32 are summed in split order by one wave, more in four ordered ranges.
+One to 512 splits: up to 32 are summed in split order by one wave, more in eight ordered ranges.
 The same rows through kv_attend_split + kv_attend_merge must give kv_attend_verify's bits."""
 import numpy as np
 import pytest
