@@ -147,6 +147,7 @@ struct PrepareArgs {
   uint32_t rows;        // rows per lane in packed / rope_cos / rope_sin
   uint32_t row_stride;  // rows between KV heads in the queries
   float eps;
+  uint32_t group_magic;  // ceil(2^32 / group): head / group = mulhi(head, group_magic) for head < 2^16
 };
 
 template <uint32_t FMT>
@@ -268,6 +269,21 @@ __device__ __forceinline__ void load_floats(const float *from, float (&out)[E]) 
 // lane exchanges, smaller ones pair a lane's own elements), then the groups in
 // order; the results are the same bits.  Needs rotary_pairs / E to be a power
 // of two, so that a pair's two dimensions sit rotary_pairs / E lanes apart.
+// x of the lane `offset` lanes away (offset a power of two below 32) through the LDS
+// crossbar's fixed patterns: no address register and no address arithmetic.
+template <uint32_t OFFSET>
+__device__ __forceinline__ float lane_xor(float x) {
+  static_assert(OFFSET && OFFSET < 32 && !(OFFSET & (OFFSET - 1)), "a power of two below 32");
+  return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(x), int((OFFSET << 10) | 0x1f)));
+}
+// bf16 (round to nearest even) of a finite value in one instruction; a NaN stays a NaN.
+__device__ __forceinline__ uint16_t f32_to_bf16_hw(float f) {
+  typedef float f32x2v __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
+  const f32x2v pair = {f, 0.0f};
+  return uint16_t(__builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2v)));
+}
+
 template <uint32_t FMT, uint32_t E>
 __device__ __forceinline__ void store_row_wave(const uint16_t (&source)[E], bool value_tensor,
                                                const Slab &s, uint32_t slot, uint32_t lane,
@@ -292,7 +308,12 @@ __device__ __forceinline__ void store_row_wave(const uint16_t (&source)[E], bool
       v[e] = bf16_to_f32(source[e]);
       m = fmaxf(m, fabsf(v[e]));
     }
-    for (int offset = 32; offset; offset >>= 1) m = fmaxf(m, __shfl_xor(m, offset));
+    m = fmaxf(m, __shfl_xor(m, 32));
+    m = fmaxf(m, lane_xor<16>(m));
+    m = fmaxf(m, lane_xor<8>(m));
+    m = fmaxf(m, lane_xor<4>(m));
+    m = fmaxf(m, lane_xor<2>(m));
+    m = fmaxf(m, lane_xor<1>(m));
     const float maximum = m;
     constexpr float qmax = FMT == KVX_FMT_INT4 ? 7.0f : FMT == KVX_FMT_INT8 ? 127.0f : 448.0f;
     const float scale = maximum == 0.0f ? 0.0f : __fdiv_rn(maximum, qmax);
@@ -339,28 +360,23 @@ __device__ __forceinline__ void store_row_wave(const uint16_t (&source)[E], bool
   }
 }
 
+// grid (blocks of four head tasks, row, lane): a wave is one (row, head) task, and which
+// one it is comes from the block's coordinates without a division or a walk over the
+// lane records.  Head tasks 0 .. QH - 1 are the query heads, QH .. QH + H - 1 the KV heads.
 template <uint32_t FMT, uint32_t E>
 __global__ __launch_bounds__(256) void prepare_append_wave_kernel(PrepareArgs p) {
 #pragma clang fp contract(off)
   constexpr uint32_t D = 64 * E;
   const AppendArgs &a = p.append;
-  const uint32_t task_id = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
-  uint32_t li = 0;
-  if (a.uniform_groups) {  // every lane has as many tasks: no walk over the lane records
-    li = min(task_id / a.uniform_groups, a.n_lanes - 1);
-  } else {
-    for (uint32_t i = 1; i < a.n_lanes; ++i)
-      if (task_id >= a.lane[i].group_base) li = i;
-  }
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t task = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t row = blockIdx.y, li = blockIdx.z;
   const AppendLane &l = a.lane[li];
   if (!append_contract(l, a)) return;
   const uint32_t H = a.kv_heads, QH = p.query_heads, G = QH / H;
-  const uint32_t local = task_id - l.group_base;
-  if (local >= l.tokens * (QH + H)) return;
-  const bool query = local < l.tokens * QH;
-  const uint32_t local_task = query ? local : local - l.tokens * QH;
-  const uint32_t heads = query ? QH : H;
-  const uint32_t row = local_task / heads, head = local_task % heads;
+  if (row >= l.tokens || task >= QH + H) return;
+  const bool query = task < QH;
+  const uint32_t head = query ? task : task - QH;
   const uint32_t d0 = E * lane;
   const uint32_t q_stride = p.query_gate ? 2 * D : D;
   const uint64_t packed_stride = uint64_t(QH) * q_stride + 2ull * H * D;
@@ -399,9 +415,12 @@ __global__ __launch_bounds__(256) void prepare_append_wave_kernel(PrepareArgs p)
     for (uint32_t e = 0; e < E; ++e) sum[e] = element[e] * element[e];
     // dimension offsets 16 .. E: the partner sits offset / E lanes away
 #pragma unroll
-    for (uint32_t offset = 16; offset >= E; offset >>= 1) {
-#pragma unroll
-      for (uint32_t e = 0; e < E; ++e) sum[e] = sum[e] + __shfl_xor(sum[e], int(offset / E));
+    for (uint32_t e = 0; e < E; ++e) {
+      sum[e] = sum[e] + lane_xor<16 / E>(sum[e]);
+      if constexpr (8 >= E) sum[e] = sum[e] + lane_xor<(8 >= E ? 8 / E : 1)>(sum[e]);
+      if constexpr (4 >= E) sum[e] = sum[e] + lane_xor<(4 >= E ? 4 / E : 1)>(sum[e]);
+      if constexpr (2 >= E) sum[e] = sum[e] + lane_xor<(2 >= E ? 2 / E : 1)>(sum[e]);
+      if constexpr (1 >= E) sum[e] = sum[e] + lane_xor<1>(sum[e]);
     }
     // dimension offsets below E pair the lane's own elements
     float group_sum;
@@ -416,7 +435,8 @@ __global__ __launch_bounds__(256) void prepare_append_wave_kernel(PrepareArgs p)
     // the groups of 32 dimensions in order; a group spans 32 / E lanes
     float total = 0.0f;
 #pragma unroll
-    for (uint32_t g = 0; g < D / 32; ++g) total = total + __shfl(group_sum, int(g * (32 / E)));
+    for (uint32_t g = 0; g < D / 32; ++g)
+      total = total + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(group_sum), int(g * (32 / E))));
     const float mean = total / float(D);
     inverse = 1.0f / sqrtf(mean + p.eps);
   }
@@ -424,14 +444,14 @@ __global__ __launch_bounds__(256) void prepare_append_wave_kernel(PrepareArgs p)
 #pragma unroll
   for (uint32_t e = 0; e < E; ++e) {
     const float unit = element[e] * inverse;
-    const uint16_t normal = f32_to_bf16(unit * scale[e]);
+    const uint16_t normal = f32_to_bf16_hw(unit * scale[e]);
     const float mine = bf16_to_f32(normal);
     const float other = __shfl_xor(mine, int(pair_lanes));
     const float mc = mine * cosine[e], os = other * sine[e];
-    prepared[e] = rotated ? f32_to_bf16(is_first ? mc - os : mc + os) : normal;
+    prepared[e] = rotated ? f32_to_bf16_hw(is_first ? mc - os : mc + os) : normal;
   }
   if (query) {
-    const uint32_t kv_head = head / G, local_head = head % G;
+    const uint32_t kv_head = __umulhi(head, p.group_magic), local_head = head - kv_head * G;
     store_bf16s<E>(p.queries + uint64_t(li) * H * p.row_stride * G * D +
                        ((uint64_t(kv_head) * p.row_stride + row) * G + local_head) * D + d0,
                    prepared);
@@ -1402,6 +1422,7 @@ int kv_prepare_append(const kvx_storage *s, uint32_t layer, const kvx_qkv_shape 
     p.rows = rows;
     p.row_stride = row_stride;
     p.eps = shape->eps != 0.0f ? shape->eps : 1e-6f;
+    p.group_magic = uint32_t((0x100000000ull + QH / H - 1) / (QH / H));
     // One wave per task where the head dimension is 64, 128 or 256 and a rotary pair's
     // dimensions are a power-of-two number of lanes apart; else one workgroup per task.
     const uint32_t E = D / 64, pair_lanes = E ? shape->rotary_pairs / E : 0;
@@ -1411,7 +1432,9 @@ int kv_prepare_append(const kvx_storage *s, uint32_t layer, const kvx_qkv_shape 
       constexpr uint32_t F = decltype(fmt)::value;
       const hipStream_t st = static_cast<hipStream_t>(stream);
       if (by_wave) {
-        const dim3 grid((groups + 3) / 4), block(256);
+        uint32_t most_rows = 0;
+        for (uint32_t i = 0; i < a.n_lanes; ++i) most_rows = std::max(most_rows, lanes[first + i].chunk_tokens);
+        const dim3 grid((QH + H + 3) / 4, most_rows, a.n_lanes), block(256);
         if (E == 4) hipLaunchKernelGGL((prepare_append_wave_kernel<F, 4>), grid, block, 0, st, p);
         else if (E == 2) hipLaunchKernelGGL((prepare_append_wave_kernel<F, 2>), grid, block, 0, st, p);
         else hipLaunchKernelGGL((prepare_append_wave_kernel<F, 1>), grid, block, 0, st, p);
