@@ -38,8 +38,9 @@ def check_row(got_bits, want_bits, want32, label, explain):
                               explain=lambda index: explain)
 
 
-@pytest.mark.parametrize("history", [131072, 260096])
-def test_long_history_verify_decode_and_prefill(history):
+@pytest.mark.parametrize("history,FMT", [(131072, ko.INT4), (260096, ko.INT4), (131072, ko.INT8),
+                                         (131072, ko.BF16)])
+def test_long_history_verify_decode_and_prefill(history, FMT):
     rows = 257                                    # the prefill chunk; verify and decode sit inside it
     total = history + rows
     n_pages = (total + 31) // 32
@@ -82,7 +83,7 @@ def test_long_history_verify_decode_and_prefill(history):
                     head=head, committed=history, active=8, splits=splits, capacity=8,
                     fused_row=row * G + g)
         want, want32 = one_row(**args)
-        check_row(got[lane, head, row, g], want, want32, f"long verify {history} {lane, head, row, g}",
+        check_row(got[lane, head, row, g], want, want32, f"long verify fmt={FMT} {history} {lane, head, row, g}",
                   dict(kv_heads=H, group=G, head_dim=D, **args))
 
     # ---- decode: one row, the decode plan (hundreds of splits, merged in eight ranges) ----
@@ -100,7 +101,7 @@ def test_long_history_verify_decode_and_prefill(history):
         args = dict(fmt=FMT, tile_queries=q1[0, head, 0].reshape(G, D), table=th, kv=kv, head=head,
                     committed=history, active=1, splits=splits, capacity=1, fused_row=g)
         want, want32 = one_row(**args)
-        check_row(got[0, head, 0, g], want, want32, f"long decode {history} {head, g} splits={splits}",
+        check_row(got[0, head, 0, g], want, want32, f"long decode fmt={FMT} {history} {head, g} splits={splits}",
                   dict(kv_heads=H, group=G, head_dim=D, **args))
 
     # ---- chunked prefill: 257 rows, the split count sized for the GPU ----
@@ -128,7 +129,7 @@ def test_long_history_verify_decode_and_prefill(history):
                     committed=history + 8 * tile, active=min(8, rows - 8 * tile), splits=splits,
                     capacity=8, fused_row=(row % 8) * G + g)
         want, want32 = one_row(**args)
-        check_row(got[head, row, g], want, want32, f"long prefill {history} {head, row, g}",
+        check_row(got[head, row, g], want, want32, f"long prefill fmt={FMT} {history} {head, row, g}",
                   dict(kv_heads=H, group=G, head_dim=D, **args))
 
     after = kvx.attend_paths()
@@ -175,4 +176,80 @@ def test_one_split_over_a_long_history():
                     head=head, committed=history, active=1, splits=1, capacity=1, fused_row=g)
         check_row(got[0, head, 0, g], want, want32, "one split over 1251 pages",
                   dict(kv_heads=H, group=G, head_dim=D, **args))
+    tw.close()
+
+
+def fill(tw, td, n_pages, total, seed):
+    """History written by the device (bit-exactness of the append is other tests' business) and
+    mirrored into the oracle's store by its bytes."""
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    done = 0
+    while done < total:
+        n = min(2048, total - done)
+        stride = (n + 31) // 32 * 32
+        ck = torch.randn((H, stride, D), generator=gen, device="cuda").clamp_(-6, 6).bfloat16()
+        cv = torch.randn((H, D, stride), generator=gen, device="cuda").clamp_(-6, 6).bfloat16()
+        kvx.append(tw.dev, 0, ck.view(torch.int16), cv.view(torch.int16), [td],
+                   [kvx.ChunkParams(done, n, stride, n_pages)], H * stride * D)
+        done += n
+    torch.cuda.synchronize()
+    tw.download()
+
+
+@pytest.mark.parametrize("fmt", [ko.INT4, ko.INT8, ko.BF16, ko.FP8])
+@pytest.mark.parametrize("history,rows", [(0, 2048), (4093, 1057), (16383, 257), (8064, 130), (6145, 2048)])
+@pytest.mark.parametrize("planned", [False, True])
+def test_reference_prefill_cases_on_sampled_rows(fmt, history, rows, planned):
+    """The large cases of the reference's prefill list (dev/tests/engine/
+    paged_attention_plan_test.mm:1018-1029; the small ones run whole in test_gpu_attention.py):
+    full chunks, chunks that start one token before a page boundary and in the middle of a
+    page, ragged last tiles.  Sampled rows, each recomputed alone by the oracle: the chunk's
+    first and last rows, rows either side of a page boundary of the history, of a tile pair
+    and of the last, partly filled tile.  With the reference's split rule and with the
+    split count sized for the GPU."""
+    total = history + rows
+    n_pages = (total + 31) // 32
+    tw = Gp.Twin(fmt, H, D, 1, n_pages)
+    th, td = tw.tables(tw.pages(n_pages, history + rows))
+    fill(tw, td, n_pages, total, history + 7 * rows)
+    kv = tw.host.layer(0)
+    rng = np.random.default_rng(history + rows)
+    stride = (rows + 31) // 32 * 32
+    qp = np.zeros((H, stride, G, D), dtype=np.uint16)
+    qp[:, :rows] = ko.f32_to_bf16(rng.standard_normal((H, rows, G, D)).astype(np.float32)
+                                  ).reshape(H, rows, G, D)
+    splits = (kvx.prefill_plan(history, rows, H, QH, fmt) if planned
+              else kvx.lib().kvx_prefill_splits(rows))
+    out = torch.full((H, stride, G, D), 0x5A5A, dtype=torch.int16, device="cuda")
+    ws = torch.empty(kvx.prefill_workspace_bytes(tw.dev, rows, QH, splits), dtype=torch.uint8,
+                     device="cuda")
+    before = kvx.attend_paths()
+    kvx.attend_prefill(tw.dev, 0, QH, Gp.dev(qp), out, td,
+                       kvx.PrefillParams(history, rows, stride, n_pages, kvx.KvLayer(), splits, 0.0), ws)
+    torch.cuda.synchronize()
+    after = kvx.attend_paths()
+    assert after[1] == before[1] + 1 and after[0] == before[0]      # the matrix-core kernels
+    got = Gp.host_u16(out)
+    tile_end = (rows + 7) // 8 * 8
+    assert not got[:, rows:tile_end].any() and (got[:, tile_end:] == 0x5A5A).all()
+    to_boundary = (32 - history % 32) % 32          # first chunk row that starts a page
+    picks = {0, 7, 8, 15, 16, rows - 1, rows - 2, (rows - 1) // 8 * 8, rows // 2,
+             to_boundary, max(to_boundary - 1, 0), to_boundary + 31, to_boundary + 32}
+    picks = sorted(r for r in picks if 0 <= r < rows)
+    tol = 1e-2 if fmt == ko.FP8 else 2e-3
+    for i, row in enumerate(picks):
+        head, g = (i * 5 + row) % H, (i * 7 + row) % G
+        tile = row // 8
+        tile_queries = np.zeros((8, G, D), dtype=np.uint16)
+        live = qp[head, 8 * tile:min(8 * tile + 8, rows)]
+        tile_queries[:live.shape[0]] = live
+        args = dict(fmt=fmt, tile_queries=tile_queries.reshape(8 * G, D), table=th, kv=kv, head=head,
+                    committed=history + 8 * tile, active=min(8, rows - 8 * tile), splits=splits,
+                    capacity=8, fused_row=(row % 8) * G + g)
+        want, want32 = one_row(**args)
+        Gp.check_attention(got[head, row, g].reshape(1, D), want.reshape(1, D), want32.reshape(1, D),
+                           np.ones(1, dtype=bool), tol,
+                           f"reference prefill case fmt={fmt} {history}+{rows} splits={splits} "
+                           f"{head, row, g}",
+                           explain=lambda index: dict(kv_heads=H, group=G, head_dim=D, **args))
     tw.close()
