@@ -247,6 +247,35 @@ def cpu_prefill(seed, fmt_name, prefix, chunk, budget_s):
 
 
 
+def cpu_qkv_prepare(seed, budget_s):
+    """The oracle on the qkv-prepare workload's chunk, one layer: 2048 rows prepared (norm,
+    rotation, layout) and stored into int4 pages."""
+    import numpy as np
+    from oracle import kvoracle as ko
+    rng = np.random.default_rng(seed)
+    pairs, width = 32, (2 * QH + 2 * H) * D
+    rows = 2048                                                      # the whole chunk: a fraction of a second
+    n_pages = rows // 32 + 1
+    store = ko.Store(1, H, D, ko.INT4, n_pages, n_pages)
+    store.allocate(0)
+    table = store.entries(np.arange(n_pages, dtype=np.uint32))
+    bf = lambda a: ko.f32_to_bf16(a.astype(np.float32)).reshape(a.shape)
+    packed = bf(rng.standard_normal((rows, width)))
+    wq, wk = bf(rng.standard_normal(D)), bf(rng.standard_normal(D))
+    cos = rng.random((rows, pairs), dtype=np.float32)
+    sin = rng.random((rows, pairs), dtype=np.float32)
+    t0 = time.perf_counter()
+    _, k, v = ko.qkv_prepare(H, G, D, pairs, True, 1e-6, rows, rows, packed, wq, wk, cos, sin)
+    stored = ko.store_chunk(ko.INT4, H, D, k, v, table, ko.ChunkParams(0, rows, rows, n_pages, store.layer(0)))
+    spent = time.perf_counter() - t0
+    store.close()
+    assert stored == 1, "the oracle refused the qkv-prepare sample"
+    return {"value": rows / spent, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"the whole {rows}-row chunk, one layer: prepare + quantize + store, "
+                      f"{spent:.2f} s of scalar C++ oracle",
+            "seconds": spent, "rows": rows}
+
+
 def profiled_traffic():
     """HBM bytes per launch of the split kernel on this workload, from the
     committed counter summary (two rocprofv3 --pmc runs of this script, scaled by
@@ -470,6 +499,8 @@ def qkv_prepare(args):
         "cpu_baseline": None,
     }
     storage.close()
+    if args.cpu_seconds > 0:
+        result["cpu_baseline"] = cpu_qkv_prepare(args.seed, args.cpu_seconds)
     print(json.dumps(result))
 
 
@@ -574,6 +605,13 @@ def shared_prefix(args):
         "cpu_baseline": None,
     }
     storage.close()
+    if args.cpu_seconds > 0 and args.format == "int4":
+        # one sequence of the 16 (the oracle has no shared form: every sequence walks its whole table)
+        spent = cpu_lane(int(committed[0]), args.seed)
+        result["cpu_baseline"] = {
+            "value": 1.0 / spent, "unit": "sequence-steps/s", "cores": 1, "kind": "port",
+            "sample": f"one sequence of the 16 ({int(committed[0]) + 1} tokens), one layer: append 1 token + "
+                      f"decode attention over its whole table, {spent:.1f} s of scalar C++ oracle"}
     print(json.dumps(result))
 
 
