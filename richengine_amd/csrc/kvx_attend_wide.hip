@@ -478,6 +478,347 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
   }
 }
 
+
+// ---- pages shared by the four waves of a workgroup: the tiles of a chunked prefill ----
+//
+// A chunk's tiles walk the same pages, and with one wave per 32 fused rows every wave
+// fetches every page for itself: a 2048-row chunk over 16 K tokens pulls 27 GB out of the L2
+// for 0.9 TFLOP of arithmetic.  Here four waves form a workgroup per (lane of up to 32 query
+// rows, split, KV head): each fetches a quarter of the page and writes it into LDS as
+// finished MFMA operands (byte formats expanded on the way, once instead of four times),
+// and all four multiply their own fused rows with the shared copy.  Two copies alternate:
+// while a page is multiplied the next one is staged, one barrier per page; each wave keeps
+// its quarters of the pages two and three ahead in flight.  An operand read from LDS must
+// feed two row blocks: four waves reading one block's worth each would ask the LDS for
+// twice what it delivers.
+constexpr uint32_t kGroupWaves = 4;
+
+// The workgroup's barrier between pages: a wave's LDS writes are done (the LDS counter at
+// zero) before it arrives, and that is all; __syncthreads() would also wait for the global
+// loads in flight, which are the pages two and three ahead.
+__device__ __forceinline__ void group_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+struct GroupOperands {
+  u32x4 keys[2][8][64];  // [token block][dims block][lane]
+  u32x4 values[16][64];  // [dims block][lane]
+};
+template <uint32_t FMT>
+struct GroupShare {  // a wave's quarter of a page as loaded: dims blocks 2w, 2w + 1 of the keys,
+                     // dims blocks 4w .. 4w + 3 of the values
+  uint32_t k[2][2][Wide<FMT>::kDwords];  // [token block][dims block of the pair]
+  uint32_t v[4][Wide<FMT>::kDwords];
+};
+
+template <uint32_t FMT, bool REUSED>
+__device__ __forceinline__ void fetch_share(GroupShare<FMT> &r, const PagePlace &p, uint32_t wave,
+                                            uint32_t t, uint32_t g) {
+  constexpr uint32_t B = Wide<FMT>::kBytes;
+#pragma unroll
+  for (uint32_t tb = 0; tb < 2; ++tb) {
+    const uint8_t *row = p.keys + (8 * (t >> 2) + 4 * tb + (t & 3)) * kD * B;
+    if constexpr (Wide<FMT>::kByte) {
+      const u32x4 x = load_streaming<u32x4, REUSED>(row + 64 * wave + 16 * g);  // dims blocks 2w, 2w + 1
+      r.k[tb][0][0] = x[0], r.k[tb][0][1] = x[1], r.k[tb][1][0] = x[2], r.k[tb][1][1] = x[3];
+    } else {
+#pragma unroll
+      for (uint32_t c = 0; c < 2; ++c) {
+        const u32x4 x = load_streaming<u32x4, REUSED>(row + key_dims<FMT>(2 * wave + c, g) * B);
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) r.k[tb][c][i] = x[i];
+      }
+    }
+  }
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i) {
+    const uint8_t *at = p.values + ((16 * (4 * wave + i) + t) * kPage + 8 * g) * B;
+    if constexpr (Wide<FMT>::kByte) {
+      const u32x2 x = load_streaming<u32x2, REUSED>(at);
+      r.v[i][0] = x[0], r.v[i][1] = x[1];
+    } else {
+      const u32x4 x = load_streaming<u32x4, REUSED>(at);
+#pragma unroll
+      for (uint32_t e = 0; e < 4; ++e) r.v[i][e] = x[e];
+    }
+  }
+}
+template <uint32_t FMT>
+__device__ __forceinline__ u32x4 share_operand(const uint32_t (&raw)[Wide<FMT>::kDwords]) {
+  if constexpr (Wide<FMT>::kFp8) return fp8_operand(raw[0], raw[1]);
+  else if constexpr (Wide<FMT>::kInt8) return int8_operand(raw[0], raw[1]);
+  else return u32x4{raw[0], raw[1], raw[2], raw[3]};
+}
+template <uint32_t FMT>
+__device__ __forceinline__ void stage_share(GroupOperands &page, const GroupShare<FMT> &r, uint32_t wave,
+                                            uint32_t lane) {
+#pragma unroll
+  for (uint32_t tb = 0; tb < 2; ++tb)
+#pragma unroll
+    for (uint32_t c = 0; c < 2; ++c) page.keys[tb][2 * wave + c][lane] = share_operand<FMT>(r.k[tb][c]);
+#pragma unroll
+  for (uint32_t i = 0; i < 4; ++i) page.values[4 * wave + i][lane] = share_operand<FMT>(r.v[i]);
+}
+
+// NB blocks of 16 fused rows per wave; the lane's fused rows are dealt to the four waves in
+// equal runs of ceil(M / 4) (at most 16 NB).
+template <uint32_t FMT, uint32_t NB, bool REUSED>
+__global__ __launch_bounds__(64 * kGroupWaves) __attribute__((amdgpu_waves_per_eu(1, 1))) void
+group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
+                  float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
+  constexpr bool kFp8 = Wide<FMT>::kFp8, kInt8 = Wide<FMT>::kInt8, kByte = Wide<FMT>::kByte;
+  constexpr uint32_t W = kGroupWaves;
+  __shared__ GroupOperands shared_page[2];
+  __shared__ u32x4 q_lds[W][NB][8][64];
+  const uint32_t item = blockIdx.x, head = blockIdx.y;
+  uint32_t li;
+  const DecodeLane l = lane_of_item(a, item, li);
+  const uint32_t split = item - l.first_item;
+  // Every wave of the workgroup takes the same way out: the barriers below are reached by
+  // all of them or by none.
+  if (split >= l.split_count) return;
+  const uint32_t visible = l.committed + l.active_rows;
+  const uint32_t pages = (visible + kPage - 1) / kPage;
+  const uint32_t per = (pages + l.split_count - 1) / l.split_count;
+  const uint32_t written = (pages + per - 1) / per;
+  const uint32_t begin = split * per;
+  if (begin >= pages) return;
+  const uint32_t end = min(pages, begin + per);
+
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t lane = threadIdx.x & 63u, t = lane & 15, g = lane >> 4;
+  const uint32_t H = a.kv_heads, G = a.group, M = a.fused_rows;
+  const uint32_t db = Wide<FMT>::kSlab * H, sb = kByte ? kPage * H * 4 : 0;
+  const RegionOffsets ro = region_offsets(a.kv.extent_pages, db, sb);
+  const float score_scale = default_score_scale(kD, l.score_scale);
+
+  const uint32_t run = (M + W - 1) / W;  // fused rows per wave
+  uint32_t m[NB];
+  bool in_tile[NB], live_row[NB];
+  Sight sight[NB];
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    m[nb] = run * wave + 16 * nb + t;
+    const uint32_t query_row = m[nb] / G;
+    in_tile[nb] = 16 * nb + t < run && m[nb] < M;
+    live_row[nb] = in_tile[nb] && query_row < l.active_rows;
+    sight[nb].committed = l.committed;
+    sight[nb].visible = visible;
+    sight[nb].limit =
+        live_row[nb] ? min(visible, l.committed + min(query_row, l.active_rows - 1) + 1) : visible;
+    sight[nb].tree = live_row[nb] && l.masks != nullptr;
+    sight[nb].mask = sight[nb].tree ? l.masks[query_row] : 0u;
+  }
+  // A wave none of whose rows is in the lane still fetches and stages its quarter.
+  const bool computes = run * wave < M;
+
+  const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    const uint16_t *q_row = q_head + uint64_t(live_row[nb] ? m[nb] : 0) * kD;
+#pragma unroll
+    for (uint32_t kb = 0; kb < 8; ++kb) {
+      u32x4 q = load_global<u32x4>(q_row + key_dims<FMT>(kb, g));
+      if constexpr (kByte) {
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+          const f16x2 pair = {_Float16(__uint_as_float(q[i] << 16)),
+                              _Float16(__uint_as_float(q[i] & 0xffff0000u))};
+          q[i] = __builtin_bit_cast(uint32_t, pair);
+        }
+      }
+      if (!live_row[nb]) q = u32x4{0u, 0u, 0u, 0u};
+      q_lds[wave][nb][kb][lane] = q;  // read back by this wave only
+    }
+  }
+
+  const uint64_t *const entries = l.table + begin;
+  const uint32_t count = end - begin, last_slot = count - 1;
+  GroupShare<FMT> raw[2];  // raw[i % 2]: this wave's quarter of the page of slot i
+  auto fetch = [&](GroupShare<FMT> &set, uint32_t slot) {
+    const PagePlace p = place_page<FMT>(scalar_entry(entries, min(slot, last_slot)), head, H, a.kv.offset, ro);
+    asm volatile("");
+    fetch_share<FMT, REUSED>(set, p, wave, t, g);
+    asm volatile("");
+  };
+  // The scales of a byte format's page, by every wave for its own lanes: they are few, and
+  // what a lane needs of them depends on its place in the wave alone.
+  f32x4 ks_even[2], vs_even[2], ks_odd[2], vs_odd[2];
+  auto fetch_scales = [&](f32x4 (&ks)[2], f32x4 (&vs)[2], uint32_t slot) {
+    if constexpr (kByte) {
+      const PagePlace p = place_page<FMT>(scalar_entry(entries, min(slot, last_slot)), head, H, a.kv.offset, ro);
+      ks[0] = load_global<f32x4>(p.key_scales + 8 * g);
+      ks[1] = load_global<f32x4>(p.key_scales + 8 * g + 4);
+      vs[0] = load_global<f32x4>(p.value_scales + 8 * g);
+      vs[1] = load_global<f32x4>(p.value_scales + 8 * g + 4);
+    }
+  };
+  fetch(raw[0], 0);
+  fetch(raw[1], 1);
+  fetch_scales(ks_even, vs_even, 0);
+  fetch_scales(ks_odd, vs_odd, 1);
+
+  f32x4 acc[NB][16];  // [block][dim block]: dims 16*mb + 4g + r of column t
+  float row_max[NB], row_sum[NB];
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+#pragma unroll
+    for (uint32_t mb = 0; mb < 16; ++mb) acc[nb][mb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    row_max[nb] = -INFINITY;
+    row_sum[nb] = 0.0f;
+  }
+
+  // One staged page against the wave's rows.  check_tokens: whether the page can hold
+  // tokens some row does not see (a page wholly inside the committed tokens cannot; one
+  // copy of the page code serves both, the test itself is skipped).
+  auto attend_page = [&](const GroupOperands &now, uint32_t page, const f32x4 (&page_ks)[2],
+                         const f32x4 (&page_vs)[2], bool check_tokens) {
+    f32x4 s[NB][2];
+#pragma unroll
+    for (uint32_t nb = 0; nb < NB; ++nb) s[nb][0] = s[nb][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (uint32_t kb = 0; kb < 8; ++kb)
+#pragma unroll
+      for (uint32_t tb = 0; tb < 2; ++tb) {
+        const u32x4 k = now.keys[tb][kb][lane];
+#pragma unroll
+        for (uint32_t nb = 0; nb < NB; ++nb) s[nb][tb] = mfma<FMT>(k, q_lds[wave][nb][kb][lane], s[nb][tb]);
+      }
+    const uint32_t first_token = page * kPage;
+    u32x4 pb[NB];
+#pragma unroll
+    for (uint32_t nb = 0; nb < NB; ++nb) {
+      float score[8], local_max = -INFINITY;
+      bool live[8];
+#pragma unroll
+      for (uint32_t i = 0; i < 8; ++i) live[i] = true;
+      if (check_tokens) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i)
+          live[i] = sight[nb].sees(first_token + 8 * g + 4 * (i >> 2) + (i & 3));
+      }
+#pragma unroll
+      for (uint32_t i = 0; i < 8; ++i) {
+        const uint32_t tb = i >> 2, rr = i & 3;
+        float v = s[nb][tb][rr];
+        if constexpr (kByte) v *= page_ks[tb][rr];
+        v *= score_scale;
+        score[i] = live[i] ? v : -INFINITY;
+        local_max = fmaxf(local_max, score[i]);
+      }
+      local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
+      local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
+      const float next_max = fmaxf(row_max[nb], local_max);
+      // A row that has seen nothing yet keeps -inf; its rescale is 1, not exp(nan).
+      const float rescale = next_max == row_max[nb]
+                                ? 1.0f
+                                : __builtin_amdgcn_exp2f((row_max[nb] - next_max) * kLog2e);
+      float weight[8], page_sum = 0.0f;
+#pragma unroll
+      for (uint32_t i = 0; i < 8; ++i) {
+        // The difference first, so the page's maximum gets exactly 1.
+        float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
+        p = live[i] ? p : 0.0f;
+        page_sum += p;
+        weight[i] = kByte ? p * page_vs[i >> 2][i & 3] : p;
+      }
+      row_sum[nb] = fmaf(row_sum[nb], rescale, page_sum);
+      row_max[nb] = next_max;
+#pragma unroll
+      for (uint32_t p = 0; p < 4; ++p) {
+        if constexpr (kFp8) {
+          const f16x2 pair = {_Float16(weight[2 * p]), _Float16(weight[2 * p + 1])};
+          pb[nb][p] = __builtin_bit_cast(uint32_t, pair);
+        } else if constexpr (kInt8) {
+          // Rounded to bf16 as the reference tile does, then carried as fp16.
+          const f32x2 wide = {weight[2 * p], weight[2 * p + 1]};
+          const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(wide, bf16x2));
+          const f16x2 pair = {_Float16(__uint_as_float(bits << 16)),
+                              _Float16(__uint_as_float(bits & 0xffff0000u))};
+          pb[nb][p] = __builtin_bit_cast(uint32_t, pair);
+        } else {
+          const f32x2 pair = {weight[2 * p], weight[2 * p + 1]};
+          pb[nb][p] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+        }
+      }
+      if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
+#pragma unroll
+        for (uint32_t mb = 0; mb < 16; ++mb) acc[nb][mb] *= rescale;
+      }
+    }
+#pragma unroll
+    for (uint32_t mb = 0; mb < 16; ++mb) {
+      const u32x4 v = now.values[mb][lane];
+#pragma unroll
+      for (uint32_t nb = 0; nb < NB; ++nb) acc[nb][mb] = mfma<FMT>(v, pb[nb], acc[nb][mb]);
+    }
+  };
+
+  // The first page into the first copy.
+  const uint32_t first_masked = l.committed / kPage;
+  stage_share<FMT>(shared_page[0], raw[0], wave, lane);
+  fetch(raw[0], 2);
+  group_barrier();
+  // Slot i of the split: copy i % 2 holds it staged when its turn comes; while it is
+  // multiplied, slot i + 1 goes from raw set (i + 1) % 2 into the other copy and that set is
+  // sent for slot i + 3 (past the end: the last page again, staged into a copy nobody
+  // reads).  Two slots per turn of the loop and no branch around the loads, so every wait
+  // names exactly the loads it needs.
+  auto turn = [&](const GroupOperands &now, GroupOperands &next, GroupShare<FMT> &next_raw, uint32_t slot,
+                  f32x4 (&ks)[2], f32x4 (&vs)[2]) {
+    stage_share<FMT>(next, next_raw, wave, lane);
+    fetch(next_raw, slot + 3);
+    if (computes && slot < count) attend_page(now, begin + slot, ks, vs, begin + slot >= first_masked);
+    fetch_scales(ks, vs, slot + 2);
+    group_barrier();
+  };
+  for (uint32_t slot = 0; slot < count; slot += 2) {
+    turn(shared_page[0], shared_page[1], raw[1], slot, ks_even, vs_even);
+    turn(shared_page[1], shared_page[0], raw[0], slot + 1, ks_odd, vs_odd);
+  }
+  if (!computes) return;
+
+#pragma unroll
+  for (uint32_t nb = 0; nb < NB; ++nb) {
+    // Lanes of one column hold disjoint tokens: combine their sums.
+    float sum = row_sum[nb];
+    sum += __shfl_xor(sum, 16);
+    sum += __shfl_xor(sum, 32);
+    uint16_t *out_head = output + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
+    if (written == 1 && !a.all_partials) {
+      // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
+      // Rows of the tile past the live ones read as zeros.
+      if (in_tile[nb]) {
+        const float denominator = live_row[nb] ? sum : 0.0f;
+#pragma unroll
+        for (uint32_t mb = 0; mb < 16; ++mb) {
+          u32x2 packed;
+#pragma unroll
+          for (uint32_t i = 0; i < 2; ++i) {
+            const float lo = acc[nb][mb][2 * i], hi = acc[nb][mb][2 * i + 1];
+            const float qlo = denominator > 0.0f ? __fdiv_rn(lo, denominator) : 0.0f;
+            const float qhi = denominator > 0.0f ? __fdiv_rn(hi, denominator) : 0.0f;
+            packed[i] = uint32_t(f32_to_bf16(qlo)) | (uint32_t(f32_to_bf16(qhi)) << 16);
+          }
+          *reinterpret_cast<u32x2 *>(out_head + uint64_t(m[nb]) * kD + 16 * mb + 4 * g) = packed;
+        }
+      }
+      continue;
+    }
+    if (live_row[nb]) {
+      const uint64_t row =
+          l.row_base + uint64_t(head) * l.split_count * M + uint64_t(split) * M + m[nb];
+      float *out = partials + row * kD;
+#pragma unroll
+      for (uint32_t mb = 0; mb < 16; ++mb) *reinterpret_cast<f32x4 *>(out + 16 * mb + 4 * g) = acc[nb][mb];
+      if (g == 0) {
+        statistics[row * 2] = row_max[nb];
+        statistics[row * 2 + 1] = sum;
+      }
+    }
+  }
+}
+
 }  // namespace
 }  // namespace kvx
 
@@ -511,6 +852,20 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   // The regular tiles of a chunked prefill (tile_rows > 0) walk the same pages
   // over and over: their loads may stay in the caches.
   const bool reused = tile_rows > 0;
+  // many_tiles == 2: lanes of several prefill tiles each, for a workgroup of four waves
+  // that shares every page through LDS, two row blocks per wave: up to 128 fused rows.
+  if (many_tiles == 2) {
+    if (!tile_rows || M > 32u * kGroupWaves) return 1;
+#define KVX_GROUP(FMT, NB)                                                                        \
+  launch_matrix_attention(group_wide_kernel<FMT, NB, true>, "group_wide_kernel", 16 * NB * kGroupWaves, \
+                          64 * kGroupWaves, s, kv, query_heads, queries, output, page_tables, lanes, \
+                          n_lanes, row_masks, row_stride, lane_stride, workspace, workspace_bytes,  \
+                          stream, nullptr, tile_rows, epilogue)
+    if (format == KVX_FMT_BF16) return KVX_GROUP(KVX_FMT_BF16, 2);
+    if (format == KVX_FMT_INT8) return KVX_GROUP(KVX_FMT_INT8, 2);
+    return KVX_GROUP(KVX_FMT_FP8E4M3, 2);
+#undef KVX_GROUP
+  }
   if (format == KVX_FMT_BF16) {
     if (M > 16) return reused ? KVX_WIDE(KVX_FMT_BF16, 2, 1, true) : KVX_WIDE(KVX_FMT_BF16, 2, 1, false);
     return reused ? KVX_WIDE(KVX_FMT_BF16, 1, 1, true) : KVX_WIDE(KVX_FMT_BF16, 1, 1, false);
