@@ -187,7 +187,12 @@ int kvx_chunk_validation(const kvx_chunk_params *params);
    launch still fits one round of slots: of the paired tiles' waves where the two tiles of
    every pair see the same number of pages (committed_tokens mod 16 is 0 or at least 9, so
    every page-aligned chunk start; int4 pages: from 512 rows on), else of tiles x splits x KV heads x ceil(8 x group / 16)
-   waves of single tiles.  Returns 0 for bad head counts.  No counterpart in the reference (its rule is
+   waves of single tiles.  bf16, fp8 and int8 pages, chunks of 64 rows and more (lanes of four tiles of
+   8 x group <= 48 fused rows, or two of <= 96, one workgroup per lane, split and KV head, one
+   workgroup per CU): one split where those workgroups fill three quarters of the 256 CUs, else
+   the count (same bounds) that fills them, where the chunk starts on a page boundary (lanes
+   of two tiles: where the tiles pair); other starts fall under the rules above.
+   Returns 0 for bad head counts.  No counterpart in the reference (its rule is
    kvx_prefill_splits); any count in 1..32 is valid for kv_attend_prefill. */
 uint32_t kvx_prefill_plan(uint32_t committed_tokens, uint32_t rows, uint32_t kv_heads,
                           uint32_t query_heads, uint32_t format);

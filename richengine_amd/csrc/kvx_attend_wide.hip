@@ -569,7 +569,6 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
   constexpr bool kFp8 = Wide<FMT>::kFp8, kInt8 = Wide<FMT>::kInt8, kByte = Wide<FMT>::kByte;
   constexpr uint32_t W = kGroupWaves;
   __shared__ GroupOperands shared_page[2];
-  __shared__ u32x4 q_lds[W][NB][8][64];
   const uint32_t item = blockIdx.x, head = blockIdx.y;
   uint32_t li;
   const DecodeLane l = lane_of_item(a, item, li);
@@ -613,6 +612,7 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
   const bool computes = run * wave < M;
 
   const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
+  u32x4 q_reg[NB][8];
 #pragma unroll
   for (uint32_t nb = 0; nb < NB; ++nb) {
     const uint16_t *q_row = q_head + uint64_t(live_row[nb] ? m[nb] : 0) * kD;
@@ -628,15 +628,26 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
         }
       }
       if (!live_row[nb]) q = u32x4{0u, 0u, 0u, 0u};
-      q_lds[wave][nb][kb][lane] = q;  // read back by this wave only
+      q_reg[nb][kb] = q;
     }
   }
 
   const uint64_t *const entries = l.table + begin;
   const uint32_t count = end - begin, last_slot = count - 1;
   GroupShare<FMT> raw[2];  // raw[i % 2]: this wave's quarter of the page of slot i
-  auto fetch = [&](GroupShare<FMT> &set, uint32_t slot) {
-    const PagePlace p = place_page<FMT>(scalar_entry(entries, min(slot, last_slot)), head, H, a.kv.offset, ro);
+  // bf16 pages: a page's entry is read a turn before the loads that need it, since one wave
+  // per SIMD has nothing else to run while a scalar load is on its way.  With the byte
+  // formats' conversions to fill that time the early read measured 10 % slower, and they
+  // read the entry where they use it.
+  uint64_t entry_ahead = kByte ? 0 : scalar_entry(entries, 0);
+  auto next_entry = [&](uint32_t following) {
+    if constexpr (kByte) return scalar_entry(entries, min(following - 1, last_slot));
+    const uint64_t entry = entry_ahead;
+    entry_ahead = scalar_entry(entries, min(following, last_slot));
+    return entry;
+  };
+  auto fetch = [&](GroupShare<FMT> &set, uint64_t entry) {
+    const PagePlace p = place_page<FMT>(entry, head, H, a.kv.offset, ro);
     asm volatile("");
     fetch_share<FMT, REUSED>(set, p, wave, t, g);
     asm volatile("");
@@ -644,19 +655,20 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
   // The scales of a byte format's page, by every wave for its own lanes: they are few, and
   // what a lane needs of them depends on its place in the wave alone.
   f32x4 ks_even[2], vs_even[2], ks_odd[2], vs_odd[2];
-  auto fetch_scales = [&](f32x4 (&ks)[2], f32x4 (&vs)[2], uint32_t slot) {
+  auto fetch_scales = [&](f32x4 (&ks)[2], f32x4 (&vs)[2], uint64_t entry) {
     if constexpr (kByte) {
-      const PagePlace p = place_page<FMT>(scalar_entry(entries, min(slot, last_slot)), head, H, a.kv.offset, ro);
+      const PagePlace p = place_page<FMT>(entry, head, H, a.kv.offset, ro);
       ks[0] = load_global<f32x4>(p.key_scales + 8 * g);
       ks[1] = load_global<f32x4>(p.key_scales + 8 * g + 4);
       vs[0] = load_global<f32x4>(p.value_scales + 8 * g);
       vs[1] = load_global<f32x4>(p.value_scales + 8 * g + 4);
     }
   };
-  fetch(raw[0], 0);
-  fetch(raw[1], 1);
-  fetch_scales(ks_even, vs_even, 0);
-  fetch_scales(ks_odd, vs_odd, 1);
+  const uint64_t entry0 = next_entry(1), entry1 = next_entry(2);
+  fetch(raw[0], entry0);
+  fetch(raw[1], entry1);
+  fetch_scales(ks_even, vs_even, entry0);
+  fetch_scales(ks_odd, vs_odd, entry1);
 
   f32x4 acc[NB][16];  // [block][dim block]: dims 16*mb + 4g + r of column t
   float row_max[NB], row_sum[NB];
@@ -682,30 +694,29 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
       for (uint32_t tb = 0; tb < 2; ++tb) {
         const u32x4 k = now.keys[tb][kb][lane];
 #pragma unroll
-        for (uint32_t nb = 0; nb < NB; ++nb) s[nb][tb] = mfma<FMT>(k, q_lds[wave][nb][kb][lane], s[nb][tb]);
+        for (uint32_t nb = 0; nb < NB; ++nb) s[nb][tb] = mfma<FMT>(k, q_reg[nb][kb], s[nb][tb]);
       }
     const uint32_t first_token = page * kPage;
     u32x4 pb[NB];
 #pragma unroll
     for (uint32_t nb = 0; nb < NB; ++nb) {
       float score[8], local_max = -INFINITY;
-      bool live[8];
-#pragma unroll
-      for (uint32_t i = 0; i < 8; ++i) live[i] = true;
-      if (check_tokens) {
-#pragma unroll
-        for (uint32_t i = 0; i < 8; ++i)
-          live[i] = sight[nb].sees(first_token + 8 * g + 4 * (i >> 2) + (i & 3));
-      }
 #pragma unroll
       for (uint32_t i = 0; i < 8; ++i) {
         const uint32_t tb = i >> 2, rr = i & 3;
         float v = s[nb][tb][rr];
         if constexpr (kByte) v *= page_ks[tb][rr];
-        v *= score_scale;
-        score[i] = live[i] ? v : -INFINITY;
-        local_max = fmaxf(local_max, score[i]);
+        score[i] = v * score_scale;
       }
+      // A token the row does not see scores -inf, and its weight below comes out as
+      // exp(-inf) = 0 by itself.
+      if (check_tokens) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i)
+          if (!sight[nb].sees(first_token + 8 * g + 4 * (i >> 2) + (i & 3))) score[i] = -INFINITY;
+      }
+#pragma unroll
+      for (uint32_t i = 0; i < 8; ++i) local_max = fmaxf(local_max, score[i]);
       local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
       local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
       const float next_max = fmaxf(row_max[nb], local_max);
@@ -713,12 +724,13 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
       const float rescale = next_max == row_max[nb]
                                 ? 1.0f
                                 : __builtin_amdgcn_exp2f((row_max[nb] - next_max) * kLog2e);
+      // A row that still has seen nothing measures from 0: -inf - -inf is no number.
+      const float reference = next_max == -INFINITY ? 0.0f : next_max;
       float weight[8], page_sum = 0.0f;
 #pragma unroll
       for (uint32_t i = 0; i < 8; ++i) {
         // The difference first, so the page's maximum gets exactly 1.
-        float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
-        p = live[i] ? p : 0.0f;
+        const float p = __builtin_amdgcn_exp2f((score[i] - reference) * kLog2e);
         page_sum += p;
         weight[i] = kByte ? p * page_vs[i >> 2][i & 3] : p;
       }
@@ -742,8 +754,14 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
         }
       }
       if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
+        // The accumulators live in the second register file and are named there on the way
+        // in, so that the moves out of it that a multiply needs stay inside this branch:
+        // left to itself the compiler moves all of them out on every page.
 #pragma unroll
-        for (uint32_t mb = 0; mb < 16; ++mb) acc[nb][mb] *= rescale;
+        for (uint32_t mb = 0; mb < 16; ++mb) {
+          asm volatile("" : "+a"(acc[nb][mb]));
+          acc[nb][mb] *= rescale;
+        }
       }
     }
 #pragma unroll
@@ -757,7 +775,8 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
   // The first page into the first copy.
   const uint32_t first_masked = l.committed / kPage;
   stage_share<FMT>(shared_page[0], raw[0], wave, lane);
-  fetch(raw[0], 2);
+  uint64_t entry_scales = next_entry(3);  // the page two slots on, whose scales are read a turn after its operands
+  fetch(raw[0], entry_scales);
   group_barrier();
   // Slot i of the split: copy i % 2 holds it staged when its turn comes; while it is
   // multiplied, slot i + 1 goes from raw set (i + 1) % 2 into the other copy and that set is
@@ -767,9 +786,11 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
   auto turn = [&](const GroupOperands &now, GroupOperands &next, GroupShare<FMT> &next_raw, uint32_t slot,
                   f32x4 (&ks)[2], f32x4 (&vs)[2]) {
     stage_share<FMT>(next, next_raw, wave, lane);
-    fetch(next_raw, slot + 3);
+    const uint64_t entry = next_entry(slot + 4);
+    fetch(next_raw, entry);
     if (computes && slot < count) attend_page(now, begin + slot, ks, vs, begin + slot >= first_masked);
-    fetch_scales(ks, vs, slot + 2);
+    fetch_scales(ks, vs, entry_scales);
+    entry_scales = entry;
     group_barrier();
   };
   for (uint32_t slot = 0; slot < count; slot += 2) {
@@ -855,12 +876,17 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   // many_tiles == 2: lanes of several prefill tiles each, for a workgroup of four waves
   // that shares every page through LDS, two row blocks per wave: up to 128 fused rows.
   if (many_tiles == 2) {
-    if (!tile_rows || M > 32u * kGroupWaves) return 1;
+    if (!tile_rows || M > 48u * kGroupWaves) return 1;
 #define KVX_GROUP(FMT, NB)                                                                        \
   launch_matrix_attention(group_wide_kernel<FMT, NB, true>, "group_wide_kernel", 16 * NB * kGroupWaves, \
                           64 * kGroupWaves, s, kv, query_heads, queries, output, page_tables, lanes, \
                           n_lanes, row_masks, row_stride, lane_stride, workspace, workspace_bytes,  \
                           stream, nullptr, tile_rows, epilogue)
+    if (M > 32u * kGroupWaves) {
+      if (format == KVX_FMT_BF16) return KVX_GROUP(KVX_FMT_BF16, 3);
+      if (format == KVX_FMT_INT8) return KVX_GROUP(KVX_FMT_INT8, 3);
+      return KVX_GROUP(KVX_FMT_FP8E4M3, 3);
+    }
     if (format == KVX_FMT_BF16) return KVX_GROUP(KVX_FMT_BF16, 2);
     if (format == KVX_FMT_INT8) return KVX_GROUP(KVX_FMT_INT8, 2);
     return KVX_GROUP(KVX_FMT_FP8E4M3, 2);

@@ -167,12 +167,22 @@ uint32_t kvx_prefill_plan(uint32_t committed, uint32_t rows, uint32_t kv_heads, 
   const uint32_t group = query_heads / kv_heads, tile_fused = KVX_PREFILL_TILE_ROWS * group;
   const uint32_t pages = pages_of(uint64_t(committed) + rows);
   constexpr uint32_t kSimds = 1024;
+  const uint32_t by_pages = std::max(1u, pages / 8);
+  // bf16, fp8 and int8 pages, long chunks: lanes of several tiles, one workgroup per lane,
+  // split and KV head, one workgroup per CU.  One split where that fills three quarters of
+  // the CUs; else as many as fill them, where the lanes' tiles cut their pages alike.
+  if (const uint32_t width = kvx::prefill_group_width(format, 256, rows, group)) {
+    constexpr uint32_t kCus = 256;
+    const uint32_t workgroups = (tiles + width - 1) / width * kv_heads;
+    if (4 * workgroups >= 3 * kCus) return 1;
+    if (kvx::prefill_group_splits_alike(width, committed))
+      return std::max(1u, std::min({(kCus + workgroups - 1) / workgroups, by_pages, KVX_PREFILL_MAX_SPLITS}));
+  }
   // One split: neighbouring tiles share a walk as lanes of 16 rows on the kernels
   // with two blocks of 16 fused rows per wave (int4: two waves per SIMD).
   const uint32_t paired_waves = kvx::prefill_paired_waves(tiles, kv_heads, group);
   const uint32_t paired_slots = kvx::prefill_paired_slots(format);
   if (tile_fused <= 16 || 2 * paired_waves >= paired_slots) return 1;
-  const uint32_t by_pages = std::max(1u, pages / 8);
   // Tiles that pair under any split count keep their shared walks: as many
   // splits as fit one round of the paired kernels' slots.
   const uint32_t paired_splits =

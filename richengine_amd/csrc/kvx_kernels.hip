@@ -1894,10 +1894,6 @@ int kv_append_attend_decode(const kvx_storage *s, uint32_t layer, const void *ch
                           row_stride, workspace, workspace_bytes, stream);
 }
 
-// Chunks from this many rows on take the lanes of several tiles whose waves share pages
-// through LDS (bf16, fp8, int8 pages); shorter ones have too few such lanes to fill the GPU.
-constexpr uint32_t kGroupedPrefillRows = 256;
-
 int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
                       const void *queries, void *output, const uint64_t *page_table,
                       const kvx_prefill_params *params, void *workspace, uint64_t workspace_bytes,
@@ -1946,23 +1942,15 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
                                                   params->split_count, H, G)))
             ? 2
             : 1;
-    // bf16, fp8 and int8 pages: lanes of four (or two) tiles for a workgroup of four waves
-    // that fetches every page once for all of them and shares it through LDS, where the
-    // lane's fused rows fit its two row blocks per wave (128).
-    // With several splits the tiles of a lane must cut their pages into the same splits,
-    // which they do when the chunk starts on a page boundary and a lane is 32 rows.
+    // bf16, fp8 and int8 pages: lanes of four (or two) tiles for a workgroup that shares
+    // every page through LDS (prefill_group_width); with several splits only where a
+    // lane's tiles cut their pages alike.
     int lane_kind = width == 1 ? 1 : 0;  // attend_matrix's many_tiles
-    if (l.format != KVX_FMT_INT4 && D == 256 && params->rows >= kGroupedPrefillRows) {
-      const uint32_t most = 128u;
-      const uint32_t grouped = 4 * T * G <= most ? 4u : 2 * T * G <= most ? 2u : 0u;
-      const bool same_splits =
-          params->split_count == 1 ||
-          (grouped == 4 && params->committed_tokens % KVX_PAGE_TOKENS == 0) ||
-          (grouped == 2 && prefill_tiles_pair(params->committed_tokens));
-      if (grouped && tiles >= grouped && same_splits) {
-        width = grouped;
-        lane_kind = 2;
-      }
+    const uint32_t grouped = prefill_group_width(l.format, D, params->rows, G);
+    if (grouped && tiles >= grouped &&
+        (params->split_count == 1 || prefill_group_splits_alike(grouped, params->committed_tokens))) {
+      width = grouped;
+      lane_kind = 2;
     }
     const uint32_t wide_lanes = tiles / width, rest = tiles - wide_lanes * width;
     std::vector<kvx_verify_params> tile_lanes(wide_lanes + rest);

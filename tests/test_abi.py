@@ -152,7 +152,18 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
             tiles = -(-rows // 8)
             paired = -(-tiles // 2) * H * -(-(16 * (QH // H)) // 32)
             want = 1
-            if 2 * paired < single_slots:
+            width = 0
+            if fmt != kvx.INT4 and rows >= 64:           # lanes of several tiles, a workgroup each
+                fused = 8 * (QH // H)
+                width = 4 if 4 * fused <= 192 else 2 if 2 * fused <= 192 else 0
+            workgroups = -(-tiles // width) * H if width else 0
+            alike = width and (committed % 32 == 0 if width == 4 else
+                               (committed % 16 == 0 or committed % 16 >= 9))
+            if width and 4 * workgroups >= 3 * 256:
+                want = 1
+            elif alike:
+                want = max(1, min(-(-256 // workgroups), max(1, pages(committed + rows) // 8), 32))
+            elif 2 * paired < single_slots:
                 by_pages = max(1, pages(committed + rows) // 8)
                 pairable = tiles >= 2 and (committed % 16 == 0 or committed % 16 >= 9)
                 if fmt == kvx.INT4 and tiles < 64:
@@ -165,7 +176,9 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
                     want = want if want >= 2 else 1
             assert kvx.prefill_plan(committed, rows, H, QH, fmt) == want
     assert kvx.prefill_plan(16384, 256, H, QH, kvx.INT4) == 5      # 384 waves of single tiles per split
-    assert kvx.prefill_plan(16384, 256, H, QH, kvx.BF16) == 5      # 192 of paired tiles
+    assert kvx.prefill_plan(16384, 256, H, QH, kvx.BF16) == 8      # 32 workgroups of four tiles each
+    assert kvx.prefill_plan(16384, 1024, H, QH, kvx.FP8) == 2      # 128 workgroups
+    assert kvx.prefill_plan(16384, 2048, H, QH, kvx.INT8) == 1     # 256 workgroups
     assert kvx.prefill_plan(16384, 1024, H, QH, kvx.INT4) == 2     # 768 of paired tiles
     assert kvx.prefill_plan(16388, 256, H, QH, kvx.BF16) == 2      # 384 of single tiles
     assert kvx.prefill_plan(16384, 2048, H, QH, kvx.INT4) == 1
@@ -208,6 +221,12 @@ def test_hot_kernels_stay_out_of_scratch_memory():
         r = one(fragment)
         assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, (fragment, r)
     assert one("decode_int4_kernelE")["occupancy"] == 2
+    # the workgroup-shared prefill kernels (int8, bf16, fp8 pages; two and three row blocks
+    # per wave): one wave per SIMD with all 512 registers, and nothing beyond them
+    for fmt in (1, 2, 4):
+        for blocks in (2, 3):
+            r = one(f"group_wide_kernelILj{fmt}ELj{blocks}ELb1E")
+            assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, (fmt, blocks, r)
     # the 48-row verify kernel keeps a few set-up values in scratch memory, none of
     # them touched inside its page loop; more than that would be accumulators or pages
     assert one("verify48_int4_kernel")["vgprs_spill"] <= 20

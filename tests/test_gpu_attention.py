@@ -98,7 +98,7 @@ def test_int4_prefill_pairs_tiles_under_several_splits():
     prefill_case(ko.INT4, 1500, 264)
 
 
-def prefill_case(fmt, committed, rows):
+def prefill_case(fmt, committed, rows, forced_splits=None):
     planned, rows = rows < 0, abs(rows)
     tw = Gp.Twin(fmt, H, D, 2, (committed + rows + 31) // 32)
     pages, th, td = fill(tw, committed + rows, seed=committed + rows)
@@ -110,6 +110,8 @@ def prefill_case(fmt, committed, rows):
     if planned:
         splits = kvx.prefill_plan(committed, rows, H, QH, fmt)
         assert splits > 1
+    if forced_splits:
+        splits = forced_splits
     hp = ko.PrefillParams(committed, rows, stride, len(pages), tw.host.layer(1), splits, 0.0)
     ok, want, want32 = ko.attend_prefill(fmt, H, G, D, q, th, hp)
     assert ok == 1
