@@ -398,7 +398,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
         }
         if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
 #pragma unroll
-          for (uint32_t mb = 0; mb < 16; ++mb) acc[nb][mb] *= rescale;
+          for (uint32_t mb = 0; mb < 16; ++mb) {
+            // Two blocks of accumulators (one wave per SIMD) live in the second register
+            // file.  Named there on the way in, the moves out of it that a multiply needs
+            // stay inside this branch; left to itself the compiler moves every accumulator
+            // out on every page.
+            if constexpr (NB == 2) asm volatile("" : "+a"(acc[nb][mb]));
+            acc[nb][mb] *= rescale;
+          }
         }
       }
       // ---- p.v ----

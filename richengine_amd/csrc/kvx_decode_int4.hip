@@ -211,7 +211,9 @@ struct RegisterPage {
 // keys_consumed() runs when the page's keys have been read for the last time:
 // the steady loop refills them from there, half a page ahead of the rest.
 // queries(nb, kb) yields the B operand of block nb for dims block kb.
-template <bool MASKED, uint32_t NB, class Page, class Queries, class KeysConsumed>
+// PINNED: the kernel runs one wave per SIMD and its accumulators live in the second
+// register file (see the rescaling below).
+template <bool MASKED, uint32_t NB, bool PINNED, class Page, class Queries, class KeysConsumed>
 __device__ __forceinline__ void attend_page(const Page &source, Queries queries,
                                             const float *q_bias, float score_scale,
                                             uint32_t first_token, const Sight *sight,
@@ -283,7 +285,13 @@ __device__ __forceinline__ void attend_page(const Page &source, Queries queries,
     st[nb].bias = fmaf(st[nb].bias, rescale, page_bias);
     if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
 #pragma unroll
-      for (uint32_t m = 0; m < 16; ++m) st[nb].acc[m] *= rescale;
+      for (uint32_t m = 0; m < 16; ++m) {
+        // Accumulators in the second register file are named there on the way in, so that
+        // the moves out of it that a multiply needs stay inside this branch; left to itself
+        // the compiler moves every accumulator out on every page.
+        if constexpr (PINNED) asm volatile("" : "+a"(st[nb].acc[m]));
+        st[nb].acc[m] *= rescale;
+      }
     }
   }
   // ---- p.v ----
@@ -432,6 +440,8 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
                                             uint16_t *__restrict__ output,
                                             float *__restrict__ partials,
                                             float *__restrict__ statistics, const DecodeArgs &a) {
+  // The forms that have a SIMD to themselves: three blocks, or two with two page sets.
+  constexpr bool kPinned = NB == 3 || (NB == 2 && kDepth >= 2);
   const uint32_t item = blockIdx.x, head = blockIdx.y;
   uint32_t li;
   const DecodeLane l = lane_of_item(a, item, li);
@@ -584,7 +594,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
 #pragma unroll
     for (uint32_t d = 0; d < kDepth; ++d) {
       // upcoming[d] is the entry of slot page + d + kDepth - begin, this set's refill
-      attend_page<false, NB>(RegisterPage{r[d], g}, staged_queries, q_bias, score_scale,
+      attend_page<false, NB, kPinned>(RegisterPage{r[d], g}, staged_queries, q_bias, score_scale,
                              (page + d) * kPage, sight, g, st, [&] { fill_keys(r[d], upcoming[d]); });
       fill_rest(r[d], upcoming[d]);
       upcoming[d] = scalar_entry(entries, min(page + d + 2 * kDepth - begin, last_slot));
@@ -595,7 +605,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   for (uint32_t k = 0; k < kUnmaskedStop - 1; ++k) {
     const uint32_t d = k % kDepth;
     if (page + k < end) {
-      attend_page<true, NB>(RegisterPage{r[d], g}, staged_queries, q_bias, score_scale,
+      attend_page<true, NB, kPinned>(RegisterPage{r[d], g}, staged_queries, q_bias, score_scale,
                             (page + k) * kPage, sight, g, st, [] {});
       if (k + kDepth < kUnmaskedStop - 1 && page + k + kDepth < end) {
         fill(r[d], upcoming[d]);  // slot page + k + kDepth - begin, and d = k here

@@ -227,14 +227,12 @@ def test_hot_kernels_stay_out_of_scratch_memory():
         for blocks in (2, 3):
             r = one(f"group_wide_kernelILj{fmt}ELj{blocks}ELb1E")
             assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, (fmt, blocks, r)
-    # the 48-row verify kernel keeps a few set-up values in scratch memory, none of
-    # them touched inside its page loop; more than that would be accumulators or pages
-    assert one("verify48_int4_kernel")["vgprs_spill"] <= 20
-    # likewise the two-block bf16 kernel (verify and prefill tiles on bf16 pages): values of its
-    # set-up and write-out are parked in scratch memory across the page loop, which had no
-    # scratch access in the assembly when this bound was set
-    for reused in (0, 1):
-        assert one(f"attend_wide_kernelILj2ELj2ELj1ELb{reused}E")["vgprs_spill"] <= 80
+    # the kernels whose accumulators fill the second register file (48-row verify, two-block
+    # bf16): since their rescaling names the accumulators there, nothing spills
+    for fragment in ("verify48_int4_kernel", "attend_wide_kernelILj2ELj2ELj1ELb0E",
+                     "attend_wide_kernelILj2ELj2ELj1ELb1E"):
+        r = one(fragment)
+        assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, (fragment, r)
     assert one("attend_wide_kernelILj1ELj1ELj2ELb0E")["occupancy"] == 2
     for fmt in (1, 2, 3, 4):
         assert one(f"13append_kernelILj{fmt}E")["scratchsize"] == 0
