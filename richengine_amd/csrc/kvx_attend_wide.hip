@@ -493,16 +493,16 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
 // for 0.9 TFLOP of arithmetic.  Here four waves form a workgroup per (lane of up to 32 query
 // rows, split, KV head): each fetches a quarter of the page and writes it into LDS as
 // finished MFMA operands (byte formats expanded on the way, once instead of four times),
-// and all four multiply their own fused rows with the shared copy.  Two copies alternate:
-// while a page is multiplied the next one is staged, one barrier per page; each wave keeps
-// its quarters of the pages two and three ahead in flight.  An operand read from LDS must
+// and all four multiply their own fused rows with the shared copy.  Two pairs of copies
+// alternate: while two pages are multiplied the next two are staged, one barrier per two
+// pages; each wave keeps its quarter of one page in flight.  An operand read from LDS must
 // feed two row blocks: four waves reading one block's worth each would ask the LDS for
 // twice what it delivers.
 constexpr uint32_t kGroupWaves = 4;
 
-// The workgroup's barrier between pages: a wave's LDS writes are done (the LDS counter at
-// zero) before it arrives, and that is all; __syncthreads() would also wait for the global
-// loads in flight, which are the pages two and three ahead.
+// The workgroup's barrier between pairs of pages: a wave's LDS writes are done (the LDS
+// counter at zero) before it arrives, and that is all; __syncthreads() would also wait for
+// the global loads in flight, which are the next page to stage.
 __device__ __forceinline__ void group_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
@@ -575,7 +575,7 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
                   float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
   constexpr bool kFp8 = Wide<FMT>::kFp8, kInt8 = Wide<FMT>::kInt8, kByte = Wide<FMT>::kByte;
   constexpr uint32_t W = kGroupWaves;
-  __shared__ GroupOperands shared_page[2];
+  __shared__ GroupOperands shared_page[4];
   const uint32_t item = blockIdx.x, head = blockIdx.y;
   uint32_t li;
   const DecodeLane l = lane_of_item(a, item, li);
@@ -641,7 +641,7 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
 
   const uint64_t *const entries = l.table + begin;
   const uint32_t count = end - begin, last_slot = count - 1;
-  GroupShare<FMT> raw[2];  // raw[i % 2]: this wave's quarter of the page of slot i
+  GroupShare<FMT> raw;  // this wave's quarter of the page two slots on
   // bf16 pages: a page's entry is read a turn before the loads that need it, since one wave
   // per SIMD has nothing else to run while a scalar load is on its way.  With the byte
   // formats' conversions to fill that time the early read measured 10 % slower, and they
@@ -672,8 +672,7 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
     }
   };
   const uint64_t entry0 = next_entry(1), entry1 = next_entry(2);
-  fetch(raw[0], entry0);
-  fetch(raw[1], entry1);
+  fetch(raw, entry0);
   fetch_scales(ks_even, vs_even, entry0);
   fetch_scales(ks_odd, vs_odd, entry1);
 
@@ -691,18 +690,30 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
   // tokens some row does not see (a page wholly inside the committed tokens cannot; one
   // copy of the page code serves both, the test itself is skipped).
   auto attend_page = [&](const GroupOperands &now, uint32_t page, const f32x4 (&page_ks)[2],
-                         const f32x4 (&page_vs)[2], bool check_tokens) {
+                         const f32x4 (&page_vs)[2], bool check_tokens) __attribute__((always_inline)) {
     f32x4 s[NB][2];
 #pragma unroll
     for (uint32_t nb = 0; nb < NB; ++nb) s[nb][0] = s[nb][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    // Operands come out of LDS kAhead reads before the MFMAs that take them: the four waves
+    // of the workgroup read at the same time, and a read comes back later than the MFMAs of
+    // two operands last.  The order is pinned, or the compiler pulls the reads back together.
+    constexpr uint32_t kAhead = kInt8 ? 3 : 4;  // int8 with four reloads spilled registers inside the page loop
+    u32x4 operand[kAhead];
 #pragma unroll
-    for (uint32_t kb = 0; kb < 8; ++kb)
+    for (uint32_t i = 0; i < kAhead; ++i) operand[i] = now.keys[i & 1][i >> 1][lane];
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (uint32_t tb = 0; tb < 2; ++tb) {
-        const u32x4 k = now.keys[tb][kb][lane];
+    for (uint32_t i = 0; i < 16; ++i) {
+      const uint32_t tb = i & 1, kb = i >> 1;
 #pragma unroll
-        for (uint32_t nb = 0; nb < NB; ++nb) s[nb][tb] = mfma<FMT>(k, q_reg[nb][kb], s[nb][tb]);
-      }
+      for (uint32_t nb = 0; nb < NB; ++nb) s[nb][tb] = mfma<FMT>(operand[i % kAhead], q_reg[nb][kb], s[nb][tb]);
+      if (i + kAhead < 16) operand[i % kAhead] = now.keys[(i + kAhead) & 1][(i + kAhead) >> 1][lane];
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // The first value operands are on their way while the softmax runs.
+#pragma unroll
+    for (uint32_t i = 0; i < kAhead; ++i) operand[i] = now.values[i][lane];
+    __builtin_amdgcn_sched_barrier(0);
     const uint32_t first_token = page * kPage;
     u32x4 pb[NB];
 #pragma unroll
@@ -771,38 +782,50 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
         }
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (uint32_t mb = 0; mb < 16; ++mb) {
-      const u32x4 v = now.values[mb][lane];
 #pragma unroll
-      for (uint32_t nb = 0; nb < NB; ++nb) acc[nb][mb] = mfma<FMT>(v, pb[nb], acc[nb][mb]);
+      for (uint32_t nb = 0; nb < NB; ++nb) acc[nb][mb] = mfma<FMT>(operand[mb % kAhead], pb[nb], acc[nb][mb]);
+      if (mb + kAhead < 16) operand[mb % kAhead] = now.values[mb + kAhead][lane];
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // The first page into the first copy.
+  // The first two pages into the first two copies.
   const uint32_t first_masked = l.committed / kPage;
-  stage_share<FMT>(shared_page[0], raw[0], wave, lane);
-  uint64_t entry_scales = next_entry(3);  // the page two slots on, whose scales are read a turn after its operands
-  fetch(raw[0], entry_scales);
+  stage_share<FMT>(shared_page[0], raw, wave, lane);
+  fetch(raw, entry1);
+  stage_share<FMT>(shared_page[1], raw, wave, lane);
+  uint64_t carried = next_entry(3);  // the entry of the page in the raw registers
+  fetch(raw, carried);
   group_barrier();
-  // Slot i of the split: copy i % 2 holds it staged when its turn comes; while it is
-  // multiplied, slot i + 1 goes from raw set (i + 1) % 2 into the other copy and that set is
-  // sent for slot i + 3 (past the end: the last page again, staged into a copy nobody
-  // reads).  Two slots per turn of the loop and no branch around the loads, so every wait
-  // names exactly the loads it needs.
-  auto turn = [&](const GroupOperands &now, GroupOperands &next, GroupShare<FMT> &next_raw, uint32_t slot,
-                  f32x4 (&ks)[2], f32x4 (&vs)[2]) {
-    stage_share<FMT>(next, next_raw, wave, lane);
-    const uint64_t entry = next_entry(slot + 4);
-    fetch(next_raw, entry);
-    if (computes && slot < count) attend_page(now, begin + slot, ks, vs, begin + slot >= first_masked);
-    fetch_scales(ks, vs, entry_scales);
-    entry_scales = entry;
+  // Four copies, two pages between barriers: while slots i and i + 1 are multiplied out of
+  // one pair of copies, slots i + 2 and i + 3 go from the raw registers into the other pair,
+  // each a page time after its loads were sent (past the end: the last page again, staged
+  // into copies nobody reads).  A barrier per page cost 5 % more: the waves leave it
+  // together and read their operands at the same time.  Four slots per turn of the loop
+  // and no branch around the loads, so every wait names exactly the loads it needs.
+  auto pair = [&](const GroupOperands &now0, const GroupOperands &now1, GroupOperands &next0,
+                  GroupOperands &next1, uint32_t slot) __attribute__((always_inline)) {
+    stage_share<FMT>(next0, raw, wave, lane);
+    const uint64_t entry_odd = next_entry(slot + 4);  // of slot + 3
+    fetch(raw, entry_odd);
+    if (computes && slot < count)
+      attend_page(now0, begin + slot, ks_even, vs_even, begin + slot >= first_masked);
+    fetch_scales(ks_even, vs_even, carried);  // of slot + 2
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    stage_share<FMT>(next1, raw, wave, lane);
+    carried = next_entry(slot + 5);  // of slot + 4
+    fetch(raw, carried);
+    if (computes && slot + 1 < count)
+      attend_page(now1, begin + slot + 1, ks_odd, vs_odd, begin + slot + 1 >= first_masked);
+    fetch_scales(ks_odd, vs_odd, entry_odd);
     group_barrier();
   };
-  for (uint32_t slot = 0; slot < count; slot += 2) {
-    turn(shared_page[0], shared_page[1], raw[1], slot, ks_even, vs_even);
-    turn(shared_page[1], shared_page[0], raw[0], slot + 1, ks_odd, vs_odd);
+  for (uint32_t slot = 0; slot < count; slot += 4) {
+    pair(shared_page[0], shared_page[1], shared_page[2], shared_page[3], slot);
+    pair(shared_page[2], shared_page[3], shared_page[0], shared_page[1], slot + 2);
   }
   if (!computes) return;
 
