@@ -486,7 +486,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
 }
 
 
-// ---- pages shared by the four waves of a workgroup: the tiles of a chunked prefill ----
+// ---- pages shared by the waves of a workgroup: the tiles of a chunked prefill, verify ----
 //
 // A chunk's tiles walk the same pages, and with one wave per 32 fused rows every wave
 // fetches every page for itself: a 2048-row chunk over 16 K tokens pulls 27 GB out of the L2
@@ -498,6 +498,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
 // pages; each wave keeps its quarter of one page in flight.  An operand read from LDS must
 // feed two row blocks: four waves reading one block's worth each would ask the LDS for
 // twice what it delivers.
+// The same with two waves per workgroup, each fetching half a page, serves verify batches of
+// 33 to 96 fused rows per lane (a chain of 8 rows or a tree of 16 nodes for a group of 6):
+// the one-wave kernels give such a lane two or three waves that each read every page, and
+// on these formats the reading is what they wait for.
 constexpr uint32_t kGroupWaves = 4;
 
 // The workgroup's barrier between pairs of pages: a wave's LDS writes are done (the LDS
@@ -511,35 +515,40 @@ struct GroupOperands {
   u32x4 keys[2][8][64];  // [token block][dims block][lane]
   u32x4 values[16][64];  // [dims block][lane]
 };
-template <uint32_t FMT>
-struct GroupShare {  // a wave's quarter of a page as loaded: dims blocks 2w, 2w + 1 of the keys,
-                     // dims blocks 4w .. 4w + 3 of the values
-  uint32_t k[2][2][Wide<FMT>::kDwords];  // [token block][dims block of the pair]
-  uint32_t v[4][Wide<FMT>::kDwords];
+template <uint32_t FMT, uint32_t W>
+struct GroupShare {  // wave w's share of a page as loaded, W waves: dims blocks (8 / W) w .. of the
+                     // keys, dims blocks (16 / W) w .. of the values
+  static constexpr uint32_t kKeyBlocks = 8 / W, kValueBlocks = 16 / W;
+  uint32_t k[2][kKeyBlocks][Wide<FMT>::kDwords];  // [token block][dims block of the share]
+  uint32_t v[kValueBlocks][Wide<FMT>::kDwords];
 };
 
-template <uint32_t FMT, bool REUSED>
-__device__ __forceinline__ void fetch_share(GroupShare<FMT> &r, const PagePlace &p, uint32_t wave,
+template <uint32_t FMT, uint32_t W, bool REUSED>
+__device__ __forceinline__ void fetch_share(GroupShare<FMT, W> &r, const PagePlace &p, uint32_t wave,
                                             uint32_t t, uint32_t g) {
   constexpr uint32_t B = Wide<FMT>::kBytes;
+  constexpr uint32_t KB = GroupShare<FMT, W>::kKeyBlocks, VB = GroupShare<FMT, W>::kValueBlocks;
 #pragma unroll
   for (uint32_t tb = 0; tb < 2; ++tb) {
     const uint8_t *row = p.keys + (8 * (t >> 2) + 4 * tb + (t & 3)) * kD * B;
     if constexpr (Wide<FMT>::kByte) {
-      const u32x4 x = load_streaming<u32x4, REUSED>(row + 64 * wave + 16 * g);  // dims blocks 2w, 2w + 1
-      r.k[tb][0][0] = x[0], r.k[tb][0][1] = x[1], r.k[tb][1][0] = x[2], r.k[tb][1][1] = x[3];
+#pragma unroll
+      for (uint32_t c = 0; c < KB; c += 2) {  // one 16-byte load holds two dims blocks
+        const u32x4 x = load_streaming<u32x4, REUSED>(row + key_dims<FMT>(KB * wave + c, g));
+        r.k[tb][c][0] = x[0], r.k[tb][c][1] = x[1], r.k[tb][c + 1][0] = x[2], r.k[tb][c + 1][1] = x[3];
+      }
     } else {
 #pragma unroll
-      for (uint32_t c = 0; c < 2; ++c) {
-        const u32x4 x = load_streaming<u32x4, REUSED>(row + key_dims<FMT>(2 * wave + c, g) * B);
+      for (uint32_t c = 0; c < KB; ++c) {
+        const u32x4 x = load_streaming<u32x4, REUSED>(row + key_dims<FMT>(KB * wave + c, g) * B);
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) r.k[tb][c][i] = x[i];
       }
     }
   }
 #pragma unroll
-  for (uint32_t i = 0; i < 4; ++i) {
-    const uint8_t *at = p.values + ((16 * (4 * wave + i) + t) * kPage + 8 * g) * B;
+  for (uint32_t i = 0; i < VB; ++i) {
+    const uint8_t *at = p.values + ((16 * (VB * wave + i) + t) * kPage + 8 * g) * B;
     if constexpr (Wide<FMT>::kByte) {
       const u32x2 x = load_streaming<u32x2, REUSED>(at);
       r.v[i][0] = x[0], r.v[i][1] = x[1];
@@ -556,25 +565,25 @@ __device__ __forceinline__ u32x4 share_operand(const uint32_t (&raw)[Wide<FMT>::
   else if constexpr (Wide<FMT>::kInt8) return int8_operand(raw[0], raw[1]);
   else return u32x4{raw[0], raw[1], raw[2], raw[3]};
 }
-template <uint32_t FMT>
-__device__ __forceinline__ void stage_share(GroupOperands &page, const GroupShare<FMT> &r, uint32_t wave,
+template <uint32_t FMT, uint32_t W>
+__device__ __forceinline__ void stage_share(GroupOperands &page, const GroupShare<FMT, W> &r, uint32_t wave,
                                             uint32_t lane) {
+  constexpr uint32_t KB = GroupShare<FMT, W>::kKeyBlocks, VB = GroupShare<FMT, W>::kValueBlocks;
 #pragma unroll
   for (uint32_t tb = 0; tb < 2; ++tb)
 #pragma unroll
-    for (uint32_t c = 0; c < 2; ++c) page.keys[tb][2 * wave + c][lane] = share_operand<FMT>(r.k[tb][c]);
+    for (uint32_t c = 0; c < KB; ++c) page.keys[tb][KB * wave + c][lane] = share_operand<FMT>(r.k[tb][c]);
 #pragma unroll
-  for (uint32_t i = 0; i < 4; ++i) page.values[4 * wave + i][lane] = share_operand<FMT>(r.v[i]);
+  for (uint32_t i = 0; i < VB; ++i) page.values[VB * wave + i][lane] = share_operand<FMT>(r.v[i]);
 }
 
-// NB blocks of 16 fused rows per wave; the lane's fused rows are dealt to the four waves in
-// equal runs of ceil(M / 4) (at most 16 NB).
-template <uint32_t FMT, uint32_t NB, bool REUSED>
-__global__ __launch_bounds__(64 * kGroupWaves) __attribute__((amdgpu_waves_per_eu(1, 1))) void
+// NB blocks of 16 fused rows per wave; the lane's fused rows are dealt to the W waves in
+// equal runs of ceil(M / W) (at most 16 NB).
+template <uint32_t FMT, uint32_t NB, uint32_t W, bool REUSED>
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 1))) void
 group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
                   float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
   constexpr bool kFp8 = Wide<FMT>::kFp8, kInt8 = Wide<FMT>::kInt8, kByte = Wide<FMT>::kByte;
-  constexpr uint32_t W = kGroupWaves;
   __shared__ GroupOperands shared_page[4];
   const uint32_t item = blockIdx.x, head = blockIdx.y;
   uint32_t li;
@@ -641,7 +650,7 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
 
   const uint64_t *const entries = l.table + begin;
   const uint32_t count = end - begin, last_slot = count - 1;
-  GroupShare<FMT> raw;  // this wave's quarter of the page two slots on
+  GroupShare<FMT, W> raw;  // this wave's share of the page two slots on
   // bf16 pages: a page's entry is read a turn before the loads that need it, since one wave
   // per SIMD has nothing else to run while a scalar load is on its way.  With the byte
   // formats' conversions to fill that time the early read measured 10 % slower, and they
@@ -653,10 +662,10 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
     entry_ahead = scalar_entry(entries, min(following, last_slot));
     return entry;
   };
-  auto fetch = [&](GroupShare<FMT> &set, uint64_t entry) {
+  auto fetch = [&](GroupShare<FMT, W> &set, uint64_t entry) {
     const PagePlace p = place_page<FMT>(entry, head, H, a.kv.offset, ro);
     asm volatile("");
-    fetch_share<FMT, REUSED>(set, p, wave, t, g);
+    fetch_share<FMT, W, REUSED>(set, p, wave, t, g);
     asm volatile("");
   };
   // The scales of a byte format's page, by every wave for its own lanes: they are few, and
@@ -794,9 +803,9 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
 
   // The first two pages into the first two copies.
   const uint32_t first_masked = l.committed / kPage;
-  stage_share<FMT>(shared_page[0], raw, wave, lane);
+  stage_share<FMT, W>(shared_page[0], raw, wave, lane);
   fetch(raw, entry1);
-  stage_share<FMT>(shared_page[1], raw, wave, lane);
+  stage_share<FMT, W>(shared_page[1], raw, wave, lane);
   uint64_t carried = next_entry(3);  // the entry of the page in the raw registers
   fetch(raw, carried);
   group_barrier();
@@ -808,14 +817,14 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
   // and no branch around the loads, so every wait names exactly the loads it needs.
   auto pair = [&](const GroupOperands &now0, const GroupOperands &now1, GroupOperands &next0,
                   GroupOperands &next1, uint32_t slot) __attribute__((always_inline)) {
-    stage_share<FMT>(next0, raw, wave, lane);
+    stage_share<FMT, W>(next0, raw, wave, lane);
     const uint64_t entry_odd = next_entry(slot + 4);  // of slot + 3
     fetch(raw, entry_odd);
     if (computes && slot < count)
       attend_page(now0, begin + slot, ks_even, vs_even, begin + slot >= first_masked);
     fetch_scales(ks_even, vs_even, carried);  // of slot + 2
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    stage_share<FMT>(next1, raw, wave, lane);
+    stage_share<FMT, W>(next1, raw, wave, lane);
     carried = next_entry(slot + 5);  // of slot + 4
     fetch(raw, carried);
     if (computes && slot + 1 < count)
@@ -903,25 +912,36 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   // The regular tiles of a chunked prefill (tile_rows > 0) walk the same pages
   // over and over: their loads may stay in the caches.
   const bool reused = tile_rows > 0;
+#define KVX_GROUP(FMT, NB, W, REUSED)                                                             \
+  launch_matrix_attention(group_wide_kernel<FMT, NB, W, REUSED>, "group_wide_kernel", 16 * NB * W, 64 * W, \
+                          s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks, \
+                          row_stride, lane_stride, workspace, workspace_bytes, stream, nullptr,     \
+                          tile_rows, epilogue)
+#define KVX_GROUP_FORMATS(NB, W, REUSED)                                                          \
+  (format == KVX_FMT_BF16   ? KVX_GROUP(KVX_FMT_BF16, NB, W, REUSED)                                \
+   : format == KVX_FMT_INT8 ? KVX_GROUP(KVX_FMT_INT8, NB, W, REUSED)                                \
+                            : KVX_GROUP(KVX_FMT_FP8E4M3, NB, W, REUSED))
   // many_tiles == 2: lanes of several prefill tiles each, for a workgroup of four waves
-  // that shares every page through LDS, two row blocks per wave: up to 128 fused rows.
+  // that shares every page through LDS, two or three row blocks per wave: up to 192 fused rows.
   if (many_tiles == 2) {
     if (!tile_rows || M > 48u * kGroupWaves) return 1;
-#define KVX_GROUP(FMT, NB)                                                                        \
-  launch_matrix_attention(group_wide_kernel<FMT, NB, true>, "group_wide_kernel", 16 * NB * kGroupWaves, \
-                          64 * kGroupWaves, s, kv, query_heads, queries, output, page_tables, lanes, \
-                          n_lanes, row_masks, row_stride, lane_stride, workspace, workspace_bytes,  \
-                          stream, nullptr, tile_rows, epilogue)
-    if (M > 32u * kGroupWaves) {
-      if (format == KVX_FMT_BF16) return KVX_GROUP(KVX_FMT_BF16, 3);
-      if (format == KVX_FMT_INT8) return KVX_GROUP(KVX_FMT_INT8, 3);
-      return KVX_GROUP(KVX_FMT_FP8E4M3, 3);
-    }
-    if (format == KVX_FMT_BF16) return KVX_GROUP(KVX_FMT_BF16, 2);
-    if (format == KVX_FMT_INT8) return KVX_GROUP(KVX_FMT_INT8, 2);
-    return KVX_GROUP(KVX_FMT_FP8E4M3, 2);
-#undef KVX_GROUP
+    if (M > 32u * kGroupWaves) return KVX_GROUP_FORMATS(3, 4, true);
+    return KVX_GROUP_FORMATS(2, 4, true);
   }
+  // Verify lanes of more than 64 fused rows (a tree of 16 nodes for a group of 6): four
+  // waves share the lane's pages, up to 32 or 48 rows each (16 nodes, batch 4 x 65 536 tokens:
+  // bf16 456 -> 270 us, int8 436 -> 307 us).  33 .. 64 rows (a chain of 8): two waves that
+  // fetch half a page each, on bf16 pages only (706 -> 559 us on a batch of 32); with one
+  // page in flight per wave the byte formats, which read half as much, were slower that way
+  // (int8 468 -> 628 us) and keep a wave per 32 rows.  Two waves with three blocks each and
+  // half a page in flight spill 21 to 45 registers.
+  // A verify lane holds 128 fused rows at most.
+  if (!tile_rows && !many_tiles && M > 32 && M <= 32u * kGroupWaves) {
+    if (M > 64) return KVX_GROUP_FORMATS(2, 4, false);
+    if (format == KVX_FMT_BF16) return KVX_GROUP(KVX_FMT_BF16, 2, 2, false);
+  }
+#undef KVX_GROUP_FORMATS
+#undef KVX_GROUP
   if (format == KVX_FMT_BF16) {
     if (M > 16) return reused ? KVX_WIDE(KVX_FMT_BF16, 2, 1, true) : KVX_WIDE(KVX_FMT_BF16, 2, 1, false);
     return reused ? KVX_WIDE(KVX_FMT_BF16, 1, 1, true) : KVX_WIDE(KVX_FMT_BF16, 1, 1, false);

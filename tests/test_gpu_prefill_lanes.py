@@ -2,7 +2,9 @@
 whose four waves share every page through LDS; shorter chunks run a wave per tile or pair of
 tiles.  Both walk the pages of a row in the same order with the same arithmetic, so a long
 chunk in one call must give, bit for bit, the rows of the same chunk attended in pieces of
-56 rows.  The pieces are the path that tests/test_gpu_attention.py holds against the
+56 rows.  Verify lanes of more than 64 fused rows (bf16 pages: more than 32) run on the same kernels;
+the layouts of tests/test_gpu_attention.py and tests/test_gpu_geometries.py give them 64, 96 and 128
+rows, the most a verify lane may hold.  The pieces are the path that tests/test_gpu_attention.py holds against the
 oracle.  Under several splits every split rounds its weights against its own running maximum,
 so those results are held against the oracle with the same splits instead."""
 import numpy as np
@@ -69,3 +71,4 @@ def test_long_chunk_under_several_splits_matches_oracle(fmt, heads, group, commi
         A.prefill_case(fmt, committed, rows, forced_splits=splits)
     finally:
         A.H, A.G, A.QH = saved
+
