@@ -320,7 +320,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
 
   // One page out of set r; keys_consumed() runs when its keys have been read for
   // the last time.
+  // Pages that lie wholly inside the committed tokens are seen whole by every row; only
+  // from this page on does a token have to be tested (one copy of the page code serves
+  // both, the test itself is skipped).  The one-block forms wait for memory, not for this
+  // arithmetic, and two of them spill with the branch: they test every token.
+  const uint32_t first_masked = l.committed / kPage;
   auto attend_page = [&](PageSet &r, uint32_t page, auto keys_consumed) {
+      const bool check_tokens = page >= first_masked;
       // ---- q.k ----
       f32x4 s[NB][2];
 #pragma unroll
@@ -350,17 +356,30 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
 #pragma unroll
       for (uint32_t nb = 0; nb < NB; ++nb) {
         float score[8], local_max = -INFINITY;
-        bool live[8];
 #pragma unroll
         for (uint32_t i = 0; i < 8; ++i) {
           const uint32_t tb = i >> 2, rr = i & 3;
           float v = s[nb][tb][rr] * kUnscale;
           if constexpr (kByte) v *= page_ks[tb][rr];
-          v *= score_scale;
-          live[i] = sight[nb].sees(first_token + 8 * g + 4 * tb + rr);
-          score[i] = live[i] ? v : -INFINITY;
-          local_max = fmaxf(local_max, score[i]);
+          score[i] = v * score_scale;
         }
+        // A token the row does not see scores -inf, and its weight below comes out as
+        // exp(-inf) = 0 by itself.  (The one-block forms, which run two waves per SIMD on the
+        // byte formats, spill with this form of it and select per token instead.)
+        bool live[8];
+        if constexpr (NB == 1) {
+#pragma unroll
+          for (uint32_t i = 0; i < 8; ++i) {
+            live[i] = sight[nb].sees(first_token + 8 * g + 4 * (i >> 2) + (i & 3));
+            score[i] = live[i] ? score[i] : -INFINITY;
+          }
+        } else if (check_tokens) {
+#pragma unroll
+          for (uint32_t i = 0; i < 8; ++i)
+            if (!sight[nb].sees(first_token + 8 * g + 4 * (i >> 2) + (i & 3))) score[i] = -INFINITY;
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i) local_max = fmaxf(local_max, score[i]);
         local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
         local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
         const float next_max = fmaxf(row_max[nb], local_max);
@@ -368,12 +387,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES
         const float rescale = next_max == row_max[nb]
                                   ? 1.0f
                                   : __builtin_amdgcn_exp2f((row_max[nb] - next_max) * kLog2e);
+        // A row that still has seen nothing measures from 0: -inf - -inf is no number.
+        const float reference = (NB == 1 || next_max != -INFINITY) ? next_max : 0.0f;
         float weight[8], page_sum = 0.0f;
 #pragma unroll
         for (uint32_t i = 0; i < 8; ++i) {
           // The difference first, so the page's maximum gets exactly 1.
-          float p = __builtin_amdgcn_exp2f((score[i] - next_max) * kLog2e);
-          p = live[i] ? p : 0.0f;
+          float p = __builtin_amdgcn_exp2f((score[i] - reference) * kLog2e);
+          if constexpr (NB == 1) p = live[i] ? p : 0.0f;
           page_sum += p;
           weight[i] = kByte ? p * page_vs[i >> 2][i & 3] : p;
         }
