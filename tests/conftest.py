@@ -12,8 +12,9 @@ def pytest_configure(config):
 
 def pytest_terminal_summary(terminalreporter):
     """How often the attention checks needed their one allowance (a row one rounding flip
-    away from the oracle, proven by recomputation): per check and in total; also written to
-    gpurun_out/parity_allowance.txt where that folder exists."""
+    away from the oracle, proven by recomputation): per check and in total; also written as
+    parity_allowance.txt into the folder KVX_TEST_REPORT_DIR names (default: the run's output
+    folder at the repository root) where that folder exists."""
     gpulib = sys.modules.get("gpulib")
     log = getattr(gpulib, "ALLOWANCE_LOG", None)
     if not log:
@@ -24,7 +25,7 @@ def pytest_terminal_summary(terminalreporter):
              f"{explained} of {rows} rows in {len(log)} checks"]
     lines += [f"  {n:4d} of {total:6d}  {label}" for label, n, total in log if n]
     terminalreporter.write_line("\n".join(lines))
-    out = os.path.join(ROOT, "gpurun_out")
+    out = os.environ.get("KVX_TEST_REPORT_DIR", os.path.join(ROOT, "gpurun_out"))
     if os.path.isdir(out):
         with open(os.path.join(out, "parity_allowance.txt"), "w") as f:
             f.write("\n".join(lines) + "\n")
