@@ -599,13 +599,20 @@ __device__ __forceinline__ void stage_share(GroupOperands &page, const GroupShar
 }
 
 // NB blocks of 16 fused rows per wave; the lane's fused rows are dealt to the W waves in
-// equal runs of ceil(M / W) (at most 16 NB).
-template <uint32_t FMT, uint32_t NB, uint32_t W, bool REUSED>
+// equal runs of ceil(M / W) (at most 16 NB).  SETS register sets hold a wave's share of
+// the pages on their way: one, whose loads have a page time to arrive, for pages that come
+// out of the caches (prefill) and for bf16, whose share is 32 to 64 registers; two, with
+// two page times, for the byte formats' verify lanes, whose pages come from HBM.
+// COPIES staged pages in LDS: four (128 KiB, a barrier every second page) where the
+// workgroup's four waves fill the CU anyway; two (64 KiB, a barrier per page) for workgroups
+// of two waves, so that two of them fit a CU and no SIMD stays empty.
+template <uint32_t FMT, uint32_t NB, uint32_t W, bool REUSED, uint32_t SETS = 1, uint32_t COPIES = 4>
 __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(1, 1))) void
 group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
                   float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
   constexpr bool kFp8 = Wide<FMT>::kFp8, kInt8 = Wide<FMT>::kInt8, kByte = Wide<FMT>::kByte;
-  __shared__ GroupOperands shared_page[4];
+  static_assert(COPIES == 4 || (COPIES == 2 && SETS == 1), "two copies: one set of page registers");
+  __shared__ GroupOperands shared_page[COPIES];
   const uint32_t item = blockIdx.x, head = blockIdx.y;
   uint32_t li;
   const DecodeLane l = lane_of_item(a, item, li);
@@ -671,7 +678,8 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
 
   const uint64_t *const entries = l.table + begin;
   const uint32_t count = end - begin, last_slot = count - 1;
-  GroupShare<FMT, W> raw;  // this wave's share of the page two slots on
+  static_assert(SETS == 1 || (SETS == 2 && Wide<FMT>::kByte), "two sets of page registers: byte formats only");
+  GroupShare<FMT, W> raw[SETS];  // this wave's share of the pages on their way
   // bf16 pages: a page's entry is read a turn before the loads that need it, since one wave
   // per SIMD has nothing else to run while a scalar load is on its way.  With the byte
   // formats' conversions to fill that time the early read measured 10 % slower, and they
@@ -702,7 +710,8 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
     }
   };
   const uint64_t entry0 = next_entry(1), entry1 = next_entry(2);
-  fetch(raw, entry0);
+  fetch(raw[0], entry0);
+  if constexpr (SETS == 2) fetch(raw[1], entry1);
   fetch_scales(ks_even, vs_even, entry0);
   fetch_scales(ks_odd, vs_odd, entry1);
 
@@ -822,40 +831,74 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
     }
   };
 
-  // The first two pages into the first two copies.
   const uint32_t first_masked = l.committed / kPage;
-  stage_share<FMT, W>(shared_page[0], raw, wave, lane);
-  fetch(raw, entry1);
-  stage_share<FMT, W>(shared_page[1], raw, wave, lane);
-  uint64_t carried = next_entry(3);  // the entry of the page in the raw registers
-  fetch(raw, carried);
-  group_barrier();
-  // Four copies, two pages between barriers: while slots i and i + 1 are multiplied out of
-  // one pair of copies, slots i + 2 and i + 3 go from the raw registers into the other pair,
-  // each a page time after its loads were sent (past the end: the last page again, staged
-  // into copies nobody reads).  A barrier per page cost 5 % more: the waves leave it
-  // together and read their operands at the same time.  Four slots per turn of the loop
-  // and no branch around the loads, so every wait names exactly the loads it needs.
-  auto pair = [&](const GroupOperands &now0, const GroupOperands &now1, GroupOperands &next0,
-                  GroupOperands &next1, uint32_t slot) __attribute__((always_inline)) {
-    stage_share<FMT, W>(next0, raw, wave, lane);
-    const uint64_t entry_odd = next_entry(slot + 4);  // of slot + 3
-    fetch(raw, entry_odd);
-    if (computes && slot < count)
-      attend_page(now0, begin + slot, ks_even, vs_even, begin + slot >= first_masked);
-    fetch_scales(ks_even, vs_even, carried);  // of slot + 2
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    stage_share<FMT, W>(next1, raw, wave, lane);
-    carried = next_entry(slot + 5);  // of slot + 4
-    fetch(raw, carried);
-    if (computes && slot + 1 < count)
-      attend_page(now1, begin + slot + 1, ks_odd, vs_odd, begin + slot + 1 >= first_masked);
-    fetch_scales(ks_odd, vs_odd, entry_odd);
+  if constexpr (COPIES == 2) {
+    // Two copies: while slot i is multiplied out of one, slot i + 1 goes from the raw
+    // registers into the other and the registers are sent for slot i + 2; a barrier per page.
+    stage_share<FMT, W>(shared_page[0], raw[0], wave, lane);
+    fetch(raw[0], entry1);
     group_barrier();
-  };
-  for (uint32_t slot = 0; slot < count; slot += 4) {
-    pair(shared_page[0], shared_page[1], shared_page[2], shared_page[3], slot);
-    pair(shared_page[2], shared_page[3], shared_page[0], shared_page[1], slot + 2);
+    auto turn = [&](const GroupOperands &now, GroupOperands &next, uint32_t slot, f32x4 (&ks)[2],
+                    f32x4 (&vs)[2]) __attribute__((always_inline)) {
+      stage_share<FMT, W>(next, raw[0], wave, lane);  // slot + 1
+      const uint64_t entry = next_entry(slot + 3);  // of slot + 2
+      fetch(raw[0], entry);
+      if (computes && slot < count) attend_page(now, begin + slot, ks, vs, begin + slot >= first_masked);
+      fetch_scales(ks, vs, entry);
+      group_barrier();
+    };
+    for (uint32_t slot = 0; slot < count; slot += 2) {
+      turn(shared_page[0], shared_page[1], slot, ks_even, vs_even);
+      turn(shared_page[1], shared_page[0], slot + 1, ks_odd, vs_odd);
+    }
+  } else {
+    // The first two pages into the first two copies; the entries of the pages whose operands are on their way (slots + 2 and + 3 of a pair):
+    // their scales are asked for a page time later.
+    uint64_t held_even, held_odd = 0;
+    stage_share<FMT, W>(shared_page[0], raw[0], wave, lane);
+    if constexpr (SETS == 1) {
+      fetch(raw[0], entry1);
+      stage_share<FMT, W>(shared_page[1], raw[0], wave, lane);
+      held_even = next_entry(3);
+      fetch(raw[0], held_even);
+    } else {
+      held_even = next_entry(3);
+      fetch(raw[0], held_even);
+      stage_share<FMT, W>(shared_page[1], raw[1], wave, lane);
+      held_odd = next_entry(4);
+      fetch(raw[1], held_odd);
+    }
+    group_barrier();
+    // Four copies, two pages between barriers: while slots i and i + 1 are multiplied out of
+    // one pair of copies, slots i + 2 and i + 3 go from the raw registers into the other pair,
+    // each one page time (two with two sets) after its loads were sent (past the end: the last
+    // page again, staged into copies nobody reads).  A barrier per page cost 5 % more: the
+    // waves leave it together and read their operands at the same time.  Four slots per turn
+    // of the loop and no branch around the loads, so every wait names exactly the loads it
+    // needs.
+    auto pair = [&](const GroupOperands &now0, const GroupOperands &now1, GroupOperands &next0,
+                    GroupOperands &next1, uint32_t slot) __attribute__((always_inline)) {
+      stage_share<FMT, W>(next0, raw[0], wave, lane);  // slot + 2
+      const uint64_t entry_a = next_entry(slot + 3 + SETS);  // of slot + 2 + SETS
+      fetch(raw[0], entry_a);
+      if (computes && slot < count)
+        attend_page(now0, begin + slot, ks_even, vs_even, begin + slot >= first_masked);
+      fetch_scales(ks_even, vs_even, held_even);  // of slot + 2
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      stage_share<FMT, W>(next1, raw[SETS - 1], wave, lane);  // slot + 3
+      const uint64_t entry_b = next_entry(slot + 4 + SETS);  // of slot + 3 + SETS
+      fetch(raw[SETS - 1], entry_b);
+      if (computes && slot + 1 < count)
+        attend_page(now1, begin + slot + 1, ks_odd, vs_odd, begin + slot + 1 >= first_masked);
+      fetch_scales(ks_odd, vs_odd, SETS == 1 ? entry_a : held_odd);  // of slot + 3
+      held_even = SETS == 1 ? entry_b : entry_a;
+      held_odd = entry_b;
+      group_barrier();
+    };
+    for (uint32_t slot = 0; slot < count; slot += 4) {
+      pair(shared_page[0], shared_page[1], shared_page[2], shared_page[3], slot);
+      pair(shared_page[2], shared_page[3], shared_page[0], shared_page[1], slot + 2);
+    }
   }
   if (!computes) return;
 
@@ -933,8 +976,8 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   // The regular tiles of a chunked prefill (tile_rows > 0) walk the same pages
   // over and over: their loads may stay in the caches.
   const bool reused = tile_rows > 0;
-#define KVX_GROUP(FMT, NB, W, REUSED)                                                             \
-  launch_matrix_attention(group_wide_kernel<FMT, NB, W, REUSED>, "group_wide_kernel", 16 * NB * W, 64 * W, \
+#define KVX_GROUP(FMT, NB, W, REUSED, ...)                                                        \
+  launch_matrix_attention(group_wide_kernel<FMT, NB, W, REUSED, ##__VA_ARGS__>, "group_wide_kernel", 16 * NB * W, 64 * W, \
                           s, kv, query_heads, queries, output, page_tables, lanes, n_lanes, row_masks, \
                           row_stride, lane_stride, workspace, workspace_bytes, stream, nullptr,     \
                           tile_rows, epilogue)
@@ -949,17 +992,19 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
     if (M > 32u * kGroupWaves) return KVX_GROUP_FORMATS(3, 4, true);
     return KVX_GROUP_FORMATS(2, 4, true);
   }
-  // Verify lanes of more than 64 fused rows (a tree of 16 nodes for a group of 6): four
-  // waves share the lane's pages, up to 32 or 48 rows each (16 nodes, batch 4 x 65 536 tokens:
-  // bf16 456 -> 270 us, int8 436 -> 307 us).  33 .. 64 rows (a chain of 8): two waves that
-  // fetch half a page each, on bf16 pages only (706 -> 559 us on a batch of 32); with one
-  // page in flight per wave the byte formats, which read half as much, were slower that way
-  // (int8 468 -> 628 us) and keep a wave per 32 rows.  Two waves with three blocks each and
+  // Verify lanes of more than 32 fused rows: the waves that the lane needs anyway share its
+  // pages.  65 .. 128 rows (a tree of 16 nodes for a group of 6): four waves, four LDS copies
+  // (16 nodes, batch 4 x 65 536 tokens: bf16 456 -> 270 us, int8 436 -> 282 us with two sets of
+  // page registers).  33 .. 64 rows (a chain of 8): two waves that fetch half a page each, with
+  // two LDS copies so that two such workgroups fit a CU (batch of 32: bf16 706 -> 413 us, int8
+  // 435 -> 387 us, fp8 405 -> 343 us; with four copies, one workgroup per CU and half of the
+  // SIMDs empty, the byte formats took 550 - 650 us).  Two waves with three blocks each and
   // half a page in flight spill 21 to 45 registers.
   // A verify lane holds 128 fused rows at most.
   if (!tile_rows && !many_tiles && M > 32 && M <= 32u * kGroupWaves) {
-    if (M > 64) return KVX_GROUP_FORMATS(2, 4, false);
-    if (format == KVX_FMT_BF16) return KVX_GROUP(KVX_FMT_BF16, 2, 2, false);
+    if (format == KVX_FMT_BF16) return M > 64 ? KVX_GROUP(KVX_FMT_BF16, 2, 4, false) : KVX_GROUP(KVX_FMT_BF16, 2, 2, false, 1, 2);
+    if (format == KVX_FMT_INT8) return M > 64 ? KVX_GROUP(KVX_FMT_INT8, 2, 4, false, 2) : KVX_GROUP(KVX_FMT_INT8, 2, 2, false, 1, 2);
+    return M > 64 ? KVX_GROUP(KVX_FMT_FP8E4M3, 2, 4, false, 2) : KVX_GROUP(KVX_FMT_FP8E4M3, 2, 2, false, 1, 2);
   }
 #undef KVX_GROUP_FORMATS
 #undef KVX_GROUP

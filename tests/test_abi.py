@@ -227,8 +227,8 @@ def test_hot_kernels_stay_out_of_scratch_memory():
     # per wave): one wave per SIMD with all 512 registers; the byte formats' three-block forms
     # park a few set-up values in scratch memory, none of them touched inside the page loop
     # (no scratch access in the loop's assembly when this bound was set)
-    # (the same kernels with loads that do not stay in the caches serve tree verify, and the
-    # bf16 one with two waves a chain of 8 rows)
+    # (the same kernels with loads that do not stay in the caches serve tree verify, and forms
+    # with two waves and two LDS copies a chain of 8 rows)
     for fmt in (1, 2, 4):
         for blocks in (2, 3):
             for reused in ((0, 1) if blocks == 2 else (1,)):
@@ -237,8 +237,9 @@ def test_hot_kernels_stay_out_of_scratch_memory():
                     assert r["vgprs_spill"] <= 10, (fmt, blocks, r)
                 else:
                     assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, (fmt, blocks, r)
-    r = one("group_wide_kernelILj2ELj2ELj2ELb0E")
-    assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, r
+    for fmt in (1, 2, 4):
+        r = one(f"group_wide_kernelILj{fmt}ELj2ELj2ELb0E")
+        assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, r
     # the kernels whose accumulators fill the second register file (48-row verify, two-block
     # bf16): since their rescaling names the accumulators there, nothing spills
     for fragment in ("verify48_int4_kernel", "attend_wide_kernelILj2ELj2ELj1ELb0E",
