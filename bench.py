@@ -86,10 +86,10 @@ def parse():
                          "prefix, the matrix-core paths (profiling)")
     ap.add_argument("--format", choices=["bf16", "fp8", "int8", "int4"], default=None,
                     help="page format of the prefill workload (default bf16) and of the shared-prefix "
-                         "workload (default int4; no fp8)")
+                         "and tree-verify workloads (default int4; no fp8)")
     args = ap.parse_args()
     if args.format is None:
-        args.format = "int4" if args.workload == "shared-prefix" else "bf16"
+        args.format = "int4" if args.workload in ("shared-prefix", "tree-verify") else "bf16"
     return args
 
 
@@ -310,10 +310,14 @@ def tree_verify(args):
     rng = np.random.default_rng(args.seed)
     lanes, context, nodes = 4, 65536, 16
     n_pages = (context + nodes + 31) // 32
-    layout = kvx.Layout(LAYERS, H, D, kvx.INT4, 0.0)
+    if args.format not in ("int4", "int8", "bf16"):
+        sys.exit("tree verify runs on int4 (BASELINE configs[4]), int8 or bf16 pages")
+    fmt = {"int4": kvx.INT4, "int8": kvx.INT8, "bf16": kvx.BF16}[args.format]
+    bytes_per_token = {"int4": BYTES_PER_TOKEN_LAYER, "int8": 2080, "bf16": 4096}[args.format]
+    layout = kvx.Layout(LAYERS, H, D, fmt, 0.0)
     extent_pages = L.kvx_layout_largest_extent_pages(C.byref(layout))
     extents = -(-lanes * n_pages // extent_pages)
-    storage = kvx.Storage(LAYERS, H, D, kvx.INT4, extents * extent_pages, extent_pages, aligned=True)
+    storage = kvx.Storage(LAYERS, H, D, fmt, extents * extent_pages, extent_pages, aligned=True)
     storage.allocate_all()
     ids = rng.permutation(extents * extent_pages)[:lanes * n_pages].astype(np.uint32)
     tables = [storage.table(ids[i * n_pages:(i + 1) * n_pages]) for i in range(lanes)]
@@ -352,7 +356,7 @@ def tree_verify(args):
     chunk_v = torch.randn((lanes, H, D, 32), generator=gen, device="cuda").bfloat16()
     queries = torch.randn((lanes, H, 32, G, D), generator=gen, device="cuda").bfloat16()
     output = torch.zeros_like(queries)
-    splits = args.verify_splits or kvx.verify_plan([context] * lanes, nodes, H, QH)[0]
+    splits = args.verify_splits or kvx.verify_plan([context] * lanes, nodes, H, QH, fmt)[0]
     cp = [kvx.ChunkParams(context, nodes, 32, n_pages) for _ in range(lanes)]
     vp = [kvx.VerifyParams(context, n_pages, kvx.KvLayer(), splits, splits, nodes, 16, 0.0)
           for _ in range(lanes)]
@@ -390,29 +394,33 @@ def tree_verify(args):
     kernel_ms = time_split()
     visible = lanes * (context + nodes)
     flops = 4 * D * (nodes * QH) * visible  # q.k and p.v, multiply and add, every row over every token
-    kv_bytes = visible * BYTES_PER_TOKEN_LAYER
+    kv_bytes = visible * bytes_per_token
     achieved = flops / (kernel_ms * 1e-3) / 1e12
     result = {
-        "metric": "int4 tree verify (16-node trees, batch 4 x 65536 tokens): verified draft tokens/s",
+        "metric": args.format + " tree verify (16-node trees, batch 4 x 65536 tokens): verified draft tokens/s",
         "value": round(lanes * nodes * args.steps / wall, 1), "unit": "draft tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int4 pages, bf16 MFMA, fp32 accumulate", "data": "synthetic",
-        "config": {"workload": "BASELINE configs[4]: speculative tree verify on int4 KV, batch 4, "
+        "dtype": {"int4": "int4 pages, bf16 MFMA", "int8": "int8 pages, fp16 MFMA",
+                  "bf16": "bf16 pages, bf16 MFMA"}[args.format] + ", fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[4]: speculative tree verify on " + args.format + " KV, batch 4, "
                                "contexts 65536, 16-node trees (branching <= 3), 16 layers: append 16 "
                                "rows + masked verify per layer, then path compaction over all layers",
-                   "batch": lanes, "layers": LAYERS, "splits_per_sequence": int(splits),
-                   "seed": args.seed},
+                   "batch": lanes, "layers": LAYERS, "format": args.format,
+                   "splits_per_sequence": int(splits), "seed": args.seed},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": None,
-                     "kernel": "verify48_int4_kernel (split kernel of verify attention, 48 fused rows per wave), one layer per launch",
+                     "kernel": ("verify48_int4_kernel (split kernel of verify attention, 48 fused rows per wave)"
+                                if args.format == "int4" else
+                                "group_wide_kernel (split kernel of verify attention, four waves of 24 fused "
+                                "rows that share every page through LDS)") + ", one layer per launch",
                      "flops_per_launch": flops, "ms_per_launch": round(kernel_ms, 4),
                      "kv_gbs": round(kv_bytes / (kernel_ms * 1e-3) / 1e9, 1)},
         "cpu_baseline": None,
     }
     storage.close()
-    if args.cpu_seconds > 0:
+    if args.cpu_seconds > 0 and args.format == "int4":
         result["cpu_baseline"] = cpu_tree_verify(args.seed, context, nodes, masks, args.cpu_seconds)
     print(json.dumps(result))
 
