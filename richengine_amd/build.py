@@ -1,4 +1,5 @@
 """Builds libkvx.so (HIP kernels + C ABI) for gfx950, in-tree."""
+import concurrent.futures
 import json
 import os
 import re
@@ -43,14 +44,20 @@ def build(verbose=True, lib=LIB, extra_flags=(), tag=""):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objects, resources = [], {}
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
-    for src in SOURCES:
+    def compile_one(src):
         obj = os.path.join(HERE, "build", src + tag + ".o")
         cmd = [hipcc, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + FLAGS + list(extra_flags)
         if src.endswith(".hip"):
             cmd.append("-Rpass-analysis=kernel-resource-usage")
         if verbose:
             print(" ".join(cmd), flush=True)
-        done = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+        return obj, cmd, subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+
+    # the sources compile side by side (the kernel files take most of the time), and their
+    # remarks are read in the order of SOURCES
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+        compiled = list(pool.map(compile_one, SOURCES))
+    for obj, cmd, done in compiled:
         # the remarks and the host pass's note about the packed-fp32 feature are not warnings
         for line in done.stderr.splitlines():
             if "kernel-resource-usage" in line or "packed-fp32-ops" in line:
