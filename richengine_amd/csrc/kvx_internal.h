@@ -157,7 +157,9 @@ constexpr uint32_t kGroupedPrefillRows = 64;
 inline uint32_t prefill_group_width(uint32_t format, uint32_t head_dim, uint32_t rows, uint32_t group) {
   if (format == KVX_FMT_INT4 || head_dim != 256 || rows < kGroupedPrefillRows) return 0;
   const uint32_t tile_fused = KVX_PREFILL_TILE_ROWS * group;
-  return 4 * tile_fused <= 192 ? 4u : 2 * tile_fused <= 192 ? 2u : 0u;
+  const uint32_t width = 4 * tile_fused <= 192 ? 4u : 2 * tile_fused <= 192 ? 2u : 0u;
+  // Groups of one or two query heads would leave three quarters of every wave's rows empty.
+  return width * tile_fused >= 96 ? width : 0u;
 }
 // Whether the tiles of every such lane see the same number of pages, so that a lane cut into
 // splits is each of its tiles cut into splits: lanes of four tiles (32 rows) when the chunk

@@ -158,6 +158,7 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
             if fmt != kvx.INT4 and rows >= 64:           # lanes of several tiles, a workgroup each
                 fused = 8 * (QH // H)
                 width = 4 if 4 * fused <= 192 else 2 if 2 * fused <= 192 else 0
+                width = width if width * fused >= 96 else 0
             workgroups = -(-tiles // width) * H if width else 0
             alike = width and (committed % 32 == 0 if width == 4 else
                                (committed % 16 == 0 or committed % 16 >= 9))

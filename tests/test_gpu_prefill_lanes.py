@@ -32,9 +32,14 @@ def attend(tw, td, n_pages, heads, group, q, committed, rows, splits):
     return Gp.host_u16(out)
 
 
-@pytest.mark.parametrize("fmt", WIDE)
-@pytest.mark.parametrize("heads,group", [(4, 6), (4, 4), (2, 8)])
-@pytest.mark.parametrize("committed,rows", [(0, 256), (1000, 296), (1024, 552)])
+@pytest.mark.parametrize("fmt,heads,group,committed,rows",
+                         [(fmt, heads, group, committed, rows)
+                          for fmt in WIDE for heads, group in [(4, 6), (4, 4), (2, 8)]
+                          for committed, rows in [(0, 256), (1000, 296), (1024, 552)]] +
+                         # groups at the ends of what the lanes of several tiles take: 3 query heads
+                         # (96 fused rows in four tiles), 12 (192 in two), and 2, which they leave alone
+                         [(fmt, heads, group, 1000, 296)
+                          for fmt in (ko.INT8, ko.BF16) for heads, group in [(8, 3), (2, 12), (4, 2)]])
 def test_long_chunk_is_its_short_pieces(fmt, heads, group, committed, rows):
     # 296 rows: 37 tiles, so lanes of four (or two) tiles and an odd tile on its own;
     # 1000 tokens before the chunk: its tiles start in the middle of a page
