@@ -618,6 +618,19 @@ int kv_append_attend_decode(const kvx_storage *storage, uint32_t layer, const vo
                             void *output, const uint64_t *const *page_tables,
                             const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
                             void *workspace, uint64_t workspace_bytes, void *stream);
+/* The same step with the merge of kv_attend_verify_hidden: the token is stored, the row attended and
+   the out-projection's operand written ([lane][1][query head][D]; gated by packed_qkv when that is
+   given, as described there) in one call, which is the reference's decode step with gateHidden bound
+   (ops::PagedAttention::addVerify, runtime/ops/PagedAttention.cpp:467-544; kernel
+   verify_attention_reduce_gate*, decode/paged_attention.metal:266-330).  output may be NULL.
+   Same page bytes, output and hidden rows as kv_append followed by kv_attend_verify_hidden. */
+int kv_append_attend_decode_hidden(const kvx_storage *storage, uint32_t layer, const void *chunk_keys,
+                                   const void *chunk_values, uint64_t chunk_lane_stride,
+                                   uint32_t chunk_stride, uint32_t query_heads, const void *queries,
+                                   void *output, const uint64_t *const *page_tables,
+                                   const kvx_verify_params *lanes, uint32_t n_lanes,
+                                   uint32_t row_stride, void *workspace, uint64_t workspace_bytes,
+                                   const void *packed_qkv, void *hidden, void *stream);
 
 /* Chunked prefill attention of one sequence: rows in tiles of 8, each tile
    causal over committed + its rows.  Replaces ops::PagedAttention::addPrefill

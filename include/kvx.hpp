@@ -504,7 +504,7 @@ public:
       throw std::invalid_argument("tree verify has no fused gather");
     const kv::Layout &layout = storage.layout();
     const uint64_t laneStride = uint64_t{layout.kvHeads} * kv::kVerifyChunkStride * layout.headDimension;
-    if (plan.rowCapacity == 1 && !gateHidden) {  // a decode step: one call stores the token and attends
+    if (plan.rowCapacity == 1) {  // a decode step: one call stores the token and attends
       std::vector<kv::VerifyAttentionParams> lanes(plan.lanes);
       for (uint32_t i = 0; i < plan.lanes; ++i) {
         if (chunks[i].chunk_tokens != 1 || chunks[i].chunk_stride != kv::kVerifyChunkStride)
@@ -512,10 +512,17 @@ public:
         lanes[i] = {chunks[i].committed_tokens, chunks[i].page_table_entries, {}, plan.laneSplits[i],
                     plan.splits, 1, 1, plan.scoreScale};
       }
-      check(kv_append_attend_decode(storage.handle(), layer, buffers.chunkKeys, buffers.chunkValues,
-                                    laneStride, kv::kVerifyChunkStride, plan.queryHeads, buffers.queries,
-                                    buffers.output, buffers.pageTables, lanes.data(), plan.lanes, 1,
-                                    buffers.workspace, buffers.workspaceBytes, stream));
+      if (gateHidden)
+        check(kv_append_attend_decode_hidden(storage.handle(), layer, buffers.chunkKeys, buffers.chunkValues,
+                                             laneStride, kv::kVerifyChunkStride, plan.queryHeads,
+                                             buffers.queries, buffers.output, buffers.pageTables,
+                                             lanes.data(), plan.lanes, 1, buffers.workspace,
+                                             buffers.workspaceBytes, gatePacked, gateHidden, stream));
+      else
+        check(kv_append_attend_decode(storage.handle(), layer, buffers.chunkKeys, buffers.chunkValues,
+                                      laneStride, kv::kVerifyChunkStride, plan.queryHeads, buffers.queries,
+                                      buffers.output, buffers.pageTables, lanes.data(), plan.lanes, 1,
+                                      buffers.workspace, buffers.workspaceBytes, stream));
       return;
     }
     check(kv_append(storage.handle(), layer, buffers.chunkKeys, buffers.chunkValues, buffers.pageTables,

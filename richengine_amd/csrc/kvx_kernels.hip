@@ -1849,14 +1849,17 @@ int kv_attend_decode_static(const kvx_storage *s, uint32_t layer, uint32_t query
                           row_stride, scratch, kStaticScratchBytes, stream);
 }
 
-int kv_append_attend_decode(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
-                            const void *chunk_values, uint64_t chunk_lane_stride,
-                            uint32_t chunk_stride, uint32_t query_heads, const void *queries,
-                            void *output, const uint64_t *const *page_tables,
-                            const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
-                            void *workspace, uint64_t workspace_bytes, void *stream) {
-  if (!s || !chunk_keys || !chunk_values || !queries || !output || !page_tables || !lanes ||
-      !n_lanes || !workspace)
+namespace {
+// kv_append_attend_decode and its form whose merge also writes the hidden rows (epilogue
+// given; `output` may then be null).
+int append_attend_decode(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
+                         const void *chunk_values, uint64_t chunk_lane_stride, uint32_t chunk_stride,
+                         uint32_t query_heads, const void *queries, void *output,
+                         const uint64_t *const *page_tables, const kvx_verify_params *lanes,
+                         uint32_t n_lanes, uint32_t row_stride, void *workspace,
+                         uint64_t workspace_bytes, const Epilogue *epilogue, void *stream) {
+  if (!s || !chunk_keys || !chunk_values || !queries || (!output && !epilogue) || !page_tables ||
+      !lanes || !n_lanes || !workspace)
     return fail(KVX_EINVAL, "kv_append_attend_decode: null argument or no lanes");
   if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
   if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
@@ -1881,7 +1884,8 @@ int kv_append_attend_decode(const kvx_storage *s, uint32_t layer, const void *ch
   const int fused = kvx_attend_int4_launch(s, kv, query_heads, queries, output, page_tables, lanes,
                                            n_lanes, nullptr, row_stride, lane_stride, workspace,
                                            workspace_bytes, 0, static_cast<hipStream_t>(stream),
-                                           chunk_keys, chunk_values, chunk_lane_stride, chunk_stride);
+                                           chunk_keys, chunk_values, chunk_lane_stride, chunk_stride, 0,
+                                           epilogue);
   if (fused <= 0) return took(fused);
   // Every other shape: the two entries one after the other.
   std::vector<kvx_chunk_params> chunks(n_lanes);
@@ -1890,8 +1894,42 @@ int kv_append_attend_decode(const kvx_storage *s, uint32_t layer, const void *ch
   if (int rc = kv_append(s, layer, chunk_keys, chunk_values, page_tables, chunks.data(), n_lanes,
                          chunk_lane_stride, 0, stream))
     return rc;
+  if (epilogue)
+    return kv_attend_verify_hidden(s, layer, query_heads, queries, output, page_tables, lanes, n_lanes,
+                                   nullptr, row_stride, workspace, workspace_bytes, epilogue->packed_qkv,
+                                   epilogue->hidden, stream);
   return kv_attend_decode(s, layer, query_heads, queries, output, page_tables, lanes, n_lanes,
                           row_stride, workspace, workspace_bytes, stream);
+}
+}  // namespace
+
+int kv_append_attend_decode(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
+                            const void *chunk_values, uint64_t chunk_lane_stride,
+                            uint32_t chunk_stride, uint32_t query_heads, const void *queries,
+                            void *output, const uint64_t *const *page_tables,
+                            const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,
+                            void *workspace, uint64_t workspace_bytes, void *stream) {
+  if (!output) return fail(KVX_EINVAL, "kv_append_attend_decode: null argument or no lanes");
+  return append_attend_decode(s, layer, chunk_keys, chunk_values, chunk_lane_stride, chunk_stride,
+                              query_heads, queries, output, page_tables, lanes, n_lanes, row_stride,
+                              workspace, workspace_bytes, nullptr, stream);
+}
+
+int kv_append_attend_decode_hidden(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
+                                   const void *chunk_values, uint64_t chunk_lane_stride,
+                                   uint32_t chunk_stride, uint32_t query_heads, const void *queries,
+                                   void *output, const uint64_t *const *page_tables,
+                                   const kvx_verify_params *lanes, uint32_t n_lanes,
+                                   uint32_t row_stride, void *workspace, uint64_t workspace_bytes,
+                                   const void *packed_qkv, void *hidden, void *stream) {
+  if (!hidden) return fail(KVX_EINVAL, "kv_append_attend_decode_hidden: null hidden rows");
+  if (hidden == queries || hidden == output || hidden == packed_qkv || hidden == chunk_keys ||
+      hidden == chunk_values)
+    return fail(KVX_EINVAL, "hidden rows must not alias another argument");
+  const Epilogue epilogue{static_cast<const uint16_t *>(packed_qkv), static_cast<uint16_t *>(hidden)};
+  return append_attend_decode(s, layer, chunk_keys, chunk_values, chunk_lane_stride, chunk_stride,
+                              query_heads, queries, output, page_tables, lanes, n_lanes, row_stride,
+                              workspace, workspace_bytes, &epilogue, stream);
 }
 
 int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads,

@@ -378,6 +378,13 @@ void testAppendDecodeSingleToken() {
     uint32_t unhalved = 0;
     for (size_t i = 0; i < hidden.size(); ++i) unhalved += f32(hidden[i]) != 0.5f * f32(two[i]);
     EXPECT(unhalved == 0);
+    // The decode step as one call with the second output: the token stored again (the same
+    // bytes), the row attended and the gathered operand written.
+    hip(hipMemset(hiddenDevice, 0x3C, hidden.size() * 2));
+    ops::PagedAttention::addVerify(nullptr, storage, 1, buffers, {chunk}, plan, nullptr, hiddenDevice);
+    hip(hipDeviceSynchronize());
+    hip(hipMemcpy(hidden.data(), hiddenDevice, hidden.size() * 2, hipMemcpyDeviceToHost));
+    EXPECT(hidden == two);
     buffers.treeMasks = static_cast<const uint32_t *>(packedDevice);  // any non-null masks: a tree plan
     EXPECT(throws<std::invalid_argument>([&] {
       ops::PagedAttention::addVerify(nullptr, storage, 1, buffers, {chunk}, plan, nullptr, hiddenDevice);

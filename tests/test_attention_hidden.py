@@ -86,6 +86,7 @@ def test_gate_reads_the_gate_half_of_each_query_head(kv_heads, group, dim, rows)
 
 def test_library_exports_the_entry():
     assert hasattr(kvx.lib(), "kv_attend_verify_hidden")
+    assert hasattr(kvx.lib(), "kv_append_attend_decode_hidden")
 
 
 # ---------------------------------------------------------------- the GPU ----
@@ -188,6 +189,70 @@ def test_decode_hidden_rows_across_launches(fmt):
     dp = [kvx.VerifyParams(committed[i], counts[i], kvx.KvLayer(), splits[i], splits[i], 1, 1, 0.0)
           for i in range(len(committed))]
     fused_against_staged(tw, fmt, H, G, D, dts, dp, None, 1, 1, 17, True)
+    tw.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fmt", [ko.INT4, ko.INT8, ko.BF16])
+def test_append_attend_decode_hidden_is_the_two_calls(fmt):
+    """kv_append_attend_decode_hidden: the page bytes of kv_append, and the staged and hidden rows
+    of kv_attend_verify_hidden over them, bit for bit, gated and gathered, with and without the
+    staged rows; int4 pages take the kernel that stores the token itself, 40 lanes two launches."""
+    import torch
+    import gpulib as Gp
+    import kvtestlib as T
+    import test_gpu_attention as A
+    rng = np.random.default_rng(77)
+    committed = [0, 31, 32, 700, 4095, 1000, 63, 2047] + [int(c) for c in rng.integers(0, 1500, 32)]
+    lanes = len(committed)
+    tw, counts, hts, dts = A.shared_pool_lanes(fmt, committed, 1, seed=78)
+    k = rng.standard_normal((lanes, H, 1, D)).astype(np.float32)
+    v = rng.standard_normal((lanes, H, 1, D)).astype(np.float32)
+    ck = np.zeros((lanes, H, 32, D), dtype=np.uint16)
+    cv = np.zeros((lanes, H, D, 32), dtype=np.uint16)
+    for lane in range(lanes):
+        ck[lane], cv[lane] = T.chunk_buffers(k[lane], v[lane], 32)
+    q = A.queries((lanes, H, 1, G, D), 79)
+    packed = rand_bf16(rng, (lanes, 1, (2 * QH + 2 * H) * D), 2.0)
+    plan = (C.c_uint32 * lanes)()
+    kvx.check(kvx.lib().kvx_decode_plan((C.c_uint32 * lanes)(*committed), lanes, H, fmt, plan))
+    dp = [kvx.VerifyParams(committed[i], counts[i], kvx.KvLayer(), plan[i], plan[i], 1, 1, 0.0)
+          for i in range(lanes)]
+    ws = torch.empty(kvx.attend_workspace_bytes(tw.dev, dp, QH), dtype=torch.uint8, device="cuda")
+    before = [tw.dev.extent_read(e).copy() for e in range(tw.extents)]
+    dq, dk, dv, dpacked = Gp.dev(q), Gp.dev(ck), Gp.dev(cv), Gp.dev(packed)
+
+    def fresh(shape, fill):
+        return torch.full(shape, fill, dtype=torch.int16, device="cuda")
+
+    # the two calls, gated and gathered
+    kvx.append(tw.dev, 1, dk, dv, dts, [kvx.ChunkParams(committed[i], 1, 32, counts[i]) for i in range(lanes)],
+               H * 32 * D)
+    want_rows, want_gated = fresh((lanes, H, 1, G, D), 0x5A5A), fresh((lanes, 1, QH, D), 0x3C3C)
+    kvx.attend_verify_hidden(tw.dev, 1, QH, dq, want_rows, dts, dp, None, 1, ws, dpacked, want_gated)
+    want_gathered = fresh((lanes, 1, QH, D), 0x3C3C)
+    kvx.attend_verify_hidden(tw.dev, 1, QH, dq, None, dts, dp, None, 1, ws, None, want_gathered)
+    torch.cuda.synchronize()
+    after_two = [tw.dev.extent_read(e).copy() for e in range(tw.extents)]
+    assert want_gated.any() and want_gathered.any()
+    for gated in (True, False):
+        for e in range(tw.extents):
+            tw.dev.extent_write(e, before[e])
+        ws.fill_(0xA5)
+        rows, hidden = fresh((lanes, H, 1, G, D), 0x5A5A), fresh((lanes, 1, QH, D), 0x3C3C)
+        paths = kvx.attend_paths()
+        kvx.append_attend_decode_hidden(tw.dev, 1, dk, dv, H * 32 * D, 32, QH, dq, rows if gated else None,
+                                        dts, dp, 1, ws, dpacked if gated else None, hidden)
+        torch.cuda.synchronize()
+        assert kvx.attend_paths()[1] > paths[1] and kvx.attend_paths()[0] == paths[0]
+        assert torch.equal(hidden, want_gated if gated else want_gathered)
+        if gated:
+            assert torch.equal(rows, want_rows)
+        for e in range(tw.extents):
+            assert np.array_equal(tw.dev.extent_read(e), after_two[e])
+    with pytest.raises(kvx.KvxError):
+        kvx.append_attend_decode_hidden(tw.dev, 1, dk, dv, H * 32 * D, 32, QH, dq, None, dts, dp, 1, ws,
+                                        dpacked, None)
     tw.close()
 
 
