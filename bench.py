@@ -65,8 +65,8 @@ def parse():
                     help="call kv_append and kv_attend_decode instead of kv_append_attend_decode")
     ap.add_argument("--hidden", choices=["none", "gate", "gather"], default="none",
                     help="decode: the merge also writes the out-projection's operand "
-                         "(kv_attend_verify_hidden), gated by packed projection rows or plainly "
-                         "gathered; implies --separate-append")
+                         "(kv_append_attend_decode_hidden; with --separate-append kv_append + "
+                         "kv_attend_verify_hidden), gated by packed projection rows or plainly gathered")
     ap.add_argument("--prepare", action="store_true",
                     help="decode: the step's queries, keys and values come from packed projection rows "
                          "through kv_prepare_append (norm, rotation, quantize, store) instead of "
@@ -977,7 +977,6 @@ def main():
     lane_stride = H * 32 * D
     hidden = packed = None
     if args.hidden != "none":
-        args.separate_append = True
         hidden = torch.zeros((BATCH, 1, QH, D), dtype=torch.bfloat16, device="cuda")
         if args.hidden == "gate":
             packed = torch.randn((BATCH, 1, (2 * QH + 2 * H) * D), generator=gen, device="cuda").bfloat16()
@@ -1009,10 +1008,17 @@ def main():
         for layer in range(LAYERS):
             if not args.separate_append:
                 # one call per layer: the token is stored by the attention kernel itself
-                rc = L.kv_append_attend_decode(storage.h, layer, chunk_k.data_ptr(), chunk_v.data_ptr(),
-                                               lane_stride, 32, QH, queries.data_ptr(),
-                                               output.data_ptr(), table_arr, vp_arr, BATCH, 1,
-                                               workspace.data_ptr(), ws_bytes, stream)
+                if hidden is None:
+                    rc = L.kv_append_attend_decode(storage.h, layer, chunk_k.data_ptr(), chunk_v.data_ptr(),
+                                                   lane_stride, 32, QH, queries.data_ptr(),
+                                                   output.data_ptr(), table_arr, vp_arr, BATCH, 1,
+                                                   workspace.data_ptr(), ws_bytes, stream)
+                else:
+                    rc = L.kv_append_attend_decode_hidden(
+                        storage.h, layer, chunk_k.data_ptr(), chunk_v.data_ptr(), lane_stride, 32, QH,
+                        queries.data_ptr(), output.data_ptr(), table_arr, vp_arr, BATCH, 1,
+                        workspace.data_ptr(), ws_bytes, packed.data_ptr() if packed is not None else None,
+                        hidden.data_ptr(), stream)
                 if rc:
                     kvx.check(rc)
                 continue
@@ -1133,8 +1139,9 @@ def main():
             "pool_gb": round(extents * extent_bytes / 1e9, 1), "extents": extents,
             "page_order": "contiguous" if args.contiguous else "seed-shuffled",
             "seed": args.seed,
-            **({"entries": ("kv_prepare_append" if args.prepare else "kv_append") + " + " +
-                           ("kv_attend_verify_hidden" if args.hidden != "none" else "kv_attend_decode"),
+            **({"entries": ("kv_append_attend_decode_hidden" if not args.separate_append else
+                            ("kv_prepare_append" if args.prepare else "kv_append") + " + " +
+                            ("kv_attend_verify_hidden" if args.hidden != "none" else "kv_attend_decode")),
                 "hidden": args.hidden}
                if args.hidden != "none" or args.prepare else {}),
         },
