@@ -351,12 +351,23 @@ uint8_t ko_float_to_fp8e4m3(float v) {
   if (e > 8 || (e == 8 && m - 8 > 6)) return uint8_t(sign | 0x7E);
   return uint8_t(sign | uint8_t(((e + 7) << 3) | (m - 8)));
 }
-float ko_fp8e4m3_to_float(uint8_t c) {
+static float fp8e4m3_value(uint8_t c) {
   const float sign = (c & 0x80) ? -1.0f : 1.0f;
   const int e = (c >> 3) & 0xF, m = c & 7;
   if (e == 0) return sign * std::ldexp(float(m), -9);
   if (e == 15 && m == 7) return std::numeric_limits<float>::quiet_NaN();
   return sign * std::ldexp(1.0f + float(m) / 8.0f, e - 7);
+}
+float ko_fp8e4m3_to_float(uint8_t c) {
+  // The 256 values of the formula above, computed once: the attention restatement decodes a
+  // code per key and value element of every row, and ldexp per element is most of its time.
+  static const struct Table {
+    float value[256];
+    Table() {
+      for (int i = 0; i < 256; ++i) value[i] = fp8e4m3_value(uint8_t(i));
+    }
+  } table;
+  return table.value[c];
 }
 float ko_round_to_f16(float v) {
   // IEEE binary16 round-to-nearest-even, returned widened to fp32.

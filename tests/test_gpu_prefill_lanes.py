@@ -63,10 +63,11 @@ def test_long_chunk_is_its_short_pieces(fmt, heads, group, committed, rows):
     tw.close()
 
 
-@pytest.mark.parametrize("fmt", WIDE)
-@pytest.mark.parametrize("heads,group,committed,rows,splits",
-                         [(4, 6, 1024, 296, 3), (4, 4, 1024, 296, 3), (2, 8, 1024, 296, 3),
-                          (4, 6, 0, 256, 8), (4, 6, 1000, 264, 2)])
+@pytest.mark.parametrize("fmt,heads,group,committed,rows,splits",
+                         [(fmt, *case) for fmt in (ko.INT8, ko.BF16)
+                          for case in [(4, 6, 1024, 296, 3), (4, 4, 1024, 136, 3), (2, 8, 1024, 136, 3),
+                                       (4, 6, 0, 256, 8), (4, 6, 1000, 264, 2)]] +
+                         [(ko.FP8, 4, 6, 1024, 136, 3)])
 def test_long_chunk_under_several_splits_matches_oracle(fmt, heads, group, committed, rows, splits):
     # after 1024 and 0 tokens the tiles of a lane cut their pages into the same splits and the
     # lanes of several tiles run; after 1000 they do not, and the chunk runs tile by tile
