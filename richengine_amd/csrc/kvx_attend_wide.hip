@@ -709,9 +709,43 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
       vs[1] = load_global<f32x4>(p.value_scales + 8 * g + 4);
     }
   };
+  // bf16 pages need no conversion on their way: in the two-copy form the wave's share of a
+  // page goes from global memory into the staged copy directly (16 bytes per lane and
+  // instruction, the lanes of an instruction one operand block), with no registers in between
+  // and no LDS writes to issue.  The copy must be free when the loads are sent, since they
+  // land whenever they arrive; the wave waits for them before the barrier that hands the copy
+  // over.  (bf16 chain verify of a batch of 32: 413 -> 396 us.  The four-copy form was slower
+  // with it, a 2048-row prefill chunk 1.19 -> 1.27 ms, and stages through registers.)
+  constexpr bool kDirect = !kByte && COPIES == 2;
+  auto direct = [&](GroupOperands &copy, uint64_t entry) {
+    constexpr uint32_t B = Wide<FMT>::kBytes;
+    constexpr uint32_t KB = GroupShare<FMT, W>::kKeyBlocks, VB = GroupShare<FMT, W>::kValueBlocks;
+    constexpr uint32_t kPolicy = REUSED ? 0u : 2u;  // 2: non-temporal, for pages read once
+    typedef __attribute__((address_space(1))) const void GlobalBytes;
+    typedef __attribute__((address_space(3))) void SharedBytes;
+    const PagePlace p = place_page<FMT>(entry, head, H, a.kv.offset, ro);
+#pragma unroll
+    for (uint32_t tb = 0; tb < 2; ++tb) {
+      const uint8_t *row = p.keys + (8 * (t >> 2) + 4 * tb + (t & 3)) * kD * B;
+#pragma unroll
+      for (uint32_t c = 0; c < KB; ++c)
+        __builtin_amdgcn_global_load_lds(
+            (GlobalBytes *)(reinterpret_cast<uintptr_t>(row + key_dims<FMT>(KB * wave + c, g) * B)),
+            (SharedBytes *)(&copy.keys[tb][KB * wave + c][0]), 16, 0, kPolicy);
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < VB; ++i)
+      __builtin_amdgcn_global_load_lds(
+          (GlobalBytes *)(reinterpret_cast<uintptr_t>(p.values + ((16 * (VB * wave + i) + t) * kPage + 8 * g) * B)),
+          (SharedBytes *)(&copy.values[VB * wave + i][0]), 16, 0, kPolicy);
+  };
+  // The barrier of the direct form: the wave's loads into the copies have landed.
+  auto landed_barrier = [&] { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
   const uint64_t entry0 = next_entry(1), entry1 = next_entry(2);
-  fetch(raw[0], entry0);
-  if constexpr (SETS == 2) fetch(raw[1], entry1);
+  if constexpr (!kDirect) {
+    fetch(raw[0], entry0);
+    if constexpr (SETS == 2) fetch(raw[1], entry1);
+  }
   fetch_scales(ks_even, vs_even, entry0);
   fetch_scales(ks_odd, vs_odd, entry1);
 
@@ -832,7 +866,21 @@ group_wide_kernel(const uint16_t *__restrict__ queries, uint16_t *__restrict__ o
   };
 
   const uint32_t first_masked = l.committed / kPage;
-  if constexpr (COPIES == 2) {
+  if constexpr (kDirect) {
+    // Two copies, loaded directly: while slot i is multiplied out of one, slot i + 1 lands in
+    // the other; a barrier per page.
+    direct(shared_page[0], entry0);
+    landed_barrier();
+    auto turn = [&](const GroupOperands &now, GroupOperands &next, uint32_t slot) __attribute__((always_inline)) {
+      direct(next, slot == 0 ? entry1 : next_entry(slot + 2));  // of slot + 1
+      if (computes && slot < count) attend_page(now, begin + slot, ks_even, vs_even, begin + slot >= first_masked);
+      landed_barrier();
+    };
+    for (uint32_t slot = 0; slot < count; slot += 2) {
+      turn(shared_page[0], shared_page[1], slot);
+      turn(shared_page[1], shared_page[0], slot + 1);
+    }
+  } else if constexpr (COPIES == 2) {
     // Two copies: while slot i is multiplied out of one, slot i + 1 goes from the raw
     // registers into the other and the registers are sent for slot i + 2; a barrier per page.
     stage_share<FMT, W>(shared_page[0], raw[0], wave, lane);
@@ -993,16 +1041,20 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
     return KVX_GROUP_FORMATS(2, 4, true);
   }
   // Verify lanes of more than 32 fused rows: the waves that the lane needs anyway share its
-  // pages.  65 .. 128 rows (a tree of 16 nodes for a group of 6): four waves, four LDS copies
-  // (16 nodes, batch 4 x 65 536 tokens: bf16 456 -> 270 us, int8 436 -> 282 us with two sets of
-  // page registers).  33 .. 64 rows (a chain of 8): two waves that fetch half a page each, with
-  // two LDS copies so that two such workgroups fit a CU (batch of 32: bf16 706 -> 413 us, int8
-  // 435 -> 387 us, fp8 405 -> 343 us; with four copies, one workgroup per CU and half of the
-  // SIMDs empty, the byte formats took 550 - 650 us).  Two waves with three blocks each and
-  // half a page in flight spill 21 to 45 registers.
+  // pages.  33 .. 64 rows (a chain of 8 for a group of 6): two waves that fetch half a page
+  // each, with two LDS copies so that two such workgroups fit a CU (batch of 32: bf16 706 ->
+  // 400 us, int8 435 -> 387 us, fp8 405 -> 343 us; with four copies, one workgroup per CU and
+  // half of the SIMDs empty, the byte formats took 550 - 650 us).  65 .. 128 rows (a tree of 16
+  // nodes): four waves over four copies, the byte formats with two sets of page registers
+  // (batch 4 x 65 536 tokens: int8 436 -> 282 us); bf16 up to 96 rows as two waves of 48, which
+  // its direct loads leave the registers for (456 -> 212 us; four waves of 24: 238 us; the
+  // byte formats spill in that form).
   // A verify lane holds 128 fused rows at most.
   if (!tile_rows && !many_tiles && M > 32 && M <= 32u * kGroupWaves) {
-    if (format == KVX_FMT_BF16) return M > 64 ? KVX_GROUP(KVX_FMT_BF16, 2, 4, false) : KVX_GROUP(KVX_FMT_BF16, 2, 2, false, 1, 2);
+    if (format == KVX_FMT_BF16)
+      return M > 96   ? KVX_GROUP(KVX_FMT_BF16, 2, 4, false)
+             : M > 64 ? KVX_GROUP(KVX_FMT_BF16, 3, 2, false, 1, 2)
+                      : KVX_GROUP(KVX_FMT_BF16, 2, 2, false, 1, 2);
     if (format == KVX_FMT_INT8) return M > 64 ? KVX_GROUP(KVX_FMT_INT8, 2, 4, false, 2) : KVX_GROUP(KVX_FMT_INT8, 2, 2, false, 1, 2);
     return M > 64 ? KVX_GROUP(KVX_FMT_FP8E4M3, 2, 4, false, 2) : KVX_GROUP(KVX_FMT_FP8E4M3, 2, 2, false, 1, 2);
   }

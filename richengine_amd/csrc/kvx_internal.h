@@ -169,7 +169,9 @@ inline bool prefill_group_splits_alike(uint32_t width, uint32_t committed) {
 }
 // Waves (row blocks) per (lane, split, KV head) of a verify launch.
 inline uint32_t verify_row_blocks(uint32_t format, uint32_t fused_rows) {
-  // bf16, fp8, int8 pages: 65 .. 128 fused rows run as four waves that share their pages.
+  // bf16, fp8, int8 pages: 65 .. 128 fused rows run as four waves that share their pages
+  // (bf16 up to 96 rows: as two waves of 48).
+  if (format == KVX_FMT_BF16 && fused_rows > 64 && fused_rows <= 96) return 2;
   if (format != KVX_FMT_INT4 && fused_rows > 64 && fused_rows <= 128) return 4;
   const uint32_t rows = verify_block_rows(format, fused_rows);
   return (fused_rows + rows - 1) / rows;

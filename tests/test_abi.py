@@ -133,6 +133,8 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
             blocks = -(-fused // 32) if fused > 16 else 1
             if fmt != kvx.INT4 and 64 < fused <= 128:
                 blocks = 4                             # waves of a workgroup that shares its pages
+                if fmt == kvx.BF16 and fused <= 96:
+                    blocks = 2                         # two waves of 48 rows
             if fmt == kvx.INT4 and fused > 16 and 7 * -(-fused // 48) < 5 * -(-fused // 32):
                 blocks = -(-fused // 48)  # the int4 kernel for 48 fused rows per wave
             counts = [pages(c + rows) for c in committed]
@@ -188,7 +190,8 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
     with pytest.raises(kvx.KvxError):
         kvx.prefill_plan(16384, 256, 4, 6)
     assert kvx.verify_plan([65536] * 4, 16, H, QH) == [32] * 4          # two waves of 48 fused rows
-    assert kvx.verify_plan([65536] * 4, 16, H, QH, kvx.BF16) == [16] * 4  # four waves that share their pages
+    assert kvx.verify_plan([65536] * 4, 16, H, QH, kvx.BF16) == [32] * 4  # two waves of 48 rows that share their pages
+    assert kvx.verify_plan([65536] * 4, 16, H, QH, kvx.INT8) == [16] * 4  # four waves that share their pages
     with pytest.raises(kvx.KvxError):
         kvx.verify_plan([10], 8, 4, 6)
 
@@ -241,6 +244,8 @@ def test_hot_kernels_stay_out_of_scratch_memory():
     for fmt in (1, 2, 4):
         r = one(f"group_wide_kernelILj{fmt}ELj2ELj2ELb0E")
         assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, r
+    r = one("group_wide_kernelILj2ELj3ELj2ELb0E")      # bf16, two waves of 48 rows, direct loads
+    assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, r
     # the kernels whose accumulators fill the second register file (48-row verify, two-block
     # bf16): since their rescaling names the accumulators there, nothing spills
     for fragment in ("verify48_int4_kernel", "attend_wide_kernelILj2ELj2ELj1ELb0E",
