@@ -157,7 +157,13 @@ uint32_t kvx_decode_splits(uint32_t committed_tokens, uint32_t rows);
    max(ceil(total page-heads / 1024), 8) (at most 32 for int4, whose kernel holds two waves per
    SIMD and is fastest at 32), which fills the GPU when the batch is small, and grows until the
    launch has no more waves than the kernel has wave slots (2048 for int4, 1024 for the other
-   formats), because waves beyond that run as a second round on a nearly empty GPU.  One-row
+   formats), because waves beyond that run as a second round on a nearly empty GPU.  An int4
+   batch of at most KVX_LANES_PER_LAUNCH lanes that needs two waves on most SIMDs is planned in
+   two classes instead, because the two waves of a SIMD do not share it evenly: lanes from the
+   longest down get splits of one length while their waves fit one per SIMD (1024), the other
+   lanes splits of 0.58 of that length, and the length is the least for which the second class
+   fits 1024 waves too; kv_attend_decode dispatches the lanes with the longest splits first, so
+   the long splits take the first wave of every SIMD and both classes end together.  One-row
    decode lanes may use up to KVX_DECODE_MAX_SPLITS splits; every other attend entry keeps the
    reference's KVX_VERIFY_MAX_SPLITS.  No counterpart in the reference, whose decode shares the
    verify plan (runtime/ops/PagedAttention.cpp:232-262). */
@@ -185,8 +191,10 @@ int kvx_chunk_validation(const kvx_chunk_params *params);
    alone.  The plan keeps one split while those waves fill at least half of the kernel's wave
    slots and otherwise takes the largest count (at most 32, at least 8 pages per split) whose
    launch still fits one round of slots: of the paired tiles' waves where the two tiles of
-   every pair see the same number of pages (committed_tokens mod 16 is 0 or at least 9, so
-   every page-aligned chunk start; int4 pages: from 512 rows on), else of tiles x splits x KV heads x ceil(8 x group / 16)
+   every pair see the same number of pages (a pair is 16 rows of 32-token pages, and its two
+   8-row tiles end in the same page exactly when committed_tokens mod 16 is 0 or at least 9:
+   then the first tile's last row and the second tile's last row, 8 tokens later, do not
+   straddle a page boundary; so every page-aligned chunk start; int4 pages: from 512 rows on), else of tiles x splits x KV heads x ceil(8 x group / 16)
    waves of single tiles.  bf16, fp8 and int8 pages, chunks of 64 rows and more (lanes of four tiles of
    8 x group <= 48 fused rows, or two of <= 96, one workgroup per lane, split and KV head, one
    workgroup per CU): one split where those workgroups fill three quarters of the 256 CUs, else
@@ -359,9 +367,11 @@ int kvx_prefix_erase(kvx_prefix *prefix, uint64_t block);
 /* KvCache::followPages: after kvx_pool_compact_extent moved pages. */
 void kvx_prefix_follow_pages(kvx_prefix *prefix, uint32_t first_page, const uint32_t *destinations,
                              uint32_t n);
-/* Cache::extendMatch (runtime/engine/cache/Cache.cpp:179-199), text-only prompts: the chain of
-   cached blocks that covers the prompt's leading whole pages, leaving at least one prompt token
-   unmatched.  Returns the number of pages looked up. */
+/* Cache::extendMatch (runtime/engine/cache/Cache.cpp:179-199): the chain of cached blocks that
+   covers the prompt's leading whole pages, leaving at least one prompt token unmatched.  Returns
+   the number of pages looked up.  kvx_prefix_match is the text-only form (every block keyed
+   with the zero identity); a prompt with images goes through kvx_prefix_match_images below,
+   or two prompts with the same placeholder tokens and different images would share pages. */
 uint64_t kvx_prefix_match(const kvx_prefix *prefix, const uint32_t *prompt, uint64_t n_tokens,
                           uint64_t *blocks, uint32_t capacity, uint32_t *matched);
 
@@ -377,6 +387,12 @@ typedef struct kvx_image_span {
 void kvx_block_image_identity(uint64_t block_begin, uint32_t block_tokens,
                               const kvx_image_span *spans, uint32_t n_spans, uint64_t *lo,
                               uint64_t *hi);
+/* Cache::extendMatch with the prompt's images (Cache.cpp:186-193: spansFrom, then
+   blockImageIdentity per block): every block is looked up under the identity of the spans
+   that overlap it.  `spans` sorted by offset and disjoint; null or none = kvx_prefix_match. */
+uint64_t kvx_prefix_match_images(const kvx_prefix *prefix, const uint32_t *prompt,
+                                 uint64_t n_tokens, const kvx_image_span *spans, uint32_t n_spans,
+                                 uint64_t *blocks, uint32_t capacity, uint32_t *matched);
 
 /* ---- per-sequence page lists: the Request records of engine::Cache
         (runtime/engine/cache/Cache.cpp:143-166, 284-333, 381-413, 700-731, 748-785) ---- */
@@ -410,7 +426,12 @@ int kvx_sequence_ensure_tokens(kvx_sequences *sequences, uint64_t id, uint64_t t
    the shared page is given back; *copied = 1 with the two page ids.  A page held by nobody
    else is written in place (*copied = 0).  KVX_ESTATE for a published page (its rows are
    final), KVX_EINVAL when the sequence holds no page for `token`, KVX_ENOMEM with nothing
-   changed when no page is to be had.  Stores into the copy go on `stream` or after it. */
+   changed when no page is to be had.  Stores into the copy go on `stream` or after it.  The
+   copy is only enqueued when the call returns, and the sequence's reference to the shared
+   page is given back at once: should every other holder let go of it too, the pool can hand
+   the page out again, and whoever gets it must not store into it before `stream` has passed
+   the copy (an event recorded on `stream` after this call, waited for by the writer's stream;
+   the same rule as after kvx_pool_compact_extent).  kvx_sequence_fork copies nothing. */
 int kvx_sequence_fork(kvx_sequences *sequences, uint64_t id, uint64_t source, uint64_t tokens);
 int kvx_sequence_ensure_writable(kvx_sequences *sequences, uint64_t id, uint64_t token,
                                  uint32_t *copied, uint32_t *from_page, uint32_t *to_page,
@@ -420,6 +441,22 @@ int kvx_sequence_ensure_writable(kvx_sequences *sequences, uint64_t id, uint64_t
    revision / first_changed say so. */
 int kvx_sequence_publish(kvx_sequences *sequences, uint64_t id, const uint32_t *tokens,
                          uint64_t n_tokens, uint32_t committed_tokens);
+/* The same with the request's images (Cache.cpp:310-318): every new block is keyed with the
+   identity of the spans that overlap it, so equal placeholder tokens under different images
+   stay apart.  kvx_sequence_publish is the text-only form (no spans). */
+int kvx_sequence_publish_images(kvx_sequences *sequences, uint64_t id, const uint32_t *tokens,
+                                uint64_t n_tokens, uint32_t committed_tokens,
+                                const kvx_image_span *spans, uint32_t n_spans);
+/* After a speculative rollback (kv_compact_path, then the host's committed count): gives the
+   pages past those that hold the first `tokens` tokens back to the pool, one active reference
+   each, and says how many in *released_pages; the view's revision / first_changed say so.
+   `tokens` is what the sequence keeps room for: the committed tokens plus the scratch rows of
+   the next step (the reference asks ensureTokens for position + 15, Engine.cpp:1190-1193, and
+   never shrinks a request; this is the other direction, for trees of 16 draft rows that can
+   leave a whole page without a committed token).  A page somebody else holds too only loses
+   this sequence's reference.  KVX_ESTATE when that would drop a published page. */
+int kvx_sequence_truncate(kvx_sequences *sequences, uint64_t id, uint64_t tokens,
+                          uint32_t *released_pages);
 int kvx_sequence_view(const kvx_sequences *sequences, uint64_t id, kvx_sequence_pages *out);
 /* Cache::compactExtent: kvx_pool_compact_extent (with its ordering rule for `stream`), then
    blocks and sequences follow their pages. */
@@ -597,8 +634,13 @@ int kv_attend_decode(const kvx_storage *storage, uint32_t layer, uint32_t query_
    KVX_EINVAL when kvx_attend_workspace_bytes() of the lanes exceeds the array (the headline batch
    of 32 sequences at 507 splits needs 12.6 MB), KVX_ESTATE when the storage's device is not the
    current device.  All calls on one GPU share the array: calls that overlap there (two streams,
-   two threads) race on it; calls on one stream, or ordered by events, do not. */
+   two threads) race on it; calls on one stream, or ordered by events, do not.
+   Where the array lies on a device is looked up once per device: kvx_storage_create does it
+   for the device it runs on, kvx_static_workspace_prime for a storage whose device became
+   current later.  A call under stream capture on a device where neither has happened is
+   refused with KVX_ESTATE instead of asking the runtime in the middle of the capture. */
 #define KVX_STATIC_WORKSPACE_BYTES (32u << 20)
+int kvx_static_workspace_prime(const kvx_storage *storage);
 int kv_attend_decode_static(const kvx_storage *storage, uint32_t layer, uint32_t query_heads,
                             const void *queries, void *output, const uint64_t *const *page_tables,
                             const kvx_verify_params *lanes, uint32_t n_lanes, uint32_t row_stride,

@@ -78,6 +78,29 @@ def lib():
     return _lib
 
 
+_ref_cache = None
+
+
+def ref_image_identity(block_begin, block_tokens, spans):
+    """(lo, hi) from the reference's own blockImageIdentity (oracle/_ref/libkvref_cache.so:
+    runtime/engine/cache/KvCache.cpp compiled where it lies), or None where it was not built.
+    spans: (offset, tokens, grid height, grid width, digest lo, digest hi) tuples."""
+    global _ref_cache
+    if _ref_cache is None:
+        path = os.path.join(_HERE, "_ref", "libkvref_cache.so")
+        if not os.path.exists(path):
+            return None
+        _ref_cache = C.CDLL(path)
+        _ref_cache.ref_image_identity.argtypes = [C.c_uint64, C.c_uint32, C.c_void_p, C.c_uint32,
+                                                  C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
+        _ref_cache.ref_image_identity.restype = None
+    words = np.array([w for span in spans for w in span], dtype=np.uint64)
+    lo, hi = C.c_uint64(), C.c_uint64()
+    _ref_cache.ref_image_identity(block_begin, block_tokens, words.ctypes.data_as(C.c_void_p),
+                                  len(spans), C.byref(lo), C.byref(hi))
+    return lo.value, hi.value
+
+
 def ref():
     """The reference's own host code (oracle/_ref), or None where it was not built."""
     global _ref

@@ -165,15 +165,22 @@ class PrefixCache:
             self.blocks[block].page = to
             self.block_on_page[to] = block
 
-    def extend_match(self, blocks, prompt):
+    def extend_match(self, blocks, prompt, spans=()):
+        """Cache::extendMatch (runtime/engine/cache/Cache.cpp:179-199); spans are the prompt's
+        images, sorted by offset: each block is looked up under blockImageIdentity of the spans
+        that have not ended before it (spansFrom, Cache.cpp:16-22)."""
         if not len(prompt):
             return 0
         maximum = (len(prompt) - 1) // PAGE_TOKENS
         hashed = 0
+        spans = list(spans)
         for index in range(len(blocks), maximum):
             parent = blocks[-1] if blocks else 0
             hashed += 1
-            match = self.find(parent, prompt[index * PAGE_TOKENS:(index + 1) * PAGE_TOKENS])
+            begin = index * PAGE_TOKENS
+            spans = spans_from(spans, begin)
+            match = self.find(parent, prompt[begin:begin + PAGE_TOKENS],
+                              block_image_identity(begin, PAGE_TOKENS, spans))
             if not match:
                 break
             blocks.append(match[0])
@@ -240,8 +247,26 @@ class SequenceCache:
         s.pages += list(self.acquire(needed - previous))
         self._changed(s, previous)
 
-    def publish(self, sequence, tokens, committed):
+    def truncate(self, sequence, tokens):
+        """No counterpart in the reference (it never shrinks a request): the pages past those of
+        the first `tokens` tokens go back to the pool; published pages may not."""
         s = self._sequence(sequence)
+        keep = (tokens + PAGE_TOKENS - 1) // PAGE_TOKENS
+        if keep < len(s.blocks):
+            raise OracleError("state", "truncation would drop a published page")
+        if keep >= len(s.pages):
+            return 0
+        dropped = s.pages[keep:]
+        for page in dropped:
+            self.pool.release(page, False)
+        del s.pages[keep:]
+        self._changed(s, keep)
+        return len(dropped)
+
+    def publish(self, sequence, tokens, committed, spans=()):
+        """Cache::publishCommittedBlocks (Cache.cpp:294-333), images included (:310-318)."""
+        s = self._sequence(sequence)
+        spans = list(spans)
         if committed > len(tokens):
             raise OracleError("invalid", "committed KV exceeds exact token history")
         full = committed // PAGE_TOKENS
@@ -253,8 +278,11 @@ class SequenceCache:
             logical = len(s.blocks)
             parent = s.blocks[-1] if logical else 0
             writer = s.pages[logical]
+            begin = logical * PAGE_TOKENS
+            spans = spans_from(spans, begin)
             block, canonical = self.prefix.insert(
-                parent, tokens[logical * PAGE_TOKENS:(logical + 1) * PAGE_TOKENS], writer)
+                parent, tokens[begin:begin + PAGE_TOKENS], writer,
+                block_image_identity(begin, PAGE_TOKENS, spans))
             replace = canonical != writer
             if replace:
                 self.pool.retain(canonical, False)
@@ -304,16 +332,27 @@ def tree_masks(parents, none=0xFFFFFFFF):
     return masks
 
 
+def spans_from(spans, block_begin):
+    """spansFrom (runtime/engine/cache/Cache.cpp:16-22): the spans that can still overlap the
+    block at block_begin or a later one."""
+    first = 0
+    while first < len(spans) and ((spans[first][0] + spans[first][1]) & 0xFFFFFFFF) <= block_begin:
+        first += 1
+    return spans[first:]
+
+
 def block_image_identity(block_begin, block_tokens, spans):
     """Restates blockImageIdentity (runtime/engine/cache/KvCache.cpp:29-52): (lo, hi) of a block
     of `block_tokens` tokens at `block_begin`; spans are (offset, tokens, grid height, grid
     width, digest lo, digest hi) sorted by offset.  Only spans that overlap the block count;
     a block without any has identity (0, 0).
 
-    The reference holds no golden value of this function, only the properties of
-    dev/tests/engine/kv_page_cache_test.cpp:44-69 (zero for text, zero after the image,
-    dependence on digest and alignment, spans outside the block ignored): PARITY UNPINNED at
-    the bit level, pinned to those properties in tests/test_prefix_cache.py."""
+    Pinned to the bit: tests/golden/reference_vectors.npz holds what the reference's own
+    compiled function returned (tests/golden/make_vectors.py through oracle/_ref), and
+    tests/test_golden.py holds this restatement and the library to those values; the
+    properties of dev/tests/engine/kv_page_cache_test.cpp:44-69 (zero for text, zero after the
+    image, dependence on digest and alignment, spans outside the block ignored) are checked in
+    tests/test_prefix_cache.py."""
     mask = (1 << 64) - 1
 
     def mix(h, v):

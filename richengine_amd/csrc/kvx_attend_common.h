@@ -69,6 +69,7 @@ struct DecodeLane {
   uint32_t split_count;
   uint32_t first_item;  // first (lane, split) work item of this lane
   float score_scale;
+  uint32_t source;      // the lane's place among the launch's lanes as the caller passed them
   uint64_t row_base;    // first fused row of the lane's slots in the workspace
   uint64_t q_offset;    // element offset of the lane's queries
 };
@@ -108,6 +109,9 @@ struct DecodeArgs {
   uint16_t *hidden;
   const uint16_t *packed_qkv;
   uint32_t all_partials;
+  // Work items in the grid's y and KV heads in its x (the heads of an item are dispatched
+  // side by side and the items in the order of the lane records) instead of items in x.
+  uint32_t item_major;
 };
 
 // The lane with this index of a launch: read from the arguments, or derived
@@ -126,6 +130,7 @@ __device__ __forceinline__ DecodeLane lane_at(const DecodeArgs &a, uint32_t inde
   l.split_count = from.split_count;
   l.first_item = a.tile_lanes ? index * from.split_count : from.first_item;
   l.score_scale = from.score_scale;
+  l.source = a.tile_lanes ? index : from.source;
   l.row_base = from.row_base + uint64_t(tile) * from.split_count * a.kv_heads * a.fused_rows;
   l.q_offset = from.q_offset + tile * a.tile_lane_stride;
   return l;
@@ -268,7 +273,7 @@ __global__ __launch_bounds__(64 * WAVES) void matrix_merge_kernel(
              : nullptr;
   // The row's place in the out-projection's operand and in the packed rows:
   // [lane][row][query head], the gate D elements after the head's query.
-  const uint64_t hidden_row = uint64_t(blockIdx.z) * (M / G) + j / G;
+  const uint64_t hidden_row = uint64_t(l.source) * (M / G) + j / G;
   const uint32_t query_head = head * G + j % G;
   uint16_t *hidden_out =
       a.hidden ? a.hidden + (hidden_row * a.kv_heads * G + query_head) * kD + 4 * lane : nullptr;
@@ -369,7 +374,8 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
                             uint32_t n_lanes, const uint32_t *row_masks, uint32_t row_stride,
                             uint64_t lane_stride, void *workspace, uint64_t workspace_bytes,
                             hipStream_t stream, const FusedAppend *fused = nullptr,
-                            uint32_t tile_rows = 0, const Epilogue *epilogue = nullptr) {
+                            uint32_t tile_rows = 0, const Epilogue *epilogue = nullptr,
+                            bool longest_first = false) {
   const bool run_split = !(epilogue && epilogue->merge_only);
   const bool run_merge = !(epilogue && epilogue->partials_only);
   const kvx_layout &l = s->layout;
@@ -408,22 +414,45 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
     }
     uint32_t items = 0, max_splits = 0;
     for (uint32_t i = 0; i < kLanes; ++i) a.item_base[i] = UINT32_MAX;
-    for (uint32_t i = 0; i < (tile_rows ? 1u : a.n_lanes); ++i) {
-      const kvx_verify_params &p = lanes[first + i];
+    // Where each lane's rows lie in the workspace follows the caller's order of lanes; the
+    // order of the lane records, which is the order the work items are dispatched in, may
+    // differ: longest_first puts the lanes with the longest splits first (a plan that pairs
+    // long and short splits on a SIMD counts on the long ones taking the first wave slots).
+    const uint32_t recorded = tile_rows ? 1u : a.n_lanes;
+    uint64_t lane_row_base[kLanes];
+    uint32_t order[kLanes];
+    for (uint32_t i = 0; i < recorded; ++i) {
+      order[i] = i;
+      lane_row_base[i] = row_base;
+      row_base += uint64_t(lanes[first + i].split_count) * H * M;
+    }
+    if (longest_first && !tile_rows) {
+      const auto split_pages = [&](uint32_t k) {
+        const kvx_verify_params &p = lanes[first + k];
+        const uint32_t pages = (p.committed_tokens + p.active_rows + kPage - 1) / kPage;
+        return (pages + p.split_count - 1) / p.split_count;
+      };
+      std::stable_sort(order, order + recorded,
+                       [&](uint32_t x, uint32_t y) { return split_pages(x) > split_pages(y); });
+      a.item_major = 1;
+    }
+    for (uint32_t i = 0; i < recorded; ++i) {
+      const uint32_t source = order[i];
+      const kvx_verify_params &p = lanes[first + source];
       DecodeLane &dl = a.lane[i];
-      dl.table = page_tables ? page_tables[first + i] : nullptr;
-      dl.masks = row_masks ? row_masks + uint64_t(first + i) * capacity : nullptr;
+      dl.table = page_tables ? page_tables[first + source] : nullptr;
+      dl.masks = row_masks ? row_masks + uint64_t(first + source) * capacity : nullptr;
       dl.committed = p.committed_tokens;
       dl.active_rows = p.active_rows;
       dl.split_count = p.split_count;
       dl.first_item = items;
       a.item_base[i] = items;
       dl.score_scale = p.score_scale != 0.0f ? p.score_scale : l.score_scale;
-      dl.row_base = row_base;
-      dl.q_offset = uint64_t(first + i) * lane_stride;
+      dl.source = source;
+      dl.row_base = lane_row_base[source];
+      dl.q_offset = uint64_t(first + source) * lane_stride;
       items += p.split_count;
       max_splits = std::max(max_splits, p.split_count);
-      row_base += uint64_t(p.split_count) * H * M;
     }
     if (tile_rows) items = n_lanes * lanes[0].split_count;
     if (epilogue && !epilogue->hidden) {
@@ -437,8 +466,10 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       a.all_partials = 1;
     }
     if (run_split) {
-      hipLaunchKernelGGL(split_kernel, dim3(items, H, (M + columns - 1) / columns), dim3(threads), 0,
-                         stream, static_cast<const uint16_t *>(queries),
+      const uint32_t column_blocks = (M + columns - 1) / columns;
+      hipLaunchKernelGGL(split_kernel,
+                         a.item_major ? dim3(H, items, column_blocks) : dim3(items, H, column_blocks),
+                         dim3(threads), 0, stream, static_cast<const uint16_t *>(queries),
                          static_cast<uint16_t *>(output), partials, statistics, a);
       const hipError_t e = hipGetLastError();
       if (e != hipSuccess) return hip_fail(e, name);

@@ -311,6 +311,23 @@ __device__ __forceinline__ void attend_page(const Page &source, Queries queries,
   }
 }
 
+// The launch-wide arguments a wave works with, in registers.  The kernels read them out
+// of DecodeArgs once; the kernel argument block itself is only ever read where this is
+// filled in, because the compiler prefers fetching an argument again where it is used
+// (one more trip to memory in a wave's set-up) to keeping it.
+struct LaunchArgs {
+  uint32_t kv_heads, group, fused_rows, row_stride;
+  kvx_kv_layer kv;
+  const uint16_t *chunk_keys, *chunk_values;
+  uint64_t chunk_lane_stride;
+  uint32_t chunk_stride;
+  uint32_t all_partials;
+};
+__device__ __forceinline__ LaunchArgs launch_args_of(const DecodeArgs &a) {
+  return {a.kv_heads,   a.group,        a.fused_rows,        a.row_stride,   a.kv,
+          a.chunk_keys, a.chunk_values, a.chunk_lane_stride, a.chunk_stride, a.all_partials};
+}
+
 // One-token append done by the wave that owns the sequence's last page, for its
 // own KV head: quantizes the token's key row and value row (bf16 -> int4 codes and
 // one fp32 scale each, the arithmetic of append_kernel: reference
@@ -318,7 +335,7 @@ __device__ __forceinline__ void attend_page(const Page &source, Queries queries,
 // page.  Each lane owns four consecutive dims.  The stores are complete before
 // the caller loads the page: the wave waits for them, and no cache of this CU can
 // hold the lines yet because only this wave reads this head of this page.
-__device__ __forceinline__ void append_decode_token(const DecodeArgs &a, const DecodeLane &l,
+__device__ __forceinline__ void append_decode_token(const LaunchArgs &a, const DecodeLane &l,
                                                     uint32_t li, uint32_t head, uint32_t lane) {
   const uint32_t H = a.kv_heads;
   const uint32_t slot = l.committed % kPage;
@@ -374,7 +391,7 @@ constexpr uint32_t kVerify48Depth = 1;
 template <uint32_t NB>
 __device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m, const bool *in_tile,
                                              const bool *live_row, const DecodeLane &l,
-                                             const DecodeArgs &a, uint32_t head, uint32_t split,
+                                             const LaunchArgs &a, uint32_t head, uint32_t split,
                                              uint32_t written, uint32_t g,
                                              uint16_t *__restrict__ output,
                                              float *__restrict__ partials,
@@ -435,16 +452,85 @@ __device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m,
 
 // The split kernel's body for NB blocks of 16 fused query rows per wave, with
 // kDepth register sets of pages.
-template <uint32_t NB, uint32_t kDepth, bool kReused = false>
+// kItemMajor: the launch has its work items in the grid's y and the KV heads in x
+// (DecodeArgs::item_major), and its lanes are plain lane records, never the regular tiles of a
+// prefill.
+template <uint32_t NB, uint32_t kDepth, bool kReused = false, bool kItemMajor = false>
 __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries,
                                             uint16_t *__restrict__ output,
                                             float *__restrict__ partials,
-                                            float *__restrict__ statistics, const DecodeArgs &a) {
+                                            float *__restrict__ statistics, const DecodeArgs &args) {
   // The forms that have a SIMD to themselves: three blocks, or two with two page sets.
   constexpr bool kPinned = NB == 3 || (NB == 2 && kDepth >= 2);
-  const uint32_t item = blockIdx.x, head = blockIdx.y;
+  const uint32_t item = kItemMajor ? blockIdx.y : blockIdx.x;
+  const uint32_t head = kItemMajor ? blockIdx.x : blockIdx.y;
   uint32_t li;
-  const DecodeLane l = lane_of_item(a, item, li);
+  DecodeLane l;
+  LaunchArgs a;
+  if constexpr (kItemMajor) {
+    // Every wave of the launch pays the way from its first instruction to its first page
+    // load at the same time, so that way is kept to three trips to memory: the launch-wide
+    // arguments with the first items of all lanes, the wave's lane record, its first page
+    // entries.  Left to itself the compiler fetches each field where it is first used, behind
+    // the branch before it, and fetches it again rather than keep it: ten trips one after the
+    // other, 5.6 us of a 100 us launch.  The empty statements below take in everything one
+    // trip brings and hand it out again as values the compiler cannot fetch anew, so the
+    // loads of a trip go out together and are waited for once.
+    uint32_t base[kLanes];
+#pragma unroll
+    for (uint32_t i = 0; i < kLanes; ++i) base[i] = args.item_base[i];
+    uint32_t kv_heads = args.kv_heads, group = args.group, fused_rows = args.fused_rows,
+             row_stride = args.row_stride, extent_pages = args.kv.extent_pages,
+             kv_offset = args.kv.offset, all_partials = args.all_partials,
+             chunk_stride = args.chunk_stride;
+    uint64_t chunk_keys = reinterpret_cast<uint64_t>(args.chunk_keys),
+             chunk_values = reinterpret_cast<uint64_t>(args.chunk_values),
+             chunk_lane_stride = args.chunk_lane_stride;
+    asm volatile("" : "+s"(base[0]), "+s"(base[1]), "+s"(base[2]), "+s"(base[3]), "+s"(base[4]),
+                      "+s"(base[5]), "+s"(base[6]), "+s"(base[7]), "+s"(base[8]), "+s"(base[9]),
+                      "+s"(base[10]), "+s"(base[11]), "+s"(base[12]), "+s"(base[13]),
+                      "+s"(base[14]), "+s"(base[15]));
+    asm volatile("" : "+s"(base[16]), "+s"(base[17]), "+s"(base[18]), "+s"(base[19]),
+                      "+s"(base[20]), "+s"(base[21]), "+s"(base[22]), "+s"(base[23]),
+                      "+s"(base[24]), "+s"(base[25]), "+s"(base[26]), "+s"(base[27]),
+                      "+s"(base[28]), "+s"(base[29]), "+s"(base[30]), "+s"(base[31]));
+    asm volatile("" : "+s"(kv_heads), "+s"(group), "+s"(fused_rows), "+s"(row_stride),
+                      "+s"(extent_pages), "+s"(kv_offset), "+s"(all_partials), "+s"(chunk_stride),
+                      "+s"(chunk_keys), "+s"(chunk_values), "+s"(chunk_lane_stride));
+    a = {kv_heads, group, fused_rows, row_stride, {extent_pages, kv_offset},
+         reinterpret_cast<const uint16_t *>(chunk_keys),
+         reinterpret_cast<const uint16_t *>(chunk_values), chunk_lane_stride, chunk_stride,
+         all_partials};
+    // base is non-decreasing: the lane is the number of later lanes that start at or
+    // before the item.
+    uint32_t index = 0;
+#pragma unroll
+    for (uint32_t i = 1; i < kLanes; ++i) index += item >= base[i] ? 1u : 0u;
+    const DecodeLane &from = args.lane[index];
+    uint64_t table = reinterpret_cast<uint64_t>(from.table),
+             masks = reinterpret_cast<uint64_t>(from.masks), row_base = from.row_base,
+             q_offset = from.q_offset;
+    uint32_t committed = from.committed, active_rows = from.active_rows,
+             split_count = from.split_count, first_item = from.first_item, source = from.source;
+    float lane_scale = from.score_scale;
+    asm volatile("" : "+s"(table), "+s"(masks), "+s"(row_base), "+s"(q_offset), "+s"(committed),
+                      "+s"(active_rows), "+s"(split_count), "+s"(first_item), "+s"(source),
+                      "+s"(lane_scale));
+    l.table = reinterpret_cast<const uint64_t *>(table);
+    l.masks = reinterpret_cast<const uint32_t *>(masks);
+    l.committed = committed;
+    l.active_rows = active_rows;
+    l.split_count = split_count;
+    l.first_item = first_item;
+    l.score_scale = lane_scale;
+    l.source = source;
+    l.row_base = row_base;
+    l.q_offset = q_offset;
+  } else {
+    l = lane_of_item(args, item, li);
+    a = launch_args_of(args);
+  }
+  li = l.source;  // the step's token rows lie in the caller's order of lanes
   const uint32_t split = item - l.first_item;
   if (split >= l.split_count) return;
   const uint32_t visible = l.committed + l.active_rows;
@@ -485,9 +571,25 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   const RegionOffsets ro = region_offsets(a.kv.extent_pages, db, sb);
   const float score_scale = default_score_scale(kD, l.score_scale);
 
+  // The split's first page entries, one per lane (lane i: slot i mod 2 kDepth, clamped), as
+  // one vector load ahead of everything else.  Every wave of a launch wants its first entries
+  // at the same moment, from cache lines nobody has touched yet: through the scalar cache,
+  // which a few CUs share and which takes few misses at a time, that trip took 3 to 4 us of
+  // the 5 a wave needs to issue its first page load; the vector path takes them all at once.
+  const uint64_t *const entries = l.table + begin;
+  const uint32_t last_slot = end - begin - 1;
+  const u32x2 first_entries = load_global<u32x2>(entries + min(lane & (2 * kDepth - 1), last_slot));
+  const auto first_entry = [&](uint32_t slot) {
+    // the builtin returns a signed int: through uint32_t, or the low half's top bit
+    // would spread over the high half
+    const uint32_t lo = uint32_t(__builtin_amdgcn_readlane(int(first_entries[0]), int(slot)));
+    const uint32_t hi = uint32_t(__builtin_amdgcn_readlane(int(first_entries[1]), int(slot)));
+    return uint64_t(lo) | uint64_t(hi) << 32;
+  };
+
   // Queries of this KV head: [row][g][D] bf16, fused row m.  Their loads go out
-  // first; everything behind them returns later, so the wait for the queries
-  // leaves the page loads in flight.  Columns without a live row carry zeros.
+  // ahead of the page loads; everything behind them returns later, so the wait for the
+  // queries leaves the page loads in flight.  Columns without a live row carry zeros.
   const uint16_t *q_head = queries + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
   u32x4 q_raw[NB][8];
 #pragma unroll
@@ -498,13 +600,11 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
       q_raw[nb][kb] = load_global<u32x4>(q_row + 8 * (16 * (kb >> 2) + 4 * g + (kb & 3)));
   }
 
-  // The split's page entries come through the scalar unit, each set's next entry
+  // The later page entries come through the scalar unit, each set's next entry
   // fetched a whole page period before the refill that uses it.
   // kDepth register sets rotate: a set is refilled with the page kDepth ahead as
   // soon as its page has been consumed, so up to kDepth pages are in flight.
   PageRegs r[kDepth];
-  const uint64_t *const entries = l.table + begin;
-  const uint32_t last_slot = end - begin - 1;
   uint64_t upcoming[kDepth];  // upcoming[d]: the entry of set d's next refill
   const LaneOffsets at = lane_offsets(t, g, uint32_t(ro.value_scales - ro.key_scales));
   // The empty asm statements pin the loads of one fill together and in place:
@@ -532,11 +632,9 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   // loads its last page again): the steady loop must be entered with the same
   // loads in flight, in the same order, as its own iterations leave behind.
 #pragma unroll
-  for (uint32_t d = 0; d < kDepth; ++d) upcoming[d] = scalar_entry(entries, min(d, last_slot));
-#pragma unroll
   for (uint32_t d = 0; d < kDepth; ++d) {
-    fill(r[d], upcoming[d]);
-    upcoming[d] = scalar_entry(entries, min(d + kDepth, last_slot));
+    fill(r[d], first_entry(d));
+    upcoming[d] = first_entry(d + kDepth);
   }
   if (appends && !appends_first) append_decode_token(a, l, li, head, lane);
 
@@ -623,7 +721,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_int4_kernel(
     const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
     float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
-  attend_int4<1, kDecodeDepth>(queries, output, partials, statistics, a);
+  attend_int4<1, kDecodeDepth, false, true>(queries, output, partials, statistics, a);
 }
 
 // The same for the 8-row tiles of a chunked prefill with several splits: every
@@ -764,7 +862,7 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   return launch_matrix_attention(decode_int4_kernel, "decode_int4_kernel", 16, 64, s, kv,
                                  query_heads, queries, output, page_tables, lanes, n_lanes,
                                  row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                 stream, fused, tile_rows, epilogue);
+                                 stream, fused, tile_rows, epilogue, /*longest_first=*/true);
 }
 
 extern "C" int kvx_calibrate_stream(const kvx_storage *s, uint32_t layer, const uint64_t *page_table,

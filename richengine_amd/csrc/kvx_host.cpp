@@ -3,6 +3,7 @@
 #include "kvx_internal.h"
 
 #include <algorithm>
+#include <vector>
 #include <chrono>
 #include <cstring>
 #include <limits>
@@ -213,24 +214,65 @@ int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_hea
   // with more waves than the kernel has wave slots: the overflow runs as a second
   // round on a nearly empty GPU (measured on 530 K tokens: int4 146 -> 115 us,
   // bf16 397 -> 350 us once the waves fit).  The int4 kernel holds two waves per
-  // SIMD and is fastest with 32 pages per split as long as those fit; the other
-  // formats' kernels are fastest with one wave per SIMD.
+  // SIMD; the other formats' kernels are fastest with one wave per SIMD.
   constexpr uint64_t kSimds = 1024;
   const uint64_t slots = format == KVX_FMT_INT4 ? 2 * kSimds : kSimds;
+  std::vector<uint32_t> pages(n_lanes);
   uint64_t page_heads = 0;
-  for (uint32_t i = 0; i < n_lanes; ++i) page_heads += uint64_t(pages_of(uint64_t(committed[i]) + 1)) * kv_heads;
+  for (uint32_t i = 0; i < n_lanes; ++i) {
+    pages[i] = pages_of(uint64_t(committed[i]) + 1);
+    page_heads += uint64_t(pages[i]) * kv_heads;
+  }
   uint32_t per = uint32_t(std::max<uint64_t>((page_heads + kSimds - 1) / kSimds, 8));
   if (format == KVX_FMT_INT4) per = std::min(per, KVX_DECODE_PAGES_PER_SPLIT);
+  uint64_t waves = 0;
   for (;; ++per) {
-    uint64_t waves = 0;
+    waves = 0;
     bool single = true;
     for (uint32_t i = 0; i < n_lanes; ++i) {
-      const uint32_t pages = pages_of(uint64_t(committed[i]) + 1);
-      split_counts[i] = std::min(std::max(1u, (pages + per - 1) / per), KVX_DECODE_MAX_SPLITS);
+      split_counts[i] = std::min(std::max(1u, (pages[i] + per - 1) / per), KVX_DECODE_MAX_SPLITS);
       waves += uint64_t(split_counts[i]) * kv_heads;
       single = single && split_counts[i] == 1;
     }
     if (waves <= slots || single) break;  // one split per lane is the fewest waves there can be
+  }
+  if (format != KVX_FMT_INT4 || n_lanes > KVX_LANES_PER_LAUNCH || waves <= kSimds) return KVX_OK;
+  // int4, a launch with two waves on most SIMDs.  The two do not share their SIMD evenly:
+  // the wave that was dispatched first runs ahead of the other (measured on splits of equal
+  // length: 2.05 against 3.9 us per page while both run), ends a quarter of the launch early
+  // and leaves the other alone, and a lone wave of this kernel cannot keep its share of the
+  // memory system busy.  So the lanes are planned in two classes: long splits for exactly the
+  // first wave of every SIMD (the launch dispatches the lanes with the longest splits first,
+  // the heads of a work item side by side), and splits of kPairedShortShare of that length
+  // for the second, which then end together (same batch and GPU: 104 -> 100 us per launch, 1.83 -> 1.76 ms per
+  // step; shares of 0.52 / 0.56 / 0.60 / 0.64 gave 1.80 / 1.767 / 1.761 / 1.785 ms).  Lanes
+  // go to the long class from the longest down while their waves fit one per SIMD, lanes that
+  // do not fit to the short class; the long length is the least whose short class fits the
+  // second waves.
+  constexpr double kPairedShortShare = 0.58;
+  std::vector<uint32_t> order(n_lanes);
+  for (uint32_t i = 0; i < n_lanes; ++i) order[i] = i;
+  std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) { return pages[x] > pages[y]; });
+  std::vector<uint32_t> paired(n_lanes);
+  for (uint32_t longer = 8; longer <= KVX_MAX_PHYSICAL_TOKENS / KVX_PAGE_TOKENS; ++longer) {
+    const uint32_t shorter = std::max(4u, uint32_t(kPairedShortShare * longer));
+    uint64_t first_waves = 0, second_waves = 0;
+    bool capped = false;
+    for (uint32_t i : order) {
+      const uint32_t as_long = (pages[i] + longer - 1) / longer;
+      if (first_waves + uint64_t(as_long) * kv_heads <= kSimds) {
+        paired[i] = as_long;
+        first_waves += uint64_t(as_long) * kv_heads;
+      } else {
+        paired[i] = (pages[i] + shorter - 1) / shorter;
+        second_waves += uint64_t(paired[i]) * kv_heads;
+      }
+      capped = capped || paired[i] > KVX_DECODE_MAX_SPLITS;
+    }
+    if (second_waves <= kSimds && !capped) {
+      std::copy(paired.begin(), paired.end(), split_counts);
+      break;
+    }
   }
   return KVX_OK;
 }
@@ -363,6 +405,10 @@ static int storage_create(const kvx_layout *layout, uint32_t page_count, uint32_
     delete s;
     return fail(KVX_EDEVICE, "no HIP device: the paged KV path needs a GPU");
   }
+  // The static workspace's address on this device, asked here so that no launch has to
+  // (a launch may be under stream capture).  A refusal only matters to the entry that
+  // uses the workspace, which then reports it.
+  if (!accounting && kvx::prime_static_workspace(s->device) != KVX_OK) (void)hipGetLastError();
   *out = s;
   return KVX_OK;
 }

@@ -13,6 +13,9 @@ namespace kvx {
 
 // ---- errors -----------------------------------------------------------------
 int fail(int code, const std::string &message);
+// Looks up, once per device, where the static workspace of kv_attend_decode_static lies
+// on `device` (the current one).
+int prime_static_workspace(int device);
 int hip_fail(hipError_t error, const char *what);
 #define KVX_HIP(call)                                     \
   do {                                                    \

@@ -4,6 +4,7 @@
 // The arithmetic of every kernel here keeps the operation order of the
 // reference kernels it replaces (cited per kernel), with products and sums
 // left unfused so the fp32 results do not depend on contraction.
+#include <atomic>
 #include <algorithm>
 #include <vector>
 
@@ -147,7 +148,7 @@ struct PrepareArgs {
   uint32_t rows;        // rows per lane in packed / rope_cos / rope_sin
   uint32_t row_stride;  // rows between KV heads in the queries
   float eps;
-  uint32_t group_magic;  // ceil(2^32 / group): head / group = mulhi(head, group_magic) for head < 2^16
+  uint32_t group_magic;  // ceil(2^32 / group) for group > 1: head / group = mulhi(head, group_magic) for head < 2^16
 };
 
 template <uint32_t FMT>
@@ -451,7 +452,10 @@ __global__ __launch_bounds__(256) void prepare_append_wave_kernel(PrepareArgs p)
     prepared[e] = rotated ? f32_to_bf16_hw(is_first ? mc - os : mc + os) : normal;
   }
   if (query) {
-    const uint32_t kv_head = __umulhi(head, p.group_magic), local_head = head - kv_head * G;
+    // A group of one query head has no reciprocal that fits 32 bits (2^32): the head is
+    // its own KV head then.
+    const uint32_t kv_head = G == 1 ? head : __umulhi(head, p.group_magic);
+    const uint32_t local_head = head - kv_head * G;
     store_bf16s<E>(p.queries + uint64_t(li) * H * p.row_stride * G * D +
                        ((uint64_t(kv_head) * p.row_stride + row) * G + local_head) * D + d0,
                    prepared);
@@ -1422,7 +1426,7 @@ int kv_prepare_append(const kvx_storage *s, uint32_t layer, const kvx_qkv_shape 
     p.rows = rows;
     p.row_stride = row_stride;
     p.eps = shape->eps != 0.0f ? shape->eps : 1e-6f;
-    p.group_magic = uint32_t((0x100000000ull + QH / H - 1) / (QH / H));
+    p.group_magic = QH / H > 1 ? uint32_t((0x100000000ull + QH / H - 1) / (QH / H)) : 0u;
     // One wave per task where the head dimension is 64, 128 or 256 and a rotary pair's
     // dimensions are a power-of-two number of lanes apart; else one workgroup per task.
     const uint32_t E = D / 64, pair_lanes = E ? shape->rotary_pairs / E : 0;
@@ -1465,7 +1469,8 @@ static int validate_attend(const kvx_storage *s, uint32_t query_heads,
       return fail(KVX_EINVAL, "verify active rows are out of range");
     if (uint64_t(p.committed_tokens) + p.active_rows > KVX_MAX_PHYSICAL_TOKENS)
       return fail(KVX_EINVAL, "verify attention history exceeds physical context");
-    if (p.page_table_entries < (uint64_t(p.committed_tokens) + p.active_rows + 31) / 32)
+    // (a call that reads no pages, the merge alone, brings no tables and need not size them)
+    if (page_tables && p.page_table_entries < (uint64_t(p.committed_tokens) + p.active_rows + 31) / 32)
       return fail(KVX_EINVAL, "page_table_too_short");
     if (!p.split_count || p.split_count > max_splits)
       return fail(KVX_EINVAL, "verify split count is out of range");
@@ -1705,15 +1710,6 @@ int kv_attend_decode_shared(const kvx_storage *s, uint32_t layer, uint32_t query
   prefix.split_count = prefix.slot_splits = prefix_splits;
   prefix.active_rows = prefix.row_capacity = n_lanes;
   prefix.score_scale = lanes[0].score_scale;
-  // The matrix-core kernels stage one split's page entries in LDS, 1024 at most.
-  const auto split_fits = [](const kvx_verify_params &p) {
-    const uint32_t pages = (p.committed_tokens + p.active_rows + kPage - 1) / kPage;
-    return (pages + p.split_count - 1) / p.split_count <= 1024;
-  };
-  bool fits = split_fits(prefix);
-  for (uint32_t i = 0; i < n_lanes; ++i) fits = fits && split_fits(own[i]);
-  if (!fits) return fail(KVX_EINVAL, "a split is longer than 1024 pages: use more splits");
-
   uint8_t *base = static_cast<uint8_t *>(workspace);
   uint16_t *staged = reinterpret_cast<uint16_t *>(base);
   base += align256(uint64_t(n_lanes) * query_heads * D * 2);
@@ -1809,25 +1805,58 @@ static __device__ __align__(256) unsigned char kvx_static_scratch[kStaticScratch
 
 namespace {
 constexpr int kMaxDevices = 64;
-void *g_static_scratch[kMaxDevices] = {};  // the array's address on each device, once known
+// The array's address on each device, once known.  Written once per device (any thread
+// that asks gets the same answer from the runtime), read by every launch.
+std::atomic<void *> g_static_scratch[kMaxDevices];
+}  // namespace
 
+// Asks the runtime for the array's address on `device`, which must be the current one.
+// Creating a storage does this for its device, so that no launch has to: asking is a
+// call of the runtime that is no stream operation and may load the library's code
+// object, neither of which belongs into a stream capture.
+extern "C++" {
+int kvx::prime_static_workspace(int device) {
+  if (device < 0 || device >= kMaxDevices) return fail(KVX_EDEVICE, "device index out of range");
+  if (g_static_scratch[device].load(std::memory_order_acquire)) return KVX_OK;
+  void *address = nullptr;
+  KVX_HIP(hipGetSymbolAddress(&address, HIP_SYMBOL(kvx_static_scratch)));
+  if (!address) return fail(KVX_EDEVICE, "the static workspace has no address on this device");
+  g_static_scratch[device].store(address, std::memory_order_release);
+  return KVX_OK;
+}
+}  // extern "C++"
+
+namespace {
 // The address of the scratch array on the current device, which must be the storage's.
-int static_scratch(const kvx_storage *s, void **out) {
+int static_scratch(const kvx_storage *s, hipStream_t stream, void **out) {
   int device = -1;
   KVX_HIP(hipGetDevice(&device));
   if (device < 0 || device >= kMaxDevices) return fail(KVX_EDEVICE, "device index out of range");
   if (device != s->device)
     return fail(KVX_ESTATE, "the storage's device is not the current device");
-  if (!g_static_scratch[device]) {
-    void *address = nullptr;
-    KVX_HIP(hipGetSymbolAddress(&address, HIP_SYMBOL(kvx_static_scratch)));
-    if (!address) return fail(KVX_EDEVICE, "the static workspace has no address on this device");
-    g_static_scratch[device] = address;
+  if (!g_static_scratch[device].load(std::memory_order_acquire)) {
+    // Not asked yet on this device (the storage was created while another was current).
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) (void)hipGetLastError();
+    if (capturing != hipStreamCaptureStatusNone)
+      return fail(KVX_ESTATE, "the static workspace's address is not known on this device yet: "
+                              "call kvx_static_workspace_prime before the capture");
+    if (const int rc = kvx::prime_static_workspace(device)) return rc;
   }
-  *out = g_static_scratch[device];
+  *out = g_static_scratch[device].load(std::memory_order_acquire);
   return KVX_OK;
 }
 }  // namespace
+
+int kvx_static_workspace_prime(const kvx_storage *s) {
+  if (!s) return fail(KVX_EINVAL, "kvx_static_workspace_prime: null storage");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
+  int device = -1;
+  KVX_HIP(hipGetDevice(&device));
+  if (device != s->device)
+    return fail(KVX_ESTATE, "the storage's device is not the current device");
+  return kvx::prime_static_workspace(device);
+}
 
 int kv_attend_decode_static(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
                             const void *queries, void *output, const uint64_t *const *page_tables,
@@ -1842,7 +1871,7 @@ int kv_attend_decode_static(const kvx_storage *s, uint32_t layer, uint32_t query
                                 std::to_string(kStaticScratchBytes) +
                                 "; use kv_attend_decode with a workspace of the caller's");
   void *scratch = nullptr;
-  if (const int rc = static_scratch(s, &scratch)) return rc;
+  if (const int rc = static_scratch(s, static_cast<hipStream_t>(stream), &scratch)) return rc;
   // Every partial row and statistic a merge reads is written by the split kernel of the
   // same call first, so nothing of the previous call's contents has to be cleared.
   return kv_attend_decode(s, layer, query_heads, queries, output, page_tables, lanes, n_lanes,

@@ -217,17 +217,62 @@ void PrefixCache::follow_pages(const PageMoves &moves) {
   }
 }
 
-uint64_t PrefixCache::extend_match(std::vector<uint64_t> *blocks, const uint32_t *prompt,
-                                   uint64_t n) const {
+// The identity is a value that travels with a block's key (and would be persisted
+// with it), so its bits are the reference's: two chains with their own seeds fold,
+// for every span that overlaps the block, the span's content digest, its grid, its
+// place in the prompt and the block's start.  `a ^= v + golden + (a << 6) + (a >> 2)`
+// is the fold of both chains; the second takes the complement of every value.
+void block_image_identity(uint64_t block_begin, uint32_t block_tokens, const kvx_image_span *spans,
+                          uint32_t n_spans, uint64_t *lo, uint64_t *hi) {
+  const auto fold = [](uint64_t a, uint64_t v) {
+    return a ^ (v + 0x9e3779b97f4a7c15ull + (a << 6) + (a >> 2));
+  };
+  uint64_t chain_lo = 0, chain_hi = 0;
+  const uint64_t block_end = block_begin + block_tokens;
+  for (uint32_t i = 0; i < n_spans; ++i) {
+    const kvx_image_span &span = spans[i];
+    if (span.offset >= block_end) break;  // spans are sorted by offset
+    if (uint32_t(span.offset + span.tokens) <= block_begin) continue;  // 32-bit end, as ImageSpan::end()
+    const uint64_t words[5] = {span.digest_lo, span.digest_hi,
+                               uint64_t(span.grid_height) << 32 | span.grid_width,
+                               uint64_t(span.offset) << 32 | span.tokens, block_begin};
+    if (!chain_lo) chain_lo = 0x243f6a8885a308d3ull;
+    if (!chain_hi) chain_hi = 0x13198a2e03707344ull;
+    for (const uint64_t word : words) {
+      chain_lo = fold(chain_lo, word);
+      chain_hi = fold(chain_hi, ~word);
+    }
+  }
+  *lo = chain_lo;
+  *hi = chain_hi;
+}
+
+namespace {
+// The spans that can still overlap the block at `block_begin` or a later one (Cache.cpp:16-22):
+// sorted and disjoint, a span that ends before a block ends before every later block too.
+void spans_from(const kvx_image_span *&spans, uint32_t &n_spans, uint64_t block_begin) {
+  while (n_spans && uint32_t(spans->offset + spans->tokens) <= block_begin) {
+    ++spans;
+    --n_spans;
+  }
+}
+}  // namespace
+
+uint64_t PrefixCache::extend_match(std::vector<uint64_t> *blocks, const uint32_t *prompt, uint64_t n,
+                                   const kvx_image_span *spans, uint32_t n_spans) const {
   if (!n) return 0;
   // Leave one real input token to compute the first logits from.
   const uint64_t maximum = (n - 1) / KVX_PAGE_TOKENS;
   uint64_t hashed = 0;
   for (uint64_t index = blocks->size(); index < maximum; ++index) {
+    const uint64_t begin = index * KVX_PAGE_TOKENS;
     const uint64_t parent = blocks->empty() ? 0 : blocks->back();
+    spans_from(spans, n_spans, begin);
+    uint64_t image_lo = 0, image_hi = 0;
+    block_image_identity(begin, KVX_PAGE_TOKENS, spans, n_spans, &image_lo, &image_hi);
     ++hashed;
     uint64_t id = 0;
-    if (!find(parent, prompt + index * KVX_PAGE_TOKENS, KVX_PAGE_TOKENS, 0, 0, &id, nullptr)) break;
+    if (!find(parent, prompt + begin, KVX_PAGE_TOKENS, image_lo, image_hi, &id, nullptr)) break;
     blocks->push_back(id);
   }
   return hashed;
@@ -310,6 +355,25 @@ int SequenceCache::fork(uint64_t id, uint64_t source, uint64_t tokens) {
   return KVX_OK;
 }
 
+// The counterpart of ensure_tokens after a speculative rollback: the reference keeps
+// "the pages of tokens + scratch" by never asking for more (Engine.cpp:1190-1193) and lets
+// rejected rows lie where they are (abi/PagedAttention.h:33-38); a tree of 16 draft rows can
+// leave a whole page without a committed token, which goes back to the pool here.
+int SequenceCache::truncate(uint64_t id, uint64_t tokens, uint32_t *released) {
+  *released = 0;
+  const auto found = sequences_.find(id);
+  if (found == sequences_.end()) return KVX_ERANGE;
+  Sequence &s = found->second;
+  const uint64_t keep = (tokens + KVX_PAGE_TOKENS - 1) / KVX_PAGE_TOKENS;
+  if (keep < s.blocks.size()) return KVX_ESTATE;  // a published page is history, not scratch
+  if (keep >= s.pages.size()) return KVX_OK;
+  for (size_t index = size_t(keep); index < s.pages.size(); ++index) pool_.release(s.pages[index], false);
+  *released = uint32_t(s.pages.size() - keep);
+  s.pages.resize(size_t(keep));
+  changed(s, uint32_t(keep));
+  return KVX_OK;
+}
+
 int SequenceCache::ensure_writable(uint64_t id, uint64_t token, bool *copied, uint32_t *from,
                                    uint32_t *to) {
   *copied = false;
@@ -342,7 +406,7 @@ int SequenceCache::ensure_writable(uint64_t id, uint64_t token, bool *copied, ui
 // becomes a block; where the content is already cached the sequence moves to
 // the canonical page and gives its own back.
 int SequenceCache::publish(uint64_t id, const uint32_t *tokens, uint64_t n_tokens,
-                           uint32_t committed) {
+                           uint32_t committed, const kvx_image_span *spans, uint32_t n_spans) {
   const auto found = sequences_.find(id);
   if (found == sequences_.end()) return KVX_ERANGE;
   Sequence &s = found->second;
@@ -357,8 +421,12 @@ int SequenceCache::publish(uint64_t id, const uint32_t *tokens, uint64_t n_token
     uint64_t block = 0;
     uint32_t canonical = 0;
     const uint32_t writer = s.pages[logical];
-    if (const int rc = prefix_.insert(parent, tokens + uint64_t(logical) * KVX_PAGE_TOKENS,
-                                      KVX_PAGE_TOKENS, writer, 0, 0, &block, &canonical))
+    const uint64_t begin = uint64_t(logical) * KVX_PAGE_TOKENS;
+    spans_from(spans, n_spans, begin);
+    uint64_t image_lo = 0, image_hi = 0;
+    block_image_identity(begin, KVX_PAGE_TOKENS, spans, n_spans, &image_lo, &image_hi);
+    if (const int rc = prefix_.insert(parent, tokens + begin, KVX_PAGE_TOKENS, writer, image_lo,
+                                      image_hi, &block, &canonical))
       return rc;
     const bool replace = canonical != writer;
     if (replace) pool_.retain(canonical, false);

@@ -24,6 +24,10 @@
 
 namespace kvx {
 
+// engine::blockImageIdentity (runtime/engine/cache/KvCache.cpp:29-52).
+void block_image_identity(uint64_t block_begin, uint32_t block_tokens, const kvx_image_span *spans,
+                          uint32_t n_spans, uint64_t *lo, uint64_t *hi);
+
 class PrefixCache {
 public:
   static constexpr uint32_t kNoPage = 0xffffffffu;
@@ -51,9 +55,12 @@ public:
   int erase(uint64_t block);
   // KvCache::followPages after an extent compaction.
   void follow_pages(const PageMoves &moves);
-  // Cache::extendMatch for text-only prompts: appends matched blocks, leaving at
-  // least one prompt token unmatched; returns how many pages were looked up.
-  uint64_t extend_match(std::vector<uint64_t> *blocks, const uint32_t *prompt, uint64_t n) const;
+  // Cache::extendMatch: appends matched blocks, leaving at least one prompt token
+  // unmatched; returns how many pages were looked up.  Every block is looked up
+  // under the identity of the prompt's images that overlap it (`spans` sorted by
+  // offset and disjoint; none for a text-only prompt).
+  uint64_t extend_match(std::vector<uint64_t> *blocks, const uint32_t *prompt, uint64_t n,
+                        const kvx_image_span *spans = nullptr, uint32_t n_spans = 0) const;
   uint64_t generation() const { return generation_; }
   uint64_t block_count() const { return blocks_.size(); }
 
@@ -107,8 +114,12 @@ public:
   // holds it is replaced by a private copy (all layers, on the pool's copy stream)
   // when anyone else holds it too; *copied says whether, *from / *to which pages.
   int fork(uint64_t id, uint64_t source, uint64_t tokens);
+  // Gives back the pages past those that hold the first `tokens` tokens (a rollback
+  // that emptied them); *released says how many.  Published pages stay.
+  int truncate(uint64_t id, uint64_t tokens, uint32_t *released);
   int ensure_writable(uint64_t id, uint64_t token, bool *copied, uint32_t *from, uint32_t *to);
-  int publish(uint64_t id, const uint32_t *tokens, uint64_t n_tokens, uint32_t committed);
+  int publish(uint64_t id, const uint32_t *tokens, uint64_t n_tokens, uint32_t committed,
+              const kvx_image_span *spans = nullptr, uint32_t n_spans = 0);
   struct View {                                             // Cache::pageTable
     const uint32_t *pages;
     uint32_t count;

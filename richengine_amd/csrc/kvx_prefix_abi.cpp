@@ -103,42 +103,23 @@ void kvx_prefix_follow_pages(kvx_prefix *prefix, uint32_t first_page, const uint
 }
 uint64_t kvx_prefix_match(const kvx_prefix *prefix, const uint32_t *prompt, uint64_t n_tokens,
                           uint64_t *blocks, uint32_t capacity, uint32_t *matched) {
+  return kvx_prefix_match_images(prefix, prompt, n_tokens, nullptr, 0, blocks, capacity, matched);
+}
+uint64_t kvx_prefix_match_images(const kvx_prefix *prefix, const uint32_t *prompt, uint64_t n_tokens,
+                                 const kvx_image_span *spans, uint32_t n_spans, uint64_t *blocks,
+                                 uint32_t capacity, uint32_t *matched) {
   std::vector<uint64_t> chain;
-  const uint64_t hashed = prefix->cache.extend_match(&chain, prompt, n_tokens);
+  const uint64_t hashed =
+      prefix->cache.extend_match(&chain, prompt, n_tokens, spans, spans ? n_spans : 0);
   if (matched) *matched = uint32_t(chain.size());
   for (uint32_t i = 0; i < chain.size() && i < capacity; ++i) blocks[i] = chain[i];
   return hashed;
 }
 
-// The identity is a value that travels with a block's key (and would be persisted
-// with it), so its bits are the reference's: two chains with their own seeds fold,
-// for every span that overlaps the block, the span's content digest, its grid, its
-// place in the prompt and the block's start.  `a ^= v + golden + (a << 6) + (a >> 2)`
-// is the fold of both chains; the second takes the complement of every value.
 void kvx_block_image_identity(uint64_t block_begin, uint32_t block_tokens,
                               const kvx_image_span *spans, uint32_t n_spans, uint64_t *lo,
                               uint64_t *hi) {
-  const auto fold = [](uint64_t a, uint64_t v) {
-    return a ^ (v + 0x9e3779b97f4a7c15ull + (a << 6) + (a >> 2));
-  };
-  uint64_t chain_lo = 0, chain_hi = 0;
-  const uint64_t block_end = block_begin + block_tokens;
-  for (uint32_t i = 0; i < n_spans; ++i) {
-    const kvx_image_span &span = spans[i];
-    if (span.offset >= block_end) break;  // spans are sorted by offset
-    if (uint32_t(span.offset + span.tokens) <= block_begin) continue;  // 32-bit end, as ImageSpan::end()
-    const uint64_t words[5] = {span.digest_lo, span.digest_hi,
-                               uint64_t(span.grid_height) << 32 | span.grid_width,
-                               uint64_t(span.offset) << 32 | span.tokens, block_begin};
-    if (!chain_lo) chain_lo = 0x243f6a8885a308d3ull;
-    if (!chain_hi) chain_hi = 0x13198a2e03707344ull;
-    for (const uint64_t word : words) {
-      chain_lo = fold(chain_lo, word);
-      chain_hi = fold(chain_hi, ~word);
-    }
-  }
-  *lo = chain_lo;
-  *hi = chain_hi;
+  kvx::block_image_identity(block_begin, block_tokens, spans, n_spans, lo, hi);
 }
 
 int kvx_sequences_create(kvx_pool *pool, kvx_prefix *prefix, kvx_sequences **out) {
@@ -171,6 +152,13 @@ int kvx_sequence_fork(kvx_sequences *s, uint64_t id, uint64_t source, uint64_t t
     return report(rc, "unknown sequence");
   }
 }
+int kvx_sequence_truncate(kvx_sequences *s, uint64_t id, uint64_t tokens, uint32_t *released_pages) {
+  uint32_t released = 0;
+  const int rc = s->sequences.truncate(id, tokens, &released);
+  if (released_pages) *released_pages = released;
+  if (rc == KVX_ESTATE) return kvx::fail(rc, "truncation would drop a published page");
+  return report(rc, "unknown sequence");
+}
 int kvx_sequence_ensure_writable(kvx_sequences *s, uint64_t id, uint64_t token, uint32_t *copied,
                                  uint32_t *from_page, uint32_t *to_page, void *stream) {
   bool did = false;
@@ -194,7 +182,13 @@ int kvx_sequence_ensure_writable(kvx_sequences *s, uint64_t id, uint64_t token, 
 }
 int kvx_sequence_publish(kvx_sequences *s, uint64_t id, const uint32_t *tokens, uint64_t n_tokens,
                          uint32_t committed_tokens) {
-  const int rc = s->sequences.publish(id, tokens, n_tokens, committed_tokens);
+  return kvx_sequence_publish_images(s, id, tokens, n_tokens, committed_tokens, nullptr, 0);
+}
+int kvx_sequence_publish_images(kvx_sequences *s, uint64_t id, const uint32_t *tokens,
+                                uint64_t n_tokens, uint32_t committed_tokens,
+                                const kvx_image_span *spans, uint32_t n_spans) {
+  const int rc =
+      s->sequences.publish(id, tokens, n_tokens, committed_tokens, spans, spans ? n_spans : 0);
   switch (rc) {
   case KVX_EINVAL:
     return kvx::fail(rc, "committed KV exceeds exact token history");

@@ -45,6 +45,8 @@ SYMBOLS = [
     "kvx_sequence_ensure_tokens", "kvx_sequence_publish", "kvx_sequence_view",
     "kvx_sequences_compact_extent", "kvx_tree_masks", "kvx_tree_path_valid",
     "kvx_sequence_fork", "kvx_sequence_ensure_writable", "kvx_block_image_identity",
+    "kvx_prefix_match_images", "kvx_sequence_publish_images", "kvx_sequence_truncate",
+    "kvx_static_workspace_prime",
 ]
 
 
@@ -190,6 +192,10 @@ def _declare(L):
     L.kvx_sequence_ensure_writable.argtypes = [vp, u64, u64, PU32, PU32, PU32, vp]
     L.kvx_block_image_identity.argtypes = [u64, u32, vp, u32, PU64, PU64]
     L.kvx_block_image_identity.restype = None
+    L.kvx_prefix_match_images.argtypes = [vp, vp, u64, vp, u32, vp, u32, PU32]
+    L.kvx_prefix_match_images.restype = u64
+    L.kvx_sequence_publish_images.argtypes = [vp, u64, vp, u64, u32, vp, u32]
+    L.kvx_sequence_truncate.argtypes = [vp, u64, u64, PU32]
     L.kvx_debug_attend_paths.argtypes, L.kvx_debug_attend_paths.restype = [PU64, PU64], None
     L.kvx_calibrate_stream.argtypes = [vp, u32, vp, u32, u32, u32, vp, vp]
     L.kvx_decode_plan.argtypes = [vp, u32, u32, u32, vp]
@@ -644,11 +650,18 @@ class Prefix:
             dest = _u32(moves["dest"])
             lib().kvx_prefix_follow_pages(self.h, moves["first"], dest, len(moves["dest"]))
 
-    def match(self, prompt):
+    def match(self, prompt, spans=()):
+        """spans: the prompt's images as (offset, tokens, grid height, grid width, digest lo,
+        digest hi) tuples sorted by offset; none for a text-only prompt."""
         capacity = max(len(prompt) // 32, 1)
         blocks, matched = (C.c_uint64 * capacity)(), C.c_uint32()
-        hashed = lib().kvx_prefix_match(self.h, _u32(prompt), len(prompt), blocks, capacity,
-                                        C.byref(matched))
+        if spans:
+            arr = (ImageSpan * len(spans))(*[ImageSpan(*s) for s in spans])
+            hashed = lib().kvx_prefix_match_images(self.h, _u32(prompt), len(prompt), arr, len(spans),
+                                                   blocks, capacity, C.byref(matched))
+        else:
+            hashed = lib().kvx_prefix_match(self.h, _u32(prompt), len(prompt), blocks, capacity,
+                                            C.byref(matched))
         return list(blocks[:matched.value]), hashed
 
 
@@ -681,9 +694,19 @@ class Sequences:
     def ensure_tokens(self, sequence, tokens):
         return check(lib().kvx_sequence_ensure_tokens(self.h, sequence, tokens))
 
-    def publish(self, sequence, tokens, committed):
+    def publish(self, sequence, tokens, committed, spans=()):
+        if spans:
+            arr = (ImageSpan * len(spans))(*[ImageSpan(*s) for s in spans])
+            return check(lib().kvx_sequence_publish_images(self.h, sequence, _u32(tokens), len(tokens),
+                                                           committed, arr, len(spans)))
         return check(lib().kvx_sequence_publish(self.h, sequence, _u32(tokens), len(tokens),
                                                 committed))
+
+    def truncate(self, sequence, tokens):
+        """Gives back the pages past those of the first `tokens` tokens; returns how many."""
+        released = C.c_uint32()
+        check(lib().kvx_sequence_truncate(self.h, sequence, tokens, C.byref(released)))
+        return released.value
 
     def fork(self, sequence, source, tokens):
         """`sequence` (empty) shares the pages of the first `tokens` tokens of `source`."""

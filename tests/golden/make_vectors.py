@@ -17,6 +17,7 @@ from the library under test.  Sources of the expected values:
   chunk_*       kv::chunkedPrefillValidationError / RequiredPages
   q8_*, f8_*    whole-page quantizers           dev/tests/engine/Q8PageFormatReference.hpp:141-180,
                                                 dev/tests/engine/Fp8PageFormatReference.hpp:147-186
+  identity_*    engine::blockImageIdentity      runtime/engine/cache/KvCache.cpp:29-52
 """
 import ctypes as C
 import os
@@ -134,6 +135,35 @@ def main():
             out[f"{name}_{case}_page"] = page
 
     path = os.path.join(HERE, "reference_vectors.npz")
+    # ---- image identities: span lists (sorted, disjoint) and blocks around them
+    if ko.ref_image_identity(0, 32, []) is None:
+        raise SystemExit("oracle/_ref/libkvref_cache.so is missing: run make -C oracle ref")
+    cases, spans_flat, spans_first, answers = [], [], [0], []
+    for case in range(48):
+        spans, at = [], int(rng.integers(0, 70))
+        for _ in range(int(rng.integers(0, 4))):
+            tokens = int(rng.integers(1, 90))
+            spans.append((at, tokens, int(rng.integers(1, 40)), int(rng.integers(1, 40)),
+                          int(rng.integers(0, 2**63)) * 2 + int(rng.integers(0, 2)),
+                          int(rng.integers(0, 2**63)) * 2 + int(rng.integers(0, 2))))
+            at += tokens + int(rng.integers(0, 50))
+        if case == 0:
+            spans = []                                      # a text-only prompt
+        if case == 1:
+            spans = [(0xFFFFFFF0, 0x20, 3, 3, 5, 7)]        # a span whose 32-bit end wraps
+        for begin in sorted({0, 32, 64, 96, 160, 320} | {s[0] // 32 * 32 for s in spans} |
+                            {(s[0] + s[1]) // 32 * 32 for s in spans}):
+            cases.append((len(spans_first) - 1, begin & 0xFFFFFFFFFFFF, 32))
+            answers.append(ko.ref_image_identity(begin, 32, spans))
+        cases.append((len(spans_first) - 1, 7, 100))         # a block that is not a page
+        answers.append(ko.ref_image_identity(7, 100, spans))
+        spans_flat += spans
+        spans_first.append(len(spans_flat))
+    out["identity_spans"] = np.array(spans_flat, dtype=np.uint64).reshape(-1, 6)
+    out["identity_spans_first"] = np.array(spans_first, dtype=np.uint32)
+    out["identity_cases"] = np.array(cases, dtype=np.uint64)      # (span list, block begin, block tokens)
+    out["identity_out"] = np.array(answers, dtype=np.uint64)      # (lo, hi)
+
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes,", len(out), "arrays")
 

@@ -126,6 +126,26 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
                 if sum(want) * H <= slots or all(s == 1 for s in want):
                     break
                 per += 1
+            if fmt == kvx.INT4 and lanes <= 32 and sum(want) * H > 1024:
+                # two waves on most SIMDs: long splits for exactly the first wave of every
+                # SIMD, from the longest lane down while they fit, and splits of 0.58
+                # of that length for the second waves; the least long length that fits
+                counts = [pages(c + 1) for c in committed]
+                order = sorted(range(lanes), key=lambda i: -counts[i])
+                for longer in range(8, 8200):
+                    shorter = max(4, int(0.58 * longer))
+                    first = second = 0
+                    want = [0] * lanes
+                    for i in order:
+                        as_long = -(-counts[i] // longer)
+                        if first + as_long * H <= 1024:
+                            want[i], first = as_long, first + as_long * H
+                        else:
+                            want[i] = -(-counts[i] // shorter)
+                            second += want[i] * H
+                    if second <= 1024 and max(want) <= 512:
+                        break
+                assert first <= 1024 and second <= 1024
             assert plan == want
         for rows, fmt in ((2, kvx.INT4), (8, kvx.INT4), (8, kvx.INT8), (16, kvx.INT4), (16, kvx.BF16)):
             plan = kvx.verify_plan(committed, rows, H, QH, fmt)

@@ -94,6 +94,37 @@ def test_planning():
         assert K.kvx_chunk_validation(C.byref(q)) == int(error)
 
 
+def identity_cases():
+    spans, first = G["identity_spans"], G["identity_spans_first"]
+    for (which, begin, tokens), want in zip(G["identity_cases"], G["identity_out"]):
+        mine = [tuple(int(w) for w in row) for row in spans[first[int(which)]:first[int(which) + 1]]]
+        yield mine, int(begin), int(tokens), (int(want[0]), int(want[1]))
+
+
+def test_image_identity_values_of_the_reference():
+    """The 128-bit values of engine::blockImageIdentity (runtime/engine/cache/KvCache.cpp:29-52),
+    written from the reference's own compiled function: the oracle's restatement and the
+    library's entry give the same bits, for pages and for blocks that are no page, for spans
+    before, inside, across and after the block, and for a span whose 32-bit end wraps."""
+    from oracle import prefix_oracle as po
+    seen_zero = seen_value = 0
+    for spans, begin, tokens, want in identity_cases():
+        assert po.block_image_identity(begin, tokens, spans) == want, (spans, begin, tokens)
+        assert kvx.block_image_identity(begin, tokens, spans) == want, (spans, begin, tokens)
+        seen_zero += want == (0, 0)
+        seen_value += want != (0, 0)
+    assert seen_zero > 50 and seen_value > 50
+
+
+def test_image_identity_fixture_is_what_the_reference_returns():
+    """Where the reference checkout was present at build time: the fixture against a fresh
+    call of the reference's function."""
+    if ko.ref_image_identity(0, 32, []) is None:
+        pytest.skip("oracle/_ref/libkvref_cache.so was not built")
+    for spans, begin, tokens, want in identity_cases():
+        assert ko.ref_image_identity(begin, tokens, spans) == want
+
+
 PAGES = [("q8", ko.INT8, "a"), ("q8", ko.INT8, "b"), ("f8", ko.FP8, "a"), ("f8", ko.FP8, "b")]
 
 

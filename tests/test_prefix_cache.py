@@ -94,9 +94,9 @@ class OracleStack:
     def touch(self, b): return self.call(self.prefix.touch, b)
     def candidate(self, after=0): return self.prefix.eviction_candidate(after)
     def erase(self, b): return self.call(self.prefix.erase, b)
-    def match(self, prompt):
+    def match(self, prompt, spans=()):
         blocks = []
-        hashed = self.prefix.extend_match(blocks, prompt)
+        hashed = self.prefix.extend_match(blocks, prompt, spans)
         return blocks, hashed
     def generation(self): return self.prefix.generation
     # sequences
@@ -104,8 +104,9 @@ class OracleStack:
     def end(self, s): return self.call(self.sequences.end, s)
     def restore(self, s, b): return self.call(self.sequences.restore, s, b)
     def ensure(self, s, n): return self.call(self.sequences.ensure_tokens, s, n)
-    def publish(self, s, tokens, committed):
-        return self.call(self.sequences.publish, s, tokens, committed)
+    def publish(self, s, tokens, committed, spans=()):
+        return self.call(self.sequences.publish, s, tokens, committed, spans)
+    def truncate(self, s, tokens): return self.call(self.sequences.truncate, s, tokens)
     def view(self, s):
         q = self.sequences.sequences[s]
         return {"pages": list(q.pages), "revision": q.revision, "first_changed": q.first_changed,
@@ -154,14 +155,15 @@ class ProductStack:
     def touch(self, b): return self._status(self.prefix.touch, b)
     def candidate(self, after=0): return self.prefix.eviction_candidate(after)
     def erase(self, b): return self._status(self.prefix.erase, b)
-    def match(self, prompt): return self.prefix.match(prompt)
+    def match(self, prompt, spans=()): return self.prefix.match(prompt, spans)
     def generation(self): return self.prefix.generation()
     def begin(self, s): return self._status(self.sequences.begin, s)
     def end(self, s): return self._status(self.sequences.end, s)
     def restore(self, s, b): return self._status(self.sequences.restore, s, b)
     def ensure(self, s, n): return self._status(self.sequences.ensure_tokens, s, n)
-    def publish(self, s, tokens, committed):
-        return self._status(self.sequences.publish, s, tokens, committed)
+    def publish(self, s, tokens, committed, spans=()):
+        return self._status(self.sequences.publish, s, tokens, committed, spans)
+    def truncate(self, s, tokens): return self.call(self.sequences.truncate, s, tokens)
     def view(self, s): return self.sequences.view(s)
     def compact(self):
         moves = self.sequences.compact_extent()
@@ -310,12 +312,97 @@ def test_publish_dedups_to_the_canonical_page(Stack):
     assert s.candidate(0) == two["blocks"][2]          # only the chain's leaf is evictable
 
 
+@pytest.mark.parametrize("Stack", STACKS)
+def test_images_keep_equal_placeholder_tokens_apart(Stack):
+    """Cache::publishCommittedBlocks and Cache::extendMatch key every block with the identity of
+    the images that overlap it (runtime/engine/cache/Cache.cpp:186-193, :310-318): two prompts
+    with the same placeholder tokens and different images neither match nor share a page, the
+    same image does both, and blocks before the image are shared whatever the image is."""
+    s = Stack(24, extent_pages=4)
+    prompt = [3] * 40 + [9] * 50 + [5] * 20            # an image of 50 placeholder tokens at 40
+    cat = [(40, 50, 5, 10, 0x1111, 0x2222)]
+    dog = [(40, 50, 5, 10, 0x3333, 0x4444)]
+    ok(s.begin(1))
+    ok(s.ensure(1, len(prompt)))
+    ok(s.publish(1, prompt, 96, cat))
+    one = s.view(1)
+    assert len(one["blocks"]) == 3
+    # the same tokens under another image: the text-only first page is shared, the rest is not
+    ok(s.begin(2))
+    ok(s.ensure(2, len(prompt)))
+    own = s.view(2)["pages"]
+    ok(s.publish(2, prompt, 96, dog))
+    two = s.view(2)
+    assert two["pages"][0] == one["pages"][0] and two["blocks"][0] == one["blocks"][0]
+    assert two["pages"][1:3] == own[1:3] and not set(two["blocks"][1:]) & set(one["blocks"][1:])
+    # the same image again: everything is found and deduplicated
+    ok(s.begin(3))
+    ok(s.ensure(3, len(prompt)))
+    ok(s.publish(3, prompt, 96, cat))
+    three = s.view(3)
+    assert three["pages"][:3] == one["pages"][:3] and three["blocks"] == one["blocks"]
+    assert s.match(prompt, cat) == (one["blocks"], 3)
+    assert s.match(prompt, dog) == (two["blocks"], 3)
+    # without its images the prompt matches the text page only, and publishing it as text
+    # makes blocks of its own for the placeholder pages
+    assert s.match(prompt) == (one["blocks"][:1], 2)
+    assert s.match(prompt, [(40, 50, 5, 10, 0x1111, 0x2223)]) == (one["blocks"][:1], 2)
+    assert s.match(prompt, [(41, 50, 5, 10, 0x1111, 0x2222)]) == (one["blocks"][:1], 2)
+    ok(s.begin(4))
+    ok(s.ensure(4, len(prompt)))
+    ok(s.publish(4, prompt, 96))
+    four = s.view(4)
+    assert four["blocks"][0] == one["blocks"][0]
+    assert not set(four["blocks"][1:]) & (set(one["blocks"]) | set(two["blocks"]))
+
+
+@pytest.mark.parametrize("Stack", STACKS)
+def test_truncate_gives_emptied_pages_back(Stack):
+    """After a speculative rollback the pages past the kept tokens go back to the pool; the
+    published pages and the pages of the kept tokens stay; the next growth takes pages again."""
+    s = Stack(16, extent_pages=4)
+    tokens = [11 * i % 997 for i in range(200)]
+    ok(s.begin(1))
+    ok(s.ensure(1, 70 + 16))                       # 70 committed tokens and a tree of 16 rows
+    before = s.view(1)
+    assert len(before["pages"]) == 3
+    ok(s.publish(1, tokens, 70))
+    counts = s.pool_counts()
+    assert ok(s.truncate(1, 70 + 16)) == 0 and s.view(1) == s.view(1)   # nothing past the kept tokens
+    assert ok(s.truncate(1, 300)) == 0
+    assert s.view(1)["revision"] == before["revision"]
+    assert ok(s.truncate(1, 64)) == 1              # the third page held no kept token
+    after = s.view(1)
+    assert after["pages"] == before["pages"][:2] and after["blocks"] == s.view(1)["blocks"]
+    assert after["revision"] == before["revision"] + 1 and after["first_changed"] == 2
+    assert s.pool_counts()[2] == counts[2] - 1 and s.pool_counts()[1] == counts[1] + 1
+    assert ok(s.truncate(1, 63)) == 0              # still two pages
+    assert s.truncate(1, 32)[0] == "state"         # the second page is published
+    assert s.truncate(9, 10)[0] == "range"
+    ok(s.ensure(1, 100))                           # growth takes pages again, from the changed end
+    grown = s.view(1)
+    assert grown["pages"][:2] == after["pages"] and len(grown["pages"]) == 4
+    assert grown["first_changed"] == 2
+    # a page another sequence holds too only loses this sequence's reference
+    ok(s.begin(2))
+    ok(s.restore(2, after["blocks"][1]))
+    ok(s.ensure(2, 96))
+    ok(s.end(1))
+    held = s.pool_counts()
+    assert ok(s.truncate(2, 64)) == 1
+    assert s.pool_counts()[2] == held[2] - 1
+    assert s.view(2)["pages"] == after["pages"]
+    ok(s.end(2))
+
+
 def test_random_walk_in_lockstep():
     rng = random.Random(20261125)
     o, p = OracleStack(24, extent_pages=4, runway=8), ProductStack(24, extent_pages=4, runway=8)
     vocab = [rng.randrange(50) for _ in range(4)]
     streams = {}          # sequence -> (tokens, committed)
+    images = {}           # sequence -> its prompt's image spans
     next_sequence = 1
+    digests = [(0xA1, 0xB1), (0xA2, 0xB2)]
 
     def both(name, *args):
         a, b = getattr(o, name)(*args), getattr(p, name)(*args)
@@ -334,7 +421,13 @@ def test_random_walk_in_lockstep():
                 tokens += [rng.choice(vocab)] * 32
             tokens += [rng.randrange(50) for _ in range(rng.randrange(1, 32))]
             streams[sequence] = [tokens, 0]
-            blocks, _ = both("match", tokens)
+            # a third of the prompts carry an image over some of their tokens
+            images[sequence] = ()
+            if rng.random() < 0.33 and len(tokens) > 40:
+                offset = rng.randrange(0, len(tokens) - 8)
+                images[sequence] = ((offset, rng.randrange(4, len(tokens) - offset), 2, 2) +
+                                    rng.choice(digests),)
+            blocks, _ = both("match", tokens, images[sequence])
             if blocks and rng.random() < 0.7:
                 assert both("restore", sequence, blocks[-1])[0] == "ok"
                 streams[sequence][1] = len(blocks) * 32
@@ -342,10 +435,13 @@ def test_random_walk_in_lockstep():
             sequence = rng.choice(live)
             tokens, committed = streams[sequence]
             target = min(len(tokens), committed + rng.randrange(1, 48))
-            kind, _ = both("ensure", sequence, target)
+            # room for a tree of draft rows past the target, given back after the step
+            kind, _ = both("ensure", sequence, target + rng.choice((0, 16)))
             if kind == "ok":
-                assert both("publish", sequence, tokens, target)[0] == "ok"
+                assert both("publish", sequence, tokens, target, images[sequence])[0] == "ok"
                 streams[sequence][1] = target
+                if rng.random() < 0.5:
+                    assert both("truncate", sequence, target)[0] == "ok"
         elif op < 0.70 and live:
             sequence = rng.choice(live)
             assert both("end", sequence)[0] == "ok"

@@ -59,7 +59,7 @@ def steps(a_bits, b_bits):
     return np.abs(key(a_bits) - key(b_bits))
 
 
-SHAPES = [(4, 6, 256, 32, True), (2, 8, 128, 64, False), (8, 4, 64, 32, False)]
+SHAPES = [(4, 6, 256, 32, True), (2, 8, 128, 64, False), (8, 4, 64, 32, False), (4, 1, 128, 32, True)]
 
 
 # ------------------------------------------------------------- the oracle ----
@@ -249,6 +249,16 @@ def test_long_chunk_of_a_narrower_head():
 @pytest.mark.parametrize("heads,group,dim,pairs,norm", [(2, 8, 128, 64, 0), (8, 4, 64, 32, 2)])
 def test_other_head_dimensions(fmt, heads, group, dim, pairs, norm):
     fused_case(fmt, heads, group, dim, pairs, False, norm, [100, 31], [8, 3], 8, 32, seed=207,
+               verify_max_rows=15)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fmt", [ko.INT4, ko.BF16])
+@pytest.mark.parametrize("dim,pairs,gate", [(128, 32, True), (256, 32, False)])
+def test_one_query_head_per_kv_head(fmt, dim, pairs, gate):
+    """A group of one: every query head is its own KV head (the reciprocal that stands for
+    the division by the group does not fit 32 bits there)."""
+    fused_case(fmt, 4, 1, dim, pairs, gate, 1, [100, 31, 0], [8, 3, 5], 8, 32, seed=209,
                verify_max_rows=15)
 
 

@@ -59,6 +59,29 @@ def test_static_workspace_decode_is_the_workspace_decode():
     # the second call in a row is smaller: what the first left in the array must not show
     both(2, 3)
     both(5, 1)
+    # under stream capture: the address of the array was looked up when the storage was made,
+    # so the call records kernel launches only; every replay, with eager work and
+    # synchronisations of the program's own between them, gives the eager rows
+    assert kvx.lib().kvx_static_workspace_prime(tw.dev.h) == 0
+    eager = torch.full((lanes, H, 1, G, D), 0x5A5A, dtype=torch.int16, device="cuda")
+    kvx.attend_decode_static(tw.dev, 1, QH, q, eager, dts, dp, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(eager, whole)
+    captured = torch.full_like(eager, 0x5A5A)
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            kvx.attend_decode_static(tw.dev, 1, QH, q, captured, dts, dp, 1,
+                                     stream=torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(3):
+        captured.fill_(0x5A5A)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, whole), f"replay {replay} of the captured call differs"
+        both(replay, 2)                      # eager calls over the same array in between
+    del graph
     # more partial rows than the array holds: refused, nothing enqueued
     huge = [kvx.VerifyParams(committed[3], counts[3], kvx.KvLayer(), 512, 512, 1, 1, 0.0)] * 32
     assert kvx.attend_workspace_bytes(tw.dev, huge, QH) > 32 << 20      # KVX_STATIC_WORKSPACE_BYTES
