@@ -318,9 +318,21 @@ def tree_verify(args):
     extent_pages = L.kvx_layout_largest_extent_pages(C.byref(layout))
     extents = -(-lanes * n_pages // extent_pages)
     storage = kvx.Storage(LAYERS, H, D, fmt, extents * extent_pages, extent_pages, aligned=True)
-    storage.allocate_all()
-    ids = rng.permutation(extents * extent_pages)[:lanes * n_pages].astype(np.uint32)
-    tables = [storage.table(ids[i * n_pages:(i + 1) * n_pages]) for i in range(lanes)]
+    # The pages belong to the pool and reach the sequences through their records, as in an
+    # engine: everything is acquired once and given back in a seed-shuffled order, so the
+    # sequences' pages come off the free stacks scattered over the extents.
+    pool = kvx.Pool(storage, storage.page_count)
+    prefix_cache = kvx.Prefix(pool)
+    sequences = kvx.Sequences(pool, prefix_cache)
+    for page in rng.permutation(pool.acquire(min(storage.page_count, lanes * n_pages + 64))):
+        pool.release(int(page))
+    tables, revisions = [], []
+    for lane in range(lanes):
+        sequences.begin(lane + 1)
+        sequences.ensure_tokens(lane + 1, context + nodes)
+        view = sequences.view(lane + 1)
+        tables.append(storage.table(np.array(view["pages"], dtype=np.uint32)))
+        revisions.append(view["revision"])
     gen = torch.Generator(device="cuda")
     gen.manual_seed(args.seed)
     for lane in range(lanes):
@@ -364,11 +376,26 @@ def tree_verify(args):
                             device="cuda")
     torch.cuda.synchronize()
 
+    released = [0]
+
     def step():
+        for lane in range(lanes):
+            # room for the step's draft rows; a page list that changed is written out again
+            sequences.ensure_tokens(lane + 1, context + nodes)
+            view = sequences.view(lane + 1)
+            if view["revision"] != revisions[lane]:
+                tables[lane] = storage.table(np.array(view["pages"], dtype=np.uint32))
+                revisions[lane] = view["revision"]
         for layer in range(LAYERS):
             kvx.append(storage, layer, chunk_k, chunk_v, tables, cp, H * 32 * D, verify_max_rows=16)
             kvx.attend_verify(storage, layer, QH, queries, output, tables, vp, masks_d, 32, workspace)
         kvx.compact_path(storage, 0xFFFFFFFF, tables, cp, paths_d, counts_d, 16)
+        for lane in range(lanes):
+            # the rollback's host side: pages that hold rejected rows only go back to the pool
+            # (none at this context, whose draft rows share a page with the accepted ones;
+            # the history itself stays where it is, so every step sees the same lanes)
+            released[0] += sequences.truncate(lane + 1, context + int(counts[lane]))
+            revisions[lane] = sequences.view(lane + 1)["revision"] if released[0] else revisions[lane]
 
     for _ in range(args.warmup):
         step()
@@ -407,10 +434,17 @@ def tree_verify(args):
                                "contexts 65536, 16-node trees (branching <= 3), 16 layers: append 16 "
                                "rows + masked verify per layer, then path compaction over all layers",
                    "batch": lanes, "layers": LAYERS, "format": args.format,
-                   "splits_per_sequence": int(splits), "seed": args.seed},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": None,
+                   "splits_per_sequence": int(splits), "seed": args.seed,
+                   "pages_released_by_rollbacks": released[0]},
+        # Verify of 16 rows is a bandwidth-bound path by its bytes (each page is read once for
+        # 96 fused rows); what holds the kernel is the work per page of its matrix and vector
+        # units, so the MFMA figures stand beside the HBM ones.
+        "roofline": {"bound": "hbm", "achieved": round(kv_bytes / (kernel_ms * 1e-3) / 1e9, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(kv_bytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "bytes_per_launch": kv_bytes,
+                     "mfma_tflops": round(achieved, 1), "mfma_peak_tflops": MFMA_BF16_PEAK_TFLOPS,
+                     "mfma_frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
                      "kernel": ("verify48_int4_kernel (split kernel of verify attention, 48 fused rows per wave)"
                                 if args.format == "int4" else
                                 "group_wide_kernel (split kernel of verify attention, four waves of 24 fused "
@@ -419,6 +453,11 @@ def tree_verify(args):
                      "kv_gbs": round(kv_bytes / (kernel_ms * 1e-3) / 1e9, 1)},
         "cpu_baseline": None,
     }
+    for lane in range(lanes):
+        sequences.end(lane + 1)
+    sequences.close()
+    prefix_cache.close()
+    pool.close()
     storage.close()
     if args.cpu_seconds > 0 and args.format == "int4":
         result["cpu_baseline"] = cpu_tree_verify(args.seed, context, nodes, masks, args.cpu_seconds)
@@ -598,11 +637,14 @@ def shared_prefix(args):
         "config": {"workload": "kv_attend_decode_shared: 16 sequences, 938 shared pages, 64..1024 own "
                                "tokens each, 4 KV heads x 256, 24 query heads, one layer per call",
                    "format": args.format, "prefix_splits": int(prefix_splits), "seed": args.seed},
-        "roofline": {"bound": "mfma", "achieved": round(4 * D * QH * sum(c + 1 for c in committed) /
-                                                        (shared_ms * 1e-3) / 1e12, 1),
-                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(4 * D * QH * sum(c + 1 for c in committed) / (shared_ms * 1e-3) / 1e12 /
-                                   MFMA_BF16_PEAK_TFLOPS, 4),
+        # Decode is bandwidth-bound: the bytes the entry has to read are the shared pages once
+        # and every sequence's own pages (`physical`), over the time of the whole call.
+        "roofline": {"bound": "hbm", "achieved": round(physical / (shared_ms * 1e-3) / 1e9, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(physical / (shared_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "bytes_per_launch": physical,
+                     "mfma_tflops": round(4 * D * QH * sum(c + 1 for c in committed) /
+                                          (shared_ms * 1e-3) / 1e12, 1),
                      "traffic": None, "kernel": "split kernels over the shared pages (stacked rows) and over the "
                                                 "sequences' own pages + shared_merge_kernel",
                      "ms_per_launch": round(shared_ms, 4)},

@@ -372,22 +372,44 @@ def test_config4_copy_on_write_of_the_partial_last_page(fmt):
     tw.close()
 
 
-def test_config5_int4_tree_verify_and_rollback():
-    # int4, batch 4, context 65536, a 16-row tree per sequence: append the rows,
-    # masked verify, a root-to-leaf path per sequence, compaction; the page bytes
-    # after the rollback must be the oracle's, bit for bit
-    lanes, committed, nodes = 4, 65536, 16
-    n_pages = (committed + nodes + 31) // 32
-    tw = Gp.Twin(ko.INT4, H, D, 1, lanes * n_pages, one_extent=True)
-    ids = np.random.default_rng(8).permutation(lanes * n_pages).astype(np.uint32)
+@pytest.mark.parametrize("rule", ["reference", "plan"])
+def test_config5_int4_tree_verify_and_rollback(rule):
+    """int4, batch 4, contexts of 65 536 tokens (two a little further, so that their 16 draft
+    rows run over a page boundary), a 16-row tree per sequence: append the rows, masked verify
+    under the reference's split rule and under kvx_verify_plan (what bench.py and the
+    integration notes use), a root-to-leaf path per sequence, compaction; the page bytes after
+    the rollback must be the oracle's, bit for bit.  The pages come from the pool through the
+    sequence records: after the rollback kvx_sequence_truncate gives the page that holds only
+    rejected rows back, the pool's counts and the page lists say so, and the next step's rows
+    land in the slots behind the accepted ones."""
+    lanes, nodes = 4, 16
+    committed = [65536, 65560, 65556, 65536]
+    n_pages = [(c + nodes + 31) // 32 for c in committed]
+    tw = Gp.Twin(ko.INT4, H, D, 1, sum(n_pages) + 8, one_extent=True)
+    tw.dev.release(0)                      # the pool allocates the device extent itself
+    pool = kvx.Pool(tw.dev, tw.dev.page_count)
+    cache = kvx.Prefix(pool)
+    seqs = kvx.Sequences(pool, cache)
+    # page ids in a seed-shuffled order: everything acquired once and given back shuffled,
+    # so that the sequences' pages come off the free stacks scattered over the extent
+    every = pool.acquire(sum(n_pages) + 4)
+    for page in np.random.default_rng(8).permutation(every):
+        pool.release(int(page))
+    assert pool.snapshot().pages_active == 0
     gen = torch.Generator(device="cuda")
     gen.manual_seed(8)
     hts, dts = [], []
     for lane in range(lanes):
-        th, td = tw.tables(ids[lane * n_pages:(lane + 1) * n_pages])
+        seqs.begin(lane + 1)
+        seqs.ensure_tokens(lane + 1, committed[lane] + nodes)
+        pages = np.array(seqs.view(lane + 1)["pages"], dtype=np.uint32)
+        assert len(pages) == n_pages[lane] and len(set(np.diff(pages.astype(np.int64)))) > 100
+        th, td = tw.tables(pages)
         hts.append(th)
         dts.append(td)
-        device_history(tw, 0, td, n_pages, 0, committed, gen)
+        device_history(tw, 0, td, n_pages[lane], 0, committed[lane], gen)
+    held = pool.snapshot().pages_active
+    assert held == sum(n_pages)
     tw.download()
     rng = np.random.default_rng(9)
     none = 0xFFFFFFFF
@@ -409,34 +431,41 @@ def test_config5_int4_tree_verify_and_rollback():
     cv = np.zeros((lanes, H, D, 32), dtype=np.uint16)
     for lane in range(lanes):
         ck[lane], cv[lane] = T.chunk_buffers(k[lane], v[lane], 32)
-    dparams = [kvx.ChunkParams(committed, nodes, 32, n_pages) for _ in range(lanes)]
+    dparams = [kvx.ChunkParams(committed[i], nodes, 32, n_pages[i]) for i in range(lanes)]
     kvx.append(tw.dev, 0, Gp.dev(ck), Gp.dev(cv), dts, dparams, H * 32 * D, verify_max_rows=16)
-    hparams = [ko.ChunkParams(committed, nodes, 32, n_pages, tw.host.layer(0)) for _ in range(lanes)]
+    hparams = [ko.ChunkParams(committed[i], nodes, 32, n_pages[i], tw.host.layer(0)) for i in range(lanes)]
     assert ko.store_verify(ko.INT4, H, D, ck, cv, hts, hparams, max_rows=16) == lanes
     # masked verify on the device; the oracle on one lane, two heads
     q = np.zeros((lanes, H, 32, G, D), dtype=np.uint16)
     q[:, :, :nodes] = bf16_rows((lanes, H, nodes, G, D), 10)
-    splits = [kvx.lib().kvx_verify_splits(committed, nodes)] * lanes
-    dp = [kvx.VerifyParams(committed, n_pages, kvx.KvLayer(), splits[i], 128, nodes, 16, 0.0)
+    if rule == "reference":
+        splits = [kvx.lib().kvx_verify_splits(c, nodes) for c in committed]
+        assert splits == [128] * lanes
+    else:
+        splits = kvx.verify_plan(committed, nodes, H, QH)
+        # two waves of 48 fused rows per split and KV head, one round of the 1024 SIMDs
+        assert splits == [32] * lanes and sum(splits) * H * 2 <= 1024
+    dp = [kvx.VerifyParams(committed[i], n_pages[i], kvx.KvLayer(), splits[i], 128, nodes, 16, 0.0)
           for i in range(lanes)]
     out = torch.zeros((lanes, H, 32, G, D), dtype=torch.int16, device="cuda")
     ws = torch.empty(kvx.attend_workspace_bytes(tw.dev, dp, QH) + 256, dtype=torch.uint8, device="cuda")
     kvx.attend_verify(tw.dev, 0, QH, Gp.dev(q), out, dts, dp, Gp.dev(masks), 32, ws)
     torch.cuda.synchronize()
     got = Gp.host_u16(out)
-    lane = 2
-    for head in (0, 3):
-        tile_q = q[lane, head, :16].reshape(16 * G, D)
-        want, want32 = Gp.oracle_tile(ko.INT4, H, G, D, tile_q, hts[lane], tw.host.layer(0), head,
-                                      committed, nodes, splits[lane], 16, masks=masks[lane])
-        mine = got[lane, head, :16].reshape(16 * G, D)
-        Gp.check_attention(
-            mine, want, want32, np.ones(16 * G, dtype=bool), tol(ko.INT4),
-            f"config 5 lane {lane} head {head}",
-            explain=lambda index: dict(fmt=ko.INT4, kv_heads=H, group=G, head_dim=D, tile_queries=tile_q,
-                                       table=hts[lane], kv=tw.host.layer(0), head=head,
-                                       committed=committed, active=nodes, splits=splits[lane],
-                                       capacity=16, fused_row=index[0], masks=masks[lane]))
+    for lane, heads in ((2, (0, 3)), (1, (2,))):
+        for head in heads:
+            tile_q = q[lane, head, :16].reshape(16 * G, D)
+            want, want32 = Gp.oracle_tile(ko.INT4, H, G, D, tile_q, hts[lane], tw.host.layer(0), head,
+                                          committed[lane], nodes, splits[lane], 16, masks=masks[lane])
+            mine = got[lane, head, :16].reshape(16 * G, D)
+            Gp.check_attention(
+                mine, want, want32, np.ones(16 * G, dtype=bool), tol(ko.INT4),
+                f"config 5 ({rule} splits) lane {lane} head {head}",
+                explain=lambda index: dict(fmt=ko.INT4, kv_heads=H, group=G, head_dim=D,
+                                           tile_queries=tile_q, table=hts[lane], kv=tw.host.layer(0),
+                                           head=head, committed=committed[lane], active=nodes,
+                                           splits=splits[lane], capacity=16, fused_row=index[0],
+                                           masks=masks[lane]))
     # a tree that is a path must see exactly what the chain sees
     chain_masks = np.zeros((lanes, nodes), dtype=np.uint32)
     chain_masks[:] = kvx.tree_masks([none] + list(range(nodes - 1)))
@@ -464,4 +493,47 @@ def test_config5_int4_tree_verify_and_rollback():
     torch.cuda.synchronize()
     assert ko.compact_tree(ko.INT4, H, D, hts, hparams, paths, counts, 16) > 0   # rows moved
     tw.assert_same_bytes()
+    # the rollback frees what it emptied: the host's committed count moves on by the accepted
+    # rows, and a page none of them reached goes back to the pool
+    after = [committed[i] + int(counts[i]) for i in range(lanes)]
+    emptied = [n_pages[i] - (after[i] + 31) // 32 for i in range(lanes)]
+    assert sum(emptied) >= 1 and emptied[0] == 0 and emptied[3] == 0   # page-aligned lanes keep theirs
+    for i in range(lanes):
+        before = seqs.view(i + 1)
+        assert seqs.truncate(i + 1, after[i]) == emptied[i]
+        view = seqs.view(i + 1)
+        assert view["pages"] == before["pages"][:n_pages[i] - emptied[i]]
+        if emptied[i]:
+            dropped = before["pages"][-1]
+            assert not pool.page_active(dropped)
+            assert view["revision"] == before["revision"] + 1
+            assert view["first_changed"] == len(view["pages"])
+    assert pool.snapshot().pages_active == held - sum(emptied)
+    # the next step: room for another tree, its rows stored behind the accepted ones
+    k2 = rng.standard_normal((lanes, H, nodes, D)).astype(np.float32)
+    v2 = rng.standard_normal((lanes, H, nodes, D)).astype(np.float32)
+    for lane in range(lanes):
+        ck[lane], cv[lane] = T.chunk_buffers(k2[lane], v2[lane], 32)
+    hts2, dts2, next_pages = [], [], []
+    for lane in range(lanes):
+        seqs.ensure_tokens(lane + 1, after[lane] + nodes)
+        pages = np.array(seqs.view(lane + 1)["pages"], dtype=np.uint32)
+        next_pages.append(len(pages))
+        assert len(pages) == (after[lane] + nodes + 31) // 32
+        th, td = tw.tables(pages)
+        hts2.append(th)
+        dts2.append(td)
+    assert pool.snapshot().pages_active == sum(next_pages)
+    dparams2 = [kvx.ChunkParams(after[i], nodes, 32, next_pages[i]) for i in range(lanes)]
+    kvx.append(tw.dev, 0, Gp.dev(ck), Gp.dev(cv), dts2, dparams2, H * 32 * D, verify_max_rows=16)
+    torch.cuda.synchronize()
+    hparams2 = [ko.ChunkParams(after[i], nodes, 32, next_pages[i], tw.host.layer(0)) for i in range(lanes)]
+    assert ko.store_verify(ko.INT4, H, D, ck, cv, hts2, hparams2, max_rows=16) == lanes
+    tw.assert_same_bytes()
+    for lane in range(lanes):
+        seqs.end(lane + 1)
+    assert pool.snapshot().pages_active == 0
+    seqs.close()
+    cache.close()
+    pool.close()
     tw.close()
