@@ -51,7 +51,7 @@ def parse():
                     help="KV pool size; 0 = 80%% of free HBM, at most 256 GB")
     ap.add_argument("--contiguous", action="store_true",
                     help="hand out pages in order instead of shuffled (TLB comparison)")
-    ap.add_argument("--cpu-seconds", type=float, default=15.0,
+    ap.add_argument("--cpu-seconds", type=float, default=30.0,
                     help="CPU oracle budget; 0 skips the CPU baseline")
     ap.add_argument("--kernel-iters", type=int, default=20)
     ap.add_argument("--uniform-context", type=int, default=0,
@@ -79,11 +79,14 @@ def parse():
                          "current stream); a sequence's layers stay in order on its stream")
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
-    ap.add_argument("--workload", choices=["decode", "decode-single", "tree-verify", "prefill", "qkv-prepare", "shared-prefix"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "decode-single", "tree-verify", "prefill", "qkv-prepare", "shared-prefix",
+                                           "stream-ceiling"], default="decode",
                     help="decode = batch-32 mixed-length int4 decode, the headline metric (default); "
                          "decode-single = one sequence of 32768 tokens, the 16 per-layer calls replayed "
                          "as one HIP graph; tree-verify = 16-node tree verify and prefill = chunked prefill with a shared "
-                         "prefix, the matrix-core paths (profiling)")
+                         "prefix, the matrix-core paths (profiling); stream-ceiling = what the memory system "
+                         "delivers for the headline batch's bytes under request shapes other than the "
+                         "decode kernel's (linear, 16-byte coalesced, page order, pool size)")
     ap.add_argument("--format", choices=["bf16", "fp8", "int8", "int4"], default=None,
                     help="page format of the prefill workload (default bf16) and of the shared-prefix "
                          "and tree-verify workloads (default int4; no fp8)")
@@ -93,9 +96,16 @@ def parse():
     return args
 
 
-def cpu_lane(ctx, seed):
-    """One sequence on the oracle: history filled untimed, then the timed decode
-    step of one layer (append one token, attend).  Returns seconds."""
+def host_cpus():
+    """What the CPU figures ran on: the machine's processors, those this process may use, and
+    the threads the all-core legs start at most (a one-GPU box's share of its host)."""
+    return {"host_cpus": os.cpu_count(), "affinity_cpus": len(os.sched_getaffinity(0)),
+            "threads_cap": 16}
+
+
+def cpu_lane_prepare(ctx, seed):
+    """One sequence on the oracle: fills the history (untimed) and returns run(), the decode
+    step of one layer (append one token, attend), which returns its seconds."""
     import numpy as np
     from oracle import kvoracle as ko
 
@@ -117,23 +127,37 @@ def cpu_lane(ctx, seed):
     q = np.zeros((1, H, 32, G, D), dtype=np.uint16)
     q[0, :, 0] = ko.f32_to_bf16(rng.standard_normal((H, G, D)).astype(np.float32)).reshape(H, G, D)
     splits = min(max(1, ((ctx + 1 + 31) // 32 + 31) // 32), 128)
-    t0 = time.perf_counter()
-    ko.store_chunk(ko.INT4, H, D, k, v, table, ko.ChunkParams(ctx, 1, 32, n_pages, store.layer(0)))
-    ko.attend_verify(ko.INT4, H, G, D, q, [table],
-                     [ko.VerifyParams(ctx, n_pages, store.layer(0), splits, 128, 1, 1, 0.0)],
-                     want_f32=False)
-    spent = time.perf_counter() - t0
-    store.close()
+
+    def run():
+        t0 = time.perf_counter()
+        ko.store_chunk(ko.INT4, H, D, k, v, table, ko.ChunkParams(ctx, 1, 32, n_pages, store.layer(0)))
+        ko.attend_verify(ko.INT4, H, G, D, q, [table],
+                         [ko.VerifyParams(ctx, n_pages, store.layer(0), splits, 128, 1, 1, 0.0)],
+                         want_f32=False)
+        return time.perf_counter() - t0
+
+    run.close = store.close
+    return run
+
+
+def cpu_lane(ctx, seed):
+    """History filled untimed, then the timed decode step of one layer.  Returns seconds."""
+    run = cpu_lane_prepare(ctx, seed)
+    spent = run()
+    run.close()
     return spent
 
 
 def cpu_baseline(contexts, seed, budget_s):
-    """The oracle (scalar C++ port) on a bounded sample of the same workload:
-    whole sequences of the batch, shortest first, one layer each (append one
-    token, then decode attention).  First on one thread, then the same sequences
-    spread over the host's cores, one sequence per thread (the oracle's calls
-    release the interpreter lock)."""
+    """The oracle (scalar C++ port) on a bounded sample of the same workload: whole sequences
+    of the batch, shortest first, one layer each (append one token, then decode attention).
+    First on one thread; then the same sequences on the host's cores, one sequence per thread
+    (the oracle's calls release the interpreter lock), all histories filled first and the
+    decode steps started together, timed by the wall clock from the common start to the last
+    thread's end.  One layer of the whole batch would take the sample's time times
+    `layer_over_sample`: the work is linear in the tokens."""
     import concurrent.futures
+    import threading
     import numpy as np
 
     order = [int(i) for i in np.argsort(contexts)]  # shortest first so the sample stays bounded
@@ -141,23 +165,52 @@ def cpu_baseline(contexts, seed, budget_s):
     for lane in order:
         ctx = int(contexts[lane])
         tokens = sum(int(contexts[i]) + 1 for i in sample)
-        if spent > 0 and spent + spent / max(tokens, 1) * ctx > budget_s / 2:
+        if spent > 0 and spent + spent / max(tokens, 1) * ctx > 0.8 * budget_s:
             break
         spent += cpu_lane(ctx, seed + lane)
         sample.append(lane)
     tokens = sum(int(contexts[i]) + 1 for i in sample)
     nbytes = tokens * BYTES_PER_TOKEN_LAYER
-    cores = max(1, min(16, len(os.sched_getaffinity(0)), len(sample)))
+    layer_tokens = sum(int(c) + 1 for c in contexts)
+    host = host_cpus()
+    cores = max(1, min(host["threads_cap"], host["affinity_cpus"], len(sample)))
+    # longest first, so that the threads' shares come out even
+    runs = [cpu_lane_prepare(int(contexts[lane]), seed + lane) for lane in sample[::-1]]
+    start = threading.Barrier(cores + 1)
+    queue, lock = list(runs), threading.Lock()
+
+    def worker():
+        start.wait()
+        while True:
+            with lock:
+                if not queue:
+                    return
+                run = queue.pop(0)
+            run()
+
     with concurrent.futures.ThreadPoolExecutor(cores) as pool:
-        busy = sum(pool.map(lambda lane: cpu_lane(int(contexts[lane]), seed + lane), sample[::-1]))
+        futures = [pool.submit(worker) for _ in range(cores)]
+        start.wait()
+        t0 = time.perf_counter()
+        for f in futures:
+            f.result()
+        wall = time.perf_counter() - t0
+    for run in runs:
+        run.close()
     return {
         "value": nbytes / spent / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-        "sample": f"{len(sample)} shortest sequences of the batch ({tokens} tokens), one layer: "
-                  f"append 1 token + decode attention each, {spent:.1f} s of scalar C++ oracle",
+        "sample": f"{len(sample)} shortest sequences of the batch of {len(contexts)} ({tokens} of the "
+                  f"layer's {layer_tokens} tokens), one layer: append 1 token + decode attention each, "
+                  f"{spent:.1f} s of scalar C++ oracle",
+        "layer_over_sample": round(layer_tokens / tokens, 2),
+        "one_layer_of_the_batch_s": round(spent * layer_tokens / tokens, 1),
         "decode_tokens_per_s_one_layer": len(sample) / spent,
-        "all_cores": {"cores": cores, "value": nbytes / (busy / cores) / 1e9, "unit": "GB/s",
-                      "note": "same sequences, one per thread; rate = bytes / (summed attention "
-                              "seconds / threads), history fills excluded"},
+        **host,
+        "all_cores": {"cores": cores, "value": nbytes / wall / 1e9, "unit": "GB/s",
+                      "wall_s": round(wall, 2),
+                      "one_layer_of_the_batch_s": round(wall * layer_tokens / tokens, 1),
+                      "note": "same sequences over the threads, longest first; wall clock from the "
+                              "threads' common start to the last one's end, history fills before it"},
     }
 
 
@@ -207,7 +260,7 @@ def cpu_tree_verify(seed, context, nodes, masks, budget_s):
     store.close()
     assert stored == 1 and attended == 1, "the oracle refused the tree-verify sample"
     full = spent * (context + nodes) / (history + nodes) * LAYERS  # one sequence, all layers, full history
-    return {"value": nodes / full, "unit": "draft tokens/s", "cores": 1, "kind": "port",
+    return {"value": nodes / full, "unit": "draft tokens/s", "cores": 1, "kind": "port", **host_cpus(),
             "sample": f"one sequence of the batch, one layer, history cut to {history} of {context} tokens: "
                       f"append {nodes} tree rows + masked verify, {spent:.1f} s of scalar C++ oracle; "
                       f"scaled linearly to the full history and {LAYERS} layers",
@@ -239,7 +292,7 @@ def cpu_prefill(seed, fmt_name, prefix, chunk, budget_s):
     spent = time.perf_counter() - t0
     store.close()
     assert stored == 1 and attended == 1, "the oracle refused the prefill sample"
-    return {"value": rows / (spent * LAYERS), "unit": "tokens/s", "cores": 1, "kind": "port",
+    return {"value": rows / (spent * LAYERS), "unit": "tokens/s", "cores": 1, "kind": "port", **host_cpus(),
             "sample": f"one sequence, one layer, the first {rows} rows of a {chunk}-row chunk over the "
                       f"{prefix}-token prefix: append + causal attention, {spent:.1f} s of scalar C++ "
                       f"oracle; rate = rows / (seconds x {LAYERS} layers)",
@@ -270,7 +323,7 @@ def cpu_qkv_prepare(seed, budget_s):
     spent = time.perf_counter() - t0
     store.close()
     assert stored == 1, "the oracle refused the qkv-prepare sample"
-    return {"value": rows / spent, "unit": "tokens/s", "cores": 1, "kind": "port",
+    return {"value": rows / spent, "unit": "tokens/s", "cores": 1, "kind": "port", **host_cpus(),
             "sample": f"the whole {rows}-row chunk, one layer: prepare + quantize + store, "
                       f"{spent:.2f} s of scalar C++ oracle",
             "seconds": spent, "rows": rows}
@@ -461,6 +514,113 @@ def tree_verify(args):
     storage.close()
     if args.cpu_seconds > 0 and args.format == "int4":
         result["cpu_baseline"] = cpu_tree_verify(args.seed, context, nodes, masks, args.cpu_seconds)
+    print(json.dumps(result))
+
+
+def stream_ceiling(args):
+    """Where the distance between the decode kernel and the 8 TB/s peak lies: the bytes of one
+    layer of the headline batch (16 743 pages x 4 KV heads x 8448 B) read by kernels that do
+    nothing else, in forms that are not the decode kernel's own (include/kvx_debug.h) --
+    a linear read from one extent; the shuffled page list with 16-byte loads of whole KiB at 2, 4
+    and 8 waves per SIMD; the decode kernel's own loads over the shuffled list, the list sorted
+    by address, a list drawn from 40 GB of the pool only, pages in address order; and twice the
+    pages per wave, whose extra time is what the bytes cost once a launch is under way.  One
+    JSON line: microseconds and GB/s per form."""
+    import numpy as np
+    import torch
+    from richengine_amd import kvx
+
+    L = kvx.lib()
+    torch.cuda.set_device(0)
+    rng = np.random.default_rng(args.seed)
+    layout = kvx.Layout(LAYERS, H, D, kvx.INT4, 0.0)
+    extent_pages = L.kvx_layout_largest_extent_pages(C.byref(layout))
+    page_bytes = L.kvx_layout_bytes_per_model_page(C.byref(layout))
+    free, _total = torch.cuda.mem_get_info()
+    pool_bytes = args.pool_gb * 1e9 if args.pool_gb > 0 else min(0.8 * free, 256e9)
+    extents = max(3, int(pool_bytes // (extent_pages * page_bytes)))
+    storage = kvx.Storage(LAYERS, H, D, kvx.INT4, extents * extent_pages, extent_pages, aligned=True)
+    storage.allocate_all()
+    n_pages = 16743
+    small = min(extents, 9)
+    lists = {
+        "shuffled over the pool": rng.permutation(extents * extent_pages)[:n_pages],
+        "the same pages sorted by address": None,
+        f"shuffled over {small} extents ({small * extent_pages * page_bytes / 1e9:.0f} GB)":
+            rng.permutation(small * extent_pages)[:n_pages],
+        "pages in address order": np.arange(n_pages),
+        "twice the pages, shuffled over the pool": rng.permutation(extents * extent_pages)[:2 * n_pages],
+    }
+    lists["the same pages sorted by address"] = np.sort(lists["shuffled over the pool"])
+    tables = {name: storage.table(ids.astype(np.uint32)) for name, ids in lists.items()}
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def timed(call):
+        for layer in range(2):
+            kvx.check(call(layer))
+        torch.cuda.synchronize()
+        k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        k0.record()
+        for it in range(args.kernel_iters):
+            call(it % LAYERS)
+        k1.record()
+        torch.cuda.synchronize()
+        return k0.elapsed_time(k1) / args.kernel_iters * 1e3  # microseconds
+
+    def kernel_loads(name, per):
+        table = tables[name]
+        return timed(lambda layer: L.kvx_calibrate_stream(storage.h, layer, table.data_ptr(), table.numel(),
+                                                          per, 1, sink.data_ptr(), stream))
+
+    def form(name, which, per, depth, waves):
+        table = tables[name]
+        return timed(lambda layer: L.kvx_calibrate_stream_form(storage.h, layer, table.data_ptr(),
+                                                               table.numel(), per, which, depth, waves,
+                                                               sink.data_ptr(), stream))
+
+    nbytes = n_pages * H * 8448
+    rows = []
+
+    def row(what, us, count=n_pages):
+        rows.append({"form": what, "us": round(us, 1), "gbs": round(count * H * 8448 / us / 1e3, 0)})
+
+    shuffled = "shuffled over the pool"
+    for per in (4, 16):
+        row(f"linear read of the same bytes from one extent, {2 * per} pieces of 4 KiB per wave",
+            form(shuffled, 2, per, 1, 8))
+    for waves in (2, 4, 8):
+        row(f"shuffled list, 16-byte loads of whole KiB, one page ahead, {waves} waves per SIMD, 34 pages per wave",
+            form(shuffled, 1, 34, 1, waves))
+    row("shuffled list, 16-byte loads of whole KiB, two pages ahead, 2 waves per SIMD, 34 pages per wave",
+        form(shuffled, 1, 34, 2, 2))
+    for per in (16, 34, 64):
+        row(f"shuffled list, the decode kernel's loads, 2 waves per SIMD, {per} pages per wave",
+            kernel_loads(shuffled, per))
+    one = rows[-2]["us"]
+    for name in list(lists)[1:4]:
+        row(f"{name}, the decode kernel's loads, 34 pages per wave", kernel_loads(name, 34))
+    two = kernel_loads("twice the pages, shuffled over the pool", 68)
+    row("twice the pages at 68 per wave (the same number of waves), the decode kernel's loads", two,
+        2 * n_pages)
+    rows.append({"form": "the second half of those bytes: what the list costs once a launch is under way",
+                 "us": round(two - one, 1), "gbs": round(nbytes / (two - one) / 1e3, 0)})
+    result = {
+        "metric": "HBM read rate for one layer of the int4 batch-32 decode step's pages, by request shape",
+        "value": rows[0]["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.kernel_iters, "warmup": 2,
+        "ms_per_step": round(rows[0]["us"] / 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "calibration: 16 743 pages x 4 KV heads x 8448 B per launch (the headline "
+                               "batch's bytes of one layer), pool of %d extents, %.1f GB" %
+                               (extents, extents * extent_pages * page_bytes / 1e9),
+                   "bytes_per_launch": nbytes, "seed": args.seed},
+        "forms": rows,
+        "roofline": {"bound": "hbm", "achieved": rows[0]["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(rows[0]["gbs"] / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "stream_linear_kernel (a plain read, no attention)"},
+        "cpu_baseline": None,
+    }
+    storage.close()
     print(json.dumps(result))
 
 
@@ -659,7 +819,7 @@ def shared_prefix(args):
         # one sequence of the 16 (the oracle has no shared form: every sequence walks its whole table)
         spent = cpu_lane(int(committed[0]), args.seed)
         result["cpu_baseline"] = {
-            "value": 1.0 / spent, "unit": "sequence-steps/s", "cores": 1, "kind": "port",
+            "value": 1.0 / spent, "unit": "sequence-steps/s", "cores": 1, "kind": "port", **host_cpus(),
             "sample": f"one sequence of the 16 ({int(committed[0]) + 1} tokens), one layer: append 1 token + "
                       f"decode attention over its whole table, {spent:.1f} s of scalar C++ oracle"}
     print(json.dumps(result))
@@ -916,7 +1076,7 @@ def single_decode(args):
     if args.cpu_seconds > 0:
         spent = cpu_lane(context, args.seed)
         result["cpu_baseline"] = {
-            "value": layer_bytes / spent / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "value": layer_bytes / spent / 1e9, "unit": "GB/s", "cores": 1, "kind": "port", **host_cpus(),
             "sample": f"the sequence itself, one layer of the 16: append 1 token + decode attention over "
                       f"{context + 1} tokens, {spent:.1f} s of scalar C++ oracle"}
     print(json.dumps(result))
@@ -935,6 +1095,8 @@ def main():
             kvx_build.build(verbose=False)
         if args.workload == "qkv-prepare":
             return qkv_prepare(args)
+        if args.workload == "stream-ceiling":
+            return stream_ceiling(args)
         if args.workload == "decode-single":
             return single_decode(args)
         if args.workload == "shared-prefix":

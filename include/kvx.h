@@ -696,23 +696,6 @@ int kv_compact_path(const kvx_storage *storage, uint32_t layer,
                     uint32_t n_lanes, const uint32_t *retained_path,
                     const uint32_t *retained_count, uint32_t path_stride, void *stream);
 
-/* Also no counterpart in the reference: how many attend calls of this process went to the
-   format-generic kernels and how many to the matrix-core (MFMA) kernels, so tests can tell
-   which path they measured. */
-void kvx_debug_attend_paths(uint64_t *generic_calls, uint64_t *matrix_core_calls);
-
-/* Calibration, no counterpart in the reference and no part of any attention path: streams
-   the pages of `page_table` (n_pages device entries of an int4, head dimension 256 storage)
-   with exactly the loads of the int4 decode kernel, two waves per SIMD, and nothing behind
-   them; workgroup x reads entries x * pages_per_wave onward, one wave per KV head,
-   heads_per_workgroup (1, 2 or 4, a divisor of the KV heads) of them in a workgroup.  Timing
-   it gives the rate the access pattern itself reaches, the ceiling the decode kernel is
-   measured against.  `sink`: one device word that is never written in practice.  KVX_EINVAL
-   for other formats. */
-int kvx_calibrate_stream(const kvx_storage *storage, uint32_t layer, const uint64_t *page_table,
-                         uint32_t n_pages, uint32_t pages_per_wave, uint32_t heads_per_workgroup,
-                         uint32_t *sink, void *stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -691,6 +691,14 @@ void ko_attention_row_weights(uint32_t format, uint32_t kv_heads, uint32_t head_
   }
 }
 
+// Threads the attention functions may spread independent rows and tiles over (the checks of
+// the GPU suite; 1, the default, for anything that is timed as a one-thread baseline).  Every
+// row is still computed by one thread in the reference's order, so the results do not depend
+// on the number.
+static int g_threads = 1;
+void ko_set_threads(int threads) { g_threads = threads > 1 ? threads : 1; }
+int ko_threads(void) { return g_threads; }
+
 int ko_attention_tile(uint32_t format, uint32_t kv_heads, uint32_t group, uint32_t head_dim,
                       uint32_t row_capacity, const uint16_t *tile_queries,
                       const uint64_t *page_table, ko_kv_layer kv, uint32_t kv_head,
@@ -709,14 +717,19 @@ int ko_attention_tile(uint32_t format, uint32_t kv_heads, uint32_t group, uint32
   const bool fp8 = format == KO_FP8E4M3;
   const bool quant = quantized(format);
   const float score_scale = default_score_scale(D, score_scale_param);
-  std::vector<float> q(D), acc(D), kc(size_t{kPage} * D);
+  // The question is the calling thread's (thread_local); the worker threads of the loop below
+  // read this copy of it and report into `turned_tokens`.
+  const Flips flips = g_flips;
+  uint32_t turned_tokens = 0;
 
+#pragma omp parallel for schedule(dynamic, 1) num_threads(g_threads) if (g_threads > 1)
   for (uint32_t r = 0; r < M; ++r) {
+    std::vector<float> q(D), acc(D);
     const uint32_t query_row = r / group;
     // Rows past the live ones are never read by the merge (it writes zeros
     // for them), so the oracle leaves their partials untouched.
     if (query_row >= active_rows) continue;
-    if (g_flips.only_row && g_flips.fused_row >= 0 && int64_t(r) != g_flips.fused_row) continue;
+    if (flips.only_row && flips.fused_row >= 0 && int64_t(r) != flips.fused_row) continue;
     for (uint32_t d = 0; d < D; ++d) {
       const float v = ko_bf16_to_float(tile_queries[uint64_t{r} * D + d]);
       q[d] = fp8 ? ko_round_to_f16(v) : v;  // fp8 tile stages queries as fp16
@@ -768,12 +781,15 @@ int ko_attention_tile(uint32_t format, uint32_t kv_heads, uint32_t group, uint32
         float w = 0.0f;
         if (admitted[j] && score[j] > -kInf) w = prob[j] * (quant ? s.value_scales[j] : 1.0f);
         weight[j] = fp8 ? ko_round_to_f16(w) : ko_bf16_to_float(ko_float_to_bf16(w));
-        if (g_flips.fused_row == int64_t(r))
-          for (uint32_t f = 0; f < g_flips.count; ++f)
-            if (g_flips.tokens[f] == token_start + j) {
+        if (flips.fused_row == int64_t(r))
+          for (uint32_t f = 0; f < flips.count; ++f)
+            if (flips.tokens[f] == token_start + j) {
               bool did = false;
-              weight[j] = turned(w, weight[j], fp8, g_flips.slack, &did);
-              if (did) g_flips.applied |= 1u << f;
+              weight[j] = turned(w, weight[j], fp8, flips.slack, &did);
+              if (did) {
+#pragma omp atomic
+                turned_tokens |= 1u << f;
+              }
             }
       }
       for (uint32_t d = 0; d < D; ++d) {
@@ -787,6 +803,7 @@ int ko_attention_tile(uint32_t format, uint32_t kv_heads, uint32_t group, uint32
     statistics[(slot * M + r) * 2] = row_max;
     statistics[(slot * M + r) * 2 + 1] = row_sum;
   }
+  g_flips.applied |= turned_tokens;
   return 1;
 }
 
@@ -834,6 +851,7 @@ int ko_attend_prefill(uint32_t format, uint32_t kv_heads, uint32_t group, uint32
   const uint32_t tiles = ko_prefill_tiles(p->rows);
   const uint64_t slots = uint64_t{tiles} * kv_heads * p->split_count;
   std::vector<float> partials(slots * M * D, 0.0f), statistics(slots * M * 2, 0.0f);
+#pragma omp parallel for schedule(dynamic, 1) num_threads(g_threads) if (g_threads > 1)
   for (uint32_t tile = 0; tile < tiles; ++tile) {
     const uint32_t tile_start = tile * R;
     const uint32_t active = std::min(R, p->rows - tile_start);

@@ -222,6 +222,12 @@ int ko_attention_tile(uint32_t format, uint32_t kv_heads, uint32_t group, uint32
 void ko_attention_flips(int64_t fused_row, const uint32_t *tokens, uint32_t count, float slack,
                         int only_row);
 uint32_t ko_attention_flips_applied(void);
+/* Threads that ko_attention_tile spreads a tile's rows over and ko_attend_prefill its tiles
+   (OpenMP; default 1).  Every row is computed by one thread in the same order whatever the
+   number, so results do not depend on it; it only shortens the checks of the GPU suite.
+   Timed baselines leave it at 1. */
+void ko_set_threads(int threads);
+int ko_threads(void);
 void ko_attention_row_weights(uint32_t format, uint32_t kv_heads, uint32_t head_dim,
                               const uint16_t *query_row, const uint64_t *page_table, ko_kv_layer kv,
                               uint32_t kv_head, uint32_t committed, uint32_t active_rows,

@@ -12,7 +12,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libkvx.so")
 SOURCES = ["kvx_host.cpp", "kvx_pool.cpp", "kvx_pool_abi.cpp", "kvx_prefix.cpp",
            "kvx_prefix_abi.cpp", "kvx_kernels.hip",
-           "kvx_decode_int4.hip", "kvx_attend_wide.hip"]
+           "kvx_decode_int4.hip", "kvx_attend_wide.hip", "kvx_calibrate.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
          # packed fp32 instructions stay off for every kernel of this library
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -27,6 +27,7 @@
 // scalar result.  The field's place costs one shift per dword.  Values use 128 +
 // field (136 + c, 135 - c): nothing is rounded after p.v but the result.
 #include "kvx_attend_common.h"
+#include "kvx_debug.h"
 
 namespace kvx {
 namespace {
@@ -67,7 +68,7 @@ __device__ __forceinline__ LaneOffsets lane_offsets(uint32_t t, uint32_t g, uint
           (lane < kPage ? 0u : scale_rows_apart) + 4u * (lane & (kPage - 1))};
 }
 
-// PARTS: bit 0 the keys, bit 1 values and both scale lines.
+// PARTS: bit 0 the keys, bit 1 the values, bit 2 the scale lines.
 template <uint32_t PARTS, bool REUSED>
 __device__ __forceinline__ void load_page(PageRegs &r, uint64_t entry, uint32_t head,
                                           uint32_t kv_heads, uint32_t layer_offset,
@@ -95,11 +96,12 @@ __device__ __forceinline__ void load_page(PageRegs &r, uint64_t entry, uint32_t 
 #pragma unroll
     for (uint32_t s = 0; s < 8; ++s)
       r.v[s] = load_streaming<u32x2, REUSED>(values + at.values + ((s < 4 ? 0 : 16) + (s & 3)) * kRowBytes);
-    // One scale per lane instead of the sixteen a lane multiplies with: they
-    // are fetched from the owning lanes when the page is attended, which keeps
-    // a register set at 33 registers.
-    r.scale = load_global<float>(region + key_scales_off + head_page * (kPage * 4u) + at.scale);
   }
+  // One scale per lane instead of the sixteen a lane multiplies with: they
+  // are fetched from the owning lanes when the page is attended, which keeps
+  // a register set at 33 registers.
+  if constexpr (PARTS & 4u)
+    r.scale = load_global<float>(region + key_scales_off + head_page * (kPage * 4u) + at.scale);
 }
 
 // x of this lane and x of the lane 16 (32) away, without the address register a
@@ -613,7 +615,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   // they would make every wait cover both.
   auto fill = [&](PageRegs &set, uint64_t entry) {
     asm volatile("");
-    load_page<3, kReused>(set, entry, head, H, a.kv.offset, ro.key_scales, ro.values, at);
+    load_page<7, kReused>(set, entry, head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
   // The same in two steps for the steady loop: the keys as soon as the page that
@@ -625,7 +627,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   };
   auto fill_rest = [&](PageRegs &set, uint64_t entry) {
     asm volatile("");
-    load_page<2, kReused>(set, entry, head, H, a.kv.offset, ro.key_scales, ro.values, at);
+    load_page<6, kReused>(set, entry, head, H, a.kv.offset, ro.key_scales, ro.values, at);
     asm volatile("");
   };
   // The first fills are unconditional too (a split shorter than kDepth pages
@@ -785,7 +787,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   uint32_t x = 0;
 #pragma unroll
   for (uint32_t d = 0; d < 2; ++d)
-    load_page<3, false>(r[d], scalar_entry(table, min(d, last_slot)), head, kv_heads, kv.offset,
+    load_page<7, false>(r[d], scalar_entry(table, min(d, last_slot)), head, kv_heads, kv.offset,
                         ro.key_scales, ro.values, at);
   for (uint32_t slot = 0; slot < count; slot += 2) {
 #pragma unroll
@@ -796,7 +798,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (uint32_t i = 0; i < 8; ++i) x ^= r[d].v[i][0] ^ r[d].v[i][1];
       x ^= __float_as_uint(r[d].scale);
       asm volatile("");
-      load_page<3, false>(r[d], scalar_entry(table, min(slot + d + 2, last_slot)), head, kv_heads,
+      load_page<7, false>(r[d], scalar_entry(table, min(slot + d + 2, last_slot)), head, kv_heads,
                           kv.offset, ro.key_scales, ro.values, at);
       asm volatile("");
     }

@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "kvx_device.h"
+#include "kvx_debug.h"
 
 namespace kvx {
 

@@ -46,7 +46,7 @@ SYMBOLS = [
     "kvx_sequences_compact_extent", "kvx_tree_masks", "kvx_tree_path_valid",
     "kvx_sequence_fork", "kvx_sequence_ensure_writable", "kvx_block_image_identity",
     "kvx_prefix_match_images", "kvx_sequence_publish_images", "kvx_sequence_truncate",
-    "kvx_static_workspace_prime",
+    "kvx_static_workspace_prime", "kvx_calibrate_stream_form",
 ]
 
 
@@ -198,6 +198,7 @@ def _declare(L):
     L.kvx_sequence_truncate.argtypes = [vp, u64, u64, PU32]
     L.kvx_debug_attend_paths.argtypes, L.kvx_debug_attend_paths.restype = [PU64, PU64], None
     L.kvx_calibrate_stream.argtypes = [vp, u32, vp, u32, u32, u32, vp, vp]
+    L.kvx_calibrate_stream_form.argtypes = [vp, u32, vp, u32, u32, u32, u32, u32, vp, vp]
     L.kvx_decode_plan.argtypes = [vp, u32, u32, u32, vp]
     L.kvx_verify_plan.argtypes = [vp, u32, u32, u32, u32, u32, vp]
     L.kvx_tree_masks.argtypes = [vp, u32, vp]

@@ -88,6 +88,9 @@ def bf16_ulp_diff(a_bits, b_bits):
 # Rows that were farther from the oracle than the tolerance and were shown to be one
 # rounding flip away from it, per check: (label, rows explained, rows checked).
 ALLOWANCE_LOG = []
+# What tests/test_gpu_score_deviation.py measured, per format: (name, samples, worst |max - max|,
+# worst |max + log(sum) - the same|, the flip slack the format's checks use).
+DEVIATION_LOG = []
 
 
 def check_attention(out_bits, want_bits, want_f32, rows_mask, tol, label="", explain=None):

@@ -14,9 +14,19 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "kvx.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(kvx?_[a-z0-9_]+)\s*\(", text)))
+    """The entries of the drop-in boundary (include/kvx.h) and the measurement and test hooks
+    beside it (include/kvx_debug.h)."""
+    names = set()
+    for header in ("kvx.h", "kvx_debug.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(kvx?_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
+
+
+def test_debug_hooks_stay_out_of_the_boundary_header():
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "kvx.h")).read(), flags=re.S)
+    assert "kvx_debug" not in text and "kvx_calibrate" not in text
 
 
 def test_library_exports_every_declared_symbol():
@@ -24,7 +34,7 @@ def test_library_exports_every_declared_symbol():
     names = declared_symbols()
     assert len(names) >= 50
     for name in names:
-        assert hasattr(L, name), f"{name} is declared in include/kvx.h but not exported"
+        assert hasattr(L, name), f"{name} is declared in include/kvx*.h but not exported"
     assert sorted(kvx.SYMBOLS) == names
 
 

@@ -153,8 +153,18 @@ def test_calibration_stream_runs_and_rejects_what_it_does_not_cover():
             for per in (1, 5, 64):
                 assert L.kvx_calibrate_stream(twin.dev.h, 1, table.data_ptr(), len(pages), per, heads,
                                               sink.data_ptr(), None) == 0
+        # the forms that are not the kernel's shape: 16-byte loads of whole KiB with 1, 2 or 4
+        # pages ahead at 1 to 8 waves per SIMD, and the linear read of as many bytes
+        for depth in (1, 2, 4):
+            for waves in (1, 2, 4, 8):
+                assert L.kvx_calibrate_stream_form(twin.dev.h, 1, table.data_ptr(), len(pages), 5,
+                                                   1, depth, waves, sink.data_ptr(), None) == 0
+        assert L.kvx_calibrate_stream_form(twin.dev.h, 1, None, 4, 2, 2, 1, 8, sink.data_ptr(), None) == 0
         torch.cuda.synchronize()
         assert int(sink.item()) == 0
+        for form, depth, waves, count in ((1, 3, 2, 4), (1, 2, 3, 4), (7, 1, 2, 4), (2, 1, 8, 1 << 20)):
+            assert L.kvx_calibrate_stream_form(twin.dev.h, 1, table.data_ptr(), count, 2, form, depth,
+                                               waves, sink.data_ptr(), None) == -1
         assert L.kvx_calibrate_stream(twin.dev.h, 1, table.data_ptr(), len(pages), 4, 3,
                                       sink.data_ptr(), None) == -1
         assert L.kvx_calibrate_stream(twin.dev.h, 2, table.data_ptr(), len(pages), 4, 1,

@@ -365,13 +365,31 @@ def test_rounding_flips_turn_only_weights_on_a_boundary(fmt):
         moved = np.linalg.norm(value(bits) - value(base[fused_row])) / np.linalg.norm(value(base[fused_row]))
         # one place of the weight's format, times at most the whole row
         assert 0 < moved <= size * (2.0 ** -7 if fmt != ko.FP8 else 2.0 ** -9) + 2e-3
-    # at the real slack a minority of the weights is that close to a boundary (about a quarter:
-    # the window is 1e-3 wide, a place 3.9e-3 to 7.8e-3); at a hundredth of it hardly any
+    # at the real slack (twice the measured score deviation of the format's kernels) a minority
+    # of bf16 weights is that close to a boundary (the window is 7.4e-4 wide, a place 3.9e-3 to
+    # 7.8e-3); an fp16 place, 4.9e-4 to 9.8e-4, is no wider than the window, so on fp8 pages
+    # most weights are; at a hundredth of the slack hardly any, in either format
     def near(slack):
         return sum(sum(1 for _, size, _ in ko.rounding_flip_rows(*args[:-1], r, top=6, slack=slack)
                        if size == 1) for r in range(0, 8 * G, 2))
-    assert near(ko.flip_slack(fmt)) <= 6 * 4 * G * 0.4 and near(ko.flip_slack(fmt) / 100) <= 2
+    considered = 6 * 4 * G
+    if fmt == ko.FP8:
+        assert near(ko.flip_slack(fmt)) >= 0.5 * considered and near(ko.flip_slack(fmt) / 100) <= 6
+    else:
+        assert near(ko.flip_slack(fmt)) <= 0.4 * considered and near(ko.flip_slack(fmt) / 100) <= 2
     again, _ = ko.attention_tile_rows(fmt, H, G, D, tile_q, table, kv, head, committed, active,
                                       splits, capacity)
     assert np.array_equal(again, base)
+    # the question belongs to the calling thread; the tile's worker threads must answer it too
+    before = ko.lib().ko_threads()
+    try:
+        ko.set_threads(4)
+        threaded = list(ko.rounding_flip_rows(*args, top=3, slack=1.0, together=3))
+        spread, _ = ko.attention_tile_rows(fmt, H, G, D, tile_q, table, kv, head, committed, active,
+                                           splits, capacity)
+    finally:
+        ko.set_threads(before)
+    assert np.array_equal(spread, base)
+    assert [(t, s) for t, s, _ in threaded] == [(t, s) for t, s, _ in rows]
+    assert all(np.array_equal(a[2], b[2]) for a, b in zip(threaded, rows))
     store.close()
