@@ -147,7 +147,10 @@ __device__ __forceinline__ u32x4 expand_key_dword(uint32_t x) {
 
 // Softmax state and accumulators of one block of 16 fused query rows.
 struct State {
-  f32x4 acc[16];  // [nibble position m]: dims 16*(4g + r) + m of column t
+  // [nibble position m]: register r holds dim 16 (4g + r) + m of fused row t; in the kernels
+  // that hold the tiles transposed (the probabilities as the A operand of p.v), dim
+  // 16 t + m of fused row 4g + r.
+  f32x4 acc[16];
   float row_max;
   float row_sum;   // this lane's tokens only; lanes of a column are summed at the end
   float bias;      // constant part carried by acc, this lane's tokens only
@@ -215,7 +218,11 @@ struct RegisterPage {
 // queries(nb, kb) yields the B operand of block nb for dims block kb.
 // PINNED: the kernel runs one wave per SIMD and its accumulators live in the second
 // register file (see the rescaling below).
-template <bool MASKED, uint32_t NB, bool PINNED, class Page, class Queries, class KeysConsumed>
+// ROWS_DOWN: the accumulator tiles are held transposed (State::acc); for kernels whose
+// accumulators live in the first register file, where one register of a tile can be
+// multiplied alone.
+template <bool MASKED, uint32_t NB, bool PINNED, bool ROWS_DOWN, class Page, class Queries,
+          class KeysConsumed>
 __device__ __forceinline__ void attend_page(const Page &source, Queries queries,
                                             const float *q_bias, float score_scale,
                                             uint32_t first_token, const Sight *sight,
@@ -285,7 +292,30 @@ __device__ __forceinline__ void attend_page(const Page &source, Queries queries,
       pb[nb][p] = bits ^ 0x80000000u;
     }
     st[nb].bias = fmaf(st[nb].bias, rescale, page_bias);
-    if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
+    const uint64_t grown = __builtin_amdgcn_ballot_w64(rescale != 1.0f);
+    if constexpr (ROWS_DOWN) {
+      // Register j of a lane holds fused row 4g + j, so the registers j need the multiply
+      // only when one of the four rows j, 4 + j, 8 + j, 12 + j has a new maximum: over a
+      // split of 64 pages that happens on about 15 pages, where some row of all sixteen
+      // grows on about 38.  The factors of those four rows come out of the lanes that hold
+      // them (lane t holds row t's).
+      if (grown) {
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+          if (uint32_t(grown) & (0x1111u << j)) {
+            const auto factor_of = [&](uint32_t row) {
+              return __uint_as_float(
+                  uint32_t(__builtin_amdgcn_readlane(int(__float_as_uint(rescale)), int(row))));
+            };
+            const float f0 = factor_of(j), f1 = factor_of(4 + j), f2 = factor_of(8 + j),
+                        f3 = factor_of(12 + j);
+            const float factor = g == 0 ? f0 : g == 1 ? f1 : g == 2 ? f2 : f3;
+#pragma unroll
+            for (uint32_t m = 0; m < 16; ++m) st[nb].acc[m][j] *= factor;
+          }
+        }
+      }
+    } else if (grown) {
 #pragma unroll
       for (uint32_t m = 0; m < 16; ++m) {
         // Accumulators in the second register file are named there on the way in, so that
@@ -307,7 +337,9 @@ __device__ __forceinline__ void attend_page(const Page &source, Queries queries,
       for (uint32_t i = 0; i < 4; ++i) {
         const uint32_t m = 8 * half + 4 * part + i;
 #pragma unroll
-        for (uint32_t nb = 0; nb < NB; ++nb) st[nb].acc[m] = mfma_bf16(vop[i], pb[nb], st[nb].acc[m]);
+        for (uint32_t nb = 0; nb < NB; ++nb)
+          st[nb].acc[m] = ROWS_DOWN ? mfma_bf16(pb[nb], vop[i], st[nb].acc[m])
+                                    : mfma_bf16(vop[i], pb[nb], st[nb].acc[m]);
       }
     }
   }
@@ -390,7 +422,7 @@ constexpr uint32_t kVerify48Depth = 1;
 
 // Writes what a wave has accumulated for its NB blocks: the finished bf16 rows
 // when the lane has a single split, else fp32 partial rows and (max, sum).
-template <uint32_t NB>
+template <uint32_t NB, bool ROWS_DOWN>
 __device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m, const bool *in_tile,
                                              const bool *live_row, const DecodeLane &l,
                                              const LaunchArgs &a, uint32_t head, uint32_t split,
@@ -400,6 +432,7 @@ __device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m,
                                              float *__restrict__ statistics) {
   const uint32_t G = a.group, M = a.fused_rows;
   uint16_t *out_head = output + l.q_offset + uint64_t(head) * a.row_stride * G * kD;
+  const uint64_t first_row = l.row_base + uint64_t(head) * l.split_count * M + uint64_t(split) * M;
 #pragma unroll
   for (uint32_t nb = 0; nb < NB; ++nb) {
     // Lanes of one column hold disjoint tokens: combine their sums and the
@@ -407,6 +440,52 @@ __device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m,
     float row_sum = st[nb].row_sum, bias = st[nb].bias;
     row_sum = column_sum(row_sum);
     bias = column_sum(bias);
+    if (written != 1 && live_row[nb] && g == 0) {
+      statistics[(first_row + m[nb]) * 2] = st[nb].row_max;
+      statistics[(first_row + m[nb]) * 2 + 1] = row_sum;
+    }
+    if constexpr (ROWS_DOWN) {
+      // Register rr of this lane holds fused row 4g + rr of the block, dims 16 t + 0 .. 15
+      // over the sixteen accumulators; the row's sum and constant part sit in lane 4g + rr.
+      const uint32_t t = threadIdx.x & 15;
+#pragma unroll
+      for (uint32_t rr = 0; rr < 4; ++rr) {
+        const uint32_t fused = m[nb] - t + 4 * g + rr;
+        const bool row_in_tile = fused < M, row_live = row_in_tile && fused / G < l.active_rows;
+        const float sum_of_row = __shfl(row_sum, int(4 * g + rr));
+        const float bias_of_row = __shfl(bias, int(4 * g + rr));
+        if (written == 1) {
+          // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
+          // Rows of the tile past the live ones read as zeros.
+          if (row_in_tile) {
+            const float denominator = row_live ? sum_of_row : 0.0f;
+#pragma unroll
+            for (uint32_t m8 = 0; m8 < 2; ++m8) {
+              u32x4 packed;
+#pragma unroll
+              for (uint32_t i = 0; i < 4; ++i) {
+                const float lo = st[nb].acc[8 * m8 + 2 * i][rr] - bias_of_row;
+                const float hi = st[nb].acc[8 * m8 + 2 * i + 1][rr] - bias_of_row;
+                const float qlo = denominator > 0.0f ? __fdiv_rn(lo, denominator) : 0.0f;
+                const float qhi = denominator > 0.0f ? __fdiv_rn(hi, denominator) : 0.0f;
+                packed[i] = uint32_t(f32_to_bf16(qlo)) | (uint32_t(f32_to_bf16(qhi)) << 16);
+              }
+              *reinterpret_cast<u32x4 *>(out_head + uint64_t(fused) * kD + 16 * t + 8 * m8) = packed;
+            }
+          }
+        } else if (row_live) {
+          float *out = partials + (first_row + fused) * kD + 16 * t;
+#pragma unroll
+          for (uint32_t m4 = 0; m4 < 4; ++m4) {
+            f32x4 v;
+#pragma unroll
+            for (uint32_t i = 0; i < 4; ++i) v[i] = st[nb].acc[4 * m4 + i][rr] - bias_of_row;
+            *reinterpret_cast<f32x4 *>(out + 4 * m4) = v;
+          }
+        }
+      }
+      continue;
+    }
     if (written == 1) {
       // One split: the merge's weights are exp(0) = 1, so the row is acc / sum.
       // Rows of the tile past the live ones read as zeros (row_sum is 0 there).
@@ -432,9 +511,7 @@ __device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m,
       continue;
     }
     if (live_row[nb]) {
-      const uint64_t row =
-          l.row_base + uint64_t(head) * l.split_count * M + uint64_t(split) * M + m[nb];
-      float *out = partials + row * kD;
+      float *out = partials + (first_row + m[nb]) * kD;
 #pragma unroll
       for (uint32_t rr = 0; rr < 4; ++rr)
 #pragma unroll
@@ -444,10 +521,6 @@ __device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m,
           for (uint32_t i = 0; i < 4; ++i) v[i] = st[nb].acc[4 * m4 + i][rr] - bias;
           *reinterpret_cast<f32x4 *>(out + 16 * (4 * g + rr) + 4 * m4) = v;
         }
-      if (g == 0) {
-        statistics[row * 2] = st[nb].row_max;
-        statistics[row * 2 + 1] = row_sum;
-      }
     }
   }
 }
@@ -464,6 +537,10 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
                                             float *__restrict__ statistics, const DecodeArgs &args) {
   // The forms that have a SIMD to themselves: three blocks, or two with two page sets.
   constexpr bool kPinned = NB == 3 || (NB == 2 && kDepth >= 2);
+  // Two blocks with one page set run two waves per SIMD with every accumulator in the first
+  // register file: they hold their tiles transposed, which needs the rescaling for a quarter
+  // of a tile's registers on a fifth of the pages instead of all of them on half.
+  constexpr bool kRowsDown = NB == 2 && kDepth == 1;
   const uint32_t item = kItemMajor ? blockIdx.y : blockIdx.x;
   const uint32_t head = kItemMajor ? blockIdx.x : blockIdx.y;
   uint32_t li;
@@ -694,7 +771,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
 #pragma unroll
     for (uint32_t d = 0; d < kDepth; ++d) {
       // upcoming[d] is the entry of slot page + d + kDepth - begin, this set's refill
-      attend_page<false, NB, kPinned>(RegisterPage{r[d], g}, staged_queries, q_bias, score_scale,
+      attend_page<false, NB, kPinned, kRowsDown>(RegisterPage{r[d], g}, staged_queries, q_bias, score_scale,
                              (page + d) * kPage, sight, g, st, [&] { fill_keys(r[d], upcoming[d]); });
       fill_rest(r[d], upcoming[d]);
       upcoming[d] = scalar_entry(entries, min(page + d + 2 * kDepth - begin, last_slot));
@@ -705,7 +782,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   for (uint32_t k = 0; k < kUnmaskedStop - 1; ++k) {
     const uint32_t d = k % kDepth;
     if (page + k < end) {
-      attend_page<true, NB, kPinned>(RegisterPage{r[d], g}, staged_queries, q_bias, score_scale,
+      attend_page<true, NB, kPinned, kRowsDown>(RegisterPage{r[d], g}, staged_queries, q_bias, score_scale,
                             (page + k) * kPage, sight, g, st, [] {});
       if (k + kDepth < kUnmaskedStop - 1 && page + k + kDepth < end) {
         fill(r[d], upcoming[d]);  // slot page + k + kDepth - begin, and d = k here
@@ -714,8 +791,8 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
     }
   }
 
-  write_blocks<NB>(st, m, in_tile, live_row, l, a, head, split, a.all_partials ? 2u : written, g, output,
-                   partials, statistics);
+  write_blocks<NB, kRowsDown>(st, m, in_tile, live_row, l, a, head, split, a.all_partials ? 2u : written,
+                              g, output, partials, statistics);
 }
 
 // One block of 16 fused rows per wave, two waves per SIMD: one-row decode, where
@@ -754,6 +831,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
     float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
   attend_int4<2, 1, true>(queries, output, partials, statistics, a);
+}
+
+// Two blocks with one register set of pages, for lanes of more than 32 fused rows that fill
+// blocks of 32 better than blocks of 48 (a tree of 16 nodes for a group of 6: three waves of
+// 32 rows).  Built for two waves per SIMD, so that every accumulator lives in the first
+// register file, where its rescaling costs one instruction a register instead of three;
+// per block and page it issues 235 vector instructions where the three-block kernel
+// issues 268, and a wave's vector instructions are what these kernels wait for.
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void verify32_int4_kernel(
+    const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
+    float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
+  attend_int4<2, 1, false>(queries, output, partials, statistics, a);
 }
 
 // Three blocks (48 fused rows: a chain of 8 rows for a group of 6 query heads, half
@@ -848,6 +937,11 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
   // read and expanded once per 48 rows instead of once per 32.
   if (verify_block_rows(KVX_FMT_INT4, fused_rows) == 48 && !many_tiles)
     return launch_matrix_attention(verify48_int4_kernel, "verify48_int4_kernel", 48, 64, s, kv,
+                                   query_heads, queries, output, page_tables, lanes, n_lanes,
+                                   row_masks, row_stride, lane_stride, workspace, workspace_bytes,
+                                   stream, nullptr, tile_rows, epilogue);
+  if (fused_rows > 32 && !many_tiles)
+    return launch_matrix_attention(verify32_int4_kernel, "verify32_int4_kernel", 32, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
                                    stream, nullptr, tile_rows, epilogue);

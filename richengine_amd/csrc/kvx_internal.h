@@ -115,12 +115,15 @@ struct Storage {
 // Fused query rows one wave of a verify launch covers: the matrix-core kernels
 // hold 32 per wave (16 when there are no more); the int4 kernels also have a
 // 48-row form, which reads and expands every page once for all three blocks of
-// 16 and costs about 1.4 waves of the 32-row form.  It is used where it leaves
-// fewer waves by more than that.
+// 16 but keeps its accumulators where rescaling them costs three times as much:
+// per page a wave of the 48-row form costs about 1.74 waves of the 32-row form
+// (5040 against 2900 cycles), and it is used where it leaves fewer waves by
+// more than that (48 fused rows: one wave against two; 96: two against three,
+// which is not enough).
 inline uint32_t verify_block_rows(uint32_t format, uint32_t fused_rows) {
   if (fused_rows <= 16) return 16;
   const uint32_t by32 = (fused_rows + 31) / 32, by48 = (fused_rows + 47) / 48;
-  if (format == KVX_FMT_INT4 && 7 * by48 < 5 * by32) return 48;
+  if (format == KVX_FMT_INT4 && 26 * by48 < 15 * by32) return 48;
   return 32;
 }
 // Whether tiles 2i and 2i + 1 of a chunked prefill that starts after `committed`

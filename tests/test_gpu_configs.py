@@ -443,8 +443,8 @@ def test_config5_int4_tree_verify_and_rollback(rule):
         assert splits == [128] * lanes
     else:
         splits = kvx.verify_plan(committed, nodes, H, QH)
-        # two waves of 48 fused rows per split and KV head, one round of the 1024 SIMDs
-        assert splits == [32] * lanes and sum(splits) * H * 2 <= 1024
+        # three waves of 32 fused rows per split and KV head, one round of the 1024 SIMDs
+        assert splits == [21] * lanes and sum(splits) * H * 3 <= 1024
     dp = [kvx.VerifyParams(committed[i], n_pages[i], kvx.KvLayer(), splits[i], 128, nodes, 16, 0.0)
           for i in range(lanes)]
     out = torch.zeros((lanes, H, 32, G, D), dtype=torch.int16, device="cuda")
