@@ -352,7 +352,7 @@ def tree_verify(args):
     sequence (branching <= 3).  A step = per layer, append the 16 draft rows and
     run masked verify attention over history + rows; then compact a seeded
     root-to-leaf path of every sequence, all layers in one call.  The dominant
-    kernel (verify48_int4_kernel) runs on the matrix cores; its line carries the
+    kernel (verify32_int4_kernel) runs on the matrix cores; its line carries the
     MFMA roofline (flops = 4 x D x fused query rows x visible tokens per layer)."""
     import numpy as np
     import torch
@@ -498,7 +498,7 @@ def tree_verify(args):
                      "traffic": None, "bytes_per_launch": kv_bytes,
                      "mfma_tflops": round(achieved, 1), "mfma_peak_tflops": MFMA_BF16_PEAK_TFLOPS,
                      "mfma_frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "kernel": ("verify48_int4_kernel (split kernel of verify attention, 48 fused rows per wave)"
+                     "kernel": ("verify32_int4_kernel (split kernel of verify attention, three waves of 32 fused rows)"
                                 if args.format == "int4" else
                                 "group_wide_kernel (split kernel of verify attention, four waves of 24 fused "
                                 "rows that share every page through LDS)") + ", one layer per launch",
