@@ -74,9 +74,11 @@ def parse():
     ap.add_argument("--prefill-chunk", type=int, default=2048, choices=[64, 128, 256, 512, 1024, 2048],
                     help="prefill: rows per chunk (BASELINE configs[3] has 2048); smaller chunks show "
                          "what kvx_prefill_plan's split counts do")
-    ap.add_argument("--prefill-streams", type=int, default=4,
+    ap.add_argument("--prefill-streams", type=int, default=None,
                     help="prefill: HIP streams the batch's sequences are spread over (1 = all on the "
-                         "current stream); a sequence's layers stay in order on its stream")
+                         "current stream); a sequence's layers stay in order on its stream.  0 = the "
+                         "batch in one kv_attend_prefill_batch call per layer on one stream.  Default: "
+                         "0 on int4 pages, 4 otherwise (the faster of the two by a few per cent)")
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
     ap.add_argument("--workload", choices=["decode", "decode-single", "tree-verify", "prefill", "qkv-prepare", "shared-prefix",
@@ -873,6 +875,11 @@ def chunked_prefill(args):
     # independent, and the 1536 waves of one sequence's launch leave half of the
     # SIMDs idle in their second round on the formats that run one wave per SIMD.
     # Launches of other sequences on other streams fill that round.
+    # --prefill-streams 0: the whole batch per layer in one kv_append and one
+    # kv_attend_prefill_batch call on one stream (every sequence's tiles in the same launch).
+    if args.prefill_streams is None:
+        args.prefill_streams = 0 if args.format == "int4" else 4
+    batched = args.prefill_streams == 0
     n_streams = max(1, min(args.prefill_streams, sequences))
     streams = [torch.cuda.Stream() for _ in range(n_streams)] if n_streams > 1 else [None]
     outputs = [torch.zeros_like(queries[0]) for _ in range(n_streams)]
@@ -883,9 +890,20 @@ def chunked_prefill(args):
     workspaces = [torch.empty(kvx.prefill_workspace_bytes(storage, chunk, QH, splits) + 4096, dtype=torch.uint8,
                               device="cuda") for _ in range(n_streams)]
     workspace = workspaces[0]
+    if batched:
+        all_k, all_v, all_q = torch.stack(chunk_k), torch.stack(chunk_v), torch.stack(queries)
+        all_out = torch.zeros_like(all_q)
+        all_ws = torch.empty(sequences * kvx.prefill_workspace_bytes(storage, chunk, QH, splits) + 4096,
+                             dtype=torch.uint8, device="cuda")
     torch.cuda.synchronize()
 
     def step():
+        if batched:
+            for layer in range(LAYERS):
+                kvx.append(storage, layer, all_k, all_v, tables, [cp] * sequences, H * chunk * D)
+                kvx.attend_prefill_batch(storage, layer, QH, all_q, all_out, tables, [pp] * sequences,
+                                         H * chunk * G * D, all_ws)
+            return
         # a sequence's layers follow one another on its stream, as they do in a model
         for layer in range(LAYERS):
             for s in range(sequences):
@@ -930,7 +948,10 @@ def chunked_prefill(args):
                                f"{chunk}-row chunks over 16384 + {chunk} tokens, 16 layers: quantize + scatter "
                                "of the chunk, then causal attention per layer and sequence",
                    "batch": sequences, "layers": LAYERS, "format": args.format, "splits": int(splits),
-                   "streams": n_streams, "seed": args.seed},
+                   "streams": 0 if batched else n_streams,
+                   "calls": "kv_attend_prefill_batch, one per layer" if batched
+                            else "kv_attend_prefill, one per layer and sequence",
+                   "seed": args.seed},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": None,
                      "kernel": "split kernel of kv_attend_prefill (prefill_int4_kernel or "

@@ -683,6 +683,22 @@ int kv_attend_prefill(const kvx_storage *storage, uint32_t layer, uint32_t query
                       const void *queries, void *output, const uint64_t *page_table,
                       const kvx_prefill_params *params, void *workspace,
                       uint64_t workspace_bytes, void *stream);
+/* The chunks of several sequences in one call, as the reference records the lanes of a step in one
+   command (ops::PagedAttention::addVerify's lane array, runtime/ops/PagedAttention.cpp:467-500; its
+   addPrefill takes one sequence).  Sequence q has params[q] and page_tables[q]; its queries and
+   output rows ([kv head][chunk_stride][group][D] as above) begin q x sequence_stride elements after
+   the first sequence's.  Chunks of the same shape (rows, chunk_stride and split_count equal, and
+   committed_tokens such that their tiles are paired or grouped alike: page-aligned starts always
+   are) share their launches, 32 sequences at a time: every sequence's tiles are lanes of one
+   launch.  Anything else runs sequence by sequence on `stream`.  Either way every sequence's
+   rows are the bits kv_attend_prefill gives for it alone.  workspace: at least the sum of the
+   sequences' kvx_prefill_workspace_for() bounds plus 256 bytes.  Nothing is enqueued unless every
+   sequence's parameters are valid. */
+int kv_attend_prefill_batch(const kvx_storage *storage, uint32_t layer, uint32_t query_heads,
+                            const void *queries, void *output, const uint64_t *const *page_tables,
+                            const kvx_prefill_params *params, uint32_t n_sequences,
+                            uint64_t sequence_stride, void *workspace, uint64_t workspace_bytes,
+                            void *stream);
 
 /* Tree-path compaction after acceptance: for i < retained_count[lane], the
    row at committed + retained_path[lane * path_stride + i] moves to

@@ -489,6 +489,22 @@ public:
     check(kv_attend_prefill(storage.handle(), layer, plan.queryHeads, queries, output, pageTable, &p,
                             workspace, workspaceBytes, stream));
   }
+  // The chunks of several sequences in one call (no counterpart in the reference, whose
+  // addPrefill takes one sequence): sequence q's queries and rows lie q x sequenceStride
+  // elements after the first's; chunks of one shape share their launches.
+  static void addPrefillBatch(void *stream, const kv::PageStorage &storage, uint32_t layer,
+                              const void *queries, void *output, void *workspace, uint64_t workspaceBytes,
+                              const uint64_t *const *pageTables,
+                              const std::vector<kv::ChunkedPrefillParams> &chunks, uint64_t sequenceStride,
+                              const PrefillAttentionPlan &plan) {
+    std::vector<kv::PrefillAttentionParams> params;
+    for (const kv::ChunkedPrefillParams &chunk : chunks)
+      params.push_back({chunk.committed_tokens, chunk.chunk_tokens, chunk.chunk_stride,
+                        chunk.page_table_entries, {}, plan.splits, plan.scoreScale});
+    check(kv_attend_prefill_batch(storage.handle(), layer, plan.queryHeads, queries, output, pageTables,
+                                  params.data(), static_cast<uint32_t>(params.size()), sequenceStride,
+                                  workspace, workspaceBytes, stream));
+  }
   // Stores each lane's chunk and attends its rows with the plan's split counts.
   // With gateHidden the merge also writes the out-projection's operand
   // ([lane][row capacity][query head][D]): scaled by the sigmoid of the gates in

@@ -97,10 +97,13 @@ struct DecodeArgs {
   // describes the first of that many lanes over one page table, each tile_rows
   // query rows and committed tokens after the one before, its queries
   // tile_lane_stride elements further on; the last holds tile_last_rows rows.
-  // Any number of them fits one launch.
+  // Any number of them fits one launch.  With tile_per_sequence < tile_lanes the
+  // lanes are runs of tile_per_sequence lanes, one run per sequence of a batch of equal
+  // chunks: lane[s] describes the first lane of run s.
   uint32_t tile_lanes;
   uint32_t tile_rows;
   uint32_t tile_last_rows;
+  uint32_t tile_per_sequence;
   uint64_t tile_lane_stride;
   // The merge's second output (see Epilogue): hidden rows of the launch's first
   // lane onwards, and the packed rows their gates come from (null = no gate).
@@ -120,13 +123,18 @@ __device__ __forceinline__ DecodeLane lane_at(const DecodeArgs &a, uint32_t inde
   // Field by field from a reference into the kernel arguments: a copy of a whole
   // lane record picked by a run-time index would make the compiler move the
   // argument block to scratch memory.
-  const uint32_t tile = a.tile_lanes ? index : 0u;
-  const DecodeLane &from = a.lane[a.tile_lanes ? 0u : index];
+  uint32_t tile = 0, record = index;
+  if (a.tile_lanes) {
+    record = a.tile_per_sequence < a.tile_lanes ? index / a.tile_per_sequence : 0u;
+    tile = index - record * a.tile_per_sequence;
+  }
+  const DecodeLane &from = a.lane[record];
   DecodeLane l;
   l.table = from.table;
   l.masks = from.masks;
   l.committed = from.committed + tile * a.tile_rows;
-  l.active_rows = (a.tile_lanes && index + 1 == a.tile_lanes) ? a.tile_last_rows : from.active_rows;
+  l.active_rows =
+      (a.tile_lanes && tile + 1 == a.tile_per_sequence) ? a.tile_last_rows : from.active_rows;
   l.split_count = from.split_count;
   l.first_item = a.tile_lanes ? index * from.split_count : from.first_item;
   l.score_scale = from.score_scale;
@@ -374,7 +382,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
                             uint32_t n_lanes, const uint32_t *row_masks, uint32_t row_stride,
                             uint64_t lane_stride, void *workspace, uint64_t workspace_bytes,
                             hipStream_t stream, const FusedAppend *fused = nullptr,
-                            uint32_t tile_rows = 0, const Epilogue *epilogue = nullptr,
+                            Tiles tile_rows = 0, const Epilogue *epilogue = nullptr,
                             bool longest_first = false) {
   const bool run_split = !(epilogue && epilogue->merge_only);
   const bool run_merge = !(epilogue && epilogue->partials_only);
@@ -397,6 +405,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
     a.n_lanes = std::min(lanes_per_launch, n_lanes - first);
     if (tile_rows) {
       a.tile_lanes = n_lanes;
+      a.tile_per_sequence = n_lanes / tile_rows.sequences;
       a.tile_rows = tile_rows;
       a.tile_last_rows = lanes[n_lanes - 1].active_rows;
       a.tile_lane_stride = lane_stride;
@@ -418,13 +427,15 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
     // order of the lane records, which is the order the work items are dispatched in, may
     // differ: longest_first puts the lanes with the longest splits first (a plan that pairs
     // long and short splits on a SIMD counts on the long ones taking the first wave slots).
-    const uint32_t recorded = tile_rows ? 1u : a.n_lanes;
+    // Regular lanes: one record per run, that of the run's first lane.
+    const uint32_t recorded = tile_rows ? tile_rows.sequences : a.n_lanes;
+    const uint32_t run = tile_rows ? n_lanes / tile_rows.sequences : 1u;
     uint64_t lane_row_base[kLanes];
     uint32_t order[kLanes];
     for (uint32_t i = 0; i < recorded; ++i) {
-      order[i] = i;
+      order[i] = i * run;
       lane_row_base[i] = row_base;
-      row_base += uint64_t(lanes[first + i].split_count) * H * M;
+      row_base += uint64_t(lanes[first + i * run].split_count) * H * M * run;
     }
     if (longest_first && !tile_rows) {
       const auto split_pages = [&](uint32_t k) {
@@ -437,7 +448,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       a.item_major = 1;
     }
     for (uint32_t i = 0; i < recorded; ++i) {
-      const uint32_t source = order[i];
+      const uint32_t source = order[i];  // index of the lane (of the run's first lane)
       const kvx_verify_params &p = lanes[first + source];
       DecodeLane &dl = a.lane[i];
       dl.table = page_tables ? page_tables[first + source] : nullptr;
@@ -449,8 +460,9 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
       a.item_base[i] = items;
       dl.score_scale = p.score_scale != 0.0f ? p.score_scale : l.score_scale;
       dl.source = source;
-      dl.row_base = lane_row_base[source];
-      dl.q_offset = uint64_t(first + source) * lane_stride;
+      dl.row_base = lane_row_base[tile_rows ? i : source];
+      dl.q_offset = tile_rows ? uint64_t(i) * tile_rows.sequence_stride
+                              : uint64_t(first + source) * lane_stride;
       items += p.split_count;
       max_splits = std::max(max_splits, p.split_count);
     }

@@ -1004,7 +1004,7 @@ int kvx_attend_wide_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                            const kvx_verify_params *lanes, uint32_t n_lanes,
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
-                           hipStream_t stream, uint32_t tile_rows, const Epilogue *epilogue) {
+                           hipStream_t stream, Tiles tile_rows, const Epilogue *epilogue) {
   const uint32_t format = s->layout.format;
   if ((format != KVX_FMT_BF16 && format != KVX_FMT_FP8E4M3 && format != KVX_FMT_INT8) ||
       !matrix_attention_covers(s, query_heads, lanes, n_lanes))

@@ -914,7 +914,7 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
                            hipStream_t stream, const void *append_keys, const void *append_values,
-                           uint64_t append_lane_stride, uint32_t append_stride, uint32_t tile_rows,
+                           uint64_t append_lane_stride, uint32_t append_stride, Tiles tile_rows,
                            const Epilogue *epilogue) {
   if (s->layout.format != KVX_FMT_INT4 || !matrix_attention_covers(s, query_heads, lanes, n_lanes))
     return 1;

@@ -95,6 +95,20 @@ struct Epilogue {
   bool merge_only = false;
 };
 
+// Regular lanes of a launch (the tiles of chunked prefill): `rows` > 0 says that the lanes
+// passed are `sequences` runs of equally many lanes, lane i of a run being its first lane
+// moved on by i x rows query rows and committed tokens over the run's one page table; the
+// runs' queries and rows lie sequence_stride elements apart.  rows = 0: ordinary lanes.
+struct Tiles {
+  uint32_t rows = 0;
+  uint32_t sequences = 1;
+  uint64_t sequence_stride = 0;
+  Tiles(uint32_t tile_rows = 0) : rows(tile_rows) {}
+  Tiles(uint32_t tile_rows, uint32_t runs, uint64_t stride)
+      : rows(tile_rows), sequences(runs), sequence_stride(stride) {}
+  operator uint32_t() const { return rows; }
+};
+
 // ---- storage ----------------------------------------------------------------
 struct Storage {
   kvx_layout layout;

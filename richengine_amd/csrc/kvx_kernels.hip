@@ -1237,7 +1237,7 @@ int kvx_attend_int4_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
                            hipStream_t stream, const void *append_keys = nullptr,
                            const void *append_values = nullptr, uint64_t append_lane_stride = 0,
-                           uint32_t append_stride = 0, uint32_t tile_rows = 0,
+                           uint32_t append_stride = 0, Tiles tile_rows = 0,
                            const Epilogue *epilogue = nullptr);
 
 int kvx_attend_wide_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t query_heads,
@@ -1245,7 +1245,7 @@ int kvx_attend_wide_launch(const kvx_storage *storage, kvx_kv_layer kv, uint32_t
                            const kvx_verify_params *lanes, uint32_t n_lanes,
                            const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                            void *workspace, uint64_t workspace_bytes, int many_tiles,
-                           hipStream_t stream, uint32_t tile_rows = 0,
+                           hipStream_t stream, Tiles tile_rows = 0,
                            const Epilogue *epilogue = nullptr);
 
 // int4 pages go to their own kernels, bf16, fp8 and int8 pages to the wide-element
@@ -1255,7 +1255,7 @@ static int attend_matrix(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_h
                          const kvx_verify_params *lanes, uint32_t n_lanes,
                          const uint32_t *row_masks, uint32_t row_stride, uint64_t lane_stride,
                          void *workspace, uint64_t workspace_bytes, int many_tiles,
-                         hipStream_t stream, uint32_t tile_rows = 0,
+                         hipStream_t stream, Tiles tile_rows = 0,
                          const Epilogue *epilogue = nullptr) {
   // tile_rows > 0: the lanes are regular (lane i = lane 0 moved on by i x tile_rows
   // rows and tokens over one table, all full but perhaps the last), which lets
@@ -1962,6 +1962,121 @@ int kv_append_attend_decode_hidden(const kvx_storage *s, uint32_t layer, const v
                               workspace, workspace_bytes, &epilogue, stream);
 }
 
+namespace {
+// How the tiles of a chunk go to the matrix-core kernels.
+// With a single split every tile walks its pages from the first, so two
+// neighbouring tiles can share one walk as a lane of 16 rows: a row's softmax
+// runs over the same pages in the same order (the page the second tile may
+// add is invisible to the first tile's rows and changes nothing), and every
+// key and value is fetched and expanded once for 16 rows instead of 8.
+// With several splits the two tiles must also cut their pages into the same
+// splits, which they do when they see the same number of pages
+// (prefill_tiles_pair: true for every pair of the chunk, or for none), and pay
+// only where the paired launch fills the GPU (prefill_pairs_with_splits).
+// bf16, fp8 and int8 pages: lanes of four (or two) tiles for a workgroup that shares
+// every page through LDS (prefill_group_width); with several splits only where a
+// lane's tiles cut their pages alike.
+struct TileShape {
+  uint32_t width;  // tiles per lane
+  int lane_kind;   // attend_matrix's many_tiles
+  bool operator==(const TileShape &o) const { return width == o.width && lane_kind == o.lane_kind; }
+};
+TileShape tile_shape(const kvx_layout &l, uint32_t query_heads, const kvx_prefill_params &p) {
+  const uint32_t H = l.kv_heads, G = query_heads / H;
+  const uint32_t tiles = (p.rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+  TileShape shape;
+  shape.width = (tiles >= 2 && (p.split_count == 1 ||
+                                prefill_pairs_with_splits(l.format, p.committed_tokens, tiles,
+                                                          p.split_count, H, G)))
+                    ? 2
+                    : 1;
+  shape.lane_kind = shape.width == 1 ? 1 : 0;
+  const uint32_t grouped = prefill_group_width(l.format, l.head_dim, p.rows, G);
+  if (grouped && tiles >= grouped &&
+      (p.split_count == 1 || prefill_group_splits_alike(grouped, p.committed_tokens))) {
+    shape.width = grouped;
+    shape.lane_kind = 2;
+  }
+  return shape;
+}
+
+int validate_prefill(const kvx_layout &l, uint32_t query_heads, const kvx_prefill_params &p) {
+  const kvx_chunk_params chunk{p.committed_tokens, p.rows, p.chunk_stride, p.page_table_entries, {}};
+  static const char *const names[] = {"", "chunk_tokens_out_of_range", "context_out_of_range",
+                                      "chunk_stride_invalid", "page_table_too_short"};
+  if (const int e = kvx_chunk_validation(&chunk)) return fail(KVX_EINVAL, names[e]);
+  if (!p.split_count || p.split_count > KVX_PREFILL_MAX_SPLITS)
+    return fail(KVX_EINVAL, "prefill split count is out of range");
+  if (KVX_PREFILL_TILE_ROWS * (query_heads / l.kv_heads) > 128)
+    return fail(KVX_EINVAL, "tile holds more than 128 fused rows");
+  return KVX_OK;
+}
+uint64_t prefill_rows(const kvx_layout &l, uint32_t query_heads, const kvx_prefill_params &p) {
+  const uint32_t tiles = (p.rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+  return uint64_t(tiles) * l.kv_heads * p.split_count * KVX_PREFILL_TILE_ROWS * (query_heads / l.kv_heads);
+}
+
+// The chunks of `sequences` sequences (equal rows, stride, split count and tile shape; one
+// sequence is the plain call) on the matrix-core kernels, every sequence's tiles in the same
+// launch: 0 when enqueued, 1 when the kernels decline the shape, or a negative status.
+int prefill_matrix(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_heads, const void *queries,
+                   void *output, const uint64_t *const *page_tables, const kvx_prefill_params *params,
+                   uint32_t sequences, uint64_t sequence_stride, void *workspace,
+                   uint64_t workspace_bytes, hipStream_t st) {
+  const kvx_layout &l = s->layout;
+  const uint32_t H = l.kv_heads, G = query_heads / H, D = l.head_dim;
+  const uint32_t T = KVX_PREFILL_TILE_ROWS;
+  const uint32_t tiles = (params[0].rows + T - 1) / T;
+  // The matrix-core kernels take the tiles as lanes: tile t attends rows 8t..8t+7
+  // over committed + 8t tokens, its queries 8 rows further on in the chunk.
+  const TileShape shape = tile_shape(l, query_heads, params[0]);
+  const uint32_t width = shape.width;
+  const uint32_t wide_lanes = tiles / width, rest = tiles - wide_lanes * width;
+  // every sequence's wide lanes, then every sequence's odd last tile
+  std::vector<kvx_verify_params> tile_lanes(size_t(sequences) * (wide_lanes + rest));
+  std::vector<const uint64_t *> tile_tables(tile_lanes.size());
+  for (uint32_t q = 0; q < sequences; ++q) {
+    const kvx_prefill_params &p = params[q];
+    for (uint32_t t = 0; t < wide_lanes + rest; ++t) {
+      const bool wide = t < wide_lanes;
+      const uint32_t first_row = wide ? T * width * t : T * (wide_lanes * width + (t - wide_lanes));
+      const uint32_t capacity = wide ? T * width : T;
+      // the odd last tiles tile by tile, so that each launch of them has one lane per sequence
+      const size_t at = wide ? size_t(q) * wide_lanes + t
+                             : size_t(sequences) * wide_lanes + size_t(t - wide_lanes) * sequences + q;
+      tile_lanes[at] = {p.committed_tokens + first_row, p.page_table_entries, {}, p.split_count,
+                        p.split_count, std::min(capacity, p.rows - first_row), capacity,
+                        p.score_scale};
+      tile_tables[at] = page_tables[q];
+    }
+  }
+  int fast = 1;
+  if (wide_lanes)
+    fast = took(attend_matrix(s, kv, query_heads, queries, output, tile_tables.data(),
+                              tile_lanes.data(), sequences * wide_lanes, nullptr,
+                              params[0].chunk_stride, uint64_t(T) * width * G * D, workspace,
+                              workspace_bytes, shape.lane_kind, st,
+                              Tiles(T * width, sequences, sequence_stride)));
+  if (!wide_lanes) fast = 0;
+  // The odd last tiles on their own, as ordinary lanes; lanes of one launch share a row
+  // capacity.  One sequence: its last tiles in one launch, a tile apart.  Several: the
+  // sequences' k-th last tiles in one launch, a sequence apart.
+  const uint32_t rest_launches = sequences > 1 ? rest : (rest ? 1u : 0u);
+  for (uint32_t k = 0; k < rest_launches && fast == 0; ++k) {
+    const uint64_t skip = uint64_t(T) * (uint64_t(width) * wide_lanes + k) * G * D;
+    const size_t at = size_t(sequences) * wide_lanes + size_t(k) * sequences;
+    fast = attend_matrix(s, kv, query_heads, static_cast<const uint16_t *>(queries) + skip,
+                         static_cast<uint16_t *>(output) + skip, tile_tables.data() + at,
+                         tile_lanes.data() + at, sequences > 1 ? sequences : rest, nullptr,
+                         params[0].chunk_stride, sequences > 1 ? sequence_stride : uint64_t(T) * G * D,
+                         workspace, workspace_bytes, 1, st);
+    if (fast > 0 && (wide_lanes || k))
+      return fail(KVX_ESTATE, "the last prefill tile was declined after the others ran");
+  }
+  return fast;
+}
+}  // namespace
+
 int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
                       const void *queries, void *output, const uint64_t *page_table,
                       const kvx_prefill_params *params, void *workspace, uint64_t workspace_bytes,
@@ -1975,79 +2090,18 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
   if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
   if (!query_heads || query_heads % l.kv_heads)
     return fail(KVX_EINVAL, "query heads are not a multiple of the KV heads");
-  const kvx_chunk_params chunk{params->committed_tokens, params->rows, params->chunk_stride,
-                               params->page_table_entries, {}};
-  static const char *const names[] = {"", "chunk_tokens_out_of_range", "context_out_of_range",
-                                      "chunk_stride_invalid", "page_table_too_short"};
-  if (const int e = kvx_chunk_validation(&chunk)) return fail(KVX_EINVAL, names[e]);
-  if (!params->split_count || params->split_count > KVX_PREFILL_MAX_SPLITS)
-    return fail(KVX_EINVAL, "prefill split count is out of range");
+  if (int rc = validate_prefill(l, query_heads, *params)) return rc;
   const uint32_t H = l.kv_heads, G = query_heads / H, D = l.head_dim;
   const uint32_t tiles = (params->rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
   const uint32_t M = KVX_PREFILL_TILE_ROWS * G;
-  if (M > 128) return fail(KVX_EINVAL, "tile holds more than 128 fused rows");
-  const uint64_t rows = uint64_t(tiles) * H * params->split_count * M;
+  const uint64_t rows = prefill_rows(l, query_heads, *params);
   const uint64_t partial_bytes = rows * D * sizeof(float);
   if (workspace_bytes < partial_bytes + rows * 2 * sizeof(float))
     return fail(KVX_EINVAL, "prefill attention scratch is smaller than its bound");
   auto st = static_cast<hipStream_t>(stream);
   {
-    // The matrix-core kernels take the tiles as lanes: tile t attends rows 8t..8t+7
-    // over committed + 8t tokens, its queries 8 rows further on in the chunk.
-    // With a single split every tile walks its pages from the first, so two
-    // neighbouring tiles can share one walk as a lane of 16 rows: a row's softmax
-    // runs over the same pages in the same order (the page the second tile may
-    // add is invisible to the first tile's rows and changes nothing), and every
-    // key and value is fetched and expanded once for 16 rows instead of 8.
-    // With several splits the two tiles must also cut their pages into the same
-    // splits, which they do when they see the same number of pages
-    // (prefill_tiles_pair: true for every pair of the chunk, or for none), and pay
-    // only where the paired launch fills the GPU (prefill_pairs_with_splits).
-    const uint32_t T = KVX_PREFILL_TILE_ROWS;
-    uint32_t width =
-        (tiles >= 2 && (params->split_count == 1 ||
-                        prefill_pairs_with_splits(l.format, params->committed_tokens, tiles,
-                                                  params->split_count, H, G)))
-            ? 2
-            : 1;
-    // bf16, fp8 and int8 pages: lanes of four (or two) tiles for a workgroup that shares
-    // every page through LDS (prefill_group_width); with several splits only where a
-    // lane's tiles cut their pages alike.
-    int lane_kind = width == 1 ? 1 : 0;  // attend_matrix's many_tiles
-    const uint32_t grouped = prefill_group_width(l.format, D, params->rows, G);
-    if (grouped && tiles >= grouped &&
-        (params->split_count == 1 || prefill_group_splits_alike(grouped, params->committed_tokens))) {
-      width = grouped;
-      lane_kind = 2;
-    }
-    const uint32_t wide_lanes = tiles / width, rest = tiles - wide_lanes * width;
-    std::vector<kvx_verify_params> tile_lanes(wide_lanes + rest);
-    std::vector<const uint64_t *> tile_tables(wide_lanes + rest, page_table);
-    for (uint32_t t = 0; t < wide_lanes + rest; ++t) {
-      const uint32_t first_row = t < wide_lanes ? T * width * t : T * (wide_lanes * width + (t - wide_lanes));
-      const uint32_t capacity = t < wide_lanes ? T * width : T;
-      tile_lanes[t] = {params->committed_tokens + first_row,
-                       params->page_table_entries,
-                       {},
-                       params->split_count,
-                       params->split_count,
-                       std::min(capacity, params->rows - first_row),
-                       capacity,
-                       params->score_scale};
-    }
-    int fast = took(attend_matrix(s, kv, query_heads, queries, output, tile_tables.data(),
-                                  tile_lanes.data(), wide_lanes, nullptr, params->chunk_stride,
-                                  uint64_t(T) * width * G * D, workspace, workspace_bytes,
-                                  lane_kind, st, T * width));
-    if (fast == 0 && rest) {
-      // The odd last tile on its own; lanes of one launch share a row capacity.
-      const uint64_t skip = uint64_t(T) * width * wide_lanes * G * D;
-      fast = attend_matrix(s, kv, query_heads, static_cast<const uint16_t *>(queries) + skip,
-                           static_cast<uint16_t *>(output) + skip, tile_tables.data(),
-                           tile_lanes.data() + wide_lanes, rest, nullptr, params->chunk_stride,
-                           uint64_t(T) * G * D, workspace, workspace_bytes, 1, st);
-      if (fast > 0) return fail(KVX_ESTATE, "the last prefill tile was declined after the others ran");
-    }
+    const int fast = prefill_matrix(s, kv, query_heads, queries, output, &page_table, params, 1, 0,
+                                    workspace, workspace_bytes, st);
     if (fast <= 0) return fast;
   }
   float *partials = static_cast<float *>(workspace);
@@ -2067,6 +2121,63 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
   hipLaunchKernelGGL(prefill_reduce_kernel, dim3(M, H, tiles), dim3(D), 0, st, partials, statistics,
                      static_cast<uint16_t *>(output), p);
   return check_launch("prefill_reduce_kernel");
+}
+
+int kv_attend_prefill_batch(const kvx_storage *s, uint32_t layer, uint32_t query_heads,
+                            const void *queries, void *output, const uint64_t *const *page_tables,
+                            const kvx_prefill_params *params, uint32_t n_sequences,
+                            uint64_t sequence_stride, void *workspace, uint64_t workspace_bytes,
+                            void *stream) {
+  if (!s || !queries || !output || !page_tables || !params || !workspace || !n_sequences)
+    return fail(KVX_EINVAL, "kv_attend_prefill_batch: null argument or no sequences");
+  if (s->accounting) return fail(KVX_ESTATE, "accounting-only storage has no memory to run on");
+  if (queries == output) return fail(KVX_EINVAL, "queries and output must not alias");
+  const kvx_layout &l = s->layout;
+  kvx_kv_layer kv;
+  if (int rc = kvx_storage_layer(s, layer, &kv)) return rc;
+  if (!query_heads || query_heads % l.kv_heads)
+    return fail(KVX_EINVAL, "query heads are not a multiple of the KV heads");
+  // Nothing is enqueued unless every sequence is valid.
+  const uint32_t G = query_heads / l.kv_heads;
+  uint64_t rows = 0;
+  bool alike = true;
+  for (uint32_t q = 0; q < n_sequences; ++q) {
+    if (!page_tables[q]) return fail(KVX_EINVAL, "null page table");
+    if (int rc = validate_prefill(l, query_heads, params[q])) return rc;
+    if (n_sequences > 1 &&
+        sequence_stride < uint64_t(l.kv_heads) * params[q].chunk_stride * G * l.head_dim)
+      return fail(KVX_EINVAL, "sequence stride is smaller than a sequence's chunk");
+    rows += prefill_rows(l, query_heads, params[q]);
+    alike = alike && params[q].rows == params[0].rows &&
+            params[q].chunk_stride == params[0].chunk_stride &&
+            params[q].split_count == params[0].split_count &&
+            tile_shape(l, query_heads, params[q]) == tile_shape(l, query_heads, params[0]);
+  }
+  if (workspace_bytes < rows * l.head_dim * sizeof(float) + 256 + rows * 2 * sizeof(float))
+    return fail(KVX_EINVAL, "prefill attention scratch is smaller than its bound");
+  auto st = static_cast<hipStream_t>(stream);
+  // Equal chunks (what a scheduler that cuts chunks of its token budget produces) share
+  // their launches, 32 sequences at a time; anything else runs sequence by sequence.
+  if (alike && n_sequences > 1) {
+    int fast = 0;
+    for (uint32_t first = 0; first < n_sequences && fast == 0; first += KVX_LANES_PER_LAUNCH) {
+      const uint32_t count = std::min<uint32_t>(KVX_LANES_PER_LAUNCH, n_sequences - first);
+      fast = prefill_matrix(s, kv, query_heads,
+                            static_cast<const uint16_t *>(queries) + first * sequence_stride,
+                            static_cast<uint16_t *>(output) + first * sequence_stride,
+                            page_tables + first, params + first, count, sequence_stride, workspace,
+                            workspace_bytes, st);
+      if (fast > 0 && first) return fail(KVX_ESTATE, "a later part of the batch was declined");
+    }
+    if (fast <= 0) return fast;
+  }
+  for (uint32_t q = 0; q < n_sequences; ++q)
+    if (int rc = kv_attend_prefill(s, layer, query_heads,
+                                   static_cast<const uint16_t *>(queries) + q * sequence_stride,
+                                   static_cast<uint16_t *>(output) + q * sequence_stride,
+                                   page_tables[q], &params[q], workspace, workspace_bytes, stream))
+      return rc;
+  return KVX_OK;
 }
 
 int kv_compact_path(const kvx_storage *s, uint32_t layer, const uint64_t *const *page_tables,

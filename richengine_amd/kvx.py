@@ -35,7 +35,7 @@ SYMBOLS = [
     "kvx_pool_acquire", "kvx_pool_retain", "kvx_pool_release", "kvx_pool_page_active",
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
     "kvx_pool_snapshot_get", "kv_append", "kv_prepare_append", "kv_attend_decode_shared", "kvx_attend_shared_workspace_bytes", "kv_attend_verify", "kv_attend_verify_hidden", "kv_attend_decode",
-    "kv_attend_prefill", "kv_compact_path", "kv_append_attend_decode", "kv_append_attend_decode_hidden", "kv_page_export", "kv_page_import", "kv_attend_split", "kv_attend_merge", "kv_attend_decode_static",
+    "kv_attend_prefill", "kv_attend_prefill_batch", "kv_compact_path", "kv_append_attend_decode", "kv_append_attend_decode_hidden", "kv_page_export", "kv_page_import", "kv_attend_split", "kv_attend_merge", "kv_attend_decode_static",
     "kvx_debug_attend_paths", "kvx_calibrate_stream", "kvx_decode_plan", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
     "kvx_prefix_chain", "kvx_prefix_retain_active", "kvx_prefix_release_active",
@@ -252,6 +252,7 @@ def _declare(L):
     L.kv_append_attend_decode_hidden.argtypes = [vp, u32, vp, vp, u64, u32, u32, vp, vp, vp, vp, u32, u32,
                                                  vp, u64, vp, vp, vp]
     L.kv_attend_prefill.argtypes = [vp, u32, u32, vp, vp, vp, C.POINTER(PrefillParams), vp, u64, vp]
+    L.kv_attend_prefill_batch.argtypes = [vp, u32, u32, vp, vp, vp, C.POINTER(PrefillParams), u32, u64, vp, u64, vp]
     L.kv_compact_path.argtypes = [vp, u32, vp, vp, u32, vp, vp, u32, vp]
 
 
@@ -512,6 +513,17 @@ def attend_prefill(storage, layer, query_heads, queries, output, table, params, 
                                          _ptr(workspace),
                                          workspace.numel() * workspace.element_size(),
                                          _stream(stream)))
+
+
+def attend_prefill_batch(storage, layer, query_heads, queries, output, tables, params,
+                         sequence_stride, workspace, stream=None):
+    """The chunks of several sequences in one call: sequence q's queries and rows begin
+    q x sequence_stride elements after the first's."""
+    arr = (PrefillParams * len(params))(*params)
+    return check(lib().kv_attend_prefill_batch(
+        storage.h, layer, query_heads, _ptr(queries), _ptr(output), _table_array(tables), arr,
+        len(params), sequence_stride, _ptr(workspace),
+        workspace.numel() * workspace.element_size(), _stream(stream)))
 
 
 def compact_path(storage, layer, tables, lanes, retained_path, retained_count, path_stride,

@@ -46,11 +46,13 @@ def tol(fmt):
     return 1e-2 if fmt == ko.FP8 else 2e-3
 
 
-def fill(tw, total, seed, layer=1, scale=1.0):
+def fill(tw, total, seed, layer=1, scale=1.0, pages=None):
     """Appends `total` tokens on the device (the path under test) and mirrors
     them into the oracle store by copying the device bytes back."""
     n_pages = (total + 31) // 32
-    pages = tw.pages(n_pages, seed)
+    if pages is None:
+        pages = tw.pages(n_pages, seed)
+    assert len(pages) == n_pages
     th, td = tw.tables(pages)
     rng = np.random.default_rng(seed)
     done = 0
