@@ -814,6 +814,314 @@ __global__ __launch_bounds__(kTileThreads) void prefill_split_kernel(
                             split, partials, statistics, slot_row, nullptr, p.score_scale);
 }
 
+// ---- head dimensions 64 and 128 on the matrix cores -------------------------
+// The same tile for the reference's narrower heads (its _hd128, _hd64, _k8q5d64 and
+// _k8q4d128 layouts, runtime/ops/PagedAttention.cpp:66-115), every format: the workgroup
+// stages a page's key and value codes in LDS as bf16 (fp16 on fp8 pages: the fp8 tile
+// multiplies fp16), which holds every code exactly, and each of its four waves multiplies
+// the blocks of 16 fused rows it owns (blocks w and w + 4) out of that copy with
+// v_mfma_f32_16x16x32: q.k as keys (16 tokens x 32 dims) x queries, p.v as values
+// (16 dims x 32 tokens) x probabilities.  A lane of q.k's result holds tokens 4g + j and
+// 16 + 4g + j of its row; the value operand is read from the staged copy in that token
+// order, so the rounded probabilities are the B operand of p.v as they stand.  Partial rows
+// and statistics go where attention_tile puts them, for the same reduce kernels.
+typedef float small_f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t small_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t small_u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 small_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 small_f16x8 __attribute__((ext_vector_type(8)));
+
+template <bool F16>
+__device__ __forceinline__ small_f32x4 small_mfma(small_u32x4 a, small_u32x4 b, small_f32x4 c) {
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(small_f16x8, a),
+                                                  __builtin_bit_cast(small_f16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(small_bf16x8, a),
+                                                   __builtin_bit_cast(small_bf16x8, b), c, 0, 0, 0);
+}
+// The 16 bits of x in the tile's operand format (x is exact in it, or is rounded to it).
+template <bool F16>
+__device__ __forceinline__ uint16_t operand_bits(float x) {
+  if constexpr (F16) return __builtin_bit_cast(uint16_t, _Float16(x));
+  else return f32_to_bf16(x);
+}
+
+constexpr uint32_t kSmallBlocks = 2;  // at most: blocks of 16 fused rows per wave, 128 rows per tile
+
+// Sixteen bytes of a page as they lie (32 int4 codes, 16 int8 or e4m3 codes, 8 bf16 values)
+// to that many 16-bit operand elements, in order: int4 and int8 codes as the bf16 numbers
+// they are (a small integer's float, cut to its upper half, is exact), e4m3 as fp16 (one
+// v_cvt_scalef32_pk_f16_fp8 per pair, exact), bf16 as it is.
+template <uint32_t FMT>
+struct SmallChunk {
+  static constexpr uint32_t kElements = FMT == KVX_FMT_INT4 ? 32 : FMT == KVX_FMT_BF16 ? 8 : 16;
+  uint32_t pair[kElements / 2];  // elements 2i (low half) and 2i + 1
+  __device__ __forceinline__ explicit SmallChunk(small_u32x4 raw) {
+    if constexpr (FMT == KVX_FMT_BF16) {
+#pragma unroll
+      for (uint32_t i = 0; i < 4; ++i) pair[i] = raw[i];
+    } else if constexpr (FMT == KVX_FMT_FP8E4M3) {
+#pragma unroll
+      for (uint32_t i = 0; i < 4; ++i) {
+        pair[2 * i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[i], 1.0f, false));
+        pair[2 * i + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[i], 1.0f, true));
+      }
+    } else if constexpr (FMT == KVX_FMT_INT8) {
+#pragma unroll
+      for (uint32_t i = 0; i < 8; ++i) {
+        const int lo = __builtin_amdgcn_sbfe(int(raw[i / 2]), 16 * (i & 1), 8);
+        const int hi = __builtin_amdgcn_sbfe(int(raw[i / 2]), 16 * (i & 1) + 8, 8);
+        pair[i] = (__float_as_uint(float(lo)) >> 16) | (__float_as_uint(float(hi)) & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (uint32_t i = 0; i < 16; ++i) {
+        const int lo = __builtin_amdgcn_sbfe(int(raw[i / 4]), 8 * (i & 3), 4);
+        const int hi = __builtin_amdgcn_sbfe(int(raw[i / 4]), 8 * (i & 3) + 4, 4);
+        pair[i] = (__float_as_uint(float(lo)) >> 16) | (__float_as_uint(float(hi)) & 0xffff0000u);
+      }
+    }
+  }
+};
+
+template <uint32_t FMT, uint32_t D, uint32_t BLOCKS>
+__device__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
+                                     const uint64_t *__restrict__ table, kvx_kv_layer kv,
+                                     uint32_t H, uint32_t G, uint32_t row_capacity, uint32_t head,
+                                     uint32_t committed, uint32_t active_rows, uint32_t splits,
+                                     uint32_t split, float *__restrict__ partials,
+                                     float *__restrict__ statistics, uint64_t slot_row,
+                                     const uint32_t *__restrict__ row_masks, float score_scale_in) {
+  constexpr bool kFp8 = FMT == KVX_FMT_FP8E4M3;
+  constexpr bool kQuant = FMT != KVX_FMT_BF16;
+  constexpr uint32_t kKeyRow = D + 8;        // staged halves per token: 16 bytes past a power of two
+  constexpr uint32_t kValueRow = kPage + 4;  // staged halves per dimension
+  constexpr uint32_t kSteps = D / 32, kTiles = D / 16;
+  __shared__ __align__(16) uint16_t k_lds[kPage * kKeyRow];
+  __shared__ __align__(16) uint16_t v_lds[D * kValueRow];
+  __shared__ float key_scale_lds[kPage], value_scale_lds[kPage];
+
+  const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, t = lane & 15u, g = lane >> 4;
+  const uint32_t M = row_capacity * G;
+  const uint32_t visible = committed + active_rows;
+  const uint32_t pages = (visible + kPage - 1) / kPage;
+  const uint32_t per = (pages + splits - 1) / splits;
+  const uint32_t begin = split * per;
+  if (begin >= pages) return;
+  const uint32_t end = min(pages, begin + per);
+  const float score_scale = default_score_scale(D, score_scale_in);
+  const bool tree = row_masks != nullptr;
+
+  small_u32x4 q[BLOCKS][kSteps];
+  small_f32x4 acc[BLOCKS][kTiles];
+  float row_max[BLOCKS], row_sum[BLOCKS];
+  uint32_t limit[BLOCKS], mask[BLOCKS], fused[BLOCKS];
+  bool live[BLOCKS], used[BLOCKS];
+#pragma unroll
+  for (uint32_t b = 0; b < BLOCKS; ++b) {
+    fused[b] = 16 * (wave + 4 * b) + t;
+    used[b] = 16 * (wave + 4 * b) < M;  // the same in every lane of the wave
+    const uint32_t query_row = fused[b] / G;
+    live[b] = fused[b] < M && query_row < active_rows;
+    limit[b] = live[b] ? min(visible, committed + min(query_row, active_rows - 1) + 1) : 0u;
+    mask[b] = (live[b] && tree) ? row_masks[query_row] : 0u;
+    row_max[b] = -INFINITY;
+    row_sum[b] = 0.0f;
+#pragma unroll
+    for (uint32_t i = 0; i < kTiles; ++i) acc[b][i] = small_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (uint32_t kb = 0; kb < kSteps; ++kb) {
+      small_u32x4 raw = {0u, 0u, 0u, 0u};
+      if (live[b])
+        raw = *reinterpret_cast<const small_u32x4 *>(tile_queries + uint64_t(fused[b]) * D + 32 * kb + 8 * g);
+      if constexpr (kFp8) {  // the fp8 tile stages its queries as fp16
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i)
+          raw[i] = uint32_t(operand_bits<true>(bf16_to_f32(uint16_t(raw[i])))) |
+                   uint32_t(operand_bits<true>(bf16_to_f32(uint16_t(raw[i] >> 16)))) << 16;
+      }
+      q[b][kb] = raw;
+    }
+  }
+
+  // A page's keys and values come in as whole 16-byte pieces, a piece (or two) per thread,
+  // one page ahead of the page being multiplied, and go to the staged copy as operand
+  // elements: keys [token][dim], values [dim][token].
+  using Chunk = SmallChunk<FMT>;
+  constexpr uint32_t kPieces = kPage * D / Chunk::kElements;         // per tensor
+  constexpr uint32_t kPerThread = (kPieces + kTileThreads - 1) / kTileThreads;
+  small_u32x4 raw_keys[kPerThread], raw_values[kPerThread];
+  float raw_scale = 1.0f;
+  const auto fetch = [&](uint32_t page) {
+    const Slab s = slab_of(FMT, H, D, kv, head, table[page]);
+#pragma unroll
+    for (uint32_t i = 0; i < kPerThread; ++i) {
+      const uint32_t piece = tid + i * kTileThreads;
+      if (kPieces % kTileThreads == 0 || piece < kPieces) {
+        raw_keys[i] = *reinterpret_cast<const small_u32x4 *>(s.keys + 16 * piece);
+        raw_values[i] = *reinterpret_cast<const small_u32x4 *>(s.values + 16 * piece);
+      }
+    }
+    if constexpr (kQuant)
+      if (tid < 2 * kPage) raw_scale = tid < kPage ? s.key_scales[tid] : s.value_scales[tid - kPage];
+  };
+  const auto stage = [&]() {
+#pragma unroll
+    for (uint32_t i = 0; i < kPerThread; ++i) {
+      const uint32_t piece = tid + i * kTileThreads;
+      if (kPieces % kTileThreads != 0 && piece >= kPieces) continue;
+      const uint32_t first = piece * Chunk::kElements;
+      {  // keys are token-major in every format
+        const Chunk c(raw_keys[i]);
+        uint32_t *to = reinterpret_cast<uint32_t *>(&k_lds[(first / D) * kKeyRow + first % D]);
+#pragma unroll
+        for (uint32_t w = 0; w < Chunk::kElements / 2; w += 4)
+          *reinterpret_cast<small_u32x4 *>(to + w) =
+              small_u32x4{c.pair[w], c.pair[w + 1], c.pair[w + 2], c.pair[w + 3]};
+      }
+      const Chunk c(raw_values[i]);
+      if constexpr (FMT == KVX_FMT_INT4) {  // token-major values: one element per staged row
+        const uint32_t token = first / D, d0 = first % D;
+#pragma unroll
+        for (uint32_t w = 0; w < Chunk::kElements / 2; ++w) {
+          v_lds[(d0 + 2 * w) * kValueRow + token] = uint16_t(c.pair[w]);
+          v_lds[(d0 + 2 * w + 1) * kValueRow + token] = uint16_t(c.pair[w] >> 16);
+        }
+      } else {  // dimension-major values: a run of tokens of one dimension
+        uint32_t *to = reinterpret_cast<uint32_t *>(&v_lds[(first / kPage) * kValueRow + first % kPage]);
+#pragma unroll
+        for (uint32_t w = 0; w < Chunk::kElements / 2; w += 2)
+          *reinterpret_cast<small_u32x2 *>(to + w) = small_u32x2{c.pair[w], c.pair[w + 1]};
+      }
+    }
+    if (tid < kPage) key_scale_lds[tid] = raw_scale;
+    else if (tid < 2 * kPage) value_scale_lds[tid - kPage] = raw_scale;
+  };
+
+  fetch(begin);
+  for (uint32_t page = begin; page < end; ++page) {
+    const uint32_t token_start = page * kPage;
+    __syncthreads();  // the previous page's products are done with the staged copy
+    stage();
+    if (page + 1 < end) fetch(page + 1);
+    __syncthreads();
+
+#pragma unroll
+    for (uint32_t b = 0; b < BLOCKS; ++b) {
+      if (!used[b]) continue;
+      small_f32x4 scores[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+#pragma unroll
+      for (uint32_t tb = 0; tb < 2; ++tb)
+#pragma unroll
+        for (uint32_t kb = 0; kb < kSteps; ++kb) {
+          const small_u32x4 keys =
+              *reinterpret_cast<const small_u32x4 *>(&k_lds[(16 * tb + t) * kKeyRow + 32 * kb + 8 * g]);
+          scores[tb] = small_mfma<kFp8>(keys, q[b][kb], scores[tb]);
+        }
+      // page softmax of the lane's eight tokens of its row (reference:
+      // common/paged_attention_tile.h:129-188)
+      float score[8], local_max = -INFINITY;
+      bool in[8];
+#pragma unroll
+      for (uint32_t i = 0; i < 8; ++i) {
+        const uint32_t token = 16 * (i >> 2) + 4 * g + (i & 3), at = token_start + token;
+        in[i] = live[b] && (tree ? (at < committed ||
+                                    (at < visible && ((mask[b] >> ((at - committed) & 31u)) & 1u)))
+                                 : at < limit[b]);
+        float v = scores[i >> 2][i & 3];
+        if constexpr (kQuant) v = __fmul_rn(v, key_scale_lds[token]);
+        v = __fmul_rn(v, score_scale);
+        score[i] = in[i] ? v : -INFINITY;
+        local_max = fmaxf(local_max, score[i]);
+      }
+      local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
+      local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
+      const float next_max = fmaxf(row_max[b], local_max);
+      const float rescale = (next_max == -INFINITY || next_max == row_max[b])
+                                ? 1.0f
+                                : expf(__fsub_rn(row_max[b], next_max));
+      float page_sum = 0.0f;
+      uint32_t bits[8];
+#pragma unroll
+      for (uint32_t i = 0; i < 8; ++i) {
+        const uint32_t token = 16 * (i >> 2) + 4 * g + (i & 3);
+        const float p = in[i] ? expf(__fsub_rn(score[i], next_max)) : 0.0f;
+        page_sum = __fadd_rn(page_sum, p);
+        float weight = 0.0f;
+        if (in[i] && score[i] > -INFINITY) weight = kQuant ? __fmul_rn(p, value_scale_lds[token]) : p;
+        bits[i] = operand_bits<kFp8>(weight);
+      }
+      row_sum[b] = __fadd_rn(__fmul_rn(row_sum[b], rescale), page_sum);
+      row_max[b] = next_max;
+      const small_u32x4 weights = {bits[0] | bits[1] << 16, bits[2] | bits[3] << 16,
+                                   bits[4] | bits[5] << 16, bits[6] | bits[7] << 16};
+      if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
+#pragma unroll
+        for (uint32_t i = 0; i < kTiles; ++i) acc[b][i] *= rescale;
+      }
+#pragma unroll
+      for (uint32_t i = 0; i < kTiles; ++i) {
+        const uint16_t *row = &v_lds[(16 * i + t) * kValueRow + 4 * g];
+        const small_u32x2 lo = *reinterpret_cast<const small_u32x2 *>(row);
+        const small_u32x2 hi = *reinterpret_cast<const small_u32x2 *>(row + 16);
+        acc[b][i] = small_mfma<kFp8>(small_u32x4{lo[0], lo[1], hi[0], hi[1]}, weights, acc[b][i]);
+      }
+    }
+  }
+
+#pragma unroll
+  for (uint32_t b = 0; b < BLOCKS; ++b) {
+    if (!used[b]) continue;
+    // the lanes of a row hold disjoint tokens
+    float sum = row_sum[b];
+    sum = __fadd_rn(sum, __shfl_xor(sum, 16));
+    sum = __fadd_rn(sum, __shfl_xor(sum, 32));
+    if (!live[b]) continue;
+    float *out = partials + (slot_row + fused[b]) * D + 4 * g;
+#pragma unroll
+    for (uint32_t i = 0; i < kTiles; ++i) *reinterpret_cast<small_f32x4 *>(out + 16 * i) = acc[b][i];
+    if (g == 0) {
+      statistics[(slot_row + fused[b]) * 2] = row_max[b];
+      statistics[(slot_row + fused[b]) * 2 + 1] = sum;
+    }
+  }
+}
+
+// BLOCKS = 1 (tiles of up to 64 fused rows) leaves registers for four waves per SIMD.
+template <uint32_t FMT, uint32_t D, uint32_t BLOCKS>
+__global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(BLOCKS == 1 ? 4 : 2, BLOCKS == 1 ? 4 : 2))) void attend_split_small_kernel(
+    const uint16_t *__restrict__ queries, float *__restrict__ partials,
+    float *__restrict__ statistics, const uint32_t *__restrict__ row_masks, AttendArgs a) {
+  const uint32_t split = blockIdx.x, head = blockIdx.y, li = blockIdx.z;
+  const AttendLane &l = a.lane[li];
+  if (!attend_contract(l, a) || split >= l.split_count) return;
+  const uint32_t M = a.row_capacity * a.group;
+  const uint16_t *tile_q = queries + l.q_offset + uint64_t(head) * a.row_stride * a.group * D;
+  const uint64_t slot_row = l.row_base + (uint64_t(head) * l.split_count + split) * M;
+  attention_tile_small<FMT, D, BLOCKS>(tile_q, l.table, a.kv, a.kv_heads, a.group, a.row_capacity, head,
+                               l.committed, l.active_rows, l.split_count, split, partials,
+                               statistics, slot_row,
+                               row_masks ? row_masks + l.mask_offset : nullptr, l.score_scale);
+}
+
+template <uint32_t FMT, uint32_t D, uint32_t BLOCKS>
+__global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(BLOCKS == 1 ? 4 : 2, BLOCKS == 1 ? 4 : 2))) void prefill_split_small_kernel(
+    const uint16_t *__restrict__ queries, float *__restrict__ partials,
+    float *__restrict__ statistics, PrefillArgs p) {
+  const uint32_t split = blockIdx.x, head = blockIdx.y, tile = blockIdx.z;
+  const uint32_t tile_start = tile * KVX_PREFILL_TILE_ROWS;
+  if (!prefill_contract(p) || tile_start >= p.rows) return;
+  const uint32_t active = min(KVX_PREFILL_TILE_ROWS, p.rows - tile_start);
+  const uint32_t M = KVX_PREFILL_TILE_ROWS * p.group;
+  const uint64_t tile_offset = (uint64_t(head) * p.stride + tile_start) * p.group * D;
+  const uint64_t slot_row = ((uint64_t(tile) * p.kv_heads + head) * p.splits + split) * M;
+  attention_tile_small<FMT, D, BLOCKS>(queries + tile_offset, p.table, p.kv, p.kv_heads, p.group,
+                               KVX_PREFILL_TILE_ROWS, head, p.committed + tile_start, active,
+                               p.splits, split, partials, statistics, slot_row, nullptr,
+                               p.score_scale);
+}
+
 // Fixed-order merge of one fused row's splits (reference:
 // common/paged_attention_tile.h:362-417).  head_dim threads, one per dimension;
 // returns the thread's bf16 element, zero for rows past the live ones.
@@ -1540,7 +1848,21 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
       max_splits = std::max(max_splits, p.split_count);
     }
     int rc = KVX_OK;
-    if (phases & 1u)
+    if ((phases & 1u) && (D == 64 || D == 128) && M <= 64 * kSmallBlocks)
+      rc = dispatch_format(l.format, [&](auto fmt) {
+        // head dimensions 64 and 128: the tile on the matrix cores
+        const auto launch = [&](auto kernel) {
+          hipLaunchKernelGGL(kernel, dim3(max_splits, H, a.n_lanes), dim3(kTileThreads), 0, stream,
+                             static_cast<const uint16_t *>(queries), partials, statistics, row_masks, a);
+        };
+        constexpr uint32_t F = decltype(fmt)::value;
+        if (D == 64 && M <= 64) launch(attend_split_small_kernel<F, 64, 1>);
+        else if (D == 64) launch(attend_split_small_kernel<F, 64, 2>);
+        else if (M <= 64) launch(attend_split_small_kernel<F, 128, 1>);
+        else launch(attend_split_small_kernel<F, 128, 2>);
+        return check_launch("attend_split_small_kernel");
+      });
+    else if (phases & 1u)
       rc = dispatch_format(l.format, [&](auto fmt) {
         return dispatch_rows(M, [&](auto maxm) {
           hipLaunchKernelGGL((attend_split_kernel<decltype(fmt)::value, decltype(maxm)::value>),
@@ -2109,7 +2431,21 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
   PrefillArgs p{page_table, params->committed_tokens, params->rows, params->chunk_stride,
                 params->page_table_entries, params->split_count, H, G, D,
                 params->score_scale != 0.0f ? params->score_scale : l.score_scale, kv};
-  int rc = dispatch_format(l.format, [&](auto fmt) {
+  int rc = KVX_OK;
+  if ((D == 64 || D == 128) && M <= 64 * kSmallBlocks)
+    rc = dispatch_format(l.format, [&](auto fmt) {
+      const auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(params->split_count, H, tiles), dim3(kTileThreads), 0, st,
+                           static_cast<const uint16_t *>(queries), partials, statistics, p);
+      };
+      constexpr uint32_t F = decltype(fmt)::value;
+      if (D == 64 && M <= 64) launch(prefill_split_small_kernel<F, 64, 1>);
+      else if (D == 64) launch(prefill_split_small_kernel<F, 64, 2>);
+      else if (M <= 64) launch(prefill_split_small_kernel<F, 128, 1>);
+      else launch(prefill_split_small_kernel<F, 128, 2>);
+      return check_launch("prefill_split_small_kernel");
+    });
+  else rc = dispatch_format(l.format, [&](auto fmt) {
     return dispatch_rows(M, [&](auto maxm) {
       hipLaunchKernelGGL((prefill_split_kernel<decltype(fmt)::value, decltype(maxm)::value>),
                          dim3(params->split_count, H, tiles), dim3(kTileThreads), 0, st,

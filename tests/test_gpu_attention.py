@@ -424,34 +424,44 @@ def test_invalid_attention_parameters_enqueue_nothing():
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
-@pytest.mark.parametrize("heads,group,dim", [(2, 3, 128), (4, 6, 128), (3, 2, 64)])
+@pytest.mark.parametrize("heads,group,dim", [(2, 3, 128), (4, 6, 128), (3, 2, 64), (2, 8, 128), (8, 4, 64),
+                                              (1, 20, 256)])
 def test_generic_kernels_cover_other_shapes(fmt, heads, group, dim):
-    """Head dimensions other than 256: chunked
-    prefill, chain verify and decode on the format-generic kernels, which keep
-    the oracle's operation order (nearly every output has the oracle's bits)."""
+    """Head dimensions other than 256: chunked prefill, chain verify and decode.  64 and 128
+    (the reference's other layouts, 2 x 8 x 128 and 8 x 4 x 64 among them) run the tile on the
+    matrix cores out of a staged copy of the page; anything else (here a group of 20 query
+    heads, whose tiles of 8 rows would exceed 128 fused rows: verify of 6 rows and decode only)
+    runs on the format-generic kernels, which keep the oracle's operation order (nearly every
+    output has the oracle's bits)."""
+    in_order = dim not in (64, 128)
     committed, rows = 300, 13
     tw = Gp.Twin(fmt, heads, dim, 2, (committed + rows + 31) // 32)
     pages, th, td = fill(tw, committed + rows, seed=dim + heads)
     tw.assert_same_bytes()
     qh = heads * group
-    # prefill
-    q = np.zeros((heads, 32, group, dim), dtype=np.uint16)
-    q[:, :rows] = queries((heads, rows, group, dim), dim)
-    splits = kvx.lib().kvx_prefill_splits(rows)
-    hp = ko.PrefillParams(committed, rows, 32, len(pages), tw.host.layer(1), splits, 0.0)
-    ok, want, want32 = ko.attend_prefill(fmt, heads, group, dim, q, th, hp)
-    assert ok == 1
-    out = torch.zeros((heads, 32, group, dim), dtype=torch.int16, device="cuda")
-    ws = torch.empty(kvx.prefill_workspace_bytes(tw.dev, rows, qh), dtype=torch.uint8, device="cuda")
-    kvx.attend_prefill(tw.dev, 1, qh, Gp.dev(q), out, td,
-                       kvx.PrefillParams(committed, rows, 32, len(pages), kvx.KvLayer(), splits, 0.0), ws)
-    torch.cuda.synchronize()
-    live = np.zeros((heads, 32), dtype=bool)
-    live[:, :rows] = True
-    stats = Gp.check_attention(Gp.host_u16(out), want, want32, live, tol(fmt), f"generic prefill {fmt}")
-    assert stats["exact"] > 0.98
-    # chain verify of 8 rows and one-row decode over the same pages
-    for active, capacity, row_stride in ((8, 8, 32), (1, 1, 1)):
+    chain = min(8, 128 // group)
+    # prefill (a tile is 8 rows x group fused rows, 128 at most)
+    if 8 * group <= 128:
+        q = np.zeros((heads, 32, group, dim), dtype=np.uint16)
+        q[:, :rows] = queries((heads, rows, group, dim), dim)
+        splits = kvx.lib().kvx_prefill_splits(rows)
+        hp = ko.PrefillParams(committed, rows, 32, len(pages), tw.host.layer(1), splits, 0.0)
+        ok, want, want32 = ko.attend_prefill(fmt, heads, group, dim, q, th, hp)
+        assert ok == 1
+        out = torch.zeros((heads, 32, group, dim), dtype=torch.int16, device="cuda")
+        ws = torch.empty(kvx.prefill_workspace_bytes(tw.dev, rows, qh), dtype=torch.uint8, device="cuda")
+        kvx.attend_prefill(tw.dev, 1, qh, Gp.dev(q), out, td,
+                           kvx.PrefillParams(committed, rows, 32, len(pages), kvx.KvLayer(), splits, 0.0), ws)
+        torch.cuda.synchronize()
+        live = np.zeros((heads, 32), dtype=bool)
+        live[:, :rows] = True
+        stats = Gp.check_attention(Gp.host_u16(out), want, want32, live, tol(fmt), f"generic prefill {fmt}",
+                                   explain=None if in_order else Gp.prefill_explainer(
+                                       fmt, heads, group, dim, q, th, tw.host.layer(1), committed, rows, splits))
+        assert stats["exact"] > 0.98 or not in_order
+        assert stats["rel_l2_mean"] < 5e-4
+    # chain verify of 8 rows (6 for the group of 20) and one-row decode over the same pages
+    for active, capacity, row_stride in ((chain, chain, 32), (1, 1, 1)):
         visible = committed + active
         q = np.zeros((1, heads, row_stride, group, dim), dtype=np.uint16)
         q[:, :, :active] = queries((1, heads, active, group, dim), active)
@@ -473,7 +483,10 @@ def test_generic_kernels_cover_other_shapes(fmt, heads, group, dim):
         live = np.zeros((1, heads, row_stride), dtype=bool)
         live[:, :, :active] = True
         Gp.check_attention(Gp.host_u16(out), want[:, :, :row_stride], want32[:, :, :row_stride], live,
-                           tol(fmt), f"generic rows={active} fmt={fmt}")
+                           tol(fmt), f"generic rows={active} fmt={fmt}",
+                           explain=None if in_order else Gp.lanes_explainer(
+                               fmt, heads, group, dim, qo, [th], tw.host.layer(1), [committed], [active],
+                               [splits], capacity))
     tw.close()
 
 
