@@ -151,11 +151,16 @@ uint32_t kvx_prefill_splits(uint32_t rows);
    floor would only add partial traffic. */
 #define KVX_DECODE_PAGES_PER_SPLIT 32u
 uint32_t kvx_decode_splits(uint32_t committed_tokens, uint32_t rows);
-/* The split counts of a whole decode batch of pages of `format`.  A launch runs (sum of splits) x
+/* The split counts of a whole decode batch of pages of `format`, planned launch by launch: the
+   attend calls take the lanes KVX_LANES_PER_LAUNCH at a time in the caller's order, and every
+   such group is planned to fill the GPU by itself.  A launch runs (sum of splits) x
    KV heads waves; the plan is a split length in pages, each lane getting
    clamp(ceil(its pages / that), 1, KVX_DECODE_MAX_SPLITS) splits.  The length starts at
-   max(ceil(total page-heads / 1024), 8) (at most 32 for int4, whose kernel holds two waves per
-   SIMD and is fastest at 32), which fills the GPU when the batch is small, and grows until the
+   max(ceil(the launch's page-heads / 1024), 8) (at most 32 for int4, whose kernel holds two waves per
+   SIMD and is fastest at 32; at least 4 instead of 8 for a launch of at most 4096 page-heads
+   on int4 pages, 2048 on the others, whose longest lane has at most 512 pages: splits of 8
+   pages would leave most SIMDs of such a launch empty),
+   which fills the GPU when the batch is small, and grows until the
    launch has no more waves than the kernel has wave slots (2048 for int4, 1024 for the other
    formats), because waves beyond that run as a second round on a nearly empty GPU.  An int4
    batch of at most KVX_LANES_PER_LAUNCH lanes that needs two waves on most SIMDs is planned in
@@ -171,11 +176,12 @@ uint32_t kvx_decode_splits(uint32_t committed_tokens, uint32_t rows);
 int kvx_decode_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t kv_heads,
                     uint32_t format, uint32_t *split_counts);
 /* Split counts of a verify batch (`rows` live rows per lane) sized for this GPU instead of
-   the reference's clamp(ceil(pages/16), 32, 128): the longest split length (at least 8 pages)
+   the reference's clamp(ceil(pages/16), 32, 128), launch by launch like kvx_decode_plan: the
+   longest split length (at least 8 pages)
    for which the launch has no more waves than the GPU has SIMDs (1024), each lane getting
    clamp(ceil(its pages / that), 1, KVX_VERIFY_MAX_SPLITS).  A launch runs (sum of splits) x
    KV heads x ceil(rows x group / 32) waves, one per SIMD; on int4 pages ceil(rows x group / 48)
-   where that is fewer by more than two fifths (33 .. 48 and 65 .. 96 fused rows among others).  No counterpart in the reference
+   where that is fewer by more than 1.74 (33 .. 48 fused rows among others).  No counterpart in the reference
    (its rule is kvx_verify_splits); any split count either rule gives is valid for
    kv_attend_verify. */
 int kvx_verify_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t rows,

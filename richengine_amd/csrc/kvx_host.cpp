@@ -204,13 +204,17 @@ uint32_t kvx_decode_splits(uint32_t committed, uint32_t rows) {
   const uint32_t wanted = (pages + KVX_DECODE_PAGES_PER_SPLIT - 1) / KVX_DECODE_PAGES_PER_SPLIT;
   return std::min(std::max(1u, wanted), KVX_VERIFY_MAX_SPLITS);
 }
-int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_heads, uint32_t format,
-                    uint32_t *split_counts) {
-  if (!committed || !split_counts || !n_lanes || !kv_heads)
-    return fail(KVX_EINVAL, "kvx_decode_plan: null argument or empty batch");
+// The decode plan of the lanes of one launch (at most KVX_LANES_PER_LAUNCH).
+static void decode_plan_of_launch(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_heads,
+                                  uint32_t format, uint32_t *split_counts) {
   // A launch runs (sum of splits) x KV heads waves.  One per SIMD of 256 CUs x 4
   // is the least that fills the GPU; shorter splits than 8 pages cost more in
-  // set-up and partial rows than they win.  What must not happen is a launch
+  // set-up and partial rows than they win, except in a launch so small that splits of 8
+  // pages leave half of the SIMDs empty (three quarters where the kernel runs one wave per
+  // SIMD): there splits go down to 4 pages, unless that gives a lane more than 128 of them
+  // to merge (one sequence of 8192 tokens: int4 21.1 -> 16.1, int8 24.0 -> 17.9, bf16 21.6 ->
+  // 16.8 us; 2048 tokens, batches of 1 to 4: 19 -> 15, 22 -> 16, 19 -> 15 us; one sequence
+  // of 32768 tokens loses 5 % to the longer merge).  What must not happen is a launch
   // with more waves than the kernel has wave slots: the overflow runs as a second
   // round on a nearly empty GPU (measured on 530 K tokens: int4 146 -> 115 us,
   // bf16 397 -> 350 us once the waves fit).  The int4 kernel holds two waves per
@@ -223,7 +227,11 @@ int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_hea
     pages[i] = pages_of(uint64_t(committed[i]) + 1);
     page_heads += uint64_t(pages[i]) * kv_heads;
   }
-  uint32_t per = uint32_t(std::max<uint64_t>((page_heads + kSimds - 1) / kSimds, 8));
+  uint32_t longest_lane = 0;
+  for (uint32_t i = 0; i < n_lanes; ++i) longest_lane = std::max(longest_lane, pages[i]);
+  const uint64_t small_launch = format == KVX_FMT_INT4 ? 4 * kSimds : 2 * kSimds;  // page-heads
+  const uint64_t shortest = (page_heads <= small_launch && longest_lane <= 512) ? 4 : 8;
+  uint32_t per = uint32_t(std::max<uint64_t>((page_heads + kSimds - 1) / kSimds, shortest));
   if (format == KVX_FMT_INT4) per = std::min(per, KVX_DECODE_PAGES_PER_SPLIT);
   uint64_t waves = 0;
   for (;; ++per) {
@@ -236,7 +244,7 @@ int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_hea
     }
     if (waves <= slots || single) break;  // one split per lane is the fewest waves there can be
   }
-  if (format != KVX_FMT_INT4 || n_lanes > KVX_LANES_PER_LAUNCH || waves <= kSimds) return KVX_OK;
+  if (format != KVX_FMT_INT4 || waves <= kSimds) return;
   // int4, a launch with two waves on most SIMDs.  The two do not share their SIMD evenly:
   // the wave that was dispatched first runs ahead of the other (measured on splits of equal
   // length: 2.05 against 3.9 us per page while both run), ends a quarter of the launch early
@@ -274,13 +282,23 @@ int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_hea
       break;
     }
   }
+}
+int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_heads, uint32_t format,
+                    uint32_t *split_counts) {
+  if (!committed || !split_counts || !n_lanes || !kv_heads)
+    return fail(KVX_EINVAL, "kvx_decode_plan: null argument or empty batch");
+  // The attend calls take the lanes KVX_LANES_PER_LAUNCH at a time, in the caller's order,
+  // and the launches follow one another: every launch is planned to fill the GPU by itself
+  // (a batch of 128 sequences of 8192 tokens planned as one: 341 us; launch by launch: 220).
+  for (uint32_t first = 0; first < n_lanes; first += KVX_LANES_PER_LAUNCH)
+    decode_plan_of_launch(committed + first, std::min(KVX_LANES_PER_LAUNCH, n_lanes - first), kv_heads,
+                          format, split_counts + first);
   return KVX_OK;
 }
-int kvx_verify_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t rows, uint32_t kv_heads,
-                    uint32_t query_heads, uint32_t format, uint32_t *split_counts) {
-  if (!committed || !split_counts || !n_lanes || !kv_heads || !rows || !query_heads ||
-      query_heads % kv_heads)
-    return fail(KVX_EINVAL, "kvx_verify_plan: null argument, empty batch or bad head counts");
+// The verify plan of the lanes of one launch (at most KVX_LANES_PER_LAUNCH).
+static void verify_plan_of_launch(const uint32_t *committed, uint32_t n_lanes, uint32_t rows,
+                                  uint32_t kv_heads, uint32_t query_heads, uint32_t format,
+                                  uint32_t *split_counts) {
   // The verify kernels keep 32 fused rows (16 when there are no more; all of 33 .. 48
   // on int4 pages) per wave and run one wave per SIMD, so a launch is (sum of splits) x KV heads x row blocks
   // waves: the plan is the longest split length that still gives every SIMD of
@@ -307,6 +325,16 @@ int kvx_verify_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t rows, 
     for (uint32_t i = 0; i < n_lanes; ++i) single = single && split_counts[i] == 1;
     if (single) break;
   }
+}
+int kvx_verify_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t rows, uint32_t kv_heads,
+                    uint32_t query_heads, uint32_t format, uint32_t *split_counts) {
+  if (!committed || !split_counts || !n_lanes || !kv_heads || !rows || !query_heads ||
+      query_heads % kv_heads)
+    return fail(KVX_EINVAL, "kvx_verify_plan: null argument, empty batch or bad head counts");
+  // launch by launch, as kvx_decode_plan
+  for (uint32_t first = 0; first < n_lanes; first += KVX_LANES_PER_LAUNCH)
+    verify_plan_of_launch(committed + first, std::min(KVX_LANES_PER_LAUNCH, n_lanes - first), rows,
+                          kv_heads, query_heads, format, split_counts + first);
   return KVX_OK;
 }
 int kvx_chunk_validation(const kvx_chunk_params *p) {

@@ -122,60 +122,76 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
     rng = np.random.default_rng(3)
     H, QH = 4, 24
     pages = lambda tokens: (tokens + 31) // 32
-    for trial in range(40):
-        lanes = int(rng.integers(1, 40))
-        committed = [int(x) for x in rng.integers(0, 70000, lanes)]
+    def decode_rule(committed, fmt, slots):
+        """The rule for the lanes of one launch, restated."""
+        lanes = len(committed)
         heads_pages = sum(pages(c + 1) for c in committed) * H
+        small = heads_pages <= (4096 if fmt == kvx.INT4 else 2048) and max(pages(c + 1) for c in committed) <= 512
+        per = max(-(-heads_pages // 1024), 4 if small else 8)
+        if fmt == kvx.INT4:
+            per = min(per, 32)
+        while True:  # the first length whose waves fit the kernel's slots
+            want = [min(max(1, -(-pages(c + 1) // per)), 512) for c in committed]
+            if sum(want) * H <= slots or all(s == 1 for s in want):
+                break
+            per += 1
+        if fmt == kvx.INT4 and sum(want) * H > 1024:
+            # two waves on most SIMDs: long splits for exactly the first wave of every
+            # SIMD, from the longest lane down while they fit, and splits of 0.58
+            # of that length for the second waves; the least long length that fits
+            counts = [pages(c + 1) for c in committed]
+            order = sorted(range(lanes), key=lambda i: -counts[i])
+            for longer in range(8, 8200):
+                shorter = max(4, int(0.58 * longer))
+                first = second = 0
+                want = [0] * lanes
+                for i in order:
+                    as_long = -(-counts[i] // longer)
+                    if first + as_long * H <= 1024:
+                        want[i], first = as_long, first + as_long * H
+                    else:
+                        want[i] = -(-counts[i] // shorter)
+                        second += want[i] * H
+                if second <= 1024 and max(want) <= 512:
+                    break
+            assert first <= 1024 and second <= 1024
+        return want
+
+    def verify_rule(committed, rows, fmt):
+        fused = rows * (QH // H)
+        blocks = -(-fused // 32) if fused > 16 else 1
+        if fmt != kvx.INT4 and 64 < fused <= 128:
+            blocks = 4                             # waves of a workgroup that shares its pages
+            if fmt == kvx.BF16 and fused <= 96:
+                blocks = 2                         # two waves of 48 rows
+        if fmt == kvx.INT4 and fused > 16 and 26 * -(-fused // 48) < 15 * -(-fused // 32):
+            blocks = -(-fused // 48)  # the int4 kernel for 48 fused rows per wave
+        counts = [pages(c + rows) for c in committed]
+        per = max(-(-sum(counts) * H * blocks // 1024), 8)
+        while True:  # the first length that fits one round of waves
+            want = [min(max(1, -(-n // per)), 128) for n in counts]
+            if sum(want) * H * blocks <= 1024 or all(s == 1 for s in want):
+                break
+            per += 1
+        return want
+
+    for trial in range(40):
+        lanes = int(rng.integers(1, 100))   # past 32 lanes: several launches, each planned alone
+        top = int(rng.choice([300, 4000, 70000]))
+        committed = [int(x) for x in rng.integers(0, top, lanes)]
+        groups = [committed[i:i + 32] for i in range(0, lanes, 32)]
         for fmt, slots in ((kvx.INT4, 2048), (kvx.INT8, 1024), (kvx.BF16, 1024), (kvx.FP8, 1024)):
             plan = kvx.decode_plan(committed, H, fmt)
-            per = max(-(-heads_pages // 1024), 8)
-            if fmt == kvx.INT4:
-                per = min(per, 32)
-            while True:  # the rule, restated: the first length whose waves fit the kernel's slots
-                want = [min(max(1, -(-pages(c + 1) // per)), 512) for c in committed]
-                if sum(want) * H <= slots or all(s == 1 for s in want):
-                    break
-                per += 1
-            if fmt == kvx.INT4 and lanes <= 32 and sum(want) * H > 1024:
-                # two waves on most SIMDs: long splits for exactly the first wave of every
-                # SIMD, from the longest lane down while they fit, and splits of 0.58
-                # of that length for the second waves; the least long length that fits
-                counts = [pages(c + 1) for c in committed]
-                order = sorted(range(lanes), key=lambda i: -counts[i])
-                for longer in range(8, 8200):
-                    shorter = max(4, int(0.58 * longer))
-                    first = second = 0
-                    want = [0] * lanes
-                    for i in order:
-                        as_long = -(-counts[i] // longer)
-                        if first + as_long * H <= 1024:
-                            want[i], first = as_long, first + as_long * H
-                        else:
-                            want[i] = -(-counts[i] // shorter)
-                            second += want[i] * H
-                    if second <= 1024 and max(want) <= 512:
-                        break
-                assert first <= 1024 and second <= 1024
-            assert plan == want
+            assert plan == sum((decode_rule(g, fmt, slots) for g in groups), [])
         for rows, fmt in ((2, kvx.INT4), (8, kvx.INT4), (8, kvx.INT8), (16, kvx.INT4), (16, kvx.BF16)):
             plan = kvx.verify_plan(committed, rows, H, QH, fmt)
-            fused = rows * (QH // H)
-            blocks = -(-fused // 32) if fused > 16 else 1
-            if fmt != kvx.INT4 and 64 < fused <= 128:
-                blocks = 4                             # waves of a workgroup that shares its pages
-                if fmt == kvx.BF16 and fused <= 96:
-                    blocks = 2                         # two waves of 48 rows
-            if fmt == kvx.INT4 and fused > 16 and 26 * -(-fused // 48) < 15 * -(-fused // 32):
-                blocks = -(-fused // 48)  # the int4 kernel for 48 fused rows per wave
+            assert plan == sum((verify_rule(g, rows, fmt) for g in groups), [])
             counts = [pages(c + rows) for c in committed]
-            per = max(-(-sum(counts) * H * blocks // 1024), 8)
-            while True:  # the rule, restated: the first length that fits one round of waves
-                want = [min(max(1, -(-n // per)), 128) for n in counts]
-                if sum(want) * H * blocks <= 1024 or all(s == 1 for s in want):
-                    break
-                per += 1
-            assert plan == want
             assert all(1 <= s <= 128 and s <= max(n, 1) for s, n in zip(plan, counts))
+    # a small launch takes shorter splits: one sequence of 8192 tokens, 64 splits of 4 pages
+    assert kvx.decode_plan([8191], H, kvx.INT4) == [64] and kvx.decode_plan([8191], H, kvx.INT8) == [64]
+    assert kvx.decode_plan([8191] * 3, H, kvx.INT4) == [64] * 3 and kvx.decode_plan([8191] * 3, H, kvx.BF16) == [32] * 3
+    assert kvx.decode_plan([32767], H, kvx.INT4) == [128]   # 256 splits would be too many to merge
     # chunked prefill: one split while the paired tiles fill half of the wave slots, else the
     # largest count whose one-tile lanes fit one round (and leave 8 pages per split)
     for fmt in (kvx.INT4, kvx.INT8, kvx.FP8, kvx.BF16):
