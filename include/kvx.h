@@ -177,8 +177,11 @@ int kvx_decode_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t
                     uint32_t format, uint32_t *split_counts);
 /* Split counts of a verify batch (`rows` live rows per lane) sized for this GPU instead of
    the reference's clamp(ceil(pages/16), 32, 128), launch by launch like kvx_decode_plan: the
-   longest split length (at least 8 pages)
-   for which the launch has no more waves than the GPU has SIMDs (1024), each lane getting
+   longest split length (at least 8 pages; 4 in a launch of at most 2048 page-waves whose
+   longest lane has at most 512 pages)
+   for which the launch has no more waves than the GPU has SIMDs (1024; 2048 for int4 lanes of
+   more than 32 fused rows in blocks of 32 from 16 lanes on, whose kernel holds two waves per
+   SIMD), each lane getting
    clamp(ceil(its pages / that), 1, KVX_VERIFY_MAX_SPLITS).  A launch runs (sum of splits) x
    KV heads x ceil(rows x group / 32) waves, one per SIMD; on int4 pages ceil(rows x group / 48)
    where that is fewer by more than 1.74 (33 .. 48 fused rows among others).  No counterpart in the reference

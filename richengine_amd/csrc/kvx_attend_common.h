@@ -371,7 +371,8 @@ __global__ __launch_bounds__(64 * WAVES) void matrix_merge_kernel(
 
 // Launches a split kernel over (work items, KV heads, column blocks) and then
 // the merge of the lanes that have more than one split.  `columns` is how many
-// fused query rows one workgroup of the split kernel covers.  Returns 1
+// fused query rows one workgroup of the split kernel covers (one wave of it where a
+// workgroup is waves_per_group independent waves, each a work item).  Returns 1
 // (declined) when the workspace cannot hold the aligned layout, 0 when
 // enqueued, or a negative status.
 template <class SplitKernel>
@@ -383,7 +384,7 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
                             uint64_t lane_stride, void *workspace, uint64_t workspace_bytes,
                             hipStream_t stream, const FusedAppend *fused = nullptr,
                             Tiles tile_rows = 0, const Epilogue *epilogue = nullptr,
-                            bool longest_first = false) {
+                            bool longest_first = false, uint32_t waves_per_group = 1) {
   const bool run_split = !(epilogue && epilogue->merge_only);
   const bool run_merge = !(epilogue && epilogue->partials_only);
   const kvx_layout &l = s->layout;
@@ -480,7 +481,8 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
     if (run_split) {
       const uint32_t column_blocks = (M + columns - 1) / columns;
       hipLaunchKernelGGL(split_kernel,
-                         a.item_major ? dim3(H, items, column_blocks) : dim3(items, H, column_blocks),
+                         a.item_major ? dim3(H, items, column_blocks)
+                                      : dim3((items + waves_per_group - 1) / waves_per_group, H, column_blocks),
                          dim3(threads), 0, stream, static_cast<const uint16_t *>(queries),
                          static_cast<uint16_t *>(output), partials, statistics, a);
       const hipError_t e = hipGetLastError();

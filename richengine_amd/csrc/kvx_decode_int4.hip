@@ -530,7 +530,13 @@ __device__ __forceinline__ void write_blocks(const State *st, const uint32_t *m,
 // kItemMajor: the launch has its work items in the grid's y and the KV heads in x
 // (DecodeArgs::item_major), and its lanes are plain lane records, never the regular tiles of a
 // prefill.
-template <uint32_t NB, uint32_t kDepth, bool kReused = false, bool kItemMajor = false>
+// kQuad: workgroups of four waves, each wave a work item of its own (items 4 x .. 4 x + 3); the
+// waves share nothing.  A kernel built for two waves per SIMD but launched with at most one
+// wave per SIMD is not always given one SIMD per wave: after another kernel the dispatcher has
+// put two single-wave workgroups on one SIMD of a CU and none on its neighbour (38 of 960
+// SIMDs, the launch 157 instead of 121 us).  The four waves of one workgroup go to the four
+// SIMDs of its CU.
+template <uint32_t NB, uint32_t kDepth, bool kReused = false, bool kItemMajor = false, bool kQuad = false>
 __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries,
                                             uint16_t *__restrict__ output,
                                             float *__restrict__ partials,
@@ -541,7 +547,8 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   // register file: they hold their tiles transposed, which needs the rescaling for a quarter
   // of a tile's registers on a fifth of the pages instead of all of them on half.
   constexpr bool kRowsDown = NB == 2 && kDepth == 1;
-  const uint32_t item = kItemMajor ? blockIdx.y : blockIdx.x;
+  const uint32_t wave = kQuad ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0u;
+  const uint32_t item = kItemMajor ? blockIdx.y : kQuad ? 4 * blockIdx.x + wave : blockIdx.x;
   const uint32_t head = kItemMajor ? blockIdx.x : blockIdx.y;
   uint32_t li;
   DecodeLane l;
@@ -620,7 +627,7 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   if (begin >= pages) return;
   const uint32_t end = min(pages, begin + per);
 
-  const uint32_t lane = threadIdx.x, t = lane & 15, g = lane >> 4;
+  const uint32_t lane = kQuad ? threadIdx.x & 63u : threadIdx.x, t = lane & 15, g = lane >> 4;
   const uint32_t H = a.kv_heads, G = a.group, M = a.fused_rows;
   // The wave that owns the sequence's last page stores the step's token: before
   // anything else when that page is among the first fills, otherwise behind them,
@@ -720,7 +727,8 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   // Register kb of the staged queries holds the 8 dims of dword
   // w = 16*(kb>>2) + 4g + (kb&3) of a key row in expansion order; odd dims are
   // negated.  q_bias is the constant part of every score.
-  __shared__ u32x4 q_lds[NB][8 * 64];
+  __shared__ u32x4 q_lds_all[kQuad ? 4 : 1][NB][8 * 64];
+  u32x4 (&q_lds)[NB][8 * 64] = q_lds_all[wave];
   float q_bias[NB];
 #pragma unroll
   for (uint32_t nb = 0; nb < NB; ++nb) {
@@ -839,10 +847,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 // register file, where its rescaling costs one instruction a register instead of three;
 // per block and page it issues 235 vector instructions where the three-block kernel
 // issues 268, and a wave's vector instructions are what these kernels wait for.
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void verify32_int4_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void verify32_int4_kernel(
     const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
     float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
-  attend_int4<2, 1, false>(queries, output, partials, statistics, a);
+  attend_int4<2, 1, false, false, true>(queries, output, partials, statistics, a);
 }
 
 // Three blocks (48 fused rows: a chain of 8 rows for a group of 6 query heads, half
@@ -941,10 +949,10 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
                                    stream, nullptr, tile_rows, epilogue);
   if (fused_rows > 32 && !many_tiles)
-    return launch_matrix_attention(verify32_int4_kernel, "verify32_int4_kernel", 32, 64, s, kv,
+    return launch_matrix_attention(verify32_int4_kernel, "verify32_int4_kernel", 32, 256, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
-                                   stream, nullptr, tile_rows, epilogue);
+                                   stream, nullptr, tile_rows, epilogue, false, /*waves_per_group=*/4);
   if (fused_rows > 16 && !many_tiles)
     return launch_matrix_attention(verify_int4_kernel, "verify_int4_kernel", 32, 64, s, kv,
                                    query_heads, queries, output, page_tables, lanes, n_lanes,

@@ -305,13 +305,26 @@ static void verify_plan_of_launch(const uint32_t *committed, uint32_t n_lanes, u
   // 256 CUs x 4 a wave, but no more waves than SIMDs, so that no second round of
   // waves starts on a nearly empty GPU; splits shorter than 8 pages cost more in
   // set-up and partial rows than they win.
-  constexpr uint64_t kSimds = 1024;
   const uint32_t fused = rows * (query_heads / kv_heads);
   const uint32_t blocks = kvx::verify_row_blocks(format, fused);
+  // The int4 kernel for lanes of more than 32 fused rows in blocks of 32 is built for two
+  // waves per SIMD, and from 16 lanes on a launch is faster with them (16 lanes of 8192
+  // tokens, 16 rows: 134 -> 118 us; 32 lanes of 4096: 152 -> 123 us); with fewer, longer
+  // lanes the second wave's partial rows cost what it gains (4 lanes of 32768: 114 -> 131).
+  const bool two_per_simd = format == KVX_FMT_INT4 && fused > 32 &&
+                            kvx::verify_block_rows(format, fused) == 32 && n_lanes >= 16;
+  const uint64_t kSimds = two_per_simd ? 2048 : 1024;
   uint64_t page_waves = 0;
   for (uint32_t i = 0; i < n_lanes; ++i)
     page_waves += uint64_t(pages_of(uint64_t(committed[i]) + rows)) * kv_heads * blocks;
-  uint32_t per = uint32_t(std::max<uint64_t>((page_waves + kSimds - 1) / kSimds, 8));
+  // A launch that splits of 8 pages would spread over a quarter of the SIMDs takes splits of 4
+  // (one lane of 2048 tokens, 4 / 8 / 16 rows: 35 -> 26, 39 -> 30, 30 -> 25 us), unless that
+  // gives a lane more than 128 splits.
+  uint32_t longest_lane = 0;
+  for (uint32_t i = 0; i < n_lanes; ++i)
+    longest_lane = std::max(longest_lane, pages_of(uint64_t(committed[i]) + rows));
+  const uint64_t shortest = (page_waves <= 2048 && longest_lane <= 512) ? 4 : 8;
+  uint32_t per = uint32_t(std::max<uint64_t>((page_waves + kSimds - 1) / kSimds, shortest));
   for (;; ++per) {
     uint64_t waves = 0;
     for (uint32_t i = 0; i < n_lanes; ++i) {

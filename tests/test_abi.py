@@ -167,10 +167,14 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
         if fmt == kvx.INT4 and fused > 16 and 26 * -(-fused // 48) < 15 * -(-fused // 32):
             blocks = -(-fused // 48)  # the int4 kernel for 48 fused rows per wave
         counts = [pages(c + rows) for c in committed]
-        per = max(-(-sum(counts) * H * blocks // 1024), 8)
+        # the int4 kernel for blocks of 32 rows of longer lanes: two waves per SIMD from 16 lanes on
+        slots = 2048 if (fmt == kvx.INT4 and fused > 32 and blocks == -(-fused // 32)
+                         and len(committed) >= 16) else 1024
+        small = sum(counts) * H * blocks <= 2048 and max(counts) <= 512
+        per = max(-(-sum(counts) * H * blocks // slots), 4 if small else 8)
         while True:  # the first length that fits one round of waves
             want = [min(max(1, -(-n // per)), 128) for n in counts]
-            if sum(want) * H * blocks <= 1024 or all(s == 1 for s in want):
+            if sum(want) * H * blocks <= slots or all(s == 1 for s in want):
                 break
             per += 1
         return want
