@@ -1376,7 +1376,7 @@ def main():
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-            "kernel": "decode_int4_kernel (split kernel of paged decode attention), one layer of the batch per launch",
+            "kernel": "decode_int4_quad_kernel (split kernel of paged decode attention, workgroups of four waves), one layer of the batch per launch",
             "bytes_per_launch": launch_bytes, "ms_per_launch": round(kernel_ms, 4),
             "merge_ms_per_launch": round(merge_ms, 4), "split_plus_merge_ms": round(both_ms, 4),
             "split_plus_merge_gbs": round(launch_bytes / (both_ms * 1e-3) / 1e9, 1),

@@ -481,8 +481,11 @@ int launch_matrix_attention(SplitKernel split_kernel, const char *name, uint32_t
     if (run_split) {
       const uint32_t column_blocks = (M + columns - 1) / columns;
       hipLaunchKernelGGL(split_kernel,
-                         a.item_major ? dim3(H, items, column_blocks)
-                                      : dim3((items + waves_per_group - 1) / waves_per_group, H, column_blocks),
+                         a.item_major
+                             ? (waves_per_group > 1
+                                    ? dim3((H * items + waves_per_group - 1) / waves_per_group, 1, column_blocks)
+                                    : dim3(H, items, column_blocks))
+                             : dim3((items + waves_per_group - 1) / waves_per_group, H, column_blocks),
                          dim3(threads), 0, stream, static_cast<const uint16_t *>(queries),
                          static_cast<uint16_t *>(output), partials, statistics, a);
       const hipError_t e = hipGetLastError();

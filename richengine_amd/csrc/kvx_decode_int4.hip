@@ -548,8 +548,10 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
   // of a tile's registers on a fifth of the pages instead of all of them on half.
   constexpr bool kRowsDown = NB == 2 && kDepth == 1;
   const uint32_t wave = kQuad ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0u;
-  const uint32_t item = kItemMajor ? blockIdx.y : kQuad ? 4 * blockIdx.x + wave : blockIdx.x;
-  const uint32_t head = kItemMajor ? blockIdx.x : blockIdx.y;
+  // item-major workgroups of four waves: (item, head) pairs in dispatch order, heads fastest
+  const uint32_t flat = 4 * blockIdx.x + wave;
+  uint32_t item = kItemMajor ? (kQuad ? 0u : blockIdx.y) : kQuad ? flat : blockIdx.x;
+  uint32_t head = kItemMajor ? (kQuad ? 0u : blockIdx.x) : blockIdx.y;
   uint32_t li;
   DecodeLane l;
   LaunchArgs a;
@@ -587,6 +589,10 @@ __device__ __forceinline__ void attend_int4(const uint16_t *__restrict__ queries
          reinterpret_cast<const uint16_t *>(chunk_keys),
          reinterpret_cast<const uint16_t *>(chunk_values), chunk_lane_stride, chunk_stride,
          all_partials};
+    if constexpr (kQuad) {
+      item = flat / kv_heads;
+      head = flat - item * kv_heads;
+    }
     // base is non-decreasing: the lane is the number of later lanes that start at or
     // before the item.
     uint32_t index = 0;
@@ -810,6 +816,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
   attend_int4<1, kDecodeDepth, false, true>(queries, output, partials, statistics, a);
 }
+// The same as workgroups of four waves, (work item, KV head) pairs in dispatch order: for
+// launches with two waves on most SIMDs, whose plan counts on the lanes with the longest
+// splits taking the first wave of every SIMD.  Single-wave workgroups get that placement only
+// while the dispatcher starts from a clean state (16 lanes of 32 768 tokens after a merge
+// kernel: 127 us, against 112 us for this form and 111 for its parts alone); a launch that
+// leaves SIMDs empty is better off with single waves spread over all CUs (one sequence of
+// 32 768 tokens: 15.5 against 16.6 us).
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void decode_int4_quad_kernel(
+    const uint16_t *__restrict__ queries, uint16_t *__restrict__ output,
+    float *__restrict__ partials, float *__restrict__ statistics, DecodeArgs a) {
+  attend_int4<1, kDecodeDepth, false, true, true>(queries, output, partials, statistics, a);
+}
 
 // The same for the 8-row tiles of a chunked prefill with several splits: every
 // tile of the chunk walks the same pages, so the loads may stay in the caches.
@@ -963,6 +981,16 @@ int kvx_attend_int4_launch(const kvx_storage *s, kvx_kv_layer kv, uint32_t query
                                    kv, query_heads, queries, output, page_tables, lanes, n_lanes,
                                    row_masks, row_stride, lane_stride, workspace, workspace_bytes,
                                    stream, nullptr, tile_rows, epilogue);
+  // two waves on most SIMDs (of the first launch's lanes): the form whose placement holds
+  uint64_t first_waves = 0;
+  for (uint32_t i = 0; i < std::min(n_lanes, kLanes); ++i)
+    first_waves += uint64_t(lanes[i].split_count) * s->layout.kv_heads;
+  if (first_waves > 1024)
+    return launch_matrix_attention(decode_int4_quad_kernel, "decode_int4_quad_kernel", 16, 256, s, kv,
+                                   query_heads, queries, output, page_tables, lanes, n_lanes,
+                                   row_masks, row_stride, lane_stride, workspace, workspace_bytes,
+                                   stream, fused, tile_rows, epilogue, /*longest_first=*/true,
+                                   /*waves_per_group=*/4);
   return launch_matrix_attention(decode_int4_kernel, "decode_int4_kernel", 16, 64, s, kv,
                                  query_heads, queries, output, page_tables, lanes, n_lanes,
                                  row_masks, row_stride, lane_stride, workspace, workspace_bytes,

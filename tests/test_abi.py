@@ -264,7 +264,7 @@ def test_hot_kernels_stay_out_of_scratch_memory():
         assert len(names) == 1, (fragment, names)
         return report[names[0]]
 
-    for fragment in ("decode_int4_kernelE", "decode_int4_tiles_kernel", "verify_int4_kernel",
+    for fragment in ("decode_int4_kernelE", "decode_int4_quad_kernel", "decode_int4_tiles_kernel", "verify_int4_kernel",
                      "verify32_int4_kernel", "verify48_int4_kernel", "prefill_int4_kernel",
                      "matrix_merge_kernelILj1E", "matrix_merge_kernelILj8E",   # one wave per row; ranged
                      "attend_wide_kernelILj1ELj1ELj2ELb0E",    # int8, one block, two waves per SIMD
@@ -277,7 +277,7 @@ def test_hot_kernels_stay_out_of_scratch_memory():
                      "attend_wide_kernelILj1ELj2ELj1ELb1E", "attend_wide_kernelILj4ELj2ELj1ELb1E"):
         r = one(fragment)
         assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, (fragment, r)
-    assert one("decode_int4_kernelE")["occupancy"] == 2
+    assert one("decode_int4_kernelE")["occupancy"] == 2 and one("decode_int4_quad_kernel")["occupancy"] == 2
     # two blocks over one page set: every accumulator in the first register file
     assert one("verify32_int4_kernel")["agprs"] == 0 and one("prefill_int4_kernel")["agprs"] == 0
     # the workgroup-shared prefill kernels (int8, bf16, fp8 pages; two and three row blocks
