@@ -884,16 +884,20 @@ def chunked_prefill(args):
     streams = [torch.cuda.Stream() for _ in range(n_streams)] if n_streams > 1 else [None]
     outputs = [torch.zeros_like(queries[0]) for _ in range(n_streams)]
     output = outputs[0]
-    splits = kvx.prefill_plan(prefix, chunk, H, QH, fmt)  # 1 for 2048 rows; chunks of 64 .. 1024 rows get more
+    # the split count fills the GPU's wave slots with the launch it is for: one sequence's tiles, or
+    # (batched) every sequence's
+    splits = kvx.prefill_plan(prefix, chunk, H, QH, fmt)
+    batch_splits = kvx.prefill_plan(prefix, chunk, H, QH, fmt, sequences=sequences)
     cp = kvx.ChunkParams(prefix, chunk, chunk, entries)
     pp = kvx.PrefillParams(prefix, chunk, chunk, entries, kvx.KvLayer(), splits, 0.0)
+    batch_pp = kvx.PrefillParams(prefix, chunk, chunk, entries, kvx.KvLayer(), batch_splits, 0.0)
     workspaces = [torch.empty(kvx.prefill_workspace_bytes(storage, chunk, QH, splits) + 4096, dtype=torch.uint8,
                               device="cuda") for _ in range(n_streams)]
     workspace = workspaces[0]
     if batched:
         all_k, all_v, all_q = torch.stack(chunk_k), torch.stack(chunk_v), torch.stack(queries)
         all_out = torch.zeros_like(all_q)
-        all_ws = torch.empty(sequences * kvx.prefill_workspace_bytes(storage, chunk, QH, splits) + 4096,
+        all_ws = torch.empty(sequences * kvx.prefill_workspace_bytes(storage, chunk, QH, batch_splits) + 4096,
                              dtype=torch.uint8, device="cuda")
     torch.cuda.synchronize()
 
@@ -901,7 +905,7 @@ def chunked_prefill(args):
         if batched:
             for layer in range(LAYERS):
                 kvx.append(storage, layer, all_k, all_v, tables, [cp] * sequences, H * chunk * D)
-                kvx.attend_prefill_batch(storage, layer, QH, all_q, all_out, tables, [pp] * sequences,
+                kvx.attend_prefill_batch(storage, layer, QH, all_q, all_out, tables, [batch_pp] * sequences,
                                          H * chunk * G * D, all_ws)
             return
         # a sequence's layers follow one another on its stream, as they do in a model
@@ -947,7 +951,8 @@ def chunked_prefill(args):
         "config": {"workload": "BASELINE configs[3]: chunked prefill with a shared prefix, batch 4, "
                                f"{chunk}-row chunks over 16384 + {chunk} tokens, 16 layers: quantize + scatter "
                                "of the chunk, then causal attention per layer and sequence",
-                   "batch": sequences, "layers": LAYERS, "format": args.format, "splits": int(splits),
+                   "batch": sequences, "layers": LAYERS, "format": args.format,
+                   "splits": int(batch_splits if batched else splits), "splits_of_one_launch": int(splits),
                    "streams": 0 if batched else n_streams,
                    "calls": "kv_attend_prefill_batch, one per layer" if batched
                             else "kv_attend_prefill, one per layer and sequence",

@@ -204,7 +204,12 @@ int kvx_chunk_validation(const kvx_chunk_params *params);
    8-row tiles end in the same page exactly when committed_tokens mod 16 is 0 or at least 9:
    then the first tile's last row and the second tile's last row, 8 tokens later, do not
    straddle a page boundary; so every page-aligned chunk start; int4 pages: from 512 rows on), else of tiles x splits x KV heads x ceil(8 x group / 16)
-   waves of single tiles.  bf16, fp8 and int8 pages, chunks of 64 rows and more (lanes of four tiles of
+   waves of single tiles.  int4 pages, chunks whose paired waves fill a quarter of the 2048
+   slots or more (from 683 rows of 24 query heads on 4 KV heads): the waves of a launch
+   are equally long and take the slots round by round, so the plan takes the fewest splits
+   (of at least 16 pages of the average tile's history each) that leave every round at least
+   nine tenths full, or failing that the fullest rounds: 4 for 2048 rows (1536 waves per
+   split) once 2048 tokens are committed, 5 for 1024 rows, 1 where there is no history to cut.  bf16, fp8 and int8 pages, chunks of 64 rows and more (lanes of four tiles of
    8 x group <= 48 fused rows, or two of <= 96, one workgroup per lane, split and KV head, one
    workgroup per CU): one split where those workgroups fill three quarters of the 256 CUs, else
    the count (same bounds) that fills them, where the chunk starts on a page boundary (lanes
@@ -213,6 +218,11 @@ int kvx_chunk_validation(const kvx_chunk_params *params);
    kvx_prefill_splits); any count in 1..32 is valid for kv_attend_prefill. */
 uint32_t kvx_prefill_plan(uint32_t committed_tokens, uint32_t rows, uint32_t kv_heads,
                           uint32_t query_heads, uint32_t format);
+/* The same for n_sequences chunks of this shape in one kv_attend_prefill_batch call, whose
+   launches hold every sequence's waves (four chunks of 2048 rows: 6144 waves, three full
+   rounds in one split each).  n_sequences = 1 is kvx_prefill_plan; 0 returns 0. */
+uint32_t kvx_prefill_plan_batch(uint32_t committed_tokens, uint32_t rows, uint32_t kv_heads,
+                                uint32_t query_heads, uint32_t format, uint32_t n_sequences);
 /* ops::PagedAttention::prefillPlan(...).workspace / prefillWorkspace / verifyWorkspace.
    Bytes of partials and statistics; a workspace buffer holds partials first,
    then statistics at the next 256-byte boundary. */

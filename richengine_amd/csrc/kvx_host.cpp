@@ -162,7 +162,11 @@ uint32_t kvx_prefill_splits(uint32_t rows) {
 }
 uint32_t kvx_prefill_plan(uint32_t committed, uint32_t rows, uint32_t kv_heads, uint32_t query_heads,
                           uint32_t format) {
-  if (!kv_heads || !query_heads || query_heads % kv_heads) return 0;
+  return kvx_prefill_plan_batch(committed, rows, kv_heads, query_heads, format, 1);
+}
+uint32_t kvx_prefill_plan_batch(uint32_t committed, uint32_t rows, uint32_t kv_heads,
+                                uint32_t query_heads, uint32_t format, uint32_t sequences) {
+  if (!kv_heads || !query_heads || query_heads % kv_heads || !sequences) return 0;
   const uint32_t tiles = (rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
   if (!tiles) return 1;
   const uint32_t group = query_heads / kv_heads, tile_fused = KVX_PREFILL_TILE_ROWS * group;
@@ -174,28 +178,51 @@ uint32_t kvx_prefill_plan(uint32_t committed, uint32_t rows, uint32_t kv_heads, 
   // the CUs; else as many as fill them, where the lanes' tiles cut their pages alike.
   if (const uint32_t width = kvx::prefill_group_width(format, 256, rows, group)) {
     constexpr uint32_t kCus = 256;
-    const uint32_t workgroups = (tiles + width - 1) / width * kv_heads;
+    const uint32_t workgroups = (tiles + width - 1) / width * kv_heads * sequences;
     if (4 * workgroups >= 3 * kCus) return 1;
     if (kvx::prefill_group_splits_alike(width, committed))
       return std::max(1u, std::min({(kCus + workgroups - 1) / workgroups, by_pages, KVX_PREFILL_MAX_SPLITS}));
   }
   // One split: neighbouring tiles share a walk as lanes of 16 rows on the kernels
   // with two blocks of 16 fused rows per wave (int4: two waves per SIMD).
-  const uint32_t paired_waves = kvx::prefill_paired_waves(tiles, kv_heads, group);
+  const uint64_t paired_waves = uint64_t(kvx::prefill_paired_waves(tiles, kv_heads, group)) * sequences;
   const uint32_t paired_slots = kvx::prefill_paired_slots(format);
-  if (tile_fused <= 16 || 2 * paired_waves >= paired_slots) return 1;
+  if (tile_fused <= 16) return 1;
+  // int4 pages, chunks whose paired waves fill a quarter of the slots or more: the waves of a
+  // launch are equally long and take their slots round by round, so a last round that is
+  // partly empty costs as much as a full one (2048 rows, one split: 1536 waves, 4.97 ms after
+  // 65536 tokens; four splits, three full rounds: 3.84 ms; 1024 rows: 2.45 -> 1.9 ms).  The
+  // fewest splits that leave every round at least nine tenths full, of at least 16 pages of
+  // the average tile's history each (shorter ones cost more in set-up and partial rows than
+  // the rounds win: 1024 rows with no history, 77 us in one split, 90 in two); failing that,
+  // the fullest rounds.
+  if (format == KVX_FMT_INT4 && 4 * paired_waves >= paired_slots) {
+    const uint32_t seen = pages_of(uint64_t(committed) + rows / 2);
+    const uint32_t most = std::max(1u, std::min(seen / 16, KVX_PREFILL_MAX_SPLITS));
+    uint32_t best = 1;
+    uint64_t best_waves = 0, best_room = 1;
+    for (uint32_t s = 1; s <= most; ++s) {
+      if (s > 1 && !kvx::prefill_pairs_with_splits(format, committed, tiles, s, kv_heads, group)) continue;
+      const uint64_t waves = paired_waves * s;
+      const uint64_t room = (waves + paired_slots - 1) / paired_slots * paired_slots;
+      if (10 * waves >= 9 * room) return s;
+      if (waves * best_room > best_waves * room) best = s, best_waves = waves, best_room = room;
+    }
+    return best;
+  }
+  if (2 * paired_waves >= paired_slots) return 1;
   // Tiles that pair under any split count keep their shared walks: as many
   // splits as fit one round of the paired kernels' slots.
   const uint32_t paired_splits =
-      std::max(1u, std::min({paired_slots / paired_waves, by_pages, KVX_PREFILL_MAX_SPLITS}));
+      std::max(1u, std::min({uint32_t(paired_slots / paired_waves), by_pages, KVX_PREFILL_MAX_SPLITS}));
   if (paired_splits >= 2 &&
       kvx::prefill_pairs_with_splits(format, committed, tiles, paired_splits, kv_heads, group))
     return paired_splits;
   // Several splits: one lane per tile on the kernels with one block per wave
   // (two waves per SIMD except for bf16 pages).
   const uint32_t slots = format == KVX_FMT_BF16 ? kSimds : 2 * kSimds;
-  const uint32_t per_split = tiles * kv_heads * ((tile_fused + 15) / 16);
-  const uint32_t fit = slots / per_split;
+  const uint64_t per_split = uint64_t(tiles) * kv_heads * ((tile_fused + 15) / 16) * sequences;
+  const uint32_t fit = uint32_t(slots / per_split);
   const uint32_t splits = std::min({fit, by_pages, KVX_PREFILL_MAX_SPLITS});
   return splits >= 2 ? splits : 1;
 }

@@ -23,7 +23,7 @@ SYMBOLS = [
     "kvx_layout_bytes_per_model_page", "kvx_layout_extent_alignment_pages",
     "kvx_layout_minimum_extent_pages", "kvx_layout_maximum_extent_pages",
     "kvx_layout_extent_pages_for", "kvx_layout_largest_extent_pages", "kvx_kv_offset",
-    "kvx_verify_splits", "kvx_prefill_splits", "kvx_prefill_plan", "kvx_decode_splits", "kvx_chunk_validation",
+    "kvx_verify_splits", "kvx_prefill_splits", "kvx_prefill_plan", "kvx_prefill_plan_batch", "kvx_decode_splits", "kvx_chunk_validation",
     "kvx_prefill_workspace", "kvx_prefill_workspace_for", "kvx_prefill_workspace_bound", "kvx_verify_workspace",
     "kvx_attend_workspace_bytes", "kvx_storage_create", "kvx_storage_destroy",
     "kvx_storage_page_count", "kvx_storage_extent_pages", "kvx_storage_bytes_per_page",
@@ -155,6 +155,7 @@ def _declare(L):
         getattr(L, n).argtypes, getattr(L, n).restype = [u32, u32], u32
     L.kvx_prefill_splits.argtypes, L.kvx_prefill_splits.restype = [u32], u32
     L.kvx_prefill_plan.argtypes, L.kvx_prefill_plan.restype = [u32, u32, u32, u32, u32], u32
+    L.kvx_prefill_plan_batch.argtypes, L.kvx_prefill_plan_batch.restype = [u32] * 6, u32
     L.kvx_chunk_validation.argtypes = [C.POINTER(ChunkParams)]
     P64 = C.POINTER(u64)
     L.kvx_prefill_workspace.argtypes = [u32, u32, LP, P64, P64]
@@ -775,9 +776,10 @@ def decode_plan(committed, kv_heads, fmt=INT4):
     return list(out)
 
 
-def prefill_plan(committed, rows, kv_heads, query_heads, fmt=INT4):
-    """Split count of a chunked prefill sized for the GPU (kvx_prefill_plan)."""
-    splits = lib().kvx_prefill_plan(committed, rows, kv_heads, query_heads, fmt)
+def prefill_plan(committed, rows, kv_heads, query_heads, fmt=INT4, sequences=1):
+    """Split count of a chunked prefill sized for the GPU (kvx_prefill_plan; for `sequences`
+    equal chunks in one kv_attend_prefill_batch call, kvx_prefill_plan_batch)."""
+    splits = lib().kvx_prefill_plan_batch(committed, rows, kv_heads, query_heads, fmt, sequences)
     if not splits:
         raise KvxError(-1, "kvx_prefill_plan: bad head counts")
     return splits

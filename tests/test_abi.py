@@ -202,7 +202,8 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
         single_slots = 2048 if fmt == kvx.INT4 else 1024
         slots = 1024 if fmt == kvx.BF16 else 2048
         for committed, rows in ((16384, 64), (16384, 256), (16384, 512), (16384, 2048), (0, 256),
-                                (100, 7), (3000, 264), (3004, 264), (16388, 512)):
+                                (100, 7), (3000, 264), (3004, 264), (16388, 512), (0, 1024), (2048, 1024),
+                                (65536, 1024), (1024, 2048), (16388, 2048), (512, 768)):
             tiles = -(-rows // 8)
             paired = -(-tiles // 2) * H * -(-(16 * (QH // H)) // 32)
             want = 1
@@ -218,6 +219,14 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
                 want = 1
             elif alike:
                 want = max(1, min(-(-256 // workgroups), max(1, pages(committed + rows) // 8), 32))
+            elif fmt == kvx.INT4 and 4 * paired >= single_slots:
+                # equally long waves take the slots round by round: the fewest splits (of 16
+                # pages of the average tile's history or more) whose rounds are nine tenths full
+                pairable = committed % 16 == 0 or committed % 16 >= 9
+                most = max(1, min(pages(committed + rows // 2) // 16, 32)) if pairable else 1
+                room = lambda s: -(-paired * s // single_slots) * single_slots
+                full = [s for s in range(1, most + 1) if 10 * paired * s >= 9 * room(s)]
+                want = full[0] if full else max(range(1, most + 1), key=lambda s: (paired * s / room(s), -s))
             elif 2 * paired < single_slots:
                 by_pages = max(1, pages(committed + rows) // 8)
                 pairable = tiles >= 2 and (committed % 16 == 0 or committed % 16 >= 9)
@@ -234,9 +243,15 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
     assert kvx.prefill_plan(16384, 256, H, QH, kvx.BF16) == 8      # 32 workgroups of four tiles each
     assert kvx.prefill_plan(16384, 1024, H, QH, kvx.FP8) == 2      # 128 workgroups
     assert kvx.prefill_plan(16384, 2048, H, QH, kvx.INT8) == 1     # 256 workgroups
-    assert kvx.prefill_plan(16384, 1024, H, QH, kvx.INT4) == 2     # 768 of paired tiles
+    assert kvx.prefill_plan(16384, 1024, H, QH, kvx.INT4) == 5     # 768 waves of paired tiles: 3840 on 4096 slots
     assert kvx.prefill_plan(16388, 256, H, QH, kvx.BF16) == 2      # 384 of single tiles
-    assert kvx.prefill_plan(16384, 2048, H, QH, kvx.INT4) == 1
+    assert kvx.prefill_plan(16384, 2048, H, QH, kvx.INT4) == 4     # 1536 waves: three full rounds of 2048
+    assert kvx.prefill_plan(0, 2048, H, QH, kvx.INT4) == 1         # 32 pages before the average tile: nothing to cut
+    assert kvx.prefill_plan(0, 1024, H, QH, kvx.INT4) == 1
+    assert kvx.prefill_plan(16384, 2048, H, QH, kvx.INT4, sequences=4) == 1   # 6144 waves already
+    assert kvx.prefill_plan(16384, 2048, H, QH, kvx.INT4, sequences=2) == 2
+    assert kvx.prefill_plan(16384, 256, H, QH, kvx.BF16, sequences=4) == 2    # 128 workgroups
+    assert kvx.lib().kvx_prefill_plan_batch(16384, 256, H, QH, kvx.INT4, 0) == 0
     with pytest.raises(kvx.KvxError):
         kvx.prefill_plan(16384, 256, 4, 6)
     assert kvx.verify_plan([65536] * 4, 16, H, QH) == [21] * 4          # three waves of 32 fused rows
