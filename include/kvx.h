@@ -170,8 +170,9 @@ uint32_t kvx_decode_splits(uint32_t committed_tokens, uint32_t rows);
    fits 1024 waves too; kv_attend_decode dispatches the lanes with the longest splits first, so
    the long splits take the first wave of every SIMD and both classes end together.  One-row
    decode lanes may use up to KVX_DECODE_MAX_SPLITS splits; every other attend entry keeps the
-   reference's KVX_VERIFY_MAX_SPLITS.  No counterpart in the reference, whose decode shares the
-   verify plan (runtime/ops/PagedAttention.cpp:232-262). */
+   reference's KVX_VERIFY_MAX_SPLITS.  KVX_EINVAL for a null argument, no lanes, no KV heads or a
+   lane whose context (committed + 1) is beyond KVX_MAX_PHYSICAL_TOKENS.  No counterpart in the
+   reference, whose decode shares the verify plan (runtime/ops/PagedAttention.cpp:232-262). */
 #define KVX_DECODE_MAX_SPLITS 512u
 int kvx_decode_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t kv_heads,
                     uint32_t format, uint32_t *split_counts);
@@ -186,7 +187,8 @@ int kvx_decode_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t
    KV heads x ceil(rows x group / 32) waves, one per SIMD; on int4 pages ceil(rows x group / 48)
    where that is fewer by more than 1.74 (33 .. 48 fused rows among others).  No counterpart in the reference
    (its rule is kvx_verify_splits); any split count either rule gives is valid for
-   kv_attend_verify. */
+   kv_attend_verify.  KVX_EINVAL for a null argument, no lanes, bad head counts or a lane whose
+   context (committed + rows) is beyond KVX_MAX_PHYSICAL_TOKENS. */
 int kvx_verify_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t rows,
                     uint32_t kv_heads, uint32_t query_heads, uint32_t format,
                     uint32_t *split_counts);

@@ -167,8 +167,12 @@ uint32_t kvx_prefill_plan(uint32_t committed, uint32_t rows, uint32_t kv_heads, 
 uint32_t kvx_prefill_plan_batch(uint32_t committed, uint32_t rows, uint32_t kv_heads,
                                 uint32_t query_heads, uint32_t format, uint32_t sequences) {
   if (!kv_heads || !query_heads || query_heads % kv_heads || !sequences) return 0;
-  const uint32_t tiles = (rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+  const uint32_t tiles = uint32_t((uint64_t(rows) + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS);
   if (!tiles) return 1;
+  // wave counts saturate instead of wrapping (no shape the kernels take comes near)
+  const auto times = [](uint64_t a, uint64_t b) {
+    return b && a > std::numeric_limits<uint64_t>::max() / b ? std::numeric_limits<uint64_t>::max() : a * b;
+  };
   const uint32_t group = query_heads / kv_heads, tile_fused = KVX_PREFILL_TILE_ROWS * group;
   const uint32_t pages = pages_of(uint64_t(committed) + rows);
   constexpr uint32_t kSimds = 1024;
@@ -178,14 +182,16 @@ uint32_t kvx_prefill_plan_batch(uint32_t committed, uint32_t rows, uint32_t kv_h
   // the CUs; else as many as fill them, where the lanes' tiles cut their pages alike.
   if (const uint32_t width = kvx::prefill_group_width(format, 256, rows, group)) {
     constexpr uint32_t kCus = 256;
-    const uint32_t workgroups = (tiles + width - 1) / width * kv_heads * sequences;
-    if (4 * workgroups >= 3 * kCus) return 1;
+    const uint64_t workgroups = times(times((tiles + width - 1) / width, kv_heads), sequences);
+    if (workgroups >= 3 * kCus / 4) return 1;
     if (kvx::prefill_group_splits_alike(width, committed))
-      return std::max(1u, std::min({(kCus + workgroups - 1) / workgroups, by_pages, KVX_PREFILL_MAX_SPLITS}));
+      return std::max(1u, std::min({uint32_t((kCus + workgroups - 1) / workgroups), by_pages,
+                                    KVX_PREFILL_MAX_SPLITS}));
   }
   // One split: neighbouring tiles share a walk as lanes of 16 rows on the kernels
   // with two blocks of 16 fused rows per wave (int4: two waves per SIMD).
-  const uint64_t paired_waves = uint64_t(kvx::prefill_paired_waves(tiles, kv_heads, group)) * sequences;
+  const uint64_t paired_waves =
+      times(times(times((uint64_t(tiles) + 1) / 2, kv_heads), (2 * uint64_t(tile_fused) + 31) / 32), sequences);
   const uint32_t paired_slots = kvx::prefill_paired_slots(format);
   if (tile_fused <= 16) return 1;
   // int4 pages, chunks whose paired waves fill a quarter of the slots or more: the waves of a
@@ -196,21 +202,22 @@ uint32_t kvx_prefill_plan_batch(uint32_t committed, uint32_t rows, uint32_t kv_h
   // the average tile's history each (shorter ones cost more in set-up and partial rows than
   // the rounds win: 1024 rows with no history, 77 us in one split, 90 in two); failing that,
   // the fullest rounds.
-  if (format == KVX_FMT_INT4 && 4 * paired_waves >= paired_slots) {
+  if (format == KVX_FMT_INT4 && paired_waves >= paired_slots / 4) {
     const uint32_t seen = pages_of(uint64_t(committed) + rows / 2);
     const uint32_t most = std::max(1u, std::min(seen / 16, KVX_PREFILL_MAX_SPLITS));
     uint32_t best = 1;
     uint64_t best_waves = 0, best_room = 1;
     for (uint32_t s = 1; s <= most; ++s) {
       if (s > 1 && !kvx::prefill_pairs_with_splits(format, committed, tiles, s, kv_heads, group)) continue;
-      const uint64_t waves = paired_waves * s;
+      const uint64_t waves = times(paired_waves, s);
+      if (waves > (1ull << 30)) return s;  // thousands of rounds: full by any count
       const uint64_t room = (waves + paired_slots - 1) / paired_slots * paired_slots;
       if (10 * waves >= 9 * room) return s;
       if (waves * best_room > best_waves * room) best = s, best_waves = waves, best_room = room;
     }
     return best;
   }
-  if (2 * paired_waves >= paired_slots) return 1;
+  if (paired_waves >= paired_slots / 2) return 1;
   // Tiles that pair under any split count keep their shared walks: as many
   // splits as fit one round of the paired kernels' slots.
   const uint32_t paired_splits =
@@ -221,7 +228,7 @@ uint32_t kvx_prefill_plan_batch(uint32_t committed, uint32_t rows, uint32_t kv_h
   // Several splits: one lane per tile on the kernels with one block per wave
   // (two waves per SIMD except for bf16 pages).
   const uint32_t slots = format == KVX_FMT_BF16 ? kSimds : 2 * kSimds;
-  const uint64_t per_split = uint64_t(tiles) * kv_heads * ((tile_fused + 15) / 16) * sequences;
+  const uint64_t per_split = times(times(times(tiles, kv_heads), (uint64_t(tile_fused) + 15) / 16), sequences);
   const uint32_t fit = uint32_t(slots / per_split);
   const uint32_t splits = std::min({fit, by_pages, KVX_PREFILL_MAX_SPLITS});
   return splits >= 2 ? splits : 1;
@@ -258,7 +265,8 @@ static void decode_plan_of_launch(const uint32_t *committed, uint32_t n_lanes, u
   for (uint32_t i = 0; i < n_lanes; ++i) longest_lane = std::max(longest_lane, pages[i]);
   const uint64_t small_launch = format == KVX_FMT_INT4 ? 4 * kSimds : 2 * kSimds;  // page-heads
   const uint64_t shortest = (page_heads <= small_launch && longest_lane <= 512) ? 4 : 8;
-  uint32_t per = uint32_t(std::max<uint64_t>((page_heads + kSimds - 1) / kSimds, shortest));
+  constexpr uint64_t kMostPages = KVX_MAX_PHYSICAL_TOKENS / KVX_PAGE_TOKENS + 1;  // one split per lane by then
+  uint32_t per = uint32_t(std::min(std::max<uint64_t>((page_heads + kSimds - 1) / kSimds, shortest), kMostPages));
   if (format == KVX_FMT_INT4) per = std::min(per, KVX_DECODE_PAGES_PER_SPLIT);
   uint64_t waves = 0;
   for (;; ++per) {
@@ -314,6 +322,9 @@ int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_hea
                     uint32_t *split_counts) {
   if (!committed || !split_counts || !n_lanes || !kv_heads)
     return fail(KVX_EINVAL, "kvx_decode_plan: null argument or empty batch");
+  for (uint32_t i = 0; i < n_lanes; ++i)
+    if (uint64_t(committed[i]) + 1 > KVX_MAX_PHYSICAL_TOKENS)
+      return fail(KVX_EINVAL, "kvx_decode_plan: context_out_of_range");
   // The attend calls take the lanes KVX_LANES_PER_LAUNCH at a time, in the caller's order,
   // and the launches follow one another: every launch is planned to fill the GPU by itself
   // (a batch of 128 sequences of 8192 tokens planned as one: 341 us; launch by launch: 220).
@@ -351,7 +362,8 @@ static void verify_plan_of_launch(const uint32_t *committed, uint32_t n_lanes, u
   for (uint32_t i = 0; i < n_lanes; ++i)
     longest_lane = std::max(longest_lane, pages_of(uint64_t(committed[i]) + rows));
   const uint64_t shortest = (page_waves <= 2048 && longest_lane <= 512) ? 4 : 8;
-  uint32_t per = uint32_t(std::max<uint64_t>((page_waves + kSimds - 1) / kSimds, shortest));
+  constexpr uint64_t kMostPages = KVX_MAX_PHYSICAL_TOKENS / KVX_PAGE_TOKENS + 1;  // one split per lane by then
+  uint32_t per = uint32_t(std::min(std::max<uint64_t>((page_waves + kSimds - 1) / kSimds, shortest), kMostPages));
   for (;; ++per) {
     uint64_t waves = 0;
     for (uint32_t i = 0; i < n_lanes; ++i) {
@@ -371,6 +383,9 @@ int kvx_verify_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t rows, 
   if (!committed || !split_counts || !n_lanes || !kv_heads || !rows || !query_heads ||
       query_heads % kv_heads)
     return fail(KVX_EINVAL, "kvx_verify_plan: null argument, empty batch or bad head counts");
+  for (uint32_t i = 0; i < n_lanes; ++i)
+    if (uint64_t(committed[i]) + rows > KVX_MAX_PHYSICAL_TOKENS)
+      return fail(KVX_EINVAL, "kvx_verify_plan: context_out_of_range");
   // launch by launch, as kvx_decode_plan
   for (uint32_t first = 0; first < n_lanes; first += KVX_LANES_PER_LAUNCH)
     verify_plan_of_launch(committed + first, std::min(KVX_LANES_PER_LAUNCH, n_lanes - first), rows,

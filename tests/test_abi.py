@@ -252,6 +252,29 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
     assert kvx.prefill_plan(16384, 2048, H, QH, kvx.INT4, sequences=2) == 2
     assert kvx.prefill_plan(16384, 256, H, QH, kvx.BF16, sequences=4) == 2    # 128 workgroups
     assert kvx.lib().kvx_prefill_plan_batch(16384, 256, H, QH, kvx.INT4, 0) == 0
+    # contexts past the interface's maximum are refused before any planning; absurd head counts
+    # neither divide by a wrapped zero nor walk the split lengths one by one for seconds
+    import time
+    for committed in ([262144 + 15], [5, 0xFFFFFFFF]):
+        with pytest.raises(kvx.KvxError):
+            kvx.decode_plan(committed, H, kvx.INT4)
+        with pytest.raises(kvx.KvxError):
+            kvx.verify_plan(committed, 16, H, QH, kvx.INT4)
+    started = time.perf_counter()
+    for fmt in (kvx.INT4, kvx.INT8, kvx.BF16):
+        for heads in (748871255, 1 << 22, 0xFFFFFFFF):
+            plan = kvx.decode_plan([262144, 32146, 6, 2048] * 8, heads, fmt)
+            assert all(1 <= s <= 512 for s in plan)
+            plan = kvx.verify_plan([262144, 32146, 6, 2048] * 8, 15, heads, heads, fmt)
+            assert all(1 <= s <= 128 for s in plan)
+    assert time.perf_counter() - started < 2.0
+    # wave counts saturate: absurd shapes get some count in 1..32 instead of a wrapped division
+    for fmt in (kvx.INT4, kvx.INT8, kvx.BF16):
+        for heads, query_heads, sequences in ((1 << 31, 1 << 31, 1 << 31), (2, 1 << 31, 0xFFFFFFFF),
+                                              (1 << 30, 3 << 30, 1 << 30), (4, 24, 0xFFFFFFFF)):
+            for rows in (8, 2048, 0xFFFFFFFF):
+                assert 1 <= kvx.lib().kvx_prefill_plan_batch(0xFFFFFFF0, rows, heads, query_heads, fmt,
+                                                             sequences) <= 32
     with pytest.raises(kvx.KvxError):
         kvx.prefill_plan(16384, 256, 4, 6)
     assert kvx.verify_plan([65536] * 4, 16, H, QH) == [21] * 4          # three waves of 32 fused rows
