@@ -250,7 +250,9 @@ uint64_t kvx_attend_workspace_bytes(const kvx_verify_params *lanes, uint32_t n_l
 typedef struct kvx_storage kvx_storage;
 /* PageStorage::PageStorage (PageStorage.mm:12-46).  aligned != 0 enforces whole
    alignment units per extent as production does; 0 takes any extent size the
-   page index allows (dev/tuning/HostKvExtents.hpp:158-169, test pools). */
+   page index allows (dev/tuning/HostKvExtents.hpp:158-169, test pools).  KVX_EINVAL beyond the
+   reference's own checks: head dimensions other than 64 / 128 / 256, more than 4096 KV heads or
+   65536 layers (the kernels index a page's bytes in 32 bits), more than 1048576 extents. */
 int kvx_storage_create(const kvx_layout *layout, uint32_t page_count, uint32_t extent_pages,
                        int aligned, kvx_storage **out);
 /* Storage with no memory behind its extents, for the page bookkeeping alone (pool,

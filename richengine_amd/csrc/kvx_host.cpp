@@ -79,11 +79,14 @@ const char *kvx_last_error(void) { return g_last_error.c_str(); }
 int kvx_layout_valid(const kvx_layout *l) {
   return l && l->layers && l->kv_heads && l->head_dim && valid_format(l->format);
 }
+// In 64 bits: the device-side forms (data_bytes_of, scale_bytes_of) hold for the layouts a
+// storage accepts, these for whatever a caller asks about.
 uint64_t kvx_layout_data_bytes_per_layer_page(const kvx_layout *l) {
-  return data_bytes_of(l->format, l->kv_heads, l->head_dim);
+  const uint64_t elements = uint64_t(KVX_PAGE_TOKENS) * l->kv_heads * l->head_dim;
+  return l->format == KVX_FMT_BF16 ? elements * 2 : l->format == KVX_FMT_INT4 ? elements / 2 : elements;
 }
 uint64_t kvx_layout_scale_bytes_per_layer_page(const kvx_layout *l) {
-  return scale_bytes_of(l->format, l->kv_heads);
+  return quantized(l->format) ? uint64_t(KVX_PAGE_TOKENS) * l->kv_heads * 4 : 0;
 }
 uint64_t kvx_layout_bytes_per_layer_page(const kvx_layout *l) {
   return 2 * (kvx_layout_data_bytes_per_layer_page(l) + kvx_layout_scale_bytes_per_layer_page(l));
@@ -468,6 +471,9 @@ static int storage_create(const kvx_layout *layout, uint32_t page_count, uint32_
   if (!kvx_layout_valid(layout)) return fail(KVX_EINVAL, "KV page storage layout is invalid");
   if (layout->head_dim != 64 && layout->head_dim != 128 && layout->head_dim != 256)
     return fail(KVX_EINVAL, "head dimension must be 64, 128 or 256");
+  // The kernels index a page's bytes in 32 bits.
+  if (layout->kv_heads > 4096 || layout->layers > 65536)
+    return fail(KVX_EINVAL, "more than 4096 KV heads or 65536 layers");
   const uint64_t extent_bytes = uint64_t(extent_pages) * kvx_layout_bytes_per_model_page(layout);
   if (!extent_pages || (aligned && extent_pages % kvx_layout_extent_alignment_pages(layout)) ||
       extent_pages > KVX_PAGE_INDEX_MASK ||
@@ -475,6 +481,8 @@ static int storage_create(const kvx_layout *layout, uint32_t page_count, uint32_
     return fail(KVX_EINVAL, "KV extent geometry is invalid");
   if (!page_count || page_count % extent_pages)
     return fail(KVX_EINVAL, "KV page pool is not a whole number of extents");
+  if (page_count / extent_pages > (1u << 20))
+    return fail(KVX_EINVAL, "KV page pool of more than 1048576 extents");
   auto *s = new kvx_storage;
   s->layout = *layout;
   s->page_count = page_count;

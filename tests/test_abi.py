@@ -347,3 +347,20 @@ def test_hot_kernels_stay_out_of_scratch_memory():
     for fmt in (1, 2, 3, 4):
         assert one(f"13append_kernelILj{fmt}E")["scratchsize"] == 0
         assert one(f"prepare_append_kernelILj{fmt}E")["scratchsize"] == 0
+
+
+def test_storage_refuses_geometry_the_kernels_cannot_index():
+    """A page's bytes are indexed in 32 bits on the device: head counts whose page bytes would
+    wrap are refused when the storage is made (with kv_heads = 2**19 + 4 the wrapped sizes are
+    those of 4 heads), the layout functions answer in 64 bits, and a pool cannot have so many
+    extents that its host tables alone take gigabytes."""
+    import ctypes as C
+    L = kvx.lib()
+    wrapped = kvx.Layout(1, (1 << 19) + 4, 256, kvx.INT8, 0.0)
+    L.kvx_layout_data_bytes_per_layer_page.restype = C.c_uint64
+    assert L.kvx_layout_data_bytes_per_layer_page(C.byref(wrapped)) == 32 * ((1 << 19) + 4) * 256
+    for heads, layers, pages, extent_pages in (((1 << 19) + 4, 1, 256, 128), (4097, 1, 256, 128),
+                                               (4, 65537, 256, 128), (1, 1, 3 << 20, 1)):
+        with pytest.raises(kvx.KvxError):
+            kvx.Storage(layers, heads, 64, kvx.INT8, pages, extent_pages, accounting=True)
+    kvx.Storage(1, 1, 64, kvx.INT8, 1 << 20, 1, accounting=True).close()
