@@ -362,109 +362,124 @@ __device__ __forceinline__ void store_row_wave(const uint16_t (&source)[E], bool
   }
 }
 
-// grid (blocks of four head tasks, row, lane): a wave is one (row, head) task, and which
-// one it is comes from the block's coordinates without a division or a walk over the
-// lane records.  Head tasks 0 .. QH - 1 are the query heads, QH .. QH + H - 1 the KV heads.
-template <uint32_t FMT, uint32_t E>
+// grid (blocks of four head tasks, group of R rows, lane): a wave is one head task of R
+// consecutive rows, and which one it is comes from the block's coordinates without a division
+// or a walk over the lane records.  Head tasks 0 .. QH - 1 are the query heads, QH .. QH + H - 1
+// the KV heads.  R = 4 for chunks: a row is 512 bytes of work behind four trips to memory, and
+// with the loads of four rows in flight at once a wave's wait is shared by them (2048 rows of
+// 28 head tasks: 37.5 us as one row per wave).
+template <uint32_t FMT, uint32_t E, uint32_t R>
 __global__ __launch_bounds__(256) void prepare_append_wave_kernel(PrepareArgs p) {
 #pragma clang fp contract(off)
   constexpr uint32_t D = 64 * E;
   const AppendArgs &a = p.append;
   const uint32_t lane = threadIdx.x & 63u;
   const uint32_t task = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t row = blockIdx.y, li = blockIdx.z;
+  const uint32_t first_row = blockIdx.y * R, li = blockIdx.z;
   const AppendLane &l = a.lane[li];
   if (!append_contract(l, a)) return;
   const uint32_t H = a.kv_heads, QH = p.query_heads, G = QH / H;
-  if (row >= l.tokens || task >= QH + H) return;
+  if (first_row >= l.tokens || task >= QH + H) return;
   const bool query = task < QH;
   const uint32_t head = query ? task : task - QH;
   const uint32_t d0 = E * lane;
   const uint32_t q_stride = p.query_gate ? 2 * D : D;
   const uint64_t packed_stride = uint64_t(QH) * q_stride + 2ull * H * D;
-  const uint16_t *source = p.packed + (uint64_t(li) * p.rows + row) * packed_stride +
-                           (query ? uint64_t(head) * q_stride : uint64_t(QH) * q_stride + uint64_t(head) * D);
-  // Everything the task reads is requested before anything waits: the row, the
-  // value row (a query task reads its own row twice), the norm weights (any
+  const uint64_t head_offset = query ? uint64_t(head) * q_stride : uint64_t(QH) * q_stride + uint64_t(head) * D;
+  // Everything the task reads is requested before anything waits: the rows, the
+  // value rows (a query task reads its own row twice), the norm weights (any
   // readable address when there are none), the rotation of the lane's
-  // dimensions (entry 0 for dimensions past the rotated ones) and the page entry.
+  // dimensions (entry 0 for dimensions past the rotated ones) and the page entries.
+  // Rows past the lane's last read the last again; nothing is stored for them.
   const bool norms = p.q_norm != nullptr;
   const uint32_t RP = p.rotary_pairs, pair_lanes = RP / E;
   const bool rotated = d0 < 2 * RP, is_first = d0 < RP;
-  uint16_t raw[E], raw_value[E], weight_bf16[E];
-  float weight_f32[E], cosine[E], sine[E];
-  load_bf16s<E>(source + d0, raw);
-  load_bf16s<E>(source + (query ? 0u : H * D) + d0, raw_value);
+  uint16_t raw[R][E], raw_value[R][E], weight_bf16[E];
+  float weight_f32[E], cosine[R][E], sine[R][E];
+  uint64_t entry[R];
+#pragma unroll
+  for (uint32_t r = 0; r < R; ++r) {
+    const uint32_t row = min(first_row + r, l.tokens - 1);
+    const uint16_t *source = p.packed + (uint64_t(li) * p.rows + row) * packed_stride + head_offset;
+    load_bf16s<E>(source + d0, raw[r]);
+    load_bf16s<E>(source + (query ? 0u : H * D) + d0, raw_value[r]);
+    const uint64_t rope_at = (uint64_t(li) * p.rows + row) * RP + (rotated ? (is_first ? d0 : d0 - RP) : 0u);
+    load_floats<E>(p.rope_cos + rope_at, cosine[r]);
+    load_floats<E>(p.rope_sin + rope_at, sine[r]);
+    entry[r] = l.table[(l.committed + row) / kPage];
+  }
   const void *weight = norms ? (query ? p.q_norm : p.k_norm) : static_cast<const void *>(p.packed);
   if (p.norm_f32) load_floats<E>(static_cast<const float *>(weight) + d0, weight_f32);
   else load_bf16s<E>(static_cast<const uint16_t *>(weight) + d0, weight_bf16);
-  const uint64_t rope_at = (uint64_t(li) * p.rows + row) * RP + (rotated ? (is_first ? d0 : d0 - RP) : 0u);
-  load_floats<E>(p.rope_cos + rope_at, cosine);
-  load_floats<E>(p.rope_sin + rope_at, sine);
-  const uint32_t logical = l.committed + row;
-  const uint64_t entry = l.table[logical / kPage];
 
-  float element[E], scale[E];
-  float inverse = 1.0f;
+  float scale[E];
 #pragma unroll
-  for (uint32_t e = 0; e < E; ++e) {
-    element[e] = bf16_to_f32(raw[e]);
+  for (uint32_t e = 0; e < E; ++e)
     scale[e] = !norms ? 1.0f : p.norm_f32 ? weight_f32[e] : bf16_to_f32(weight_bf16[e]);
-  }
-  if (norms) {
-    float sum[E];
 #pragma unroll
-    for (uint32_t e = 0; e < E; ++e) sum[e] = element[e] * element[e];
-    // dimension offsets 16 .. E: the partner sits offset / E lanes away
+  for (uint32_t r = 0; r < R; ++r) {
+    const uint32_t row = first_row + r;
+    if (row >= l.tokens) break;
+    float element[E];
+    float inverse = 1.0f;
+#pragma unroll
+    for (uint32_t e = 0; e < E; ++e) element[e] = bf16_to_f32(raw[r][e]);
+    if (norms) {
+      float sum[E];
+#pragma unroll
+      for (uint32_t e = 0; e < E; ++e) sum[e] = element[e] * element[e];
+      // dimension offsets 16 .. E: the partner sits offset / E lanes away
+#pragma unroll
+      for (uint32_t e = 0; e < E; ++e) {
+        sum[e] = sum[e] + lane_xor<16 / E>(sum[e]);
+        if constexpr (8 >= E) sum[e] = sum[e] + lane_xor<(8 >= E ? 8 / E : 1)>(sum[e]);
+        if constexpr (4 >= E) sum[e] = sum[e] + lane_xor<(4 >= E ? 4 / E : 1)>(sum[e]);
+        if constexpr (2 >= E) sum[e] = sum[e] + lane_xor<(2 >= E ? 2 / E : 1)>(sum[e]);
+        if constexpr (1 >= E) sum[e] = sum[e] + lane_xor<1>(sum[e]);
+      }
+      // dimension offsets below E pair the lane's own elements
+      float group_sum;
+      if constexpr (E == 4) {
+        const float a02 = sum[0] + sum[2], a13 = sum[1] + sum[3];
+        group_sum = a02 + a13;
+      } else if constexpr (E == 2) {
+        group_sum = sum[0] + sum[1];
+      } else {
+        group_sum = sum[0];
+      }
+      // the groups of 32 dimensions in order; a group spans 32 / E lanes
+      float total = 0.0f;
+#pragma unroll
+      for (uint32_t g = 0; g < D / 32; ++g)
+        total = total + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(group_sum), int(g * (32 / E))));
+      const float mean = total / float(D);
+      inverse = 1.0f / sqrtf(mean + p.eps);
+    }
+    uint16_t prepared[E];
 #pragma unroll
     for (uint32_t e = 0; e < E; ++e) {
-      sum[e] = sum[e] + lane_xor<16 / E>(sum[e]);
-      if constexpr (8 >= E) sum[e] = sum[e] + lane_xor<(8 >= E ? 8 / E : 1)>(sum[e]);
-      if constexpr (4 >= E) sum[e] = sum[e] + lane_xor<(4 >= E ? 4 / E : 1)>(sum[e]);
-      if constexpr (2 >= E) sum[e] = sum[e] + lane_xor<(2 >= E ? 2 / E : 1)>(sum[e]);
-      if constexpr (1 >= E) sum[e] = sum[e] + lane_xor<1>(sum[e]);
+      const float unit = element[e] * inverse;
+      const uint16_t normal = f32_to_bf16_hw(unit * scale[e]);
+      const float mine = bf16_to_f32(normal);
+      const float other = __shfl_xor(mine, int(pair_lanes));
+      const float mc = mine * cosine[r][e], os = other * sine[r][e];
+      prepared[e] = rotated ? f32_to_bf16_hw(is_first ? mc - os : mc + os) : normal;
     }
-    // dimension offsets below E pair the lane's own elements
-    float group_sum;
-    if constexpr (E == 4) {
-      const float a02 = sum[0] + sum[2], a13 = sum[1] + sum[3];
-      group_sum = a02 + a13;
-    } else if constexpr (E == 2) {
-      group_sum = sum[0] + sum[1];
-    } else {
-      group_sum = sum[0];
+    if (query) {
+      // A group of one query head has no reciprocal that fits 32 bits (2^32): the head is
+      // its own KV head then.
+      const uint32_t kv_head = G == 1 ? head : __umulhi(head, p.group_magic);
+      const uint32_t local_head = head - kv_head * G;
+      store_bf16s<E>(p.queries + uint64_t(li) * H * p.row_stride * G * D +
+                         ((uint64_t(kv_head) * p.row_stride + row) * G + local_head) * D + d0,
+                     prepared);
+      continue;
     }
-    // the groups of 32 dimensions in order; a group spans 32 / E lanes
-    float total = 0.0f;
-#pragma unroll
-    for (uint32_t g = 0; g < D / 32; ++g)
-      total = total + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(group_sum), int(g * (32 / E))));
-    const float mean = total / float(D);
-    inverse = 1.0f / sqrtf(mean + p.eps);
+    const uint32_t logical = l.committed + row;
+    const Slab s = slab_of(FMT, H, D, a.kv, head, entry[r]);
+    store_row_wave<FMT, E>(prepared, false, s, logical % kPage, lane, D);
+    store_row_wave<FMT, E>(raw_value[r], true, s, logical % kPage, lane, D);
   }
-  uint16_t prepared[E];
-#pragma unroll
-  for (uint32_t e = 0; e < E; ++e) {
-    const float unit = element[e] * inverse;
-    const uint16_t normal = f32_to_bf16_hw(unit * scale[e]);
-    const float mine = bf16_to_f32(normal);
-    const float other = __shfl_xor(mine, int(pair_lanes));
-    const float mc = mine * cosine[e], os = other * sine[e];
-    prepared[e] = rotated ? f32_to_bf16_hw(is_first ? mc - os : mc + os) : normal;
-  }
-  if (query) {
-    // A group of one query head has no reciprocal that fits 32 bits (2^32): the head is
-    // its own KV head then.
-    const uint32_t kv_head = G == 1 ? head : __umulhi(head, p.group_magic);
-    const uint32_t local_head = head - kv_head * G;
-    store_bf16s<E>(p.queries + uint64_t(li) * H * p.row_stride * G * D +
-                       ((uint64_t(kv_head) * p.row_stride + row) * G + local_head) * D + d0,
-                   prepared);
-    return;
-  }
-  const Slab s = slab_of(FMT, H, D, a.kv, head, entry);
-  store_row_wave<FMT, E>(prepared, false, s, logical % kPage, lane, D);
-  store_row_wave<FMT, E>(raw_value, true, s, logical % kPage, lane, D);
 }
 
 // The same store for chunks of many tokens: one workgroup per (lane, logical page
@@ -1747,10 +1762,16 @@ int kv_prepare_append(const kvx_storage *s, uint32_t layer, const kvx_qkv_shape 
       if (by_wave) {
         uint32_t most_rows = 0;
         for (uint32_t i = 0; i < a.n_lanes; ++i) most_rows = std::max(most_rows, lanes[first + i].chunk_tokens);
-        const dim3 grid((QH + H + 3) / 4, most_rows, a.n_lanes), block(256);
-        if (E == 4) hipLaunchKernelGGL((prepare_append_wave_kernel<F, 4>), grid, block, 0, st, p);
-        else if (E == 2) hipLaunchKernelGGL((prepare_append_wave_kernel<F, 2>), grid, block, 0, st, p);
-        else hipLaunchKernelGGL((prepare_append_wave_kernel<F, 1>), grid, block, 0, st, p);
+        // chunks: four rows per wave; a decode or verify step's few rows one each
+        const auto launch = [&](auto rows_per_wave) {
+          constexpr uint32_t R = decltype(rows_per_wave)::value;
+          const dim3 grid((QH + H + 3) / 4, (most_rows + R - 1) / R, a.n_lanes), block(256);
+          if (E == 4) hipLaunchKernelGGL((prepare_append_wave_kernel<F, 4, R>), grid, block, 0, st, p);
+          else if (E == 2) hipLaunchKernelGGL((prepare_append_wave_kernel<F, 2, R>), grid, block, 0, st, p);
+          else hipLaunchKernelGGL((prepare_append_wave_kernel<F, 1, R>), grid, block, 0, st, p);
+        };
+        if (most_rows >= 64) launch(std::integral_constant<uint32_t, 4>{});
+        else launch(std::integral_constant<uint32_t, 1>{});
         return check_launch("prepare_append_wave_kernel");
       }
       hipLaunchKernelGGL((prepare_append_kernel<F>), dim3(groups), dim3(D), 0, st, p);
