@@ -700,7 +700,7 @@ def qkv_prepare(args):
                    "seed": args.seed},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "prepare_append_wave_kernel<int4, 4> (one wave per row and head; bound by its vector instructions)", "bytes_per_launch": chunk_bytes,
+                     "kernel": "prepare_append_wave_kernel<int4, 4, 4> (one wave per head and four rows; bound by its vector instructions)", "bytes_per_launch": chunk_bytes,
                      "ms_per_launch": round(chunk_ms, 4)},
         "kv_append_alone_ms": round(chunk_store_ms, 4),
         "decode_batch32_one_row": {"prepare_append_ms": round(step_ms, 4),
