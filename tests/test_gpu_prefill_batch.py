@@ -73,6 +73,18 @@ def test_equal_chunks_share_their_launches(fmt, committed, rows, planned):
     tw.close()
 
 
+@pytest.mark.parametrize("fmt", [ko.INT4, ko.INT8])
+def test_more_sequences_than_one_launch_takes(fmt):
+    """35 equal chunks: the launches take 32 sequences at a time, the last three their own."""
+    n = 35
+    committed = [32 * (1 + i % 3) for i in range(n)]
+    splits = 2 if fmt == ko.INT8 else 1
+    together, alone, tw = run_batch(fmt, committed, [72] * n, [splits] * n)
+    assert np.array_equal(together, alone)
+    assert (alone[-1] != 0x5A5A).any() and (alone[32] != 0x5A5A).any()
+    tw.close()
+
+
 @pytest.mark.parametrize("fmt", [ko.INT4, ko.BF16])
 def test_unequal_chunks_run_one_after_the_other(fmt):
     committed, rows = [1000, 64, 3000], [77, 264, 8]
