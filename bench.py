@@ -959,8 +959,8 @@ def chunked_prefill(args):
                    "seed": args.seed},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": None,
-                     "kernel": "split kernel of kv_attend_prefill (prefill_int4_kernel or "
-                               "attend_wide_kernel), one sequence and layer per launch",
+                     "kernel": "kv_attend_prefill of one sequence and layer: the split kernel (prefill_int4_kernel or "
+                               "group_wide_kernel) and, with several splits, the merge behind it",
                      "flops_per_launch": flops, "ms_per_launch": round(kernel_ms, 4)},
         "cpu_baseline": None,
     }
