@@ -935,8 +935,19 @@ def chunked_prefill(args):
                            tables[it % sequences], pp, workspace)
     k1.record()
     torch.cuda.synchronize()
-    kernel_ms = k0.elapsed_time(k1) / iters
+    single_ms = k0.elapsed_time(k1) / iters
     flops = 4 * D * QH * sum(prefix + r + 1 for r in range(chunk))
+    kernel_ms, launch_sequences = single_ms, 1
+    if batched:
+        # the launch the step runs: every sequence's tiles in one kv_attend_prefill_batch call
+        k0.record()
+        for it in range(iters):
+            kvx.attend_prefill_batch(storage, it % LAYERS, QH, all_q, all_out, tables, [batch_pp] * sequences,
+                                     H * chunk * G * D, all_ws)
+        k1.record()
+        torch.cuda.synchronize()
+        kernel_ms, launch_sequences = k0.elapsed_time(k1) / iters, sequences
+    flops *= launch_sequences
     achieved = flops / (kernel_ms * 1e-3) / 1e12
     result = {
         "metric": f"{args.format} chunked prefill ({chunk}-token chunks onto a shared 16384-token prefix, "
@@ -959,9 +970,13 @@ def chunked_prefill(args):
                    "seed": args.seed},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": None,
-                     "kernel": "kv_attend_prefill of one sequence and layer: the split kernel (prefill_int4_kernel or "
-                               "group_wide_kernel) and, with several splits, the merge behind it",
-                     "flops_per_launch": flops, "ms_per_launch": round(kernel_ms, 4)},
+                     "kernel": ("kv_attend_prefill_batch of one layer: every sequence's tiles in one launch of "
+                                "the split kernel (prefill_int4_kernel or group_wide_kernel)" if batched else
+                                "kv_attend_prefill of one sequence and layer: the split kernel (prefill_int4_kernel "
+                                "or group_wide_kernel) and, with several splits, the merge behind it"),
+                     "flops_per_launch": flops, "ms_per_launch": round(kernel_ms, 4),
+                     "sequences_per_launch": launch_sequences,
+                     "one_sequence_ms_per_launch": round(single_ms, 4)},
         "cpu_baseline": None,
     }
     storage.close()
