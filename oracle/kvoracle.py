@@ -448,13 +448,14 @@ def attention_tile_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv,
 # is off by d moves its probability by d, relatively.  That deviation is measured, not argued:
 # every split reports the maximum of its scores and the sum of its probabilities, on both sides,
 # and tests/test_gpu_score_deviation.py compares them over 8000 split statistics per format --
-# long histories with 20x outlier channels in the keys, one-row decode and 8-row chains, plain
+# long histories with 20x outlier channels in the keys, one-row decode, 8-row chains and lanes of
+# 12 and 16 rows (the kernels of wide lanes), plain
 # queries and queries that carry the keys' outlier channels too (scores of a hundred and more,
 # harsher than anything else the suite holds).  Worst |max - max| it found:
 #              plain queries   outlier queries
 #   int4         4.8e-05          1.8e-04
 #   int8         1.9e-06          1.2e-04
-#   bf16         1.1e-05          3.1e-04
+#   bf16         1.1e-05          3.4e-04
 #   fp8          5.7e-06          2.8e-04
 # The slack of a format is twice its worst figure; the test holds every new measurement to half
 # of the slack and prints what it measured in the run's summary.  A bf16 place is 3.9e-3 to
@@ -462,7 +463,7 @@ def attention_tile_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv,
 # weights on fp8 pages) is 4.9e-4 to 9.8e-4, so on those pages nearly every weight does, which
 # is what the measurement says: at such scores the fp16 rounding of a weight is not determined
 # by the inputs alone.
-FLIP_SLACK = {INT4: 3.7e-4, INT8: 2.5e-4, BF16: 6.2e-4, FP8: 5.5e-4}
+FLIP_SLACK = {INT4: 3.7e-4, INT8: 2.5e-4, BF16: 6.8e-4, FP8: 5.5e-4}
 
 
 def flip_slack(fmt):
@@ -471,7 +472,7 @@ def flip_slack(fmt):
 
 
 def rounding_flip_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv, head, committed,
-                       active, splits, capacity, fused_row, masks=None, score_scale=0.0, top=32,
+                       active, splits, capacity, fused_row, masks=None, score_scale=0.0, top=64,
                        slack=None, together=2):
     """What one fused row of a tile would be had the rounding of some of its heaviest
     probabilities fallen the other way.  Of the row's `top` heaviest tokens (softmax weight x
@@ -483,7 +484,9 @@ def rounding_flip_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv, 
     How much one turned rounding moves a row: a place of a weight in [0.25, 0.5) is 2^-9, and
     the row is a sum of value rows with weights w, so it moves by about 2^-9 / sqrt(sum w^2) --
     1e-3 to 3e-3 when the attention is spread over some ten heavy tokens, each of which can be
-    the one.  Hence `top` reaches well past the few heaviest.
+    the one.  Hence `top` reaches well past the few heaviest: a row over 150 tokens was moved
+    past the tolerance by its 40th heaviest token (weight 8.4e-3, 1.1e-7 from a tie), exactly one
+    place of that weight in one split's partial row and nothing else.
 
     A kernel that sums q.k in another order than this oracle differs from it in the last bits of
     a score, and so in the rounding of a probability that sits on a rounding boundary; a token
@@ -514,8 +517,11 @@ def rounding_flip_rows(fmt, kv_heads, group, head_dim, tile_queries, table, kv, 
         finally:
             L.ko_attention_flips(-1, None, 0, 0.0, 0)
 
-    _, applied = recompute(heaviest)          # which of them sit on a boundary at all
-    near = [t for i, t in enumerate(heaviest) if applied >> i & 1]
+    near = []                                 # which of them sit on a boundary at all
+    for first in range(0, len(heaviest), 32):  # the tile takes 32 tokens to turn at a time
+        some = heaviest[first:first + 32]
+        _, applied = recompute(some)
+        near += [t for i, t in enumerate(some) if applied >> i & 1]
     for size in range(1, min(together, len(near)) + 1):
         for tokens in itertools.combinations(near, size):
             bits, _ = recompute(list(tokens))
