@@ -304,7 +304,10 @@ class Storage:
             self.h = None
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except TypeError:   # the interpreter is shutting down and this module's names are gone
+            pass
 
     def allocate(self, extent):
         return check(lib().kvx_storage_allocate_extent(self.h, extent))
@@ -551,7 +554,10 @@ class Pool:
             self.h = None
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except TypeError:   # the interpreter is shutting down and this module's names are gone
+            pass
 
     def acquire(self, count):
         out = (C.c_uint32 * max(count, 1))()
@@ -610,7 +616,10 @@ class Prefix:
             self.h = None
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except TypeError:   # the interpreter is shutting down and this module's names are gone
+            pass
 
     def find(self, parent, tokens, images=(0, 0)):
         block, page = C.c_uint64(), C.c_uint32()
@@ -694,7 +703,10 @@ class Sequences:
             self.h = None
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except TypeError:   # the interpreter is shutting down and this module's names are gone
+            pass
 
     def begin(self, sequence):
         return check(lib().kvx_sequence_begin(self.h, sequence))
