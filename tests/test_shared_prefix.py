@@ -13,7 +13,10 @@ rounded to bf16 relative to the running maximum of their split (P = bf16(p x val
 scale), the reference's rule), so another partition into splits rounds every
 probability differently; on random values those roundings do not average out (the
 output is itself a sum of as many random terms), which leaves about 1.5e-3 between
-any two partitions, the oracle's own included.
+any two partitions, the oracle's own included, and up to 4.5e-3 on sequences of under a
+hundred tokens (a seeded search over random shapes: int8 pages, a prefix of one or two pages;
+the oracle's two arrangements lay exactly as far apart as the library's).  So the library is
+held to the oracle's own distance between the two arrangements, row by row, plus the bar.
 """
 import numpy as np
 import pytest
@@ -110,7 +113,9 @@ def test_shared_prefix_decode_matches_oracle(fmt, shared_pages, own_tokens, pref
     # the ordinary decode of every sequence, another partition: see the module's note
     value = lambda bits: ko.bf16_to_f32(bits).reshape(bits.shape).astype(np.float64)
     apart = np.linalg.norm(value(got) - value(want), axis=-1) / np.linalg.norm(value(want), axis=-1)
-    assert apart.max() <= 2 * A.tol(fmt), apart.max()
+    between = np.linalg.norm(value(same) - value(want), axis=-1) / np.linalg.norm(value(want), axis=-1)
+    # no farther from the ordinary decode than the oracle's own shared arrangement is, plus the bar
+    assert (apart <= between + A.tol(fmt)).all(), (apart.max(), between.max())
     # the unshared entry over the same tables
     plain = torch.zeros_like(out)
     up = [kvx.VerifyParams(committed[i], entries[i], kvx.KvLayer(), kvx.lib().kvx_decode_splits(committed[i], 1),
@@ -121,7 +126,7 @@ def test_shared_prefix_decode_matches_oracle(fmt, shared_pages, own_tokens, pref
     a = ko.bf16_to_f32(got).reshape(got.shape).astype(np.float64)
     b = ko.bf16_to_f32(Gp.host_u16(plain)[:, :, 0]).reshape(got.shape).astype(np.float64)
     relative = np.linalg.norm(a - b, axis=-1) / np.linalg.norm(b, axis=-1)
-    assert relative.max() <= 2 * A.tol(fmt), relative.max()
+    assert (relative <= between + 2 * A.tol(fmt)).all(), (relative.max(), between.max())
     # the same call again gives the same bits
     again = torch.zeros_like(out)
     kvx.attend_decode_shared(tw.dev, 1, QH, Gp.dev(q), again, dts, dp, shared_pages, prefix_splits, 1, ws)
