@@ -3,6 +3,8 @@ and statistics go to the library's static device array instead of a caller's wor
 output must be kv_attend_decode's, bit for bit (the same kernels over other scratch memory), on
 two calls in a row, the second with a smaller batch, and sizes past the array are refused with
 nothing enqueued."""
+import gc
+
 import numpy as np
 import pytest
 import torch
@@ -33,11 +35,16 @@ def test_static_workspace_decode_is_the_workspace_decode():
                           dp[first:first + count], 1, ws)
         got = torch.full_like(want, 0x5A5A)
         torch.cuda.synchronize()
-        allocated = torch.cuda.memory_allocated()
+        # Tensors that earlier tests left in reference cycles must not be released between the
+        # two readings; free device memory as the driver reports it also sees an allocation that
+        # does not go through torch.
+        gc.collect()
+        allocated, free = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
         kvx.attend_decode_static(tw.dev, 1, QH, q[first:first + count], got, dts[first:first + count],
                                  dp[first:first + count], 1)
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() == allocated
+        assert torch.cuda.mem_get_info()[0] == free
         assert torch.equal(got, want)
         return got
 
