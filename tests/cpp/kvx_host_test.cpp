@@ -118,6 +118,13 @@ void testPlans() {
   const auto sized = ops::PagedAttention::prefillPlan(16384, 256, 24, layout);
   EXPECT(sized.splits > 1 && sized.splits <= 32);
   EXPECT(sized.workspace.partialsBytes == uint64_t(32) * sized.splits * 8 * 24 * 256 * 4);
+  // int4 pages: 2048 rows alone take four splits (three full rounds of wave slots), four such
+  // chunks in one batched call fill them in one split each
+  const Layout int4Layout{16, 4, 256, Format::Int4};
+  EXPECT(ops::PagedAttention::prefillPlan(16384, 2048, 24, int4Layout).splits == 4);
+  EXPECT(ops::PagedAttention::prefillPlan(16384, 2048, 24, int4Layout, 4).splits == 1);
+  EXPECT(throws<std::invalid_argument>(
+      [&] { (void)ops::PagedAttention::prefillPlan(16384, 2048, 24, int4Layout, 0); }));
   const auto bound = ops::PagedAttention::prefillWorkspace(2048, 24, layout);
   EXPECT(bound.partialsBytes >= full.workspace.partialsBytes);
   const auto verify = ops::PagedAttention::verifyPlan(2, 24, layout, {0, 131072});
