@@ -21,8 +21,7 @@ def pytest_sessionstart(session):
 def pytest_terminal_summary(terminalreporter):
     """How often the attention checks needed their one allowance (a row one rounding flip
     away from the oracle, proven by recomputation): per check and in total; also written as
-    parity_allowance.txt into the folder KVX_TEST_REPORT_DIR names (default: the run's output
-    folder at the repository root) where that folder exists."""
+    parity_allowance.txt into the folder KVX_TEST_REPORT_DIR names, where that is set and exists."""
     gpulib = sys.modules.get("gpulib")
     log = getattr(gpulib, "ALLOWANCE_LOG", None)
     if not log and not getattr(gpulib, "DEVIATION_LOG", None):
@@ -38,7 +37,7 @@ def pytest_terminal_summary(terminalreporter):
     lines += [f"  {n:4d} of {total:6d}  {label}" for label, n, total in log if n]
     lines += measured
     terminalreporter.write_line("\n".join(lines))
-    out = os.environ.get("KVX_TEST_REPORT_DIR", os.path.join(ROOT, "gpurun_out"))
-    if os.path.isdir(out):
+    out = os.environ.get("KVX_TEST_REPORT_DIR")
+    if out and os.path.isdir(out):
         with open(os.path.join(out, "parity_allowance.txt"), "w") as f:
             f.write("\n".join(lines) + "\n")
