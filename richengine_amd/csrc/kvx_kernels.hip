@@ -900,7 +900,13 @@ struct SmallChunk {
   }
 };
 
-template <uint32_t FMT, uint32_t D, uint32_t BLOCKS>
+// PRIVATE = 0: the four waves of the workgroup share the tile (row blocks by wave, the page
+// staged by all 256 threads, a barrier on either side of the staging).  PRIVATE = n: the
+// workgroup is n independent waves, each with a tile of at most 16 fused rows (one-row decode,
+// short chains of small groups) and a staged copy of its own: a wave's LDS operations complete
+// in the order it issues them, so it needs no barrier, and every wave of a CU multiplies
+// instead of one in four.
+template <uint32_t FMT, uint32_t D, uint32_t BLOCKS, uint32_t PRIVATE = 0>
 __device__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
                                      const uint64_t *__restrict__ table, kvx_kv_layer kv,
                                      uint32_t H, uint32_t G, uint32_t row_capacity, uint32_t head,
@@ -913,11 +919,21 @@ __device__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
   constexpr uint32_t kKeyRow = D + 8;        // staged halves per token: 16 bytes past a power of two
   constexpr uint32_t kValueRow = kPage + 4;  // staged halves per dimension
   constexpr uint32_t kSteps = D / 32, kTiles = D / 16;
-  __shared__ __align__(16) uint16_t k_lds[kPage * kKeyRow];
-  __shared__ __align__(16) uint16_t v_lds[D * kValueRow];
-  __shared__ float key_scale_lds[kPage], value_scale_lds[kPage];
+  static_assert(!PRIVATE || BLOCKS == 1, "a private tile is one block of 16 fused rows");
+  constexpr uint32_t kCopies = PRIVATE ? PRIVATE : 1, kThreads = PRIVATE ? 64u : kTileThreads;
+  __shared__ __align__(16) uint16_t k_lds_all[kCopies][kPage * kKeyRow];
+  __shared__ __align__(16) uint16_t v_lds_all[kCopies][D * kValueRow];
+  __shared__ float key_scale_all[kCopies][kPage], value_scale_all[kCopies][kPage];
+  const uint32_t copy = PRIVATE ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0u;
+  uint16_t *const k_lds = k_lds_all[copy], *const v_lds = v_lds_all[copy];
+  float *const key_scale_lds = key_scale_all[copy], *const value_scale_lds = value_scale_all[copy];
+  const auto tile_barrier = [] {
+    if constexpr (PRIVATE) __builtin_amdgcn_wave_barrier();
+    else __syncthreads();
+  };
 
-  const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, t = lane & 15u, g = lane >> 4;
+  const uint32_t lane = threadIdx.x & 63u, t = lane & 15u, g = lane >> 4;
+  const uint32_t tid = PRIVATE ? lane : threadIdx.x, wave = PRIVATE ? 0u : threadIdx.x >> 6;
   const uint32_t M = row_capacity * G;
   const uint32_t visible = committed + active_rows;
   const uint32_t pages = (visible + kPage - 1) / kPage;
@@ -965,15 +981,15 @@ __device__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
   // elements: keys [token][dim], values [dim][token].
   using Chunk = SmallChunk<FMT>;
   constexpr uint32_t kPieces = kPage * D / Chunk::kElements;         // per tensor
-  constexpr uint32_t kPerThread = (kPieces + kTileThreads - 1) / kTileThreads;
+  constexpr uint32_t kPerThread = (kPieces + kThreads - 1) / kThreads;
   small_u32x4 raw_keys[kPerThread], raw_values[kPerThread];
   float raw_scale = 1.0f;
   const auto fetch = [&](uint32_t page) {
     const Slab s = slab_of(FMT, H, D, kv, head, table[page]);
 #pragma unroll
     for (uint32_t i = 0; i < kPerThread; ++i) {
-      const uint32_t piece = tid + i * kTileThreads;
-      if (kPieces % kTileThreads == 0 || piece < kPieces) {
+      const uint32_t piece = tid + i * kThreads;
+      if (kPieces % kThreads == 0 || piece < kPieces) {
         raw_keys[i] = *reinterpret_cast<const small_u32x4 *>(s.keys + 16 * piece);
         raw_values[i] = *reinterpret_cast<const small_u32x4 *>(s.values + 16 * piece);
       }
@@ -984,8 +1000,8 @@ __device__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
   const auto stage = [&]() {
 #pragma unroll
     for (uint32_t i = 0; i < kPerThread; ++i) {
-      const uint32_t piece = tid + i * kTileThreads;
-      if (kPieces % kTileThreads != 0 && piece >= kPieces) continue;
+      const uint32_t piece = tid + i * kThreads;
+      if (kPieces % kThreads != 0 && piece >= kPieces) continue;
       const uint32_t first = piece * Chunk::kElements;
       {  // keys are token-major in every format
         const Chunk c(raw_keys[i]);
@@ -1017,10 +1033,10 @@ __device__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
   fetch(begin);
   for (uint32_t page = begin; page < end; ++page) {
     const uint32_t token_start = page * kPage;
-    __syncthreads();  // the previous page's products are done with the staged copy
+    tile_barrier();  // the previous page's products are done with the staged copy
     stage();
     if (page + 1 < end) fetch(page + 1);
-    __syncthreads();
+    tile_barrier();
 
 #pragma unroll
     for (uint32_t b = 0; b < BLOCKS; ++b) {
@@ -1118,6 +1134,28 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(BL
                                l.committed, l.active_rows, l.split_count, split, partials,
                                statistics, slot_row,
                                row_masks ? row_masks + l.mask_offset : nullptr, l.score_scale);
+}
+
+// Tiles of at most 16 fused rows: a wave per (split, KV head, lane), PRIVATE of them to a
+// workgroup (what the staged copies leave room for: 18 KiB a wave at head dimension 128).
+template <uint32_t D>
+constexpr uint32_t kSmallPrivateWaves = D == 128 ? 2 : 4;
+template <uint32_t FMT, uint32_t D>
+__global__ __launch_bounds__(64 * kSmallPrivateWaves<D>) void attend_split_small_wave_kernel(
+    const uint16_t *__restrict__ queries, float *__restrict__ partials,
+    float *__restrict__ statistics, const uint32_t *__restrict__ row_masks, AttendArgs a) {
+  constexpr uint32_t kWaves = kSmallPrivateWaves<D>;
+  const uint32_t split = kWaves * blockIdx.x + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t head = blockIdx.y, li = blockIdx.z;
+  const AttendLane &l = a.lane[li];
+  if (!attend_contract(l, a) || split >= l.split_count) return;
+  const uint32_t M = a.row_capacity * a.group;
+  const uint16_t *tile_q = queries + l.q_offset + uint64_t(head) * a.row_stride * a.group * D;
+  const uint64_t slot_row = l.row_base + (uint64_t(head) * l.split_count + split) * M;
+  attention_tile_small<FMT, D, 1, kWaves>(tile_q, l.table, a.kv, a.kv_heads, a.group, a.row_capacity, head,
+                                          l.committed, l.active_rows, l.split_count, split, partials,
+                                          statistics, slot_row,
+                                          row_masks ? row_masks + l.mask_offset : nullptr, l.score_scale);
 }
 
 template <uint32_t FMT, uint32_t D, uint32_t BLOCKS>
@@ -1877,6 +1915,15 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
                              static_cast<const uint16_t *>(queries), partials, statistics, row_masks, a);
         };
         constexpr uint32_t F = decltype(fmt)::value;
+        if (M <= 16) {  // one wave per tile
+          const auto wave_launch = [&](auto kernel, uint32_t waves) {
+            hipLaunchKernelGGL(kernel, dim3((max_splits + waves - 1) / waves, H, a.n_lanes), dim3(64 * waves), 0,
+                               stream, static_cast<const uint16_t *>(queries), partials, statistics, row_masks, a);
+          };
+          if (D == 64) wave_launch(attend_split_small_wave_kernel<F, 64>, kSmallPrivateWaves<64>);
+          else wave_launch(attend_split_small_wave_kernel<F, 128>, kSmallPrivateWaves<128>);
+          return check_launch("attend_split_small_wave_kernel");
+        }
         if (D == 64 && M <= 64) launch(attend_split_small_kernel<F, 64, 1>);
         else if (D == 64) launch(attend_split_small_kernel<F, 64, 2>);
         else if (M <= 64) launch(attend_split_small_kernel<F, 128, 1>);

@@ -337,6 +337,12 @@ def test_hot_kernels_stay_out_of_scratch_memory():
         assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, r
     r = one("group_wide_kernelILj2ELj3ELj2ELb0E")      # bf16, two waves of 48 rows, direct loads
     assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, r
+    # head dimensions 64 and 128, a wave per tile: no scratch, and two (128) or three and more
+    # (64) waves per SIMD beside the staged copies
+    for fmt in (1, 2, 3, 4):
+        for dim, least in ((128, 2), (64, 3)):
+            r = one(f"attend_split_small_wave_kernelILj{fmt}ELj{dim}E")
+            assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0 and r["occupancy"] >= least, (fmt, dim, r)
     # the kernels whose accumulators fill the second register file (48-row verify, two-block
     # bf16): since their rescaling names the accumulators there, nothing spills
     for fragment in ("verify48_int4_kernel", "attend_wide_kernelILj2ELj2ELj1ELb0E",
