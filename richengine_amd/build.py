@@ -16,6 +16,11 @@ SOURCES = ["kvx_host.cpp", "kvx_pool.cpp", "kvx_pool_abi.cpp", "kvx_prefix.cpp",
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall",
          # packed fp32 instructions stay off for every kernel of this library
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         # no fused multiply-adds but the ones the sources spell out (fmaf): the oracle is built the
+         # same way, and a product fused into the difference behind it turns a score minus the
+         # maximum it equals into the product's rounding error (__fmul_rn and its like are plain
+         # operators in HIP's headers and fuse like any other, whatever pragma surrounds the call)
+         "-ffp-contract=off",
          "-I", os.path.join(ROOT, "include"), "-I", CSRC]
 # What the compiler reports per kernel (registers, scratch bytes per lane, spills,
 # waves per SIMD) goes to this file next to the library, so that a change that
