@@ -918,11 +918,17 @@ __device__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
   constexpr bool kQuant = FMT != KVX_FMT_BF16;
   constexpr uint32_t kKeyRow = D + 8;        // staged halves per token: 16 bytes past a power of two
   constexpr uint32_t kValueRow = kPage + 4;  // staged halves per dimension
+  // Where dimension d's staged values begin.  int4 values lie token-major in the page, and a
+  // thread that holds 32 dimensions of a token writes them two bytes at a time, the threads of
+  // a wave 32 dimensions apart: a multiple of 32 rows is a multiple of 32 banks whatever the
+  // row length, so every group of 32 rows starts 16 halves (8 banks) further on.
+  constexpr uint32_t kValueSkew = FMT == KVX_FMT_INT4 ? 16u : 0u;
+  const auto value_row = [](uint32_t d) { return d * kValueRow + (d >> 5) * kValueSkew; };
   constexpr uint32_t kSteps = D / 32, kTiles = D / 16;
   static_assert(!PRIVATE || BLOCKS == 1, "a private tile is one block of 16 fused rows");
   constexpr uint32_t kCopies = PRIVATE ? PRIVATE : 1, kThreads = PRIVATE ? 64u : kTileThreads;
   __shared__ __align__(16) uint16_t k_lds_all[kCopies][kPage * kKeyRow];
-  __shared__ __align__(16) uint16_t v_lds_all[kCopies][D * kValueRow];
+  __shared__ __align__(16) uint16_t v_lds_all[kCopies][D * kValueRow + (D / 32) * 16];
   __shared__ float key_scale_all[kCopies][kPage], value_scale_all[kCopies][kPage];
   const uint32_t copy = PRIVATE ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0u;
   uint16_t *const k_lds = k_lds_all[copy], *const v_lds = v_lds_all[copy];
@@ -1016,11 +1022,11 @@ __device__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
         const uint32_t token = first / D, d0 = first % D;
 #pragma unroll
         for (uint32_t w = 0; w < Chunk::kElements / 2; ++w) {
-          v_lds[(d0 + 2 * w) * kValueRow + token] = uint16_t(c.pair[w]);
-          v_lds[(d0 + 2 * w + 1) * kValueRow + token] = uint16_t(c.pair[w] >> 16);
+          v_lds[value_row(d0 + 2 * w) + token] = uint16_t(c.pair[w]);
+          v_lds[value_row(d0 + 2 * w + 1) + token] = uint16_t(c.pair[w] >> 16);
         }
       } else {  // dimension-major values: a run of tokens of one dimension
-        uint32_t *to = reinterpret_cast<uint32_t *>(&v_lds[(first / kPage) * kValueRow + first % kPage]);
+        uint32_t *to = reinterpret_cast<uint32_t *>(&v_lds[value_row(first / kPage) + first % kPage]);
 #pragma unroll
         for (uint32_t w = 0; w < Chunk::kElements / 2; w += 2)
           *reinterpret_cast<small_u32x2 *>(to + w) = small_u32x2{c.pair[w], c.pair[w + 1]};
@@ -1093,7 +1099,7 @@ __device__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
       }
 #pragma unroll
       for (uint32_t i = 0; i < kTiles; ++i) {
-        const uint16_t *row = &v_lds[(16 * i + t) * kValueRow + 4 * g];
+        const uint16_t *row = &v_lds[value_row(16 * i + t) + 4 * g];
         const small_u32x2 lo = *reinterpret_cast<const small_u32x2 *>(row);
         const small_u32x2 hi = *reinterpret_cast<const small_u32x2 *>(row + 16);
         acc[b][i] = small_mfma<kFp8>(small_u32x4{lo[0], lo[1], hi[0], hi[1]}, weights, acc[b][i]);
