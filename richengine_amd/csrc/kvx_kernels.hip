@@ -907,7 +907,7 @@ struct SmallChunk {
 // in the order it issues them, so it needs no barrier, and every wave of a CU multiplies
 // instead of one in four.
 template <uint32_t FMT, uint32_t D, uint32_t BLOCKS, uint32_t PRIVATE = 0>
-__device__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
+__device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
                                      const uint64_t *__restrict__ table, kvx_kv_layer kv,
                                      uint32_t H, uint32_t G, uint32_t row_capacity, uint32_t head,
                                      uint32_t committed, uint32_t active_rows, uint32_t splits,

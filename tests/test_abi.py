@@ -343,6 +343,14 @@ def test_hot_kernels_stay_out_of_scratch_memory():
         for dim, least in ((128, 2), (64, 3)):
             r = one(f"attend_split_small_wave_kernelILj{fmt}ELj{dim}E")
             assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0 and r["occupancy"] >= least, (fmt, dim, r)
+    # the same tiles shared by four waves (verify and prefill of more than 16 fused rows): the tile
+    # is inlined into its kernels; called as a function it cost them 200 to 300 bytes of stack
+    for kernel in ("attend_split_small_kernel", "prefill_split_small_kernel"):
+        for fmt in (1, 2, 3, 4):
+            for dim in (128, 64):
+                for blocks in (1, 2):
+                    r = one(f"{kernel}ILj{fmt}ELj{dim}ELj{blocks}E")
+                    assert r["scratchsize"] == 0 and r["vgprs_spill"] == 0, (kernel, fmt, dim, blocks, r)
     # the kernels whose accumulators fill the second register file (48-row verify, two-block
     # bf16): since their rescaling names the accumulators there, nothing spills
     for fragment in ("verify48_int4_kernel", "attend_wide_kernelILj2ELj2ELj1ELb0E",
