@@ -646,7 +646,7 @@ constexpr uint32_t kKeyPitch = kMaxD + 2;  // bf16 elements; odd word pitch avoi
 // K and V codes are staged in LDS as bf16, which holds every int4 / int8 /
 // e4m3 / bf16 code exactly.
 template <uint32_t FMT, uint32_t MAXM>
-__device__ void attention_tile(const uint16_t *__restrict__ tile_queries,
+__device__ __forceinline__ void attention_tile(const uint16_t *__restrict__ tile_queries,
                                const uint64_t *__restrict__ table, kvx_kv_layer kv,
                                uint32_t H, uint32_t G, uint32_t D, uint32_t row_capacity,
                                uint32_t head, uint32_t committed, uint32_t active_rows,
@@ -1184,7 +1184,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(BL
 // Fixed-order merge of one fused row's splits (reference:
 // common/paged_attention_tile.h:362-417).  head_dim threads, one per dimension;
 // returns the thread's bf16 element, zero for rows past the live ones.
-__device__ uint16_t reduce_row(const float *__restrict__ partials,
+__device__ __forceinline__ uint16_t reduce_row(const float *__restrict__ partials,
                                const float *__restrict__ statistics, uint32_t G, uint32_t D,
                                uint32_t M, uint32_t committed, uint32_t active_rows,
                                uint32_t splits, uint64_t head_row, uint32_t fused_row) {
