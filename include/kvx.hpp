@@ -380,7 +380,7 @@ public:
   }
   // decode = true selects the batched-decode split rule of this library
   // (rows = 1 per lane, one split per 32 visible pages).  sizedForGpu = true
-  // takes the split counts from kvx_decode_plan / kvx_verify_plan, which look at
+  // takes the split counts from kvx_decode_plan_for / kvx_verify_plan, which look at
   // the whole batch and give the launch one round of waves, instead of the
   // reference's per-lane rules.
   static VerifyAttentionPlan verifyPlan(uint32_t lanes, uint32_t queryHeads, kv::Layout layout,
@@ -395,8 +395,8 @@ public:
     VerifyAttentionPlan plan{layout.format, lanes, {}, 0, {}, rows, queryHeads, layout.scoreScale};
     if (sizedForGpu) {
       plan.laneSplits.resize(lanes);
-      check(decode ? kvx_decode_plan(historyTokens.data(), lanes, layout.kvHeads,
-                                     static_cast<uint32_t>(layout.format), plan.laneSplits.data())
+      const kvx_layout l = layout.c();
+      check(decode ? kvx_decode_plan_for(&l, historyTokens.data(), lanes, plan.laneSplits.data())
                    : kvx_verify_plan(historyTokens.data(), lanes, rows, layout.kvHeads, queryHeads,
                                      static_cast<uint32_t>(layout.format), plan.laneSplits.data()));
       for (uint32_t splits : plan.laneSplits) plan.splits = std::max(plan.splits, splits);

@@ -336,6 +336,37 @@ int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_hea
                           format, split_counts + first);
   return KVX_OK;
 }
+int kvx_decode_plan_for(const kvx_layout *layout, const uint32_t *committed, uint32_t n_lanes,
+                        uint32_t *split_counts) {
+  if (!kvx_layout_valid(layout)) return fail(KVX_EINVAL, "kvx_decode_plan_for: invalid layout");
+  if (layout->head_dim != 64 && layout->head_dim != 128)
+    return kvx_decode_plan(committed, n_lanes, layout->kv_heads, layout->format, split_counts);
+  if (!committed || !split_counts || !n_lanes)
+    return fail(KVX_EINVAL, "kvx_decode_plan_for: null argument or empty batch");
+  for (uint32_t i = 0; i < n_lanes; ++i)
+    if (uint64_t(committed[i]) + 1 > KVX_MAX_PHYSICAL_TOKENS)
+      return fail(KVX_EINVAL, "kvx_decode_plan_for: context_out_of_range");
+  // Head dimensions 64 and 128: a wave per (lane, KV head, split) over a staged copy of its
+  // own, eight waves to a CU at head dimension 128 and sixteen at 64 (what the copies leave
+  // room for); one round of them, splits of at least 4 pages (32 sequences of 8192 tokens,
+  // 2 x 8 x 128: 63 us at 32 splits, 84 at 16; 8 x 4 x 64: 90 us at 16, 93 at 32).  bf16 pages
+  // are read at close to the memory's rate with half as many waves, and the other half only
+  // adds partial rows (2 x 8 x 128: 59 us at 16 splits, 70 at 32; 8 x 4 x 64: 119 at 8, 131 at 16).
+  const uint64_t slots = (layout->head_dim == 128 ? 2048 : 4096) / (layout->format == KVX_FMT_BF16 ? 2 : 1);
+  for (uint32_t first = 0; first < n_lanes; first += KVX_LANES_PER_LAUNCH) {
+    const uint32_t count = std::min(KVX_LANES_PER_LAUNCH, n_lanes - first);
+    uint64_t page_heads = 0;
+    for (uint32_t i = 0; i < count; ++i)
+      page_heads += uint64_t(pages_of(uint64_t(committed[first + i]) + 1)) * layout->kv_heads;
+    const uint64_t per = std::max<uint64_t>((page_heads + slots - 1) / slots, 4);
+    for (uint32_t i = 0; i < count; ++i) {
+      const uint64_t pages = pages_of(uint64_t(committed[first + i]) + 1);
+      split_counts[first + i] =
+          uint32_t(std::min<uint64_t>(std::max<uint64_t>(1, (pages + per - 1) / per), KVX_VERIFY_MAX_SPLITS));
+    }
+  }
+  return KVX_OK;
+}
 // The verify plan of the lanes of one launch (at most KVX_LANES_PER_LAUNCH).
 static void verify_plan_of_launch(const uint32_t *committed, uint32_t n_lanes, uint32_t rows,
                                   uint32_t kv_heads, uint32_t query_heads, uint32_t format,

@@ -36,7 +36,7 @@ SYMBOLS = [
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
     "kvx_pool_snapshot_get", "kv_append", "kv_prepare_append", "kv_attend_decode_shared", "kvx_attend_shared_workspace_bytes", "kv_attend_verify", "kv_attend_verify_hidden", "kv_attend_decode",
     "kv_attend_prefill", "kv_attend_prefill_batch", "kv_compact_path", "kv_append_attend_decode", "kv_append_attend_decode_hidden", "kv_page_export", "kv_page_import", "kv_attend_split", "kv_attend_merge", "kv_attend_decode_static",
-    "kvx_debug_attend_paths", "kvx_calibrate_stream", "kvx_decode_plan", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
+    "kvx_debug_attend_paths", "kvx_calibrate_stream", "kvx_decode_plan", "kvx_decode_plan_for", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
     "kvx_prefix_chain", "kvx_prefix_retain_active", "kvx_prefix_release_active",
     "kvx_prefix_touch", "kvx_prefix_eviction_candidate", "kvx_prefix_erase",
@@ -201,6 +201,7 @@ def _declare(L):
     L.kvx_calibrate_stream.argtypes = [vp, u32, vp, u32, u32, u32, vp, vp]
     L.kvx_calibrate_stream_form.argtypes = [vp, u32, vp, u32, u32, u32, u32, u32, vp, vp]
     L.kvx_decode_plan.argtypes = [vp, u32, u32, u32, vp]
+    L.kvx_decode_plan_for.argtypes = [LP, vp, u32, vp]
     L.kvx_verify_plan.argtypes = [vp, u32, u32, u32, u32, u32, vp]
     L.kvx_tree_masks.argtypes = [vp, u32, vp]
     L.kvx_tree_path_valid.argtypes = [vp, u32, vp, u32]
@@ -785,6 +786,13 @@ def decode_plan(committed, kv_heads, fmt=INT4):
     """Split counts of a decode batch of pages of format `fmt` (kvx_decode_plan)."""
     out = (C.c_uint32 * len(committed))()
     check(lib().kvx_decode_plan(_u32(committed), len(committed), kv_heads, fmt, out))
+    return list(out)
+
+
+def decode_plan_for(storage, committed):
+    """Split counts of a decode batch sized for the GPU and the storage's layout (kvx_decode_plan_for)."""
+    out = (C.c_uint32 * len(committed))()
+    check(lib().kvx_decode_plan_for(C.byref(storage.layout), _u32(committed), len(committed), out))
     return list(out)
 
 

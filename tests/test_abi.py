@@ -192,6 +192,21 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
             assert plan == sum((verify_rule(g, rows, fmt) for g in groups), [])
             counts = [pages(c + rows) for c in committed]
             assert all(1 <= s <= 128 and s <= max(n, 1) for s, n in zip(plan, counts))
+    # by layout: head dimension 256 is the plan above; 128 and 64 plan one round of single waves
+    import ctypes as C
+    for heads, dim, fmt, want in ((4, 256, kvx.INT4, kvx.decode_plan([8191] * 32, 4, kvx.INT4)),
+                                  (2, 128, kvx.INT4, [32] * 32),    # 256 pages x 2 heads x 32 lanes on 2048 waves: 8 pages a split
+                                  (8, 64, kvx.INT8, [16] * 32),     # 256 x 8 x 32 on 4096: 16 pages a split
+                                  (2, 128, kvx.BF16, [16] * 32)):    # bf16 pages: half the waves
+        layout = kvx.Layout(1, heads, dim, fmt, 0.0)
+        out = (C.c_uint32 * 32)()
+        kvx.check(kvx.lib().kvx_decode_plan_for(C.byref(layout), (C.c_uint32 * 32)(*([8191] * 32)), 32, out))
+        assert list(out) == want, (heads, dim, list(out)[:3])
+    layout = kvx.Layout(1, 2, 128, kvx.INT4, 0.0)
+    out = (C.c_uint32 * 2)()
+    kvx.check(kvx.lib().kvx_decode_plan_for(C.byref(layout), (C.c_uint32 * 2)(0, 100000), 2, out))
+    assert list(out) == [1, 128]                                  # at most 128 splits, at least 4 pages each
+    assert kvx.lib().kvx_decode_plan_for(C.byref(layout), (C.c_uint32 * 1)(262144 + 15), 1, out) != 0
     # a small launch takes shorter splits: one sequence of 8192 tokens, 64 splits of 4 pages
     assert kvx.decode_plan([8191], H, kvx.INT4) == [64] and kvx.decode_plan([8191], H, kvx.INT8) == [64]
     assert kvx.decode_plan([8191] * 3, H, kvx.INT4) == [64] * 3 and kvx.decode_plan([8191] * 3, H, kvx.BF16) == [32] * 3

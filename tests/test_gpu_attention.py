@@ -325,12 +325,13 @@ def test_int4_small_tree_verify_in_one_wave(nodes, capacity):
     tw.close()
 
 
-def decode_case(fmt, committed, seed, row_stride=1, layers=2, layer=1):
+def decode_case(fmt, committed, seed, row_stride=1, layers=2, layer=1, planned=False):
     lanes = len(committed)
     tw, counts, hts, dts = shared_pool_lanes(fmt, committed, 1, seed=seed, layers=layers, layer=layer)
     q = np.zeros((lanes, H, row_stride, G, D), dtype=np.uint16)
     q[:, :, 0] = queries((lanes, H, G, D), seed)
-    splits = [kvx.lib().kvx_decode_splits(c, 1) for c in committed]
+    splits = (kvx.decode_plan_for(tw.dev, committed) if planned
+              else [kvx.lib().kvx_decode_splits(c, 1) for c in committed])
     want = np.zeros((lanes, H, G, D), dtype=np.uint16)
     want32 = np.zeros((lanes, H, G, D), dtype=np.float32)
     for i in range(lanes):
@@ -363,6 +364,22 @@ def decode_case(fmt, committed, seed, row_stride=1, layers=2, layer=1):
 @pytest.mark.parametrize("fmt", FORMATS)
 def test_decode_matches_oracle(fmt):
     decode_case(fmt, [0, 1, 31, 32, 511, 512, 1000, 2047, 4095, 600, 33, 5000], seed=80 + fmt)
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("heads,group,dim", [(2, 8, 128), (8, 4, 64)])
+def test_decode_under_the_plan_of_its_layout(fmt, heads, group, dim):
+    """kvx_decode_plan_for's splits (one round of single waves at head dimensions 64 and 128)
+    over ragged lanes, more of them than one launch takes."""
+    global H, G, D, QH
+    saved = (H, G, D, QH)
+    H, G, D, QH = heads, group, dim, heads * group
+    try:
+        rng = np.random.default_rng(dim + fmt)
+        committed = [0, 31, 32, 127, 128, 4095] + [int(x) for x in rng.integers(0, 2500, 30)]
+        decode_case(fmt, committed, seed=300 + fmt + dim, planned=True)
+    finally:
+        H, G, D, QH = saved
 
 
 @pytest.mark.parametrize("row_stride", [1, 32])
