@@ -82,13 +82,14 @@ def parse():
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
     ap.add_argument("--workload", choices=["decode", "decode-single", "tree-verify", "prefill", "qkv-prepare", "shared-prefix",
-                                           "stream-ceiling"], default="decode",
+                                           "stream-ceiling", "control-plane"], default="decode",
                     help="decode = batch-32 mixed-length int4 decode, the headline metric (default); "
                          "decode-single = one sequence of 32768 tokens, the 16 per-layer calls replayed "
                          "as one HIP graph; tree-verify = 16-node tree verify and prefill = chunked prefill with a shared "
                          "prefix, the matrix-core paths (profiling); stream-ceiling = what the memory system "
                          "delivers for the headline batch's bytes under request shapes other than the "
-                         "decode kernel's (linear, 16-byte coalesced, page order, pool size)")
+                         "decode kernel's (linear, 16-byte coalesced, page order, pool size); control-plane = "
+                         "the host calls of a batch-32 step (prefix page cache, sequence records), no GPU work")
     ap.add_argument("--format", choices=["bf16", "fp8", "int8", "int4"], default=None,
                     help="page format of the prefill workload (default bf16) and of the shared-prefix "
                          "and tree-verify workloads (default int4; no fp8)")
@@ -827,6 +828,200 @@ def shared_prefix(args):
     print(json.dumps(result))
 
 
+def control_plane(args):
+    """The host side of a serving step at batch 32, no GPU work: the prefix page cache and the
+    sequence records (kvx_prefix_*, kvx_sequence_*) over an accounting-only storage of the
+    benchmark's layout.  32 requests of 16 384 prompt tokens whose first 8192 are shared are
+    admitted (match, restore, then chunks of 2048 tokens: pages, publish, page list), decode
+    `--steps` x 32 steps of one token (pages, publish, page list per sequence), run as many
+    16-row tree-verify steps (pages for the tree, publish what was accepted, truncate) and
+    end (every block evicted).  The calls go through ctypes with arguments built beforehand;
+    the cost of an empty ctypes call is measured beside them and `value` is the decode step
+    with that taken off.  The CPU baseline is the oracle's restatement of the reference's
+    cache (Python over the oracle's page pool) on a shorter run of the same steps."""
+    import random
+    import time
+    from richengine_amd import kvx
+
+    L = kvx.lib()
+    rng = random.Random(args.seed)
+    sequences, shared, prompt_tokens, chunk = 32, 8192, 16384, 2048
+    steps = max(32 * args.steps, 32)
+    most = prompt_tokens + 2 * steps * 6 + 64
+    pages = sequences * ((most + 31) // 32 + 1)
+    extent_pages = 1024
+    pages = (pages + extent_pages - 1) // extent_pages * extent_pages
+    prefix_tokens = [rng.randrange(150000) for _ in range(shared)]
+    streams = [prefix_tokens + [rng.randrange(150000) for _ in range(most - shared)]
+               for _ in range(sequences)]
+
+    def product():
+        storage = kvx.Storage(LAYERS, H, D, kvx.INT4, pages, extent_pages, accounting=True)
+        pool = kvx.Pool(storage, extent_pages)
+        prefix = kvx.Prefix(pool)
+        records = kvx.Sequences(pool, prefix)
+        tokens = [(C.c_uint32 * most)(*t) for t in streams]
+        blocks, matched = (C.c_uint64 * (prompt_tokens // 32))(), C.c_uint32()
+        view, released = kvx.SequencePages(), C.c_uint32()
+        S, P = records.h, prefix.h
+        calls = 0
+
+        def ok(rc):
+            if rc:
+                raise kvx.KvxError(rc, kvx.lib().kvx_last_error().decode())
+
+        now = time.perf_counter_ns
+        # the cost of a ctypes call that does nothing
+        t0 = now()
+        for _ in range(200000):
+            L.kvx_prefix_generation(P)
+        empty_ns = (now() - t0) / 200000
+        admit_ns, admit_calls, hit_blocks = [], [], []
+        for i in range(sequences):
+            t0, n = now(), 3
+            ok(L.kvx_sequence_begin(S, i + 1))
+            L.kvx_prefix_match(P, tokens[i], prompt_tokens, blocks, len(blocks), C.byref(matched))
+            if matched.value:
+                ok(L.kvx_sequence_restore(S, i + 1, blocks[matched.value - 1]))
+                n += 1
+            committed = 32 * matched.value
+            while committed < prompt_tokens:
+                committed = min(prompt_tokens, committed + chunk)
+                ok(L.kvx_sequence_ensure_tokens(S, i + 1, committed))
+                ok(L.kvx_sequence_publish(S, i + 1, tokens[i], prompt_tokens, committed))
+                ok(L.kvx_sequence_view(S, i + 1, C.byref(view)))
+                n += 3
+            admit_ns.append(now() - t0)
+            admit_calls.append(n)
+            hit_blocks.append(matched.value)
+        length = [prompt_tokens] * sequences
+        t0 = now()
+        for _ in range(steps):
+            for i in range(sequences):
+                length[i] += 1
+                ok(L.kvx_sequence_ensure_tokens(S, i + 1, length[i]))
+                ok(L.kvx_sequence_publish(S, i + 1, tokens[i], length[i], length[i]))
+                ok(L.kvx_sequence_view(S, i + 1, C.byref(view)))
+        decode_ns = (now() - t0) / steps
+        accepted = [[rng.randrange(1, 6) for _ in range(sequences)] for _ in range(steps)]
+        t0 = now()
+        for step in range(steps):
+            for i in range(sequences):
+                ok(L.kvx_sequence_ensure_tokens(S, i + 1, length[i] + 16))
+                length[i] += accepted[step][i]
+                ok(L.kvx_sequence_publish(S, i + 1, tokens[i], length[i], length[i]))
+                ok(L.kvx_sequence_truncate(S, i + 1, length[i], C.byref(released)))
+                ok(L.kvx_sequence_view(S, i + 1, C.byref(view)))
+        verify_ns = (now() - t0) / steps
+        resident = L.kvx_prefix_block_count(P)
+        t0 = now()
+        for i in range(sequences):
+            ok(L.kvx_sequence_end(S, i + 1))
+        block, evicted = C.c_uint64(), 0
+        while L.kvx_prefix_eviction_candidate(P, 0, C.byref(block)) == 1:
+            ok(L.kvx_prefix_erase(P, block.value))
+            evicted += 1
+        end_ns = now() - t0
+        snapshot = pool.snapshot()
+        assert evicted == resident and snapshot.pages_active == 0 and snapshot.pages_prefix == 0
+        records.close(); prefix.close(); pool.close(); storage.close()
+        return {"empty_ns": empty_ns, "admit_ns": admit_ns, "admit_calls": admit_calls,
+                "hit_blocks": hit_blocks, "decode_ns": decode_ns, "verify_ns": verify_ns,
+                "end_ns": end_ns, "evicted": evicted, "final_length": length}
+
+    def port(budget_s):
+        from oracle import kvoracle as ko
+        from oracle import prefix_oracle as po
+        import numpy as np
+        KL = ko.lib()
+
+        class Pages:   # the oracle's page pool behind the three calls the cache makes
+            def __init__(self):
+                self.h = KL.ko_pool_create(pages, 100, extent_pages, extent_pages, 0xFFFFFFFF)
+                self.pages, self.extent_pages = pages, extent_pages
+            def acquire(self, count):
+                out = np.zeros(max(count, 1), dtype=np.uint32)
+                if KL.ko_pool_acquire(self.h, count, ko.ptr(out)) != count:
+                    raise po.OracleError("nomem")
+                return [int(x) for x in out[:count]]
+            def retain(self, page, prefix_owner):
+                if KL.ko_pool_retain(self.h, page, int(prefix_owner)):
+                    raise po.OracleError("state")
+            def release(self, page, prefix_owner):
+                if KL.ko_pool_release(self.h, page, int(prefix_owner)):
+                    raise po.OracleError("state")
+
+        pool = Pages()
+        prefix = po.PrefixCache(pool, pages)
+        records = po.SequenceCache(pool, prefix, pool.acquire)
+        started = time.perf_counter()
+        admitted = 0
+        t0 = time.perf_counter_ns()
+        for i in range(sequences):
+            records.begin(i + 1)
+            found = []
+            prefix.extend_match(found, streams[i][:prompt_tokens])
+            if found:
+                records.restore(i + 1, found[-1])
+            committed = 32 * len(found)
+            while committed < prompt_tokens:
+                committed = min(prompt_tokens, committed + chunk)
+                records.ensure_tokens(i + 1, committed)
+                records.publish(i + 1, streams[i][:prompt_tokens], committed)
+            admitted += 1
+        admit_ns = (time.perf_counter_ns() - t0) / admitted
+        length = [prompt_tokens] * sequences
+        done = 0
+        t0 = time.perf_counter_ns()
+        while done < steps and time.perf_counter() - started < budget_s:
+            for i in range(sequences):
+                length[i] += 1
+                records.ensure_tokens(i + 1, length[i])
+                records.publish(i + 1, streams[i][:length[i]], length[i])
+            done += 1
+        decode_ns = (time.perf_counter_ns() - t0) / max(done, 1)
+        return {"admit_us": admit_ns / 1e3, "decode_step_us": decode_ns / 1e3, "steps": done}
+
+    for _ in range(max(args.warmup, 0) and 1):
+        product()
+    m = product()
+    per_step_calls = 3 * sequences
+    net_decode_us = (m["decode_ns"] - per_step_calls * m["empty_ns"]) / 1e3
+    warm = [i for i in range(sequences) if m["hit_blocks"][i]]
+    cold_us = m["admit_ns"][0] / 1e3
+    warm_us = sum(m["admit_ns"][i] for i in warm) / max(len(warm), 1) / 1e3
+    baseline = port(args.cpu_seconds) if args.cpu_seconds > 0 else None
+    result = {
+        "metric": "kv_control_plane_decode_step_us", "value": round(net_decode_us, 2), "unit": "us per step of 32 sequences",
+        "n_gpus": 1, "steps": steps, "warmup": 1 if args.warmup else 0,
+        "ms_per_step": round(m["decode_ns"] / 1e6, 5), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "host", "data": "synthetic",
+        "config": {"workload": "host control plane at batch 32: prefix page cache and sequence records over "
+                               "accounting-only storage, 32 x 16384-token prompts sharing 8192 tokens, then "
+                               "one-token decode steps and 16-row tree-verify steps",
+                   "layers": LAYERS, "kv_heads": H, "head_dim": D, "format": "int4", "pool_pages": pages},
+        "roofline": None,
+        "calls": {
+            "empty_ctypes_call_ns": round(m["empty_ns"], 1),
+            "decode_step_us_with_call_overhead": round(m["decode_ns"] / 1e3, 2),
+            "decode_step_calls": per_step_calls,
+            "tree_verify_step_us_with_call_overhead": round(m["verify_ns"] / 1e3, 2),
+            "tree_verify_step_calls": 4 * sequences,
+            "admission_cold_us": round(cold_us, 1), "admission_cold_calls": m["admit_calls"][0],
+            "admission_shared_prefix_us": round(warm_us, 1),
+            "admission_shared_prefix_calls": m["admit_calls"][-1],
+            "admission_matched_blocks": m["hit_blocks"][-1],
+            "end_and_evict_us": round(m["end_ns"] / 1e3, 1), "blocks_evicted": m["evicted"],
+        },
+        "cpu_baseline": None if baseline is None else {
+            "value": round(baseline["decode_step_us"], 1), "unit": "us per step of 32 sequences", "cores": 1,
+            "kind": "port",
+            "sample": f"oracle/prefix_oracle.py over the oracle's page pool: the same admissions "
+                      f"({baseline['admit_us']:.0f} us each on average) and {baseline['steps']} of the decode steps"},
+    }
+    print(json.dumps(result))
+
+
 def chunked_prefill(args):
     """Chunked prefill with prefix reuse: batch 4, a 2048-token chunk per sequence appended onto a
     shared 16384-token prefix (the prefix pages are the same physical pages in every
@@ -1142,6 +1337,8 @@ def main():
             return single_decode(args)
         if args.workload == "shared-prefix":
             return shared_prefix(args)
+        if args.workload == "control-plane":
+            return control_plane(args)
         return tree_verify(args) if args.workload == "tree-verify" else chunked_prefill(args)
     import numpy as np
     import torch
