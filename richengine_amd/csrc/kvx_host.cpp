@@ -349,9 +349,9 @@ int kvx_decode_plan_for(const kvx_layout *layout, const uint32_t *committed, uin
   // Head dimensions 64 and 128: a wave per (lane, KV head, split) over a staged copy of its
   // own, eight waves to a CU at head dimension 128 and sixteen at 64 (what the copies leave
   // room for); one round of them, splits of at least 4 pages (32 sequences of 8192 tokens,
-  // 2 x 8 x 128: 63 us at 32 splits, 84 at 16; 8 x 4 x 64: 90 us at 16, 93 at 32).  bf16 pages
-  // are read at close to the memory's rate with half as many waves, and the other half only
-  // adds partial rows (2 x 8 x 128: 59 us at 16 splits, 70 at 32; 8 x 4 x 64: 119 at 8, 131 at 16).
+  // 2 x 8 x 128: 51 us at 32 splits, 80 at 16, 65 at 64; 8 x 4 x 64: 87 us at 16, 86 at 32).
+  // bf16 pages are read at close to the memory's rate with half as many waves, and the other half
+  // only adds partial rows (2 x 8 x 128: 54 us at 16 splits, 60 at 32; 8 x 4 x 64: 113 at 8, 125 at 16).
   const uint64_t slots = (layout->head_dim == 128 ? 2048 : 4096) / (layout->format == KVX_FMT_BF16 ? 2 : 1);
   for (uint32_t first = 0; first < n_lanes; first += KVX_LANES_PER_LAUNCH) {
     const uint32_t count = std::min(KVX_LANES_PER_LAUNCH, n_lanes - first);

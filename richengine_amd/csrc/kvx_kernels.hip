@@ -990,8 +990,8 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
   constexpr uint32_t kPerThread = (kPieces + kThreads - 1) / kThreads;
   small_u32x4 raw_keys[kPerThread], raw_values[kPerThread];
   float raw_scale = 1.0f;
-  const auto fetch = [&](uint32_t page) {
-    const Slab s = slab_of(FMT, H, D, kv, head, table[page]);
+  const auto fetch = [&](uint64_t entry) {
+    const Slab s = slab_of(FMT, H, D, kv, head, entry);
 #pragma unroll
     for (uint32_t i = 0; i < kPerThread; ++i) {
       const uint32_t piece = tid + i * kThreads;
@@ -1036,12 +1036,19 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
     else if (tid < 2 * kPage) value_scale_lds[tid - kPage] = raw_scale;
   };
 
-  fetch(begin);
+  // A page's table entry is read one page before its bytes are asked for, so that a fetch
+  // is one trip to memory and not two in a row.
+  uint64_t entry_ahead = table[min(begin + 1, end - 1)];
+  fetch(table[begin]);
   for (uint32_t page = begin; page < end; ++page) {
     const uint32_t token_start = page * kPage;
     tile_barrier();  // the previous page's products are done with the staged copy
     stage();
-    if (page + 1 < end) fetch(page + 1);
+    if (page + 1 < end) {
+      const uint64_t entry = entry_ahead;
+      entry_ahead = table[min(page + 2, end - 1)];
+      fetch(entry);
+    }
     tile_barrier();
 
 #pragma unroll
@@ -1182,26 +1189,51 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(BL
 }
 
 // Fixed-order merge of one fused row's splits (reference:
-// common/paged_attention_tile.h:362-417).  head_dim threads, one per dimension;
+// common/paged_attention_tile.h:362-417).  One thread per dimension, in whole waves;
 // returns the thread's bf16 element, zero for rows past the live ones.
 __device__ __forceinline__ uint16_t reduce_row(const float *__restrict__ partials,
                                const float *__restrict__ statistics, uint32_t G, uint32_t D,
                                uint32_t M, uint32_t committed, uint32_t active_rows,
                                uint32_t splits, uint64_t head_row, uint32_t fused_row) {
-  const uint32_t d = threadIdx.x;
+  // Workgroups of whole waves: thread d sums dimension d (threads past D only lend their
+  // lanes).  Lane i of every wave holds the statistics of split base + i, 64 splits at a
+  // time, and hands weight and term round with shuffles; the partial values of eight splits
+  // are asked for together and then added in split order.
+  const uint32_t d = threadIdx.x, lane = threadIdx.x & 63u;
   if (fused_row / G >= active_rows) return 0;
   const uint32_t pages = (committed + active_rows + kPage - 1) / kPage;
   const uint32_t per = (pages + splits - 1) / splits;
   const uint32_t written = (pages + per - 1) / per;
+  const auto statistic = [&](uint32_t s) { return statistics + (head_row + uint64_t(s) * M + fused_row) * 2; };
   float maximum = -INFINITY;
-  for (uint32_t s = 0; s < written; ++s)
-    maximum = fmaxf(maximum, statistics[(head_row + uint64_t(s) * M + fused_row) * 2]);
+  for (uint32_t base = 0; base < written; base += 64)
+    if (base + lane < written) maximum = fmaxf(maximum, statistic(base + lane)[0]);
+  for (int offset = 32; offset; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset));
+  constexpr uint32_t kAhead = 8;
   float numerator = 0.0f, denominator = 0.0f;
-  for (uint32_t s = 0; s < written; ++s) {  // split order is part of the contract
-    const uint64_t row = head_row + uint64_t(s) * M + fused_row;
-    const float weight = expf(__fsub_rn(statistics[row * 2], maximum));
-    numerator = __fadd_rn(numerator, __fmul_rn(weight, partials[row * D + d]));
-    denominator = __fadd_rn(denominator, __fmul_rn(weight, statistics[row * 2 + 1]));
+  for (uint32_t base = 0; base < written; base += 64) {
+    const uint32_t count = min(64u, written - base);
+    float my_weight = 0.0f, my_term = 0.0f;
+    if (lane < count) {
+      const float *stat = statistic(base + lane);
+      my_weight = expf(__fsub_rn(stat[0], maximum));
+      my_term = __fmul_rn(my_weight, stat[1]);
+    }
+    for (uint32_t i = 0; i < count; i += kAhead) {
+      float part[kAhead];
+#pragma unroll
+      for (uint32_t u = 0; u < kAhead; ++u) {
+        const uint64_t row = head_row + uint64_t(base + min(i + u, count - 1)) * M + fused_row;
+        part[u] = d < D ? partials[row * D + d] : 0.0f;
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < kAhead; ++u) {
+        if (i + u < count) {  // split order is part of the contract
+          numerator = __fadd_rn(numerator, __fmul_rn(__shfl(my_weight, i + u), part[u]));
+          denominator = __fadd_rn(denominator, __shfl(my_term, i + u));
+        }
+      }
+    }
   }
   return f32_to_bf16(denominator > 0.0f ? __fdiv_rn(numerator, denominator) : 0.0f);
 }
@@ -1217,6 +1249,7 @@ __global__ __launch_bounds__(256) void attend_reduce_kernel(const float *__restr
   const uint16_t value =
       reduce_row(partials, statistics, a.group, D, M, l.committed, l.active_rows, l.split_count,
                  l.row_base + uint64_t(head) * l.split_count * M, fused_row);
+  if (d >= D) return;
   if (output)
     output[l.q_offset + uint64_t(head) * a.row_stride * a.group * D + uint64_t(fused_row) * D + d] =
         value;
@@ -1246,9 +1279,10 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float *__rest
   const uint32_t active = min(KVX_PREFILL_TILE_ROWS, p.rows - tile_start);
   const uint32_t M = KVX_PREFILL_TILE_ROWS * p.group, D = p.head_dim;
   const uint64_t tile_offset = (uint64_t(head) * p.stride + tile_start) * p.group * D;
-  output[tile_offset + uint64_t(fused_row) * D + threadIdx.x] =
+  const uint16_t value =
       reduce_row(partials, statistics, p.group, D, M, p.committed + tile_start, active, p.splits,
                  (uint64_t(tile) * p.kv_heads + head) * p.splits * M, fused_row);
+  if (threadIdx.x < D) output[tile_offset + uint64_t(fused_row) * D + threadIdx.x] = value;
 }
 
 // =========================================================== compaction ====
@@ -1948,7 +1982,7 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
       });
     if (rc) return rc;
     if (phases & 2u) {
-      hipLaunchKernelGGL(attend_reduce_kernel, dim3(M, H, a.n_lanes), dim3(D), 0, stream, partials,
+      hipLaunchKernelGGL(attend_reduce_kernel, dim3(M, H, a.n_lanes), dim3((D + 63) / 64 * 64), 0, stream, partials,
                          statistics, static_cast<uint16_t *>(output), a);
       if ((rc = check_launch("attend_reduce_kernel"))) return rc;
     }
@@ -2528,7 +2562,7 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
     });
   });
   if (rc) return rc;
-  hipLaunchKernelGGL(prefill_reduce_kernel, dim3(M, H, tiles), dim3(D), 0, st, partials, statistics,
+  hipLaunchKernelGGL(prefill_reduce_kernel, dim3(M, H, tiles), dim3((D + 63) / 64 * 64), 0, st, partials, statistics,
                      static_cast<uint16_t *>(output), p);
   return check_launch("prefill_reduce_kernel");
 }
