@@ -179,8 +179,8 @@ int kvx_decode_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t
 /* The same by layout: head dimension 256 is kvx_decode_plan; head dimensions 64 and 128 (the
    reference's other layouts, runtime/ops/PagedAttention.cpp:66-115), whose one-row tiles run a
    wave each over a staged copy of their own, get the split length (at least 4 pages) that makes
-   one round of those waves, 2048 at head dimension 128 and 4096 at 64 (half as many over bf16
-   pages), launch by launch, at most KVX_VERIFY_MAX_SPLITS per lane.  Same errors, and KVX_EINVAL
+   one round of those waves, 4096 (2048 at head dimension 128 over pages other than int4; half as
+   many over bf16 pages), launch by launch, at most KVX_VERIFY_MAX_SPLITS per lane.  Same errors, and KVX_EINVAL
    for an invalid layout. */
 int kvx_decode_plan_for(const kvx_layout *layout, const uint32_t *committed_tokens, uint32_t n_lanes,
                         uint32_t *split_counts);

@@ -346,13 +346,16 @@ int kvx_decode_plan_for(const kvx_layout *layout, const uint32_t *committed, uin
   for (uint32_t i = 0; i < n_lanes; ++i)
     if (uint64_t(committed[i]) + 1 > KVX_MAX_PHYSICAL_TOKENS)
       return fail(KVX_EINVAL, "kvx_decode_plan_for: context_out_of_range");
-  // Head dimensions 64 and 128: a wave per (lane, KV head, split) over a staged copy of its
-  // own, eight waves to a CU at head dimension 128 and sixteen at 64 (what the copies leave
-  // room for); one round of them, splits of at least 4 pages (32 sequences of 8192 tokens,
-  // 2 x 8 x 128: 51 us at 32 splits, 80 at 16, 65 at 64; 8 x 4 x 64: 87 us at 16, 86 at 32).
-  // bf16 pages are read at close to the memory's rate with half as many waves, and the other half
-  // only adds partial rows (2 x 8 x 128: 54 us at 16 splits, 60 at 32; 8 x 4 x 64: 113 at 8, 125 at 16).
-  const uint64_t slots = (layout->head_dim == 128 ? 2048 : 4096) / (layout->format == KVX_FMT_BF16 ? 2 : 1);
+  // Head dimensions 64 and 128: a wave per (lane, KV head, split) over a staged copy of the
+  // page's values of its own, sixteen waves to a CU (eight at head dimension 128 over pages
+  // other than int4, whose raw bytes take more registers); one round of them, splits of at
+  // least 4 pages (32 sequences of 8192 tokens, int4, 2 x 8 x 128: 48 us at 64 splits, 51 at
+  // 32, 60 at 128; 8 x 4 x 64: 83 us at 16, 82 at 32, 85 at 64; int8 2 x 8 x 128: 44 us at 32,
+  // 49 at 64).  bf16 pages are read at close to the memory's rate with half as many waves, and
+  // the other half only adds partial rows (2 x 8 x 128: 54 us at 16 splits, 55 at 32; 8 x 4 x 64:
+  // 106 at 8, 110 at 16).
+  const bool sixteen = layout->head_dim == 64 || layout->format == KVX_FMT_INT4;
+  const uint64_t slots = (sixteen ? 4096 : 2048) / (layout->format == KVX_FMT_BF16 ? 2 : 1);
   for (uint32_t first = 0; first < n_lanes; first += KVX_LANES_PER_LAUNCH) {
     const uint32_t count = std::min(KVX_LANES_PER_LAUNCH, n_lanes - first);
     uint64_t page_heads = 0;

@@ -900,12 +900,57 @@ struct SmallChunk {
   }
 };
 
+// Eight key elements of one token as they lie in the page (16 bytes of bf16, 8 of int8 or
+// e4m3, 4 of int4), which is a lane's share of q.k's key operand: a wave whose tile is its
+// own reads its keys straight from the page and keeps no staged copy of them.
+template <uint32_t FMT>
+struct SmallKeyPiece {
+  static constexpr uint32_t kWords = FMT == KVX_FMT_BF16 ? 4 : FMT == KVX_FMT_INT4 ? 1 : 2;
+  uint32_t raw[kWords];
+  __device__ __forceinline__ void load(const uint8_t *from) {
+    if constexpr (kWords == 4) {
+      const small_u32x4 v = *reinterpret_cast<const small_u32x4 *>(from);
+      raw[0] = v[0]; raw[1] = v[1]; raw[2] = v[2]; raw[3] = v[3];
+    } else if constexpr (kWords == 2) {
+      const small_u32x2 v = *reinterpret_cast<const small_u32x2 *>(from);
+      raw[0] = v[0]; raw[1] = v[1];
+    } else {
+      raw[0] = *reinterpret_cast<const uint32_t *>(from);
+    }
+  }
+  // The eight elements as 16-bit operand elements, as SmallChunk makes them.
+  __device__ __forceinline__ small_u32x4 operand() const {
+    small_u32x4 out;
+    if constexpr (FMT == KVX_FMT_BF16) {
+      out = small_u32x4{raw[0], raw[1], raw[2], raw[3]};
+    } else if constexpr (FMT == KVX_FMT_FP8E4M3) {
+#pragma unroll
+      for (uint32_t i = 0; i < 2; ++i) {
+        out[2 * i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[i], 1.0f, false));
+        out[2 * i + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[i], 1.0f, true));
+      }
+    } else {
+      constexpr uint32_t kBits = FMT == KVX_FMT_INT8 ? 8 : 4;
+#pragma unroll
+      for (uint32_t i = 0; i < 4; ++i) {
+        const uint32_t word = raw[(2 * i * kBits) / 32];
+        const int lo = __builtin_amdgcn_sbfe(int(word), (2 * i * kBits) % 32, kBits);
+        const int hi = __builtin_amdgcn_sbfe(int(word), (2 * i * kBits) % 32 + kBits, kBits);
+        out[i] = (__float_as_uint(float(lo)) >> 16) | (__float_as_uint(float(hi)) & 0xffff0000u);
+      }
+    }
+    return out;
+  }
+};
+
 // PRIVATE = 0: the four waves of the workgroup share the tile (row blocks by wave, the page
 // staged by all 256 threads, a barrier on either side of the staging).  PRIVATE = n: the
 // workgroup is n independent waves, each with a tile of at most 16 fused rows (one-row decode,
 // short chains of small groups) and a staged copy of its own: a wave's LDS operations complete
 // in the order it issues them, so it needs no barrier, and every wave of a CU multiplies
-// instead of one in four.
+// instead of one in four.  Such a wave stages the values only: a lane's share of the key
+// operand is eight consecutive elements of one token, which it reads from the page itself,
+// and half the staged bytes leave room for twice the waves.
 template <uint32_t FMT, uint32_t D, uint32_t BLOCKS, uint32_t PRIVATE = 0>
 __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
                                      const uint64_t *__restrict__ table, kvx_kv_layer kv,
@@ -927,7 +972,8 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
   constexpr uint32_t kSteps = D / 32, kTiles = D / 16;
   static_assert(!PRIVATE || BLOCKS == 1, "a private tile is one block of 16 fused rows");
   constexpr uint32_t kCopies = PRIVATE ? PRIVATE : 1, kThreads = PRIVATE ? 64u : kTileThreads;
-  __shared__ __align__(16) uint16_t k_lds_all[kCopies][kPage * kKeyRow];
+  constexpr bool kDirectKeys = PRIVATE != 0;
+  __shared__ __align__(16) uint16_t k_lds_all[kCopies][kDirectKeys ? 8 : kPage * kKeyRow];
   __shared__ __align__(16) uint16_t v_lds_all[kCopies][D * kValueRow + (D / 32) * 16];
   __shared__ float key_scale_all[kCopies][kPage], value_scale_all[kCopies][kPage];
   const uint32_t copy = PRIVATE ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0u;
@@ -988,15 +1034,25 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
   using Chunk = SmallChunk<FMT>;
   constexpr uint32_t kPieces = kPage * D / Chunk::kElements;         // per tensor
   constexpr uint32_t kPerThread = (kPieces + kThreads - 1) / kThreads;
-  small_u32x4 raw_keys[kPerThread], raw_values[kPerThread];
+  small_u32x4 raw_keys[kDirectKeys ? 1 : kPerThread], raw_values[kPerThread];
+  SmallKeyPiece<FMT> key_piece[2][kDirectKeys ? kSteps : 1];  // tokens 16 tb + t, dims 32 kb + 8 g ..
+  constexpr uint32_t kKeyRowBytes = D * 16 / Chunk::kElements;
   float raw_scale = 1.0f;
+  const auto fetch_keys = [&](uint64_t entry) {
+    const Slab s = slab_of(FMT, H, D, kv, head, entry);
+#pragma unroll
+    for (uint32_t tb = 0; tb < 2; ++tb)
+#pragma unroll
+      for (uint32_t kb = 0; kb < kSteps; ++kb)
+        key_piece[tb][kb].load(s.keys + (16 * tb + t) * kKeyRowBytes + (32 * kb + 8 * g) * 16 / Chunk::kElements);
+  };
   const auto fetch = [&](uint64_t entry) {
     const Slab s = slab_of(FMT, H, D, kv, head, entry);
 #pragma unroll
     for (uint32_t i = 0; i < kPerThread; ++i) {
       const uint32_t piece = tid + i * kThreads;
       if (kPieces % kThreads == 0 || piece < kPieces) {
-        raw_keys[i] = *reinterpret_cast<const small_u32x4 *>(s.keys + 16 * piece);
+        if constexpr (!kDirectKeys) raw_keys[i] = *reinterpret_cast<const small_u32x4 *>(s.keys + 16 * piece);
         raw_values[i] = *reinterpret_cast<const small_u32x4 *>(s.values + 16 * piece);
       }
     }
@@ -1009,7 +1065,7 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
       const uint32_t piece = tid + i * kThreads;
       if (kPieces % kThreads != 0 && piece >= kPieces) continue;
       const uint32_t first = piece * Chunk::kElements;
-      {  // keys are token-major in every format
+      if constexpr (!kDirectKeys) {  // keys are token-major in every format
         const Chunk c(raw_keys[i]);
         uint32_t *to = reinterpret_cast<uint32_t *>(&k_lds[(first / D) * kKeyRow + first % D]);
 #pragma unroll
@@ -1040,12 +1096,13 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
   // is one trip to memory and not two in a row.
   uint64_t entry_ahead = table[min(begin + 1, end - 1)];
   fetch(table[begin]);
+  if constexpr (kDirectKeys) fetch_keys(table[begin]);
   for (uint32_t page = begin; page < end; ++page) {
     const uint32_t token_start = page * kPage;
     tile_barrier();  // the previous page's products are done with the staged copy
     stage();
+    const uint64_t entry = entry_ahead;
     if (page + 1 < end) {
-      const uint64_t entry = entry_ahead;
       entry_ahead = table[min(page + 2, end - 1)];
       fetch(entry);
     }
@@ -1059,10 +1116,14 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
       for (uint32_t tb = 0; tb < 2; ++tb)
 #pragma unroll
         for (uint32_t kb = 0; kb < kSteps; ++kb) {
-          const small_u32x4 keys =
-              *reinterpret_cast<const small_u32x4 *>(&k_lds[(16 * tb + t) * kKeyRow + 32 * kb + 8 * g]);
+          small_u32x4 keys;
+          if constexpr (kDirectKeys) keys = key_piece[tb][kb].operand();
+          else keys = *reinterpret_cast<const small_u32x4 *>(&k_lds[(16 * tb + t) * kKeyRow + 32 * kb + 8 * g]);
           scores[tb] = small_mfma<kFp8>(keys, q[b][kb], scores[tb]);
         }
+      // the next page's keys, now that this page's are multiplied (a private tile is one block)
+      if constexpr (kDirectKeys)
+        if (page + 1 < end) fetch_keys(entry);
       // page softmax of the lane's eight tokens of its row (reference:
       // common/paged_attention_tile.h:129-188)
       float score[8], local_max = -INFINITY;
@@ -1150,11 +1211,16 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(BL
 }
 
 // Tiles of at most 16 fused rows: a wave per (split, KV head, lane), PRIVATE of them to a
-// workgroup (what the staged copies leave room for: 18 KiB a wave at head dimension 128).
+// workgroup (the staged values take 9.3 KiB a wave at head dimension 128).
 template <uint32_t D>
 constexpr uint32_t kSmallPrivateWaves = D == 128 ? 2 : 4;
+// Four waves to a SIMD where the page's raw bytes leave the registers for it: at head dimension
+// 128, bf16 pages keep 64 registers of them in flight, and int8 and e4m3 pages would spill a few.
 template <uint32_t FMT, uint32_t D>
-__global__ __launch_bounds__(64 * kSmallPrivateWaves<D>) void attend_split_small_wave_kernel(
+constexpr uint32_t kSmallPrivatePerSimd = D != 128 || FMT == KVX_FMT_INT4 ? 4 : FMT == KVX_FMT_BF16 ? 2 : 3;
+template <uint32_t FMT, uint32_t D>
+__global__ __launch_bounds__(64 * kSmallPrivateWaves<D>)
+__attribute__((amdgpu_waves_per_eu(kSmallPrivatePerSimd<FMT, D>, kSmallPrivatePerSimd<FMT, D>))) void attend_split_small_wave_kernel(
     const uint16_t *__restrict__ queries, float *__restrict__ partials,
     float *__restrict__ statistics, const uint32_t *__restrict__ row_masks, AttendArgs a) {
   constexpr uint32_t kWaves = kSmallPrivateWaves<D>;

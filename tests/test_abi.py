@@ -195,7 +195,8 @@ def test_decode_and_verify_plans_size_the_launch_for_the_gpu():
     # by layout: head dimension 256 is the plan above; 128 and 64 plan one round of single waves
     import ctypes as C
     for heads, dim, fmt, want in ((4, 256, kvx.INT4, kvx.decode_plan([8191] * 32, 4, kvx.INT4)),
-                                  (2, 128, kvx.INT4, [32] * 32),    # 256 pages x 2 heads x 32 lanes on 2048 waves: 8 pages a split
+                                  (2, 128, kvx.INT4, [64] * 32),    # 256 pages x 2 heads x 32 lanes on 4096 waves: 4 pages a split
+                                  (2, 128, kvx.FP8, [32] * 32),     # other than int4 at 128: 2048 waves, 8 pages a split
                                   (8, 64, kvx.INT8, [16] * 32),     # 256 x 8 x 32 on 4096: 16 pages a split
                                   (2, 128, kvx.BF16, [16] * 32)):    # bf16 pages: half the waves
         layout = kvx.Layout(1, heads, dim, fmt, 0.0)
