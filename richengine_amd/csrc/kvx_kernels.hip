@@ -1738,10 +1738,10 @@ static int attend_matrix(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_h
 }
 
 namespace {
-uint64_t g_generic_attends = 0, g_matrix_attends = 0;
+std::atomic<uint64_t> g_generic_attends{0}, g_matrix_attends{0};  // callers may be on several threads
 int took(int fast) {  // counts which kernels an attend call went to
-  if (fast == 0) ++g_matrix_attends;
-  if (fast > 0) ++g_generic_attends;
+  if (fast == 0) g_matrix_attends.fetch_add(1, std::memory_order_relaxed);
+  if (fast > 0) g_generic_attends.fetch_add(1, std::memory_order_relaxed);
   return fast;
 }
 }  // namespace
@@ -1749,8 +1749,8 @@ int took(int fast) {  // counts which kernels an attend call went to
 extern "C" {
 
 void kvx_debug_attend_paths(uint64_t *generic_calls, uint64_t *matrix_core_calls) {
-  if (generic_calls) *generic_calls = g_generic_attends;
-  if (matrix_core_calls) *matrix_core_calls = g_matrix_attends;
+  if (generic_calls) *generic_calls = g_generic_attends.load(std::memory_order_relaxed);
+  if (matrix_core_calls) *matrix_core_calls = g_matrix_attends.load(std::memory_order_relaxed);
 }
 
 int kv_append(const kvx_storage *s, uint32_t layer, const void *chunk_keys,
