@@ -19,7 +19,11 @@
  *    last failure.
  *  - Lanes whose parameters fail the kernel contract write nothing (as the
  *    reference kernels do); host-side validation reports them first.
- *  - One caller thread per storage/pool (as the reference's engine thread).
+ *  - One caller thread per storage/pool (as the reference's engine thread) for
+ *    what changes them: extents, pool, prefix cache, sequence records.  The kv_*
+ *    entries only read the storage's description and keep nothing between
+ *    calls, so several threads may call them at once over one storage, each on
+ *    a stream and a workspace of its own.
  */
 #ifndef KVX_H
 #define KVX_H
