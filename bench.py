@@ -82,20 +82,23 @@ def parse():
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
     ap.add_argument("--workload", choices=["decode", "decode-single", "tree-verify", "prefill", "qkv-prepare", "shared-prefix",
-                                           "stream-ceiling", "control-plane"], default="decode",
+                                           "stream-ceiling", "control-plane", "decode-layout"], default="decode",
                     help="decode = batch-32 mixed-length int4 decode, the headline metric (default); "
                          "decode-single = one sequence of 32768 tokens, the 16 per-layer calls replayed "
                          "as one HIP graph; tree-verify = 16-node tree verify and prefill = chunked prefill with a shared "
                          "prefix, the matrix-core paths (profiling); stream-ceiling = what the memory system "
                          "delivers for the headline batch's bytes under request shapes other than the "
                          "decode kernel's (linear, 16-byte coalesced, page order, pool size); control-plane = "
-                         "the host calls of a batch-32 step (prefix page cache, sequence records), no GPU work")
+                         "the host calls of a batch-32 step (prefix page cache, sequence records), no GPU work; "
+                         "decode-layout = one-row decode over the reference's other layouts (--layout)")
+    ap.add_argument("--layout", choices=["hd128", "hd64"], default="hd128",
+                    help="decode-layout: 2 KV heads x 8 x 128 or 8 x 4 x 64")
     ap.add_argument("--format", choices=["bf16", "fp8", "int8", "int4"], default=None,
                     help="page format of the prefill workload (default bf16) and of the shared-prefix "
                          "and tree-verify workloads (default int4; no fp8)")
     args = ap.parse_args()
     if args.format is None:
-        args.format = "int4" if args.workload in ("shared-prefix", "tree-verify") else "bf16"
+        args.format = "int4" if args.workload in ("shared-prefix", "tree-verify", "decode-layout") else "bf16"
     return args
 
 
@@ -106,15 +109,16 @@ def host_cpus():
             "threads_cap": 16}
 
 
-def cpu_lane_prepare(ctx, seed):
+def cpu_lane_prepare(ctx, seed, H=H, G=G, D=D, fmt=None):
     """One sequence on the oracle: fills the history (untimed) and returns run(), the decode
     step of one layer (append one token, attend), which returns its seconds."""
     import numpy as np
     from oracle import kvoracle as ko
 
+    page_format = ko.INT4 if fmt is None else fmt
     rng = np.random.default_rng(seed)
     n_pages = (ctx + 1 + 31) // 32
-    store = ko.Store(1, H, D, ko.INT4, n_pages, n_pages)
+    store = ko.Store(1, H, D, page_format, n_pages, n_pages)
     store.allocate(0)
     table = store.entries(np.arange(n_pages, dtype=np.uint32))
     done = 0
@@ -123,7 +127,7 @@ def cpu_lane_prepare(ctx, seed):
         stride = (n + 31) // 32 * 32
         k = ko.f32_to_bf16(rng.standard_normal((H, stride, D)).astype(np.float32)).reshape(H, stride, D)
         v = ko.f32_to_bf16(rng.standard_normal((H, D, stride)).astype(np.float32)).reshape(H, D, stride)
-        ko.store_chunk(ko.INT4, H, D, k, v, table, ko.ChunkParams(done, n, stride, n_pages, store.layer(0)))
+        ko.store_chunk(page_format, H, D, k, v, table, ko.ChunkParams(done, n, stride, n_pages, store.layer(0)))
         done += n
     k = ko.f32_to_bf16(rng.standard_normal((H, 32, D)).astype(np.float32)).reshape(H, 32, D)
     v = ko.f32_to_bf16(rng.standard_normal((H, D, 32)).astype(np.float32)).reshape(H, D, 32)
@@ -133,8 +137,8 @@ def cpu_lane_prepare(ctx, seed):
 
     def run():
         t0 = time.perf_counter()
-        ko.store_chunk(ko.INT4, H, D, k, v, table, ko.ChunkParams(ctx, 1, 32, n_pages, store.layer(0)))
-        ko.attend_verify(ko.INT4, H, G, D, q, [table],
+        ko.store_chunk(page_format, H, D, k, v, table, ko.ChunkParams(ctx, 1, 32, n_pages, store.layer(0)))
+        ko.attend_verify(page_format, H, G, D, q, [table],
                          [ko.VerifyParams(ctx, n_pages, store.layer(0), splits, 128, 1, 1, 0.0)],
                          want_f32=False)
         return time.perf_counter() - t0
@@ -143,9 +147,9 @@ def cpu_lane_prepare(ctx, seed):
     return run
 
 
-def cpu_lane(ctx, seed):
+def cpu_lane(ctx, seed, **layout):
     """History filled untimed, then the timed decode step of one layer.  Returns seconds."""
-    run = cpu_lane_prepare(ctx, seed)
+    run = cpu_lane_prepare(ctx, seed, **layout)
     spent = run()
     run.close()
     return spent
@@ -1318,6 +1322,91 @@ def single_decode(args):
     print(json.dumps(result))
 
 
+def decode_layout(args):
+    """One-row decode attention over the reference's other shipped layouts (2 KV heads x 8 x 128
+    and 8 x 4 x 64, runtime/ops/PagedAttention.cpp:66-115): 32 sequences of 8192 tokens, one
+    layer per call, split counts from kvx_decode_plan_for.  `value` is KV bytes per second of
+    kv_attend_decode (split + reduce); the roofline leg times the split kernel alone."""
+    import numpy as np
+    import torch
+    from richengine_amd import kvx
+
+    torch.cuda.set_device(0)
+    heads, group, dim = {"hd128": (2, 8, 128), "hd64": (8, 4, 64)}[args.layout]
+    fmt = {"bf16": kvx.BF16, "fp8": kvx.FP8, "int8": kvx.INT8, "int4": kvx.INT4}[args.format]
+    per_token = heads * {"bf16": 4 * dim, "fp8": 2 * dim + 8, "int8": 2 * dim + 8, "int4": dim + 8}[args.format]
+    lanes, context = 32, 8192
+    n_pages = (context + 31) // 32
+    query_heads = heads * group
+    pool_pages = 8192 * (-(-lanes * n_pages // 8192))
+    storage = kvx.Storage(1, heads, dim, fmt, pool_pages, 8192, aligned=True)
+    storage.allocate_all()
+    rng = np.random.default_rng(args.seed)
+    ids = rng.permutation(lanes * n_pages).astype(np.uint32)
+    tables = [storage.table(ids[i * n_pages:(i + 1) * n_pages]) for i in range(lanes)]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(args.seed)
+    for i in range(lanes):
+        for done in range(0, context, 2048):
+            k = torch.randn((heads, 2048, dim), generator=gen, device="cuda").bfloat16()
+            v = torch.randn((heads, dim, 2048), generator=gen, device="cuda").bfloat16()
+            kvx.append(storage, 0, k, v, [tables[i]], [kvx.ChunkParams(done, 2048, 2048, n_pages)],
+                       heads * 2048 * dim)
+    q = torch.randn((lanes, heads, 1, group, dim), generator=gen, device="cuda").bfloat16()
+    out = torch.zeros_like(q)
+    splits = kvx.decode_plan_for(storage, [context - 1] * lanes)
+    dp = [kvx.VerifyParams(context - 1, n_pages, kvx.KvLayer(), splits[i], splits[i], 1, 1, 0.0)
+          for i in range(lanes)]
+    ws = torch.empty(kvx.attend_workspace_bytes(storage, dp, query_heads), dtype=torch.uint8, device="cuda")
+
+    def timed(fn, n):
+        for _ in range(max(args.warmup, 1)):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n * 1e-3
+
+    call_s = timed(lambda: kvx.attend_decode(storage, 0, query_heads, q, out, tables, dp, 1, ws), args.steps)
+    split_s = timed(lambda: kvx.attend_split(storage, 0, query_heads, q, tables, dp, None, 1, ws), args.kernel_iters)
+    merge_s = timed(lambda: kvx.attend_merge(storage, query_heads, out, dp, 1, ws), args.kernel_iters)
+    kv_bytes = lanes * context * per_token
+    value = kv_bytes / call_s / 1e9
+    achieved = kv_bytes / split_s / 1e9
+    result = {
+        "metric": "decode_kv_read_GBps", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": max(args.warmup, 1), "ms_per_step": round(call_s * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {"int4": "int4 codes -> bf16 MFMA", "int8": "int8 codes -> bf16 MFMA",
+                  "fp8": "e4m3 -> fp16 MFMA", "bf16": "bf16 MFMA"}[args.format],
+        "data": "synthetic",
+        "config": {"workload": f"one-row decode attention, {heads} KV heads x {group} x {dim} ({args.layout}), "
+                               f"{args.format} pages, batch {lanes} x {context} tokens, one layer per call",
+                   "splits_per_sequence": int(splits[0]), "seed": args.seed},
+        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "attend_split_small_wave_kernel (a wave per sequence, KV head and split)",
+                     "bytes_per_launch": kv_bytes, "ms_per_launch": round(split_s * 1e3, 4),
+                     "reduce_ms_per_launch": round(merge_s * 1e3, 4)},
+        "cpu_baseline": None,
+    }
+    storage.close()
+    if args.cpu_seconds > 0:
+        from oracle import kvoracle as ko
+        oracle_fmt = {"bf16": ko.BF16, "fp8": ko.FP8, "int8": ko.INT8, "int4": ko.INT4}[args.format]
+        spent = cpu_lane(context - 1, args.seed, H=heads, G=group, D=dim, fmt=oracle_fmt)
+        result["cpu_baseline"] = {
+            "value": context * per_token / spent / 1e9, "unit": "GB/s", "cores": 1, "kind": "port", **host_cpus(),
+            "sample": f"one of the 32 sequences: append 1 token + decode attention over {context} tokens, "
+                      f"{spent:.2f} s of scalar C++ oracle"}
+    print(json.dumps(result))
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -1339,6 +1428,8 @@ def main():
             return shared_prefix(args)
         if args.workload == "control-plane":
             return control_plane(args)
+        if args.workload == "decode-layout":
+            return decode_layout(args)
         return tree_verify(args) if args.workload == "tree-verify" else chunked_prefill(args)
     import numpy as np
     import torch

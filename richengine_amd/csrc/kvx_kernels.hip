@@ -1263,7 +1263,7 @@ __device__ __forceinline__ uint16_t reduce_row(const float *__restrict__ partial
                                uint32_t splits, uint64_t head_row, uint32_t fused_row) {
   // Workgroups of whole waves: thread d sums dimension d (threads past D only lend their
   // lanes).  Lane i of every wave holds the statistics of split base + i, 64 splits at a
-  // time, and hands weight and term round with shuffles; the partial values of eight splits
+  // time, and hands weight and term round with shuffles; the partial values of 32 splits
   // are asked for together and then added in split order.
   const uint32_t d = threadIdx.x, lane = threadIdx.x & 63u;
   if (fused_row / G >= active_rows) return 0;
@@ -1271,27 +1271,42 @@ __device__ __forceinline__ uint16_t reduce_row(const float *__restrict__ partial
   const uint32_t per = (pages + splits - 1) / splits;
   const uint32_t written = (pages + per - 1) / per;
   const auto statistic = [&](uint32_t s) { return statistics + (head_row + uint64_t(s) * M + fused_row) * 2; };
-  float maximum = -INFINITY;
-  for (uint32_t base = 0; base < written; base += 64)
+  const auto partial = [&](uint32_t s) {
+    return d < D ? partials[(head_row + uint64_t(s) * M + fused_row) * D + d] : 0.0f;
+  };
+  // The statistics of the first 64 splits and the partial values of the first kAhead are asked
+  // for together, before anything waits.
+  constexpr uint32_t kAhead = 32;
+  float first_max = -INFINITY, first_sum = 0.0f;
+  if (lane < written) {
+    first_max = statistic(lane)[0];
+    first_sum = statistic(lane)[1];
+  }
+  float early[kAhead];
+#pragma unroll
+  for (uint32_t u = 0; u < kAhead; ++u) early[u] = partial(min(u, written - 1));
+  float maximum = first_max;
+  for (uint32_t base = 64; base < written; base += 64)
     if (base + lane < written) maximum = fmaxf(maximum, statistic(base + lane)[0]);
   for (int offset = 32; offset; offset >>= 1) maximum = fmaxf(maximum, __shfl_xor(maximum, offset));
-  constexpr uint32_t kAhead = 8;
   float numerator = 0.0f, denominator = 0.0f;
   for (uint32_t base = 0; base < written; base += 64) {
     const uint32_t count = min(64u, written - base);
+    float my_max = first_max, my_sum = first_sum;
+    if (base && lane < count) {
+      my_max = statistic(base + lane)[0];
+      my_sum = statistic(base + lane)[1];
+    }
     float my_weight = 0.0f, my_term = 0.0f;
     if (lane < count) {
-      const float *stat = statistic(base + lane);
-      my_weight = expf(__fsub_rn(stat[0], maximum));
-      my_term = __fmul_rn(my_weight, stat[1]);
+      my_weight = expf(__fsub_rn(my_max, maximum));
+      my_term = __fmul_rn(my_weight, my_sum);
     }
     for (uint32_t i = 0; i < count; i += kAhead) {
       float part[kAhead];
 #pragma unroll
-      for (uint32_t u = 0; u < kAhead; ++u) {
-        const uint64_t row = head_row + uint64_t(base + min(i + u, count - 1)) * M + fused_row;
-        part[u] = d < D ? partials[row * D + d] : 0.0f;
-      }
+      for (uint32_t u = 0; u < kAhead; ++u)
+        part[u] = (base == 0 && i == 0) ? early[u] : partial(base + min(i + u, count - 1));
 #pragma unroll
       for (uint32_t u = 0; u < kAhead; ++u) {
         if (i + u < count) {  // split order is part of the contract
