@@ -862,6 +862,13 @@ __device__ __forceinline__ uint16_t operand_bits(float x) {
   else return f32_to_bf16(x);
 }
 
+// exp of a difference of scores as the head-dimension-256 kernels take it: one v_exp_f32 of the
+// difference in units of log 2 (exactly 1 at a difference of 0; within an ulp or two of expf
+// elsewhere, far inside the scores' own deviation from the oracle's).
+__device__ __forceinline__ float small_exp(float difference) {
+  return __builtin_amdgcn_exp2f(__fmul_rn(difference, 1.4426950408889634f));
+}
+
 constexpr uint32_t kSmallBlocks = 2;  // at most: blocks of 16 fused rows per wave, 128 rows per tile
 
 // Sixteen bytes of a page as they lie (32 int4 codes, 16 int8 or e4m3 codes, 8 bf16 values)
@@ -1145,13 +1152,13 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
       const float next_max = fmaxf(row_max[b], local_max);
       const float rescale = (next_max == -INFINITY || next_max == row_max[b])
                                 ? 1.0f
-                                : expf(__fsub_rn(row_max[b], next_max));
+                                : small_exp(__fsub_rn(row_max[b], next_max));
       float page_sum = 0.0f;
       uint32_t bits[8];
 #pragma unroll
       for (uint32_t i = 0; i < 8; ++i) {
         const uint32_t token = 16 * (i >> 2) + 4 * g + (i & 3);
-        const float p = in[i] ? expf(__fsub_rn(score[i], next_max)) : 0.0f;
+        const float p = in[i] ? small_exp(__fsub_rn(score[i], next_max)) : 0.0f;
         page_sum = __fadd_rn(page_sum, p);
         float weight = 0.0f;
         if (in[i] && score[i] > -INFINITY) weight = kQuant ? __fmul_rn(p, value_scale_lds[token]) : p;
