@@ -844,6 +844,8 @@ typedef float small_f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t small_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t small_u32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 small_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 small_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float small_f32x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 small_f16x8 __attribute__((ext_vector_type(8)));
 
 template <bool F16>
@@ -1132,42 +1134,56 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
       if constexpr (kDirectKeys)
         if (page + 1 < end) fetch_keys(entry);
       // page softmax of the lane's eight tokens of its row (reference:
-      // common/paged_attention_tile.h:129-188)
-      float score[8], local_max = -INFINITY;
-      bool in[8];
+      // common/paged_attention_tile.h:129-188).  A page that lies wholly in the committed
+      // history is seen by every row, so its tokens skip the tests (rows past the live ones
+      // then hold numbers instead of nothing, and are not written either way).
+      float rescale;
+      small_u32x4 weights;
+      const auto page_softmax = [&](auto whole_page) {
+        constexpr bool kWhole = decltype(whole_page)::value;
+        float score[8], local_max = -INFINITY;
+        bool in[8];
 #pragma unroll
-      for (uint32_t i = 0; i < 8; ++i) {
-        const uint32_t token = 16 * (i >> 2) + 4 * g + (i & 3), at = token_start + token;
-        in[i] = live[b] && (tree ? (at < committed ||
-                                    (at < visible && ((mask[b] >> ((at - committed) & 31u)) & 1u)))
-                                 : at < limit[b]);
-        float v = scores[i >> 2][i & 3];
-        if constexpr (kQuant) v = __fmul_rn(v, key_scale_lds[token]);
-        v = __fmul_rn(v, score_scale);
-        score[i] = in[i] ? v : -INFINITY;
-        local_max = fmaxf(local_max, score[i]);
-      }
-      local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
-      local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
-      const float next_max = fmaxf(row_max[b], local_max);
-      const float rescale = (next_max == -INFINITY || next_max == row_max[b])
-                                ? 1.0f
-                                : small_exp(__fsub_rn(row_max[b], next_max));
-      float page_sum = 0.0f;
-      uint32_t bits[8];
+        for (uint32_t i = 0; i < 8; ++i) {
+          const uint32_t token = 16 * (i >> 2) + 4 * g + (i & 3), at = token_start + token;
+          in[i] = kWhole || (live[b] && (tree ? (at < committed || (at < visible && ((mask[b] >> ((at - committed) & 31u)) & 1u)))
+                                              : at < limit[b]));
+          float v = scores[i >> 2][i & 3];
+          if constexpr (kQuant) v = __fmul_rn(v, key_scale_lds[token]);
+          v = __fmul_rn(v, score_scale);
+          score[i] = in[i] ? v : -INFINITY;
+          local_max = fmaxf(local_max, score[i]);
+        }
+        local_max = fmaxf(local_max, __shfl_xor(local_max, 16));
+        local_max = fmaxf(local_max, __shfl_xor(local_max, 32));
+        const float next_max = fmaxf(row_max[b], local_max);
+        rescale = (next_max == -INFINITY || next_max == row_max[b])
+                      ? 1.0f
+                      : small_exp(__fsub_rn(row_max[b], next_max));
+        float page_sum = 0.0f, weight[8];
 #pragma unroll
-      for (uint32_t i = 0; i < 8; ++i) {
-        const uint32_t token = 16 * (i >> 2) + 4 * g + (i & 3);
-        const float p = in[i] ? small_exp(__fsub_rn(score[i], next_max)) : 0.0f;
-        page_sum = __fadd_rn(page_sum, p);
-        float weight = 0.0f;
-        if (in[i] && score[i] > -INFINITY) weight = kQuant ? __fmul_rn(p, value_scale_lds[token]) : p;
-        bits[i] = operand_bits<kFp8>(weight);
-      }
-      row_sum[b] = __fadd_rn(__fmul_rn(row_sum[b], rescale), page_sum);
-      row_max[b] = next_max;
-      const small_u32x4 weights = {bits[0] | bits[1] << 16, bits[2] | bits[3] << 16,
-                                   bits[4] | bits[5] << 16, bits[6] | bits[7] << 16};
+        for (uint32_t i = 0; i < 8; ++i) {
+          const uint32_t token = 16 * (i >> 2) + 4 * g + (i & 3);
+          const float p = in[i] ? small_exp(__fsub_rn(score[i], next_max)) : 0.0f;
+          page_sum = __fadd_rn(page_sum, p);
+          weight[i] = 0.0f;
+          if (kWhole || (in[i] && score[i] > -INFINITY))
+            weight[i] = kQuant ? __fmul_rn(p, value_scale_lds[token]) : p;
+        }
+        row_sum[b] = __fadd_rn(__fmul_rn(row_sum[b], rescale), page_sum);
+        row_max[b] = next_max;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+          // two weights to their 16-bit operand elements, round to nearest even, in one
+          // instruction where the operand is bf16
+          if constexpr (kFp8)
+            weights[i] = uint32_t(operand_bits<true>(weight[2 * i])) | uint32_t(operand_bits<true>(weight[2 * i + 1])) << 16;
+          else
+            weights[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(small_f32x2{weight[2 * i], weight[2 * i + 1]}, small_bf16x2));
+        }
+      };
+      if (token_start + kPage <= committed) page_softmax(std::true_type{});
+      else page_softmax(std::false_type{});
       if (__builtin_amdgcn_ballot_w64(rescale != 1.0f)) {
 #pragma unroll
         for (uint32_t i = 0; i < kTiles; ++i) acc[b][i] *= rescale;
