@@ -16,6 +16,12 @@ extern "C" {
    matrix-core (MFMA) kernels, so tests can tell which path they measured. */
 void kvx_debug_attend_paths(uint64_t *generic_calls, uint64_t *matrix_core_calls);
 
+/* How many consecutive 8-row tiles of a kv_attend_prefill call at head dimension 64 or 128 share
+   a workgroup and a staged page (1 = every tile on its own; 0 = invalid arguments), so tests can
+   tell which kernel a chunk ran on. */
+uint32_t kvx_debug_prefill_tiles_together(const kvx_layout *layout, uint32_t query_heads,
+                                          uint32_t committed_tokens, uint32_t rows, uint32_t splits);
+
 /* Streams the pages of `page_table` (n_pages device entries of an int4, head dimension 256
    storage) with exactly the loads of the int4 decode kernel, two waves per SIMD, and nothing
    behind them; workgroup x reads entries x * pages_per_wave onward, one wave per KV head,

@@ -960,6 +960,19 @@ struct SmallKeyPiece {
 // instead of one in four.  Such a wave stages the values only: a lane's share of the key
 // operand is eight consecutive elements of one token, which it reads from the page itself,
 // and half the staged bytes leave room for twice the waves.
+// Several consecutive prefill tiles of one (KV head, split) on one staged page: tile k of the
+// group lies `row_capacity` rows further on in the chunk (its history, its queries) and
+// `slot_stride` rows further on in the workspace.  The caller sees to it that every tile of a
+// group has the same pages under the same split (a history that ends on a page boundary and
+// groups that do not straddle one).  The blocks of 16 fused rows of all tiles are dealt to the
+// four waves in turn.  {1, 4 * BLOCKS, .., 0} is a single tile.
+struct SmallGroup {
+  uint32_t tiles;        // tiles of the group that have rows
+  uint32_t blocks;       // blocks of 16 fused rows to a tile
+  uint32_t rows_left;    // chunk rows from the group's first tile on
+  uint64_t slot_stride;  // workspace rows from a tile's slot to the next tile's
+};
+
 template <uint32_t FMT, uint32_t D, uint32_t BLOCKS, uint32_t PRIVATE = 0>
 __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict__ tile_queries,
                                      const uint64_t *__restrict__ table, kvx_kv_layer kv,
@@ -967,7 +980,8 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
                                      uint32_t committed, uint32_t active_rows, uint32_t splits,
                                      uint32_t split, float *__restrict__ partials,
                                      float *__restrict__ statistics, uint64_t slot_row,
-                                     const uint32_t *__restrict__ row_masks, float score_scale_in) {
+                                     const uint32_t *__restrict__ row_masks, float score_scale_in,
+                                     SmallGroup group = SmallGroup{1u, 4u * BLOCKS, 0u, 0u}) {
   constexpr bool kFp8 = FMT == KVX_FMT_FP8E4M3;
   constexpr bool kQuant = FMT != KVX_FMT_BF16;
   constexpr uint32_t kKeyRow = D + 8;        // staged halves per token: 16 bytes past a power of two
@@ -1009,15 +1023,24 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
   small_f32x4 acc[BLOCKS][kTiles];
   float row_max[BLOCKS], row_sum[BLOCKS];
   uint32_t limit[BLOCKS], mask[BLOCKS], fused[BLOCKS];
+  uint64_t out_row[BLOCKS];
   bool live[BLOCKS], used[BLOCKS];
 #pragma unroll
   for (uint32_t b = 0; b < BLOCKS; ++b) {
-    fused[b] = 16 * (wave + 4 * b) + t;
-    used[b] = 16 * (wave + 4 * b) < M;  // the same in every lane of the wave
+    // the wave's b-th block: block `block` of tile `k` of the group
+    const uint32_t dealt = wave + 4 * b, k = dealt / group.blocks, block = dealt % group.blocks;
+    const uint32_t tile_committed = committed + k * row_capacity;
+    const uint32_t tile_rows =
+        group.tiles == 1 ? active_rows
+                         : min(row_capacity, group.rows_left - min(group.rows_left, k * row_capacity));
+    fused[b] = 16 * block + t;
+    used[b] = k < group.tiles && 16 * block < M && tile_rows > 0;  // the same in every lane of the wave
     const uint32_t query_row = fused[b] / G;
-    live[b] = fused[b] < M && query_row < active_rows;
-    limit[b] = live[b] ? min(visible, committed + min(query_row, active_rows - 1) + 1) : 0u;
+    live[b] = used[b] && fused[b] < M && query_row < tile_rows;
+    limit[b] = live[b] ? min(tile_committed + tile_rows, tile_committed + min(query_row, tile_rows - 1) + 1) : 0u;
     mask[b] = (live[b] && tree) ? row_masks[query_row] : 0u;
+    out_row[b] = slot_row + k * group.slot_stride + fused[b];
+    const uint16_t *block_queries = tile_queries + uint64_t(k) * row_capacity * G * D;
     row_max[b] = -INFINITY;
     row_sum[b] = 0.0f;
 #pragma unroll
@@ -1026,7 +1049,7 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
     for (uint32_t kb = 0; kb < kSteps; ++kb) {
       small_u32x4 raw = {0u, 0u, 0u, 0u};
       if (live[b])
-        raw = *reinterpret_cast<const small_u32x4 *>(tile_queries + uint64_t(fused[b]) * D + 32 * kb + 8 * g);
+        raw = *reinterpret_cast<const small_u32x4 *>(block_queries + uint64_t(fused[b]) * D + 32 * kb + 8 * g);
       if constexpr (kFp8) {  // the fp8 tile stages its queries as fp16
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i)
@@ -1206,12 +1229,12 @@ __device__ __forceinline__ void attention_tile_small(const uint16_t *__restrict_
     sum = __fadd_rn(sum, __shfl_xor(sum, 16));
     sum = __fadd_rn(sum, __shfl_xor(sum, 32));
     if (!live[b]) continue;
-    float *out = partials + (slot_row + fused[b]) * D + 4 * g;
+    float *out = partials + out_row[b] * D + 4 * g;
 #pragma unroll
     for (uint32_t i = 0; i < kTiles; ++i) *reinterpret_cast<small_f32x4 *>(out + 16 * i) = acc[b][i];
     if (g == 0) {
-      statistics[(slot_row + fused[b]) * 2] = row_max[b];
-      statistics[(slot_row + fused[b]) * 2 + 1] = sum;
+      statistics[out_row[b] * 2] = row_max[b];
+      statistics[out_row[b] * 2 + 1] = sum;
     }
   }
 }
@@ -1275,6 +1298,29 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(BL
                                KVX_PREFILL_TILE_ROWS, head, p.committed + tile_start, active,
                                p.splits, split, partials, statistics, slot_row, nullptr,
                                p.score_scale);
+}
+
+// The same for `tiles_per_group` consecutive tiles of a chunk at once, on a history that ends
+// on a page boundary: the page is staged once for all of them, and every wave multiplies one
+// or two blocks of 16 fused rows a page where a single tile of a small group of query heads
+// leaves it one, or none.  Slots and results are those of the tile-by-tile launch.
+template <uint32_t FMT, uint32_t D, uint32_t BLOCKS>
+__global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void prefill_group_small_kernel(
+    const uint16_t *__restrict__ queries, float *__restrict__ partials,
+    float *__restrict__ statistics, PrefillArgs p, uint32_t tiles_per_group) {
+  const uint32_t split = blockIdx.x, head = blockIdx.y, tile = blockIdx.z * tiles_per_group;
+  const uint32_t tile_start = tile * KVX_PREFILL_TILE_ROWS;
+  if (!prefill_contract(p) || tile_start >= p.rows) return;
+  const uint32_t rows_left = p.rows - tile_start;
+  const uint32_t M = KVX_PREFILL_TILE_ROWS * p.group;
+  const uint64_t tile_offset = (uint64_t(head) * p.stride + tile_start) * p.group * D;
+  const uint64_t slot_row = ((uint64_t(tile) * p.kv_heads + head) * p.splits + split) * M;
+  const SmallGroup group = {min(tiles_per_group, (rows_left + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS),
+                            (M + 15) / 16, rows_left, uint64_t(p.kv_heads) * p.splits * M};
+  attention_tile_small<FMT, D, BLOCKS>(queries + tile_offset, p.table, p.kv, p.kv_heads, p.group,
+                               KVX_PREFILL_TILE_ROWS, head, p.committed + tile_start,
+                               min(KVX_PREFILL_TILE_ROWS, rows_left), p.splits, split, partials,
+                               statistics, slot_row, nullptr, p.score_scale, group);
 }
 
 // Fixed-order merge of one fused row's splits (reference:
@@ -1775,6 +1821,28 @@ static int attend_matrix(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_h
                                 many_tiles, stream, tile_rows, epilogue);
 }
 
+// How many consecutive tiles of a chunked prefill at head dimension 64 or 128 share a workgroup
+// and a staged page (prefill_group_small_kernel): 1 = tile by tile.  A history that ends on a
+// page boundary is what gives the tiles that begin in the same 32 (or 16) rows of the chunk the
+// same pages under the same splits.  As many tiles as keep four waves to a SIMD: a wave then
+// holds the accumulators of two blocks of 16 fused rows at head dimension 64 and of one at 128
+// (two at 128, on two waves a SIMD: 2048 rows over 16 384 tokens at 2 x 8 x 128 took 789 us
+// against 742 tile by tile on int4 pages, 596 against 550 on bf16).  Groups make a launch
+// of fewer workgroups, so a small launch stays tile by tile: where a tile alone leaves waves
+// without a block the groups win from 256 workgroups on (8 x 4 x 64, 512 rows over 16 384 tokens,
+// int4: 504 us against 484 at 256, 311 against 467 at 512), where it does not, from 1024
+// (2 x 8 x 64, 2048 rows: 647 against 593 at 512, 454 against 562 at 1024).
+static uint32_t small_prefill_tiles_together(uint32_t D, uint32_t H, uint32_t G, uint32_t committed,
+                                             uint32_t rows, uint32_t splits) {
+  if ((D != 64 && D != 128) || committed % kPage) return 1;
+  const uint32_t blocks = (KVX_PREFILL_TILE_ROWS * G + 15) / 16, most = D == 64 ? 8u : 4u;
+  const uint32_t together = 4 * blocks <= most ? 4u : 2 * blocks <= most ? 2u : 1u;
+  const uint64_t tiles = (rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+  if (together == 1 || tiles < 2) return 1;
+  const uint64_t workgroups = (tiles + together - 1) / together * H * splits;
+  return workgroups >= (blocks < 4 ? 256u : 1024u) ? together : 1u;
+}
+
 namespace {
 std::atomic<uint64_t> g_generic_attends{0}, g_matrix_attends{0};  // callers may be on several threads
 int took(int fast) {  // counts which kernels an attend call went to
@@ -1785,6 +1853,13 @@ int took(int fast) {  // counts which kernels an attend call went to
 }  // namespace
 
 extern "C" {
+
+uint32_t kvx_debug_prefill_tiles_together(const kvx_layout *layout, uint32_t query_heads,
+                                          uint32_t committed_tokens, uint32_t rows, uint32_t splits) {
+  if (!kvx_layout_valid(layout) || !query_heads || query_heads % layout->kv_heads) return 0;
+  return small_prefill_tiles_together(layout->head_dim, layout->kv_heads, query_heads / layout->kv_heads,
+                                      committed_tokens, rows, splits);
+}
 
 void kvx_debug_attend_paths(uint64_t *generic_calls, uint64_t *matrix_core_calls) {
   if (generic_calls) *generic_calls = g_generic_attends.load(std::memory_order_relaxed);
@@ -2651,6 +2726,21 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
                            static_cast<const uint16_t *>(queries), partials, statistics, p);
       };
       constexpr uint32_t F = decltype(fmt)::value;
+      const uint32_t blocks = (M + 15) / 16;
+      const uint32_t together = small_prefill_tiles_together(D, H, G, params->committed_tokens,
+                                                             params->rows, params->split_count);
+      if (together > 1) {
+        const uint32_t per_wave = (blocks * together + 3) / 4;  // 1 or 2
+        const auto group_launch = [&](auto kernel) {
+          hipLaunchKernelGGL(kernel, dim3(params->split_count, H, (tiles + together - 1) / together),
+                             dim3(kTileThreads), 0, st, static_cast<const uint16_t *>(queries), partials,
+                             statistics, p, together);
+        };
+        if (D == 128) group_launch(prefill_group_small_kernel<F, 128, 1>);
+        else if (per_wave <= 1) group_launch(prefill_group_small_kernel<F, 64, 1>);
+        else group_launch(prefill_group_small_kernel<F, 64, 2>);
+        return check_launch("prefill_group_small_kernel");
+      }
       if (D == 64 && M <= 64) launch(prefill_split_small_kernel<F, 64, 1>);
       else if (D == 64) launch(prefill_split_small_kernel<F, 64, 2>);
       else if (M <= 64) launch(prefill_split_small_kernel<F, 128, 1>);

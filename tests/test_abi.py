@@ -394,3 +394,26 @@ def test_storage_refuses_geometry_the_kernels_cannot_index():
         with pytest.raises(kvx.KvxError):
             kvx.Storage(layers, heads, 64, kvx.INT8, pages, extent_pages, accounting=True)
     kvx.Storage(1, 1, 64, kvx.INT8, 1 << 20, 1, accounting=True).close()
+
+
+def test_prefill_groups_of_tiles_rule():
+    """kvx_debug_prefill_tiles_together: groups only on a history that ends on a page boundary, only
+    at head dimensions 64 and 128, as many tiles as keep four waves to a SIMD, and only in launches
+    of enough workgroups (256 where a tile alone leaves waves idle, 1024 otherwise)."""
+    import ctypes as C
+
+    def together(heads, group, dim, committed, rows, splits, fmt=kvx.INT4):
+        layout = kvx.Layout(1, heads, dim, fmt, 0.0)
+        return kvx.lib().kvx_debug_prefill_tiles_together(C.byref(layout), heads * group, committed, rows, splits)
+
+    assert together(8, 4, 64, 16384, 2048, 1) == 4          # 64 groups x 8 heads = 512 workgroups
+    assert together(8, 4, 64, 16385, 2048, 1) == 1          # not on a page boundary
+    assert together(8, 4, 64, 16384, 512, 1) == 1           # 128 workgroups
+    assert together(8, 4, 64, 16384, 512, 2) == 4           # 256
+    assert together(2, 8, 64, 16384, 2048, 2) == 1          # every wave has a block: 512 < 1024
+    assert together(2, 8, 64, 16384, 2048, 4) == 2
+    assert together(2, 8, 128, 16384, 2048, 8) == 1         # two blocks a wave at 128: never
+    assert together(2, 4, 128, 16384, 2048, 1) == 2 and together(4, 2, 128, 16384, 2048, 1) == 4
+    assert together(4, 6, 256, 16384, 2048, 4) == 1         # head dimension 256 has kernels of its own
+    assert together(8, 4, 64, 0, 8, 32) == 1                # one tile
+    assert together(8, 3, 64, 0, 8, 32) == 1 and together(8, 0, 64, 0, 8, 32) == 0
