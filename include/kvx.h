@@ -180,6 +180,13 @@ uint32_t kvx_decode_splits(uint32_t committed_tokens, uint32_t rows);
 #define KVX_DECODE_MAX_SPLITS 512u
 int kvx_decode_plan(const uint32_t *committed_tokens, uint32_t n_lanes, uint32_t kv_heads,
                     uint32_t format, uint32_t *split_counts);
+/* kvx_prefill_plan_batch by layout: head dimension 256 is that plan; at head dimensions 64 and
+   128 (runtime/ops/PagedAttention.cpp:66-115), whose tiles run a workgroup each, or one for the
+   four or two tiles that begin in the same page of a chunk on a page-aligned history, the fewest
+   splits that make 4096 workgroups, none shorter than 4 pages, at most KVX_PREFILL_MAX_SPLITS.
+   0 for an invalid layout, bad head counts or no sequences. */
+uint32_t kvx_prefill_plan_for(const kvx_layout *layout, uint32_t committed_tokens, uint32_t rows,
+                              uint32_t query_heads, uint32_t n_sequences);
 /* The same by layout: head dimension 256 is kvx_decode_plan; head dimensions 64 and 128 (the
    reference's other layouts, runtime/ops/PagedAttention.cpp:66-115), whose one-row tiles run a
    wave each over a staged copy of their own, get the split length (at least 4 pages) that makes

@@ -362,7 +362,7 @@ public:
                                 &plan.workspace.statisticsBytes));
     return plan;
   }
-  // The same with the split count sized for the GPU (kvx_prefill_plan): the
+  // The same with the split count sized for the GPU (kvx_prefill_plan_for): the
   // reference rule gives chunks of 256 rows and more one split, which leaves
   // most of 1024 SIMDs idle until the chunk has about 2048 rows.
   // sequences: how many chunks of this shape one addPrefillBatch call holds (its launches
@@ -370,10 +370,9 @@ public:
   static PrefillAttentionPlan prefillPlan(uint32_t historyTokens, uint32_t rows, uint32_t queryHeads,
                                           kv::Layout layout, uint32_t sequences = 1) {
     PrefillAttentionPlan plan = prefillPlan(rows, queryHeads, layout);
-    plan.splits = kvx_prefill_plan_batch(historyTokens, rows, layout.kvHeads, queryHeads,
-                                         static_cast<uint32_t>(layout.format), sequences);
-    if (!plan.splits) throw std::invalid_argument("paged prefill plan: no sequences");
     const kvx_layout l = layout.c();
+    plan.splits = kvx_prefill_plan_for(&l, historyTokens, rows, queryHeads, sequences);
+    if (!plan.splits) throw std::invalid_argument("paged prefill plan: no sequences");
     check(kvx_prefill_workspace_for(rows, plan.splits, queryHeads, &l, &plan.workspace.partialsBytes,
                                     &plan.workspace.statisticsBytes));
     return plan;

@@ -336,6 +336,29 @@ int kvx_decode_plan(const uint32_t *committed, uint32_t n_lanes, uint32_t kv_hea
                           format, split_counts + first);
   return KVX_OK;
 }
+uint32_t kvx_prefill_plan_for(const kvx_layout *layout, uint32_t committed, uint32_t rows,
+                              uint32_t query_heads, uint32_t sequences) {
+  if (!kvx_layout_valid(layout) || !query_heads || query_heads % layout->kv_heads || !sequences) return 0;
+  if (layout->head_dim != 64 && layout->head_dim != 128)
+    return kvx_prefill_plan_batch(committed, rows, layout->kv_heads, query_heads, layout->format, sequences);
+  // Head dimensions 64 and 128: a workgroup of four waves per (tile or group of tiles, KV head,
+  // split), four of them to a CU at a time.  The fewest splits that make four rounds of them
+  // (4096 workgroups), none shorter than 4 pages (2048 rows over 16 384 tokens, int4, in 1 / 2 /
+  // 4 / 8 splits: 8 x 4 x 64 1562 / 1173 / 1092 / 1051 us, 2 x 8 x 128 1311 / 963 / 887 / 833;
+  // 256 rows over 8192 tokens in 4 / 8 / 16 / 32: 173 / 116 / 96 / 102 and 132 / 97 / 82 / 88).
+  // The sequences of a batch run one after the other at these head dimensions.
+  const uint64_t tiles = (uint64_t(rows) + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+  if (!tiles) return 1;
+  const uint64_t seen = pages_of(uint64_t(committed) + rows / 2);
+  const uint32_t most = uint32_t(std::max<uint64_t>(1, std::min<uint64_t>(seen / 4, KVX_PREFILL_MAX_SPLITS)));
+  const uint32_t group = query_heads / layout->kv_heads;
+  for (uint32_t s = 1; s < most; ++s) {
+    const uint32_t together =
+        kvx::small_prefill_tiles_together(layout->head_dim, layout->kv_heads, group, committed, rows, s);
+    if ((tiles + together - 1) / together * layout->kv_heads * s >= 4096) return s;
+  }
+  return most;
+}
 int kvx_decode_plan_for(const kvx_layout *layout, const uint32_t *committed, uint32_t n_lanes,
                         uint32_t *split_counts) {
   if (!kvx_layout_valid(layout)) return fail(KVX_EINVAL, "kvx_decode_plan_for: invalid layout");

@@ -197,6 +197,28 @@ inline uint32_t verify_row_blocks(uint32_t format, uint32_t fused_rows) {
   return (fused_rows + rows - 1) / rows;
 }
 
+// How many consecutive tiles of a chunked prefill at head dimension 64 or 128 share a workgroup
+// and a staged page (prefill_group_small_kernel): 1 = tile by tile.  A history that ends on a
+// page boundary is what gives the tiles that begin in the same 32 (or 16) rows of the chunk the
+// same pages under the same splits.  As many tiles as keep four waves to a SIMD: a wave then
+// holds the accumulators of two blocks of 16 fused rows at head dimension 64 and of one at 128
+// (two at 128, on two waves a SIMD: 2048 rows over 16 384 tokens at 2 x 8 x 128 took 789 us
+// against 742 tile by tile on int4 pages, 596 against 550 on bf16).  Groups make a launch
+// of fewer workgroups, so a small launch stays tile by tile: where a tile alone leaves waves
+// without a block the groups win from 256 workgroups on (8 x 4 x 64, 512 rows over 16 384 tokens,
+// int4: 504 us against 484 at 256, 311 against 467 at 512), where it does not, from 1024
+// (2 x 8 x 64, 2048 rows: 647 against 593 at 512, 454 against 562 at 1024).
+inline uint32_t small_prefill_tiles_together(uint32_t D, uint32_t H, uint32_t G, uint32_t committed,
+                                             uint32_t rows, uint32_t splits) {
+  if ((D != 64 && D != 128) || committed % KVX_PAGE_TOKENS) return 1;
+  const uint32_t blocks = (KVX_PREFILL_TILE_ROWS * G + 15) / 16, most = D == 64 ? 8u : 4u;
+  const uint32_t together = 4 * blocks <= most ? 4u : 2 * blocks <= most ? 2u : 1u;
+  const uint64_t tiles = (rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
+  if (together == 1 || tiles < 2) return 1;
+  const uint64_t workgroups = (tiles + together - 1) / together * H * splits;
+  return workgroups >= (blocks < 4 ? 256u : 1024u) ? together : 1u;
+}
+
 }  // namespace kvx
 
 struct kvx_storage : kvx::Storage {};

@@ -864,12 +864,12 @@ __device__ __forceinline__ uint16_t operand_bits(float x) {
   else return f32_to_bf16(x);
 }
 
-// exp of a difference of scores as the head-dimension-256 kernels take it: one v_exp_f32 of the
-// difference in units of log 2 (exactly 1 at a difference of 0; within an ulp or two of expf
-// elsewhere, far inside the scores' own deviation from the oracle's).
-__device__ __forceinline__ float small_exp(float difference) {
-  return __builtin_amdgcn_exp2f(__fmul_rn(difference, 1.4426950408889634f));
-}
+// exp of a difference of scores: expf, as the oracle takes it.  With the same exponentials the
+// rounded weights are the oracle's, and most rows of these tiles come out as its bits; one
+// v_exp_f32 of the difference in units of log 2 (the head-dimension-256 kernels' form, up to
+// 3.5e-6 from expf) was 6 to 16 per cent faster, but turned enough roundings that a row of 64
+// elements could land 2.2e-3 from the oracle with seven of them rounded the other way.
+__device__ __forceinline__ float small_exp(float difference) { return expf(difference); }
 
 constexpr uint32_t kSmallBlocks = 2;  // at most: blocks of 16 fused rows per wave, 128 rows per tile
 
@@ -1821,28 +1821,6 @@ static int attend_matrix(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_h
                                 many_tiles, stream, tile_rows, epilogue);
 }
 
-// How many consecutive tiles of a chunked prefill at head dimension 64 or 128 share a workgroup
-// and a staged page (prefill_group_small_kernel): 1 = tile by tile.  A history that ends on a
-// page boundary is what gives the tiles that begin in the same 32 (or 16) rows of the chunk the
-// same pages under the same splits.  As many tiles as keep four waves to a SIMD: a wave then
-// holds the accumulators of two blocks of 16 fused rows at head dimension 64 and of one at 128
-// (two at 128, on two waves a SIMD: 2048 rows over 16 384 tokens at 2 x 8 x 128 took 789 us
-// against 742 tile by tile on int4 pages, 596 against 550 on bf16).  Groups make a launch
-// of fewer workgroups, so a small launch stays tile by tile: where a tile alone leaves waves
-// without a block the groups win from 256 workgroups on (8 x 4 x 64, 512 rows over 16 384 tokens,
-// int4: 504 us against 484 at 256, 311 against 467 at 512), where it does not, from 1024
-// (2 x 8 x 64, 2048 rows: 647 against 593 at 512, 454 against 562 at 1024).
-static uint32_t small_prefill_tiles_together(uint32_t D, uint32_t H, uint32_t G, uint32_t committed,
-                                             uint32_t rows, uint32_t splits) {
-  if ((D != 64 && D != 128) || committed % kPage) return 1;
-  const uint32_t blocks = (KVX_PREFILL_TILE_ROWS * G + 15) / 16, most = D == 64 ? 8u : 4u;
-  const uint32_t together = 4 * blocks <= most ? 4u : 2 * blocks <= most ? 2u : 1u;
-  const uint64_t tiles = (rows + KVX_PREFILL_TILE_ROWS - 1) / KVX_PREFILL_TILE_ROWS;
-  if (together == 1 || tiles < 2) return 1;
-  const uint64_t workgroups = (tiles + together - 1) / together * H * splits;
-  return workgroups >= (blocks < 4 ? 256u : 1024u) ? together : 1u;
-}
-
 namespace {
 std::atomic<uint64_t> g_generic_attends{0}, g_matrix_attends{0};  // callers may be on several threads
 int took(int fast) {  // counts which kernels an attend call went to
@@ -1857,7 +1835,7 @@ extern "C" {
 uint32_t kvx_debug_prefill_tiles_together(const kvx_layout *layout, uint32_t query_heads,
                                           uint32_t committed_tokens, uint32_t rows, uint32_t splits) {
   if (!kvx_layout_valid(layout) || !query_heads || query_heads % layout->kv_heads) return 0;
-  return small_prefill_tiles_together(layout->head_dim, layout->kv_heads, query_heads / layout->kv_heads,
+  return kvx::small_prefill_tiles_together(layout->head_dim, layout->kv_heads, query_heads / layout->kv_heads,
                                       committed_tokens, rows, splits);
 }
 
@@ -2727,7 +2705,7 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
       };
       constexpr uint32_t F = decltype(fmt)::value;
       const uint32_t blocks = (M + 15) / 16;
-      const uint32_t together = small_prefill_tiles_together(D, H, G, params->committed_tokens,
+      const uint32_t together = kvx::small_prefill_tiles_together(D, H, G, params->committed_tokens,
                                                              params->rows, params->split_count);
       if (together > 1) {
         const uint32_t per_wave = (blocks * together + 3) / 4;  // 1 or 2

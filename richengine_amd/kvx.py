@@ -36,7 +36,7 @@ SYMBOLS = [
     "kvx_pool_free_pages", "kvx_pool_reclaim_empty", "kvx_pool_compact_extent",
     "kvx_pool_snapshot_get", "kv_append", "kv_prepare_append", "kv_attend_decode_shared", "kvx_attend_shared_workspace_bytes", "kv_attend_verify", "kv_attend_verify_hidden", "kv_attend_decode",
     "kv_attend_prefill", "kv_attend_prefill_batch", "kv_compact_path", "kv_append_attend_decode", "kv_append_attend_decode_hidden", "kv_page_export", "kv_page_import", "kv_attend_split", "kv_attend_merge", "kv_attend_decode_static",
-    "kvx_debug_attend_paths", "kvx_debug_prefill_tiles_together", "kvx_calibrate_stream", "kvx_decode_plan", "kvx_decode_plan_for", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
+    "kvx_debug_attend_paths", "kvx_debug_prefill_tiles_together", "kvx_calibrate_stream", "kvx_decode_plan", "kvx_decode_plan_for", "kvx_prefill_plan_for", "kvx_verify_plan", "kvx_storage_create_accounting", "kvx_prefix_create", "kvx_prefix_destroy", "kvx_prefix_find",
     "kvx_prefix_insert", "kvx_prefix_contains", "kvx_prefix_generation", "kvx_prefix_block_count",
     "kvx_prefix_chain", "kvx_prefix_retain_active", "kvx_prefix_release_active",
     "kvx_prefix_touch", "kvx_prefix_eviction_candidate", "kvx_prefix_erase",
@@ -204,6 +204,7 @@ def _declare(L):
     L.kvx_calibrate_stream_form.argtypes = [vp, u32, vp, u32, u32, u32, u32, u32, vp, vp]
     L.kvx_decode_plan.argtypes = [vp, u32, u32, u32, vp]
     L.kvx_decode_plan_for.argtypes = [LP, vp, u32, vp]
+    L.kvx_prefill_plan_for.argtypes, L.kvx_prefill_plan_for.restype = [LP, u32, u32, u32, u32], u32
     L.kvx_verify_plan.argtypes = [vp, u32, u32, u32, u32, u32, vp]
     L.kvx_tree_masks.argtypes = [vp, u32, vp]
     L.kvx_tree_path_valid.argtypes = [vp, u32, vp, u32]
@@ -796,6 +797,14 @@ def decode_plan_for(storage, committed):
     out = (C.c_uint32 * len(committed))()
     check(lib().kvx_decode_plan_for(C.byref(storage.layout), _u32(committed), len(committed), out))
     return list(out)
+
+
+def prefill_plan_for(storage, committed, rows, query_heads, sequences=1):
+    """Split count of a chunked prefill sized for the GPU and the storage's layout (kvx_prefill_plan_for)."""
+    splits = lib().kvx_prefill_plan_for(C.byref(storage.layout), committed, rows, query_heads, sequences)
+    if not splits:
+        raise KvxError(-1, "kvx_prefill_plan_for: bad layout or head counts")
+    return splits
 
 
 def prefill_plan(committed, rows, kv_heads, query_heads, fmt=INT4, sequences=1):

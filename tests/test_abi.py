@@ -417,3 +417,29 @@ def test_prefill_groups_of_tiles_rule():
     assert together(4, 6, 256, 16384, 2048, 4) == 1         # head dimension 256 has kernels of its own
     assert together(8, 4, 64, 0, 8, 32) == 1                # one tile
     assert together(8, 3, 64, 0, 8, 32) == 1 and together(8, 0, 64, 0, 8, 32) == 0
+
+
+def test_prefill_plan_by_layout():
+    """kvx_prefill_plan_for: head dimension 256 is kvx_prefill_plan_batch; 64 and 128 take the fewest
+    splits that make 4096 workgroups (groups of tiles counted as the kernels form them), none
+    shorter than 4 pages."""
+    import ctypes as C
+
+    def plan(heads, group, dim, committed, rows, sequences=1, fmt=kvx.INT4):
+        layout = kvx.Layout(1, heads, dim, fmt, 0.0)
+        return kvx.lib().kvx_prefill_plan_for(C.byref(layout), committed, rows, heads * group, sequences)
+
+    assert plan(8, 4, 64, 16384, 2048) == 8         # 64 groups of four tiles x 8 heads x 8 splits
+    assert plan(8, 4, 64, 16385, 2048) == 2         # tile by tile: 256 tiles x 8 heads x 2
+    assert plan(2, 8, 128, 16384, 2048) == 8        # 256 tiles x 2 heads x 8
+    assert plan(8, 4, 64, 8192, 256) == 32          # 8 groups x 8 heads: 32 splits are the most there are
+    assert plan(2, 8, 128, 0, 64) == 1              # two pages of history: nothing to cut
+    assert plan(2, 8, 128, 1000, 64) == 8           # 33 pages: at least 4 to a split
+    for committed, rows, sequences in ((16384, 2048, 1), (16384, 2048, 4), (100, 256, 2)):
+        assert plan(4, 6, 256, committed, rows, sequences) == kvx.prefill_plan(committed, rows, 4, 24, kvx.INT4, sequences)
+    assert plan(8, 0, 64, 0, 8) == 0 and plan(8, 4, 64, 0, 8, sequences=0) == 0
+    bad = kvx.Layout(1, 0, 64, kvx.INT4, 0.0)
+    assert kvx.lib().kvx_prefill_plan_for(C.byref(bad), 0, 8, 8, 1) == 0
+    # absurd sizes neither hang nor wrap
+    for committed, rows in ((0xFFFFFFFF, 0xFFFFFFFF), (0, 0), (0xFFFFFFFF, 1), (5, 0xFFFFFFFF)):
+        assert 0 <= plan(8, 4, 64, committed, rows) <= 32

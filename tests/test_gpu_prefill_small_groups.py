@@ -46,7 +46,14 @@ def test_grouped_tiles_match_the_oracle(layout, fmt):
     # a launch too small for groups, then one of the size that takes them: 32 splits of a ragged
     # chunk (the last group and the last tile partly filled)
     cases = ((0, 40, 1, False), (32 * int(rng.integers(4, 14)), 251, 32, True))
+    heads, group, dim = layout
+    planned = kvx.lib().kvx_prefill_plan_for(C.byref(kvx.Layout(1, heads, dim, fmt, 0.0)), 32 * 40, 251, heads * group, 1)
+    assert 1 <= planned <= 12        # 48 pages: at least 4 to a split
+    cases += ((32 * 40, 251, planned, None),)
     for committed, rows, splits, large in cases:
+        if large is None:            # the plan's splits, grouped or not as the rule has it
+            A.prefill_case(fmt, committed, rows, forced_splits=splits)
+            continue
         print(f"grouped prefill layout={layout} fmt={fmt} committed={committed} rows={rows} splits={splits}",
               flush=True)
         assert together(layout, fmt, committed, rows, splits) == (LAYOUTS[layout] if large else 1)
