@@ -82,7 +82,7 @@ def parse():
     ap.add_argument("--verify-splits", type=int, default=0,
                     help="tree-verify: splits per sequence instead of the library's plan (experiments)")
     ap.add_argument("--workload", choices=["decode", "decode-single", "tree-verify", "prefill", "qkv-prepare", "shared-prefix",
-                                           "stream-ceiling", "control-plane", "decode-layout"], default="decode",
+                                           "stream-ceiling", "control-plane", "decode-layout", "prefill-layout"], default="decode",
                     help="decode = batch-32 mixed-length int4 decode, the headline metric (default); "
                          "decode-single = one sequence of 32768 tokens, the 16 per-layer calls replayed "
                          "as one HIP graph; tree-verify = 16-node tree verify and prefill = chunked prefill with a shared "
@@ -90,15 +90,18 @@ def parse():
                          "delivers for the headline batch's bytes under request shapes other than the "
                          "decode kernel's (linear, 16-byte coalesced, page order, pool size); control-plane = "
                          "the host calls of a batch-32 step (prefix page cache, sequence records), no GPU work; "
-                         "decode-layout = one-row decode over the reference's other layouts (--layout)")
-    ap.add_argument("--layout", choices=["hd128", "hd64"], default="hd128",
-                    help="decode-layout: 2 KV heads x 8 x 128 or 8 x 4 x 64")
+                         "decode-layout = one-row decode, prefill-layout = a prefill chunk, over the reference's "
+                         "other layouts (--layout)")
+    ap.add_argument("--layout", choices=["hd128", "hd64", "k2q4d128", "k4q2d128"], default="hd128",
+                    help="decode-layout, prefill-layout: 2 KV heads x 8 x 128 or 8 x 4 x 64; prefill-layout "
+                         "also 2 x 4 x 128 and 4 x 2 x 128")
     ap.add_argument("--format", choices=["bf16", "fp8", "int8", "int4"], default=None,
                     help="page format of the prefill workload (default bf16) and of the shared-prefix "
                          "and tree-verify workloads (default int4; no fp8)")
     args = ap.parse_args()
     if args.format is None:
-        args.format = "int4" if args.workload in ("shared-prefix", "tree-verify", "decode-layout") else "bf16"
+        args.format = "int4" if args.workload in ("shared-prefix", "tree-verify", "decode-layout",
+                                                   "prefill-layout") else "bf16"
     return args
 
 
@@ -1407,6 +1410,84 @@ def decode_layout(args):
     print(json.dumps(result))
 
 
+def prefill_layout(args):
+    """A chunk of chunked prefill over the reference's other shipped layouts (2 KV heads x 8 x 128,
+    8 x 4 x 64) and two with smaller groups of query heads (2 x 4 x 128, 4 x 2 x 128): `--prefill-chunk`
+    rows (2048 by default) over 16 384 tokens of history, one sequence, one layer per call, splits
+    from kvx_prefill_plan_for.  Timed on a history that ends on a page boundary, where the tiles that
+    begin in the same page share a workgroup and a staged page, and on the same history plus one
+    token, where every tile runs on its own.  `value` is the matrix-core rate of the first."""
+    import numpy as np
+    import torch
+    from richengine_amd import kvx
+
+    torch.cuda.set_device(0)
+    heads, group, dim = {"hd128": (2, 8, 128), "hd64": (8, 4, 64), "k2q4d128": (2, 4, 128),
+                         "k4q2d128": (4, 2, 128)}[args.layout]
+    fmt = {"bf16": kvx.BF16, "fp8": kvx.FP8, "int8": kvx.INT8, "int4": kvx.INT4}[args.format]
+    rows, history = args.prefill_chunk, 16384
+    query_heads = heads * group
+    n_pages = (history + 1 + rows + 31) // 32
+    storage = kvx.Storage(1, heads, dim, fmt, 8192, 8192, aligned=True)
+    storage.allocate_all()
+    table = storage.table(np.random.default_rng(args.seed).permutation(n_pages).astype(np.uint32))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(args.seed)
+    for done in range(0, n_pages * 32, 2048):
+        n = min(2048, n_pages * 32 - done)
+        k = torch.randn((heads, n, dim), generator=gen, device="cuda").bfloat16()
+        v = torch.randn((heads, dim, n), generator=gen, device="cuda").bfloat16()
+        kvx.append(storage, 0, k, v, [table], [kvx.ChunkParams(done, n, n, n_pages)], heads * n * dim)
+    q = torch.randn((heads, rows, group, dim), generator=gen, device="cuda").bfloat16()
+    out = torch.zeros_like(q)
+    layout = kvx.Layout(1, heads, dim, fmt, 0.0)
+
+    def timed(committed):
+        splits = kvx.prefill_plan_for(storage, committed, rows, query_heads)
+        together = kvx.lib().kvx_debug_prefill_tiles_together(C.byref(layout), query_heads, committed, rows, splits)
+        params = kvx.PrefillParams(committed, rows, rows, n_pages, kvx.KvLayer(), splits, 0.0)
+        ws = torch.empty(kvx.prefill_workspace_bytes(storage, rows, query_heads, splits), dtype=torch.uint8,
+                         device="cuda")
+        call = lambda: kvx.attend_prefill(storage, 0, query_heads, q, out, table, params, ws)
+        for _ in range(max(args.warmup, 1)):
+            call()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps * 1e-3, int(splits), int(together)
+
+    aligned_s, aligned_splits, together = timed(history)
+    alone_s, alone_splits, alone_together = timed(history + 1)
+    flops = 4.0 * dim * query_heads * rows * (history + (rows + 1) / 2)
+    peak = 2500.0   # the tiles multiply bf16 (fp16 on fp8 pages): 2.5 PFLOP/s dense either way
+    achieved = flops / aligned_s / 1e12
+    result = {
+        "metric": "prefill_attention_TFLOPs", "value": round(achieved, 1), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": max(args.warmup, 1), "ms_per_step": round(aligned_s * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16 MFMA" if args.format == "fp8" else "bf16 MFMA", "data": "synthetic",
+        "config": {"workload": f"chunked prefill attention, {heads} KV heads x {group} x {dim} ({args.layout}), "
+                               f"{args.format} pages, {rows} rows over {history} tokens, one sequence, one layer "
+                               f"per call", "splits": aligned_splits, "tiles_per_workgroup": together,
+                   "seed": args.seed},
+        "one_token_past_the_page_boundary": {"ms_per_step": round(alone_s * 1e3, 4), "splits": alone_splits,
+                                             "tiles_per_workgroup": alone_together,
+                                             "TFLOPs": round(flops / alone_s / 1e12, 1)},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "kernel": "prefill_group_small_kernel / prefill_split_small_kernel + prefill_reduce_kernel "
+                               "(the call; the split kernel is all but a few microseconds of it)",
+                     "flops_per_launch": flops, "ms_per_launch": round(aligned_s * 1e3, 4)},
+        "cpu_baseline": None,
+    }
+    storage.close()
+    print(json.dumps(result))
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -1429,7 +1510,11 @@ def main():
         if args.workload == "control-plane":
             return control_plane(args)
         if args.workload == "decode-layout":
+            if args.layout not in ("hd128", "hd64"):
+                sys.exit("decode-layout takes --layout hd128 or hd64")
             return decode_layout(args)
+        if args.workload == "prefill-layout":
+            return prefill_layout(args)
         return tree_verify(args) if args.workload == "tree-verify" else chunked_prefill(args)
     import numpy as np
     import torch
