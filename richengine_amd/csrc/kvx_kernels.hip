@@ -1392,10 +1392,12 @@ __global__ __launch_bounds__(256) void attend_reduce_kernel(const float *__restr
                                                             const float *__restrict__ statistics,
                                                             uint16_t *__restrict__ output,
                                                             AttendArgs a) {
-  const uint32_t fused_row = blockIdx.x, head = blockIdx.y, li = blockIdx.z;
+  // blockDim.y rows to a workgroup, each on waves of its own (no row waits for another)
+  const uint32_t fused_row = blockIdx.x * blockDim.y + threadIdx.y, head = blockIdx.y, li = blockIdx.z;
   const AttendLane &l = a.lane[li];
   if (!attend_contract(l, a)) return;
   const uint32_t M = a.row_capacity * a.group, D = a.head_dim, d = threadIdx.x;
+  if (fused_row >= M) return;
   const uint16_t value =
       reduce_row(partials, statistics, a.group, D, M, l.committed, l.active_rows, l.split_count,
                  l.row_base + uint64_t(head) * l.split_count * M, fused_row);
@@ -1423,11 +1425,12 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float *__rest
                                                              const float *__restrict__ statistics,
                                                              uint16_t *__restrict__ output,
                                                              PrefillArgs p) {
-  const uint32_t fused_row = blockIdx.x, head = blockIdx.y, tile = blockIdx.z;
+  const uint32_t fused_row = blockIdx.x * blockDim.y + threadIdx.y, head = blockIdx.y, tile = blockIdx.z;
   const uint32_t tile_start = tile * KVX_PREFILL_TILE_ROWS;
   if (!prefill_contract(p) || tile_start >= p.rows) return;
   const uint32_t active = min(KVX_PREFILL_TILE_ROWS, p.rows - tile_start);
   const uint32_t M = KVX_PREFILL_TILE_ROWS * p.group, D = p.head_dim;
+  if (fused_row >= M) return;
   const uint64_t tile_offset = (uint64_t(head) * p.stride + tile_start) * p.group * D;
   const uint16_t value =
       reduce_row(partials, statistics, p.group, D, M, p.committed + tile_start, active, p.splits,
@@ -2139,7 +2142,9 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
       });
     if (rc) return rc;
     if (phases & 2u) {
-      hipLaunchKernelGGL(attend_reduce_kernel, dim3(M, H, a.n_lanes), dim3((D + 63) / 64 * 64), 0, stream, partials,
+      const uint32_t row_threads = (D + 63) / 64 * 64, together = 256 / row_threads;  // rows to a workgroup
+      hipLaunchKernelGGL(attend_reduce_kernel, dim3((M + together - 1) / together, H, a.n_lanes),
+                         dim3(row_threads, together), 0, stream, partials,
                          statistics, static_cast<uint16_t *>(output), a);
       if ((rc = check_launch("attend_reduce_kernel"))) return rc;
     }
@@ -2734,7 +2739,9 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
     });
   });
   if (rc) return rc;
-  hipLaunchKernelGGL(prefill_reduce_kernel, dim3(M, H, tiles), dim3((D + 63) / 64 * 64), 0, st, partials, statistics,
+  const uint32_t row_threads = (D + 63) / 64 * 64, together = 256 / row_threads;  // rows to a workgroup
+  hipLaunchKernelGGL(prefill_reduce_kernel, dim3((M + together - 1) / together, H, tiles),
+                     dim3(row_threads, together), 0, st, partials, statistics,
                      static_cast<uint16_t *>(output), p);
   return check_launch("prefill_reduce_kernel");
 }
