@@ -1326,14 +1326,15 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
 // Fixed-order merge of one fused row's splits (reference:
 // common/paged_attention_tile.h:362-417).  One thread per dimension, in whole waves;
 // returns the thread's bf16 element, zero for rows past the live ones.
+template <uint32_t kAhead>
 __device__ __forceinline__ uint16_t reduce_row(const float *__restrict__ partials,
                                const float *__restrict__ statistics, uint32_t G, uint32_t D,
                                uint32_t M, uint32_t committed, uint32_t active_rows,
                                uint32_t splits, uint64_t head_row, uint32_t fused_row) {
   // Workgroups of whole waves: thread d sums dimension d (threads past D only lend their
   // lanes).  Lane i of every wave holds the statistics of split base + i, 64 splits at a
-  // time, and hands weight and term round with shuffles; the partial values of 32 splits
-  // are asked for together and then added in split order.
+  // time, and hands weight and term round with shuffles; the partial values of kAhead splits
+  // (32; 8 for launches of at most 8 splits) are asked for together and then added in split order.
   const uint32_t d = threadIdx.x, lane = threadIdx.x & 63u;
   if (fused_row / G >= active_rows) return 0;
   const uint32_t pages = (committed + active_rows + kPage - 1) / kPage;
@@ -1345,7 +1346,6 @@ __device__ __forceinline__ uint16_t reduce_row(const float *__restrict__ partial
   };
   // The statistics of the first 64 splits and the partial values of the first kAhead are asked
   // for together, before anything waits.
-  constexpr uint32_t kAhead = 32;
   float first_max = -INFINITY, first_sum = 0.0f;
   if (lane < written) {
     first_max = statistic(lane)[0];
@@ -1388,6 +1388,7 @@ __device__ __forceinline__ uint16_t reduce_row(const float *__restrict__ partial
   return f32_to_bf16(denominator > 0.0f ? __fdiv_rn(numerator, denominator) : 0.0f);
 }
 
+template <uint32_t AHEAD>
 __global__ __launch_bounds__(256) void attend_reduce_kernel(const float *__restrict__ partials,
                                                             const float *__restrict__ statistics,
                                                             uint16_t *__restrict__ output,
@@ -1399,7 +1400,7 @@ __global__ __launch_bounds__(256) void attend_reduce_kernel(const float *__restr
   const uint32_t M = a.row_capacity * a.group, D = a.head_dim, d = threadIdx.x;
   if (fused_row >= M) return;
   const uint16_t value =
-      reduce_row(partials, statistics, a.group, D, M, l.committed, l.active_rows, l.split_count,
+      reduce_row<AHEAD>(partials, statistics, a.group, D, M, l.committed, l.active_rows, l.split_count,
                  l.row_base + uint64_t(head) * l.split_count * M, fused_row);
   if (d >= D) return;
   if (output)
@@ -1421,6 +1422,7 @@ __global__ __launch_bounds__(256) void attend_reduce_kernel(const float *__restr
   a.hidden[(hidden_row * query_heads + query_head) * D + d] = hidden;
 }
 
+template <uint32_t AHEAD>
 __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float *__restrict__ partials,
                                                              const float *__restrict__ statistics,
                                                              uint16_t *__restrict__ output,
@@ -1433,7 +1435,7 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float *__rest
   if (fused_row >= M) return;
   const uint64_t tile_offset = (uint64_t(head) * p.stride + tile_start) * p.group * D;
   const uint16_t value =
-      reduce_row(partials, statistics, p.group, D, M, p.committed + tile_start, active, p.splits,
+      reduce_row<AHEAD>(partials, statistics, p.group, D, M, p.committed + tile_start, active, p.splits,
                  (uint64_t(tile) * p.kv_heads + head) * p.splits * M, fused_row);
   if (threadIdx.x < D) output[tile_offset + uint64_t(fused_row) * D + threadIdx.x] = value;
 }
@@ -2143,7 +2145,8 @@ static int attend_generic(const kvx_storage *s, kvx_kv_layer kv, uint32_t query_
     if (rc) return rc;
     if (phases & 2u) {
       const uint32_t row_threads = (D + 63) / 64 * 64, together = 256 / row_threads;  // rows to a workgroup
-      hipLaunchKernelGGL(attend_reduce_kernel, dim3((M + together - 1) / together, H, a.n_lanes),
+      hipLaunchKernelGGL(max_splits <= 8 ? attend_reduce_kernel<8> : attend_reduce_kernel<32>,
+                         dim3((M + together - 1) / together, H, a.n_lanes),
                          dim3(row_threads, together), 0, stream, partials,
                          statistics, static_cast<uint16_t *>(output), a);
       if ((rc = check_launch("attend_reduce_kernel"))) return rc;
@@ -2740,7 +2743,8 @@ int kv_attend_prefill(const kvx_storage *s, uint32_t layer, uint32_t query_heads
   });
   if (rc) return rc;
   const uint32_t row_threads = (D + 63) / 64 * 64, together = 256 / row_threads;  // rows to a workgroup
-  hipLaunchKernelGGL(prefill_reduce_kernel, dim3((M + together - 1) / together, H, tiles),
+  hipLaunchKernelGGL(params->split_count <= 8 ? prefill_reduce_kernel<8> : prefill_reduce_kernel<32>,
+                     dim3((M + together - 1) / together, H, tiles),
                      dim3(row_threads, together), 0, st, partials, statistics,
                      static_cast<uint16_t *>(output), p);
   return check_launch("prefill_reduce_kernel");
